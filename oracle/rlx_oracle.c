@@ -1,0 +1,481 @@
+/*
+ * CPU oracle for the GGUF dequant-matmul / FakeQuantize path of MIT-RLX/rlx.
+ *
+ * TEST INFRASTRUCTURE ONLY.  This file restates, in plain C, the algorithm the
+ * reference runs on its CPU backend.  It is the checker the HIP kernels are
+ * compared against; nothing in the shipped library links or calls it.
+ * Build: `make -C oracle` (gcc -O2 -ffp-contract=off -fno-fast-math), so no
+ * multiply-add is ever fused and every rounding step matches the scalar Rust.
+ *
+ * Pinning status (which independent check pins each function):
+ *   f16 -> f32            exhaustive 65536 values vs numpy.float16 (library routine)
+ *   f32 -> f16 / bf16     RNE, vs numpy.float16 cast / closed-form bit rule
+ *   Q8_0 / Q4_0 / Q4_K    the reference's own known-answer blocks
+ *                         (rlx-gguf/src/lib.rs:1187-1264) + independent numpy
+ *                         bit-field restatements on random bytes
+ *   gguf_matmul_bt        reference tests rlx-cpu/src/gguf_matmul.rs:238-277 and
+ *                         rlx-runtime/tests/dequant_matmul_gguf.rs:176-308
+ *                         (layout idx = j*k + p), f64 dense matmul (textbook)
+ *   fake_quantize         closed forms (channel max -> code +-q_max, all-zero
+ *                         channel, constructed ties, NaN), shapes/inputs of
+ *                         rlx-mlx/tests/autodiff_fakequant_parity.rs:189-308
+ *   philox4x32            Random123 known-answer vectors when run with the
+ *                         standard multiplier; the reference's own multiplier
+ *                         (rlx-ir/src/rng.rs:55) only changes that constant
+ *   philox normal()       PARITY UNPINNED in the last ulp: the reference calls
+ *                         Rust std ln/sqrt/cos (platform libm); no reference test
+ *                         holds literal values (rlx-ir/src/rng.rs:149-205)
+ *   encoders              not here: the reference has none (rlx-gguf is
+ *                         decode-only), so there is nothing to restate
+ */
+#include <math.h>
+#include <stddef.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+#define QK8_0 32
+#define QK4_0 32
+#define QK_K 256
+#define K_SCALE_SIZE 12
+
+/* scheme ids shared with include/rlx_mi355x.h (rlx-ir/src/quant.rs:39-79 order) */
+enum { ORC_Q4K = 5, ORC_Q4_0 = 11, ORC_Q8_0 = 12 };
+
+/* ---- half / bfloat16 -------------------------------------------------- */
+
+/* half::f16::to_f32 as used by rlx-gguf/src/lib.rs:569-571: exact IEEE widening. */
+float orc_f16_to_f32(uint16_t h) {
+    uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+    uint32_t exp = (h >> 10) & 0x1Fu;
+    uint32_t man = h & 0x3FFu;
+    uint32_t bits;
+    if (exp == 0) {
+        if (man == 0) {
+            bits = sign;
+        } else { /* subnormal: normalise */
+            int e = -1;
+            do {
+                man <<= 1;
+                e++;
+            } while (!(man & 0x400u));
+            man &= 0x3FFu;
+            bits = sign | ((uint32_t)(127 - 15 - e) << 23) | (man << 13);
+        }
+    } else if (exp == 31) {
+        bits = sign | 0x7F800000u | (man << 13);
+    } else {
+        bits = sign | ((exp + 127 - 15) << 23) | (man << 13);
+    }
+    float f;
+    memcpy(&f, &bits, 4);
+    return f;
+}
+
+/* half::f16::from_f32 (rlx-driver/src/arena.rs:72-76): round-to-nearest-even, NaN kept quiet. */
+uint16_t orc_f32_to_f16(float f) {
+    uint32_t x;
+    memcpy(&x, &f, 4);
+    uint16_t sign = (uint16_t)((x >> 16) & 0x8000u);
+    uint32_t exp = (x >> 23) & 0xFFu;
+    uint32_t man = x & 0x7FFFFFu;
+    if (exp == 255) {
+        if (man) return (uint16_t)(sign | 0x7E00u | (man >> 13));
+        return (uint16_t)(sign | 0x7C00u);
+    }
+    int e = (int)exp - 127 + 15;
+    if (e >= 31) return (uint16_t)(sign | 0x7C00u);
+    if (e <= 0) {
+        if (e < -10) return sign;
+        man |= 0x800000u;
+        int shift = 14 - e; /* 14..24 */
+        uint32_t half_man = man >> shift;
+        uint32_t rem = man & ((1u << shift) - 1);
+        uint32_t halfway = 1u << (shift - 1);
+        if (rem > halfway || (rem == halfway && (half_man & 1))) half_man++;
+        return (uint16_t)(sign | half_man);
+    }
+    uint32_t half_man = man >> 13;
+    uint32_t rem = man & 0x1FFFu;
+    uint16_t out = (uint16_t)(sign | ((uint32_t)e << 10) | half_man);
+    if (rem > 0x1000u || (rem == 0x1000u && (half_man & 1))) out++; /* carry may roll into exp/inf: correct */
+    return out;
+}
+
+/* half::bf16::from_f32 (rlx-driver/src/arena.rs:78-83): RNE on the upper 16 bits. */
+uint16_t orc_f32_to_bf16(float f) {
+    uint32_t x;
+    memcpy(&x, &f, 4);
+    if ((x & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((x >> 16) | 0x0040u);
+    uint32_t round_bit = 0x8000u;
+    if ((x & round_bit) && (x & (3u * round_bit - 1u))) return (uint16_t)((x >> 16) + 1);
+    return (uint16_t)(x >> 16);
+}
+
+float orc_bf16_to_f32(uint16_t h) {
+    uint32_t x = (uint32_t)h << 16;
+    float f;
+    memcpy(&f, &x, 4);
+    return f;
+}
+
+/* ---- block geometry (rlx-ir/src/quant.rs:138-164, rlx-gguf/src/lib.rs:393-414) ---- */
+
+int orc_block_elems(int scheme) {
+    switch (scheme) {
+    case ORC_Q4K: return QK_K;
+    case ORC_Q4_0: return QK4_0;
+    case ORC_Q8_0: return QK8_0;
+    default: return 0;
+    }
+}
+
+int orc_block_bytes(int scheme) {
+    switch (scheme) {
+    case ORC_Q4K: return 2 + 2 + K_SCALE_SIZE + QK_K / 2; /* 144 */
+    case ORC_Q4_0: return 2 + QK4_0 / 2;                  /* 18 */
+    case ORC_Q8_0: return 2 + QK8_0;                      /* 34 */
+    default: return 0;
+    }
+}
+
+/* bytes_for (rlx-gguf/src/lib.rs:393-399): -1 when n is not a multiple of the block. */
+int64_t orc_bytes_for(int scheme, int64_t n) {
+    int be = orc_block_elems(scheme);
+    if (be == 0 || n % be != 0) return -1;
+    return (n / be) * orc_block_bytes(scheme);
+}
+
+/* ---- block decoders ---------------------------------------------------- */
+
+static float read_f16_le(const uint8_t *b) { return orc_f16_to_f32((uint16_t)(b[0] | (b[1] << 8))); }
+
+/* rlx-gguf/src/lib.rs:574-581 */
+void orc_dequant_q8_0_block(const uint8_t *block, float *out) {
+    float d = read_f16_le(block);
+    const uint8_t *qs = block + 2;
+    for (int i = 0; i < QK8_0; i++) out[i] = d * (float)(int8_t)qs[i];
+}
+
+/* rlx-gguf/src/lib.rs:584-597: low nibbles -> first half, high nibbles -> second half. */
+void orc_dequant_q4_0_block(const uint8_t *block, float *out) {
+    float d = read_f16_le(block);
+    const uint8_t *qs = block + 2;
+    for (int j = 0; j < QK4_0 / 2; j++) {
+        int v0 = (int)(qs[j] & 0x0F) - 8;
+        out[j] = d * (float)v0;
+    }
+    for (int j = 0; j < QK4_0 / 2; j++) {
+        int v1 = (int)(qs[j] >> 4) - 8;
+        out[QK4_0 / 2 + j] = d * (float)v1;
+    }
+}
+
+/* rlx-gguf/src/lib.rs:743-751 */
+void orc_get_scale_min_k4(int j, const uint8_t *q, uint8_t *sc, uint8_t *mn) {
+    if (j < 4) {
+        *sc = q[j] & 63;
+        *mn = q[j + 4] & 63;
+    } else {
+        *sc = (uint8_t)((q[j + 4] & 0x0F) | ((q[j - 4] >> 6) << 4));
+        *mn = (uint8_t)((q[j + 4] >> 4) | ((q[j] >> 6) << 4));
+    }
+}
+
+/* rlx-gguf/src/lib.rs:754-780: four roundings per element, none fused. */
+void orc_dequant_q4_k_block(const uint8_t *block, float *out) {
+    float d = read_f16_le(block);
+    float dmin = read_f16_le(block + 2);
+    const uint8_t *scales = block + 4;
+    const uint8_t *qs = block + 4 + K_SCALE_SIZE;
+    int is = 0, oi = 0;
+    for (int j = 0; j < 8; j += 2) {
+        uint8_t sc0, m0, sc1, m1;
+        orc_get_scale_min_k4(j, scales, &sc0, &m0);
+        orc_get_scale_min_k4(j + 1, scales, &sc1, &m1);
+        float d0 = d * (float)sc0;
+        float m0f = dmin * (float)m0;
+        float d1 = d * (float)sc1;
+        float m1f = dmin * (float)m1;
+        for (int l = 0; l < 32; l++) {
+            uint8_t q = qs[is + l];
+            float t = d0 * (float)(q & 0x0F);
+            out[oi++] = t - m0f;
+        }
+        for (int l = 0; l < 32; l++) {
+            uint8_t q = qs[is + l];
+            float t = d1 * (float)(q >> 4);
+            out[oi++] = t - m1f;
+        }
+        is += 32;
+    }
+}
+
+/* rlx-cpu/src/gguf_matmul.rs:25-37 */
+static void dequant_block(int scheme, const uint8_t *block, float *out) {
+    switch (scheme) {
+    case ORC_Q4K: orc_dequant_q4_k_block(block, out); break;
+    case ORC_Q4_0: orc_dequant_q4_0_block(block, out); break;
+    case ORC_Q8_0: orc_dequant_q8_0_block(block, out); break;
+    default: break;
+    }
+}
+
+/* Whole-tensor forms (rlx-gguf/src/lib.rs:600-633, 974-1013). Returns 0, or -1 on a bad size. */
+int orc_dequant(int scheme, const uint8_t *bytes, int64_t nbytes, int64_t n, float *out) {
+    int be = orc_block_elems(scheme), bb = orc_block_bytes(scheme);
+    if (be == 0 || n % be != 0) return -1;
+    int64_t nb = n / be;
+    if (nbytes != nb * bb) return -1;
+    float tmp[QK_K];
+    for (int64_t i = 0; i < nb; i++) {
+        dequant_block(scheme, bytes + i * bb, tmp);
+        memcpy(out + i * be, tmp, (size_t)be * sizeof(float));
+    }
+    return 0;
+}
+
+/* ---- matmul ------------------------------------------------------------ */
+
+/* rlx-cpu/src/gguf_matmul.rs:40-95, loop for loop: out zeroed, then for each block in
+ * storage order, for each element t: j = idx / k, p = idx % k, out[mi*n+j] += x[mi*k+p]*w. */
+int orc_gguf_matmul_bt(const float *x, const uint8_t *w_bytes, int64_t w_nbytes, float *out, int64_t m, int64_t k,
+                       int64_t n, int scheme) {
+    int be = orc_block_elems(scheme), bb = orc_block_bytes(scheme);
+    if (be == 0) return -1;
+    int64_t total = k * n;
+    if (total % be != 0) return -1;
+    int64_t num_blocks = total / be;
+    if (w_nbytes != num_blocks * bb) return -1;
+    for (int64_t i = 0; i < m * n; i++) out[i] = 0.0f;
+    float blk[QK_K];
+    if (m == 1) {
+        for (int64_t bi = 0; bi < num_blocks; bi++) {
+            dequant_block(scheme, w_bytes + bi * bb, blk);
+            int64_t idx0 = bi * be;
+            for (int t = 0; t < be; t++) {
+                int64_t idx = idx0 + t;
+                int64_t j = idx / k;
+                int64_t p = idx % k;
+                float prod = x[p] * blk[t];
+                out[j] = out[j] + prod;
+            }
+        }
+        return 0;
+    }
+    for (int64_t bi = 0; bi < num_blocks; bi++) {
+        dequant_block(scheme, w_bytes + bi * bb, blk);
+        int64_t idx0 = bi * be;
+        for (int t = 0; t < be; t++) {
+            int64_t idx = idx0 + t;
+            int64_t j = idx / k;
+            int64_t p = idx % k;
+            float w_val = blk[t];
+            for (int64_t mi = 0; mi < m; mi++) {
+                float prod = x[mi * k + p] * w_val;
+                out[mi * n + j] = out[mi * n + j] + prod;
+            }
+        }
+    }
+    return 0;
+}
+
+/* Error yardstick: same decoded weights, products and sums in f64. Rows [n0, n1) only. */
+int orc_gguf_matmul_f64(const float *x, const uint8_t *w_bytes, int64_t w_nbytes, double *out, int64_t m, int64_t k,
+                        int64_t n, int scheme, int64_t n0, int64_t n1) {
+    int be = orc_block_elems(scheme), bb = orc_block_bytes(scheme);
+    if (be == 0 || k % be != 0) return -1;
+    if (w_nbytes != (k * n / be) * bb) return -1;
+    int64_t bpr = k / be;
+    float blk[QK_K];
+    for (int64_t j = n0; j < n1; j++) {
+        for (int64_t mi = 0; mi < m; mi++) out[mi * (n1 - n0) + (j - n0)] = 0.0;
+        for (int64_t b = 0; b < bpr; b++) {
+            dequant_block(scheme, w_bytes + (j * bpr + b) * bb, blk);
+            for (int64_t mi = 0; mi < m; mi++) {
+                double acc = 0.0;
+                const float *xr = x + mi * k + b * be;
+                for (int t = 0; t < be; t++) acc += (double)xr[t] * (double)blk[t];
+                out[mi * (n1 - n0) + (j - n0)] += acc;
+            }
+        }
+    }
+    return 0;
+}
+
+/* ---- FakeQuantize (rlx-cpu/src/thunk.rs:11159-11253, 14163-14175) ------- */
+
+enum { ORC_SCALE_PER_BATCH = 0, ORC_SCALE_EMA = 1, ORC_SCALE_FIXED = 2 };
+enum { ORC_ROUND_HALF_AWAY = 0, ORC_ROUND_HALF_EVEN = 1 };
+
+static float clampf(float v, float lo, float hi) {
+    /* Rust f32::clamp: NaN passes through. */
+    if (v < lo) return lo;
+    if (v > hi) return hi;
+    return v;
+}
+
+static float fmax_rust(float a, float b) {
+    /* Rust f32::max: if one side is NaN the other is returned. */
+    if (a != a) return b;
+    if (b != b) return a;
+    return a > b ? a : b;
+}
+
+/* x, out: len floats. codes (optional): len int8 integer codes q. state: chan_dim floats for
+ * EMA (updated in place) / Fixed. scales_out (optional): chan_dim. Returns 0, -1 on bad bits. */
+int orc_fake_quantize(const float *x, float *out, int8_t *codes, int64_t len, int64_t chan_dim, int64_t inner, int bits,
+                      int scale_mode, float decay, float *state, int round_mode, float *scales_out) {
+    float q_max;
+    switch (bits) {
+    case 8: q_max = 127.0f; break;
+    case 4: q_max = 7.0f; break;
+    case 2: q_max = 1.0f; break;
+    default: return -1;
+    }
+    if (chan_dim < 1) chan_dim = 1;
+    float *scale = scales_out;
+    float local_scale[1];
+    float *heap = NULL;
+    if (!scale) {
+        if (chan_dim == 1) scale = local_scale;
+        else scale = heap = (float *)malloc((size_t)chan_dim * sizeof(float));
+    }
+    if (scale_mode == ORC_SCALE_PER_BATCH || scale_mode == ORC_SCALE_EMA) {
+        float *max_abs = (float *)malloc((size_t)chan_dim * sizeof(float));
+        for (int64_t c = 0; c < chan_dim; c++) max_abs[c] = 0.0f;
+        for (int64_t i = 0; i < len; i++) {
+            int64_t c = chan_dim == 1 ? 0 : (i / inner) % chan_dim;
+            float a = fabsf(x[i]);
+            if (a > max_abs[c]) max_abs[c] = a;
+        }
+        for (int64_t c = 0; c < chan_dim; c++) {
+            float cur = fmax_rust(max_abs[c] / q_max, 1e-12f);
+            if (scale_mode == ORC_SCALE_EMA) {
+                float blended;
+                if (state[c] <= 0.0f) {
+                    blended = cur;
+                } else {
+                    float a = decay * state[c];
+                    float b = (1.0f - decay) * cur;
+                    blended = a + b;
+                }
+                state[c] = blended;
+                scale[c] = blended;
+            } else {
+                scale[c] = cur;
+            }
+        }
+        free(max_abs);
+    } else {
+        for (int64_t c = 0; c < chan_dim; c++) scale[c] = fmax_rust(state[c], 1e-12f);
+    }
+    for (int64_t i = 0; i < len; i++) {
+        int64_t c = chan_dim == 1 ? 0 : (i / inner) % chan_dim;
+        float s = scale[c];
+        float r = x[i] / s;
+        r = round_mode == ORC_ROUND_HALF_EVEN ? rintf(r) : roundf(r);
+        float qv = clampf(r, -q_max, q_max);
+        out[i] = qv * s;
+        if (codes) codes[i] = (qv != qv) ? 0 : (int8_t)qv;
+    }
+    if (heap) free(heap);
+    return 0;
+}
+
+/* ---- Philox4x32-10 (rlx-ir/src/rng.rs:43-143) ---------------------------- */
+
+typedef struct {
+    uint32_t seed[2];
+    uint32_t counter[4];
+    uint32_t buffer[4];
+    uint32_t cursor;
+    uint32_t m0; /* 0xD2561A75 in the reference (rng.rs:55); Random123's is 0xD2511F53 */
+} orc_philox;
+
+void orc_philox_init(orc_philox *p, uint64_t seed, uint32_t m0) {
+    p->seed[0] = (uint32_t)(seed & 0xFFFFFFFFu);
+    p->seed[1] = (uint32_t)(seed >> 32);
+    memset(p->counter, 0, sizeof p->counter);
+    memset(p->buffer, 0, sizeof p->buffer);
+    p->cursor = 4;
+    p->m0 = m0;
+}
+
+void orc_philox_set_counter(orc_philox *p, const uint32_t c[4]) {
+    memcpy(p->counter, c, sizeof p->counter);
+    p->cursor = 4;
+}
+
+static void philox_fill(orc_philox *p) {
+    uint32_t s[4], key[2];
+    memcpy(s, p->counter, sizeof s);
+    key[0] = p->seed[0];
+    key[1] = p->seed[1];
+    for (int r = 0; r < 10; r++) {
+        uint64_t p0 = (uint64_t)s[0] * (uint64_t)p->m0;
+        uint64_t p1 = (uint64_t)s[2] * 0xCD9E8D57ull;
+        uint32_t hi0 = (uint32_t)(p0 >> 32), lo0 = (uint32_t)p0;
+        uint32_t hi1 = (uint32_t)(p1 >> 32), lo1 = (uint32_t)p1;
+        uint32_t n0 = hi1 ^ s[1] ^ key[0];
+        uint32_t n2 = hi0 ^ s[3] ^ key[1];
+        s[0] = n0;
+        s[1] = lo1;
+        s[2] = n2;
+        s[3] = lo0;
+        key[0] += 0x9E3779B9u;
+        key[1] += 0xBB67AE85u;
+    }
+    memcpy(p->buffer, s, sizeof s);
+    p->cursor = 0;
+    if (++p->counter[0] == 0)
+        if (++p->counter[1] == 0)
+            if (++p->counter[2] == 0) ++p->counter[3];
+}
+
+uint32_t orc_philox_next_u32(orc_philox *p) {
+    if (p->cursor >= 4) philox_fill(p);
+    return p->buffer[p->cursor++];
+}
+
+float orc_philox_next_f32(orc_philox *p) {
+    uint32_t bits = orc_philox_next_u32(p) >> 8;
+    return (float)bits / (float)(1u << 24);
+}
+
+/* rng.rs:121-127. Uses this platform's f32 libm (logf/sqrtf/cosf): last-ulp parity unpinned. */
+float orc_philox_normal(orc_philox *p) {
+    float u1 = orc_philox_next_f32(p);
+    if (u1 < 1.17549435e-38f) u1 = 1.17549435e-38f;
+    float u2 = orc_philox_next_f32(p);
+    float r = sqrtf(-2.0f * logf(u1));
+    float theta = 2.0f * 3.14159274101257324f * u2;
+    return r * cosf(theta);
+}
+
+void orc_philox_fill_u32(uint64_t seed, uint32_t m0, uint32_t *out, int64_t n) {
+    orc_philox p;
+    orc_philox_init(&p, seed, m0);
+    for (int64_t i = 0; i < n; i++) out[i] = orc_philox_next_u32(&p);
+}
+
+void orc_philox_fill_uniform(uint64_t seed, float *out, int64_t n) {
+    orc_philox p;
+    orc_philox_init(&p, seed, 0xD2561A75u);
+    for (int64_t i = 0; i < n; i++) out[i] = orc_philox_next_f32(&p);
+}
+
+void orc_philox_fill_normal(uint64_t seed, float *out, int64_t n) {
+    orc_philox p;
+    orc_philox_init(&p, seed, 0xD2561A75u);
+    for (int64_t i = 0; i < n; i++) out[i] = orc_philox_normal(&p);
+}
+
+/* One Philox block for an explicit (counter, key): used by the known-answer test. */
+void orc_philox_block(const uint32_t counter[4], const uint32_t key[2], uint32_t m0, uint32_t out[4]) {
+    orc_philox p;
+    orc_philox_init(&p, ((uint64_t)key[1] << 32) | key[0], m0);
+    orc_philox_set_counter(&p, counter);
+    philox_fill(&p);
+    memcpy(out, p.buffer, sizeof p.buffer);
+}
