@@ -1,0 +1,270 @@
+/*
+ * rlx_mi355x.h — C ABI of the MI355X (gfx950) backend for RLX's GGUF dequant-matmul
+ * and FakeQuantize path.
+ *
+ * Two levels, both plain C (pointers and sizes only):
+ *
+ *   1. Operator level: the device-side replacements for the functions the reference
+ *      calls on its CPU hot path (rlx_gguf::dequant_*, rlx_cpu::gguf_matmul::gguf_matmul_bt,
+ *      the FakeQuantize thunk). Device pointers in, device pointers out, on a stream.
+ *
+ *   2. Graph level: a mirror of rlx-runtime's `Backend` / `ExecutableGraph` traits
+ *      (rlx-runtime/src/backend.rs:146-426) so that a `Device::Mi355x` variant can
+ *      forward `Session::new(dev).compile(g)`, `set_param[_typed]`, `run[_typed]`.
+ *
+ * Every function returns RLX_OK (0) or a negative rlx_status; the text of the last
+ * failure on the calling thread is available from rlx_mi355x_last_error(). No HIP error
+ * is ever swallowed (the reference's ROCm launcher drops them, rlx-rocm/src/launch.rs:53-55).
+ */
+#ifndef RLX_MI355X_H
+#define RLX_MI355X_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define RLX_MI355X_ABI_VERSION 1
+
+typedef enum rlx_status {
+    RLX_OK = 0,
+    RLX_WARN_UNKNOWN_NAME = 1, /* set_param/run given a name the graph does not have: ignored, as the
+                                  reference does silently (rlx-runtime/src/backend.rs:883-901,916-922) */
+    RLX_ERR_INVALID = -1,      /* bad argument / shape / size */
+    RLX_ERR_UNSUPPORTED = -2,  /* op, scheme or dtype this backend does not claim */
+    RLX_ERR_HIP = -3,          /* a HIP call failed; text in last_error */
+    RLX_ERR_NO_DEVICE = -4     /* no gfx950 device / HIP runtime unusable */
+} rlx_status;
+
+/* rlx_ir::DType, declaration order (rlx-ir/src/dtype.rs:20-44). */
+typedef enum rlx_dtype {
+    RLX_F32 = 0, RLX_F16 = 1, RLX_BF16 = 2, RLX_F64 = 3, RLX_I8 = 4, RLX_I16 = 5,
+    RLX_I32 = 6, RLX_I64 = 7, RLX_U8 = 8, RLX_U32 = 9, RLX_BOOL = 10, RLX_C64 = 11
+} rlx_dtype;
+
+/* rlx_ir::quant::QuantScheme, declaration order (rlx-ir/src/quant.rs:39-79). Only the three
+ * GGUF schemes below are claimed; any other value is RLX_ERR_UNSUPPORTED. */
+typedef enum rlx_quant_scheme {
+    RLX_SCHEME_GGUF_Q4K = 5,  /* 256 elems / 144 bytes */
+    RLX_SCHEME_GGUF_Q4_0 = 11, /* 32 elems / 18 bytes  */
+    RLX_SCHEME_GGUF_Q8_0 = 12  /* 32 elems / 34 bytes  */
+} rlx_quant_scheme;
+
+/* rlx_ir::op::ScaleMode (rlx-ir/src/op.rs:73-82). */
+typedef enum rlx_scale_mode { RLX_SCALE_PER_BATCH = 0, RLX_SCALE_EMA = 1, RLX_SCALE_FIXED = 2 } rlx_scale_mode;
+
+/* Rounding of x/s inside FakeQuantize. HALF_AWAY is what rlx-cpu does (f32::round,
+ * rlx-cpu/src/thunk.rs:11249) and is the default; HALF_EVEN is offered because some callers
+ * specify ties-to-even. They differ only on exact .5 ties. */
+typedef enum rlx_round_mode { RLX_ROUND_HALF_AWAY = 0, RLX_ROUND_HALF_EVEN = 1 } rlx_round_mode;
+
+/* ------------------------------------------------------------------------------------------
+ * Device / runtime
+ * ---------------------------------------------------------------------------------------- */
+
+/* 1 when a gfx950 device is present and the kernel module loads; 0 otherwise. Mirrors
+ * `HipRuntime::load() -> None` / `is_available()` (rlx-rocm/src/hip.rs:223-235, rlx-rocm/src/lib.rs:73-75). */
+int rlx_mi355x_is_available(void);
+/* "MI355X" — what `Device::name()` would return for the new variant (rlx-driver/src/device.rs:66-81). */
+const char *rlx_mi355x_device_name(void);
+int rlx_mi355x_abi_version(void);
+/* Thread-local text of the most recent failure ("" if none). Replaces the reference's panics. */
+const char *rlx_mi355x_last_error(void);
+/* gcnArchName, CU count and peak clocks of device 0 as a short text (for bench output). */
+int rlx_mi355x_device_info(char *buf, size_t cap);
+
+/* Raw device memory and streams, for callers without their own HIP binding
+ * (the reference's FFI table: rlx-rocm/src/hip.rs:102-163). `stream` is a hipStream_t; NULL = default stream. */
+int rlx_mi355x_malloc(void **dptr, size_t nbytes);
+int rlx_mi355x_free(void *dptr);
+int rlx_mi355x_memcpy_h2d(void *dst, const void *src, size_t nbytes);
+int rlx_mi355x_memcpy_d2h(void *dst, const void *src, size_t nbytes);
+int rlx_mi355x_memset_u32(void *dst, uint32_t value, size_t n_words, void *stream); /* fill kernel, graph-safe */
+int rlx_mi355x_stream_create(void **stream);
+int rlx_mi355x_stream_destroy(void *stream);
+int rlx_mi355x_stream_sync(void *stream);
+int rlx_mi355x_event_create(void **event);
+int rlx_mi355x_event_destroy(void *event);
+int rlx_mi355x_event_record(void *event, void *stream);
+int rlx_mi355x_event_elapsed_ms(void *start, void *stop, float *ms); /* synchronises on `stop` */
+
+/* ------------------------------------------------------------------------------------------
+ * Format constants (rlx-ir/src/quant.rs:138-183, rlx-gguf/src/lib.rs:377-419)
+ * ---------------------------------------------------------------------------------------- */
+
+int rlx_mi355x_block_elems(int scheme);            /* QuantScheme::gguf_block_size(): 32 / 32 / 256, else 0 */
+int rlx_mi355x_block_bytes(int scheme);            /* QuantScheme::gguf_block_bytes(): 18 / 34 / 144, else 0 */
+int64_t rlx_mi355x_bytes_for(int scheme, int64_t n_elems); /* rlx_gguf bytes_for: -1 if n % block != 0 */
+
+/* ------------------------------------------------------------------------------------------
+ * Packed weights resident in HBM
+ * ---------------------------------------------------------------------------------------- */
+
+/* A GGUF-packed [n, k] matrix (row-major, blocks along k: rlx-cpu/src/gguf_matmul.rs:15-20) repacked once
+ * into the device layout the kernels stream (same byte count per block; 16-row x 128/256-k tiles whose
+ * 16-byte lane slots hold MFMA operand fragments). */
+typedef struct rlx_qweight rlx_qweight;
+
+/* Repack `gguf_bytes` (host, exactly bytes_for(scheme, n*k) long) and upload. Where the reference memcpy's the
+ * bytes into the arena (`set_param_bytes`, rlx-runtime/src/backend.rs:1175-1187). */
+int rlx_mi355x_qweight_create(int scheme, const void *gguf_bytes, size_t nbytes, int64_t n, int64_t k,
+                              rlx_qweight **out);
+/* Same, into caller-owned device memory of rlx_mi355x_qweight_device_bytes_for() bytes (256-byte aligned). */
+int rlx_mi355x_qweight_create_at(int scheme, const void *gguf_bytes, size_t nbytes, int64_t n, int64_t k,
+                                 void *device_mem, rlx_qweight **out);
+void rlx_mi355x_qweight_destroy(rlx_qweight *w);
+size_t rlx_mi355x_qweight_device_bytes(const rlx_qweight *w);
+size_t rlx_mi355x_qweight_device_bytes_for(int scheme, int64_t n, int64_t k);
+/* Host-side repack only (no device): writes device-layout bytes to `out` (size from ..._device_bytes_for). */
+int rlx_mi355x_repack_host(int scheme, const void *gguf_bytes, size_t nbytes, int64_t n, int64_t k, void *out);
+
+/* rlx_gguf::dequant_q8_0 / dequant_q4_0 / dequant_q4_k (rlx-gguf/src/lib.rs:600-633,974-1013) on the device:
+ * out_dev[n*k] f32, row-major [n,k], bit-identical to the reference decoders. */
+int rlx_mi355x_dequant(const rlx_qweight *w, float *out_dev, void *stream);
+
+/* rlx_cpu::gguf_matmul::gguf_matmul_bt (rlx-cpu/src/gguf_matmul.rs:40-95):
+ *   out[m, n] = x[m, k] . W^T, W = decoded [n, k]; out is overwritten (the reference zero-fills first).
+ * x_dev is [m,k] row-major of x_dtype in {RLX_F32, RLX_BF16, RLX_F16}; 16-bit activations stand for the values
+ * the reference's typed boundary would widen to f32 (rlx-runtime/src/backend.rs:49-53). out_dev is f32.
+ * `workspace` must hold rlx_mi355x_gguf_matmul_workspace() bytes (may be NULL when that is 0).
+ * m <= 16 runs the decode kernel (weights streamed once, MFMA 16x16x32); larger m runs the prefill GEMM. */
+int rlx_mi355x_gguf_matmul_bt(const void *x_dev, int x_dtype, const rlx_qweight *w, float *out_dev, int64_t m,
+                              void *workspace, size_t workspace_bytes, void *stream);
+size_t rlx_mi355x_gguf_matmul_workspace(int scheme, int x_dtype, int64_t m, int64_t k, int64_t n);
+
+/* Thunk::FakeQuantize (rlx-cpu/src/thunk.rs:11159-11253) with the layout of quant_layout()
+ * (thunk.rs:14163-14175): channel of flat element i is (i / inner) % chan_dim.
+ *   x_dev, out_dev : len f32 (may alias)
+ *   codes_dev      : optional len int8, the integer codes clamp(round(x/s)) (NULL to skip)
+ *   state_dev      : chan_dim f32; read for FIXED, read+written for EMA, ignored (may be NULL) for PER_BATCH
+ *   scratch_dev    : chan_dim * 4 bytes of device scratch for the per-channel maxima (PER_BATCH / EMA)
+ * bits in {8,4,2} -> q_max {127,7,1}; anything else is RLX_ERR_UNSUPPORTED (the reference panics). */
+int rlx_mi355x_fake_quantize(const float *x_dev, float *out_dev, int8_t *codes_dev, int64_t len, int64_t chan_dim,
+                             int64_t inner, int bits, int scale_mode, float ema_decay, float *state_dev,
+                             int round_mode, void *scratch_dev, void *stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Host utilities that exist because the path needs inputs: the reference has no GGUF encoder
+ * (rlx-gguf is decode-only) and seeds its tensors with Philox (rlx-ir/src/rng.rs:43-143).
+ * ---------------------------------------------------------------------------------------- */
+
+/* Encode a row-major f32 [n_elems] tensor (n_elems % block == 0) into GGUF bytes. Host code, deterministic.
+ * Q8_0/Q4_0 follow the llama.cpp reference quantizers; Q4_K is a simple min/max variant (documented in the
+ * source). `out` must hold rlx_mi355x_bytes_for(scheme, n_elems) bytes. */
+int rlx_mi355x_quantize(int scheme, const float *src, int64_t n_elems, void *out);
+
+/* Philox4x32-10 stream exactly as rlx_ir::rng::Philox4x32 (same constants, key schedule, counter order). */
+void rlx_mi355x_philox_u32(uint64_t seed, uint32_t *out, int64_t n);
+void rlx_mi355x_philox_uniform(uint64_t seed, float *out, int64_t n); /* next_f32(): (u32 >> 8) / 2^24 */
+void rlx_mi355x_philox_normal(uint64_t seed, float *out, int64_t n);  /* normal(): Box-Muller, 2 uniforms/sample */
+
+/* ------------------------------------------------------------------------------------------
+ * Graph level: Backend / ExecutableGraph mirror
+ * ---------------------------------------------------------------------------------------- */
+
+typedef enum rlx_op_kind {
+    RLX_OP_INPUT = 0,          /* OpKind::Input  */
+    RLX_OP_PARAM = 1,          /* OpKind::Param  */
+    RLX_OP_DEQUANT_MATMUL = 2, /* OpKind::DequantMatMul, Op::DequantMatMul{scheme} (rlx-ir/src/op.rs:736-752) */
+    RLX_OP_FAKE_QUANTIZE = 3   /* OpKind::FakeQuantize,  Op::FakeQuantize{bits,axis,ste,scale_mode} (op.rs:407-432) */
+} rlx_op_kind;
+
+#define RLX_MAX_RANK 6
+#define RLX_MAX_INPUTS 2
+
+/* One rlx_ir::Node{id, op, inputs, shape, name} (rlx-ir/src/graph.rs:40-81); id = index in the array. */
+typedef struct rlx_node_desc {
+    uint32_t op_kind;                 /* rlx_op_kind */
+    uint32_t dtype;                   /* rlx_dtype of the node's shape */
+    uint32_t rank;
+    int64_t dims[RLX_MAX_RANK];
+    uint32_t n_inputs;
+    uint32_t inputs[RLX_MAX_INPUTS];  /* node ids */
+    const char *name;                 /* Input / Param name (may be NULL for op nodes) */
+    /* DequantMatMul */
+    uint32_t scheme;                  /* rlx_quant_scheme */
+    /* FakeQuantize */
+    uint32_t bits;                    /* 8, 4, 2 */
+    int32_t axis;                     /* -1 = None (per tensor) */
+    uint32_t scale_mode;              /* rlx_scale_mode; EMA / FIXED take a second input: state [chan_dim] */
+    float ema_decay;
+    uint32_t ste;                     /* SteKind; forward-only backend: carried, not used */
+} rlx_node_desc;
+
+typedef struct rlx_graph_desc {
+    const char *name;
+    const rlx_node_desc *nodes;
+    uint32_t n_nodes;
+    const uint32_t *outputs; /* Graph::set_outputs */
+    uint32_t n_outputs;
+} rlx_graph_desc;
+
+/* The subset of rlx_runtime::CompileOptions (rlx-runtime/src/options.rs:41-87) that means something here. */
+typedef struct rlx_compile_opts {
+    uint32_t arena_alignment; /* bytes, power of two; 0 = 256 */
+    uint32_t fq_round_mode;   /* rlx_round_mode for every FakeQuantize node */
+    uint32_t verbose;         /* RLX_VERBOSE-style plan dump to stderr */
+    uint32_t reserved[5];
+} rlx_compile_opts;
+
+typedef struct rlx_exec rlx_exec; /* Box<dyn ExecutableGraph>: Send, not Sync — one thread at a time */
+
+/* Backend::supported_ops(): the op kinds this backend lowers. Returns the count. */
+size_t rlx_mi355x_supported_ops(const uint32_t **kinds);
+
+/* Backend::compile(graph, options): validates (legalize: unsupported op / scheme / dtype -> NULL with the
+ * reference's legalize message shape), infers (m,k,n) and (chan_dim, inner) as the CPU thunk compiler does
+ * (rlx-cpu/src/thunk.rs:3027-3043, 2567-2598), plans the arena and allocates it. NULL on failure. */
+rlx_exec *rlx_mi355x_compile(const rlx_graph_desc *graph, const rlx_compile_opts *opts);
+void rlx_exec_destroy(rlx_exec *e);
+
+/* ExecutableGraph::set_param(name, &[f32]). */
+int rlx_exec_set_param(rlx_exec *e, const char *name, const float *data, size_t n);
+/* ExecutableGraph::set_param_typed(name, &[u8], dtype). U8/I8 = raw GGUF bytes for a DequantMatMul weight: this is
+ * where the one-time repack into the device layout happens. F16/BF16 are widened to f32 as the reference does. */
+int rlx_exec_set_param_typed(rlx_exec *e, const char *name, const void *data, size_t nbytes, uint32_t dtype);
+
+typedef struct rlx_named_buf {
+    const char *name;
+    const void *data; /* host */
+    size_t nbytes;
+    uint32_t dtype;   /* rlx_dtype of `data` */
+} rlx_named_buf;
+
+typedef struct rlx_out_buf {
+    void *data;       /* host, caller-owned */
+    size_t capacity;  /* bytes available */
+    size_t nbytes;    /* bytes written (set by the call) */
+    uint32_t dtype;   /* dtype written (the output node's declared dtype) */
+} rlx_out_buf;
+
+/* ExecutableGraph::run(&[(name, &[f32])]) -> Vec<Vec<f32>>: host f32 in, host f32 out (synchronous). */
+int rlx_exec_run(rlx_exec *e, const rlx_named_buf *inputs, size_t n_inputs, rlx_out_buf *outputs, size_t n_outputs);
+/* ExecutableGraph::run_typed: inputs in F32/F16/BF16 bytes. 16-bit inputs stay 16-bit on the device. */
+int rlx_exec_run_typed(rlx_exec *e, const rlx_named_buf *inputs, size_t n_inputs, rlx_out_buf *outputs,
+                       size_t n_outputs);
+
+/* run_slots / arena_ptr analogue (rlx-runtime/src/backend.rs:169-178): device-resident execution.
+ * rlx_exec_slot gives the device address and byte size of an Input/Param/output node's buffer;
+ * rlx_exec_launch enqueues the whole schedule on the executable's stream without any host copy;
+ * rlx_exec_sync waits for it (sync_pending). */
+int rlx_exec_slot(rlx_exec *e, const char *name, void **dptr, size_t *nbytes);
+int rlx_exec_output_slot(rlx_exec *e, uint32_t output_index, void **dptr, size_t *nbytes);
+int rlx_exec_write_input(rlx_exec *e, const char *name, const void *data, size_t nbytes, uint32_t dtype);
+int rlx_exec_launch(rlx_exec *e);
+int rlx_exec_sync(rlx_exec *e);
+void *rlx_exec_stream(rlx_exec *e);
+
+/* MemoryPlan{arena_size, assignments} (rlx-compile/src/memory.rs:76-94) as planned for this executable,
+ * including the persistent repacked-weight slots. Writes a short text table. */
+size_t rlx_exec_arena_bytes(const rlx_exec *e);
+int rlx_exec_describe_plan(const rlx_exec *e, char *buf, size_t cap);
+/* FakeQuantize node's integer codes from the last run (int8, len elements), by output index; for parity checks. */
+int rlx_exec_read_fq_codes(rlx_exec *e, uint32_t node_id, int8_t *codes, size_t n);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RLX_MI355X_H */

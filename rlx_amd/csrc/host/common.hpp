@@ -1,0 +1,62 @@
+// Host-side plumbing shared by every translation unit of librlx_mi355x.so: error text, HIP call checking,
+// the embedded gfx950 code object and the kernel launcher (hipModuleLoadData / hipModuleLaunchKernel only;
+// no hipBLAS, MIOpen or runtime compilation anywhere).
+#pragma once
+#include <hip/hip_runtime_api.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <string>
+
+#include "../../../include/rlx_mi355x.h"
+#include "../layout.h"
+
+namespace rlx {
+
+void set_error(const char *fmt, ...) __attribute__((format(printf, 1, 2)));
+void clear_error();
+
+// Evaluates a HIP call; on failure records "<call>: <hipGetErrorString>" and returns RLX_ERR_HIP from the caller.
+#define RLX_HIP(call)                                                                               \
+    do {                                                                                            \
+        hipError_t e_ = (call);                                                                     \
+        if (e_ != hipSuccess) {                                                                     \
+            ::rlx::set_error("%s failed: %s (%d) at %s:%d", #call, hipGetErrorString(e_), (int)e_, \
+                             __FILE__, __LINE__);                                                   \
+            return RLX_ERR_HIP;                                                                     \
+        }                                                                                           \
+    } while (0)
+
+#define RLX_TRY(expr)             \
+    do {                          \
+        int rc_ = (expr);         \
+        if (rc_ < 0) return rc_;  \
+    } while (0)
+
+enum KernelId : int {
+    K_DEQUANT_Q4_0, K_DEQUANT_Q8_0, K_DEQUANT_Q4_K,
+    K_FQ_COL_ABSMAX, K_FQ_SEG_ABSMAX, K_FQ_FLAT_ABSMAX, K_FQ_SCALE, K_FQ_COL_APPLY, K_FQ_FLAT_APPLY, K_FQ_FLAT4_APPLY,
+    K_FILL_U32,
+    K_GEMV_Q4_0_T1_R2, K_GEMV_Q4_0_T2_R2, K_GEMV_Q4_0_T1_R4, K_GEMV_Q4_0_T2_R4, K_GEMV_Q4_0_T4_R4,
+    K_GEMV_Q8_0_T1_R2, K_GEMV_Q8_0_T1_R4, K_GEMV_Q8_0_T2_R4,
+    K_GEMV_Q4_K_T1_R2, K_GEMV_Q4_K_T1_R4, K_GEMV_Q4_K_T2_R4,
+    K_COUNT
+};
+
+// Loads the embedded code object on first use (device 0). RLX_OK or an error code with text.
+int runtime_init();
+// Launches kernel `id`; `args` points at the kernel's single by-value argument struct (or packed scalars).
+int launch(KernelId id, unsigned gx, unsigned gy, unsigned bx, unsigned shmem, hipStream_t stream, void **params);
+
+struct DeviceProps {
+    int cu_count;
+    int clock_khz;
+    int mem_clock_khz;
+    size_t lds_per_block;
+    char arch[64];
+    char name[128];
+};
+const DeviceProps &device_props();
+
+}  // namespace rlx

@@ -1,0 +1,553 @@
+// Graph level: the Backend / ExecutableGraph mirror (rlx-runtime/src/backend.rs:146-426).
+//
+// compile() does what the reference's CPU thunk compiler does for the two ops this backend claims
+// (rlx-cpu/src/thunk.rs:3027-3043 for DequantMatMul, 2567-2598 for FakeQuantize), plans one device arena in the
+// shape of rlx-compile's MemoryPlan (slots of {offset, size}; params and inputs live for the whole run,
+// rlx-compile/src/memory.rs:76-94,203-219) and extends it the way a quantized GPU backend needs: a packed U8
+// param owns a slot sized for the *device layout* of its weights, filled once by set_param_typed.
+#include <algorithm>
+#include <cstring>
+#include <map>
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "common.hpp"
+
+struct rlx_qweight;
+extern "C" int rlx_mi355x_qweight_create_at(int, const void *, size_t, int64_t, int64_t, void *, rlx_qweight **);
+extern "C" void rlx_mi355x_qweight_destroy(rlx_qweight *);
+
+namespace {
+
+using namespace rlx;
+
+const uint32_t kSupportedOps[] = {RLX_OP_INPUT, RLX_OP_PARAM, RLX_OP_DEQUANT_MATMUL, RLX_OP_FAKE_QUANTIZE};
+const char *op_name(uint32_t k) {
+    switch (k) {
+    case RLX_OP_INPUT: return "Input";
+    case RLX_OP_PARAM: return "Param";
+    case RLX_OP_DEQUANT_MATMUL: return "DequantMatMul";
+    case RLX_OP_FAKE_QUANTIZE: return "FakeQuantize";
+    default: return "?";
+    }
+}
+
+size_t dtype_size(uint32_t dt) {
+    switch (dt) {
+    case RLX_BOOL: case RLX_I8: case RLX_U8: return 1;
+    case RLX_F16: case RLX_BF16: case RLX_I16: return 2;
+    case RLX_F32: case RLX_I32: case RLX_U32: return 4;
+    case RLX_F64: case RLX_I64: case RLX_C64: return 8;
+    default: return 0;
+    }
+}
+
+struct Slot {
+    size_t offset = 0, size = 0;
+};
+
+struct Node {
+    rlx_node_desc d;
+    std::string name;
+    int64_t numel = 0;
+    Slot slot;          // the node's value
+    Slot aux;           // FakeQuantize: maxima + scales; DequantMatMul: workspace
+    Slot codes;         // FakeQuantize: int8 codes
+    uint32_t cur_dtype = RLX_F32;  // dtype of the bytes currently in an Input slot
+    // DequantMatMul
+    int64_t m = 0, k = 0, n = 0;
+    // FakeQuantize
+    int64_t chan_dim = 1, inner = 1;
+    // packed weight param
+    bool is_packed = false;
+    int scheme = 0;
+    int64_t w_n = 0, w_k = 0;
+    rlx_qweight *qw = nullptr;
+};
+
+// f32 <-> half / bfloat16 as the reference's typed boundary does (rlx-driver/src/arena.rs:69-119, `half` crate).
+float f16_to_f32(uint16_t h) {
+    uint32_t sign = (uint32_t)(h & 0x8000u) << 16, exp = (h >> 10) & 0x1Fu, man = h & 0x3FFu, bits;
+    if (exp == 0) {
+        if (!man) bits = sign;
+        else {
+            int e = -1;
+            do { man <<= 1; e++; } while (!(man & 0x400u));
+            bits = sign | ((uint32_t)(112 - e) << 23) | ((man & 0x3FFu) << 13);
+        }
+    } else if (exp == 31) bits = sign | 0x7F800000u | (man << 13);
+    else bits = sign | ((exp + 112) << 23) | (man << 13);
+    float f;
+    memcpy(&f, &bits, 4);
+    return f;
+}
+float bf16_to_f32(uint16_t h) {
+    uint32_t bits = (uint32_t)h << 16;
+    float f;
+    memcpy(&f, &bits, 4);
+    return f;
+}
+
+}  // namespace
+
+struct rlx_exec {
+    std::string name;
+    std::vector<Node> nodes;
+    std::vector<uint32_t> outputs;
+    std::map<std::string, uint32_t> inputs, params;
+    rlx_compile_opts opts{};
+    size_t arena_bytes = 0;
+    uint8_t *arena = nullptr;
+    hipStream_t stream = nullptr;
+
+    ~rlx_exec() {
+        for (auto &nd : nodes)
+            if (nd.qw) rlx_mi355x_qweight_destroy(nd.qw);
+        if (arena) (void)hipFree(arena);
+        if (stream) (void)hipStreamDestroy(stream);
+    }
+    void *ptr(const Slot &s) const { return arena + s.offset; }
+};
+
+extern "C" {
+
+size_t rlx_mi355x_supported_ops(const uint32_t **kinds) {
+    if (kinds) *kinds = kSupportedOps;
+    return sizeof kSupportedOps / sizeof kSupportedOps[0];
+}
+
+rlx_exec *rlx_mi355x_compile(const rlx_graph_desc *g, const rlx_compile_opts *opts) {
+    clear_error();
+    if (!g || !g->nodes || g->n_nodes == 0 || !g->outputs || g->n_outputs == 0) {
+        set_error("compile: empty graph or no outputs");
+        return nullptr;
+    }
+    auto e = std::unique_ptr<rlx_exec>(new rlx_exec);
+    e->name = g->name ? g->name : "";
+    if (opts) e->opts = *opts;
+    size_t align = e->opts.arena_alignment ? e->opts.arena_alignment : 256;
+    if (align & (align - 1)) {
+        set_error("compile: arena_alignment %zu is not a power of two", align);
+        return nullptr;
+    }
+    align = std::max<size_t>(align, 256);
+
+    // Legalize: every op kind must be claimed (rlx-compile/src/legalize.rs:61-76 message shape).
+    std::string bad;
+    int n_bad = 0;
+    for (uint32_t i = 0; i < g->n_nodes; i++) {
+        uint32_t k = g->nodes[i].op_kind;
+        if (k > RLX_OP_FAKE_QUANTIZE) {
+            n_bad++;
+            bad += "\n  - node " + std::to_string(i) + ": op kind " + std::to_string(k);
+        }
+    }
+    if (n_bad) {
+        set_error("rlx-opt: backend \"MI355X\" doesn't claim support for %d op kind(s):%s", n_bad, bad.c_str());
+        return nullptr;
+    }
+
+    e->nodes.resize(g->n_nodes);
+    for (uint32_t i = 0; i < g->n_nodes; i++) {
+        Node &nd = e->nodes[i];
+        nd.d = g->nodes[i];
+        nd.name = nd.d.name ? nd.d.name : "";
+        nd.d.name = nullptr;
+        if (nd.d.rank > RLX_MAX_RANK || nd.d.n_inputs > RLX_MAX_INPUTS) {
+            set_error("compile: node %u has rank %u / %u inputs (max %d / %d)", i, nd.d.rank, nd.d.n_inputs, RLX_MAX_RANK,
+                      RLX_MAX_INPUTS);
+            return nullptr;
+        }
+        nd.numel = 1;
+        for (uint32_t r = 0; r < nd.d.rank; r++) {
+            if (nd.d.dims[r] < 0) {
+                set_error("compile: node %u has a negative / symbolic dim", i);
+                return nullptr;
+            }
+            nd.numel *= nd.d.dims[r];
+        }
+        for (uint32_t j = 0; j < nd.d.n_inputs; j++)
+            if (nd.d.inputs[j] >= i) {
+                set_error("compile: node %u reads node %u, which is not earlier in the schedule", i, nd.d.inputs[j]);
+                return nullptr;
+            }
+        if (dtype_size(nd.d.dtype) == 0) {
+            set_error("compile: node %u has unknown dtype %u", i, nd.d.dtype);
+            return nullptr;
+        }
+    }
+    for (uint32_t i = 0; i < g->n_outputs; i++) {
+        if (g->outputs[i] >= g->n_nodes) {
+            set_error("compile: output %u names node %u of %u", i, g->outputs[i], g->n_nodes);
+            return nullptr;
+        }
+        e->outputs.push_back(g->outputs[i]);
+    }
+
+    // Per-op lowering.
+    for (uint32_t i = 0; i < g->n_nodes; i++) {
+        Node &nd = e->nodes[i];
+        switch (nd.d.op_kind) {
+        case RLX_OP_INPUT:
+            if (nd.d.dtype != RLX_F32 && nd.d.dtype != RLX_F16 && nd.d.dtype != RLX_BF16) {
+                set_error("compile: input '%s' has dtype %u; only F32/F16/BF16 cross the host boundary", nd.name.c_str(),
+                          nd.d.dtype);
+                return nullptr;
+            }
+            e->inputs[nd.name] = i;
+            break;
+        case RLX_OP_PARAM:
+            e->params[nd.name] = i;
+            break;
+        case RLX_OP_DEQUANT_MATMUL: {
+            if (layout_of((int)nd.d.scheme).unit_k == 0) {
+                set_error("compile: node %u: DequantMatMul scheme %u is not claimed (GGUF Q4_K=5, Q4_0=11, Q8_0=12)", i,
+                          nd.d.scheme);
+                return nullptr;
+            }
+            if (nd.d.n_inputs != 2 || nd.d.rank == 0 || nd.d.dtype != RLX_F32) {
+                set_error("compile: node %u: GGUF DequantMatMul takes [x, packed_w] and yields an F32 tensor of rank >= 1", i);
+                return nullptr;
+            }
+            Node &x = e->nodes[nd.d.inputs[0]];
+            Node &w = e->nodes[nd.d.inputs[1]];
+            // n = last dim of the declared output, m = numel(out)/n, k = numel(x)/m (thunk.rs:3029-3033)
+            nd.n = nd.d.dims[nd.d.rank - 1];
+            nd.m = nd.numel / std::max<int64_t>(nd.n, 1);
+            nd.k = x.numel / std::max<int64_t>(nd.m, 1);
+            if (nd.n <= 0 || nd.m <= 0 || nd.k <= 0 || nd.m * nd.k != x.numel) {
+                set_error("compile: node %u: cannot derive (m,k,n) from out numel %lld, x numel %lld", i,
+                          (long long)nd.numel, (long long)x.numel);
+                return nullptr;
+            }
+            Layout L = layout_of((int)nd.d.scheme);
+            int64_t want = (nd.k * nd.n) % L.block_elems == 0 ? nd.k * nd.n / L.block_elems * L.block_bytes : -1;
+            if (w.d.op_kind != RLX_OP_PARAM || (w.d.dtype != RLX_U8 && w.d.dtype != RLX_I8) || w.numel != want ||
+                nd.k % L.block_elems != 0) {
+                set_error("compile: node %u: packed weight must be a U8 param of %lld bytes ([n=%lld, k=%lld], k %% %d == 0); "
+                          "got %lld elements of dtype %u",
+                          i, (long long)want, (long long)nd.n, (long long)nd.k, L.block_elems, (long long)w.numel, w.d.dtype);
+                return nullptr;
+            }
+            if (w.is_packed && (w.scheme != (int)nd.d.scheme || w.w_n != nd.n || w.w_k != nd.k)) {
+                set_error("compile: packed param '%s' is used with two different (scheme, n, k)", w.name.c_str());
+                return nullptr;
+            }
+            if (x.d.dtype != RLX_F32 && x.d.dtype != RLX_F16 && x.d.dtype != RLX_BF16) {
+                set_error("compile: node %u: activation dtype %u unsupported", i, x.d.dtype);
+                return nullptr;
+            }
+            w.is_packed = true;
+            w.scheme = (int)nd.d.scheme;
+            w.w_n = nd.n;
+            w.w_k = nd.k;
+            break;
+        }
+        case RLX_OP_FAKE_QUANTIZE: {
+            if (nd.d.bits != 8 && nd.d.bits != 4 && nd.d.bits != 2) {
+                set_error("FakeQuantize: unsupported bits %u", nd.d.bits);
+                return nullptr;
+            }
+            bool stateful = nd.d.scale_mode == RLX_SCALE_EMA || nd.d.scale_mode == RLX_SCALE_FIXED;
+            if (nd.d.scale_mode > RLX_SCALE_FIXED || nd.d.n_inputs != (stateful ? 2u : 1u) || nd.d.dtype != RLX_F32) {
+                set_error("compile: node %u: FakeQuantize takes 1 input (PerBatch) or [x, state] (EMA/Fixed), F32", i);
+                return nullptr;
+            }
+            Node &x = e->nodes[nd.d.inputs[0]];
+            if (x.numel != nd.numel || x.d.dtype != RLX_F32) {
+                set_error("compile: node %u: FakeQuantize input must be F32 with the output's element count", i);
+                return nullptr;
+            }
+            // quant_layout (thunk.rs:14163-14175)
+            if (nd.d.axis < 0) {
+                nd.chan_dim = 1;
+                nd.inner = std::max<int64_t>(nd.numel, 1);
+            } else {
+                if ((uint32_t)nd.d.axis >= nd.d.rank) {
+                    set_error("compile: node %u: FakeQuantize axis %d out of range for rank %u", i, nd.d.axis, nd.d.rank);
+                    return nullptr;
+                }
+                nd.chan_dim = nd.d.dims[nd.d.axis];
+                nd.inner = 1;
+                for (uint32_t r = nd.d.axis + 1; r < nd.d.rank; r++) nd.inner *= nd.d.dims[r];
+                nd.inner = std::max<int64_t>(nd.inner, 1);
+            }
+            if (stateful) {
+                Node &st = e->nodes[nd.d.inputs[1]];
+                if (st.numel != nd.chan_dim || st.d.dtype != RLX_F32) {
+                    set_error("compile: node %u: FakeQuantize state must be F32 [%lld]", i, (long long)nd.chan_dim);
+                    return nullptr;
+                }
+            }
+            break;
+        }
+        }
+    }
+
+    // Memory plan.
+    size_t off = 0;
+    auto take = [&](size_t bytes) {
+        Slot s;
+        s.offset = off;
+        s.size = bytes;
+        off = (off + std::max<size_t>(bytes, 1) + align - 1) & ~(align - 1);
+        return s;
+    };
+    for (Node &nd : e->nodes) {
+        if (nd.is_packed) {
+            nd.slot = take((size_t)weight_dims(nd.scheme, nd.w_n, nd.w_k).bytes);  // device layout, resident
+        } else if (nd.d.op_kind == RLX_OP_INPUT) {
+            nd.slot = take((size_t)nd.numel * 4);  // room for an f32 upload even when declared 16-bit
+            nd.cur_dtype = nd.d.dtype;
+        } else {
+            nd.slot = take((size_t)nd.numel * dtype_size(nd.d.dtype));
+        }
+        if (nd.d.op_kind == RLX_OP_FAKE_QUANTIZE) {
+            nd.aux = take((size_t)nd.chan_dim * 8);
+            nd.codes = take((size_t)nd.numel);
+        }
+    }
+    e->arena_bytes = off;
+
+    if (runtime_init() != RLX_OK) return nullptr;
+    if (hipMalloc((void **)&e->arena, std::max<size_t>(off, 256)) != hipSuccess) {
+        set_error("compile: hipMalloc(%zu) for the arena failed", off);
+        return nullptr;
+    }
+    if (hipMemset(e->arena, 0, std::max<size_t>(off, 256)) != hipSuccess || hipStreamCreate(&e->stream) != hipSuccess) {
+        set_error("compile: arena clear / stream creation failed");
+        return nullptr;
+    }
+    if (e->opts.verbose) {
+        char buf[4096];
+        rlx_exec_describe_plan(e.get(), buf, sizeof buf);
+        fprintf(stderr, "%s", buf);
+    }
+    return e.release();
+}
+
+void rlx_exec_destroy(rlx_exec *e) { delete e; }
+
+int rlx_exec_set_param_typed(rlx_exec *e, const char *name, const void *data, size_t nbytes, uint32_t dtype) {
+    clear_error();
+    if (!e || !name || !data) {
+        set_error("set_param_typed: null argument");
+        return RLX_ERR_INVALID;
+    }
+    auto it = e->params.find(name);
+    if (it == e->params.end()) return RLX_WARN_UNKNOWN_NAME;
+    Node &nd = e->nodes[it->second];
+    if (dtype == RLX_U8 || dtype == RLX_I8) {
+        if (nd.is_packed) {
+            if (nd.qw) {
+                rlx_mi355x_qweight_destroy(nd.qw);
+                nd.qw = nullptr;
+            }
+            return rlx_mi355x_qweight_create_at(nd.scheme, data, nbytes, nd.w_n, nd.w_k, e->ptr(nd.slot), &nd.qw);
+        }
+        if (nbytes > nd.slot.size) {
+            set_error("set_param_typed: '%s' holds %zu bytes, got %zu", name, nd.slot.size, nbytes);
+            return RLX_ERR_INVALID;
+        }
+        RLX_HIP(hipMemcpy(e->ptr(nd.slot), data, nbytes, hipMemcpyHostToDevice));
+        return RLX_OK;
+    }
+    if (nd.is_packed) {
+        set_error("set_param_typed: '%s' is a packed GGUF weight; pass its bytes as U8", name);
+        return RLX_ERR_INVALID;
+    }
+    std::vector<float> wide;
+    const float *src = nullptr;
+    size_t n = 0;
+    if (dtype == RLX_F32) {
+        if (nbytes % 4) {
+            set_error("set_param_typed F32: data length %zu not a multiple of 4", nbytes);
+            return RLX_ERR_INVALID;
+        }
+        src = (const float *)data;
+        n = nbytes / 4;
+    } else if (dtype == RLX_F16 || dtype == RLX_BF16) {
+        n = nbytes / 2;
+        wide.resize(n);
+        const uint16_t *h = (const uint16_t *)data;
+        for (size_t i = 0; i < n; i++) wide[i] = dtype == RLX_F16 ? f16_to_f32(h[i]) : bf16_to_f32(h[i]);
+        src = wide.data();
+    } else {
+        set_error("set_param_typed: dtype %u unsupported (only F32/F16/BF16/U8/I8 are accepted on the host I/O surface)", dtype);
+        return RLX_ERR_UNSUPPORTED;
+    }
+    if (nd.d.dtype != RLX_F32 || n * 4 > nd.slot.size) {
+        set_error("set_param: '%s' is %lld elements of dtype %u; got %zu f32 values", name, (long long)nd.numel, nd.d.dtype, n);
+        return RLX_ERR_INVALID;
+    }
+    RLX_HIP(hipMemcpy(e->ptr(nd.slot), src, n * 4, hipMemcpyHostToDevice));
+    return RLX_OK;
+}
+
+int rlx_exec_set_param(rlx_exec *e, const char *name, const float *data, size_t n) {
+    return rlx_exec_set_param_typed(e, name, data, n * 4, RLX_F32);
+}
+
+int rlx_exec_write_input(rlx_exec *e, const char *name, const void *data, size_t nbytes, uint32_t dtype) {
+    if (!e || !name || !data) {
+        set_error("write_input: null argument");
+        return RLX_ERR_INVALID;
+    }
+    auto it = e->inputs.find(name);
+    if (it == e->inputs.end()) return RLX_WARN_UNKNOWN_NAME;
+    Node &nd = e->nodes[it->second];
+    size_t es = dtype == RLX_F32 ? 4 : (dtype == RLX_F16 || dtype == RLX_BF16) ? 2 : 0;
+    if (es == 0) {
+        set_error("run: input '%s' dtype %u unsupported (F32/F16/BF16 only)", name, dtype);
+        return RLX_ERR_UNSUPPORTED;
+    }
+    if (nbytes != (size_t)nd.numel * es) {
+        set_error("run: input '%s' needs %lld elements, got %zu bytes of dtype %u", name, (long long)nd.numel, nbytes, dtype);
+        return RLX_ERR_INVALID;
+    }
+    RLX_HIP(hipMemcpyAsync(e->ptr(nd.slot), data, nbytes, hipMemcpyHostToDevice, e->stream));
+    nd.cur_dtype = dtype;
+    return RLX_OK;
+}
+
+int rlx_exec_launch(rlx_exec *e) {
+    if (!e) {
+        set_error("launch: null executable");
+        return RLX_ERR_INVALID;
+    }
+    for (Node &nd : e->nodes) {
+        if (nd.d.op_kind == RLX_OP_DEQUANT_MATMUL) {
+            Node &x = e->nodes[nd.d.inputs[0]];
+            Node &w = e->nodes[nd.d.inputs[1]];
+            if (!w.qw) {
+                set_error("run: packed weight '%s' was never set (set_param_typed(.., U8))", w.name.c_str());
+                return RLX_ERR_INVALID;
+            }
+            uint32_t xdt = x.d.op_kind == RLX_OP_INPUT ? x.cur_dtype : x.d.dtype;
+            RLX_TRY(rlx_mi355x_gguf_matmul_bt(e->ptr(x.slot), (int)xdt, w.qw, (float *)e->ptr(nd.slot), nd.m, nullptr, 0,
+                                              e->stream));
+        } else if (nd.d.op_kind == RLX_OP_FAKE_QUANTIZE) {
+            Node &x = e->nodes[nd.d.inputs[0]];
+            if (x.d.op_kind == RLX_OP_INPUT && x.cur_dtype != RLX_F32) {
+                set_error("run: FakeQuantize input '%s' must be written as F32", x.name.c_str());
+                return RLX_ERR_INVALID;
+            }
+            float *state = nd.d.n_inputs == 2 ? (float *)e->ptr(e->nodes[nd.d.inputs[1]].slot) : nullptr;
+            RLX_TRY(rlx_mi355x_fake_quantize((const float *)e->ptr(x.slot), (float *)e->ptr(nd.slot),
+                                             (int8_t *)e->ptr(nd.codes), nd.numel, nd.chan_dim, nd.inner, (int)nd.d.bits,
+                                             (int)nd.d.scale_mode, nd.d.ema_decay, state, (int)e->opts.fq_round_mode,
+                                             e->ptr(nd.aux), e->stream));
+        }
+    }
+    return RLX_OK;
+}
+
+int rlx_exec_sync(rlx_exec *e) {
+    RLX_HIP(hipStreamSynchronize(e->stream));
+    return RLX_OK;
+}
+
+void *rlx_exec_stream(rlx_exec *e) { return e ? e->stream : nullptr; }
+
+static int run_common(rlx_exec *e, const rlx_named_buf *inputs, size_t n_inputs, rlx_out_buf *outputs, size_t n_outputs,
+                      bool typed) {
+    clear_error();
+    if (!e || (n_inputs && !inputs) || (n_outputs && !outputs)) {
+        set_error("run: null argument");
+        return RLX_ERR_INVALID;
+    }
+    int warn = RLX_OK;
+    for (size_t i = 0; i < n_inputs; i++) {
+        int rc = rlx_exec_write_input(e, inputs[i].name, inputs[i].data, inputs[i].nbytes, typed ? inputs[i].dtype : RLX_F32);
+        if (rc < 0) return rc;
+        if (rc > 0) warn = rc;
+    }
+    RLX_TRY(rlx_exec_launch(e));
+    if (n_outputs > e->outputs.size()) {
+        set_error("run: %zu output buffers for a graph with %zu outputs", n_outputs, e->outputs.size());
+        return RLX_ERR_INVALID;
+    }
+    for (size_t i = 0; i < n_outputs; i++) {
+        Node &nd = e->nodes[e->outputs[i]];
+        size_t bytes = (size_t)nd.numel * dtype_size(nd.d.dtype);
+        if (outputs[i].capacity < bytes || !outputs[i].data) {
+            set_error("run: output %zu needs %zu bytes, buffer has %zu", i, bytes, outputs[i].capacity);
+            return RLX_ERR_INVALID;
+        }
+        RLX_HIP(hipMemcpyAsync(outputs[i].data, e->ptr(nd.slot), bytes, hipMemcpyDeviceToHost, e->stream));
+        outputs[i].nbytes = bytes;
+        outputs[i].dtype = nd.d.dtype;
+    }
+    RLX_HIP(hipStreamSynchronize(e->stream));
+    return warn;
+}
+
+int rlx_exec_run(rlx_exec *e, const rlx_named_buf *inputs, size_t n_inputs, rlx_out_buf *outputs, size_t n_outputs) {
+    return run_common(e, inputs, n_inputs, outputs, n_outputs, false);
+}
+int rlx_exec_run_typed(rlx_exec *e, const rlx_named_buf *inputs, size_t n_inputs, rlx_out_buf *outputs, size_t n_outputs) {
+    return run_common(e, inputs, n_inputs, outputs, n_outputs, true);
+}
+
+int rlx_exec_slot(rlx_exec *e, const char *name, void **dptr, size_t *nbytes) {
+    if (!e || !name) return RLX_ERR_INVALID;
+    auto it = e->inputs.find(name);
+    if (it == e->inputs.end()) {
+        it = e->params.find(name);
+        if (it == e->params.end()) return RLX_WARN_UNKNOWN_NAME;
+    }
+    Node &nd = e->nodes[it->second];
+    if (dptr) *dptr = e->ptr(nd.slot);
+    if (nbytes) *nbytes = nd.slot.size;
+    return RLX_OK;
+}
+
+int rlx_exec_output_slot(rlx_exec *e, uint32_t idx, void **dptr, size_t *nbytes) {
+    if (!e || idx >= e->outputs.size()) {
+        set_error("output_slot: index %u out of range", idx);
+        return RLX_ERR_INVALID;
+    }
+    Node &nd = e->nodes[e->outputs[idx]];
+    if (dptr) *dptr = e->ptr(nd.slot);
+    if (nbytes) *nbytes = nd.slot.size;
+    return RLX_OK;
+}
+
+size_t rlx_exec_arena_bytes(const rlx_exec *e) { return e ? e->arena_bytes : 0; }
+
+int rlx_exec_describe_plan(const rlx_exec *e, char *buf, size_t cap) {
+    if (!e || !buf || cap == 0) return RLX_ERR_INVALID;
+    size_t pos = 0;
+    auto put = [&](const char *fmt, auto... a) {
+        if (pos < cap) pos += (size_t)snprintf(buf + pos, cap - pos, fmt, a...);
+    };
+    put("graph '%s': arena %zu bytes\n", e->name.c_str(), e->arena_bytes);
+    for (size_t i = 0; i < e->nodes.size(); i++) {
+        const Node &nd = e->nodes[i];
+        put("  node %zu %-13s %-12s off=%zu size=%zu", i, op_name(nd.d.op_kind), nd.name.c_str(), nd.slot.offset, nd.slot.size);
+        if (nd.is_packed) put(" [device layout, scheme %d, n=%lld k=%lld]", nd.scheme, (long long)nd.w_n, (long long)nd.w_k);
+        if (nd.d.op_kind == RLX_OP_DEQUANT_MATMUL) put(" m=%lld k=%lld n=%lld", (long long)nd.m, (long long)nd.k, (long long)nd.n);
+        if (nd.d.op_kind == RLX_OP_FAKE_QUANTIZE)
+            put(" chan_dim=%lld inner=%lld aux@%zu codes@%zu", (long long)nd.chan_dim, (long long)nd.inner, nd.aux.offset, nd.codes.offset);
+        put("\n");
+    }
+    return RLX_OK;
+}
+
+int rlx_exec_read_fq_codes(rlx_exec *e, uint32_t node_id, int8_t *codes, size_t n) {
+    if (!e || node_id >= e->nodes.size() || e->nodes[node_id].d.op_kind != RLX_OP_FAKE_QUANTIZE || !codes) {
+        set_error("read_fq_codes: node %u is not a FakeQuantize node", node_id);
+        return RLX_ERR_INVALID;
+    }
+    Node &nd = e->nodes[node_id];
+    if (n != (size_t)nd.numel) {
+        set_error("read_fq_codes: node has %lld elements, buffer %zu", (long long)nd.numel, n);
+        return RLX_ERR_INVALID;
+    }
+    RLX_HIP(hipStreamSynchronize(e->stream));
+    RLX_HIP(hipMemcpy(codes, e->ptr(nd.codes), n, hipMemcpyDeviceToHost));
+    return RLX_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,243 @@
+// Operator-level entry points: packed weights in HBM, dequant, matmul dispatch, FakeQuantize.
+#include <algorithm>
+#include <cstring>
+#include <vector>
+
+#include "common.hpp"
+
+namespace rlx {
+int repack_host(int scheme, const uint8_t *src, size_t nbytes, int64_t n, int64_t k, uint8_t *out);
+}
+
+struct rlx_qweight {
+    int scheme;
+    rlx::WeightDims dims;
+    uint8_t *dev;
+    bool owns;
+};
+
+namespace rlx {
+
+// Kernel argument blocks: must match the structs in kernels/*.hip field for field.
+struct DequantArgs {
+    const uint8_t *w;
+    float *out;
+    long long n, k, units;
+};
+struct GemvArgs {
+    const uint8_t *w;
+    const void *x;
+    float *out;
+    int m, k, n, units, row_tiles, kc_units, x_dtype;
+};
+struct FqArgs {
+    const float *x;
+    float *out;
+    int8_t *codes;
+    uint32_t *max_bits;
+    float *scale;
+    float *state;
+    long long len, chan_dim, inner;
+    float q_max, decay;
+    int scale_mode, round_mode, rows_per_block;
+};
+
+static int x_kind(int x_dtype) {
+    switch (x_dtype) {
+    case RLX_F32: return 0;
+    case RLX_BF16: return 1;
+    case RLX_F16: return 2;
+    default: return -1;
+    }
+}
+
+static int launch_gemv(const void *x, int xk, const rlx_qweight *w, float *out, int m, hipStream_t stream) {
+    const Layout L = layout_of(w->scheme);
+    const int rv = xk == 0 ? 2 * m : m;
+    const int units = (int)w->dims.units, tiles = (int)w->dims.row_tiles;
+    const bool r2 = rv <= 2;
+    // Row tiles per workgroup: one, unless N is large enough that two or four still leave >= 512 workgroups.
+    const int max_rtw = w->scheme == SCHEME_Q4_0 ? (r2 ? 2 : 4) : (r2 ? 1 : 2);
+    int rtw = 1;
+    while (rtw * 2 <= max_rtw && tiles / (rtw * 2) >= 512) rtw *= 2;
+    KernelId id;
+    if (w->scheme == SCHEME_Q4_0)
+        id = r2 ? (rtw == 2 ? K_GEMV_Q4_0_T2_R2 : K_GEMV_Q4_0_T1_R2)
+                : (rtw == 4 ? K_GEMV_Q4_0_T4_R4 : rtw == 2 ? K_GEMV_Q4_0_T2_R4 : K_GEMV_Q4_0_T1_R4);
+    else if (w->scheme == SCHEME_Q8_0)
+        id = r2 ? K_GEMV_Q8_0_T1_R2 : (rtw == 2 ? K_GEMV_Q8_0_T2_R4 : K_GEMV_Q8_0_T1_R4);
+    else
+        id = r2 ? K_GEMV_Q4_K_T1_R2 : (rtw == 2 ? K_GEMV_Q4_K_T2_R4 : K_GEMV_Q4_K_T1_R4);
+
+    // LDS: the staged activation chunk (rv rows of halfs, 16 B row padding) plus, for Q4_K, the per-block sums.
+    const size_t budget = 48 * 1024;
+    auto stage_bytes = [&](int kcu) {
+        size_t b = ((size_t)rv * ((size_t)kcu * L.unit_k + 8) * 2 + 15) & ~(size_t)15;
+        if (w->scheme == SCHEME_Q4K) b += (size_t)kcu * (L.unit_k / 32) * 16 * 4;
+        return b;
+    };
+    int kcu = units;
+    while (kcu > 1 && stage_bytes(kcu) > budget) kcu--;
+    if (stage_bytes(kcu) > budget) {
+        set_error("gemv: one K unit of %d activation rows does not fit LDS", rv);
+        return RLX_ERR_INVALID;
+    }
+    int nwaves = std::min(16, std::max(1, kcu));
+    size_t red_bytes = (size_t)nwaves * rtw * 1024;
+    size_t shmem = std::max(stage_bytes(kcu), red_bytes);
+    GemvArgs a{w->dev, x, out, m, (int)w->dims.k, (int)w->dims.n, units, tiles, kcu, xk};
+    void *params[] = {&a};
+    return launch(id, (unsigned)((tiles + rtw - 1) / rtw), 1, (unsigned)nwaves * 64, (unsigned)shmem, stream, params);
+}
+
+}  // namespace rlx
+
+extern "C" {
+
+int rlx_mi355x_qweight_create_at(int scheme, const void *gguf_bytes, size_t nbytes, int64_t n, int64_t k,
+                                 void *device_mem, rlx_qweight **out) {
+    using namespace rlx;
+    RLX_TRY(runtime_init());
+    WeightDims D = weight_dims(scheme, n, k);
+    std::vector<uint8_t> staging;
+    if (D.bytes == 0) {
+        set_error("qweight: scheme %d is not a claimed GGUF scheme", scheme);
+        return RLX_ERR_UNSUPPORTED;
+    }
+    staging.resize((size_t)D.bytes);
+    RLX_TRY(repack_host(scheme, (const uint8_t *)gguf_bytes, nbytes, n, k, staging.data()));
+    bool owns = device_mem == nullptr;
+    if (owns) RLX_HIP(hipMalloc(&device_mem, (size_t)D.bytes));
+    hipError_t e = hipMemcpy(device_mem, staging.data(), (size_t)D.bytes, hipMemcpyHostToDevice);
+    if (e != hipSuccess) {
+        if (owns) (void)hipFree(device_mem);
+        set_error("qweight upload: %s", hipGetErrorString(e));
+        return RLX_ERR_HIP;
+    }
+    *out = new rlx_qweight{scheme, D, (uint8_t *)device_mem, owns};
+    return RLX_OK;
+}
+
+int rlx_mi355x_qweight_create(int scheme, const void *gguf_bytes, size_t nbytes, int64_t n, int64_t k,
+                              rlx_qweight **out) {
+    return rlx_mi355x_qweight_create_at(scheme, gguf_bytes, nbytes, n, k, nullptr, out);
+}
+
+void rlx_mi355x_qweight_destroy(rlx_qweight *w) {
+    if (!w) return;
+    if (w->owns) (void)hipFree(w->dev);
+    delete w;
+}
+
+size_t rlx_mi355x_qweight_device_bytes(const rlx_qweight *w) { return w ? (size_t)w->dims.bytes : 0; }
+
+int rlx_mi355x_dequant(const rlx_qweight *w, float *out_dev, void *stream) {
+    using namespace rlx;
+    if (!w || !out_dev) {
+        set_error("dequant: null argument");
+        return RLX_ERR_INVALID;
+    }
+    DequantArgs a{w->dev, out_dev, w->dims.n, w->dims.k, w->dims.units};
+    void *params[] = {&a};
+    KernelId id = w->scheme == SCHEME_Q4_0 ? K_DEQUANT_Q4_0 : w->scheme == SCHEME_Q8_0 ? K_DEQUANT_Q8_0 : K_DEQUANT_Q4_K;
+    return launch(id, (unsigned)w->dims.units, (unsigned)w->dims.row_tiles, 64, 0, (hipStream_t)stream, params);
+}
+
+size_t rlx_mi355x_gguf_matmul_workspace(int scheme, int x_dtype, int64_t m, int64_t k, int64_t n) {
+    (void)scheme; (void)x_dtype; (void)m; (void)k; (void)n;
+    return 0;
+}
+
+int rlx_mi355x_gguf_matmul_bt(const void *x_dev, int x_dtype, const rlx_qweight *w, float *out_dev, int64_t m,
+                              void *workspace, size_t workspace_bytes, void *stream) {
+    using namespace rlx;
+    (void)workspace; (void)workspace_bytes;
+    if (!x_dev || !w || !out_dev || m <= 0) {
+        set_error("gguf_matmul_bt: null argument or m=%lld", (long long)m);
+        return RLX_ERR_INVALID;
+    }
+    int xk = x_kind(x_dtype);
+    if (xk < 0) {
+        set_error("gguf_matmul_bt: activation dtype %d unsupported (F32, BF16, F16 only)", x_dtype);
+        return RLX_ERR_UNSUPPORTED;
+    }
+    const int64_t cap = xk == 0 ? 8 : 16;  // activation rows one MFMA pass holds
+    const size_t xrow = (size_t)w->dims.k * (xk == 0 ? 4 : 2);
+    for (int64_t r0 = 0; r0 < m; r0 += cap) {
+        int rows = (int)std::min<int64_t>(cap, m - r0);
+        RLX_TRY(launch_gemv((const uint8_t *)x_dev + r0 * xrow, xk, w, out_dev + r0 * w->dims.n, rows,
+                            (hipStream_t)stream));
+    }
+    return RLX_OK;
+}
+
+int rlx_mi355x_fake_quantize(const float *x_dev, float *out_dev, int8_t *codes_dev, int64_t len, int64_t chan_dim,
+                             int64_t inner, int bits, int scale_mode, float ema_decay, float *state_dev,
+                             int round_mode, void *scratch_dev, void *stream) {
+    using namespace rlx;
+    float q_max;
+    switch (bits) {
+    case 8: q_max = 127.0f; break;
+    case 4: q_max = 7.0f; break;
+    case 2: q_max = 1.0f; break;
+    default:
+        set_error("FakeQuantize: unsupported bits %d", bits);  // the reference panics with this text (thunk.rs:11179)
+        return RLX_ERR_UNSUPPORTED;
+    }
+    if (chan_dim < 1) chan_dim = 1;
+    if (inner < 1) inner = 1;
+    if (!x_dev || !out_dev || !scratch_dev || len < 0 || scale_mode < 0 || scale_mode > 2) {
+        set_error("FakeQuantize: null buffer, negative length or bad scale mode %d", scale_mode);
+        return RLX_ERR_INVALID;
+    }
+    if (scale_mode != RLX_SCALE_PER_BATCH && !state_dev) {
+        set_error("FakeQuantize: EMA / Fixed scale modes need the state tensor");  // "EMA needs state_off"
+        return RLX_ERR_INVALID;
+    }
+    if (len == 0) return RLX_OK;
+    hipStream_t s = (hipStream_t)stream;
+    uint32_t *max_bits = (uint32_t *)scratch_dev;
+    float *scale = (float *)scratch_dev + chan_dim;
+    const bool col = inner == 1 && chan_dim >= 4 && chan_dim % 4 == 0 && len % chan_dim == 0 &&
+                     ((uintptr_t)x_dev % 16 == 0) && ((uintptr_t)out_dev % 16 == 0) &&
+                     (!codes_dev || (uintptr_t)codes_dev % 4 == 0);
+    FqArgs a{x_dev, out_dev, codes_dev, max_bits, scale, state_dev, len, chan_dim, inner, q_max, ema_decay,
+             scale_mode, round_mode, 0};
+    void *params[] = {&a};
+    unsigned gx_col = (unsigned)((chan_dim / 4 + 255) / 256), gy_col = 1;
+    if (col) {
+        int64_t rows = len / chan_dim;
+        int64_t want = std::max<int64_t>(1, 512 / gx_col);
+        int64_t rpb = std::max<int64_t>(16, (rows + want - 1) / want);
+        a.rows_per_block = (int)rpb;
+        gy_col = (unsigned)((rows + rpb - 1) / rpb);
+    }
+    if (scale_mode != RLX_SCALE_FIXED) {
+        RLX_TRY(rlx_mi355x_memset_u32(max_bits, 0, (size_t)chan_dim, stream));
+        if (col) {
+            RLX_TRY(launch(K_FQ_COL_ABSMAX, gx_col, gy_col, 256, 0, s, params));
+        } else if (inner >= 256 && len % inner == 0 && len / inner <= 0x7FFFFFFF) {
+            // one workgroup per contiguous run of `inner` elements, long runs split into parts of >= 16K elements
+            unsigned bx = inner >= 4096 ? 1024 : 256;
+            unsigned parts = (unsigned)std::min<int64_t>(1024, std::max<int64_t>(1, inner / 16384));
+            a.rows_per_block = (int)((inner + parts - 1) / parts);
+            RLX_TRY(launch(K_FQ_SEG_ABSMAX, (unsigned)(len / inner), parts, bx, 0, s, params));
+        } else {
+            int64_t threads = (len + 31) / 32;
+            RLX_TRY(launch(K_FQ_FLAT_ABSMAX, (unsigned)((threads + 255) / 256), 1, 256, 0, s, params));
+        }
+    }
+    RLX_TRY(launch(K_FQ_SCALE, (unsigned)((chan_dim + 255) / 256), 1, 256, 0, s, params));
+    if (col) {
+        RLX_TRY(launch(K_FQ_COL_APPLY, gx_col, gy_col, 256, 0, s, params));
+    } else {
+        bool v4 = inner % 4 == 0 && len % 4 == 0 && ((uintptr_t)x_dev % 16 == 0) && ((uintptr_t)out_dev % 16 == 0) &&
+                  (!codes_dev || (uintptr_t)codes_dev % 4 == 0);
+        int64_t work = v4 ? len / 4 : len;
+        unsigned blocks = (unsigned)std::min<int64_t>((work + 255) / 256, 256 * 16);
+        RLX_TRY(launch(v4 ? K_FQ_FLAT4_APPLY : K_FQ_FLAT_APPLY, blocks, 1, 256, 0, s, params));
+    }
+    return RLX_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,177 @@
+#include "common.hpp"
+
+#include <cstring>
+#include <mutex>
+
+extern "C" const unsigned char rlx_kernels_blob[];
+extern "C" const unsigned char rlx_kernels_blob_end[];
+
+namespace rlx {
+
+static thread_local std::string g_error;
+
+void set_error(const char *fmt, ...) {
+    char buf[1024];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    g_error = buf;
+}
+void clear_error() { g_error.clear(); }
+const char *last_error_cstr() { return g_error.c_str(); }
+
+static const char *const kKernelNames[K_COUNT] = {
+    "rlx_dequant_q4_0", "rlx_dequant_q8_0", "rlx_dequant_q4_k",
+    "rlx_fq_col_absmax", "rlx_fq_seg_absmax", "rlx_fq_flat_absmax", "rlx_fq_scale", "rlx_fq_col_apply",
+    "rlx_fq_flat_apply", "rlx_fq_flat4_apply",
+    "rlx_fill_u32",
+    "rlx_gemv_q4_0_t1_r2", "rlx_gemv_q4_0_t2_r2", "rlx_gemv_q4_0_t1_r4", "rlx_gemv_q4_0_t2_r4", "rlx_gemv_q4_0_t4_r4",
+    "rlx_gemv_q8_0_t1_r2", "rlx_gemv_q8_0_t1_r4", "rlx_gemv_q8_0_t2_r4",
+    "rlx_gemv_q4_k_t1_r2", "rlx_gemv_q4_k_t1_r4", "rlx_gemv_q4_k_t2_r4",
+};
+
+static std::once_flag g_once;
+static int g_init_rc = RLX_ERR_NO_DEVICE;
+static std::string g_init_error;
+static hipModule_t g_module;
+static hipFunction_t g_fn[K_COUNT];
+static DeviceProps g_props;
+
+static int do_init() {
+    int count = 0;
+    hipError_t e = hipGetDeviceCount(&count);
+    if (e != hipSuccess || count <= 0) {
+        set_error("no HIP device (hipGetDeviceCount: %s, count=%d)", hipGetErrorString(e), count);
+        return RLX_ERR_NO_DEVICE;
+    }
+    RLX_HIP(hipSetDevice(0));
+    hipDeviceProp_t p;
+    RLX_HIP(hipGetDeviceProperties(&p, 0));
+    if (strncmp(p.gcnArchName, "gfx950", 6) != 0) {
+        set_error("device 0 is %s (%s); this library carries gfx950 code only", p.name, p.gcnArchName);
+        return RLX_ERR_NO_DEVICE;
+    }
+    g_props.cu_count = p.multiProcessorCount;
+    g_props.clock_khz = p.clockRate;
+    g_props.mem_clock_khz = p.memoryClockRate;
+    g_props.lds_per_block = p.sharedMemPerBlock;
+    snprintf(g_props.arch, sizeof g_props.arch, "%s", p.gcnArchName);
+    snprintf(g_props.name, sizeof g_props.name, "%s", p.name);
+    RLX_HIP(hipModuleLoadData(&g_module, rlx_kernels_blob));
+    for (int i = 0; i < K_COUNT; i++) {
+        hipError_t fe = hipModuleGetFunction(&g_fn[i], g_module, kKernelNames[i]);
+        if (fe != hipSuccess) {
+            set_error("hipModuleGetFunction(%s): %s", kKernelNames[i], hipGetErrorString(fe));
+            return RLX_ERR_HIP;
+        }
+    }
+    return RLX_OK;
+}
+
+int runtime_init() {
+    std::call_once(g_once, [] {
+        g_init_rc = do_init();
+        if (g_init_rc != RLX_OK) g_init_error = last_error_cstr();
+    });
+    if (g_init_rc != RLX_OK) set_error("%s", g_init_error.c_str());
+    return g_init_rc;
+}
+
+const DeviceProps &device_props() { return g_props; }
+
+int launch(KernelId id, unsigned gx, unsigned gy, unsigned bx, unsigned shmem, hipStream_t stream, void **params) {
+    RLX_TRY(runtime_init());
+    if (gx == 0 || gy == 0 || bx == 0 || bx > 1024 || gy > 65535) {
+        set_error("launch(%s): bad geometry grid=(%u,%u) block=%u", kKernelNames[id], gx, gy, bx);
+        return RLX_ERR_INVALID;
+    }
+    hipError_t e = hipModuleLaunchKernel(g_fn[id], gx, gy, 1, bx, 1, 1, shmem, stream, params, nullptr);
+    if (e != hipSuccess) {
+        set_error("hipModuleLaunchKernel(%s, grid=(%u,%u), block=%u, lds=%u): %s", kKernelNames[id], gx, gy, bx, shmem,
+                  hipGetErrorString(e));
+        return RLX_ERR_HIP;
+    }
+    return RLX_OK;
+}
+
+}  // namespace rlx
+
+namespace rlx { const char *last_error_cstr(); }
+
+extern "C" {
+
+int rlx_mi355x_is_available(void) { return rlx::runtime_init() == RLX_OK ? 1 : 0; }
+const char *rlx_mi355x_device_name(void) { return "MI355X"; }
+int rlx_mi355x_abi_version(void) { return RLX_MI355X_ABI_VERSION; }
+const char *rlx_mi355x_last_error(void) { return rlx::last_error_cstr(); }
+
+int rlx_mi355x_device_info(char *buf, size_t cap) {
+    RLX_TRY(rlx::runtime_init());
+    const rlx::DeviceProps &p = rlx::device_props();
+    snprintf(buf, cap, "%s (%s), %d CUs, %.0f MHz core, %.0f MHz mem, %zu B LDS/block", p.name, p.arch, p.cu_count,
+             p.clock_khz / 1000.0, p.mem_clock_khz / 1000.0, p.lds_per_block);
+    return RLX_OK;
+}
+
+int rlx_mi355x_malloc(void **dptr, size_t nbytes) {
+    RLX_TRY(rlx::runtime_init());
+    RLX_HIP(hipMalloc(dptr, nbytes ? nbytes : 1));
+    return RLX_OK;
+}
+int rlx_mi355x_free(void *dptr) {
+    RLX_HIP(hipFree(dptr));
+    return RLX_OK;
+}
+int rlx_mi355x_memcpy_h2d(void *dst, const void *src, size_t nbytes) {
+    RLX_HIP(hipMemcpy(dst, src, nbytes, hipMemcpyHostToDevice));
+    return RLX_OK;
+}
+int rlx_mi355x_memcpy_d2h(void *dst, const void *src, size_t nbytes) {
+    RLX_HIP(hipMemcpy(dst, src, nbytes, hipMemcpyDeviceToHost));
+    return RLX_OK;
+}
+int rlx_mi355x_memset_u32(void *dst, uint32_t value, size_t n_words, void *stream) {
+    if (n_words == 0) return RLX_OK;
+    long long n = (long long)n_words;
+    unsigned blocks = (unsigned)((n + 255) / 256 > 4096 ? 4096 : (n + 255) / 256);
+    void *params[] = {&dst, &value, &n};
+    return rlx::launch(rlx::K_FILL_U32, blocks, 1, 256, 0, (hipStream_t)stream, params);
+}
+int rlx_mi355x_stream_create(void **stream) {
+    RLX_TRY(rlx::runtime_init());
+    hipStream_t s;
+    RLX_HIP(hipStreamCreate(&s));  // default priority
+    *stream = s;
+    return RLX_OK;
+}
+int rlx_mi355x_stream_destroy(void *stream) {
+    RLX_HIP(hipStreamDestroy((hipStream_t)stream));
+    return RLX_OK;
+}
+int rlx_mi355x_stream_sync(void *stream) {
+    RLX_HIP(hipStreamSynchronize((hipStream_t)stream));
+    return RLX_OK;
+}
+int rlx_mi355x_event_create(void **event) {
+    RLX_TRY(rlx::runtime_init());
+    hipEvent_t ev;
+    RLX_HIP(hipEventCreate(&ev));
+    *event = ev;
+    return RLX_OK;
+}
+int rlx_mi355x_event_destroy(void *event) {
+    RLX_HIP(hipEventDestroy((hipEvent_t)event));
+    return RLX_OK;
+}
+int rlx_mi355x_event_record(void *event, void *stream) {
+    RLX_HIP(hipEventRecord((hipEvent_t)event, (hipStream_t)stream));
+    return RLX_OK;
+}
+int rlx_mi355x_event_elapsed_ms(void *start, void *stop, float *ms) {
+    RLX_HIP(hipEventSynchronize((hipEvent_t)stop));
+    RLX_HIP(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop));
+    return RLX_OK;
+}
+
+}  // extern "C"

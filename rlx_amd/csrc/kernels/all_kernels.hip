@@ -1,0 +1,4 @@
+// Single translation unit for the gfx950 code object the host library embeds and loads with hipModuleLoadData.
+#include "dequant.hip"
+#include "fakequant.hip"
+#include "gemv.hip"

@@ -1,0 +1,109 @@
+// Device-side helpers shared by every kernel: vector types, granule -> packed-half unpackers, MFMA wrappers.
+// gfx950 only.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../layout.h"
+
+namespace rlx {
+
+typedef _Float16 half_t;
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t uint2_t __attribute__((ext_vector_type(2)));
+
+union Frag {  // one MFMA A/B operand: 8 halfs = 4 dwords
+    half8_t h8;
+    half2_t h2[4];
+    uint32_t u[4];
+    uint4_t u4;
+};
+
+__device__ __forceinline__ half2_t as_half2(uint32_t u) { return __builtin_bit_cast(half2_t, u); }
+__device__ __forceinline__ uint32_t as_u32(half2_t h) { return __builtin_bit_cast(uint32_t, h); }
+__device__ __forceinline__ float half_bits_to_float(uint32_t bits16) {
+    return (float)__builtin_bit_cast(half_t, (uint16_t)bits16);  // exact IEEE widening (v_cvt_f32_f16)
+}
+
+// 0x6400 is 1024.0 in binary16 and its ulp is 1, so (0x6400 | v) is the half 1024 + v for 0 <= v < 1024.
+constexpr uint32_t MAGIC = 0x64006400u;
+
+// 4-bit granule word -> four half2 registers holding (q - OFF) for the 8 weights, fragment order.
+// OFF = 8 for Q4_0 (signed codes), 0 for Q4_K. All results are exact integers.
+template <int OFF>
+__device__ __forceinline__ void unpack_q4(uint32_t w, Frag &f) {
+    const half2_t sub_lo = {(half_t)(-(1024 + OFF)), (half_t)(-(1024 + OFF))};
+    const half2_t mul_hi = {(half_t)0.0625f, (half_t)0.0625f};
+    const half2_t sub_hi = {(half_t)(-(64 + OFF)), (half_t)(-(64 + OFF))};
+    uint32_t w2 = w >> 8;
+    half2_t a0 = as_half2((w & 0x000F000Fu) | MAGIC);   // 1024 + q
+    half2_t a1 = as_half2((w & 0x00F000F0u) | MAGIC);   // 1024 + 16 q
+    half2_t a2 = as_half2((w2 & 0x000F000Fu) | MAGIC);
+    half2_t a3 = as_half2((w2 & 0x00F000F0u) | MAGIC);
+    f.h2[0] = a0 + sub_lo;
+    f.h2[1] = __builtin_elementwise_fma(a1, mul_hi, sub_hi);  // (1024+16q)/16 - 64 - OFF, single rounding of an exact value
+    f.h2[2] = a2 + sub_lo;
+    f.h2[3] = __builtin_elementwise_fma(a3, mul_hi, sub_hi);
+}
+
+// Q4_K granule word -> sc * q (exact integers <= 945) given sc as a half2 splat.
+__device__ __forceinline__ void unpack_q4_scaled(uint32_t w, half2_t sc, Frag &f) {
+    const half2_t k1024 = {(half_t)1024.0f, (half_t)1024.0f};
+    const half2_t k64 = {(half_t)64.0f, (half_t)64.0f};
+    const half2_t r16 = {(half_t)0.0625f, (half_t)0.0625f};
+    half2_t neg_lo = -(sc * k1024);  // exact: sc < 64
+    half2_t neg_hi = -(sc * k64);
+    half2_t sc16 = sc * r16;         // exact power-of-two scaling
+    uint32_t w2 = w >> 8;
+    half2_t a0 = as_half2((w & 0x000F000Fu) | MAGIC);
+    half2_t a1 = as_half2((w & 0x00F000F0u) | MAGIC);
+    half2_t a2 = as_half2((w2 & 0x000F000Fu) | MAGIC);
+    half2_t a3 = as_half2((w2 & 0x00F000F0u) | MAGIC);
+    f.h2[0] = __builtin_elementwise_fma(a0, sc, neg_lo);
+    f.h2[1] = __builtin_elementwise_fma(a1, sc16, neg_hi);
+    f.h2[2] = __builtin_elementwise_fma(a2, sc, neg_lo);
+    f.h2[3] = __builtin_elementwise_fma(a3, sc16, neg_hi);
+}
+
+// Q8_0 granule (two words of offset-binary bytes) -> signed codes as halfs, fragment order.
+__device__ __forceinline__ void unpack_q8(uint32_t w0, uint32_t w1, Frag &f) {
+    const half2_t sub = {(half_t)(-1152.0f), (half_t)(-1152.0f)};  // 1024 + 128
+    const uint32_t c64 = 0x64646464u;
+    // v_perm_b32: selector byte 0..3 picks from the second source, 4..7 from the first.
+    half2_t a0 = as_half2(__builtin_amdgcn_perm(c64, w0, 0x04010400u));  // bytes 0,1
+    half2_t a1 = as_half2(__builtin_amdgcn_perm(c64, w0, 0x04030402u));  // bytes 2,3
+    half2_t a2 = as_half2(__builtin_amdgcn_perm(c64, w1, 0x04010400u));
+    half2_t a3 = as_half2(__builtin_amdgcn_perm(c64, w1, 0x04030402u));
+    f.h2[0] = a0 + sub;
+    f.h2[1] = a1 + sub;
+    f.h2[2] = a2 + sub;
+    f.h2[3] = a3 + sub;
+}
+
+// Q4_K: the eight 6-bit (scale, min) pairs of a super-block from its 12 packed bytes held in three words,
+// all eight at once (rlx-gguf/src/lib.rs:743-751). Byte j%4 of sc[j/4] / mn[j/4] is the field of sub-block j.
+__device__ __forceinline__ void q4k_scales(uint32_t s0, uint32_t s1, uint32_t s2, uint32_t sc[2], uint32_t mn[2]) {
+    sc[0] = s0 & 0x3F3F3F3Fu;
+    mn[0] = s1 & 0x3F3F3F3Fu;
+    sc[1] = (s2 & 0x0F0F0F0Fu) | ((s0 >> 2) & 0x30303030u);
+    mn[1] = ((s2 >> 4) & 0x0F0F0F0Fu) | ((s1 >> 2) & 0x30303030u);
+}
+
+__device__ __forceinline__ float ubyte_to_float(uint32_t w, int byte) { return (float)((w >> (8 * byte)) & 0xFFu); }
+
+// D(16x16) += A(16x32) * B(32x16), halfs in, f32 accumulate. Lane l: A row / B column l & 15, k-slice 8*(l>>4)..+7;
+// D column l & 15, rows 4*(l>>4)..+3.
+__device__ __forceinline__ float4_t mfma16(const Frag &a, const Frag &b, float4_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a.h8, b.h8, c, 0, 0, 0);
+}
+// D(32x32) += A(32x16) * B(16x32). Lane l: A row / B column l & 31, k-slice 8*(l>>5)..+7;
+// D column l & 31, rows 8*(i/4) + 4*(l>>5) + i%4 for register i.
+__device__ __forceinline__ float16_t mfma32(const Frag &a, const Frag &b, float16_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a.h8, b.h8, c, 0, 0, 0);
+}
+
+}  // namespace rlx

@@ -1,0 +1,80 @@
+// Device layout of GGUF-packed weights in HBM. Shared by the host repacker and the kernels.
+//
+// A weight is a row-major [N, K] matrix packed in GGUF blocks along K (rlx-cpu/src/gguf_matmul.rs:15-20).
+// The device layout keeps every bit of every block (same byte count per block) but regroups it into
+// tiles of 16 rows x UNIT_K columns so that one 64-lane wavefront reads a tile with 16-byte loads and
+// every 4-byte word it gets is one MFMA operand fragment:
+//
+//   lane l of the wave:  n = l & 15  (row inside the tile),  g = l >> 4  (which 8 of every 32 columns)
+//   "granule" (n, blk, g) = the 8 weights of row n, 32-column block blk, columns 8g .. 8g+7
+//
+//   4-bit schemes: a granule is one 32-bit word; element e (0..7) sits in nibble NIB_POS[e] so that
+//       (w      & 0x000F000F) -> elements 0,1      (w      & 0x00F000F0) -> elements 2,3 (times 16)
+//       (w >> 8 & 0x000F000F) -> elements 4,5      (w >> 8 & 0x00F000F0) -> elements 6,7 (times 16)
+//     i.e. two masks and one shift split a word into four packed-half pairs in fragment order.
+//   Q8_0: a granule is 8 bytes, byte e = q_e XOR 0x80 (offset binary, so a byte permute builds 1024+u halfs).
+//
+// Tile ("unit") contents, in bytes:
+//   Q4_0 : [0,1024)  lane slots: 16 B at 16*l = granules of blocks 4u+0..3        [1024,1152) f16 d[n][4]
+//   Q8_0 : [0,2048)  two halves h: 16 B at 1024*h + 16*l = granules of blocks 4u+2h, 4u+2h+1
+//          [2048,2176) f16 d[n][4]
+//   Q4_K : [0,2048)  two halves h: 16 B at 1024*h + 16*l = granules of sub-blocks 4h+0..3 of super-block u
+//          [2048,2304) per row n: 16 B = f16 d, f16 dmin, 12 scale bytes (verbatim from the GGUF block)
+// Units are stored [row_tile][unit] with the unit index (K direction) fastest.
+// N is padded to a multiple of 16 and K to a multiple of UNIT_K with zero-scale blocks.
+#pragma once
+#include <stdint.h>
+
+#ifdef __HIPCC__
+#define RLX_HD __host__ __device__
+#else
+#define RLX_HD
+#endif
+
+namespace rlx {
+
+enum Scheme : int { SCHEME_Q4K = 5, SCHEME_Q4_0 = 11, SCHEME_Q8_0 = 12 };
+
+constexpr int TILE_ROWS = 16;
+
+struct Layout {
+    int unit_k;        // columns per unit
+    int unit_bytes;    // bytes per unit
+    int quant_bytes;   // bytes of lane slots at the start of a unit
+    int block_elems;   // GGUF block size
+    int block_bytes;   // GGUF block bytes
+};
+
+RLX_HD constexpr Layout layout_of(int scheme) {
+    return scheme == SCHEME_Q4_0   ? Layout{128, 1152, 1024, 32, 18}
+           : scheme == SCHEME_Q8_0 ? Layout{128, 2176, 2048, 32, 34}
+           : scheme == SCHEME_Q4K  ? Layout{256, 2304, 2048, 256, 144}
+                                   : Layout{0, 0, 0, 0, 0};
+}
+
+// nibble position of fragment element e inside a granule word
+RLX_HD constexpr int nib_pos(int e) { return ((e & 1) << 2) | (e >> 1); }
+
+struct WeightDims {
+    int64_t n, k;        // logical
+    int64_t row_tiles;   // ceil(n / 16)
+    int64_t units;       // ceil(k / unit_k)
+    int64_t n_pad, k_pad;
+    int64_t bytes;       // device bytes
+};
+
+RLX_HD inline WeightDims weight_dims(int scheme, int64_t n, int64_t k) {
+    Layout L = layout_of(scheme);
+    WeightDims d{};
+    d.n = n;
+    d.k = k;
+    if (L.unit_k == 0) return d;
+    d.row_tiles = (n + TILE_ROWS - 1) / TILE_ROWS;
+    d.units = (k + L.unit_k - 1) / L.unit_k;
+    d.n_pad = d.row_tiles * TILE_ROWS;
+    d.k_pad = d.units * L.unit_k;
+    d.bytes = d.row_tiles * d.units * (int64_t)L.unit_bytes;
+    return d;
+}
+
+}  // namespace rlx

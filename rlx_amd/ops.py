@@ -1,0 +1,186 @@
+"""Operator-level wrappers over the C ABI: device buffers, packed weights, dequant, matmul, FakeQuantize,
+plus the host utilities (encoders, repack, Philox). Thin: every call goes to librlx_mi355x.so."""
+import ctypes as C
+
+import numpy as np
+
+from . import _lib
+from .ir import DType, QuantScheme, RoundMode, ScaleMode
+
+
+class DeviceBuffer:
+    def __init__(self, nbytes):
+        self.nbytes = int(nbytes)
+        p = C.c_void_p()
+        _lib.check(_lib.lib().rlx_mi355x_malloc(C.byref(p), self.nbytes))
+        self.ptr = p.value
+
+    @staticmethod
+    def from_numpy(a):
+        a = np.ascontiguousarray(a)
+        b = DeviceBuffer(a.nbytes)
+        _lib.check(_lib.lib().rlx_mi355x_memcpy_h2d(b.ptr, a.ctypes.data, a.nbytes))
+        return b
+
+    def to_numpy(self, dtype, count=None):
+        dtype = np.dtype(dtype)
+        count = self.nbytes // dtype.itemsize if count is None else count
+        out = np.empty(count, dtype=dtype)
+        _lib.check(_lib.lib().rlx_mi355x_memcpy_d2h(out.ctypes.data, self.ptr, out.nbytes))
+        return out
+
+    def free(self):
+        if self.ptr:
+            _lib.check(_lib.lib().rlx_mi355x_free(self.ptr))
+            self.ptr = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+def sync(stream=None):
+    _lib.check(_lib.lib().rlx_mi355x_stream_sync(stream))
+
+
+def device_info():
+    buf = C.create_string_buffer(512)
+    _lib.check(_lib.lib().rlx_mi355x_device_info(buf, len(buf)))
+    return buf.value.decode()
+
+
+class Event:
+    def __init__(self):
+        p = C.c_void_p()
+        _lib.check(_lib.lib().rlx_mi355x_event_create(C.byref(p)))
+        self.ptr = p.value
+
+    def record(self, stream=None):
+        _lib.check(_lib.lib().rlx_mi355x_event_record(self.ptr, stream))
+
+    def elapsed_ms(self, stop):
+        ms = C.c_float()
+        _lib.check(_lib.lib().rlx_mi355x_event_elapsed_ms(self.ptr, stop.ptr, C.byref(ms)))
+        return ms.value
+
+    def __del__(self):
+        try:
+            if self.ptr:
+                _lib.lib().rlx_mi355x_event_destroy(self.ptr)
+                self.ptr = None
+        except Exception:
+            pass
+
+
+# ---- host utilities ------------------------------------------------------------------------------------
+
+def bytes_for(scheme, n_elems):
+    return _lib.lib().rlx_mi355x_bytes_for(int(scheme), n_elems)
+
+
+def quantize(scheme, x):
+    """f32 tensor -> GGUF bytes (uint8 array). This repo's encoders; the reference has none."""
+    x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1)
+    nb = bytes_for(scheme, x.size)
+    if nb < 0:
+        raise ValueError(f"{x.size} elements is not a multiple of the block size of {scheme!r}")
+    out = np.empty(nb, dtype=np.uint8)
+    _lib.check(_lib.lib().rlx_mi355x_quantize(int(scheme), x.ctypes.data, x.size, out.ctypes.data))
+    return out
+
+
+def repack_host(scheme, packed, n, k):
+    packed = np.ascontiguousarray(packed, dtype=np.uint8)
+    out = np.empty(_lib.lib().rlx_mi355x_qweight_device_bytes_for(int(scheme), n, k), dtype=np.uint8)
+    _lib.check(_lib.lib().rlx_mi355x_repack_host(int(scheme), packed.ctypes.data, packed.size, n, k, out.ctypes.data))
+    return out
+
+
+def philox_u32(seed, n):
+    out = np.empty(n, dtype=np.uint32)
+    _lib.lib().rlx_mi355x_philox_u32(seed, out.ctypes.data, n)
+    return out
+
+
+def philox_uniform(seed, n):
+    out = np.empty(n, dtype=np.float32)
+    _lib.lib().rlx_mi355x_philox_uniform(seed, out.ctypes.data, n)
+    return out
+
+
+def philox_normal(seed, n):
+    out = np.empty(n, dtype=np.float32)
+    _lib.lib().rlx_mi355x_philox_normal(seed, out.ctypes.data, n)
+    return out
+
+
+# ---- device operators ------------------------------------------------------------------------------------
+
+class QWeight:
+    """GGUF-packed [n, k] matrix resident in HBM in the device layout."""
+
+    def __init__(self, scheme, packed, n, k):
+        packed = np.ascontiguousarray(packed, dtype=np.uint8)
+        self.scheme, self.n, self.k = QuantScheme(scheme), int(n), int(k)
+        p = C.c_void_p()
+        _lib.check(_lib.lib().rlx_mi355x_qweight_create(int(scheme), packed.ctypes.data, packed.size, n, k, C.byref(p)))
+        self.ptr = p.value
+
+    def device_bytes(self):
+        return _lib.lib().rlx_mi355x_qweight_device_bytes(self.ptr)
+
+    def dequant(self, stream=None):
+        """rlx_gguf::dequant_* on the device -> f32 [n, k] (numpy)."""
+        out = DeviceBuffer(self.n * self.k * 4)
+        _lib.check(_lib.lib().rlx_mi355x_dequant(self.ptr, out.ptr, stream))
+        sync(stream)
+        return out.to_numpy(np.float32).reshape(self.n, self.k)
+
+    def free(self):
+        if self.ptr:
+            _lib.lib().rlx_mi355x_qweight_destroy(self.ptr)
+            self.ptr = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+def gguf_matmul_bt_device(x_dev, x_dtype, w: QWeight, out_dev, m, stream=None):
+    _lib.check(_lib.lib().rlx_mi355x_gguf_matmul_bt(x_dev.ptr, int(x_dtype), w.ptr, out_dev.ptr, m, None, 0, stream))
+
+
+def gguf_matmul_bt(x, w: QWeight, m, x_dtype=DType.F32):
+    """Host convenience: upload x ([m,k]; f32, or uint16 bit patterns for BF16 / float16 for F16), run, download [m,n]."""
+    xd = DeviceBuffer.from_numpy(x)
+    od = DeviceBuffer(m * w.n * 4)
+    gguf_matmul_bt_device(xd, x_dtype, w, od, m)
+    sync()
+    return od.to_numpy(np.float32).reshape(m, w.n)
+
+
+def fake_quantize(x, shape, axis, bits, scale_mode=ScaleMode.PerBatch, decay=0.0, state=None,
+                  round_mode=RoundMode.HalfAway):
+    """Host convenience around rlx_mi355x_fake_quantize. Returns (out f32, codes i8, scales f32); EMA updates `state`."""
+    x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1)
+    if axis is None:
+        chan_dim, inner = 1, max(x.size, 1)
+    else:
+        chan_dim = shape[axis]
+        inner = max(int(np.prod(shape[axis + 1:], dtype=np.int64)), 1)
+    xd = DeviceBuffer.from_numpy(x)
+    od = DeviceBuffer(max(x.nbytes, 4))
+    cd = DeviceBuffer(max(x.size, 4))
+    scratch = DeviceBuffer(chan_dim * 8)
+    sd = DeviceBuffer.from_numpy(state) if state is not None else None
+    _lib.check(_lib.lib().rlx_mi355x_fake_quantize(xd.ptr, od.ptr, cd.ptr, x.size, chan_dim, inner, bits, int(scale_mode),
+                                                  decay, sd.ptr if sd else None, int(round_mode), scratch.ptr, None))
+    sync()
+    if sd is not None and scale_mode == ScaleMode.EMA:
+        state[...] = sd.to_numpy(np.float32)
+    scales = scratch.to_numpy(np.float32)[chan_dim:]
+    return od.to_numpy(np.float32, x.size).reshape(shape), cd.to_numpy(np.int8, x.size).reshape(shape), scales

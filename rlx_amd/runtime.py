@@ -1,0 +1,176 @@
+"""Session / CompiledGraph over the C ABI: the Python-side stand-in for what rlx-runtime's `Session` does once a
+`Device::Mi355x` backend is registered (rlx-runtime/src/session.rs:42-158, compiled.rs:27-206)."""
+import ctypes as C
+import enum
+
+import numpy as np
+
+from . import _lib
+from .ir import DType, Graph, OpKind, RoundMode
+
+
+class Device(enum.Enum):
+    Mi355x = "MI355X"  # the new rlx_driver::Device variant (rlx-driver/src/device.rs:23-59)
+
+    def name_str(self):
+        return _lib.lib().rlx_mi355x_device_name().decode()
+
+
+def is_available(device=Device.Mi355x):
+    return bool(_lib.lib().rlx_mi355x_is_available())
+
+
+_NP = {DType.F32: np.float32, DType.F16: np.float16, DType.BF16: np.uint16, DType.U8: np.uint8, DType.I8: np.int8}
+
+
+def _graph_desc(graph: Graph):
+    n = len(graph.nodes)
+    nodes = (_lib.NodeDesc * n)()
+    keep = []
+    for i, nd in enumerate(graph.nodes):
+        d = nodes[i]
+        d.op_kind = int(nd.op.kind)
+        d.dtype = int(nd.shape.dtype)
+        d.rank = len(nd.shape.dims)
+        for r, v in enumerate(nd.shape.dims):
+            d.dims[r] = v
+        d.n_inputs = len(nd.inputs)
+        for j, v in enumerate(nd.inputs):
+            d.inputs[j] = v
+        if nd.name is not None:
+            b = nd.name.encode()
+            keep.append(b)
+            d.name = b
+        d.scheme = int(nd.op.scheme) if nd.op.scheme is not None else 0
+        d.bits = nd.op.bits
+        d.axis = -1 if nd.op.axis is None else nd.op.axis
+        d.scale_mode = int(nd.op.scale_mode)
+        d.ema_decay = nd.op.ema_decay
+        d.ste = int(nd.op.ste)
+    outs = (C.c_uint32 * len(graph.outputs))(*graph.outputs)
+    gname = graph.name.encode()
+    keep += [nodes, outs, gname]
+    g = _lib.GraphDesc(gname, nodes, n, outs, len(graph.outputs))
+    return g, keep
+
+
+class CompiledGraph:
+    """Box<dyn ExecutableGraph> (rlx-runtime/src/backend.rs:146-371)."""
+
+    def __init__(self, handle, graph):
+        self._h = handle
+        self.graph = graph
+
+    def close(self):
+        if self._h:
+            _lib.lib().rlx_exec_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def set_param(self, name, data):
+        a = np.ascontiguousarray(data, dtype=np.float32)
+        return _lib.check(_lib.lib().rlx_exec_set_param(self._h, name.encode(), a.ctypes.data, a.size))
+
+    def set_param_typed(self, name, data, dtype):
+        a = np.ascontiguousarray(data)
+        return _lib.check(_lib.lib().rlx_exec_set_param_typed(self._h, name.encode(), a.ctypes.data, a.nbytes, int(dtype)))
+
+    def _outs(self):
+        bufs, arr = [], (_lib.OutBuf * len(self.graph.outputs))()
+        for i, o in enumerate(self.graph.outputs):
+            sh = self.graph.nodes[o].shape
+            b = np.empty(sh.num_elements(), dtype=_NP[sh.dtype])
+            bufs.append(b)
+            arr[i].data = b.ctypes.data
+            arr[i].capacity = b.nbytes
+        return bufs, arr
+
+    def run(self, inputs):
+        """run(&[(name, &[f32])]) -> Vec<Vec<f32>>"""
+        keep = [np.ascontiguousarray(v, dtype=np.float32) for _, v in inputs]
+        ins = (_lib.NamedBuf * max(len(inputs), 1))()
+        for i, ((name, _), a) in enumerate(zip(inputs, keep)):
+            ins[i] = _lib.NamedBuf(name.encode(), a.ctypes.data, a.nbytes, int(DType.F32))
+        bufs, outs = self._outs()
+        _lib.check(_lib.lib().rlx_exec_run(self._h, ins, len(inputs), outs, len(bufs)))
+        return bufs
+
+    def run_typed(self, inputs):
+        """run_typed(&[(name, &[u8], DType)]) -> Vec<(Vec<u8>, DType)>; arrays are passed as raw bytes of `dtype`."""
+        keep = [np.ascontiguousarray(v) for _, v, _ in inputs]
+        ins = (_lib.NamedBuf * max(len(inputs), 1))()
+        for i, ((name, _, dt), a) in enumerate(zip(inputs, keep)):
+            ins[i] = _lib.NamedBuf(name.encode(), a.ctypes.data, a.nbytes, int(dt))
+        bufs, outs = self._outs()
+        _lib.check(_lib.lib().rlx_exec_run_typed(self._h, ins, len(inputs), outs, len(bufs)))
+        return [(b, DType(outs[i].dtype)) for i, b in enumerate(bufs)]
+
+    # device-resident execution (run_slots / arena_ptr analogue)
+    def write_input(self, name, data, dtype=DType.F32):
+        a = np.ascontiguousarray(data)
+        return _lib.check(_lib.lib().rlx_exec_write_input(self._h, name.encode(), a.ctypes.data, a.nbytes, int(dtype)))
+
+    def launch(self):
+        _lib.check(_lib.lib().rlx_exec_launch(self._h))
+
+    def sync(self):
+        _lib.check(_lib.lib().rlx_exec_sync(self._h))
+
+    def stream(self):
+        return _lib.lib().rlx_exec_stream(self._h)
+
+    def arena_bytes(self):
+        return _lib.lib().rlx_exec_arena_bytes(self._h)
+
+    def describe_plan(self):
+        buf = C.create_string_buffer(16384)
+        _lib.check(_lib.lib().rlx_exec_describe_plan(self._h, buf, len(buf)))
+        return buf.value.decode()
+
+    def read_output(self, index=0):
+        sh = self.graph.nodes[self.graph.outputs[index]].shape
+        out = np.empty(sh.num_elements(), dtype=_NP[sh.dtype])
+        p, n = C.c_void_p(), C.c_size_t()
+        _lib.check(_lib.lib().rlx_exec_output_slot(self._h, index, C.byref(p), C.byref(n)))
+        self.sync()
+        _lib.check(_lib.lib().rlx_mi355x_memcpy_d2h(out.ctypes.data, p, out.nbytes))
+        return out
+
+    def fq_codes(self, node_id):
+        n = self.graph.nodes[node_id].shape.num_elements()
+        out = np.empty(n, dtype=np.int8)
+        _lib.check(_lib.lib().rlx_exec_read_fq_codes(self._h, node_id, out.ctypes.data, n))
+        return out
+
+
+class Session:
+    """Session::new(device).compile(graph) (rlx-runtime/src/session.rs:42-136)."""
+
+    def __init__(self, device=Device.Mi355x, fq_round_mode=RoundMode.HalfAway, verbose=False):
+        self.device = device
+        self.fq_round_mode = fq_round_mode
+        self.verbose = verbose
+
+    @staticmethod
+    def new(device=Device.Mi355x):
+        return Session(device)
+
+    def compile(self, graph: Graph) -> CompiledGraph:
+        g, keep = _graph_desc(graph)
+        opts = _lib.CompileOpts(0, int(self.fq_round_mode), int(self.verbose))
+        h = _lib.lib().rlx_mi355x_compile(C.byref(g), C.byref(opts))
+        del keep
+        if not h:
+            raise _lib.RlxError(-1, _lib.last_error())
+        return CompiledGraph(h, graph)
+
+
+def supported_ops():
+    p = C.POINTER(C.c_uint32)()
+    n = _lib.lib().rlx_mi355x_supported_ops(C.byref(p))
+    return [OpKind(p[i]) for i in range(n)]

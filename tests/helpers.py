@@ -1,0 +1,89 @@
+"""Shared test helpers: seeded inputs, packed weights, a numpy reader of the device layout, error metrics."""
+import numpy as np
+
+Q4K, Q4_0, Q8_0 = 5, 11, 12
+SCHEME_NAMES = {Q4K: "q4_k", Q4_0: "q4_0", Q8_0: "q8_0"}
+NIB_POS = [0, 4, 1, 5, 2, 6, 3, 7]
+UNIT = {Q4_0: (128, 1152, 1024), Q8_0: (128, 2176, 2048), Q4K: (256, 2304, 2048)}
+
+
+def make_weights(scheme, n, k, std=0.02, seed=0):
+    """f32 ~N(0,std) weights -> GGUF bytes through the library's encoders (identical bytes feed oracle and GPU)."""
+    from rlx_amd import ops
+
+    rng = np.random.default_rng(seed)
+    w = (rng.standard_normal((n, k)) * std).astype(np.float32)
+    return ops.quantize(scheme, w), w
+
+
+def random_blocks(scheme, n, k, seed=0):
+    """Arbitrary block bytes (every bit pattern in codes and 6-bit fields) with finite f16 scales."""
+    rng = np.random.default_rng(seed)
+    be, bb = {Q4_0: (32, 18), Q8_0: (32, 34), Q4K: (256, 144)}[scheme]
+    nb = n * k // be
+    p = rng.integers(0, 256, (nb, bb), dtype=np.uint8)
+    d = (rng.standard_normal(nb) * 0.02).astype(np.float16)
+    d[::11] = np.float16(3e-6)   # subnormal halfs
+    d[::13] = np.float16(0.0)
+    p[:, 0:2] = d.view(np.uint8).reshape(nb, 2)
+    if scheme == Q4K:
+        dm = (np.abs(rng.standard_normal(nb)) * 0.01).astype(np.float16)
+        p[:, 2:4] = dm.view(np.uint8).reshape(nb, 2)
+    return p.reshape(-1)
+
+
+def decode_device_layout(scheme, dev, n, k):
+    """Read the device layout back into f32 [n,k] following csrc/layout.h, with the reference's arithmetic."""
+    unit_k, unit_bytes, qbytes = UNIT[scheme]
+    tiles, units = (n + 15) // 16, (k + unit_k - 1) // unit_k
+    dev = dev.reshape(tiles, units, unit_bytes)
+    out = np.zeros((tiles * 16, units * unit_k), np.float32)
+    for l in range(64):
+        nrow, g = l & 15, l >> 4
+        rows = np.arange(tiles) * 16 + nrow
+        if scheme in (Q4_0, Q8_0):
+            for t in range(4):
+                d = dev[:, :, qbytes + nrow * 8 + 2 * t: qbytes + nrow * 8 + 2 * t + 2].copy().view(np.float16)
+                d = d.astype(np.float32).reshape(tiles, units)
+                for e in range(8):
+                    if scheme == Q4_0:
+                        w = dev[:, :, l * 16 + 4 * t: l * 16 + 4 * t + 4].copy().view(np.uint32).reshape(tiles, units)
+                        code = ((w >> (4 * NIB_POS[e])) & 0xF).astype(np.int32) - 8
+                    else:
+                        b = dev[:, :, (t >> 1) * 1024 + l * 16 + (t & 1) * 8 + e].astype(np.int32)
+                        code = b - 128
+                    cols = np.arange(units) * unit_k + t * 32 + g * 8 + e
+                    out[np.ix_(rows, cols)] = d * code.astype(np.float32)
+        else:
+            meta = dev[:, :, qbytes + nrow * 16: qbytes + nrow * 16 + 16]
+            d = meta[:, :, 0:2].copy().view(np.float16).astype(np.float32).reshape(tiles, units)
+            dmin = meta[:, :, 2:4].copy().view(np.float16).astype(np.float32).reshape(tiles, units)
+            q = meta[:, :, 4:16].astype(np.uint32)
+            for j in range(8):
+                if j < 4:
+                    sc, mn = q[:, :, j] & 63, q[:, :, j + 4] & 63
+                else:
+                    sc = (q[:, :, j + 4] & 0xF) | ((q[:, :, j - 4] >> 6) << 4)
+                    mn = (q[:, :, j + 4] >> 4) | ((q[:, :, j] >> 6) << 4)
+                dj = (d * sc.astype(np.float32)).astype(np.float32)
+                mj = (dmin * mn.astype(np.float32)).astype(np.float32)
+                off = (j >> 2) * 1024 + l * 16 + (j & 3) * 4
+                w = dev[:, :, off: off + 4].copy().view(np.uint32).reshape(tiles, units)
+                for e in range(8):
+                    code = ((w >> (4 * NIB_POS[e])) & 0xF).astype(np.float32)
+                    cols = np.arange(units) * unit_k + j * 32 + g * 8 + e
+                    out[np.ix_(rows, cols)] = ((dj * code).astype(np.float32) - mj).astype(np.float32)
+    return out[:n, :k]
+
+
+def rel_err(got, want):
+    """The reference tests' convention: |delta| / max(|expected|, 1) (rlx-runtime/tests/dequant_matmul_gguf.rs:231-233)."""
+    got = np.asarray(got, np.float64)
+    want = np.asarray(want, np.float64)
+    return float(np.max(np.abs(got - want) / np.maximum(np.abs(want), 1.0)))
+
+
+def f32_to_bf16_bits(x):
+    u = np.ascontiguousarray(x, np.float32).view(np.uint32).astype(np.uint64)
+    r = (u + 0x7FFF + ((u >> 16) & 1)) >> 16
+    return r.astype(np.uint16)

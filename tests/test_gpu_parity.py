@@ -1,0 +1,344 @@
+"""GPU parity: the HIP path (through the C ABI) against the CPU oracle on identical seeded inputs.
+Bars: decoded weights and FakeQuantize outputs / integer codes bit-exact; matmul outputs within max relative error
+2e-3 against the f64-accumulated oracle, with the reference tests' normalisation |delta| / max(|expected|, 1)."""
+import numpy as np
+import pytest
+
+import rlx_amd
+from rlx_amd import DType, Graph, Op, QuantScheme, RoundMode, ScaleMode, Session, Shape, ops
+from helpers import Q4K, Q4_0, Q8_0, SCHEME_NAMES, f32_to_bf16_bits, make_weights, random_blocks, rel_err
+
+pytestmark = pytest.mark.gpu
+TOL = 2e-3
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _need_gpu():
+    assert rlx_amd.is_available(), "no MI355X / kernel module failed to load: " + rlx_amd._lib.last_error()
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+# ------------------------------------------------------------------ dequant: bit-exact
+
+@pytest.mark.parametrize("scheme", [Q4_0, Q8_0, Q4K])
+@pytest.mark.parametrize("n,k", [(16, 256), (50, 768), (256, 4096), (1, 256)])
+def test_dequant_bit_exact_random_bytes(oracle, scheme, n, k):
+    say("dequant", SCHEME_NAMES[scheme], n, k)
+    packed = random_blocks(scheme, n, k, seed=3 * n + k)
+    w = ops.QWeight(scheme, packed, n, k)
+    got = w.dequant()
+    want = oracle.dequant(scheme, packed, n * k).reshape(n, k)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("scheme", [Q4_0, Q8_0, Q4K])
+def test_dequant_bit_exact_llama_shape(oracle, scheme):
+    n, k = 1024, 4096
+    packed, _ = make_weights(scheme, n, k, seed=5)
+    got = ops.QWeight(scheme, packed, n, k).dequant()
+    want = oracle.dequant(scheme, packed, n * k).reshape(n, k)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+# ------------------------------------------------------------------ reference test cases through Session
+
+def f16_bytes(v):
+    return np.array([v], dtype=np.float16).view(np.uint8).tolist()
+
+
+def run_dq(packed, scheme, x, m, k, n, typed=None):
+    g = Graph.new("dq")
+    x_in = g.input("x", Shape.new([m, k], DType.F32))
+    w = g.param("w_packed", Shape.new([len(packed)], DType.U8))
+    y = g.add_node(Op.DequantMatMul(QuantScheme(scheme)), [x_in, w], Shape.new([m, n], DType.F32))
+    g.set_outputs([y])
+    compiled = Session.new(rlx_amd.Device.Mi355x).compile(g)
+    compiled.set_param_typed("w_packed", packed, DType.U8)
+    if typed is None:
+        return compiled.run([("x", x)])[0].reshape(m, n)
+    return compiled.run_typed([("x", x, typed)])[0][0].reshape(m, n)
+
+
+def test_reference_q4k_case():
+    # rlx-runtime/tests/dequant_matmul_gguf.rs:249-303
+    packed = np.array(f16_bytes(1.0) + f16_bytes(1.0) + [1, 1, 1, 1] + [0] * 8 + [0x77] * 128, dtype=np.uint8)
+    k, n, m = 256, 1, 2
+    x = (0.01 * (np.arange(m * k, dtype=np.float32) + 1.0)).astype(np.float32)
+    w_ref = np.concatenate([np.full(128, 7.0, np.float32), np.zeros(128, np.float32)])
+    exp = (x.reshape(m, k).astype(np.float64) @ w_ref.astype(np.float64)).reshape(m, n)
+    got = run_dq(packed, Q4K, x, m, k, n)
+    assert rel_err(got, exp) < 1e-3
+
+
+@pytest.mark.parametrize("scheme", [Q8_0, Q4_0])
+def test_reference_layout_case_n_gt_1(oracle, scheme):
+    # run_q8k_layout_case (dequant_matmul_gguf.rs:176-241) restated for the claimed schemes: rows differ, so an
+    # [k,n] reading of the bytes fails.
+    k, n, m = 256, 4, 2
+    rows = []
+    for j in range(n):
+        for b in range(k // 32):
+            if scheme == Q8_0:
+                qs = np.clip(np.arange(32) - 16 + 30 * j, -128, 127).astype(np.int8).view(np.uint8)
+            else:
+                qs = (((np.arange(16) + j) % 16) | (((np.arange(16) + 3 * j + b) % 16) << 4)).astype(np.uint8)
+            rows.append(np.concatenate([np.array(f16_bytes(0.25 * (j + 1)), np.uint8), qs]))
+    packed = np.concatenate(rows)
+    x = (0.01 * (np.arange(m * k, dtype=np.float32) + 1.0)).astype(np.float32)
+    exp = oracle.gguf_matmul_f64(x, packed, m, k, n, scheme)
+    got = run_dq(packed, scheme, x, m, k, n)
+    assert rel_err(got, exp) < 1e-4
+
+
+def test_unknown_names_are_ignored_with_a_warning_code():
+    packed, _ = make_weights(Q4_0, 16, 128)
+    g = Graph.new("names")
+    x_in = g.input("x", Shape.new([1, 128], DType.F32))
+    w = g.param("w", Shape.new([len(packed)], DType.U8))
+    g.set_outputs([g.add_node(Op.DequantMatMul(QuantScheme.GgufQ4_0), [x_in, w], Shape.new([1, 16], DType.F32))])
+    c = Session.new().compile(g)
+    assert c.set_param("nope", np.zeros(4, np.float32)) == 1
+    with pytest.raises(rlx_amd.RlxError) as ei:
+        c.run([("x", np.zeros(128, np.float32))])
+    assert "never set" in str(ei.value)
+    assert c.set_param_typed("w", packed, DType.U8) == 0
+    assert np.all(c.run([("x", np.zeros(128, np.float32)), ("bogus", np.zeros(128, np.float32))])[0] == 0)
+    with pytest.raises(rlx_amd.RlxError):
+        c.run([("x", np.zeros(64, np.float32))])  # wrong length is an error, not a silent truncation
+
+
+# ------------------------------------------------------------------ decode matmul (m <= 16)
+
+def check_matmul(oracle, scheme, n, k, m, x_dtype=DType.F32, std=0.02, seed=0, cols=None):
+    say("matmul", SCHEME_NAMES[scheme], "n", n, "k", k, "m", m, x_dtype.name)
+    packed, _ = make_weights(scheme, n, k, std=std, seed=seed)
+    rng = np.random.default_rng(seed + 1000)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    if x_dtype == DType.BF16:
+        x = oracle.bf16_round(x)            # what the typed boundary widens to f32 (rlx-runtime/src/backend.rs:49-53)
+        xin = f32_to_bf16_bits(x)
+    elif x_dtype == DType.F16:
+        x = x.astype(np.float16).astype(np.float32)
+        xin = x.astype(np.float16)
+    else:
+        xin = x
+    w = ops.QWeight(scheme, packed, n, k)
+    got = ops.gguf_matmul_bt(xin, w, m, x_dtype)
+    n0, n1 = (0, n) if cols is None else cols
+    ref64 = oracle.gguf_matmul_f64(x, packed, m, k, n, scheme, n0, n1)
+    err = rel_err(got[:, n0:n1], ref64)
+    say("   max rel err vs f64 oracle:", err)
+    assert err <= TOL
+    return got, x, packed, err
+
+
+def test_config1_q8_0_gemv_4096(oracle):
+    # BASELINE config 1: W 4096x4096 ~N(0,0.02) Q8_0, x [1,4096] f32 ~N(0,1)
+    got, x, packed, err = check_matmul(oracle, Q8_0, 4096, 4096, 1)
+    cpu = oracle.gguf_matmul_bt(x, packed, 1, 4096, 4096, Q8_0)     # the reference CPU path, f32
+    ref64 = oracle.gguf_matmul_f64(x, packed, 1, 4096, 4096, Q8_0)
+    cpu_err = rel_err(cpu, ref64)
+    say("   cpu path err", cpu_err, "gpu err", err)
+    assert err <= max(cpu_err, 2e-6) * 4   # no worse than the CPU path's own rounding, up to a small factor
+
+
+@pytest.mark.parametrize("n,k", [(4096, 4096), (1024, 4096), (14336, 4096), (4096, 14336)])
+def test_config2_q4_0_gemv_llama8b(oracle, n, k):
+    got, x, packed, err = check_matmul(oracle, Q4_0, n, k, 1, seed=n % 97)
+    cpu = oracle.gguf_matmul_bt(x, packed, 1, k, n, Q4_0)
+    cpu_err = rel_err(cpu, oracle.gguf_matmul_f64(x, packed, 1, k, n, Q4_0))
+    say("   cpu path err", cpu_err, "gpu err", err)
+    assert err <= max(cpu_err, 2e-6) * 4
+
+
+@pytest.mark.parametrize("scheme", [Q4_0, Q8_0, Q4K])
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 8])
+def test_decode_batch_f32(oracle, scheme, m):
+    check_matmul(oracle, scheme, 512, 1024, m, seed=m)
+
+
+@pytest.mark.parametrize("scheme", [Q4_0, Q8_0, Q4K])
+@pytest.mark.parametrize("m", [1, 4, 16])
+def test_decode_batch_bf16(oracle, scheme, m):
+    check_matmul(oracle, scheme, 512, 2048, m, x_dtype=DType.BF16, seed=10 + m)
+
+
+def test_decode_f16_activations(oracle):
+    check_matmul(oracle, Q4_0, 256, 512, 5, x_dtype=DType.F16, seed=3)
+
+
+@pytest.mark.parametrize("scheme,n,k", [(Q4_0, 50, 96), (Q8_0, 17, 32), (Q4K, 33, 768), (Q4_0, 2064, 160)])
+def test_decode_ragged_shapes(oracle, scheme, n, k):
+    # n not a multiple of 16, k not a multiple of the 128/256-column unit: exercises the zero-padded tiles
+    check_matmul(oracle, scheme, n, k, 3, seed=n)
+
+
+def test_decode_more_rows_than_one_pass(oracle):
+    check_matmul(oracle, Q4_0, 128, 256, 20, seed=4)           # f32: 8 rows per pass -> 3 passes
+    check_matmul(oracle, Q4K, 64, 512, 37, x_dtype=DType.BF16, seed=5)  # 16 rows per pass -> 3 passes
+
+
+def test_decode_large_k_is_chunked(oracle):
+    # 70B down projection width: the staged activations exceed one LDS chunk
+    check_matmul(oracle, Q4_0, 64, 28672, 4, std=0.015, seed=6)
+    check_matmul(oracle, Q4K, 32, 14336, 8, seed=7)
+
+
+def test_q4k_gemv_llama_shape(oracle):
+    check_matmul(oracle, Q4K, 4096, 4096, 1, seed=8)
+
+
+def test_matmul_is_deterministic(oracle):
+    packed, _ = make_weights(Q4_0, 1024, 4096, seed=9)
+    x = np.random.default_rng(9).standard_normal((1, 4096)).astype(np.float32)
+    w = ops.QWeight(Q4_0, packed, 1024, 4096)
+    a = ops.gguf_matmul_bt(x, w, 1)
+    b = ops.gguf_matmul_bt(x, w, 1)
+    assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+
+
+def test_matmul_linearity_full_size(oracle):
+    # size-independent property at a BASELINE shape: W(x1 + 2 x2) = W x1 + 2 W x2 up to f32 rounding
+    n, k = 14336, 4096
+    packed, _ = make_weights(Q4_0, n, k, seed=11)
+    w = ops.QWeight(Q4_0, packed, n, k)
+    rng = np.random.default_rng(12)
+    x1, x2 = rng.standard_normal((1, k)).astype(np.float32), rng.standard_normal((1, k)).astype(np.float32)
+    y1, y2 = ops.gguf_matmul_bt(x1, w, 1), ops.gguf_matmul_bt(x2, w, 1)
+    y3 = ops.gguf_matmul_bt((x1 + 2 * x2).astype(np.float32), w, 1)
+    assert rel_err(y3, y1.astype(np.float64) + 2 * y2.astype(np.float64)) < 1e-4
+
+
+# ------------------------------------------------------------------ FakeQuantize: bit-exact
+
+def check_fq(oracle, x, shape, axis, bits, scale_mode=ScaleMode.PerBatch, decay=0.0, state=None,
+             round_mode=RoundMode.HalfAway):
+    st_o = None if state is None else state.copy()
+    st_g = None if state is None else state.copy()
+    want, wcodes, wscales = oracle.fake_quantize(x, shape, axis, bits, int(scale_mode), decay, st_o, int(round_mode))
+    got, codes, scales = ops.fake_quantize(x, shape, axis, bits, scale_mode, decay, st_g, round_mode)
+    assert np.array_equal(scales.view(np.uint32), wscales.view(np.uint32))
+    assert np.array_equal(codes, wcodes), f"{np.sum(codes != wcodes)} integer codes differ"
+    nan = np.isnan(want)
+    assert np.array_equal(np.isnan(got), nan)
+    assert np.array_equal(got.view(np.uint32)[~nan], want.view(np.uint32)[~nan])
+    if state is not None:
+        assert np.array_equal(st_g.view(np.uint32), st_o.view(np.uint32))
+    return got, codes
+
+
+@pytest.mark.parametrize("shape,axis,bits", [((6,), None, 8), ((3, 4), 0, 8), ((2, 5, 3), 1, 4), ((3, 4), 0, 2)])
+def test_fq_reference_shapes(oracle, shape, axis, bits):
+    # rlx-mlx/tests/autodiff_fakequant_parity.rs:189-214, 280-308
+    total = int(np.prod(shape))
+    x = (np.float32(0.07) * np.arange(total, dtype=np.float32) - np.float32(1.3)).astype(np.float32)
+    check_fq(oracle, x, shape, axis, bits)
+    cd = 1 if axis is None else shape[axis]
+    state = (np.float32(0.01) + np.float32(0.05) * np.arange(cd, dtype=np.float32)).astype(np.float32)
+    check_fq(oracle, x, shape, axis, bits, ScaleMode.Fixed, state=state)
+
+
+def heavy_tailed(rows, cols, seed):
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal((rows, cols)).astype(np.float32)
+    mask = rng.random((rows, cols)) < 0.001
+    x[mask] *= 20.0
+    return x
+
+
+def test_config4_fq_columns_full_size(oracle):
+    # BASELINE config 4: [8192, 4096] f32, N(0,1) with 0.1% of entries x20; int8 per channel along the last axis
+    x = heavy_tailed(8192, 4096, 21)
+    for mode in (RoundMode.HalfAway, RoundMode.HalfEven):
+        got, codes = check_fq(oracle, x, x.shape, 1, 8, round_mode=mode)
+    r = x / (np.max(np.abs(x), axis=0) / np.float32(127)).astype(np.float32)
+    say("   exact .5 ties in x/s:", int(np.sum(np.abs(r - np.trunc(r)) == 0.5)))
+    assert int(np.abs(codes.astype(int)).max()) == 127
+
+
+@pytest.mark.parametrize("shape,axis", [((8192, 4096), 0), ((8, 64, 28, 28), 1), ((1000, 33), 1), ((1000, 33), 0),
+                                         ((5, 7, 9), 2), ((70000,), None), ((4, 300000), None)])
+def test_fq_layouts(oracle, shape, axis):
+    say("fq layout", shape, axis)
+    x = np.random.default_rng(sum(shape)).standard_normal(shape).astype(np.float32)
+    for bits in (8, 4, 2):
+        check_fq(oracle, x, shape, axis, bits)
+
+
+def test_fq_special_values(oracle):
+    rng = np.random.default_rng(33)
+    x = rng.standard_normal((256, 64)).astype(np.float32)
+    x[:, 5] = 0.0
+    x[3, 7] = np.nan
+    x[10, 9] = np.float32(1e-41)   # subnormal input
+    x[:, 11] = np.float32(1e-30)   # scale above the 1e-12 floor but tiny
+    x[:, 12] = np.float32(1e-15)   # max/127 below the floor -> floor wins
+    x[4, 13] = -0.0
+    got, codes = check_fq(oracle, x, x.shape, 1, 8)
+    assert np.isnan(got[3, 7]) and codes[3, 7] == 0 and np.all(codes[:, 5] == 0)
+    # constructed ties: s is a power of two, x = (k + 0.5) s
+    s = np.float32(2.0 ** -5)
+    ks = np.arange(-20, 21, dtype=np.float32)
+    t = np.concatenate([(ks + np.float32(0.5)) * s, [np.float32(127.0) * s, np.float32(0.49999997) * s]]).astype(np.float32)
+    _, ca = check_fq(oracle, t, t.shape, None, 8, round_mode=RoundMode.HalfAway)
+    _, ce = check_fq(oracle, t, t.shape, None, 8, round_mode=RoundMode.HalfEven)
+    assert np.any(ca != ce) and ca[-1] == 0
+
+
+def test_fq_ema_and_fixed(oracle):
+    x = heavy_tailed(512, 256, 34)
+    state = np.abs(np.random.default_rng(35).standard_normal(256)).astype(np.float32) * 0.05
+    state[::5] = 0.0
+    state[3] = -1.0
+    check_fq(oracle, x, x.shape, 1, 8, ScaleMode.EMA, decay=0.99, state=state)
+    check_fq(oracle, x, x.shape, 1, 4, ScaleMode.Fixed, state=np.maximum(state, 0.001).astype(np.float32))
+    check_fq(oracle, x, x.shape, 0, 8, ScaleMode.EMA, decay=0.9, state=np.zeros(512, np.float32))
+
+
+def test_fq_idempotent_full_size(oracle):
+    # size-independent property: fake-quantizing an already fake-quantized tensor changes nothing
+    x = heavy_tailed(8192, 4096, 36)
+    y, c1, _ = ops.fake_quantize(x, x.shape, 1, 8)
+    z, c2, _ = ops.fake_quantize(y, y.shape, 1, 8)
+    assert np.array_equal(c1, c2)
+    assert np.max(np.abs(z - y)) <= np.max(np.abs(y)) * 2e-7
+
+
+def test_fq_unsupported_bits():
+    with pytest.raises(rlx_amd.RlxError) as ei:
+        ops.fake_quantize(np.zeros(8, np.float32), (8,), None, 3)
+    assert "unsupported bits 3" in str(ei.value)
+
+
+# ------------------------------------------------------------------ graph level: FakeQuantize -> Q8_0 matmul (config 4 chain)
+
+def test_graph_fq_then_q8_0_matmul(oracle):
+    rows, k, n = 64, 4096, 256
+    x = heavy_tailed(rows, k, 41)
+    packed, _ = make_weights(Q8_0, n, k, seed=42)
+    g = Graph.new("cfg4")
+    xi = g.input("x", Shape.new([rows, k], DType.F32))
+    fq = g.add_node(Op.FakeQuantize(8, 1), [xi], Shape.new([rows, k], DType.F32))
+    w = g.param("w", Shape.new([len(packed)], DType.U8))
+    y = g.add_node(Op.DequantMatMul(QuantScheme.GgufQ8_0), [fq, w], Shape.new([rows, n], DType.F32))
+    g.set_outputs([y, fq])
+    c = Session.new().compile(g)
+    say(c.describe_plan())
+    c.set_param_typed("w", packed, DType.U8)
+    y_got, fq_got = c.run([("x", x)])
+    fq_ref, codes_ref, _ = oracle.fake_quantize(x, x.shape, 1, 8)
+    assert np.array_equal(fq_got.reshape(rows, k).view(np.uint32), fq_ref.view(np.uint32))
+    assert np.array_equal(c.fq_codes(fq).reshape(rows, k), codes_ref)
+    ref64 = oracle.gguf_matmul_f64(fq_ref, packed, rows, k, n, Q8_0)
+    assert rel_err(y_got.reshape(rows, n), ref64) <= TOL
+
+
+def test_graph_typed_bf16_input(oracle):
+    m, k, n = 4, 512, 64
+    packed, _ = make_weights(Q4K, n, k, seed=43)
+    x = oracle.bf16_round(np.random.default_rng(44).standard_normal((m, k)).astype(np.float32))
+    got = run_dq(packed, Q4K, f32_to_bf16_bits(x), m, k, n, typed=DType.BF16)
+    assert rel_err(got, oracle.gguf_matmul_f64(x, packed, m, k, n, Q4K)) <= TOL

@@ -1,0 +1,178 @@
+"""CPU-side tests of the shipped library: the C ABI loads and exports every declared symbol, the host logic
+(format constants, repack into the device layout, encoders, Philox, graph validation) behaves, all without a GPU."""
+import os
+import re
+
+import numpy as np
+import pytest
+
+import rlx_amd
+from rlx_amd import DType, Graph, Op, QuantScheme, ScaleMode, Session, Shape, ops
+from helpers import Q4K, Q4_0, Q8_0, decode_device_layout, make_weights, random_blocks
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_header_symbols_all_exported():
+    hdr = open(os.path.join(ROOT, "include", "rlx_mi355x.h")).read()
+    hdr = re.sub(r"/\*.*?\*/", "", hdr, flags=re.S)
+    declared = set(re.findall(r"\b(rlx_(?:mi355x|exec)_[a-z0-9_]+)\s*\(", hdr))
+    assert len(declared) > 40
+    L = rlx_amd._lib.lib()
+    missing = [s for s in declared if not hasattr(L, s)]
+    assert not missing, missing
+    assert declared == set(rlx_amd._lib.SIGNATURES), declared ^ set(rlx_amd._lib.SIGNATURES)
+    assert L.rlx_mi355x_abi_version() == 1
+    assert L.rlx_mi355x_device_name() == b"MI355X"
+
+
+def test_format_constants_match_reference_and_oracle(oracle):
+    for s in (Q4K, Q4_0, Q8_0):
+        L = rlx_amd._lib.lib()
+        assert L.rlx_mi355x_block_elems(s) == oracle.block_elems(s) == QuantScheme(s).gguf_block_size()
+        assert L.rlx_mi355x_block_bytes(s) == oracle.block_bytes(s) == QuantScheme(s).gguf_block_bytes()
+        for n in (0, 256, 4096 * 4096, 255, 33):
+            assert ops.bytes_for(s, n) == oracle.bytes_for(s, n)
+    assert ops.bytes_for(3, 256) == -1  # Fp8E4m3: not a GGUF scheme
+
+
+@pytest.mark.parametrize("scheme", [Q4_0, Q8_0, Q4K])
+@pytest.mark.parametrize("n,k", [(16, 256), (40, 512), (3, 768)])
+def test_repack_is_lossless_and_matches_oracle_decode(oracle, scheme, n, k):
+    packed = random_blocks(scheme, n, k, seed=n + k)
+    dev = ops.repack_host(scheme, packed, n, k)
+    got = decode_device_layout(scheme, dev, n, k)
+    want = oracle.dequant(scheme, packed, n * k).reshape(n, k)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_repack_rejects_bad_sizes():
+    with pytest.raises(rlx_amd.RlxError):
+        ops.repack_host(Q4_0, np.zeros(18, np.uint8), 1, 33)
+    with pytest.raises(rlx_amd.RlxError):
+        ops.repack_host(Q4_0, np.zeros(17, np.uint8), 1, 32)
+    with pytest.raises(rlx_amd.RlxError) as ei:
+        ops.repack_host(Q4K, np.zeros(144, np.uint8), 1, 128)
+    assert "multiple" in str(ei.value)
+
+
+# ---- encoders: no reference exists (rlx-gguf is decode-only), so they are pinned by properties only ----
+
+def test_encoder_q8_0_properties(oracle):
+    packed, w = make_weights(Q8_0, 8, 256, seed=1)
+    deq = oracle.dequant(Q8_0, packed, w.size).reshape(w.shape)
+    d = packed.reshape(-1, 34)[:, :2].copy().view(np.float16).astype(np.float32).reshape(8, 8)
+    err = np.abs(deq - w).reshape(8, 8, 32).max(axis=2)
+    assert np.all(err <= d * (0.5 + 127 * 2.0 ** -11) + 1e-9)  # half a step plus the f16 rounding of d times the code
+    codes = packed.reshape(-1, 34)[:, 2:].view(np.int8)
+    assert np.all(np.abs(codes.astype(int)).max(axis=1) == 127)  # block max hits +-127
+    assert np.array_equal(ops.quantize(Q8_0, np.zeros(64, np.float32)).reshape(2, 34)[:, 2:], np.zeros((2, 32), np.uint8))
+
+
+def test_encoder_q4_0_properties(oracle):
+    packed, w = make_weights(Q4_0, 8, 256, seed=2)
+    deq = oracle.dequant(Q4_0, packed, w.size).reshape(w.shape)
+    d = np.abs(packed.reshape(-1, 18)[:, :2].copy().view(np.float16).astype(np.float32)).reshape(8, 8)
+    err = np.abs(deq - w).reshape(8, 8, 32).max(axis=2)
+    assert np.all(err <= d * (1.0 + 8 * 2.0 ** -11) + 1e-9)
+    assert len(np.unique(packed.reshape(-1, 18)[:, 2:] & 0xF)) == 16   # all codes used
+    # the element of largest magnitude maps to code 0 (value -8 d)
+    b0 = w.reshape(-1, 32)[0]
+    i = int(np.argmax(np.abs(b0)))
+    q = packed.reshape(-1, 18)[0, 2 + (i % 16)]
+    assert ((q & 0xF) if i < 16 else (q >> 4)) == 0
+
+
+def test_encoder_q4_k_properties(oracle):
+    rng = np.random.default_rng(3)
+    w = (rng.standard_normal((4, 512)) * 0.02).astype(np.float32)
+    w[0, :32] += 0.05      # shifted sub-block: exercises the min term
+    w[1, 128:160] *= 8.0   # large sub-block: exercises 6-bit scale high bits (j >= 4)
+    packed = ops.quantize(Q4K, w)
+    deq = oracle.dequant(Q4K, packed, w.size).reshape(w.shape)
+    blocks = packed.reshape(-1, 144)
+    scs = np.array([[oracle.get_scale_min_k4(j, b[4:16]) for j in range(8)] for b in blocks])
+    assert scs.max() <= 63 and scs[:, :, 0].max() >= 32 and scs[:, 4:, :].max() >= 16  # high bits of the j>=4 fields used
+    d = blocks[:, 0:2].copy().view(np.float16).astype(np.float32).reshape(-1)
+    step = (d[:, None] * scs[:, :, 0]).reshape(4, 2, 8)
+    err = np.abs(deq - w).reshape(4, 2, 8, 32).max(axis=3)
+    dmin = blocks[:, 2:4].copy().view(np.float16).astype(np.float32).reshape(4, 2, 1)
+    assert np.all(err <= step * 0.5 + dmin * 0.5 + d.reshape(4, 2, 1) * 8 + 1e-7)
+    assert np.sqrt(np.mean((deq - w) ** 2)) < 0.1 * np.sqrt(np.mean(w ** 2))
+
+
+def test_philox_matches_oracle(oracle):
+    for seed in (0, 7, 0x123456789ABCDEF):
+        assert np.array_equal(ops.philox_u32(seed, 1000), oracle.philox_u32(seed, 1000))
+        assert np.array_equal(ops.philox_uniform(seed, 1000), oracle.philox_uniform(seed, 1000))
+    a, b = ops.philox_normal(42, 4096), oracle.philox_normal(42, 4096)
+    assert np.allclose(a, b, rtol=0, atol=1e-6)  # same libm here; last-ulp parity with Rust std is unpinned
+
+
+# ---- graph validation (no device needed: errors are found before any HIP call) ----
+
+def dq_graph(m, k, n, scheme, nbytes=None, wdtype=DType.U8):
+    g = Graph.new("t")
+    x = g.input("x", Shape.new([m, k], DType.F32))
+    nb = QuantScheme(scheme).gguf_block_bytes() * (k * n // QuantScheme(scheme).gguf_block_size()) if nbytes is None else nbytes
+    w = g.param("w_packed", Shape.new([nb], wdtype))
+    y = g.add_node(Op.DequantMatMul(QuantScheme(scheme)), [x, w], Shape.new([m, n], DType.F32))
+    g.set_outputs([y])
+    return g
+
+
+def compile_error(g):
+    with pytest.raises(rlx_amd.RlxError) as ei:
+        Session.new().compile(g)
+    return str(ei.value)
+
+
+def test_supported_ops():
+    assert [int(k) for k in rlx_amd.supported_ops()] == [0, 1, 2, 3]
+
+
+def test_compile_rejects_wrong_weight_size():
+    assert "packed weight must be a U8 param" in compile_error(dq_graph(2, 256, 4, Q4K, nbytes=100))
+
+
+def test_compile_rejects_unclaimed_scheme():
+    g = dq_graph(1, 256, 1, Q4K)
+    g.nodes[2] = type(g.nodes[2])(2, Op.DequantMatMul(QuantScheme.GgufQ6K), g.nodes[2].inputs, g.nodes[2].shape)
+    assert "not claimed" in compile_error(g)
+
+
+def test_compile_rejects_unknown_op_kind_with_legalize_message():
+    g = dq_graph(1, 256, 1, Q4K)
+    desc, keep = rlx_amd.runtime._graph_desc(g)
+    desc.nodes[2].op_kind = 77
+    import ctypes as C
+    h = rlx_amd._lib.lib().rlx_mi355x_compile(C.byref(desc), None)
+    assert not h
+    assert "doesn't claim support for 1 op kind(s)" in rlx_amd._lib.last_error()
+
+
+def test_compile_rejects_bad_fake_quantize():
+    g = Graph.new("fq")
+    x = g.input("x", Shape.new([3, 4], DType.F32))
+    q = g.add_node(Op.FakeQuantize(3, 0), [x], Shape.new([3, 4], DType.F32))
+    g.set_outputs([q])
+    assert "unsupported bits 3" in compile_error(g)
+    g = Graph.new("fq")
+    x = g.input("x", Shape.new([3, 4], DType.F32))
+    q = g.add_node(Op.FakeQuantize(8, 0, scale_mode=ScaleMode.Fixed), [x], Shape.new([3, 4], DType.F32))
+    g.set_outputs([q])
+    assert "state" in compile_error(g) or "input" in compile_error(g)
+    g = Graph.new("fq")
+    x = g.input("x", Shape.new([3, 4], DType.F32))
+    q = g.add_node(Op.FakeQuantize(8, 2), [x], Shape.new([3, 4], DType.F32))
+    g.set_outputs([q])
+    assert "axis" in compile_error(g)
+
+
+def test_compile_without_device_fails_loudly():
+    if rlx_amd.is_available():
+        pytest.skip("a GPU is present")
+    msg = compile_error(dq_graph(2, 256, 4, Q4K))
+    assert "no HIP device" in msg or "gfx950" in msg
+    with pytest.raises(rlx_amd.RlxError):
+        ops.DeviceBuffer(16)
