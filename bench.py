@@ -1,0 +1,267 @@
+#!/usr/bin/env python3
+"""Headline benchmark: Q4_0 decode GEMV (batch 1) over the seven Llama-3-8B layer projections on one MI355X.
+
+A step is one pass over one layer's seven projections (q, k, v, o, gate, up, down): seven DequantMatMul nodes of one
+compiled graph wired like the real layer (q/k/v read one activation vector, gate/up another, o and down their own),
+so the backend fuses them into four launches (qkv, o, gate+up, down), replayed as a hipGraph. The layers rotate through LAYERS distinct weight sets (~123 MB each), far
+more than the 256 MB of last-level cache, so every launch streams its weights from HBM. Inputs and weights are
+resident in HBM before the timed region. One JSON line is printed; `value` is algorithmic bytes per second
+(packed weights + f32 activations in + f32 outputs out), the figure the roofline fraction is taken from.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--no-cpu] [--extra]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0       # MI355X published HBM3E bandwidth
+MFMA_F16_PEAK_TFLOPS = 2500.0  # dense f16/bf16 MFMA peak
+
+# (name, N, K) — BASELINE config 2
+LLAMA8B = [("q", 4096, 4096), ("k", 1024, 4096), ("v", 1024, 4096), ("o", 4096, 4096),
+           ("gate", 14336, 4096), ("up", 14336, 4096), ("down", 4096, 14336)]
+
+
+# which activation vector each projection reads (the layer's real data flow)
+X_OF = {"q": "x_attn", "k": "x_attn", "v": "x_attn", "o": "x_o", "gate": "x_mlp", "up": "x_mlp", "down": "x_down"}
+LAUNCHES_PER_STEP = 4  # qkv, o, gate+up, down
+
+
+def gemv_bytes(n, k, scheme_bytes_per_block=18, block=32, m=1):
+    return n * k // block * scheme_bytes_per_block + 4 * k * m + 4 * n * m
+
+
+def build_layer_graph(rlx, li):
+    from rlx_amd import DType, Graph, Op, QuantScheme, Shape
+
+    g = Graph.new(f"llama8b_layer{li}")
+    outs, xin = [], {}
+    for name, n, k in LLAMA8B:
+        src = X_OF[name]
+        if src not in xin:
+            xin[src] = g.input(src, Shape.new([1, k], DType.F32))
+        w = g.param(f"w_{name}", Shape.new([n * k // 32 * 18], DType.U8))
+        outs.append(g.add_node(Op.DequantMatMul(QuantScheme.GgufQ4_0), [xin[src], w], Shape.new([1, n], DType.F32)))
+    g.set_outputs(outs)
+    return g
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--layers", type=int, default=8, help="distinct weight sets rotated through (8 x 123 MB)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-graph", action="store_true", help="launch kernels one by one instead of replaying a hipGraph")
+    ap.add_argument("--extra", action="store_true", help="also time the other BASELINE configs (reported under 'extra')")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import rlx_amd
+    from rlx_amd import DType, QuantScheme, Session, ops
+
+    if not rlx_amd.is_available():
+        print("bench.py: no MI355X or the HIP library failed to load: " + rlx_amd._lib.last_error(), file=sys.stderr)
+        sys.exit(1)
+    info = ops.device_info()
+
+    # ---- synthetic weights / activations (seeded), quantized by the library's Q4_0 encoder ----
+    t0 = time.time()
+    base = {}
+    for name, n, k in LLAMA8B:
+        w = (ops.philox_normal(1000 + len(base), n * k) * np.float32(0.02)).astype(np.float32)
+        base[name] = ops.quantize(QuantScheme.GgufQ4_0, w).reshape(n, -1)
+    xsrc = {src: ops.philox_normal(2000 + i, 14336 if src == "x_down" else 4096)
+            for i, src in enumerate(sorted(set(X_OF.values())))}
+    xs = {name: xsrc[X_OF[name]] for name, _, _ in LLAMA8B}
+    layers = []
+    stream = rlx_amd._lib.C.c_void_p()
+    rlx_amd._lib.check(rlx_amd._lib.lib().rlx_mi355x_stream_create(rlx_amd._lib.C.byref(stream)))
+    for li in range(args.layers):
+        c = Session.new(rlx_amd.Device.Mi355x).compile(build_layer_graph(rlx_amd, li))
+        for name, n, k in LLAMA8B:
+            # distinct bytes per layer: rotate the rows of the base matrix (same statistics, different memory)
+            c.set_param_typed(f"w_{name}", np.roll(base[name], 37 * li, axis=0).reshape(-1), DType.U8)
+        for src, v in xsrc.items():
+            c.write_input(src, v)
+        c.sync()
+        c.set_stream(stream)
+        if not args.no_graph:
+            c.capture()
+        layers.append(c)
+    setup_s = time.time() - t0
+
+    layer_bytes = sum(gemv_bytes(n, k) for _, n, k in LLAMA8B)
+    launches_per_step = LAUNCHES_PER_STEP
+
+    def run_steps(count, offset=0):
+        seq = [layers[(offset + i) % len(layers)] for i in range(count)]
+        rlx_amd.launch_sequence(seq)
+
+    run_steps(args.warmup)
+    ops.sync(stream)
+    ev0, ev1 = ops.Event(), ops.Event()
+    ev0.record(stream)
+    run_steps(args.steps, args.warmup)
+    ev1.record(stream)
+    ms = ev0.elapsed_ms(ev1)
+    ops.sync(stream)
+    ms_per_step = ms / args.steps
+    gbs = layer_bytes / (ms_per_step * 1e-3) / 1e9
+    us_per_launch = ms_per_step * 1e3 / launches_per_step
+
+    # parity spot check of what was just timed (not in the timed region)
+    import oracle
+    y = layers[1].read_output(4)
+    packed1 = np.roll(base["gate"], 37, axis=0).reshape(-1)
+    ref = oracle.gguf_matmul_f64(xs["gate"], packed1, 1, 4096, 14336, oracle.Q4_0, 0, 512)
+    parity = float(np.max(np.abs(y[:512] - ref[0]) / np.maximum(np.abs(ref[0]), 1.0)))
+
+    result = {
+        "metric": "Q4_0 GEMV HBM GB/s (% of 8 TB/s peak); Q4_K GEMM M=512 TFLOP/s (% MFMA)",
+        "value": round(gbs, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 6),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "u4 codes x f16 scale, f32 accumulate",
+        "data": "synthetic",
+        "config": {"workload": "Q4_0 decode GEMV, batch 1, seven Llama-3-8B layer projections per step "
+                               "(q,k,v,o,gate,up,down), f32 activations, weights ~N(0,0.02)",
+                   "layers_rotated": args.layers, "hip_graph": not args.no_graph,
+                   "algorithmic_bytes_per_step": layer_bytes, "launches_per_step": launches_per_step},
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "rlx_gemv_q4_0_r2", "avg_launch_us": round(us_per_launch, 3),
+                     "algorithmic_bytes_per_launch": layer_bytes // launches_per_step},
+        "parity_max_rel_err": parity,
+        "device": info,
+        "setup_s": round(setup_s, 1),
+    }
+
+    if args.extra:
+        result["extra"] = extra_configs(rlx_amd, stream)
+
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(base, xs)
+    print(json.dumps(result), flush=True)
+
+
+def time_launches(ops, stream, fn, reps, warm):
+    for _ in range(warm):
+        fn()
+    ops.sync(stream)
+    e0, e1 = ops.Event(), ops.Event()
+    e0.record(stream)
+    for _ in range(reps):
+        fn()
+    e1.record(stream)
+    ms = e0.elapsed_ms(e1)
+    return ms / reps
+
+
+def extra_configs(rlx_amd, stream):
+    """Other BASELINE configs, each as back-to-back launches on rotating buffers (reported, not the headline)."""
+    from rlx_amd import DType, QuantScheme, ops
+    L = rlx_amd._lib.lib()
+    out = {}
+    # per-projection Q4_0 GEMV, cold (rotating over >= 512 MB of weights)
+    for name, n, k in [("q/o", 4096, 4096), ("k/v", 1024, 4096), ("gate/up", 14336, 4096), ("down", 4096, 14336)]:
+        wbytes = n * k // 32 * 18
+        copies = max(2, int(600e6 // wbytes) + 1)
+        w = (ops.philox_normal(5, n * k) * np.float32(0.02)).astype(np.float32)
+        packed = ops.quantize(QuantScheme.GgufQ4_0, w).reshape(n, -1)
+        qws = [ops.QWeight(QuantScheme.GgufQ4_0, np.roll(packed, i, axis=0).reshape(-1), n, k) for i in range(copies)]
+        x = ops.DeviceBuffer.from_numpy(ops.philox_normal(6, k))
+        y = ops.DeviceBuffer(n * 4)
+        state = {"i": 0}
+
+        def fn():
+            q = qws[state["i"] % copies]
+            state["i"] += 1
+            rlx_amd._lib.check(L.rlx_mi355x_gguf_matmul_bt(x.ptr, int(DType.F32), q.ptr, y.ptr, 1, None, 0, stream))
+
+        ms = time_launches(ops, stream, fn, 400, 50)
+        b = gemv_bytes(n, k)
+        out[f"q4_0_gemv_{name}"] = {"us": round(ms * 1e3, 3), "GB/s": round(b / ms / 1e6, 1),
+                                    "frac_hbm": round(b / ms / 1e6 / HBM_PEAK_GBS, 4), "copies": copies}
+        for q in qws:
+            q.free()
+    # config 1: Q8_0 GEMV 4096x4096
+    n = k = 4096
+    w = (ops.philox_normal(7, n * k) * np.float32(0.02)).astype(np.float32)
+    packed = ops.quantize(QuantScheme.GgufQ8_0, w).reshape(n, -1)
+    copies = 34
+    qws = [ops.QWeight(QuantScheme.GgufQ8_0, np.roll(packed, i, axis=0).reshape(-1), n, k) for i in range(copies)]
+    x = ops.DeviceBuffer.from_numpy(ops.philox_normal(8, k))
+    y = ops.DeviceBuffer(n * 4)
+    state = {"i": 0}
+
+    def fn8():
+        q = qws[state["i"] % copies]
+        state["i"] += 1
+        rlx_amd._lib.check(L.rlx_mi355x_gguf_matmul_bt(x.ptr, int(DType.F32), q.ptr, y.ptr, 1, None, 0, stream))
+
+    ms = time_launches(ops, stream, fn8, 400, 50)
+    b = gemv_bytes(n, k, 34)
+    out["q8_0_gemv_4096x4096"] = {"us": round(ms * 1e3, 3), "GB/s": round(b / ms / 1e6, 1),
+                                  "frac_hbm": round(b / ms / 1e6 / HBM_PEAK_GBS, 4)}
+    for q in qws:
+        q.free()
+    # config 4: FakeQuantize [8192, 4096], int8 per column
+    rows, cols = 8192, 4096
+    xq = ops.philox_normal(9, rows * cols)
+    xd = ops.DeviceBuffer.from_numpy(xq)
+    od = ops.DeviceBuffer(rows * cols * 4)
+    scratch = ops.DeviceBuffer(cols * 8)
+
+    def fq():
+        rlx_amd._lib.check(L.rlx_mi355x_fake_quantize(xd.ptr, od.ptr, None, rows * cols, cols, 1, 8, 0, 0.0, None, 0,
+                                                      scratch.ptr, stream))
+
+    ms = time_launches(ops, stream, fq, 50, 5)
+    b = 2 * rows * cols * 4
+    out["fake_quantize_8192x4096_cols"] = {"us": round(ms * 1e3, 2), "GB/s_1R1W": round(b / ms / 1e6, 1),
+                                           "frac_hbm_1R1W": round(b / ms / 1e6 / HBM_PEAK_GBS, 4),
+                                           "GB/s_2R1W": round(1.5 * b / ms / 1e6, 1)}
+    return out
+
+
+def cpu_baseline(base, xs):
+    """The reference CPU path (oracle restatement of rlx-cpu gguf_matmul_bt: scalar, one thread) on this box's host
+    cores, over the same seven projections, for about 10 s."""
+    import oracle
+
+    t_end = time.time() + 10.0
+    reps, spent = 0, 0.0
+    while True:
+        t0 = time.time()
+        for name, n, k in LLAMA8B:
+            oracle.gguf_matmul_bt(xs[name], base[name].reshape(-1), 1, k, n, oracle.Q4_0)
+        spent += time.time() - t0
+        reps += 1
+        if time.time() > t_end or reps >= 50:
+            break
+    layer_bytes = sum(gemv_bytes(n, k) for _, n, k in LLAMA8B)
+    return {"value": round(layer_bytes * reps / spent / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"{reps} pass(es) over the same seven Q4_0 projections of one layer, {spent:.1f} s, "
+                      f"C restatement of rlx-cpu gguf_matmul_bt (scalar, single thread, as the reference runs it)",
+            "host_cpus": os.cpu_count()}
+
+
+if __name__ == "__main__":
+    main()

@@ -133,6 +133,12 @@ int rlx_mi355x_dequant(const rlx_qweight *w, float *out_dev, void *stream);
 int rlx_mi355x_gguf_matmul_bt(const void *x_dev, int x_dtype, const rlx_qweight *w, float *out_dev, int64_t m,
                               void *workspace, size_t workspace_bytes, void *stream);
 size_t rlx_mi355x_gguf_matmul_workspace(int scheme, int x_dtype, int64_t m, int64_t k, int64_t n);
+/* `count` matmuls that share the activations, the scheme and k (q/k/v or gate/up of one layer) in one launch per
+ * four weights: outs_dev[i][m, n_i] = x . W_i^T. No counterpart in the reference, which runs one thunk per node; the
+ * graph level uses it to fuse DequantMatMul nodes that read the same input. */
+int rlx_mi355x_gguf_matmul_bt_grouped(const void *x_dev, int x_dtype, const rlx_qweight *const *ws,
+                                      float *const *outs_dev, int count, int64_t m, void *workspace,
+                                      size_t workspace_bytes, void *stream);
 
 /* Thunk::FakeQuantize (rlx-cpu/src/thunk.rs:11159-11253) with the layout of quant_layout()
  * (thunk.rs:14163-14175): channel of flat element i is (i / inner) % chan_dim.
@@ -256,6 +262,16 @@ int rlx_exec_write_input(rlx_exec *e, const char *name, const void *data, size_t
 int rlx_exec_launch(rlx_exec *e);
 int rlx_exec_sync(rlx_exec *e);
 void *rlx_exec_stream(rlx_exec *e);
+/* Run on a caller-owned stream from now on (several executables can share one; the executable's own stream
+ * is kept but unused). Drops a captured graph. */
+int rlx_exec_set_stream(rlx_exec *e, void *stream);
+/* Record the schedule once into a hipGraph (stream capture of the same kernel launches; fills are kernels, never
+ * memset nodes); rlx_exec_launch then replays it with one hipGraphLaunch. The reference's ROCm backend does the
+ * same for its Step list (rlx-rocm/src/backend.rs:1501-1537). Re-capture after changing an input's dtype. */
+int rlx_exec_capture(rlx_exec *e);
+/* commit_no_wait for a whole batch (rlx-runtime/src/backend.rs:275-293): enqueue each executable once, in order,
+ * without returning to the caller in between. All must share a stream for the order to mean anything. */
+int rlx_mi355x_launch_sequence(rlx_exec *const *execs, size_t n);
 
 /* MemoryPlan{arena_size, assignments} (rlx-compile/src/memory.rs:76-94) as planned for this executable,
  * including the persistent repacked-weight slots. Writes a short text table. */

@@ -5,7 +5,7 @@ the thin host-side mirror of the reference's Session / Graph surface used by tes
 from . import _lib, ops
 from ._lib import RlxError, build
 from .ir import DType, Graph, Op, OpKind, QuantScheme, RoundMode, ScaleMode, Shape, SteKind
-from .runtime import CompiledGraph, Device, Session, is_available, supported_ops
+from .runtime import CompiledGraph, Device, Session, is_available, launch_sequence, supported_ops
 
 __all__ = ["_lib", "ops", "RlxError", "build", "DType", "Graph", "Op", "OpKind", "QuantScheme", "RoundMode", "ScaleMode",
-           "Shape", "SteKind", "CompiledGraph", "Device", "Session", "is_available", "supported_ops"]
+           "Shape", "SteKind", "CompiledGraph", "Device", "Session", "is_available", "launch_sequence", "supported_ops"]

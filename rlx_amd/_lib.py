@@ -76,6 +76,7 @@ SIGNATURES = {
     "rlx_mi355x_dequant": (_i, [_vp, _vp, _vp]),
     "rlx_mi355x_gguf_matmul_bt": (_i, [_vp, _i, _vp, _vp, _i64, _vp, _sz, _vp]),
     "rlx_mi355x_gguf_matmul_workspace": (_sz, [_i, _i, _i64, _i64, _i64]),
+    "rlx_mi355x_gguf_matmul_bt_grouped": (_i, [_vp, _i, _pvp, _pvp, _i, _i64, _vp, _sz, _vp]),
     "rlx_mi355x_fake_quantize": (_i, [_vp, _vp, _vp, _i64, _i64, _i64, _i, _i, _f, _vp, _i, _vp, _vp]),
     "rlx_mi355x_quantize": (_i, [_i, _vp, _i64, _vp]),
     "rlx_mi355x_philox_u32": (None, [C.c_uint64, _vp, _i64]),
@@ -94,6 +95,9 @@ SIGNATURES = {
     "rlx_exec_launch": (_i, [_vp]),
     "rlx_exec_sync": (_i, [_vp]),
     "rlx_exec_stream": (_vp, [_vp]),
+    "rlx_exec_set_stream": (_i, [_vp, _vp]),
+    "rlx_exec_capture": (_i, [_vp]),
+    "rlx_mi355x_launch_sequence": (_i, [_pvp, _sz]),
     "rlx_exec_arena_bytes": (_sz, [_vp]),
     "rlx_exec_describe_plan": (_i, [_vp, C.c_char_p, _sz]),
     "rlx_exec_read_fq_codes": (_i, [_vp, _u32, _vp, _sz]),

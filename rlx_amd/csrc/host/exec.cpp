@@ -15,8 +15,12 @@
 #include "common.hpp"
 
 struct rlx_qweight;
+extern "C" int rlx_mi355x_fake_quantize(const float *, float *, int8_t *, int64_t, int64_t, int64_t, int, int, float, float *, int,
+                                        void *, void *);
 extern "C" int rlx_mi355x_qweight_create_at(int, const void *, size_t, int64_t, int64_t, void *, rlx_qweight **);
 extern "C" void rlx_mi355x_qweight_destroy(rlx_qweight *);
+extern "C" int rlx_mi355x_gguf_matmul_bt_grouped(const void *, int, const rlx_qweight *const *, float *const *, int, int64_t,
+                                                 void *, size_t, void *);
 
 namespace {
 
@@ -96,16 +100,30 @@ struct rlx_exec {
     std::vector<Node> nodes;
     std::vector<uint32_t> outputs;
     std::map<std::string, uint32_t> inputs, params;
+    // Launch schedule: one entry per kernel group. DequantMatMul nodes that read the same activations with the
+    // same scheme and k (q/k/v, gate/up) are fused into one grouped launch at the position of the first of them;
+    // they depend only on that input and on params, so moving the later ones up is safe.
+    std::vector<std::vector<uint32_t>> steps;
     rlx_compile_opts opts{};
     size_t arena_bytes = 0;
     uint8_t *arena = nullptr;
-    hipStream_t stream = nullptr;
+    hipStream_t stream = nullptr;      // the stream work is enqueued on
+    hipStream_t own_stream = nullptr;  // created at compile time
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t graph_exec = nullptr;
 
     ~rlx_exec() {
         for (auto &nd : nodes)
             if (nd.qw) rlx_mi355x_qweight_destroy(nd.qw);
+        drop_graph();
         if (arena) (void)hipFree(arena);
-        if (stream) (void)hipStreamDestroy(stream);
+        if (own_stream) (void)hipStreamDestroy(own_stream);
+    }
+    void drop_graph() {
+        if (graph_exec) (void)hipGraphExecDestroy(graph_exec);
+        if (graph) (void)hipGraphDestroy(graph);
+        graph_exec = nullptr;
+        graph = nullptr;
     }
     void *ptr(const Slot &s) const { return arena + s.offset; }
 };
@@ -285,6 +303,24 @@ rlx_exec *rlx_mi355x_compile(const rlx_graph_desc *g, const rlx_compile_opts *op
         }
     }
 
+    std::vector<bool> grouped(e->nodes.size(), false);
+    for (uint32_t i = 0; i < g->n_nodes; i++) {
+        Node &nd = e->nodes[i];
+        if (grouped[i] || (nd.d.op_kind != RLX_OP_DEQUANT_MATMUL && nd.d.op_kind != RLX_OP_FAKE_QUANTIZE)) continue;
+        std::vector<uint32_t> step{i};
+        if (nd.d.op_kind == RLX_OP_DEQUANT_MATMUL) {
+            for (uint32_t j = i + 1; j < g->n_nodes; j++) {
+                Node &o = e->nodes[j];
+                if (!grouped[j] && o.d.op_kind == RLX_OP_DEQUANT_MATMUL && o.d.inputs[0] == nd.d.inputs[0] &&
+                    o.d.scheme == nd.d.scheme && o.k == nd.k && o.m == nd.m) {
+                    grouped[j] = true;
+                    step.push_back(j);
+                }
+            }
+        }
+        e->steps.push_back(step);
+    }
+
     // Memory plan.
     size_t off = 0;
     auto take = [&](size_t bytes) {
@@ -315,10 +351,11 @@ rlx_exec *rlx_mi355x_compile(const rlx_graph_desc *g, const rlx_compile_opts *op
         set_error("compile: hipMalloc(%zu) for the arena failed", off);
         return nullptr;
     }
-    if (hipMemset(e->arena, 0, std::max<size_t>(off, 256)) != hipSuccess || hipStreamCreate(&e->stream) != hipSuccess) {
+    if (hipMemset(e->arena, 0, std::max<size_t>(off, 256)) != hipSuccess || hipStreamCreate(&e->own_stream) != hipSuccess) {
         set_error("compile: arena clear / stream creation failed");
         return nullptr;
     }
+    e->stream = e->own_stream;
     if (e->opts.verbose) {
         char buf[4096];
         rlx_exec_describe_plan(e.get(), buf, sizeof buf);
@@ -407,27 +444,31 @@ int rlx_exec_write_input(rlx_exec *e, const char *name, const void *data, size_t
         return RLX_ERR_INVALID;
     }
     RLX_HIP(hipMemcpyAsync(e->ptr(nd.slot), data, nbytes, hipMemcpyHostToDevice, e->stream));
+    if (nd.cur_dtype != dtype) e->drop_graph();  // the captured launches were specialised on the old dtype
     nd.cur_dtype = dtype;
     return RLX_OK;
 }
 
-int rlx_exec_launch(rlx_exec *e) {
-    if (!e) {
-        set_error("launch: null executable");
-        return RLX_ERR_INVALID;
-    }
-    for (Node &nd : e->nodes) {
+static int enqueue_schedule(rlx_exec *e) {
+    for (const std::vector<uint32_t> &step : e->steps) {
+        Node &nd = e->nodes[step[0]];
         if (nd.d.op_kind == RLX_OP_DEQUANT_MATMUL) {
             Node &x = e->nodes[nd.d.inputs[0]];
-            Node &w = e->nodes[nd.d.inputs[1]];
-            if (!w.qw) {
-                set_error("run: packed weight '%s' was never set (set_param_typed(.., U8))", w.name.c_str());
-                return RLX_ERR_INVALID;
+            std::vector<const rlx_qweight *> ws;
+            std::vector<float *> outs;
+            for (uint32_t id : step) {
+                Node &w = e->nodes[e->nodes[id].d.inputs[1]];
+                if (!w.qw) {
+                    set_error("run: packed weight '%s' was never set (set_param_typed(.., U8))", w.name.c_str());
+                    return RLX_ERR_INVALID;
+                }
+                ws.push_back(w.qw);
+                outs.push_back((float *)e->ptr(e->nodes[id].slot));
             }
             uint32_t xdt = x.d.op_kind == RLX_OP_INPUT ? x.cur_dtype : x.d.dtype;
-            RLX_TRY(rlx_mi355x_gguf_matmul_bt(e->ptr(x.slot), (int)xdt, w.qw, (float *)e->ptr(nd.slot), nd.m, nullptr, 0,
-                                              e->stream));
-        } else if (nd.d.op_kind == RLX_OP_FAKE_QUANTIZE) {
+            RLX_TRY(rlx_mi355x_gguf_matmul_bt_grouped(e->ptr(x.slot), (int)xdt, ws.data(), outs.data(), (int)ws.size(), nd.m,
+                                                      nullptr, 0, e->stream));
+        } else {
             Node &x = e->nodes[nd.d.inputs[0]];
             if (x.d.op_kind == RLX_OP_INPUT && x.cur_dtype != RLX_F32) {
                 set_error("run: FakeQuantize input '%s' must be written as F32", x.name.c_str());
@@ -440,6 +481,56 @@ int rlx_exec_launch(rlx_exec *e) {
                                              e->ptr(nd.aux), e->stream));
         }
     }
+    return RLX_OK;
+}
+
+int rlx_exec_launch(rlx_exec *e) {
+    if (!e) {
+        set_error("launch: null executable");
+        return RLX_ERR_INVALID;
+    }
+    if (e->graph_exec) {
+        RLX_HIP(hipGraphLaunch(e->graph_exec, e->stream));
+        return RLX_OK;
+    }
+    return enqueue_schedule(e);
+}
+
+int rlx_exec_set_stream(rlx_exec *e, void *stream) {
+    if (!e) return RLX_ERR_INVALID;
+    e->drop_graph();
+    e->stream = stream ? (hipStream_t)stream : e->own_stream;
+    return RLX_OK;
+}
+
+int rlx_exec_capture(rlx_exec *e) {
+    if (!e) return RLX_ERR_INVALID;
+    e->drop_graph();
+    RLX_TRY(runtime_init());
+    RLX_HIP(hipStreamSynchronize(e->stream));
+    RLX_HIP(hipStreamBeginCapture(e->stream, hipStreamCaptureModeThreadLocal));
+    int rc = enqueue_schedule(e);
+    hipError_t ce = hipStreamEndCapture(e->stream, &e->graph);
+    if (rc < 0) {
+        e->drop_graph();
+        return rc;
+    }
+    if (ce != hipSuccess) {
+        set_error("hipStreamEndCapture: %s", hipGetErrorString(ce));
+        e->graph = nullptr;
+        return RLX_ERR_HIP;
+    }
+    hipError_t ie = hipGraphInstantiate(&e->graph_exec, e->graph, nullptr, nullptr, 0);
+    if (ie != hipSuccess) {
+        set_error("hipGraphInstantiate: %s", hipGetErrorString(ie));
+        e->drop_graph();
+        return RLX_ERR_HIP;
+    }
+    return RLX_OK;
+}
+
+int rlx_mi355x_launch_sequence(rlx_exec *const *execs, size_t n) {
+    for (size_t i = 0; i < n; i++) RLX_TRY(rlx_exec_launch(execs[i]));
     return RLX_OK;
 }
 

@@ -24,11 +24,16 @@ struct DequantArgs {
     float *out;
     long long n, k, units;
 };
-struct GemvArgs {
+constexpr int GEMV_MAX_SEG = 4;
+struct GemvSeg {
     const uint8_t *w;
-    const void *x;
     float *out;
-    int m, k, n, units, row_tiles, kc_units, x_dtype;
+    int n, row_tiles, wg_begin, pad;
+};
+struct GemvArgs {
+    GemvSeg seg[GEMV_MAX_SEG];
+    const void *x;
+    int nseg, m, k, units, kc_units, x_dtype, tiles_per_wg;
 };
 struct FqArgs {
     const float *x;
@@ -51,43 +56,57 @@ static int x_kind(int x_dtype) {
     }
 }
 
-static int launch_gemv(const void *x, int xk, const rlx_qweight *w, float *out, int m, hipStream_t stream) {
-    const Layout L = layout_of(w->scheme);
+// One decode launch over `count` (<= 4) weights that share scheme, k and the activations.
+static int launch_gemv(const void *x, int xk, const rlx_qweight *const *ws, float *const *outs, int count, int m,
+                       hipStream_t stream) {
+    const rlx_qweight *w0 = ws[0];
+    const Layout L = layout_of(w0->scheme);
     const int rv = xk == 0 ? 2 * m : m;
-    const int units = (int)w->dims.units, tiles = (int)w->dims.row_tiles;
+    const int ng = (rv + 3) / 4;
+    const int units = (int)w0->dims.units;
     const bool r2 = rv <= 2;
-    // Row tiles per workgroup: one, unless N is large enough that two or four still leave >= 512 workgroups.
-    const int max_rtw = w->scheme == SCHEME_Q4_0 ? (r2 ? 2 : 4) : (r2 ? 1 : 2);
-    int rtw = 1;
-    while (rtw * 2 <= max_rtw && tiles / (rtw * 2) >= 512) rtw *= 2;
-    KernelId id;
-    if (w->scheme == SCHEME_Q4_0)
-        id = r2 ? (rtw == 2 ? K_GEMV_Q4_0_T2_R2 : K_GEMV_Q4_0_T1_R2)
-                : (rtw == 4 ? K_GEMV_Q4_0_T4_R4 : rtw == 2 ? K_GEMV_Q4_0_T2_R4 : K_GEMV_Q4_0_T1_R4);
-    else if (w->scheme == SCHEME_Q8_0)
-        id = r2 ? K_GEMV_Q8_0_T1_R2 : (rtw == 2 ? K_GEMV_Q8_0_T2_R4 : K_GEMV_Q8_0_T1_R4);
-    else
-        id = r2 ? K_GEMV_Q4_K_T1_R2 : (rtw == 2 ? K_GEMV_Q4_K_T2_R4 : K_GEMV_Q4_K_T1_R4);
-
-    // LDS: the staged activation chunk (rv rows of halfs, 16 B row padding) plus, for Q4_K, the per-block sums.
-    const size_t budget = 48 * 1024;
+    KernelId id = w0->scheme == SCHEME_Q4_0   ? (r2 ? K_GEMV_Q4_0_R2 : K_GEMV_Q4_0_R4)
+                  : w0->scheme == SCHEME_Q8_0 ? (r2 ? K_GEMV_Q8_0_R2 : K_GEMV_Q8_0_R4)
+                                              : (r2 ? K_GEMV_Q4_K_R2 : K_GEMV_Q4_K_R4);
+    const int nwaves = std::max(1, std::min(8, units));
+    long long total_tiles = 0;
+    for (int i = 0; i < count; i++) total_tiles += ws[i]->dims.row_tiles;
+    // Row tiles per workgroup: the fewest that keep the grid within two workgroups per CU, so every workgroup is
+    // resident at once and the activations are staged once per ~36 KB x tiles of weights.
+    const int cus = std::max(1, device_props().cu_count);
+    int tpw = (int)std::max<long long>(1, (total_tiles + 2 * cus - 1) / (2 * cus));
+    const size_t slot_bytes = (size_t)ng * 256;
+    tpw = (int)std::min<size_t>(tpw, std::max<size_t>(1, (32 * 1024) / (nwaves * slot_bytes)));
+    const size_t part_bytes = (size_t)tpw * nwaves * slot_bytes;
+    // LDS: partial sums + the staged activation chunk (rv rows of halfs, 16 B row padding) + Q4_K block sums.
+    const size_t budget = 64 * 1024;
     auto stage_bytes = [&](int kcu) {
-        size_t b = ((size_t)rv * ((size_t)kcu * L.unit_k + 8) * 2 + 15) & ~(size_t)15;
-        if (w->scheme == SCHEME_Q4K) b += (size_t)kcu * (L.unit_k / 32) * 16 * 4;
+        size_t b = ((size_t)(rv + 1) * ((size_t)kcu * L.unit_k + 8) * 2 + 15) & ~(size_t)15;  // + the all-zero row
+        if (w0->scheme == SCHEME_Q4K) b += (size_t)kcu * (L.unit_k / 32) * 16 * 4;
         return b;
     };
     int kcu = units;
-    while (kcu > 1 && stage_bytes(kcu) > budget) kcu--;
-    if (stage_bytes(kcu) > budget) {
+    while (kcu > 1 && part_bytes + stage_bytes(kcu) > budget) kcu--;
+    if (part_bytes + stage_bytes(kcu) > budget) {
         set_error("gemv: one K unit of %d activation rows does not fit LDS", rv);
         return RLX_ERR_INVALID;
     }
-    int nwaves = std::min(16, std::max(1, kcu));
-    size_t red_bytes = (size_t)nwaves * rtw * 1024;
-    size_t shmem = std::max(stage_bytes(kcu), red_bytes);
-    GemvArgs a{w->dev, x, out, m, (int)w->dims.k, (int)w->dims.n, units, tiles, kcu, xk};
+    GemvArgs a{};
+    int wg = 0;
+    for (int i = 0; i < count; i++) {
+        a.seg[i] = GemvSeg{ws[i]->dev, outs[i], (int)ws[i]->dims.n, (int)ws[i]->dims.row_tiles, wg, 0};
+        wg += (int)((ws[i]->dims.row_tiles + tpw - 1) / tpw);
+    }
+    a.x = x;
+    a.nseg = count;
+    a.m = m;
+    a.k = (int)w0->dims.k;
+    a.units = units;
+    a.kc_units = kcu;
+    a.x_dtype = xk;
+    a.tiles_per_wg = tpw;
     void *params[] = {&a};
-    return launch(id, (unsigned)((tiles + rtw - 1) / rtw), 1, (unsigned)nwaves * 64, (unsigned)shmem, stream, params);
+    return launch(id, (unsigned)wg, 1, (unsigned)nwaves * 64, (unsigned)(part_bytes + stage_bytes(kcu)), stream, params);
 }
 
 }  // namespace rlx
@@ -148,13 +167,24 @@ size_t rlx_mi355x_gguf_matmul_workspace(int scheme, int x_dtype, int64_t m, int6
     return 0;
 }
 
-int rlx_mi355x_gguf_matmul_bt(const void *x_dev, int x_dtype, const rlx_qweight *w, float *out_dev, int64_t m,
-                              void *workspace, size_t workspace_bytes, void *stream) {
+int rlx_mi355x_gguf_matmul_bt_grouped(const void *x_dev, int x_dtype, const rlx_qweight *const *ws,
+                                      float *const *outs_dev, int count, int64_t m, void *workspace,
+                                      size_t workspace_bytes, void *stream) {
     using namespace rlx;
     (void)workspace; (void)workspace_bytes;
-    if (!x_dev || !w || !out_dev || m <= 0) {
-        set_error("gguf_matmul_bt: null argument or m=%lld", (long long)m);
+    if (!x_dev || !ws || !outs_dev || count <= 0 || m <= 0) {
+        set_error("gguf_matmul_bt: null argument, count=%d or m=%lld", count, (long long)m);
         return RLX_ERR_INVALID;
+    }
+    for (int i = 0; i < count; i++) {
+        if (!ws[i] || !outs_dev[i]) {
+            set_error("gguf_matmul_bt: null weight / output %d", i);
+            return RLX_ERR_INVALID;
+        }
+        if (ws[i]->scheme != ws[0]->scheme || ws[i]->dims.k != ws[0]->dims.k) {
+            set_error("gguf_matmul_bt_grouped: weight %d differs in scheme or k from weight 0", i);
+            return RLX_ERR_INVALID;
+        }
     }
     int xk = x_kind(x_dtype);
     if (xk < 0) {
@@ -162,13 +192,22 @@ int rlx_mi355x_gguf_matmul_bt(const void *x_dev, int x_dtype, const rlx_qweight 
         return RLX_ERR_UNSUPPORTED;
     }
     const int64_t cap = xk == 0 ? 8 : 16;  // activation rows one MFMA pass holds
-    const size_t xrow = (size_t)w->dims.k * (xk == 0 ? 4 : 2);
+    const size_t xrow = (size_t)ws[0]->dims.k * (xk == 0 ? 4 : 2);
     for (int64_t r0 = 0; r0 < m; r0 += cap) {
         int rows = (int)std::min<int64_t>(cap, m - r0);
-        RLX_TRY(launch_gemv((const uint8_t *)x_dev + r0 * xrow, xk, w, out_dev + r0 * w->dims.n, rows,
-                            (hipStream_t)stream));
+        for (int c0 = 0; c0 < count; c0 += GEMV_MAX_SEG) {
+            int c = std::min(GEMV_MAX_SEG, count - c0);
+            float *outs[GEMV_MAX_SEG];
+            for (int i = 0; i < c; i++) outs[i] = outs_dev[c0 + i] + r0 * ws[c0 + i]->dims.n;
+            RLX_TRY(launch_gemv((const uint8_t *)x_dev + r0 * xrow, xk, ws + c0, outs, c, rows, (hipStream_t)stream));
+        }
     }
     return RLX_OK;
+}
+
+int rlx_mi355x_gguf_matmul_bt(const void *x_dev, int x_dtype, const rlx_qweight *w, float *out_dev, int64_t m,
+                              void *workspace, size_t workspace_bytes, void *stream) {
+    return rlx_mi355x_gguf_matmul_bt_grouped(x_dev, x_dtype, &w, &out_dev, 1, m, workspace, workspace_bytes, stream);
 }
 
 int rlx_mi355x_fake_quantize(const float *x_dev, float *out_dev, int8_t *codes_dev, int64_t len, int64_t chan_dim,

@@ -32,6 +32,16 @@ __device__ __forceinline__ float half_bits_to_float(uint32_t bits16) {
 // 0x6400 is 1024.0 in binary16 and its ulp is 1, so (0x6400 | v) is the half 1024 + v for 0 <= v < 1024.
 constexpr uint32_t MAGIC = 0x64006400u;
 
+// (a & mask) | magic in one VALU op (v_and_or_b32). gfx9 VOP3 encodings take no literal and at most one scalar
+// operand, so with three compile-time constants the compiler emits v_and + v_or instead. The two empty asm
+// statements only hide the constants from constant folding (mask in an SGPR, magic in a VGPR); the and/or itself
+// stays ordinary code, so the compiler's MFMA hazard tracking sees every register it writes.
+__device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t mask, uint32_t magic) {
+    asm("" : "+s"(mask));
+    asm("" : "+v"(magic));
+    return (a & mask) | magic;
+}
+
 // 4-bit granule word -> four half2 registers holding (q - OFF) for the 8 weights, fragment order.
 // OFF = 8 for Q4_0 (signed codes), 0 for Q4_K. All results are exact integers.
 template <int OFF>
@@ -40,10 +50,10 @@ __device__ __forceinline__ void unpack_q4(uint32_t w, Frag &f) {
     const half2_t mul_hi = {(half_t)0.0625f, (half_t)0.0625f};
     const half2_t sub_hi = {(half_t)(-(64 + OFF)), (half_t)(-(64 + OFF))};
     uint32_t w2 = w >> 8;
-    half2_t a0 = as_half2((w & 0x000F000Fu) | MAGIC);   // 1024 + q
-    half2_t a1 = as_half2((w & 0x00F000F0u) | MAGIC);   // 1024 + 16 q
-    half2_t a2 = as_half2((w2 & 0x000F000Fu) | MAGIC);
-    half2_t a3 = as_half2((w2 & 0x00F000F0u) | MAGIC);
+    half2_t a0 = as_half2(and_or(w, 0x000F000Fu, MAGIC));   // 1024 + q
+    half2_t a1 = as_half2(and_or(w, 0x00F000F0u, MAGIC));   // 1024 + 16 q
+    half2_t a2 = as_half2(and_or(w2, 0x000F000Fu, MAGIC));
+    half2_t a3 = as_half2(and_or(w2, 0x00F000F0u, MAGIC));
     f.h2[0] = a0 + sub_lo;
     f.h2[1] = __builtin_elementwise_fma(a1, mul_hi, sub_hi);  // (1024+16q)/16 - 64 - OFF, single rounding of an exact value
     f.h2[2] = a2 + sub_lo;
@@ -59,10 +69,10 @@ __device__ __forceinline__ void unpack_q4_scaled(uint32_t w, half2_t sc, Frag &f
     half2_t neg_hi = -(sc * k64);
     half2_t sc16 = sc * r16;         // exact power-of-two scaling
     uint32_t w2 = w >> 8;
-    half2_t a0 = as_half2((w & 0x000F000Fu) | MAGIC);
-    half2_t a1 = as_half2((w & 0x00F000F0u) | MAGIC);
-    half2_t a2 = as_half2((w2 & 0x000F000Fu) | MAGIC);
-    half2_t a3 = as_half2((w2 & 0x00F000F0u) | MAGIC);
+    half2_t a0 = as_half2(and_or(w, 0x000F000Fu, MAGIC));
+    half2_t a1 = as_half2(and_or(w, 0x00F000F0u, MAGIC));
+    half2_t a2 = as_half2(and_or(w2, 0x000F000Fu, MAGIC));
+    half2_t a3 = as_half2(and_or(w2, 0x00F000F0u, MAGIC));
     f.h2[0] = __builtin_elementwise_fma(a0, sc, neg_lo);
     f.h2[1] = __builtin_elementwise_fma(a1, sc16, neg_hi);
     f.h2[2] = __builtin_elementwise_fma(a2, sc, neg_lo);

@@ -7,24 +7,33 @@
 // per-block scale is applied to the block result in f32 (acc += d * blk), so nothing is rounded to 16 bits
 // except the activations, and f32 activations are carried as an exact hi + lo pair of halfs in two A rows.
 //
-// Workgroup = row tiles [T0, T0+RTW) x all of K. Activations for a K chunk are converted into LDS once per
-// workgroup; the waves take units (128 or 256 columns) round-robin, keep per-wave partial sums, and a final
-// LDS pass adds the waves' partials in a fixed order (deterministic output).
+// Work decomposition and the LDS protocol are described above gemv_body().
 #include "common.h"
 
 namespace rlx {
 
 enum XType : int { X_F32 = 0, X_BF16 = 1, X_F16 = 2 };
 
-struct GemvArgs {
+constexpr int GEMV_MAX_SEG = 4;
+
+struct GemvSeg {
     const uint8_t *w;
-    const void *x;
     float *out;
-    int m, k, n;
-    int units;      // K units in the device layout
-    int row_tiles;  // 16-row tiles in the device layout
-    int kc_units;   // units per LDS chunk
+    int n;          // logical rows of this matrix
+    int row_tiles;  // 16-row tiles in its device layout
+    int wg_begin;   // first workgroup of this segment
+    int pad;
+};
+
+struct GemvArgs {
+    GemvSeg seg[GEMV_MAX_SEG];
+    const void *x;
+    int nseg;
+    int m, k;
+    int units;         // K units in the device layout
+    int kc_units;      // units per LDS chunk
     int x_dtype;
+    int tiles_per_wg;  // row tiles per workgroup
 };
 
 constexpr int XS_PAD_HALFS = 8;      // 16 bytes of padding per LDS row: rows land in different bank groups
@@ -38,9 +47,10 @@ template <>
 struct UnitRegs<SCHEME_Q4_0> {
     uint4_t q;
     uint2_t s;
-    __device__ __forceinline__ void load(const uint8_t *unit, int l, int nrow) {
+    // `meta` is false for lanes whose accumulators hold no real row: they skip the scale load
+    __device__ __forceinline__ void load(const uint8_t *unit, int l, int nrow, bool meta) {
         q = *(const uint4_t *)(unit + l * 16);
-        s = *(const uint2_t *)(unit + 1024 + nrow * 8);
+        if (meta) s = *(const uint2_t *)(unit + 1024 + nrow * 8);
     }
     __device__ __forceinline__ void clear() {
         q = uint4_t{0, 0, 0, 0};
@@ -51,10 +61,10 @@ template <>
 struct UnitRegs<SCHEME_Q8_0> {
     uint4_t q0, q1;
     uint2_t s;
-    __device__ __forceinline__ void load(const uint8_t *unit, int l, int nrow) {
+    __device__ __forceinline__ void load(const uint8_t *unit, int l, int nrow, bool meta) {
         q0 = *(const uint4_t *)(unit + l * 16);
         q1 = *(const uint4_t *)(unit + 1024 + l * 16);
-        s = *(const uint2_t *)(unit + 2048 + nrow * 8);
+        if (meta) s = *(const uint2_t *)(unit + 2048 + nrow * 8);
     }
     __device__ __forceinline__ void clear() {
         q0 = q1 = uint4_t{0, 0, 0, 0};
@@ -64,10 +74,10 @@ struct UnitRegs<SCHEME_Q8_0> {
 template <>
 struct UnitRegs<SCHEME_Q4K> {
     uint4_t q0, q1, meta;
-    __device__ __forceinline__ void load(const uint8_t *unit, int l, int nrow) {
+    __device__ __forceinline__ void load(const uint8_t *unit, int l, int nrow, bool want_meta) {
         q0 = *(const uint4_t *)(unit + l * 16);
         q1 = *(const uint4_t *)(unit + 1024 + l * 16);
-        meta = *(const uint4_t *)(unit + 2048 + nrow * 16);
+        if (want_meta) meta = *(const uint4_t *)(unit + 2048 + nrow * 16);
     }
     __device__ __forceinline__ void clear() { q0 = q1 = meta = uint4_t{0, 0, 0, 0}; }  // d = dmin = 0
 };
@@ -76,39 +86,49 @@ __device__ __forceinline__ float scale_of(uint2_t s, int t) {
     return half_bits_to_float((t & 1) ? (s[t >> 1] >> 16) : (s[t >> 1] & 0xFFFFu));
 }
 
-// A fragment of virtual row i for the 8 columns starting at `col` of the staged chunk; rows >= rv give zeros.
-__device__ __forceinline__ void load_afrag(const half_t *xs, int row_stride, int i, int rv, int col, Frag &a) {
-    a.u4 = uint4_t{0, 0, 0, 0};
-    if (i < rv) a.u4 = *(const uint4_t *)(xs + i * row_stride + col);
+// A fragments of one lane for the NB 32-column blocks starting at staged column `col`. `xrow` already points at
+// the lane's virtual row and 8-column slice; lanes past the last real row point at an all-zero LDS row, so the
+// reads need no masking.
+template <int NB>
+__device__ __forceinline__ void load_afrags(const half_t *xrow, int col, Frag (&a)[NB]) {
+#pragma unroll
+    for (int t = 0; t < NB; t++) a[t].u4 = *(const uint4_t *)(xrow + col + t * 32);
 }
 
 template <int SCHEME, int NREG>
-__device__ __forceinline__ void compute_unit(const UnitRegs<SCHEME> &w, const half_t *xs, const float *sxs,
-                                             int row_stride, int i, int g, int rv, int ucol, int ublk,
-                                             float acc[4]) {
+__device__ __forceinline__ void compute_unit(const UnitRegs<SCHEME> &w, const half_t *xrow, const float *sxs, int g,
+                                             int ucol, int ublk, float acc[4]) {
     const float4_t zero = {0.f, 0.f, 0.f, 0.f};
     if constexpr (SCHEME == SCHEME_Q4_0) {
+        Frag a[4], b[4];
+        load_afrags<4>(xrow, ucol, a);
+#pragma unroll
+        for (int t = 0; t < 4; t++) unpack_q4<8>(w.q[t], b[t]);
+        float4_t blk[4];
+#pragma unroll
+        for (int t = 0; t < 4; t++) blk[t] = mfma16(a[t], b[t], zero);
 #pragma unroll
         for (int t = 0; t < 4; t++) {
-            Frag a, b;
-            load_afrag(xs, row_stride, i, rv, ucol + t * 32 + g * 8, a);
-            unpack_q4<8>(w.q[t], b);
-            float4_t blk = mfma16(a, b, zero);
             float d = scale_of(w.s, t);
 #pragma unroll
-            for (int r = 0; r < NREG; r++) acc[r] = __builtin_fmaf(d, blk[r], acc[r]);
+            for (int r = 0; r < NREG; r++) acc[r] = __builtin_fmaf(d, blk[t][r], acc[r]);
         }
     } else if constexpr (SCHEME == SCHEME_Q8_0) {
+        Frag a[4], b[4];
+        load_afrags<4>(xrow, ucol, a);
 #pragma unroll
         for (int t = 0; t < 4; t++) {
-            Frag a, b;
-            load_afrag(xs, row_stride, i, rv, ucol + t * 32 + g * 8, a);
             const uint4_t &q = (t < 2) ? w.q0 : w.q1;
-            unpack_q8(q[2 * (t & 1)], q[2 * (t & 1) + 1], b);
-            float4_t blk = mfma16(a, b, zero);
+            unpack_q8(q[2 * (t & 1)], q[2 * (t & 1) + 1], b[t]);
+        }
+        float4_t blk[4];
+#pragma unroll
+        for (int t = 0; t < 4; t++) blk[t] = mfma16(a[t], b[t], zero);
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
             float d = scale_of(w.s, t);
 #pragma unroll
-            for (int r = 0; r < NREG; r++) acc[r] = __builtin_fmaf(d, blk[r], acc[r]);
+            for (int r = 0; r < NREG; r++) acc[r] = __builtin_fmaf(d, blk[t][r], acc[r]);
         }
     } else {
         float d = half_bits_to_float(w.meta[0] & 0xFFFFu);
@@ -116,20 +136,26 @@ __device__ __forceinline__ void compute_unit(const UnitRegs<SCHEME> &w, const ha
         uint32_t sc[2], mn[2];
         q4k_scales(w.meta[1], w.meta[2], w.meta[3], sc, mn);
 #pragma unroll
-        for (int j = 0; j < 8; j++) {
-            Frag a, b;
-            load_afrag(xs, row_stride, i, rv, ucol + j * 32 + g * 8, a);
-            const uint4_t &q = (j < 4) ? w.q0 : w.q1;
-            unpack_q4<0>(q[j & 3], b);
-            float4_t blk = mfma16(a, b, zero);
-            float dj = d * ubyte_to_float(sc[j >> 2], j & 3);
-            float mj = dmin * ubyte_to_float(mn[j >> 2], j & 3);
-            // sum of the activations of this 32-column block for the four output rows this lane holds
-            float4_t sx = *(const float4_t *)(sxs + (ublk + j) * 16 + 4 * g);
+        for (int h = 0; h < 2; h++) {
+            Frag a[4], b[4];
+            load_afrags<4>(xrow, ucol + h * 128, a);
+            const uint4_t &q = h ? w.q1 : w.q0;
 #pragma unroll
-            for (int r = 0; r < NREG; r++) {
-                acc[r] = __builtin_fmaf(dj, blk[r], acc[r]);
-                acc[r] = __builtin_fmaf(-mj, sx[r], acc[r]);
+            for (int t = 0; t < 4; t++) unpack_q4<0>(q[t], b[t]);
+            float4_t blk[4];
+#pragma unroll
+            for (int t = 0; t < 4; t++) blk[t] = mfma16(a[t], b[t], zero);
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                float dj = d * ubyte_to_float(sc[h], t);
+                float mj = dmin * ubyte_to_float(mn[h], t);
+                // sum of the activations of this 32-column block for the four output rows this lane holds
+                float4_t sx = *(const float4_t *)(sxs + (ublk + 4 * h + t) * 16 + 4 * g);
+#pragma unroll
+                for (int r = 0; r < NREG; r++) {
+                    acc[r] = __builtin_fmaf(dj, blk[t][r], acc[r]);
+                    acc[r] = __builtin_fmaf(-mj, sx[r], acc[r]);
+                }
             }
         }
     }
@@ -171,50 +197,78 @@ __device__ __forceinline__ void stage_x(const GemvArgs &a, half_t *xs, int row_s
     }
 }
 
-template <int SCHEME, int RTW, int NREG, int DEPTH>
+// One workgroup = a contiguous run of row tiles of one weight segment x all of K.
+//   * the activations are converted into LDS once per workgroup (per K chunk when they do not fit);
+//   * wave w walks the (tile, unit) items with unit = w, w + nwaves, ... of every tile in the run, keeping DEPTH
+//     units of weights in flight in registers, so the stream of 16-byte loads never drains between tiles;
+//   * at the end of each (tile, chunk) the wave adds its partial sums into its own LDS slot; one barrier at the
+//     very end, then the slots of all waves are added in a fixed order and written out (deterministic).
+// A launch can carry up to GEMV_MAX_SEG weight matrices that share the activations (q/k/v, gate/up).
+template <int SCHEME, int NREG, int DEPTH>
 __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
     constexpr Layout L = layout_of(SCHEME);
     constexpr int BLK_PER_UNIT = L.unit_k / 32;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
 
-    const int tid = threadIdx.x, l = tid & 63, wave = tid >> 6, nwaves = blockDim.x >> 6;
+    const int tid = threadIdx.x, l = tid & 63;
+    // wave-uniform values live in SGPRs so that unit addresses are scalar arithmetic
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), nwaves = blockDim.x >> 6;
     const int nrow = l & 15, g = l >> 4;
     const int rv = (a.x_dtype == X_F32) ? 2 * a.m : a.m;  // virtual A rows
-    const int tile0 = blockIdx.x * RTW;
+    const int ng = (rv + 3) >> 2;                         // lane groups whose accumulators hold real rows
+    const bool has_rows = g < ng;
+
+    int s = 0;
+#pragma unroll
+    for (int i = 1; i < GEMV_MAX_SEG; i++)
+        if (i < a.nseg && (int)blockIdx.x >= a.seg[i].wg_begin) s = i;
+    const GemvSeg seg = a.seg[s];
+    const int tile0 = ((int)blockIdx.x - seg.wg_begin) * a.tiles_per_wg;
+    const int ntiles = min(a.tiles_per_wg, seg.row_tiles - tile0);
+
     const int kc = a.kc_units * L.unit_k;
     const int row_stride = kc + XS_PAD_HALFS;
-    half_t *xs = (half_t *)smem;
-    float *sxs = (float *)(smem + (((size_t)rv * row_stride * 2 + 15) & ~(size_t)15));  // Q4_K only: [blk][16]
+    // LDS: [partial sums: tiles_per_wg x nwaves x (4 ng) x 16 f32][staged activations: rv rows + one zero row]
+    //      [Q4_K block sums]
+    const int slot_floats = ng * 64;
+    float *part = (float *)smem;
+    const size_t part_bytes = (size_t)a.tiles_per_wg * nwaves * slot_floats * 4;
+    half_t *xs = (half_t *)(smem + part_bytes);
+    float *sxs = (float *)(smem + part_bytes + (((size_t)(rv + 1) * row_stride * 2 + 15) & ~(size_t)15));  // [blk][16]
+    const half_t *xrow = xs + min(nrow, rv) * row_stride + g * 8;  // this lane's A row (row rv is all zeros)
 
-    float acc[RTW][4];
-#pragma unroll
-    for (int t = 0; t < RTW; t++)
-#pragma unroll
-        for (int r = 0; r < 4; r++) acc[t][r] = 0.f;
+    for (int i = tid; i < a.tiles_per_wg * nwaves * slot_floats; i += blockDim.x) part[i] = 0.f;
+    for (int i = tid; i < row_stride / 2; i += blockDim.x) ((uint32_t *)(xs + rv * row_stride))[i] = 0u;
 
-    const uint8_t *tile_base[RTW];
-    bool tile_ok[RTW];
-#pragma unroll
-    for (int t = 0; t < RTW; t++) {
-        int tile = tile0 + t;
-        tile_ok[t] = tile < a.row_tiles;
-        tile_base[t] = a.w + (long long)(tile_ok[t] ? tile : a.row_tiles - 1) * a.units * L.unit_bytes;
-    }
+    const uint8_t *wbase = seg.w + (long long)tile0 * a.units * L.unit_bytes;
+    const long long tile_bytes = (long long)a.units * L.unit_bytes;
 
     for (int u0 = 0; u0 < a.units; u0 += a.kc_units) {
         const int nu = min(a.kc_units, a.units - u0);  // units in this chunk
-        // This wave's units: u0 + wave + s * nwaves. Software pipeline of DEPTH units of weights in registers;
-        // the first loads are issued before the staging barrier so HBM latency overlaps the conversion.
-        UnitRegs<SCHEME> wr[DEPTH][RTW];
+        // This wave's items: for each tile, units wave, wave + nwaves, ... < nu. Two cursors walk them: `pf_*` issues
+        // loads DEPTH items ahead into a register ring, `cu_*` consumes.
+        const int my_units = wave < nu ? (nu - wave + nwaves - 1) / nwaves : 0;
+        const int nitems = ntiles * my_units;
+        int pf_t = 0, pf_u = wave, pf_n = 0;
+        const uint8_t *pf_ptr = wbase + (long long)(u0 + wave) * L.unit_bytes;
+        UnitRegs<SCHEME> ring[DEPTH];
+        auto prefetch = [&](UnitRegs<SCHEME> &slot) {
+            if (pf_n < nitems) {
+                slot.load(pf_ptr, l, nrow, has_rows);
+                pf_n++;
+                pf_u += nwaves;
+                pf_ptr += (long long)nwaves * L.unit_bytes;
+                if (pf_u >= nu) {
+                    pf_t++;
+                    pf_u = wave;
+                    pf_ptr = wbase + pf_t * tile_bytes + (long long)(u0 + wave) * L.unit_bytes;
+                }
+            }
+        };
 #pragma unroll
         for (int d = 0; d < DEPTH; d++) {
-            int ul = wave + d * nwaves;
-            bool ok = ul < nu;
-#pragma unroll
-            for (int t = 0; t < RTW; t++) {
-                wr[d][t].clear();
-                if (ok && tile_ok[t]) wr[d][t].load(tile_base[t] + (long long)(u0 + ul) * L.unit_bytes, l, nrow);
-            }
+            ring[d].clear();
+            prefetch(ring[d]);
         }
         if (u0 > 0) __syncthreads();  // previous chunk fully consumed
         stage_x(a, xs, row_stride, u0 * L.unit_k, nu * L.unit_k);
@@ -223,85 +277,73 @@ __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
             const int nblk = nu * BLK_PER_UNIT;
             for (int idx = tid; idx < nblk * 16; idx += blockDim.x) {
                 int blk = idx >> 4, i = idx & 15;
-                float s = 0.f;
+                float sum = 0.f;
                 if (i < rv) {
 #pragma unroll
                     for (int e4 = 0; e4 < 4; e4++) {
                         Frag f;
                         f.u4 = *(const uint4_t *)(xs + i * row_stride + blk * 32 + e4 * 8);
 #pragma unroll
-                        for (int e = 0; e < 8; e++) s += (float)f.h8[e];
+                        for (int e = 0; e < 8; e++) sum += (float)f.h8[e];
                     }
                 }
-                sxs[blk * 16 + i] = s;
+                sxs[blk * 16 + i] = sum;
             }
             __syncthreads();
         }
-        for (int base = 0; wave + base * nwaves < nu; base += DEPTH) {
+        float acc[4] = {0.f, 0.f, 0.f, 0.f};
+        int cu_t = 0, cu_u = wave;
+        for (int base = 0; base < nitems; base += DEPTH) {
 #pragma unroll
             for (int d = 0; d < DEPTH; d++) {
-                int ul = wave + (base + d) * nwaves;
-                UnitRegs<SCHEME> cur[RTW];
+                if (base + d < nitems) {
+                    UnitRegs<SCHEME> cur = ring[d];
+                    prefetch(ring[d]);
+                    compute_unit<SCHEME, NREG>(cur, xrow, sxs, g, cu_u * L.unit_k, cu_u * BLK_PER_UNIT, acc);
+                    cu_u += nwaves;
+                    if (cu_u >= nu) {  // last unit of this tile for this wave: bank the partial sums
+                        if (has_rows) {
+                            float *slot = part + ((size_t)cu_t * nwaves + wave) * slot_floats + g * 64 + nrow;
 #pragma unroll
-                for (int t = 0; t < RTW; t++) cur[t] = wr[d][t];
-                // refill this pipeline slot with the unit DEPTH rounds ahead
-                int ul_next = ul + DEPTH * nwaves;
-                bool ok_next = ul_next < nu;
-#pragma unroll
-                for (int t = 0; t < RTW; t++) {
-                    if (ok_next && tile_ok[t])
-                        wr[d][t].load(tile_base[t] + (long long)(u0 + ul_next) * L.unit_bytes, l, nrow);
-                }
-                if (ul < nu) {
-#pragma unroll
-                    for (int t = 0; t < RTW; t++)
-                        compute_unit<SCHEME, NREG>(cur[t], xs, sxs, row_stride, nrow, g, rv, ul * L.unit_k,
-                                                   ul * BLK_PER_UNIT, acc[t]);
+                            for (int r = 0; r < 4; r++) {
+                                if (r < NREG) slot[r * 16] += acc[r];
+                                acc[r] = 0.f;
+                            }
+                        }
+                        cu_t++;
+                        cu_u = wave;
+                    }
                 }
             }
         }
     }
 
-    // Cross-wave reduction in a fixed order. Lane (nrow, g) register r holds virtual row 4g + r, column nrow.
     __syncthreads();
-    float *red = (float *)smem;  // [wave][tile][16 rows][16 cols]
-    const int ng = (rv + 3) >> 2;
-    if (g < ng) {
-#pragma unroll
-        for (int t = 0; t < RTW; t++)
-#pragma unroll
-            for (int r = 0; r < 4; r++) red[((wave * RTW + t) * 16 + 4 * g + r) * 16 + nrow] = acc[t][r];
-    }
-    __syncthreads();
-    for (int idx = tid; idx < RTW * a.m * 16; idx += blockDim.x) {
-        int col = idx & 15, mr = (idx >> 4) % a.m, t = idx / (16 * a.m);
-        float s = 0.f;
+    // out[mr][tile*16 + col] = sum over waves of row mr (+ 2^-11 * row m+mr for f32 activations)
+    for (int idx = tid; idx < ntiles * a.m * 16; idx += blockDim.x) {
+        const int col = idx & 15, mr = (idx >> 4) % a.m, t = idx / (16 * a.m);
+        float sum = 0.f;
         for (int wv = 0; wv < nwaves; wv++) {
-            const float *p = red + ((wv * RTW + t) * 16) * 16 + col;
-            s += p[mr * 16];
-            if (a.x_dtype == X_F32) s += p[(a.m + mr) * 16] * (1.0f / LO_SCALE);
+            const float *slot = part + ((size_t)t * nwaves + wv) * slot_floats + col;
+            sum += slot[mr * 16];
+            if (a.x_dtype == X_F32) sum += slot[(a.m + mr) * 16] * (1.0f / LO_SCALE);
         }
-        int n_out = (tile0 + t) * 16 + col;
-        if (n_out < a.n) a.out[(long long)mr * a.n + n_out] = s;
+        const int n_out = (tile0 + t) * 16 + col;
+        if (n_out < seg.n) seg.out[(long long)mr * seg.n + n_out] = sum;
     }
 }
 
 }  // namespace rlx
 
-#define RLX_GEMV_INST(name, SCHEME, RTW, NREG, DEPTH)                                                       \
-    extern "C" __global__ __launch_bounds__(1024) void name(rlx::GemvArgs a) {                               \
-        rlx::gemv_body<SCHEME, RTW, NREG, DEPTH>(a);                                                          \
+#define RLX_GEMV_INST(name, SCHEME, NREG, DEPTH)                                                            \
+    extern "C" __global__ __launch_bounds__(512) void name(rlx::GemvArgs a) {                                \
+        rlx::gemv_body<SCHEME, NREG, DEPTH>(a);                                                               \
     }
 
 // NREG = 2: at most two virtual rows (m = 1 f32, or m <= 2 16-bit); NREG = 4 otherwise.
-RLX_GEMV_INST(rlx_gemv_q4_0_t1_r2, rlx::SCHEME_Q4_0, 1, 2, 4)
-RLX_GEMV_INST(rlx_gemv_q4_0_t2_r2, rlx::SCHEME_Q4_0, 2, 2, 2)
-RLX_GEMV_INST(rlx_gemv_q4_0_t1_r4, rlx::SCHEME_Q4_0, 1, 4, 4)
-RLX_GEMV_INST(rlx_gemv_q4_0_t2_r4, rlx::SCHEME_Q4_0, 2, 4, 2)
-RLX_GEMV_INST(rlx_gemv_q4_0_t4_r4, rlx::SCHEME_Q4_0, 4, 4, 1)
-RLX_GEMV_INST(rlx_gemv_q8_0_t1_r2, rlx::SCHEME_Q8_0, 1, 2, 2)
-RLX_GEMV_INST(rlx_gemv_q8_0_t1_r4, rlx::SCHEME_Q8_0, 1, 4, 2)
-RLX_GEMV_INST(rlx_gemv_q8_0_t2_r4, rlx::SCHEME_Q8_0, 2, 4, 2)
-RLX_GEMV_INST(rlx_gemv_q4_k_t1_r2, rlx::SCHEME_Q4K, 1, 2, 2)
-RLX_GEMV_INST(rlx_gemv_q4_k_t1_r4, rlx::SCHEME_Q4K, 1, 4, 2)
-RLX_GEMV_INST(rlx_gemv_q4_k_t2_r4, rlx::SCHEME_Q4K, 2, 4, 2)
+RLX_GEMV_INST(rlx_gemv_q4_0_r2, rlx::SCHEME_Q4_0, 2, 4)
+RLX_GEMV_INST(rlx_gemv_q4_0_r4, rlx::SCHEME_Q4_0, 4, 4)
+RLX_GEMV_INST(rlx_gemv_q8_0_r2, rlx::SCHEME_Q8_0, 2, 3)
+RLX_GEMV_INST(rlx_gemv_q8_0_r4, rlx::SCHEME_Q8_0, 4, 3)
+RLX_GEMV_INST(rlx_gemv_q4_k_r2, rlx::SCHEME_Q4K, 2, 3)
+RLX_GEMV_INST(rlx_gemv_q4_k_r4, rlx::SCHEME_Q4K, 4, 3)

@@ -124,6 +124,13 @@ class CompiledGraph:
     def stream(self):
         return _lib.lib().rlx_exec_stream(self._h)
 
+    def set_stream(self, stream):
+        _lib.check(_lib.lib().rlx_exec_set_stream(self._h, stream))
+
+    def capture(self):
+        """Record the schedule into a hipGraph; later launch() calls replay it."""
+        _lib.check(_lib.lib().rlx_exec_capture(self._h))
+
     def arena_bytes(self):
         return _lib.lib().rlx_exec_arena_bytes(self._h)
 
@@ -168,6 +175,12 @@ class Session:
         if not h:
             raise _lib.RlxError(-1, _lib.last_error())
         return CompiledGraph(h, graph)
+
+
+def launch_sequence(compiled_graphs):
+    """Enqueue each executable once, in order, from C (no Python between launches)."""
+    arr = (C.c_void_p * len(compiled_graphs))(*[c._h for c in compiled_graphs])
+    _lib.check(_lib.lib().rlx_mi355x_launch_sequence(arr, len(compiled_graphs)))
 
 
 def supported_ops():

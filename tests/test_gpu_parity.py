@@ -342,3 +342,37 @@ def test_graph_typed_bf16_input(oracle):
     x = oracle.bf16_round(np.random.default_rng(44).standard_normal((m, k)).astype(np.float32))
     got = run_dq(packed, Q4K, f32_to_bf16_bits(x), m, k, n, typed=DType.BF16)
     assert rel_err(got, oracle.gguf_matmul_f64(x, packed, m, k, n, Q4K)) <= TOL
+
+
+def test_graph_fuses_matmuls_that_share_an_input(oracle):
+    # q/k/v-style: three weights, one activation vector -> one grouped launch; outputs must be those of three
+    # separate matmuls. A fourth weight with a different k stays on its own.
+    k, ns = 1024, [256, 64, 48]
+    rng = np.random.default_rng(50)
+    x = rng.standard_normal((2, k)).astype(np.float32)
+    x2 = rng.standard_normal((2, 512)).astype(np.float32)
+    g = Graph.new("qkv")
+    xi = g.input("x", Shape.new([2, k], DType.F32))
+    xj = g.input("x2", Shape.new([2, 512], DType.F32))
+    packs, outs = [], []
+    for i, n in enumerate(ns):
+        p, _ = make_weights(Q4_0, n, k, seed=60 + i)
+        packs.append(p)
+        w = g.param(f"w{i}", Shape.new([len(p)], DType.U8))
+        outs.append(g.add_node(Op.DequantMatMul(QuantScheme.GgufQ4_0), [xi, w], Shape.new([2, n], DType.F32)))
+    p4, _ = make_weights(Q4_0, 32, 512, seed=70)
+    w4 = g.param("w4", Shape.new([len(p4)], DType.U8))
+    outs.append(g.add_node(Op.DequantMatMul(QuantScheme.GgufQ4_0), [xj, w4], Shape.new([2, 32], DType.F32)))
+    g.set_outputs(outs)
+    c = Session.new().compile(g)
+    for i, p in enumerate(packs):
+        c.set_param_typed(f"w{i}", p, DType.U8)
+    c.set_param_typed("w4", p4, DType.U8)
+    for attempt in ("eager", "hipGraph replay 1", "hipGraph replay 2"):
+        got = c.run([("x", x), ("x2", x2)])
+        for i, n in enumerate(ns):
+            assert rel_err(got[i].reshape(2, n), oracle.gguf_matmul_f64(x, packs[i], 2, k, n, Q4_0)) <= TOL, attempt
+        assert rel_err(got[3].reshape(2, 32), oracle.gguf_matmul_f64(x2, p4, 2, 512, 32, Q4_0)) <= TOL, attempt
+        if attempt == "eager":
+            c.capture()
+        x = (x * np.float32(1.5)).astype(np.float32)  # new inputs each replay: the graph must read them afresh
