@@ -2,8 +2,9 @@
 """Headline benchmark: Q4_0 decode GEMV (batch 1) over the seven Llama-3-8B layer projections on one MI355X.
 
 A step is one pass over one layer's seven projections (q, k, v, o, gate, up, down): seven DequantMatMul nodes of one
-compiled graph wired like the real layer (q/k/v read one activation vector, gate/up another, o and down their own),
-so the backend fuses them into four launches (qkv, o, gate+up, down), replayed as a hipGraph. The layers rotate through LAYERS distinct weight sets (~123 MB each), far
+compiled graph, each with its own f32 activation vector as BASELINE's config states, which the backend issues as one
+batched launch replayed as a hipGraph (`--wiring layer` orders them like a transformer layer instead: four dependent
+launches). The layers rotate through LAYERS distinct weight sets (~123 MB each), far
 more than the 256 MB of last-level cache, so every launch streams its weights from HBM. Inputs and weights are
 resident in HBM before the timed region. One JSON line is printed; `value` is algorithmic bytes per second
 (packed weights + f32 activations in + f32 outputs out), the figure the roofline fraction is taken from.
@@ -29,28 +30,75 @@ LLAMA8B = [("q", 4096, 4096), ("k", 1024, 4096), ("v", 1024, 4096), ("o", 4096, 
            ("gate", 14336, 4096), ("up", 14336, 4096), ("down", 4096, 14336)]
 
 
-# which activation vector each projection reads (the layer's real data flow)
-X_OF = {"q": "x_attn", "k": "x_attn", "v": "x_attn", "o": "x_o", "gate": "x_mlp", "up": "x_mlp", "down": "x_down"}
-LAUNCHES_PER_STEP = 4  # qkv, o, gate+up, down
+# Which activations each projection reads ("@p" = the output of projection p). "independent" is the workload as
+# BASELINE states it: seven GEMVs, each with its own seeded f32 activation vector; nothing orders them, so the backend
+# issues all seven as one batched launch. "layer" chains them the way a transformer layer's data flow does
+# (x -> q,k,v; q -> o; o -> gate,up; gate -> down; the attention / activation math in between is not part of this
+# path), which forces four dependent launches; it is reported under "extra" for comparison.
+WIRING = {
+    "independent": {n: f"x_{n}" for n in ("q", "k", "v", "o", "gate", "up", "down")},
+    "layer": {"q": "x_attn", "k": "x_attn", "v": "x_attn", "o": "@q", "gate": "@o", "up": "@o", "down": "@gate"},
+}
 
 
 def gemv_bytes(n, k, scheme_bytes_per_block=18, block=32, m=1):
     return n * k // block * scheme_bytes_per_block + 4 * k * m + 4 * n * m
 
 
-def build_layer_graph(rlx, li):
+def build_layer_graph(li, wiring):
     from rlx_amd import DType, Graph, Op, QuantScheme, Shape
 
+    x_of = WIRING[wiring]
     g = Graph.new(f"llama8b_layer{li}")
-    outs, xin = [], {}
+    outs, src_node = [], {}
     for name, n, k in LLAMA8B:
-        src = X_OF[name]
-        if src not in xin:
-            xin[src] = g.input(src, Shape.new([1, k], DType.F32))
+        src = x_of[name]
+        if src not in src_node:
+            src_node[src] = g.input(src, Shape.new([1, k], DType.F32))
         w = g.param(f"w_{name}", Shape.new([n * k // 32 * 18], DType.U8))
-        outs.append(g.add_node(Op.DequantMatMul(QuantScheme.GgufQ4_0), [xin[src], w], Shape.new([1, n], DType.F32)))
+        y = g.add_node(Op.DequantMatMul(QuantScheme.GgufQ4_0), [src_node[src], w], Shape.new([1, n], DType.F32))
+        src_node["@" + name] = y
+        outs.append(y)
     g.set_outputs(outs)
     return g
+
+
+def time_layers(rlx_amd, ops, stream, base, wiring, n_layers, steps, warmup, use_graph):
+    """Build n_layers executables (distinct weight bytes), replay them round-robin, return (ms_per_step, layers, xs)."""
+    from rlx_amd import DType, Session
+
+    x_of = WIRING[wiring]
+    xsrc = {}
+    for i, (name, n, k) in enumerate(LLAMA8B):
+        if not x_of[name].startswith("@"):
+            xsrc.setdefault(x_of[name], ops.philox_normal(2000 + i, k))
+    xs = {name: xsrc.get(x_of[name]) for name, _, _ in LLAMA8B}
+    layers = []
+    for li in range(n_layers):
+        c = Session.new(rlx_amd.Device.Mi355x).compile(build_layer_graph(li, wiring))
+        for name, n, k in LLAMA8B:
+            # distinct bytes per layer: rotate the rows of the base matrix (same statistics, different memory)
+            c.set_param_typed(f"w_{name}", np.roll(base[name], 37 * li, axis=0).reshape(-1), DType.U8)
+        for src, v in xsrc.items():
+            c.write_input(src, v)
+        c.sync()
+        c.set_stream(stream)
+        if use_graph:
+            c.capture()
+        layers.append(c)
+
+    def run_steps(count, offset=0):
+        rlx_amd.launch_sequence([layers[(offset + i) % len(layers)] for i in range(count)])
+
+    run_steps(warmup)
+    ops.sync(stream)
+    ev0, ev1 = ops.Event(), ops.Event()
+    ev0.record(stream)
+    run_steps(steps, warmup)
+    ev1.record(stream)
+    ms = ev0.elapsed_ms(ev1)
+    ops.sync(stream)
+    return ms / steps, layers, xs
 
 
 def main():
@@ -59,8 +107,11 @@ def main():
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--layers", type=int, default=8, help="distinct weight sets rotated through (8 x 123 MB)")
+    ap.add_argument("--wiring", choices=sorted(WIRING), default="independent")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--no-graph", action="store_true", help="launch kernels one by one instead of replaying a hipGraph")
+    ap.add_argument("--graph", action="store_true",
+                    help="replay each layer as a hipGraph instead of launching its kernel directly (one-node graphs "
+                         "cost more per launch than a plain launch on this runtime)")
     ap.add_argument("--extra", action="store_true", help="also time the other BASELINE configs (reported under 'extra')")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -81,50 +132,21 @@ def main():
     for name, n, k in LLAMA8B:
         w = (ops.philox_normal(1000 + len(base), n * k) * np.float32(0.02)).astype(np.float32)
         base[name] = ops.quantize(QuantScheme.GgufQ4_0, w).reshape(n, -1)
-    xsrc = {src: ops.philox_normal(2000 + i, 14336 if src == "x_down" else 4096)
-            for i, src in enumerate(sorted(set(X_OF.values())))}
-    xs = {name: xsrc[X_OF[name]] for name, _, _ in LLAMA8B}
-    layers = []
     stream = rlx_amd._lib.C.c_void_p()
     rlx_amd._lib.check(rlx_amd._lib.lib().rlx_mi355x_stream_create(rlx_amd._lib.C.byref(stream)))
-    for li in range(args.layers):
-        c = Session.new(rlx_amd.Device.Mi355x).compile(build_layer_graph(rlx_amd, li))
-        for name, n, k in LLAMA8B:
-            # distinct bytes per layer: rotate the rows of the base matrix (same statistics, different memory)
-            c.set_param_typed(f"w_{name}", np.roll(base[name], 37 * li, axis=0).reshape(-1), DType.U8)
-        for src, v in xsrc.items():
-            c.write_input(src, v)
-        c.sync()
-        c.set_stream(stream)
-        if not args.no_graph:
-            c.capture()
-        layers.append(c)
-    setup_s = time.time() - t0
-
     layer_bytes = sum(gemv_bytes(n, k) for _, n, k in LLAMA8B)
-    launches_per_step = LAUNCHES_PER_STEP
-
-    def run_steps(count, offset=0):
-        seq = [layers[(offset + i) % len(layers)] for i in range(count)]
-        rlx_amd.launch_sequence(seq)
-
-    run_steps(args.warmup)
-    ops.sync(stream)
-    ev0, ev1 = ops.Event(), ops.Event()
-    ev0.record(stream)
-    run_steps(args.steps, args.warmup)
-    ev1.record(stream)
-    ms = ev0.elapsed_ms(ev1)
-    ops.sync(stream)
-    ms_per_step = ms / args.steps
+    ms_per_step, layers, xs = time_layers(rlx_amd, ops, stream, base, args.wiring, args.layers, args.steps, args.warmup,
+                                          args.graph)
+    setup_s = time.time() - t0
+    launches_per_step = 1 if args.wiring == "independent" else 4
     gbs = layer_bytes / (ms_per_step * 1e-3) / 1e9
     us_per_launch = ms_per_step * 1e3 / launches_per_step
 
     # parity spot check of what was just timed (not in the timed region)
     import oracle
-    y = layers[1].read_output(4)
-    packed1 = np.roll(base["gate"], 37, axis=0).reshape(-1)
-    ref = oracle.gguf_matmul_f64(xs["gate"], packed1, 1, 4096, 14336, oracle.Q4_0, 0, 512)
+    y = layers[1].read_output(0)
+    packed1 = np.roll(base["q"], 37, axis=0).reshape(-1)
+    ref = oracle.gguf_matmul_f64(xs["q"], packed1, 1, 4096, 4096, oracle.Q4_0, 0, 512)
     parity = float(np.max(np.abs(y[:512] - ref[0]) / np.maximum(np.abs(ref[0]), 1.0)))
 
     result = {
@@ -142,7 +164,7 @@ def main():
         "data": "synthetic",
         "config": {"workload": "Q4_0 decode GEMV, batch 1, seven Llama-3-8B layer projections per step "
                                "(q,k,v,o,gate,up,down), f32 activations, weights ~N(0,0.02)",
-                   "layers_rotated": args.layers, "hip_graph": not args.no_graph,
+                   "wiring": args.wiring, "layers_rotated": args.layers, "hip_graph": args.graph,
                    "algorithmic_bytes_per_step": layer_bytes, "launches_per_step": launches_per_step},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
@@ -154,7 +176,14 @@ def main():
     }
 
     if args.extra:
+        del layers
         result["extra"] = extra_configs(rlx_amd, stream)
+        other = "layer" if args.wiring == "independent" else "independent"
+        ms_o, lay_o, _ = time_layers(rlx_amd, ops, stream, base, other, args.layers, args.steps, args.warmup, args.graph)
+        result["extra"][f"q4_0_gemv_llama8b_{other}_wiring"] = {
+            "ms_per_step": round(ms_o, 6), "GB/s": round(layer_bytes / ms_o / 1e6, 1),
+            "launches_per_step": 1 if other == "independent" else 4}
+        del lay_o
 
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(base, xs)
@@ -251,7 +280,8 @@ def cpu_baseline(base, xs):
     while True:
         t0 = time.time()
         for name, n, k in LLAMA8B:
-            oracle.gguf_matmul_bt(xs[name], base[name].reshape(-1), 1, k, n, oracle.Q4_0)
+            oracle.gguf_matmul_bt(xs[name] if xs[name] is not None else np.ones(k, np.float32), base[name].reshape(-1), 1, k, n,
+                                  oracle.Q4_0)
         spent += time.time() - t0
         reps += 1
         if time.time() > t_end or reps >= 50:

@@ -133,12 +133,13 @@ int rlx_mi355x_dequant(const rlx_qweight *w, float *out_dev, void *stream);
 int rlx_mi355x_gguf_matmul_bt(const void *x_dev, int x_dtype, const rlx_qweight *w, float *out_dev, int64_t m,
                               void *workspace, size_t workspace_bytes, void *stream);
 size_t rlx_mi355x_gguf_matmul_workspace(int scheme, int x_dtype, int64_t m, int64_t k, int64_t n);
-/* `count` matmuls that share the activations, the scheme and k (q/k/v or gate/up of one layer) in one launch per
- * four weights: outs_dev[i][m, n_i] = x . W_i^T. No counterpart in the reference, which runs one thunk per node; the
- * graph level uses it to fuse DequantMatMul nodes that read the same input. */
-int rlx_mi355x_gguf_matmul_bt_grouped(const void *x_dev, int x_dtype, const rlx_qweight *const *ws,
-                                      float *const *outs_dev, int count, int64_t m, void *workspace,
-                                      size_t workspace_bytes, void *stream);
+/* `count` independent matmuls of one scheme, batch size m and activation dtype in one launch per eight of them:
+ * outs_dev[i][m, n_i] = xs_dev[i][m, k_i] . W_i^T. No counterpart in the reference, which runs one thunk per node;
+ * the graph level uses it to issue together every DequantMatMul whose inputs are ready at the same point of the
+ * schedule (q/k/v and gate/up of a layer share their activations; independent projections need not). */
+int rlx_mi355x_gguf_matmul_bt_batch(const void *const *xs_dev, int x_dtype, const rlx_qweight *const *ws,
+                                    float *const *outs_dev, int count, int64_t m, void *workspace, size_t workspace_bytes,
+                                    void *stream);
 
 /* Thunk::FakeQuantize (rlx-cpu/src/thunk.rs:11159-11253) with the layout of quant_layout()
  * (thunk.rs:14163-14175): channel of flat element i is (i / inner) % chan_dim.

@@ -19,8 +19,8 @@ extern "C" int rlx_mi355x_fake_quantize(const float *, float *, int8_t *, int64_
                                         void *, void *);
 extern "C" int rlx_mi355x_qweight_create_at(int, const void *, size_t, int64_t, int64_t, void *, rlx_qweight **);
 extern "C" void rlx_mi355x_qweight_destroy(rlx_qweight *);
-extern "C" int rlx_mi355x_gguf_matmul_bt_grouped(const void *, int, const rlx_qweight *const *, float *const *, int, int64_t,
-                                                 void *, size_t, void *);
+extern "C" int rlx_mi355x_gguf_matmul_bt_batch(const void *const *, int, const rlx_qweight *const *, float *const *, int, int64_t,
+                                               void *, size_t, void *);
 
 namespace {
 
@@ -100,9 +100,10 @@ struct rlx_exec {
     std::vector<Node> nodes;
     std::vector<uint32_t> outputs;
     std::map<std::string, uint32_t> inputs, params;
-    // Launch schedule: one entry per kernel group. DequantMatMul nodes that read the same activations with the
-    // same scheme and k (q/k/v, gate/up) are fused into one grouped launch at the position of the first of them;
-    // they depend only on that input and on params, so moving the later ones up is safe.
+    // Launch schedule: one entry per kernel group. DequantMatMul nodes of the same scheme, batch and activation
+    // dtype whose activations are all produced before the first of them runs (same depth in the dependency graph)
+    // are issued as one batched launch at that position; they depend on nothing in between, so moving the later
+    // ones up is safe.
     std::vector<std::vector<uint32_t>> steps;
     rlx_compile_opts opts{};
     size_t arena_bytes = 0;
@@ -303,16 +304,27 @@ rlx_exec *rlx_mi355x_compile(const rlx_graph_desc *g, const rlx_compile_opts *op
         }
     }
 
+    // depth[i] = longest chain of compute nodes below node i (inputs and params are depth 0)
+    std::vector<int> depth(e->nodes.size(), 0);
+    for (uint32_t i = 0; i < g->n_nodes; i++) {
+        Node &nd = e->nodes[i];
+        if (nd.d.op_kind == RLX_OP_INPUT || nd.d.op_kind == RLX_OP_PARAM) continue;
+        int dmax = 0;
+        for (uint32_t j = 0; j < nd.d.n_inputs; j++) dmax = std::max(dmax, depth[nd.d.inputs[j]]);
+        depth[i] = dmax + 1;
+    }
     std::vector<bool> grouped(e->nodes.size(), false);
     for (uint32_t i = 0; i < g->n_nodes; i++) {
         Node &nd = e->nodes[i];
         if (grouped[i] || (nd.d.op_kind != RLX_OP_DEQUANT_MATMUL && nd.d.op_kind != RLX_OP_FAKE_QUANTIZE)) continue;
         std::vector<uint32_t> step{i};
         if (nd.d.op_kind == RLX_OP_DEQUANT_MATMUL) {
+            const uint32_t xdt = e->nodes[nd.d.inputs[0]].d.dtype;
             for (uint32_t j = i + 1; j < g->n_nodes; j++) {
                 Node &o = e->nodes[j];
-                if (!grouped[j] && o.d.op_kind == RLX_OP_DEQUANT_MATMUL && o.d.inputs[0] == nd.d.inputs[0] &&
-                    o.d.scheme == nd.d.scheme && o.k == nd.k && o.m == nd.m) {
+                if (!grouped[j] && o.d.op_kind == RLX_OP_DEQUANT_MATMUL && depth[j] == depth[i] &&
+                    o.d.scheme == nd.d.scheme && o.m == nd.m && e->nodes[o.d.inputs[0]].d.dtype == xdt &&
+                    (o.d.inputs[0] < i || e->nodes[o.d.inputs[0]].d.op_kind == RLX_OP_INPUT)) {
                     grouped[j] = true;
                     step.push_back(j);
                 }
@@ -453,21 +465,33 @@ static int enqueue_schedule(rlx_exec *e) {
     for (const std::vector<uint32_t> &step : e->steps) {
         Node &nd = e->nodes[step[0]];
         if (nd.d.op_kind == RLX_OP_DEQUANT_MATMUL) {
-            Node &x = e->nodes[nd.d.inputs[0]];
             std::vector<const rlx_qweight *> ws;
             std::vector<float *> outs;
-            for (uint32_t id : step) {
-                Node &w = e->nodes[e->nodes[id].d.inputs[1]];
+            std::vector<const void *> xs;
+            uint32_t xdt = RLX_F32;
+            for (size_t si = 0; si < step.size(); si++) {
+                Node &mm = e->nodes[step[si]];
+                Node &x = e->nodes[mm.d.inputs[0]];
+                Node &w = e->nodes[mm.d.inputs[1]];
                 if (!w.qw) {
                     set_error("run: packed weight '%s' was never set (set_param_typed(.., U8))", w.name.c_str());
                     return RLX_ERR_INVALID;
                 }
+                uint32_t dt = x.d.op_kind == RLX_OP_INPUT ? x.cur_dtype : x.d.dtype;
+                if (si > 0 && dt != xdt) {  // inputs of one batch were written with different dtypes: flush and start anew
+                    RLX_TRY(rlx_mi355x_gguf_matmul_bt_batch(xs.data(), (int)xdt, ws.data(), outs.data(), (int)ws.size(), nd.m,
+                                                            nullptr, 0, e->stream));
+                    ws.clear();
+                    outs.clear();
+                    xs.clear();
+                }
+                xdt = dt;
                 ws.push_back(w.qw);
-                outs.push_back((float *)e->ptr(e->nodes[id].slot));
+                outs.push_back((float *)e->ptr(mm.slot));
+                xs.push_back(e->ptr(x.slot));
             }
-            uint32_t xdt = x.d.op_kind == RLX_OP_INPUT ? x.cur_dtype : x.d.dtype;
-            RLX_TRY(rlx_mi355x_gguf_matmul_bt_grouped(e->ptr(x.slot), (int)xdt, ws.data(), outs.data(), (int)ws.size(), nd.m,
-                                                      nullptr, 0, e->stream));
+            RLX_TRY(rlx_mi355x_gguf_matmul_bt_batch(xs.data(), (int)xdt, ws.data(), outs.data(), (int)ws.size(), nd.m, nullptr,
+                                                    0, e->stream));
         } else {
             Node &x = e->nodes[nd.d.inputs[0]];
             if (x.d.op_kind == RLX_OP_INPUT && x.cur_dtype != RLX_F32) {

@@ -1,5 +1,6 @@
 // Operator-level entry points: packed weights in HBM, dequant, matmul dispatch, FakeQuantize.
 #include <algorithm>
+#include <cstdlib>
 #include <cstring>
 #include <vector>
 
@@ -24,16 +25,16 @@ struct DequantArgs {
     float *out;
     long long n, k, units;
 };
-constexpr int GEMV_MAX_SEG = 4;
+constexpr int GEMV_MAX_SEG = 8;
 struct GemvSeg {
     const uint8_t *w;
+    const void *x;
     float *out;
-    int n, row_tiles, wg_begin, pad;
+    int n, k, row_tiles, units, wg_begin, tiles_per_wg;
 };
 struct GemvArgs {
     GemvSeg seg[GEMV_MAX_SEG];
-    const void *x;
-    int nseg, m, k, units, kc_units, x_dtype, tiles_per_wg;
+    int nseg, m, kc_units, x_dtype, max_tiles_per_wg;
 };
 struct FqArgs {
     const float *x;
@@ -56,55 +57,65 @@ static int x_kind(int x_dtype) {
     }
 }
 
-// One decode launch over `count` (<= 4) weights that share scheme, k and the activations.
-static int launch_gemv(const void *x, int xk, const rlx_qweight *const *ws, float *const *outs, int count, int m,
+// One decode launch over `count` (<= GEMV_MAX_SEG) matmuls of one scheme, batch and activation dtype; each has
+// its own activations, K and N.
+static int launch_gemv(const void *const *xs, int xk, const rlx_qweight *const *ws, float *const *outs, int count, int m,
                        hipStream_t stream) {
-    const rlx_qweight *w0 = ws[0];
-    const Layout L = layout_of(w0->scheme);
+    const int scheme = ws[0]->scheme;
+    const Layout L = layout_of(scheme);
     const int rv = xk == 0 ? 2 * m : m;
     const int ng = (rv + 3) / 4;
-    const int units = (int)w0->dims.units;
     const bool r2 = rv <= 2;
-    KernelId id = w0->scheme == SCHEME_Q4_0   ? (r2 ? K_GEMV_Q4_0_R2 : K_GEMV_Q4_0_R4)
-                  : w0->scheme == SCHEME_Q8_0 ? (r2 ? K_GEMV_Q8_0_R2 : K_GEMV_Q8_0_R4)
-                                              : (r2 ? K_GEMV_Q4_K_R2 : K_GEMV_Q4_K_R4);
-    const int nwaves = std::max(1, std::min(8, units));
-    long long total_tiles = 0;
-    for (int i = 0; i < count; i++) total_tiles += ws[i]->dims.row_tiles;
-    // Row tiles per workgroup: the fewest that keep the grid within two workgroups per CU, so every workgroup is
-    // resident at once and the activations are staged once per ~36 KB x tiles of weights.
+    KernelId id = scheme == SCHEME_Q4_0   ? (r2 ? K_GEMV_Q4_0_R2 : K_GEMV_Q4_0_R4)
+                  : scheme == SCHEME_Q8_0 ? (r2 ? K_GEMV_Q8_0_R2 : K_GEMV_Q8_0_R4)
+                                          : (r2 ? K_GEMV_Q4_K_R2 : K_GEMV_Q4_K_R4);
+    static const int env_waves = getenv("RLX_GEMV_WAVES") ? atoi(getenv("RLX_GEMV_WAVES")) : 8;
+    static const int env_depth = getenv("RLX_GEMV_DEPTH") ? atoi(getenv("RLX_GEMV_DEPTH")) : 4;
+    static const int env_wgs_per_cu = getenv("RLX_GEMV_WGS_PER_CU") ? atoi(getenv("RLX_GEMV_WGS_PER_CU")) : 2;
+    if (id == K_GEMV_Q4_0_R2 && env_depth == 8) id = K_GEMV_Q4_0_R2_D8;
+    int max_units = 0;
+    long long work = 0;  // (tile, unit) items in the launch
+    for (int i = 0; i < count; i++) {
+        max_units = std::max(max_units, (int)ws[i]->dims.units);
+        work += ws[i]->dims.row_tiles * ws[i]->dims.units;
+    }
+    const int nwaves = std::max(1, std::min(std::min(16, std::max(1, env_waves)), max_units));
+    // Grid: about env_wgs_per_cu workgroups per CU, every one resident at once, each with the same number of
+    // (tile, unit) items: a segment with a longer K gets fewer row tiles per workgroup.
     const int cus = std::max(1, device_props().cu_count);
-    int tpw = (int)std::max<long long>(1, (total_tiles + 2 * cus - 1) / (2 * cus));
+    const long long target_items = std::max<long long>(1, (work + (long long)env_wgs_per_cu * cus - 1) / ((long long)env_wgs_per_cu * cus));
     const size_t slot_bytes = (size_t)ng * 256;
-    tpw = (int)std::min<size_t>(tpw, std::max<size_t>(1, (32 * 1024) / (nwaves * slot_bytes)));
-    const size_t part_bytes = (size_t)tpw * nwaves * slot_bytes;
+    const int tpw_cap = (int)std::max<size_t>(1, (32 * 1024) / (nwaves * slot_bytes));
+    GemvArgs a{};
+    int wg = 0, max_tpw = 1;
+    for (int i = 0; i < count; i++) {
+        const WeightDims &D = ws[i]->dims;
+        int tpw = (int)std::max<long long>(1, (target_items + D.units / 2) / D.units);
+        tpw = std::min(tpw, tpw_cap);
+        max_tpw = std::max(max_tpw, tpw);
+        a.seg[i] = GemvSeg{ws[i]->dev, xs[i], outs[i], (int)D.n, (int)D.k, (int)D.row_tiles, (int)D.units, wg, tpw};
+        wg += (int)((D.row_tiles + tpw - 1) / tpw);
+    }
+    const size_t part_bytes = (size_t)max_tpw * nwaves * slot_bytes;
     // LDS: partial sums + the staged activation chunk (rv rows of halfs, 16 B row padding) + Q4_K block sums.
-    const size_t budget = 64 * 1024;
+    // 80 KB keeps two workgroups per CU (160 KB LDS) and holds a 14336-wide f32 vector (hi + lo rows) in one chunk.
+    const size_t budget = 80 * 1024;
     auto stage_bytes = [&](int kcu) {
-        size_t b = ((size_t)(rv + 1) * ((size_t)kcu * L.unit_k + 8) * 2 + 15) & ~(size_t)15;  // + the all-zero row
-        if (w0->scheme == SCHEME_Q4K) b += (size_t)kcu * (L.unit_k / 32) * 16 * 4;
+        size_t b = ((size_t)rv * ((size_t)kcu * L.unit_k + 8) * 2 + 15) & ~(size_t)15;
+        if (scheme == SCHEME_Q4K) b += (size_t)kcu * (L.unit_k / 32) * 16 * 4;
         return b;
     };
-    int kcu = units;
+    int kcu = max_units;
     while (kcu > 1 && part_bytes + stage_bytes(kcu) > budget) kcu--;
     if (part_bytes + stage_bytes(kcu) > budget) {
         set_error("gemv: one K unit of %d activation rows does not fit LDS", rv);
         return RLX_ERR_INVALID;
     }
-    GemvArgs a{};
-    int wg = 0;
-    for (int i = 0; i < count; i++) {
-        a.seg[i] = GemvSeg{ws[i]->dev, outs[i], (int)ws[i]->dims.n, (int)ws[i]->dims.row_tiles, wg, 0};
-        wg += (int)((ws[i]->dims.row_tiles + tpw - 1) / tpw);
-    }
-    a.x = x;
     a.nseg = count;
     a.m = m;
-    a.k = (int)w0->dims.k;
-    a.units = units;
     a.kc_units = kcu;
     a.x_dtype = xk;
-    a.tiles_per_wg = tpw;
+    a.max_tiles_per_wg = max_tpw;
     void *params[] = {&a};
     return launch(id, (unsigned)wg, 1, (unsigned)nwaves * 64, (unsigned)(part_bytes + stage_bytes(kcu)), stream, params);
 }
@@ -167,22 +178,22 @@ size_t rlx_mi355x_gguf_matmul_workspace(int scheme, int x_dtype, int64_t m, int6
     return 0;
 }
 
-int rlx_mi355x_gguf_matmul_bt_grouped(const void *x_dev, int x_dtype, const rlx_qweight *const *ws,
-                                      float *const *outs_dev, int count, int64_t m, void *workspace,
-                                      size_t workspace_bytes, void *stream) {
+int rlx_mi355x_gguf_matmul_bt_batch(const void *const *xs_dev, int x_dtype, const rlx_qweight *const *ws,
+                                    float *const *outs_dev, int count, int64_t m, void *workspace, size_t workspace_bytes,
+                                    void *stream) {
     using namespace rlx;
     (void)workspace; (void)workspace_bytes;
-    if (!x_dev || !ws || !outs_dev || count <= 0 || m <= 0) {
+    if (!xs_dev || !ws || !outs_dev || count <= 0 || m <= 0) {
         set_error("gguf_matmul_bt: null argument, count=%d or m=%lld", count, (long long)m);
         return RLX_ERR_INVALID;
     }
     for (int i = 0; i < count; i++) {
-        if (!ws[i] || !outs_dev[i]) {
-            set_error("gguf_matmul_bt: null weight / output %d", i);
+        if (!ws[i] || !outs_dev[i] || !xs_dev[i]) {
+            set_error("gguf_matmul_bt: null activations / weight / output %d", i);
             return RLX_ERR_INVALID;
         }
-        if (ws[i]->scheme != ws[0]->scheme || ws[i]->dims.k != ws[0]->dims.k) {
-            set_error("gguf_matmul_bt_grouped: weight %d differs in scheme or k from weight 0", i);
+        if (ws[i]->scheme != ws[0]->scheme) {
+            set_error("gguf_matmul_bt_batch: weight %d differs in scheme from weight 0", i);
             return RLX_ERR_INVALID;
         }
     }
@@ -192,14 +203,18 @@ int rlx_mi355x_gguf_matmul_bt_grouped(const void *x_dev, int x_dtype, const rlx_
         return RLX_ERR_UNSUPPORTED;
     }
     const int64_t cap = xk == 0 ? 8 : 16;  // activation rows one MFMA pass holds
-    const size_t xrow = (size_t)ws[0]->dims.k * (xk == 0 ? 4 : 2);
+    const size_t esz = xk == 0 ? 4 : 2;
     for (int64_t r0 = 0; r0 < m; r0 += cap) {
         int rows = (int)std::min<int64_t>(cap, m - r0);
         for (int c0 = 0; c0 < count; c0 += GEMV_MAX_SEG) {
             int c = std::min(GEMV_MAX_SEG, count - c0);
             float *outs[GEMV_MAX_SEG];
-            for (int i = 0; i < c; i++) outs[i] = outs_dev[c0 + i] + r0 * ws[c0 + i]->dims.n;
-            RLX_TRY(launch_gemv((const uint8_t *)x_dev + r0 * xrow, xk, ws + c0, outs, c, rows, (hipStream_t)stream));
+            const void *xs[GEMV_MAX_SEG];
+            for (int i = 0; i < c; i++) {
+                outs[i] = outs_dev[c0 + i] + r0 * ws[c0 + i]->dims.n;
+                xs[i] = (const uint8_t *)xs_dev[c0 + i] + (size_t)r0 * ws[c0 + i]->dims.k * esz;
+            }
+            RLX_TRY(launch_gemv(xs, xk, ws + c0, outs, c, rows, (hipStream_t)stream));
         }
     }
     return RLX_OK;
@@ -207,7 +222,7 @@ int rlx_mi355x_gguf_matmul_bt_grouped(const void *x_dev, int x_dtype, const rlx_
 
 int rlx_mi355x_gguf_matmul_bt(const void *x_dev, int x_dtype, const rlx_qweight *w, float *out_dev, int64_t m,
                               void *workspace, size_t workspace_bytes, void *stream) {
-    return rlx_mi355x_gguf_matmul_bt_grouped(x_dev, x_dtype, &w, &out_dev, 1, m, workspace, workspace_bytes, stream);
+    return rlx_mi355x_gguf_matmul_bt_batch(&x_dev, x_dtype, &w, &out_dev, 1, m, workspace, workspace_bytes, stream);
 }
 
 int rlx_mi355x_fake_quantize(const float *x_dev, float *out_dev, int8_t *codes_dev, int64_t len, int64_t chan_dim,

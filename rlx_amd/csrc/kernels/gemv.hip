@@ -14,26 +14,28 @@ namespace rlx {
 
 enum XType : int { X_F32 = 0, X_BF16 = 1, X_F16 = 2 };
 
-constexpr int GEMV_MAX_SEG = 4;
+constexpr int GEMV_MAX_SEG = 8;
 
+// One weight matrix of a launch with its own activations, K and share of the grid.
 struct GemvSeg {
     const uint8_t *w;
-    float *out;
-    int n;          // logical rows of this matrix
-    int row_tiles;  // 16-row tiles in its device layout
-    int wg_begin;   // first workgroup of this segment
-    int pad;
+    const void *x;     // [m, k] activations this matrix multiplies
+    float *out;        // [m, n]
+    int n;             // logical rows of this matrix
+    int k;             // logical columns
+    int row_tiles;     // 16-row tiles in its device layout
+    int units;         // K units in its device layout
+    int wg_begin;      // first workgroup of this segment
+    int tiles_per_wg;  // row tiles per workgroup
 };
 
 struct GemvArgs {
     GemvSeg seg[GEMV_MAX_SEG];
-    const void *x;
     int nseg;
-    int m, k;
-    int units;         // K units in the device layout
-    int kc_units;      // units per LDS chunk
+    int m;
+    int kc_units;      // most units staged in LDS at once
     int x_dtype;
-    int tiles_per_wg;  // row tiles per workgroup
+    int max_tiles_per_wg;
 };
 
 constexpr int XS_PAD_HALFS = 8;      // 16 bytes of padding per LDS row: rows land in different bank groups
@@ -86,22 +88,24 @@ __device__ __forceinline__ float scale_of(uint2_t s, int t) {
     return half_bits_to_float((t & 1) ? (s[t >> 1] >> 16) : (s[t >> 1] & 0xFFFFu));
 }
 
-// A fragments of one lane for the NB 32-column blocks starting at staged column `col`. `xrow` already points at
-// the lane's virtual row and 8-column slice; lanes past the last real row point at an all-zero LDS row, so the
-// reads need no masking.
+// A fragments of one lane for the NB 32-column blocks starting at staged column `col`. `xrow` points at the lane's
+// virtual row and 8-column slice. Only lanes that own a real row (`live`) read LDS; the others keep whatever their
+// registers held: row i of A only feeds row i of the product, and product rows >= rv are never read back.
 template <int NB>
-__device__ __forceinline__ void load_afrags(const half_t *xrow, int col, Frag (&a)[NB]) {
+__device__ __forceinline__ void load_afrags(const half_t *xrow, bool live, int col, Frag (&a)[NB]) {
+    if (live) {
 #pragma unroll
-    for (int t = 0; t < NB; t++) a[t].u4 = *(const uint4_t *)(xrow + col + t * 32);
+        for (int t = 0; t < NB; t++) a[t].u4 = *(const uint4_t *)(xrow + col + t * 32);
+    }
 }
 
 template <int SCHEME, int NREG>
-__device__ __forceinline__ void compute_unit(const UnitRegs<SCHEME> &w, const half_t *xrow, const float *sxs, int g,
-                                             int ucol, int ublk, float acc[4]) {
+__device__ __forceinline__ void compute_unit(const UnitRegs<SCHEME> &w, const half_t *xrow, bool live, Frag (&a)[4],
+                                             const float *sxs, int g, int ucol, int ublk, float acc[4]) {
     const float4_t zero = {0.f, 0.f, 0.f, 0.f};
     if constexpr (SCHEME == SCHEME_Q4_0) {
-        Frag a[4], b[4];
-        load_afrags<4>(xrow, ucol, a);
+        Frag b[4];
+        load_afrags<4>(xrow, live, ucol, a);
 #pragma unroll
         for (int t = 0; t < 4; t++) unpack_q4<8>(w.q[t], b[t]);
         float4_t blk[4];
@@ -114,8 +118,8 @@ __device__ __forceinline__ void compute_unit(const UnitRegs<SCHEME> &w, const ha
             for (int r = 0; r < NREG; r++) acc[r] = __builtin_fmaf(d, blk[t][r], acc[r]);
         }
     } else if constexpr (SCHEME == SCHEME_Q8_0) {
-        Frag a[4], b[4];
-        load_afrags<4>(xrow, ucol, a);
+        Frag b[4];
+        load_afrags<4>(xrow, live, ucol, a);
 #pragma unroll
         for (int t = 0; t < 4; t++) {
             const uint4_t &q = (t < 2) ? w.q0 : w.q1;
@@ -137,8 +141,8 @@ __device__ __forceinline__ void compute_unit(const UnitRegs<SCHEME> &w, const ha
         q4k_scales(w.meta[1], w.meta[2], w.meta[3], sc, mn);
 #pragma unroll
         for (int h = 0; h < 2; h++) {
-            Frag a[4], b[4];
-            load_afrags<4>(xrow, ucol + h * 128, a);
+            Frag b[4];
+            load_afrags<4>(xrow, live, ucol + h * 128, a);
             const uint4_t &q = h ? w.q1 : w.q0;
 #pragma unroll
             for (int t = 0; t < 4; t++) unpack_q4<0>(q[t], b[t]);
@@ -162,7 +166,7 @@ __device__ __forceinline__ void compute_unit(const UnitRegs<SCHEME> &w, const ha
 }
 
 // Convert one K chunk of the activations into LDS as halfs: f32 -> hi rows [0,m) + lo rows [m,2m); 16-bit -> rows [0,m).
-__device__ __forceinline__ void stage_x(const GemvArgs &a, half_t *xs, int row_stride, int k0, int kc) {
+__device__ __forceinline__ void stage_x(const GemvArgs &a, const GemvSeg &sg, half_t *xs, int row_stride, int k0, int kc) {
     const int tid = threadIdx.x, nt = blockDim.x;
     const int q4 = kc >> 2;  // groups of 4 columns
     for (int idx = tid; idx < a.m * q4; idx += nt) {
@@ -170,7 +174,7 @@ __device__ __forceinline__ void stage_x(const GemvArgs &a, half_t *xs, int row_s
         int kk = k0 + c;
         if (a.x_dtype == X_F32) {
             float4_t v = {0.f, 0.f, 0.f, 0.f};
-            if (kk < a.k) v = *(const float4_t *)((const float *)a.x + (long long)row * a.k + kk);
+            if (kk < sg.k) v = *(const float4_t *)((const float *)sg.x + (long long)row * sg.k + kk);
             half4_t hi, lo;
 #pragma unroll
             for (int e = 0; e < 4; e++) {
@@ -182,7 +186,7 @@ __device__ __forceinline__ void stage_x(const GemvArgs &a, half_t *xs, int row_s
             *(half4_t *)(xs + (a.m + row) * row_stride + c) = lo;
         } else {
             uint2_t raw = {0, 0};
-            if (kk < a.k) raw = *(const uint2_t *)((const uint16_t *)a.x + (long long)row * a.k + kk);
+            if (kk < sg.k) raw = *(const uint2_t *)((const uint16_t *)sg.x + (long long)row * sg.k + kk);
             if (a.x_dtype == X_BF16) {
                 half4_t h;
 #pragma unroll
@@ -203,7 +207,8 @@ __device__ __forceinline__ void stage_x(const GemvArgs &a, half_t *xs, int row_s
 //     units of weights in flight in registers, so the stream of 16-byte loads never drains between tiles;
 //   * at the end of each (tile, chunk) the wave adds its partial sums into its own LDS slot; one barrier at the
 //     very end, then the slots of all waves are added in a fixed order and written out (deterministic).
-// A launch can carry up to GEMV_MAX_SEG weight matrices that share the activations (q/k/v, gate/up).
+// A launch can carry up to GEMV_MAX_SEG independent matmuls (each with its own activations, K and N): q/k/v and
+// gate/up of a layer, or every projection whose inputs are ready at the same point of the schedule.
 template <int SCHEME, int NREG, int DEPTH>
 __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
     constexpr Layout L = layout_of(SCHEME);
@@ -223,28 +228,27 @@ __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
     for (int i = 1; i < GEMV_MAX_SEG; i++)
         if (i < a.nseg && (int)blockIdx.x >= a.seg[i].wg_begin) s = i;
     const GemvSeg seg = a.seg[s];
-    const int tile0 = ((int)blockIdx.x - seg.wg_begin) * a.tiles_per_wg;
-    const int ntiles = min(a.tiles_per_wg, seg.row_tiles - tile0);
+    const int tile0 = ((int)blockIdx.x - seg.wg_begin) * seg.tiles_per_wg;
+    const int ntiles = min(seg.tiles_per_wg, seg.row_tiles - tile0);
+    const int kc_units = min(a.kc_units, seg.units);
 
-    const int kc = a.kc_units * L.unit_k;
+    const int kc = kc_units * L.unit_k;
     const int row_stride = kc + XS_PAD_HALFS;
-    // LDS: [partial sums: tiles_per_wg x nwaves x (4 ng) x 16 f32][staged activations: rv rows + one zero row]
-    //      [Q4_K block sums]
+    // LDS: [partial sums: tiles_per_wg x nwaves x (4 ng) x 16 f32][staged activations: rv rows][Q4_K block sums]
     const int slot_floats = ng * 64;
     float *part = (float *)smem;
-    const size_t part_bytes = (size_t)a.tiles_per_wg * nwaves * slot_floats * 4;
+    const size_t part_bytes = (size_t)a.max_tiles_per_wg * nwaves * slot_floats * 4;
     half_t *xs = (half_t *)(smem + part_bytes);
-    float *sxs = (float *)(smem + part_bytes + (((size_t)(rv + 1) * row_stride * 2 + 15) & ~(size_t)15));  // [blk][16]
-    const half_t *xrow = xs + min(nrow, rv) * row_stride + g * 8;  // this lane's A row (row rv is all zeros)
+    float *sxs = (float *)(smem + part_bytes + (((size_t)rv * row_stride * 2 + 15) & ~(size_t)15));  // [blk][16]
+    const half_t *xrow = xs + min(nrow, rv - 1) * row_stride + g * 8;  // this lane's A row
 
-    for (int i = tid; i < a.tiles_per_wg * nwaves * slot_floats; i += blockDim.x) part[i] = 0.f;
-    for (int i = tid; i < row_stride / 2; i += blockDim.x) ((uint32_t *)(xs + rv * row_stride))[i] = 0u;
+    for (int i = tid; i < ntiles * nwaves * slot_floats; i += blockDim.x) part[i] = 0.f;
 
-    const uint8_t *wbase = seg.w + (long long)tile0 * a.units * L.unit_bytes;
-    const long long tile_bytes = (long long)a.units * L.unit_bytes;
+    const uint8_t *wbase = seg.w + (long long)tile0 * seg.units * L.unit_bytes;
+    const long long tile_bytes = (long long)seg.units * L.unit_bytes;
 
-    for (int u0 = 0; u0 < a.units; u0 += a.kc_units) {
-        const int nu = min(a.kc_units, a.units - u0);  // units in this chunk
+    for (int u0 = 0; u0 < seg.units; u0 += kc_units) {
+        const int nu = min(kc_units, seg.units - u0);  // units in this chunk
         // This wave's items: for each tile, units wave, wave + nwaves, ... < nu. Two cursors walk them: `pf_*` issues
         // loads DEPTH items ahead into a register ring, `cu_*` consumes.
         const int my_units = wave < nu ? (nu - wave + nwaves - 1) / nwaves : 0;
@@ -271,7 +275,7 @@ __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
             prefetch(ring[d]);
         }
         if (u0 > 0) __syncthreads();  // previous chunk fully consumed
-        stage_x(a, xs, row_stride, u0 * L.unit_k, nu * L.unit_k);
+        stage_x(a, seg, xs, row_stride, u0 * L.unit_k, nu * L.unit_k);
         __syncthreads();
         if constexpr (SCHEME == SCHEME_Q4K) {
             const int nblk = nu * BLK_PER_UNIT;
@@ -292,6 +296,9 @@ __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
             __syncthreads();
         }
         float acc[4] = {0.f, 0.f, 0.f, 0.f};
+        Frag afr[4];
+#pragma unroll
+        for (int t = 0; t < 4; t++) afr[t].u4 = uint4_t{0, 0, 0, 0};
         int cu_t = 0, cu_u = wave;
         for (int base = 0; base < nitems; base += DEPTH) {
 #pragma unroll
@@ -299,7 +306,7 @@ __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
                 if (base + d < nitems) {
                     UnitRegs<SCHEME> cur = ring[d];
                     prefetch(ring[d]);
-                    compute_unit<SCHEME, NREG>(cur, xrow, sxs, g, cu_u * L.unit_k, cu_u * BLK_PER_UNIT, acc);
+                    compute_unit<SCHEME, NREG>(cur, xrow, nrow < rv, afr, sxs, g, cu_u * L.unit_k, cu_u * BLK_PER_UNIT, acc);
                     cu_u += nwaves;
                     if (cu_u >= nu) {  // last unit of this tile for this wave: bank the partial sums
                         if (has_rows) {
@@ -336,12 +343,13 @@ __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
 }  // namespace rlx
 
 #define RLX_GEMV_INST(name, SCHEME, NREG, DEPTH)                                                            \
-    extern "C" __global__ __launch_bounds__(512) void name(rlx::GemvArgs a) {                                \
+    extern "C" __global__ __launch_bounds__(1024) void name(rlx::GemvArgs a) {                               \
         rlx::gemv_body<SCHEME, NREG, DEPTH>(a);                                                               \
     }
 
 // NREG = 2: at most two virtual rows (m = 1 f32, or m <= 2 16-bit); NREG = 4 otherwise.
 RLX_GEMV_INST(rlx_gemv_q4_0_r2, rlx::SCHEME_Q4_0, 2, 4)
+RLX_GEMV_INST(rlx_gemv_q4_0_r2_d8, rlx::SCHEME_Q4_0, 2, 8)
 RLX_GEMV_INST(rlx_gemv_q4_0_r4, rlx::SCHEME_Q4_0, 4, 4)
 RLX_GEMV_INST(rlx_gemv_q8_0_r2, rlx::SCHEME_Q8_0, 2, 3)
 RLX_GEMV_INST(rlx_gemv_q8_0_r4, rlx::SCHEME_Q8_0, 4, 3)

@@ -344,9 +344,10 @@ def test_graph_typed_bf16_input(oracle):
     assert rel_err(got, oracle.gguf_matmul_f64(x, packed, m, k, n, Q4K)) <= TOL
 
 
-def test_graph_fuses_matmuls_that_share_an_input(oracle):
-    # q/k/v-style: three weights, one activation vector -> one grouped launch; outputs must be those of three
-    # separate matmuls. A fourth weight with a different k stays on its own.
+def test_graph_batches_independent_matmuls(oracle):
+    # q/k/v-style: three weights on one activation vector plus a fourth matmul with its own activations and a
+    # different k: all four are ready at the same point of the schedule and go out as one batched launch; outputs
+    # must be those of four separate matmuls, eagerly and on every hipGraph replay.
     k, ns = 1024, [256, 64, 48]
     rng = np.random.default_rng(50)
     x = rng.standard_normal((2, k)).astype(np.float32)
