@@ -39,6 +39,7 @@ enum KernelId : int {
     K_FQ_COL_ABSMAX, K_FQ_SEG_ABSMAX, K_FQ_FLAT_ABSMAX, K_FQ_SCALE, K_FQ_COL_APPLY, K_FQ_FLAT_APPLY, K_FQ_FLAT4_APPLY,
     K_FILL_U32,
     K_GEMV_Q4_0_R2, K_GEMV_Q4_0_R2_D8, K_GEMV_Q4_0_R4, K_GEMV_Q8_0_R2, K_GEMV_Q8_0_R4, K_GEMV_Q4_K_R2, K_GEMV_Q4_K_R4,
+    K_GEMM_Q4_K, K_GEMM_Q4_0, K_GEMM_Q8_0, K_XPREP,
     K_COUNT
 };
 
@@ -46,6 +47,7 @@ enum KernelId : int {
 int runtime_init();
 // Launches kernel `id`; `args` points at the kernel's single by-value argument struct (or packed scalars).
 int launch(KernelId id, unsigned gx, unsigned gy, unsigned bx, unsigned shmem, hipStream_t stream, void **params);
+int launch3(KernelId id, unsigned gx, unsigned gy, unsigned gz, unsigned bx, unsigned shmem, hipStream_t stream, void **params);
 
 struct DeviceProps {
     int cu_count;

@@ -15,6 +15,8 @@
 #include "common.hpp"
 
 struct rlx_qweight;
+extern "C" int rlx_mi355x_gguf_matmul_bt(const void *, int, const rlx_qweight *, float *, int64_t, void *, size_t, void *);
+extern "C" size_t rlx_mi355x_gguf_matmul_workspace(int, int, int64_t, int64_t, int64_t);
 extern "C" int rlx_mi355x_fake_quantize(const float *, float *, int8_t *, int64_t, int64_t, int64_t, int, int, float, float *, int,
                                         void *, void *);
 extern "C" int rlx_mi355x_qweight_create_at(int, const void *, size_t, int64_t, int64_t, void *, rlx_qweight **);
@@ -355,6 +357,8 @@ rlx_exec *rlx_mi355x_compile(const rlx_graph_desc *g, const rlx_compile_opts *op
             nd.aux = take((size_t)nd.chan_dim * 8);
             nd.codes = take((size_t)nd.numel);
         }
+        if (nd.d.op_kind == RLX_OP_DEQUANT_MATMUL && nd.m > 8)  // prefill workspace, sized for f32 activations
+            nd.aux = take(rlx_mi355x_gguf_matmul_workspace((int)nd.d.scheme, RLX_F32, nd.m, nd.k, nd.n));
     }
     e->arena_bytes = off;
 
@@ -464,7 +468,20 @@ int rlx_exec_write_input(rlx_exec *e, const char *name, const void *data, size_t
 static int enqueue_schedule(rlx_exec *e) {
     for (const std::vector<uint32_t> &step : e->steps) {
         Node &nd = e->nodes[step[0]];
-        if (nd.d.op_kind == RLX_OP_DEQUANT_MATMUL) {
+        if (nd.d.op_kind == RLX_OP_DEQUANT_MATMUL && nd.m > 8) {
+            for (uint32_t id : step) {  // prefill: one GEMM per node, each with its own workspace slot
+                Node &mm = e->nodes[id];
+                Node &x = e->nodes[mm.d.inputs[0]];
+                Node &w = e->nodes[mm.d.inputs[1]];
+                if (!w.qw) {
+                    set_error("run: packed weight '%s' was never set (set_param_typed(.., U8))", w.name.c_str());
+                    return RLX_ERR_INVALID;
+                }
+                uint32_t dt = x.d.op_kind == RLX_OP_INPUT ? x.cur_dtype : x.d.dtype;
+                RLX_TRY(rlx_mi355x_gguf_matmul_bt(e->ptr(x.slot), (int)dt, w.qw, (float *)e->ptr(mm.slot), mm.m, e->ptr(mm.aux),
+                                                  mm.aux.size, e->stream));
+            }
+        } else if (nd.d.op_kind == RLX_OP_DEQUANT_MATMUL) {
             std::vector<const rlx_qweight *> ws;
             std::vector<float *> outs;
             std::vector<const void *> xs;

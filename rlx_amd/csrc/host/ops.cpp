@@ -48,6 +48,20 @@ struct FqArgs {
     int scale_mode, round_mode, rows_per_block;
 };
 
+struct GemmArgs {
+    const uint8_t *w;
+    const void *xh;
+    const void *sxh;
+    float *out;
+    int m_rows, m_out, n, k_pad, units, row_tiles, pair_rows, steps_per_split, use_atomics;
+};
+struct XPrepArgs {
+    const void *x;
+    void *xh;
+    void *sxh;
+    int m, k, k_pad, m_rows, x_dtype;
+};
+
 static int x_kind(int x_dtype) {
     switch (x_dtype) {
     case RLX_F32: return 0;
@@ -120,6 +134,60 @@ static int launch_gemv(const void *const *xs, int xk, const rlx_qweight *const *
     return launch(id, (unsigned)wg, 1, (unsigned)nwaves * 64, (unsigned)(part_bytes + stage_bytes(kcu)), stream, params);
 }
 
+struct GemmPlan {
+    int64_t m_rows, k_pad;
+    size_t xh_bytes, sxh_bytes;
+};
+static GemmPlan gemm_plan(int scheme, int xk, int64_t m, int64_t k) {
+    GemmPlan p;
+    const int64_t rv = xk == 0 ? 2 * m : m;
+    p.m_rows = (rv + 255) / 256 * 256;
+    p.k_pad = (k + 255) / 256 * 256;
+    p.xh_bytes = ((size_t)p.m_rows * p.k_pad * 2 + 255) & ~(size_t)255;
+    p.sxh_bytes = scheme == SCHEME_Q4K ? (size_t)p.m_rows * (p.k_pad / 256) * 32 : 0;
+    return p;
+}
+
+// Prefill path: convert the activations once (xprep), then the MFMA GEMM; K is split across workgroups (atomic
+// accumulation into a zeroed output) only when the tile grid alone would leave most CUs idle.
+static int launch_gemm(const void *x, int xk, const rlx_qweight *w, float *out, int64_t m, void *workspace,
+                       size_t workspace_bytes, hipStream_t stream) {
+    const Layout L = layout_of(w->scheme);
+    const GemmPlan p = gemm_plan(w->scheme, xk, m, w->dims.k);
+    if (!workspace || workspace_bytes < p.xh_bytes + p.sxh_bytes) {
+        set_error("gguf_matmul_bt: m=%lld needs a %zu-byte workspace, got %zu", (long long)m, p.xh_bytes + p.sxh_bytes,
+                  workspace_bytes);
+        return RLX_ERR_INVALID;
+    }
+    if ((uintptr_t)workspace % 16 != 0 || (uintptr_t)x % 16 != 0) {
+        set_error("gguf_matmul_bt: activations and workspace must be 16-byte aligned");
+        return RLX_ERR_INVALID;
+    }
+    void *xh = workspace;
+    void *sxh = p.sxh_bytes ? (uint8_t *)workspace + p.xh_bytes : nullptr;
+    XPrepArgs xa{x, xh, sxh, (int)m, (int)w->dims.k, (int)p.k_pad, (int)p.m_rows, xk};
+    void *xparams[] = {&xa};
+    const long long waves = p.m_rows * (p.k_pad / 256);
+    RLX_TRY(launch(K_XPREP, (unsigned)((waves + 3) / 4), 1, 256, 0, stream, xparams));
+
+    const int steps_per_unit = L.unit_k / 64;
+    const int gx = (int)((w->dims.row_tiles * 16 + 127) / 128), gy = (int)(p.m_rows / 256);
+    const int cus = std::max(1, device_props().cu_count);
+    int split = 1;
+    if ((long long)gx * gy * 5 < (long long)cus * 4) split = (int)std::min<long long>(w->dims.units, cus / ((long long)gx * gy));
+    split = std::max(1, split);
+    const int units_per_split = (int)((w->dims.units + split - 1) / split);
+    split = (int)((w->dims.units + units_per_split - 1) / units_per_split);
+    if (split > 1) RLX_TRY(rlx_mi355x_memset_u32(out, 0, (size_t)m * w->dims.n, stream));
+    GemmArgs a{w->dev, xh, sxh, out, (int)p.m_rows, (int)m, (int)w->dims.n, (int)p.k_pad, (int)w->dims.units,
+               (int)w->dims.row_tiles, xk == 0 ? 1 : 0, units_per_split * steps_per_unit, split > 1 ? 1 : 0};
+    void *params[] = {&a};
+    KernelId id = w->scheme == SCHEME_Q4K ? K_GEMM_Q4_K : w->scheme == SCHEME_Q4_0 ? K_GEMM_Q4_0 : K_GEMM_Q8_0;
+    RLX_TRY(runtime_init());
+    RLX_TRY(launch3(id, (unsigned)gx, (unsigned)gy, (unsigned)split, 512, 2 * (32 + 16) * 1024, stream, params));
+    return RLX_OK;
+}
+
 }  // namespace rlx
 
 extern "C" {
@@ -174,15 +242,18 @@ int rlx_mi355x_dequant(const rlx_qweight *w, float *out_dev, void *stream) {
 }
 
 size_t rlx_mi355x_gguf_matmul_workspace(int scheme, int x_dtype, int64_t m, int64_t k, int64_t n) {
-    (void)scheme; (void)x_dtype; (void)m; (void)k; (void)n;
-    return 0;
+    using namespace rlx;
+    (void)n;
+    int xk = x_kind(x_dtype);
+    if (xk < 0 || layout_of(scheme).unit_k == 0 || m <= (xk == 0 ? 8 : 16)) return 0;  // decode path: no workspace
+    GemmPlan p = gemm_plan(scheme, xk, m, k);
+    return p.xh_bytes + p.sxh_bytes;
 }
 
 int rlx_mi355x_gguf_matmul_bt_batch(const void *const *xs_dev, int x_dtype, const rlx_qweight *const *ws,
                                     float *const *outs_dev, int count, int64_t m, void *workspace, size_t workspace_bytes,
                                     void *stream) {
     using namespace rlx;
-    (void)workspace; (void)workspace_bytes;
     if (!xs_dev || !ws || !outs_dev || count <= 0 || m <= 0) {
         set_error("gguf_matmul_bt: null argument, count=%d or m=%lld", count, (long long)m);
         return RLX_ERR_INVALID;
@@ -202,8 +273,13 @@ int rlx_mi355x_gguf_matmul_bt_batch(const void *const *xs_dev, int x_dtype, cons
         set_error("gguf_matmul_bt: activation dtype %d unsupported (F32, BF16, F16 only)", x_dtype);
         return RLX_ERR_UNSUPPORTED;
     }
-    const int64_t cap = xk == 0 ? 8 : 16;  // activation rows one MFMA pass holds
+    const int64_t cap = xk == 0 ? 8 : 16;  // activation rows one decode pass holds
     const size_t esz = xk == 0 ? 4 : 2;
+    if (m > cap) {  // prefill: one GEMM per weight, sharing the workspace (same stream, so launches are ordered)
+        for (int i = 0; i < count; i++)
+            RLX_TRY(launch_gemm(xs_dev[i], xk, ws[i], outs_dev[i], m, workspace, workspace_bytes, (hipStream_t)stream));
+        return RLX_OK;
+    }
     for (int64_t r0 = 0; r0 < m; r0 += cap) {
         int rows = (int)std::min<int64_t>(cap, m - r0);
         for (int c0 = 0; c0 < count; c0 += GEMV_MAX_SEG) {

@@ -27,6 +27,7 @@ static const char *const kKernelNames[K_COUNT] = {
     "rlx_fq_flat_apply", "rlx_fq_flat4_apply",
     "rlx_fill_u32",
     "rlx_gemv_q4_0_r2", "rlx_gemv_q4_0_r2_d8", "rlx_gemv_q4_0_r4", "rlx_gemv_q8_0_r2", "rlx_gemv_q8_0_r4", "rlx_gemv_q4_k_r2", "rlx_gemv_q4_k_r4",
+    "rlx_gemm_q4_k", "rlx_gemm_q4_0", "rlx_gemm_q8_0", "rlx_xprep",
 };
 
 static std::once_flag g_once;
@@ -78,19 +79,24 @@ int runtime_init() {
 
 const DeviceProps &device_props() { return g_props; }
 
-int launch(KernelId id, unsigned gx, unsigned gy, unsigned bx, unsigned shmem, hipStream_t stream, void **params) {
+int launch3(KernelId id, unsigned gx, unsigned gy, unsigned gz, unsigned bx, unsigned shmem, hipStream_t stream,
+            void **params) {
     RLX_TRY(runtime_init());
-    if (gx == 0 || gy == 0 || bx == 0 || bx > 1024 || gy > 65535) {
-        set_error("launch(%s): bad geometry grid=(%u,%u) block=%u", kKernelNames[id], gx, gy, bx);
+    if (gx == 0 || gy == 0 || gz == 0 || bx == 0 || bx > 1024 || gy > 65535 || gz > 65535 || shmem > 160 * 1024) {
+        set_error("launch(%s): bad geometry grid=(%u,%u,%u) block=%u lds=%u", kKernelNames[id], gx, gy, gz, bx, shmem);
         return RLX_ERR_INVALID;
     }
-    hipError_t e = hipModuleLaunchKernel(g_fn[id], gx, gy, 1, bx, 1, 1, shmem, stream, params, nullptr);
+    hipError_t e = hipModuleLaunchKernel(g_fn[id], gx, gy, gz, bx, 1, 1, shmem, stream, params, nullptr);
     if (e != hipSuccess) {
-        set_error("hipModuleLaunchKernel(%s, grid=(%u,%u), block=%u, lds=%u): %s", kKernelNames[id], gx, gy, bx, shmem,
-                  hipGetErrorString(e));
+        set_error("hipModuleLaunchKernel(%s, grid=(%u,%u,%u), block=%u, lds=%u): %s", kKernelNames[id], gx, gy, gz, bx,
+                  shmem, hipGetErrorString(e));
         return RLX_ERR_HIP;
     }
     return RLX_OK;
+}
+
+int launch(KernelId id, unsigned gx, unsigned gy, unsigned bx, unsigned shmem, hipStream_t stream, void **params) {
+    return launch3(id, gx, gy, 1, bx, shmem, stream, params);
 }
 
 }  // namespace rlx

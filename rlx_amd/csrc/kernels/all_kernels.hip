@@ -1,4 +1,5 @@
 // Single translation unit for the gfx950 code object the host library embeds and loads with hipModuleLoadData.
 #include "dequant.hip"
 #include "fakequant.hip"
+#include "gemm.hip"
 #include "gemv.hip"

@@ -150,16 +150,28 @@ class QWeight:
             pass
 
 
-def gguf_matmul_bt_device(x_dev, x_dtype, w: QWeight, out_dev, m, stream=None):
-    _lib.check(_lib.lib().rlx_mi355x_gguf_matmul_bt(x_dev.ptr, int(x_dtype), w.ptr, out_dev.ptr, m, None, 0, stream))
+def matmul_workspace_bytes(w: QWeight, x_dtype, m):
+    return _lib.lib().rlx_mi355x_gguf_matmul_workspace(int(w.scheme), int(x_dtype), m, w.k, w.n)
+
+
+def gguf_matmul_bt_device(x_dev, x_dtype, w: QWeight, out_dev, m, stream=None, workspace=None):
+    """out_dev[m, n] = x_dev[m, k] . W^T on `stream`. `workspace`: DeviceBuffer of matmul_workspace_bytes() (prefill only)."""
+    need = matmul_workspace_bytes(w, x_dtype, m)
+    if need and workspace is None:
+        workspace = DeviceBuffer(need)
+    _lib.check(_lib.lib().rlx_mi355x_gguf_matmul_bt(x_dev.ptr, int(x_dtype), w.ptr, out_dev.ptr, m,
+                                                   workspace.ptr if workspace else None,
+                                                   workspace.nbytes if workspace else 0, stream))
+    return workspace
 
 
 def gguf_matmul_bt(x, w: QWeight, m, x_dtype=DType.F32):
     """Host convenience: upload x ([m,k]; f32, or uint16 bit patterns for BF16 / float16 for F16), run, download [m,n]."""
     xd = DeviceBuffer.from_numpy(x)
     od = DeviceBuffer(m * w.n * 4)
-    gguf_matmul_bt_device(xd, x_dtype, w, od, m)
+    ws = gguf_matmul_bt_device(xd, x_dtype, w, od, m)
     sync()
+    del ws
     return od.to_numpy(np.float32).reshape(m, w.n)
 
 

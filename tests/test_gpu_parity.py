@@ -176,9 +176,9 @@ def test_decode_ragged_shapes(oracle, scheme, n, k):
     check_matmul(oracle, scheme, n, k, 3, seed=n)
 
 
-def test_decode_more_rows_than_one_pass(oracle):
-    check_matmul(oracle, Q4_0, 128, 256, 20, seed=4)           # f32: 8 rows per pass -> 3 passes
-    check_matmul(oracle, Q4K, 64, 512, 37, x_dtype=DType.BF16, seed=5)  # 16 rows per pass -> 3 passes
+def test_rows_just_past_the_decode_limit(oracle):
+    check_matmul(oracle, Q4_0, 128, 256, 20, seed=4)           # f32: more than 8 rows -> prefill kernel
+    check_matmul(oracle, Q4K, 64, 512, 37, x_dtype=DType.BF16, seed=5)  # more than 16 rows -> prefill kernel
 
 
 def test_decode_large_k_is_chunked(oracle):
@@ -377,3 +377,52 @@ def test_graph_batches_independent_matmuls(oracle):
         if attempt == "eager":
             c.capture()
         x = (x * np.float32(1.5)).astype(np.float32)  # new inputs each replay: the graph must read them afresh
+
+
+# ------------------------------------------------------------------ prefill GEMM (m > 16)
+
+@pytest.mark.parametrize("scheme", [Q4K, Q4_0, Q8_0])
+@pytest.mark.parametrize("m,n,k,x_dtype", [(64, 256, 512, DType.BF16), (300, 200, 768, DType.BF16),
+                                           (40, 128, 1024, DType.F32), (512, 384, 2048, DType.F16)])
+def test_gemm_small(oracle, scheme, m, n, k, x_dtype):
+    check_matmul(oracle, scheme, n, k, m, x_dtype=x_dtype, seed=m + n)
+
+
+def test_config3_q4k_gemm_m512_slices(oracle):
+    # BASELINE config 3 shapes at full size; the f64 oracle is run on column windows (it is O(m n k) scalar work)
+    for n, k in [(14336, 4096), (4096, 14336)]:
+        packed, _ = make_weights(Q4K, n, k, seed=n % 89)
+        x = oracle.bf16_round(np.random.default_rng(n).standard_normal((512, k)).astype(np.float32))
+        w = ops.QWeight(Q4K, packed, n, k)
+        got = ops.gguf_matmul_bt(f32_to_bf16_bits(x), w, 512, DType.BF16)
+        for n0 in (0, n // 2 - 8, n - 24):
+            ref = oracle.gguf_matmul_f64(x, packed, 512, k, n, Q4K, n0, n0 + 24)
+            err = rel_err(got[:, n0:n0 + 24], ref)
+            say("   q4_k gemm", n, k, "cols", n0, "max rel err", err)
+            assert err <= TOL
+        # every output at once through a size-independent property: row sums of y against (x . sum of W rows)
+        wsum = oracle.dequant(Q4K, packed, n * k).reshape(n, k).astype(np.float64).sum(axis=0)
+        want = x.astype(np.float64) @ wsum
+        assert np.max(np.abs(got.astype(np.float64).sum(axis=1) - want) / np.maximum(np.abs(want), 1.0)) < 2e-3
+
+
+def test_gemm_q4_0_70b_shape_bf16(oracle):
+    # BASELINE config 5, one projection at M = 64 and 256
+    n, k = 1024, 8192
+    packed, _ = make_weights(Q4_0, n, k, std=0.015, seed=77)
+    w = ops.QWeight(Q4_0, packed, n, k)
+    for m in (64, 256):
+        x = oracle.bf16_round(np.random.default_rng(m).standard_normal((m, k)).astype(np.float32))
+        got = ops.gguf_matmul_bt(f32_to_bf16_bits(x), w, m, DType.BF16)
+        ref = oracle.gguf_matmul_f64(x, packed, m, k, n, Q4_0, 0, 64)
+        err = rel_err(got[:, :64], ref)
+        say("   q4_0 gemm m", m, "max rel err", err)
+        assert err <= TOL
+
+
+def test_graph_prefill_through_session(oracle):
+    m, k, n = 96, 512, 160
+    packed, _ = make_weights(Q4K, n, k, seed=81)
+    x = np.random.default_rng(82).standard_normal((m, k)).astype(np.float32)
+    got = run_dq(packed, Q4K, x, m, k, n)
+    assert rel_err(got, oracle.gguf_matmul_f64(x, packed, m, k, n, Q4K)) <= TOL
