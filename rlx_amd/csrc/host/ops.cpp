@@ -176,7 +176,8 @@ static int launch_gemm(const void *x, int xk, const rlx_qweight *w, float *out, 
     int split = 1;
     if ((long long)gx * gy * 5 < (long long)cus * 4) split = (int)std::min<long long>(w->dims.units, cus / ((long long)gx * gy));
     split = std::max(1, split);
-    const int units_per_split = (int)((w->dims.units + split - 1) / split);
+    int units_per_split = (int)((w->dims.units + split - 1) / split);
+    if (steps_per_unit == 2) units_per_split = (units_per_split + 1) & ~1;  // keep every split a multiple of 4 steps
     split = (int)((w->dims.units + units_per_split - 1) / units_per_split);
     if (split > 1) RLX_TRY(rlx_mi355x_memset_u32(out, 0, (size_t)m * w->dims.n, stream));
     GemmArgs a{w->dev, xh, sxh, out, (int)p.m_rows, (int)m, (int)w->dims.n, (int)p.k_pad, (int)w->dims.units,
@@ -184,7 +185,7 @@ static int launch_gemm(const void *x, int xk, const rlx_qweight *w, float *out, 
     void *params[] = {&a};
     KernelId id = w->scheme == SCHEME_Q4K ? K_GEMM_Q4_K : w->scheme == SCHEME_Q4_0 ? K_GEMM_Q4_0 : K_GEMM_Q8_0;
     RLX_TRY(runtime_init());
-    RLX_TRY(launch3(id, (unsigned)gx, (unsigned)gy, (unsigned)split, 512, 2 * (32 + 16) * 1024, stream, params));
+    RLX_TRY(launch3(id, (unsigned)gx, (unsigned)gy, (unsigned)split, 512, 2 * 48 * 1024, stream, params));
     return RLX_OK;
 }
 

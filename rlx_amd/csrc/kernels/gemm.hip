@@ -1,11 +1,7 @@
 // Prefill matmul: out[m, n] = x[m, k] . W^T for m > 16, W in the device layout (see layout.h).
 // Replaces rlx_cpu::gguf_matmul::gguf_matmul_bt (rlx-cpu/src/gguf_matmul.rs:40-95) for the batched case.
 //
-// Workgroup tile 256 (rows of x) x 128 (rows of W), 8 waves as 4 x 2, each wave 64 x 64 = 2 x 2 MFMA tiles of
-// v_mfma_f32_32x32x16_f16. K advances in steps of 64 columns through two LDS stages (96 KB): while the matrix
-// cores work on one stage the same waves fetch the next step's activations and packed weights, decode the
-// weights to binary16 and store both as MFMA fragments (16 B per lane, XOR-swizzled so stores and loads are
-// bank-conflict free) into the other stage. One barrier per step.
+// Workgroup tile 256 (rows of x) x 128 (rows of W); the decomposition is described above gemm_body().
 //
 // Numerics. Activations are binary16: bf16 / f16 inputs convert exactly (normal range); f32 inputs are carried
 // as two rows hi + lo/2048 and recombined in the epilogue. Weights:
@@ -19,13 +15,13 @@
 namespace rlx {
 
 constexpr int GEMM_MT = 256, GEMM_NT = 128, GEMM_KS = 64, GEMM_THREADS = 512;
-constexpr int GEMM_STAGE_A = 4 * 8 * 1024, GEMM_STAGE_B = 4 * 4 * 1024;  // [k-slice][sub-tile][lane][16 B]
+constexpr int GEMM_STAGE_A = 4 * 8 * 1024, GEMM_STAGE_B = 4 * 4 * 1024;  // [k-slice][32-row sub-tile][lane][16 B]
 constexpr int GEMM_STAGE = GEMM_STAGE_A + GEMM_STAGE_B;
 constexpr float GEMM_LO_SCALE = 2048.0f;
 
 struct GemmArgs {
     const uint8_t *w;
-    const half_t *xh;   // [m_rows][k_pad] binary16 activations (rows padded to 256, columns to the K unit)
+    const half_t *xh;   // [m_rows][k_pad] binary16 activations (rows padded to 256, columns to a multiple of 256)
     const half_t *sxh;  // Q4_K: [m_rows][k_pad / 256][16]: per 32-column block sums, 8 x hi then 8 x lo*2048
     float *out;         // [m_out][n]
     int m_rows;         // rows of xh
@@ -35,244 +31,280 @@ struct GemmArgs {
     int units;          // K units of the device layout
     int row_tiles;      // 16-row tiles of the device layout
     int pair_rows;      // 1: rows 2i, 2i+1 of xh are hi / lo*2048 of logical row i (f32 activations)
-    int steps_per_split;  // 64-column steps per grid.z slice
+    int steps_per_split;  // 64-column steps per grid.z slice (a multiple of 4)
     int use_atomics;      // split K: accumulate into a zeroed `out` with atomic adds
 };
 
-// LDS fragment slot of (sub-tile s, k-slice ks, row r in 0..31, half h): lanes r + 32 h; the low three bits of the
-// lane are XORed with c = 2 ks + h so that the eight 16-byte stores of one activation row, and the stores of the
-// decode threads, land in eight different bank groups.
-__device__ __forceinline__ int frag_offset(int nsub_per_ks, int ks, int s, int r, int h) {
-    int c = 2 * ks + h;
-    return ((ks * nsub_per_ks + s) * 64 + ((r ^ c) & 31) + 32 * h) * 16;
-}
-
-__device__ __forceinline__ uint32_t splat_code_half(uint32_t word, int byte) {
-    // half2 (v, v) with v = byte `byte` of word as an exact binary16 integer: bytes [b, 0x64, b, 0x64] = 1024 + b
+// half2 (v, v) with v = byte `byte` of word as an exact binary16 integer: bytes [b, 0x64, b, 0x64] = 1024 + b
+__device__ __forceinline__ half2_t splat_code_half(uint32_t word, int byte) {
     uint32_t sel = 0x04000400u | (uint32_t)byte | ((uint32_t)byte << 16);
     half2_t t = as_half2(__builtin_amdgcn_perm(0x64646464u, word, sel));
     const half2_t k1024 = {(half_t)1024.0f, (half_t)1024.0f};
-    return as_u32(t - k1024);
+    return t - k1024;
 }
 
+// LDS slot of (k-slice ks, sub-tile s of NS, row r in 0..31, half h): lanes r + 32 h; the low bits of the lane are
+// XORed with c = 2 ks + h so that the eight 16-byte stores of one activation row, and the stores of the decode
+// threads, land in eight different bank groups. Reads of one fragment are a permutation of 64 consecutive slots.
+__device__ __forceinline__ int frag_offset(int ns, int ks, int s, int r, int h) {
+    int c = 2 * ks + h;
+    return ((ks * ns + s) * 64 + ((r ^ c) & 31) + 32 * h) * 16;
+}
+
+// Workgroup = 8 waves (two per SIMD) as 4 x 2, tile 256 rows of x by 128 rows of W, each wave 64 x 64 = 2 x 2 tiles of
+// v_mfma_f32_32x32x16_f16. K advances in 64-column steps through two LDS stages (96 KB). On gfx950 a matrix
+// instruction leaves room for only about four other vector instructions in its shadow, so the step is written as
+// four k-slice groups, each: LDS reads of the next slice's fragments, the slice's four MFMAs, and one quarter of the
+// work that prepares the next step (LDS stores of activations fetched two steps ago, decode + store of the packed
+// weights), with scheduling fences so the compiler keeps that interleaving. Global loads run two steps ahead in
+// registers. The loop is unrolled by four steps (one Q4_K super-block) so every phase test and register-set index
+// is a compile-time constant.
 template <int SCHEME>
 __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
     constexpr Layout L = layout_of(SCHEME);
-    constexpr int STEPS_PER_UNIT = L.unit_k / GEMM_KS;  // 4 for Q4_K, 2 for Q4_0 / Q8_0
+    constexpr bool K4 = SCHEME == SCHEME_Q4K;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = wave >> 1, wn = wave & 1;  // wave grid 4 x 2
+    const int wm = wave >> 1, wn = wave & 1;
     const int lr = lane & 31, lh = lane >> 5;
     const int n_tile0 = blockIdx.x * GEMM_NT, m_tile0 = blockIdx.y * GEMM_MT;
     const int step0 = blockIdx.z * a.steps_per_split;
-    const int total_steps = a.units * STEPS_PER_UNIT;
+    const int total_steps = a.units * (L.unit_k / GEMM_KS);
     const int step1 = min(step0 + a.steps_per_split, total_steps);
 
-    // ---- loader roles -------------------------------------------------------------------------------
-    // activations: thread -> (row = tid/8 + 64 i, 16-byte chunk c = tid%8), i = 0..3
+    // ---- A loader: thread -> 16-byte chunk c = tid % 8 of rows tid/8 + 64 i, i = 0..3 (sub-tile (tid/8)/32 + 2 i) ----
     const int a_row = tid >> 3, a_c = tid & 7;
-    const half_t *a_src = a.xh + (long long)(m_tile0 + a_row) * a.k_pad + a_c * 8;
-    int a_dst[4];
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        int row = a_row + 64 * i;
-        a_dst[i] = frag_offset(8, a_c >> 1, row >> 5, row & 31, a_c & 1);
-    }
-    // weights: thread -> lane slot (tile16 = tid/64, n16 = lane%16, g = lane/16) of the unit that holds this step
+    const uint8_t *a_base = (const uint8_t *)(a.xh + (long long)m_tile0 * a.k_pad);  // wave-uniform
+    const uint32_t a_off0 = ((uint32_t)a_row * (uint32_t)a.k_pad + (uint32_t)a_c * 8u) * 2u;
+    const uint32_t a_stride64 = (uint32_t)a.k_pad * 128u;  // bytes between rows r and r + 64
+    const int a_dst0 = frag_offset(8, a_c >> 1, a_row >> 5, a_row & 31, a_c & 1);  // + i * 2048 for rows + 64 i
+
+    // ---- B loader: thread -> lane slot (n16 = lane % 16, g = lane / 16) of 16-row tile `wave` ---------------
     const int b_n16 = lane & 15, b_g = lane >> 4;
-    const int b_tile = blockIdx.x * (GEMM_NT / 16) + wave;
-    const bool b_live = b_tile < a.row_tiles;
-    const uint8_t *b_tile_base = a.w + (long long)(b_live ? b_tile : 0) * a.units * L.unit_bytes;
-    const int b_row = wave * 16 + b_n16;  // row inside the 128-row tile
-    // destination of the granule of block jl (0/1 within the step): k-slice 2 jl + g/2, half g%2
-    int b_dst[2];
+    const int b_t16 = blockIdx.x * (GEMM_NT / 16) + wave;
+    const bool b_live = b_t16 < a.row_tiles;
+    const uint8_t *b_tile = a.w + (long long)(b_live ? b_t16 : 0) * a.units * L.unit_bytes;
+    const uint32_t b_keep = b_live ? 0xFFFFFFFFu : 0u;
+    int b_dst[2];  // [block jl of the step]: k-slice 2 jl + g/2, half g%2
+    {
+        const int row = wave * 16 + b_n16;
 #pragma unroll
-    for (int jl = 0; jl < 2; jl++) b_dst[jl] = GEMM_STAGE_A + frag_offset(4, 2 * jl + (b_g >> 1), b_row >> 5, b_row & 31, b_g & 1);
+        for (int jl = 0; jl < 2; jl++)
+            b_dst[jl] = GEMM_STAGE_A + frag_offset(4, 2 * jl + (b_g >> 1), row >> 5, row & 31, b_g & 1);
+    }
 
-    uint4_t a_reg[4];
-    uint4_t b_q = {0, 0, 0, 0}, b_q2 = {0, 0, 0, 0};  // packed codes of the current half unit (Q8_0: two words per block)
-    uint4_t b_meta = {0, 0, 0, 0};                     // Q4_K: d, dmin, 12 scale bytes of (row, super-block); else scales
+    // Register-resident prefetch: activations one step ahead, packed weights two.
+    uint4_t a_reg[4];                                   // activations of the next step
+    uint4_t b_q[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};      // [chunk parity] packed codes of a two-step chunk (Q8_0: [step parity])
+    uint4_t b_meta[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};   // Q4_K: [0] = meta of the super-block decoded next; else [chunk parity] .x/.y = four f16 scales
+    uint32_t b_sc[2] = {0, 0};                          // Q4_K: 6-bit scales of sub-blocks 0-3 / 4-7 being decoded
 
-    auto fetch = [&](int step) {
-        const int kcol = step * GEMM_KS;
+    auto fetch_a = [&](int step) {
+        const uint8_t *p = a_base + (long long)step * (GEMM_KS * 2) + a_off0;
 #pragma unroll
-        for (int i = 0; i < 4; i++) a_reg[i] = *(const uint4_t *)(a_src + (long long)(64 * i) * a.k_pad + kcol);
-        const int u = step / STEPS_PER_UNIT, sub = step % STEPS_PER_UNIT;
-        const uint8_t *unit = b_tile_base + (long long)u * L.unit_bytes;
-        if (b_live) {
-            if constexpr (SCHEME == SCHEME_Q4K) {
-                if ((sub & 1) == 0) b_q = *(const uint4_t *)(unit + (sub >> 1) * 1024 + lane * 16);
-                if (sub == 0) b_meta = *(const uint4_t *)(unit + 2048 + b_n16 * 16);
-            } else if constexpr (SCHEME == SCHEME_Q4_0) {
-                if (sub == 0) {
-                    b_q = *(const uint4_t *)(unit + lane * 16);
-                    uint2_t s = *(const uint2_t *)(unit + 1024 + b_n16 * 8);
-                    b_meta[0] = s[0];
-                    b_meta[1] = s[1];
-                }
-            } else {
-                b_q = *(const uint4_t *)(unit + sub * 1024 + lane * 16);
-                if (sub == 0) {
-                    uint2_t s = *(const uint2_t *)(unit + 2048 + b_n16 * 8);
-                    b_meta[0] = s[0];
-                    b_meta[1] = s[1];
-                }
+        for (int i = 0; i < 4; i++) a_reg[i] = *(const uint4_t *)(p + (size_t)i * a_stride64);
+    };
+    auto fetch_b = [&](int step, int q) {  // q = step & 3, compile-time at every call site
+        if constexpr (K4) {  // dead tiles read tile 0 (valid memory) and are zeroed when stored
+            const uint8_t *unit = b_tile + (long long)(step >> 2) * L.unit_bytes;
+            if ((q & 1) == 0) b_q[(q >> 1) & 1] = *(const uint4_t *)(unit + (q >> 1) * 1024 + lane * 16);
+            if (q == 0) b_meta[0] = *(const uint4_t *)(unit + 2048 + b_n16 * 16);  // consumed one step later, before the next fetch
+        } else if constexpr (SCHEME == SCHEME_Q4_0) {
+            const uint8_t *unit = b_tile + (long long)(step >> 1) * L.unit_bytes;
+            if ((q & 1) == 0) {
+                b_q[(q >> 1) & 1] = *(const uint4_t *)(unit + lane * 16);
+                uint2_t sc = *(const uint2_t *)(unit + 1024 + b_n16 * 8);
+                b_meta[(q >> 1) & 1][0] = sc[0];
+                b_meta[(q >> 1) & 1][1] = sc[1];
+            }
+        } else {
+            const uint8_t *unit = b_tile + (long long)(step >> 1) * L.unit_bytes;
+            b_q[q & 1] = *(const uint4_t *)(unit + (q & 1) * 1024 + lane * 16);
+            if ((q & 1) == 0) {
+                uint2_t sc = *(const uint2_t *)(unit + 2048 + b_n16 * 8);
+                b_meta[(q >> 1) & 1][0] = sc[0];
+                b_meta[(q >> 1) & 1][1] = sc[1];
             }
         }
     };
-
-    auto store_stage = [&](int step, uint8_t *stage) {
+    auto store_a2 = [&](uint8_t *stage, int i0) {  // two of the four activation chunks
 #pragma unroll
-        for (int i = 0; i < 4; i++) *(uint4_t *)(stage + a_dst[i]) = a_reg[i];
-        const int sub = step % STEPS_PER_UNIT;
-        Frag f[2];
-        if constexpr (SCHEME == SCHEME_Q4K) {
-            uint32_t sc[2], mn[2];
-            q4k_scales(b_meta[1], b_meta[2], b_meta[3], sc, mn);
-            const uint32_t scw = (sub >> 1) ? sc[1] : sc[0];  // scales of sub-blocks 4*(sub/2) .. +3
-#pragma unroll
-            for (int jl = 0; jl < 2; jl++) {
-                const int t = 2 * (sub & 1) + jl;  // word of b_q = sub-block 4*(sub/2) + t
-                uint32_t s2 = (t == 0) ? splat_code_half(scw, 0) : (t == 1) ? splat_code_half(scw, 1)
-                              : (t == 2) ? splat_code_half(scw, 2) : splat_code_half(scw, 3);
-                uint32_t word = (t == 0) ? b_q[0] : (t == 1) ? b_q[1] : (t == 2) ? b_q[2] : b_q[3];
-                unpack_q4_scaled(word, as_half2(s2), f[jl]);
+        for (int i = i0; i < i0 + 2; i++) *(uint4_t *)(stage + a_dst0 + i * 2048) = a_reg[i];
+    };
+    // decode block jl (0/1) of the step `step` with phase q into LDS
+    auto store_b1 = [&](int step, int q, int jl, uint8_t *stage) {
+        const int cp = (q >> 1) & 1;
+        const int t = 2 * (q & 1) + jl;
+        Frag f;
+        if constexpr (K4) {
+            if (q == 0 && jl == 0) {
+                uint32_t mn[2];
+                const uint4_t &m4 = b_meta[0];
+                q4k_scales(m4[1], m4[2], m4[3], b_sc, mn);
             }
-        } else if constexpr (SCHEME == SCHEME_Q4_0) {
-#pragma unroll
-            for (int jl = 0; jl < 2; jl++) {
-                const int t = 2 * sub + jl;  // block 4u + t
-                uint32_t word = (t == 0) ? b_q[0] : (t == 1) ? b_q[1] : (t == 2) ? b_q[2] : b_q[3];
-                uint32_t dbits = (t & 1) ? (b_meta[t >> 1] >> 16) : (b_meta[t >> 1] & 0xFFFFu);
-                half2_t d2 = as_half2(dbits | (dbits << 16));
-                unpack_q4<8>(word, f[jl]);
-#pragma unroll
-                for (int e = 0; e < 4; e++) f[jl].h2[e] = f[jl].h2[e] * d2;
-            }
+            unpack_q4_scaled(b_q[cp][t], splat_code_half(b_sc[q >> 1], t), f);
         } else {
+            const uint32_t dbits = (t & 1) ? (b_meta[cp][t >> 1] >> 16) : (b_meta[cp][t >> 1] & 0xFFFFu);
+            const half2_t d2 = as_half2(dbits | (dbits << 16));
+            if constexpr (SCHEME == SCHEME_Q4_0) unpack_q4<8>(b_q[cp][t], f);
+            else unpack_q8(b_q[q & 1][2 * jl], b_q[q & 1][2 * jl + 1], f);
 #pragma unroll
-            for (int jl = 0; jl < 2; jl++) {
-                const int t = 2 * sub + jl;
-                uint32_t dbits = (t & 1) ? (b_meta[t >> 1] >> 16) : (b_meta[t >> 1] & 0xFFFFu);
-                half2_t d2 = as_half2(dbits | (dbits << 16));
-                unpack_q8(b_q[2 * jl], b_q[2 * jl + 1], f[jl]);
-#pragma unroll
-                for (int e = 0; e < 4; e++) f[jl].h2[e] = f[jl].h2[e] * d2;
-            }
-        }
-        if (!b_live) {
-            f[0].u4 = uint4_t{0, 0, 0, 0};
-            f[1].u4 = uint4_t{0, 0, 0, 0};
+            for (int e = 0; e < 4; e++) f.h2[e] = f.h2[e] * d2;
         }
 #pragma unroll
-        for (int jl = 0; jl < 2; jl++) *(uint4_t *)(stage + b_dst[jl]) = f[jl].u4;
+        for (int e = 0; e < 4; e++) f.u[e] &= b_keep;
+        *(uint4_t *)(stage + b_dst[jl]) = f.u4;
     };
 
     // ---- accumulators ----------------------------------------------------------------------------------
-    float16_t total[2][2], part[2][2];
+    float16_t total[2][2], part[2][2], zero16;
 #pragma unroll
-    for (int i = 0; i < 2; i++)
-#pragma unroll
-        for (int j = 0; j < 2; j++)
-#pragma unroll
-            for (int e = 0; e < 16; e++) {
-                total[i][j][e] = 0.f;
-                part[i][j][e] = 0.f;
-            }
-
-    // this lane's two W rows (one per 32-column MFMA tile) for the Q4_K per-super-block scaling
-    int my_row[2];
-#pragma unroll
-    for (int j = 0; j < 2; j++) my_row[j] = n_tile0 + wn * 64 + 32 * j + lr;
-
-    if (step0 < step1) {
-        fetch(step0);
-        store_stage(step0, smem);
-    }
-    __syncthreads();
-
-    for (int step = step0; step < step1; step++) {
-        const int cur = (step - step0) & 1;
-        uint8_t *stage = smem + cur * GEMM_STAGE;
-        uint8_t *next = smem + (cur ^ 1) * GEMM_STAGE;
-        const bool more = step + 1 < step1;
-        if (more) fetch(step + 1);
-
-#pragma unroll
-        for (int ks = 0; ks < 4; ks++) {
-            Frag fa[2], fb[2];
-#pragma unroll
-            for (int i = 0; i < 2; i++) fa[i].u4 = *(const uint4_t *)(stage + frag_offset(8, ks, wm * 2 + i, lr, lh));
-#pragma unroll
-            for (int j = 0; j < 2; j++)
-                fb[j].u4 = *(const uint4_t *)(stage + GEMM_STAGE_A + frag_offset(4, ks, wn * 2 + j, lr, lh));
-#pragma unroll
-            for (int i = 0; i < 2; i++)
-#pragma unroll
-                for (int j = 0; j < 2; j++) {
-                    if constexpr (SCHEME == SCHEME_Q4K) part[i][j] = mfma32(fa[i], fb[j], part[i][j]);
-                    else total[i][j] = mfma32(fa[i], fb[j], total[i][j]);
-                }
-        }
-
-        if constexpr (SCHEME == SCHEME_Q4K) {
-            if ((step & 3) == 3) {  // a 256-column super-block is complete: total += d * P - dmin * (mn . sx)
-                const int sb = step >> 2;
-                Frag fs[2];
-#pragma unroll
-                for (int i = 0; i < 2; i++) {
-                    long long row = m_tile0 + (wm * 2 + i) * 32 + lr;
-                    fs[i].u4 = *(const uint4_t *)(a.sxh + (row * (a.k_pad / 256) + sb) * 16 + lh * 8);
-                }
-#pragma unroll
-                for (int j = 0; j < 2; j++) {
-                    const int row = my_row[j];
-                    uint4_t meta = {0, 0, 0, 0};
-                    if ((row >> 4) < a.row_tiles)
-                        meta = *(const uint4_t *)(a.w + ((long long)(row >> 4) * a.units + sb) * L.unit_bytes + 2048 + (row & 15) * 16);
-                    const float d = half_bits_to_float(meta[0] & 0xFFFFu), dmin = half_bits_to_float(meta[0] >> 16);
-                    uint32_t sc[2], mn[2];
-                    q4k_scales(meta[1], meta[2], meta[3], sc, mn);
-                    // B' fragment: half 0 holds mn_0..7, half 1 holds mn_0..7 / 2048 (pairs with the lo sums)
-                    Frag fm;
-                    const half2_t k1024 = {(half_t)1024.0f, (half_t)1024.0f};
-                    const half2_t lo_scale = {(half_t)(1.0f / GEMM_LO_SCALE), (half_t)(1.0f / GEMM_LO_SCALE)};
-#pragma unroll
-                    for (int e = 0; e < 4; e++) {
-                        uint32_t src = (e < 2) ? mn[0] : mn[1];
-                        uint32_t sel = (e & 1) ? 0x04030402u : 0x04010400u;  // bytes (2,3) or (0,1) -> [b,0x64,b',0x64]
-                        half2_t v = as_half2(__builtin_amdgcn_perm(0x64646464u, src, sel)) - k1024;
-                        fm.h2[e] = lh ? v * lo_scale : v;
-                    }
-#pragma unroll
-                    for (int i = 0; i < 2; i++) {
-                        float16_t zero;
-#pragma unroll
-                        for (int e = 0; e < 16; e++) zero[e] = 0.f;
-                        float16_t q = mfma32(fs[i], fm, zero);
-#pragma unroll
-                        for (int e = 0; e < 16; e++) {
-                            total[i][j][e] = __builtin_fmaf(d, part[i][j][e], total[i][j][e]);
-                            total[i][j][e] = __builtin_fmaf(-dmin, q[e], total[i][j][e]);
-                            part[i][j][e] = 0.f;
-                        }
-                    }
-                }
-            }
-        }
-
-        if (more) store_stage(step + 1, next);
-        __syncthreads();
-    }
-
-    // ---- epilogue: register i of tile (i_m, j_n) is row 8 (i/4) + 4 lh + i%4, column lr ------------------
+    for (int e = 0; e < 16; e++) zero16[e] = 0.f;
 #pragma unroll
     for (int i = 0; i < 2; i++)
 #pragma unroll
         for (int j = 0; j < 2; j++) {
-            const int col = n_tile0 + wn * 64 + 32 * j + lr;
+            total[i][j] = zero16;
+            part[i][j] = zero16;
+        }
+    // this lane's two W rows (one per 32-column MFMA tile) for the Q4_K per-super-block scaling
+    int my_row[2];
+    const uint8_t *my_meta[2];
+    bool my_ok[2];
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+        my_row[j] = n_tile0 + wn * 64 + 32 * j + lr;
+        my_ok[j] = (my_row[j] >> 4) < a.row_tiles;
+        my_meta[j] = a.w + (long long)(my_ok[j] ? (my_row[j] >> 4) : 0) * a.units * L.unit_bytes + 2048 + (my_row[j] & 15) * 16;
+    }
+    uint4_t w_meta[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};
+    Frag fs[2];
+    int a_rd[4], b_rd[4];  // per k-slice read offsets of this lane; + sub-tile * 1024
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) {
+        a_rd[ks] = frag_offset(8, ks, wm * 2, lr, lh);
+        b_rd[ks] = GEMM_STAGE_A + frag_offset(4, ks, wn * 2, lr, lh);
+    }
+    Frag fa[2][2], fb[2][2];  // [buffer][tile]
+    auto load_frags = [&](const uint8_t *stage, int ks, int buf) {
+#pragma unroll
+        for (int i = 0; i < 2; i++) fa[buf][i].u4 = *(const uint4_t *)(stage + a_rd[ks] + i * 1024);
+#pragma unroll
+        for (int j = 0; j < 2; j++) fb[buf][j].u4 = *(const uint4_t *)(stage + b_rd[ks] + j * 1024);
+    };
+
+    if (step0 < step1) {  // step0 is a multiple of 4
+        fetch_a(step0);
+        fetch_b(step0, 0);
+        fetch_b(min(step0 + 1, step1 - 1), 1);
+        store_a2(smem, 0);
+        store_a2(smem, 2);
+        store_b1(step0, 0, 0, smem);
+        store_b1(step0, 0, 1, smem);
+    }
+    __syncthreads();
+
+    for (int sbase = step0; sbase < step1; sbase += 4) {
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            const int step = sbase + q;
+            if (step < step1) {
+                const uint8_t *stage = smem + (q & 1) * GEMM_STAGE;
+                uint8_t *next = smem + ((q & 1) ^ 1) * GEMM_STAGE;
+                // No branches inside a step: the last steps re-fetch / re-store the final step into a stage nobody
+                // reads again, so each k-slice group below is one scheduling region.
+                const int nstep = min(step + 1, step1 - 1);
+                load_frags(stage, 0, 0);
+                fetch_a(nstep);
+                fetch_b(min(step + 2, step1 - 1), (q + 2) & 3);
+                if constexpr (K4) {
+                    if (q == 0) {  // this wave's rows: meta and activation block sums of the super-block, used at q == 3
+                        const int sb = step >> 2;
+#pragma unroll
+                        for (int j = 0; j < 2; j++) w_meta[j] = *(const uint4_t *)(my_meta[j] + (long long)sb * L.unit_bytes);
+#pragma unroll
+                        for (int i = 0; i < 2; i++) {
+                            long long row = m_tile0 + (wm * 2 + i) * 32 + lr;
+                            fs[i].u4 = *(const uint4_t *)(a.sxh + (row * (a.k_pad / 256) + sb) * 16 + lh * 8);
+                        }
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int ks = 0; ks < 4; ks++) {
+                    const int buf = ks & 1;
+                    if (ks < 3) load_frags(stage, ks + 1, buf ^ 1);
+#pragma unroll
+                    for (int i = 0; i < 2; i++)
+#pragma unroll
+                        for (int j = 0; j < 2; j++) {
+                            if constexpr (K4) {
+                                // the first slice of a super-block starts the partial product from zero
+                                part[i][j] = mfma32(fa[buf][i], fb[buf][j], (q == 0 && ks == 0) ? zero16 : part[i][j]);
+                            } else {
+                                total[i][j] = mfma32(fa[buf][i], fb[buf][j], total[i][j]);
+                            }
+                        }
+                    // weights first: the activations were fetched only at the top of this step
+                    if (ks == 0) store_b1(nstep, (q + 1) & 3, 0, next);
+                    if (ks == 1) store_b1(nstep, (q + 1) & 3, 1, next);
+                    if (ks == 2) store_a2(next, 0);
+                    if (ks == 3) store_a2(next, 2);
+                    // order inside the group: the LDS reads of the next slice, then MFMA / few VALU alternating
+                    __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+                    }
+                    __builtin_amdgcn_sched_group_barrier(0x200, 2, 0);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                if constexpr (K4) {
+                    if (q == 3) {  // a 256-column super-block is complete: total += d * P - dmin * (mn . sx)
+#pragma unroll
+                        for (int j = 0; j < 2; j++) {
+                            const uint4_t meta = w_meta[j];
+                            const float d = my_ok[j] ? half_bits_to_float(meta[0] & 0xFFFFu) : 0.f;
+                            const float dmin = my_ok[j] ? half_bits_to_float(meta[0] >> 16) : 0.f;
+                            uint32_t sc[2], mn[2];
+                            q4k_scales(meta[1], meta[2], meta[3], sc, mn);
+                            // B' fragment: half 0 holds mn_0..7, half 1 holds mn_0..7 / 2048 (pairs with the lo sums)
+                            Frag fm;
+                            const half2_t k1024 = {(half_t)1024.0f, (half_t)1024.0f};
+                            const half2_t lo_scale = {(half_t)(1.0f / GEMM_LO_SCALE), (half_t)(1.0f / GEMM_LO_SCALE)};
+#pragma unroll
+                            for (int e = 0; e < 4; e++) {
+                                uint32_t src = (e < 2) ? mn[0] : mn[1];
+                                uint32_t sel = (e & 1) ? 0x04030402u : 0x04010400u;  // bytes (2,3) or (0,1) -> [b,0x64,b',0x64]
+                                half2_t v = as_half2(__builtin_amdgcn_perm(0x64646464u, src, sel)) - k1024;
+                                fm.h2[e] = lh ? v * lo_scale : v;
+                            }
+#pragma unroll
+                            for (int i = 0; i < 2; i++) {
+                                float16_t qq = mfma32(fs[i], fm, zero16);
+#pragma unroll
+                                for (int e = 0; e < 16; e++) {
+                                    total[i][j][e] = __builtin_fmaf(d, part[i][j][e], total[i][j][e]);
+                                    total[i][j][e] = __builtin_fmaf(-dmin, qq[e], total[i][j][e]);
+                                }
+                            }
+                        }
+                    }
+                }
+                __syncthreads();
+            }
+        }
+    }
+
+    // ---- epilogue: register e of tile (i, j) is row 8 (e/4) + 4 lh + e%4, column lr ------------------------
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            const int col = my_row[j];
             if (col >= a.n) continue;
 #pragma unroll
             for (int e = 0; e < 16; e++) {
