@@ -24,6 +24,10 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0       # MI355X published HBM3E bandwidth
 MFMA_F16_PEAK_TFLOPS = 2500.0  # dense f16/bf16 MFMA peak
+CALIBRATION_COPY_BYTES = 256 << 20
+# HBM bytes per launch of the headline kernel (FETCH_SIZE + WRITE_SIZE of two rocprofv3 --pmc runs of this command,
+# each scaled by the same counter's reading for the copy kernel above); profiles/gemv_q4_0_llama8b_layer_traffic.txt.
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 124216599
 
 # (name, N, K) — BASELINE config 2
 LLAMA8B = [("q", 4096, 4096), ("k", 1024, 4096), ("v", 1024, 4096), ("o", 4096, 4096),
@@ -112,6 +116,8 @@ def main():
     ap.add_argument("--graph", action="store_true",
                     help="replay each layer as a hipGraph instead of launching its kernel directly (one-node graphs "
                          "cost more per launch than a plain launch on this runtime)")
+    ap.add_argument("--calibration-copies", type=int, default=3,
+                    help="untimed launches of the 256 MiB copy kernel before the run (counter calibration)")
     ap.add_argument("--extra", action="store_true", help="also time the other BASELINE configs (reported under 'extra')")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -135,6 +141,17 @@ def main():
     stream = rlx_amd._lib.C.c_void_p()
     rlx_amd._lib.check(rlx_amd._lib.lib().rlx_mi355x_stream_create(rlx_amd._lib.C.byref(stream)))
     layer_bytes = sum(gemv_bytes(n, k) for _, n, k in LLAMA8B)
+    # A few launches of the plain copy kernel on a buffer of known size, outside the timed region: the unit against
+    # which a counter run of this same command scales FETCH_SIZE / WRITE_SIZE.
+    if args.calibration_copies:
+        src = ops.DeviceBuffer(CALIBRATION_COPY_BYTES)
+        dst = ops.DeviceBuffer(CALIBRATION_COPY_BYTES)
+        rlx_amd._lib.check(rlx_amd._lib.lib().rlx_mi355x_memset_u32(src.ptr, 0x3f800000, CALIBRATION_COPY_BYTES // 4, stream))
+        for _ in range(args.calibration_copies):
+            rlx_amd._lib.check(rlx_amd._lib.lib().rlx_mi355x_memcpy_d2d(dst.ptr, src.ptr, CALIBRATION_COPY_BYTES, stream))
+        ops.sync(stream)
+        src.free()
+        dst.free()
     ms_per_step, layers, xs = time_layers(rlx_amd, ops, stream, base, args.wiring, args.layers, args.steps, args.warmup,
                                           args.graph)
     setup_s = time.time() - t0
@@ -160,14 +177,16 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "u4 codes x f16 scale, f32 accumulate",
+        "dtype": "f16",
+        "dtype_note": "4-bit codes and activations as exact f16 MFMA operands, f32 accumulate, f16 block scale applied in f32",
         "data": "synthetic",
         "config": {"workload": "Q4_0 decode GEMV, batch 1, seven Llama-3-8B layer projections per step "
                                "(q,k,v,o,gate,up,down), f32 activations, weights ~N(0,0.02)",
                    "wiring": args.wiring, "layers_rotated": args.layers, "hip_graph": args.graph,
                    "algorithmic_bytes_per_step": layer_bytes, "launches_per_step": launches_per_step},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(gbs / HBM_PEAK_GBS, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH if args.wiring == "independent" else None,
                      "kernel": "rlx_gemv_q4_0_r2", "avg_launch_us": round(us_per_launch, 3),
                      "algorithmic_bytes_per_launch": layer_bytes // launches_per_step},
         "parity_max_rel_err": parity,
@@ -267,6 +286,89 @@ def extra_configs(rlx_amd, stream):
     out["fake_quantize_8192x4096_cols"] = {"us": round(ms * 1e3, 2), "GB/s_1R1W": round(b / ms / 1e6, 1),
                                            "frac_hbm_1R1W": round(b / ms / 1e6 / HBM_PEAK_GBS, 4),
                                            "GB/s_2R1W": round(1.5 * b / ms / 1e6, 1)}
+    out.update(gemm_configs(rlx_amd, stream))
+    return out
+
+
+def f32_to_bf16_bits(x):
+    """Round-to-nearest-even f32 -> bf16 bit patterns (uint16)."""
+    u = np.ascontiguousarray(x, np.float32).view(np.uint32).astype(np.uint64)
+    return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+
+
+def tiled_weight(ops, scheme, n, k, seed, sigma):
+    """[n, k] quantized weight built from one 4096-row seeded normal slab rolled per repetition (same statistics as a
+    fresh draw, a fraction of the host time)."""
+    slab_rows = min(n, 4096)
+    w = (ops.philox_normal(seed, slab_rows * k) * np.float32(sigma)).astype(np.float32)
+    slab = ops.quantize(scheme, w).reshape(slab_rows, -1)
+    reps = (n + slab_rows - 1) // slab_rows
+    packed = np.concatenate([np.roll(slab, 131 * r, axis=0) for r in range(reps)], axis=0)[:n]
+    return ops.QWeight(scheme, np.ascontiguousarray(packed).reshape(-1), n, k)
+
+
+def gemm_configs(rlx_amd, stream):
+    """Prefill GEMM and the batch sweep: Q4_K M=512 on the 8B MLP shapes, FakeQuantize -> Q8_0 GEMM, and the Q4_0
+    M sweep over one Llama-3-70B layer. Times include the activation-preparation kernel the GEMM path launches."""
+    from rlx_amd import DType, QuantScheme, ops
+    L = rlx_amd._lib.lib()
+    out = {}
+
+    def run_matmul(qw, m, k, x_dtype, reps, warm, copies=1):
+        xbits = f32_to_bf16_bits(ops.philox_normal(31, m * k)) if x_dtype == DType.BF16 else ops.philox_normal(31, m * k)
+        xd = ops.DeviceBuffer.from_numpy(xbits)
+        od = ops.DeviceBuffer(m * qw[0].n * 4)
+        need = ops.matmul_workspace_bytes(qw[0], x_dtype, m)
+        ws = ops.DeviceBuffer(need) if need else None
+        state = {"i": 0}
+
+        def fn():
+            q = qw[state["i"] % len(qw)]
+            state["i"] += 1
+            rlx_amd._lib.check(L.rlx_mi355x_gguf_matmul_bt(xd.ptr, int(x_dtype), q.ptr, od.ptr, m, ws.ptr if ws else None,
+                                                           need, stream))
+
+        ms = time_launches(ops, stream, fn, reps, warm)
+        ops.sync(stream)
+        return ms
+
+    # config 3: Q4_K, M = 512, bf16 activations
+    for name, n, k in [("gate_up_4096x14336", 14336, 4096), ("down_14336x4096", 4096, 14336)]:
+        qw = [tiled_weight(ops, QuantScheme.GgufQ4K, n, k, 41 + i, 0.02) for i in range(2)]
+        ms = run_matmul(qw, 512, k, DType.BF16, 100, 10)
+        tf = 2.0 * 512 * n * k / ms / 1e9
+        out[f"q4_k_gemm_m512_{name}"] = {"us": round(ms * 1e3, 2), "TFLOP/s": round(tf, 1),
+                                        "frac_mfma_f16": round(tf / MFMA_F16_PEAK_TFLOPS, 4)}
+        for q in qw:
+            q.free()
+
+    # config 4 (second half): the fake-quantized [8192, 4096] f32 tensor against a Q8_0 4096x4096 weight
+    qw = [tiled_weight(ops, QuantScheme.GgufQ8_0, 4096, 4096, 45, 0.02)]
+    ms = run_matmul(qw, 8192, 4096, DType.F32, 30, 5)
+    tf = 2.0 * 8192 * 4096 * 4096 / ms / 1e9
+    out["q8_0_gemm_m8192_4096x4096_f32"] = {"us": round(ms * 1e3, 2), "TFLOP/s": round(tf, 1),
+                                          "frac_mfma_f16": round(tf / MFMA_F16_PEAK_TFLOPS, 4),
+                                          "note": "f32 activations run as hi + lo f16 rows: two MFMA rows per token"}
+    qw[0].free()
+
+    # config 5: Q4_0 batch sweep over the seven projections of one Llama-3-70B layer, bf16 activations
+    shapes70 = [("q", 8192, 8192), ("k", 1024, 8192), ("v", 1024, 8192), ("o", 8192, 8192),
+                ("gate", 28672, 8192), ("up", 28672, 8192), ("down", 8192, 28672)]
+    weights = {name: tiled_weight(ops, QuantScheme.GgufQ4_0, n, k, 50 + i, 0.015) for i, (name, n, k) in enumerate(shapes70)}
+    wbytes = sum(n * k // 32 * 18 for _, n, k in shapes70)
+    sweep = {}
+    for m in (1, 4, 16, 64, 256):
+        total_ms = 0.0
+        for name, n, k in shapes70:
+            total_ms += run_matmul([weights[name]], m, k, DType.BF16, 30 if m > 16 else 100, 5)
+        flops = sum(2.0 * m * n * k for _, n, k in shapes70)
+        algo = wbytes + sum(2 * m * k + 4 * m * n for _, n, k in shapes70)
+        sweep[f"M={m}"] = {"us_layer": round(total_ms * 1e3, 1), "GB/s": round(algo / total_ms / 1e6, 1),
+                           "TFLOP/s": round(flops / total_ms / 1e9, 2),
+                           "path": "gemv" if m <= 16 else "gemm"}
+    out["q4_0_batch_sweep_llama70b_layer"] = sweep
+    for q in weights.values():
+        q.free()
     return out
 
 

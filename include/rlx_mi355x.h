@@ -82,6 +82,7 @@ int rlx_mi355x_free(void *dptr);
 int rlx_mi355x_memcpy_h2d(void *dst, const void *src, size_t nbytes);
 int rlx_mi355x_memcpy_d2h(void *dst, const void *src, size_t nbytes);
 int rlx_mi355x_memset_u32(void *dst, uint32_t value, size_t n_words, void *stream); /* fill kernel, graph-safe */
+int rlx_mi355x_memcpy_d2d(void *dst, const void *src, size_t nbytes, void *stream); /* copy kernel; 16-byte multiples */
 int rlx_mi355x_stream_create(void **stream);
 int rlx_mi355x_stream_destroy(void *stream);
 int rlx_mi355x_stream_sync(void *stream);
@@ -146,7 +147,7 @@ int rlx_mi355x_gguf_matmul_bt_batch(const void *const *xs_dev, int x_dtype, cons
  *   x_dev, out_dev : len f32 (may alias)
  *   codes_dev      : optional len int8, the integer codes clamp(round(x/s)) (NULL to skip)
  *   state_dev      : chan_dim f32; read for FIXED, read+written for EMA, ignored (may be NULL) for PER_BATCH
- *   scratch_dev    : chan_dim * 4 bytes of device scratch for the per-channel maxima (PER_BATCH / EMA)
+ *   scratch_dev    : chan_dim * 8 bytes of device scratch: per-channel maxima, then per-channel scales
  * bits in {8,4,2} -> q_max {127,7,1}; anything else is RLX_ERR_UNSUPPORTED (the reference panics). */
 int rlx_mi355x_fake_quantize(const float *x_dev, float *out_dev, int8_t *codes_dev, int64_t len, int64_t chan_dim,
                              int64_t inner, int bits, int scale_mode, float ema_decay, float *state_dev,

@@ -57,6 +57,7 @@ SIGNATURES = {
     "rlx_mi355x_memcpy_h2d": (_i, [_vp, _vp, _sz]),
     "rlx_mi355x_memcpy_d2h": (_i, [_vp, _vp, _sz]),
     "rlx_mi355x_memset_u32": (_i, [_vp, _u32, _sz, _vp]),
+    "rlx_mi355x_memcpy_d2d": (_i, [_vp, _vp, _sz, _vp]),
     "rlx_mi355x_stream_create": (_i, [_pvp]),
     "rlx_mi355x_stream_destroy": (_i, [_vp]),
     "rlx_mi355x_stream_sync": (_i, [_vp]),

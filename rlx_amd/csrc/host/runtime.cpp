@@ -25,7 +25,7 @@ static const char *const kKernelNames[K_COUNT] = {
     "rlx_dequant_q4_0", "rlx_dequant_q8_0", "rlx_dequant_q4_k",
     "rlx_fq_col_absmax", "rlx_fq_seg_absmax", "rlx_fq_flat_absmax", "rlx_fq_scale", "rlx_fq_col_apply",
     "rlx_fq_flat_apply", "rlx_fq_flat4_apply",
-    "rlx_fill_u32",
+    "rlx_fill_u32", "rlx_copy_u128",
     "rlx_gemv_q4_0_r2", "rlx_gemv_q4_0_r2_d8", "rlx_gemv_q4_0_r4", "rlx_gemv_q8_0_r2", "rlx_gemv_q8_0_r4", "rlx_gemv_q4_k_r2", "rlx_gemv_q4_k_r4",
     "rlx_gemm_q4_k", "rlx_gemm_q4_0", "rlx_gemm_q8_0", "rlx_xprep",
 };
@@ -141,6 +141,17 @@ int rlx_mi355x_memset_u32(void *dst, uint32_t value, size_t n_words, void *strea
     unsigned blocks = (unsigned)((n + 255) / 256 > 4096 ? 4096 : (n + 255) / 256);
     void *params[] = {&dst, &value, &n};
     return rlx::launch(rlx::K_FILL_U32, blocks, 1, 256, 0, (hipStream_t)stream, params);
+}
+int rlx_mi355x_memcpy_d2d(void *dst, const void *src, size_t nbytes, void *stream) {
+    if (nbytes == 0) return RLX_OK;
+    if ((nbytes | (uintptr_t)dst | (uintptr_t)src) & 15) {
+        rlx::set_error("memcpy_d2d: pointers and size must be multiples of 16 bytes");
+        return RLX_ERR_INVALID;
+    }
+    long long n = (long long)(nbytes / 16);
+    unsigned blocks = (unsigned)((n + 255) / 256 > 8192 ? 8192 : (n + 255) / 256);
+    void *params[] = {&dst, &src, &n};
+    return rlx::launch(rlx::K_COPY_U128, blocks, 1, 256, 0, (hipStream_t)stream, params);
 }
 int rlx_mi355x_stream_create(void **stream) {
     RLX_TRY(rlx::runtime_init());

@@ -229,3 +229,10 @@ extern "C" __global__ __launch_bounds__(256) void rlx_fill_u32(uint32_t *dst, ui
     const long long stride = (long long)gridDim.x * blockDim.x;
     for (; i < n; i += stride) dst[i] = value;
 }
+
+// Plain device-to-device copy of n 16-byte words (graph-safe; also the unit against which HBM counters are scaled).
+extern "C" __global__ __launch_bounds__(256) void rlx_copy_u128(rlx::uint4_t *dst, const rlx::uint4_t *src, long long n) {
+    long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long long stride = (long long)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) dst[i] = src[i];
+}
