@@ -167,14 +167,20 @@ static int launch_gemm(const void *x, int xk, const rlx_qweight *w, float *out, 
     void *sxh = p.sxh_bytes ? (uint8_t *)workspace + p.xh_bytes : nullptr;
     XPrepArgs xa{x, xh, sxh, (int)m, (int)w->dims.k, (int)p.k_pad, (int)p.m_rows, xk};
     void *xparams[] = {&xa};
-    const long long waves = p.m_rows * (p.k_pad / 256);
-    RLX_TRY(launch(K_XPREP, (unsigned)((waves + 3) / 4), 1, 256, 0, stream, xparams));
+    const long long xblocks = (p.m_rows / 256) * (p.k_pad / 64) * 8;  // (tile, step, 32-row sub-tile)
+    RLX_TRY(launch(K_XPREP, (unsigned)xblocks, 1, 256, 0, stream, xparams));
 
     const int steps_per_unit = L.unit_k / 64;
-    const int gx = (int)((w->dims.row_tiles * 16 + 127) / 128), gy = (int)(p.m_rows / 256);
-    const int cus = std::max(1, device_props().cu_count);
+    // Up to 128 activation rows run the 64-row tile (the weights are decoded once per 64 rows, but nothing is spent on
+    // padding rows); beyond that the 256-row tile.
+    const int64_t rv = xk == 0 ? 2 * m : m;
+    const bool skinny = rv <= 128;
+    const int gx = (int)((w->dims.row_tiles * 16 + 127) / 128);
+    const int gy = skinny ? (int)((rv + 63) / 64) : (int)(p.m_rows / 256);
+    // workgroup slots to fill: one per CU for the 256-row tile (144 KB of LDS), two for the 64-row tile
+    const long long slots = (long long)std::max(1, device_props().cu_count) * (skinny ? 2 : 1);
     int split = 1;
-    if ((long long)gx * gy * 5 < (long long)cus * 4) split = (int)std::min<long long>(w->dims.units, cus / ((long long)gx * gy));
+    if ((long long)gx * gy * 5 < slots * 4) split = (int)std::min<long long>(w->dims.units, slots / ((long long)gx * gy));
     split = std::max(1, split);
     int units_per_split = (int)((w->dims.units + split - 1) / split);
     if (steps_per_unit == 2) units_per_split = (units_per_split + 1) & ~1;  // keep every split a multiple of 4 steps
@@ -183,9 +189,11 @@ static int launch_gemm(const void *x, int xk, const rlx_qweight *w, float *out, 
     GemmArgs a{w->dev, xh, sxh, out, (int)p.m_rows, (int)m, (int)w->dims.n, (int)p.k_pad, (int)w->dims.units,
                (int)w->dims.row_tiles, xk == 0 ? 1 : 0, units_per_split * steps_per_unit, split > 1 ? 1 : 0};
     void *params[] = {&a};
-    KernelId id = w->scheme == SCHEME_Q4K ? K_GEMM_Q4_K : w->scheme == SCHEME_Q4_0 ? K_GEMM_Q4_0 : K_GEMM_Q8_0;
+    KernelId id = w->scheme == SCHEME_Q4K    ? (skinny ? K_GEMM64_Q4_K : K_GEMM_Q4_K)
+                  : w->scheme == SCHEME_Q4_0 ? (skinny ? K_GEMM64_Q4_0 : K_GEMM_Q4_0)
+                                             : (skinny ? K_GEMM64_Q8_0 : K_GEMM_Q8_0);
     RLX_TRY(runtime_init());
-    RLX_TRY(launch3(id, (unsigned)gx, (unsigned)gy, (unsigned)split, 512, 2 * 48 * 1024, stream, params));
+    RLX_TRY(launch3(id, (unsigned)gx, (unsigned)gy, (unsigned)split, 512, skinny ? 3 * 24 * 1024 : 3 * 48 * 1024, stream, params));
     return RLX_OK;
 }
 

@@ -21,7 +21,7 @@ constexpr float GEMM_LO_SCALE = 2048.0f;
 
 struct GemmArgs {
     const uint8_t *w;
-    const half_t *xh;   // [m_rows][k_pad] binary16 activations (rows padded to 256, columns to a multiple of 256)
+    const half_t *xh;   // binary16 activations as LDS stage images: [m_rows / 256][k_pad / 64][32 KB] (see rlx_xprep)
     const half_t *sxh;  // Q4_K: [m_rows][k_pad / 256][16]: per 32-column block sums, 8 x hi then 8 x lo*2048
     float *out;         // [m_out][n]
     int m_rows;         // rows of xh
@@ -52,34 +52,39 @@ __device__ __forceinline__ int frag_offset(int ns, int ks, int s, int r, int h) 
 }
 
 // Workgroup = 8 waves (two per SIMD) as 4 x 2, tile 256 rows of x by 128 rows of W, each wave 64 x 64 = 2 x 2 tiles of
-// v_mfma_f32_32x32x16_f16. K advances in 64-column steps through two LDS stages (96 KB). On gfx950 a matrix
+// v_mfma_f32_32x32x16_f16. K advances in 64-column steps through three LDS stages (144 KB). On gfx950 a matrix
 // instruction leaves room for only about four other vector instructions in its shadow, so the step is written as
 // four k-slice groups, each: LDS reads of the next slice's fragments, the slice's four MFMAs, and one quarter of the
 // work that prepares the next step (LDS stores of activations fetched two steps ago, decode + store of the packed
 // weights), with scheduling fences so the compiler keeps that interleaving. Global loads run two steps ahead in
 // registers. The loop is unrolled by four steps (one Q4_K super-block) so every phase test and register-set index
 // is a compile-time constant.
-template <int SCHEME>
+// TI x TJ = MFMA tiles per wave: 2 x 2 is the prefill shape above; 1 x 1 puts the eight waves as 2 x 4 over a 64 x 128
+// tile for batches of a few dozen rows, where the job is to stream the weights and most of a 256-row tile would be
+// padding. Both read the same activation workspace (a 64-row tile is two 32-row sub-tiles of a 256-row image).
+template <int SCHEME, int TI, int TJ>
 __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
     constexpr Layout L = layout_of(SCHEME);
     constexpr bool K4 = SCHEME == SCHEME_Q4K;
+    constexpr int WN = GEMM_NT / (32 * TJ), WM = 8 / WN, MT = WM * TI * 32;  // wave grid and rows per workgroup
+    constexpr int NSA = MT / 32, SA = 4 * NSA * 1024, ST = SA + GEMM_STAGE_B;  // LDS stage: activations [4][NSA][1 KB], then weights
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave / WN, wn = wave % WN;
     const int lr = lane & 31, lh = lane >> 5;
-    const int n_tile0 = blockIdx.x * GEMM_NT, m_tile0 = blockIdx.y * GEMM_MT;
+    const int n_tile0 = blockIdx.x * GEMM_NT, m_tile0 = blockIdx.y * MT;
     const int step0 = blockIdx.z * a.steps_per_split;
     const int total_steps = a.units * (L.unit_k / GEMM_KS);
     const int step1 = min(step0 + a.steps_per_split, total_steps);
 
-    // ---- A loader: thread -> 16-byte chunk c = tid % 8 of rows tid/8 + 64 i, i = 0..3 (sub-tile (tid/8)/32 + 2 i) ----
-    const int a_row = tid >> 3, a_c = tid & 7;
-    const uint8_t *a_base = (const uint8_t *)(a.xh + (long long)m_tile0 * a.k_pad);  // wave-uniform
-    const uint32_t a_off0 = ((uint32_t)a_row * (uint32_t)a.k_pad + (uint32_t)a_c * 8u) * 2u;
-    const uint32_t a_stride64 = (uint32_t)a.k_pad * 128u;  // bytes between rows r and r + 64
-    const int a_dst0 = frag_offset(8, a_c >> 1, a_row >> 5, a_row & 31, a_c & 1);  // + i * 2048 for rows + 64 i
+    // ---- A loader: the activation workspace already holds, per (256-row tile, 64-column step), the 32 KB image of
+    // the LDS stage (fragment order, swizzle included), so thread t moves 16-byte chunks t, t + 512, ... unchanged.
+    const uint8_t *a_base = (const uint8_t *)a.xh + (long long)(m_tile0 / GEMM_MT) * (a.k_pad / GEMM_KS) * GEMM_STAGE_A;  // wave-uniform
+    const int a_sub0 = (m_tile0 % GEMM_MT) / 32;                 // first sub-tile of the image this workgroup uses
+    const bool a_mine = MT == GEMM_MT || (wave >= a_sub0 && wave < a_sub0 + MT / 32);  // chunk t + 512 i belongs to sub-tile t / 64 = wave
+    const int a_src0 = tid * 16, a_dst0 = ((wave - a_sub0) * 64 + lane) * 16;
 
     // ---- B loader: thread -> lane slot (n16 = lane % 16, g = lane / 16) of 16-row tile `wave` ---------------
     const int b_n16 = lane & 15, b_g = lane >> 4;
@@ -92,19 +97,24 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
         const int row = wave * 16 + b_n16;
 #pragma unroll
         for (int jl = 0; jl < 2; jl++)
-            b_dst[jl] = GEMM_STAGE_A + frag_offset(4, 2 * jl + (b_g >> 1), row >> 5, row & 31, b_g & 1);
+            b_dst[jl] = SA + frag_offset(4, 2 * jl + (b_g >> 1), row >> 5, row & 31, b_g & 1);
     }
 
     // Register-resident prefetch: activations one step ahead, packed weights two.
-    uint4_t a_reg[4];                                   // activations of the next step
+    uint4_t a_reg[2][4];                                // activations of the next steps, [step parity] (Q4_K: one set)
     uint4_t b_q[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};      // [chunk parity] packed codes of a two-step chunk (Q8_0: [step parity])
     uint4_t b_meta[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};   // Q4_K: [0] = meta of the super-block decoded next; else [chunk parity] .x/.y = four f16 scales
     uint32_t b_sc[2] = {0, 0};                          // Q4_K: 6-bit scales of sub-blocks 0-3 / 4-7 being decoded
 
-    auto fetch_a = [&](int step) {
-        const uint8_t *p = a_base + (long long)step * (GEMM_KS * 2) + a_off0;
+    // Activations run AD steps ahead of their LDS store: two where registers allow (their loads come through L2 with
+    // the whole workgroup's 32 KB per step behind them), one for Q4_K whose second accumulator set takes the room.
+    constexpr int AD = K4 ? 1 : 2;
+    auto fetch_a = [&](int step, int set) {
+        const uint8_t *p = a_base + (long long)step * GEMM_STAGE_A + a_src0;
+        if (a_mine) {
 #pragma unroll
-        for (int i = 0; i < 4; i++) a_reg[i] = *(const uint4_t *)(p + (size_t)i * a_stride64);
+            for (int i = 0; i < 4; i++) a_reg[AD == 2 ? set : 0][i] = *(const uint4_t *)(p + i * 8192);
+        }
     };
     auto fetch_b = [&](int step, int q) {  // q = step & 3, compile-time at every call site
         if constexpr (K4) {  // dead tiles read tile 0 (valid memory) and are zeroed when stored
@@ -129,9 +139,10 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
             }
         }
     };
-    auto store_a2 = [&](uint8_t *stage, int i0) {  // two of the four activation chunks
+    auto store_a2 = [&](uint8_t *stage, int i0, int set) {  // two of the four activation chunks
 #pragma unroll
-        for (int i = i0; i < i0 + 2; i++) *(uint4_t *)(stage + a_dst0 + i * 2048) = a_reg[i];
+        for (int i = i0; i < i0 + 2; i++)
+            if (a_mine) *(uint4_t *)(stage + a_dst0 + i * (NSA * 1024)) = a_reg[AD == 2 ? set : 0][i];
     };
     // decode block jl (0/1) of the step `step` with phase q into LDS
     auto store_b1 = [&](int step, int q, int jl, uint8_t *stage) {
@@ -159,74 +170,82 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
     };
 
     // ---- accumulators ----------------------------------------------------------------------------------
-    float16_t total[2][2], part[2][2], zero16;
+    float16_t total[TI][TJ], part[TI][TJ], zero16;
 #pragma unroll
     for (int e = 0; e < 16; e++) zero16[e] = 0.f;
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int i = 0; i < TI; i++)
 #pragma unroll
-        for (int j = 0; j < 2; j++) {
+        for (int j = 0; j < TJ; j++) {
             total[i][j] = zero16;
             part[i][j] = zero16;
         }
     // this lane's two W rows (one per 32-column MFMA tile) for the Q4_K per-super-block scaling
-    int my_row[2];
-    const uint8_t *my_meta[2];
-    bool my_ok[2];
+    int my_row[TJ];
+    const uint8_t *my_meta[TJ];
+    bool my_ok[TJ];
 #pragma unroll
-    for (int j = 0; j < 2; j++) {
-        my_row[j] = n_tile0 + wn * 64 + 32 * j + lr;
+    for (int j = 0; j < TJ; j++) {
+        my_row[j] = n_tile0 + (wn * TJ + j) * 32 + lr;
         my_ok[j] = (my_row[j] >> 4) < a.row_tiles;
         my_meta[j] = a.w + (long long)(my_ok[j] ? (my_row[j] >> 4) : 0) * a.units * L.unit_bytes + 2048 + (my_row[j] & 15) * 16;
     }
-    uint4_t w_meta[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};
-    Frag fs[2];
+    uint4_t w_meta[TJ];
+    Frag fs[TI];
+#pragma unroll
+    for (int j = 0; j < TJ; j++) w_meta[j] = uint4_t{0, 0, 0, 0};
     int a_rd[4], b_rd[4];  // per k-slice read offsets of this lane; + sub-tile * 1024
 #pragma unroll
     for (int ks = 0; ks < 4; ks++) {
-        a_rd[ks] = frag_offset(8, ks, wm * 2, lr, lh);
-        b_rd[ks] = GEMM_STAGE_A + frag_offset(4, ks, wn * 2, lr, lh);
+        a_rd[ks] = frag_offset(NSA, ks, wm * TI, lr, lh);
+        b_rd[ks] = SA + frag_offset(4, ks, wn * TJ, lr, lh);
     }
-    Frag fa[2][2], fb[2][2];  // [buffer][tile]
+    Frag fa[2][TI], fb[2][TJ];  // [buffer][tile]
     auto load_frags = [&](const uint8_t *stage, int ks, int buf) {
 #pragma unroll
-        for (int i = 0; i < 2; i++) fa[buf][i].u4 = *(const uint4_t *)(stage + a_rd[ks] + i * 1024);
+        for (int i = 0; i < TI; i++) fa[buf][i].u4 = *(const uint4_t *)(stage + a_rd[ks] + i * 1024);
 #pragma unroll
-        for (int j = 0; j < 2; j++) fb[buf][j].u4 = *(const uint4_t *)(stage + b_rd[ks] + j * 1024);
+        for (int j = 0; j < TJ; j++) fb[buf][j].u4 = *(const uint4_t *)(stage + b_rd[ks] + j * 1024);
     };
 
     if (step0 < step1) {  // step0 is a multiple of 4
-        fetch_a(step0);
+        fetch_a(step0, 0);
         fetch_b(step0, 0);
+        if (AD == 2) fetch_a(min(step0 + 1, step1 - 1), 1);
         fetch_b(min(step0 + 1, step1 - 1), 1);
-        store_a2(smem, 0);
-        store_a2(smem, 2);
+        store_a2(smem, 0, 0);
+        store_a2(smem, 2, 0);
         store_b1(step0, 0, 0, smem);
         store_b1(step0, 0, 1, smem);
     }
     __syncthreads();
+    if (step0 < step1) load_frags(smem, 0, 0);
+    // Three LDS stages: step s reads stage s % 3 and fills stage (s + 1) % 3, whose last readers (step s - 2) all
+    // passed the barrier of step s - 1. The one barrier per step sits after the third k-slice, when this step's
+    // stores are long issued, and the last slice already reads the first fragments of the next step: no wave
+    // starts a step by waiting for LDS.
+    int rd_off = 0, wr_off = ST;  // wave-uniform
 
     for (int sbase = step0; sbase < step1; sbase += 4) {
 #pragma unroll
         for (int q = 0; q < 4; q++) {
             const int step = sbase + q;
             if (step < step1) {
-                const uint8_t *stage = smem + (q & 1) * GEMM_STAGE;
-                uint8_t *next = smem + ((q & 1) ^ 1) * GEMM_STAGE;
+                const uint8_t *stage = smem + rd_off;
+                uint8_t *next = smem + wr_off;
                 // No branches inside a step: the last steps re-fetch / re-store the final step into a stage nobody
                 // reads again, so each k-slice group below is one scheduling region.
                 const int nstep = min(step + 1, step1 - 1);
-                load_frags(stage, 0, 0);
-                fetch_a(nstep);
+                fetch_a(AD == 2 ? min(step + 2, step1 - 1) : nstep, q & 1);
                 fetch_b(min(step + 2, step1 - 1), (q + 2) & 3);
                 if constexpr (K4) {
                     if (q == 0) {  // this wave's rows: meta and activation block sums of the super-block, used at q == 3
                         const int sb = step >> 2;
 #pragma unroll
-                        for (int j = 0; j < 2; j++) w_meta[j] = *(const uint4_t *)(my_meta[j] + (long long)sb * L.unit_bytes);
+                        for (int j = 0; j < TJ; j++) w_meta[j] = *(const uint4_t *)(my_meta[j] + (long long)sb * L.unit_bytes);
 #pragma unroll
-                        for (int i = 0; i < 2; i++) {
-                            long long row = m_tile0 + (wm * 2 + i) * 32 + lr;
+                        for (int i = 0; i < TI; i++) {
+                            long long row = m_tile0 + (wm * TI + i) * 32 + lr;
                             fs[i].u4 = *(const uint4_t *)(a.sxh + (row * (a.k_pad / 256) + sb) * 16 + lh * 8);
                         }
                     }
@@ -236,10 +255,11 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
                 for (int ks = 0; ks < 4; ks++) {
                     const int buf = ks & 1;
                     if (ks < 3) load_frags(stage, ks + 1, buf ^ 1);
+                    else load_frags(next, 0, 0);  // after this step's barrier
 #pragma unroll
-                    for (int i = 0; i < 2; i++)
+                    for (int i = 0; i < TI; i++)
 #pragma unroll
-                        for (int j = 0; j < 2; j++) {
+                        for (int j = 0; j < TJ; j++) {
                             if constexpr (K4) {
                                 // the first slice of a super-block starts the partial product from zero
                                 part[i][j] = mfma32(fa[buf][i], fb[buf][j], (q == 0 && ks == 0) ? zero16 : part[i][j]);
@@ -250,22 +270,26 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
                     // weights first: the activations were fetched only at the top of this step
                     if (ks == 0) store_b1(nstep, (q + 1) & 3, 0, next);
                     if (ks == 1) store_b1(nstep, (q + 1) & 3, 1, next);
-                    if (ks == 2) store_a2(next, 0);
-                    if (ks == 3) store_a2(next, 2);
+                    if (ks == 2) {
+                        store_a2(next, 0, (q + 1) & 1);
+                        store_a2(next, 2, (q + 1) & 1);
+                    }
                     // order inside the group: the LDS reads of the next slice, then MFMA / few VALU alternating
-                    __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x100, TI + TJ, 0);
 #pragma unroll
                     for (int r = 0; r < 4; r++) {
-                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                        if (r < TI * TJ) __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
                         __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+                        if (ks == 2) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
                     }
-                    __builtin_amdgcn_sched_group_barrier(0x200, 2, 0);
+                    if (ks < 2) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
                     __builtin_amdgcn_sched_barrier(0);
+                    if (ks == 2) __syncthreads();
                 }
                 if constexpr (K4) {
                     if (q == 3) {  // a 256-column super-block is complete: total += d * P - dmin * (mn . sx)
 #pragma unroll
-                        for (int j = 0; j < 2; j++) {
+                        for (int j = 0; j < TJ; j++) {
                             const uint4_t meta = w_meta[j];
                             const float d = my_ok[j] ? half_bits_to_float(meta[0] & 0xFFFFu) : 0.f;
                             const float dmin = my_ok[j] ? half_bits_to_float(meta[0] >> 16) : 0.f;
@@ -283,7 +307,7 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
                                 fm.h2[e] = lh ? v * lo_scale : v;
                             }
 #pragma unroll
-                            for (int i = 0; i < 2; i++) {
+                            for (int i = 0; i < TI; i++) {
                                 float16_t qq = mfma32(fs[i], fm, zero16);
 #pragma unroll
                                 for (int e = 0; e < 16; e++) {
@@ -294,21 +318,22 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
                         }
                     }
                 }
-                __syncthreads();
+                rd_off = wr_off;
+                wr_off = wr_off == 2 * ST ? 0 : wr_off + ST;
             }
         }
     }
 
     // ---- epilogue: register e of tile (i, j) is row 8 (e/4) + 4 lh + e%4, column lr ------------------------
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int i = 0; i < TI; i++)
 #pragma unroll
-        for (int j = 0; j < 2; j++) {
+        for (int j = 0; j < TJ; j++) {
             const int col = my_row[j];
             if (col >= a.n) continue;
 #pragma unroll
             for (int e = 0; e < 16; e++) {
-                const int vrow = m_tile0 + (wm * 2 + i) * 32 + 8 * (e >> 2) + 4 * lh + (e & 3);
+                const int vrow = m_tile0 + (wm * TI + i) * 32 + 8 * (e >> 2) + 4 * lh + (e & 3);
                 float v = total[i][j][e];
                 int orow = vrow;
                 if (a.pair_rows) {
@@ -326,7 +351,9 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
 }
 
 // ---- activation preparation -------------------------------------------------------------------------
-// x [m, k] (f32 / bf16 / f16) -> xh [m_rows][k_pad] binary16 (+ zero padding), and for Q4_K the per-block sums.
+// x [m, k] (f32 / bf16 / f16) -> binary16 in the order the GEMM's LDS stage wants it: for each 256-row tile and
+// 64-column step one 32 KB image [k-slice][32-row sub-tile][slot][8 halfs] (frag_offset), zero padded; and for Q4_K
+// the per-32-column sums of the rounded values, as hi / lo*2048 halfs: sxh[row][k_pad / 256][16].
 struct XPrepArgs {
     const void *x;
     half_t *xh;
@@ -335,60 +362,75 @@ struct XPrepArgs {
     int x_dtype;  // 0 f32 (rows become hi / lo*2048 pairs), 1 bf16, 2 f16
 };
 
+// One workgroup of four waves per (tile, step, sub-tile); wave = k-slice, lane = slot of the 1 KB fragment block.
 __device__ __forceinline__ void xprep_body(const XPrepArgs &a) {
-    // one wave per (virtual row, 256-column span): lane handles 4 columns; 8 lanes = one 32-column block
-    const int lane = threadIdx.x & 63, wave_in_block = threadIdx.x >> 6;
-    const long long gw = (long long)blockIdx.x * (blockDim.x >> 6) + wave_in_block;
-    const int spans = a.k_pad / 256;
-    const long long vrow = gw / spans;
-    const int span = (int)(gw % spans);
-    if (vrow >= a.m_rows) return;
-    const int col = span * 256 + lane * 4;
+    __shared__ float part[4][32];
+    const int lane = threadIdx.x & 63, ks = threadIdx.x >> 6;
+    const int steps = a.k_pad / GEMM_KS;
+    const int sub = blockIdx.x & 7;
+    const int step = (blockIdx.x >> 3) % steps;
+    const int tile = (blockIdx.x >> 3) / steps;
+    const int h = lane >> 5, c = 2 * ks + h;
+    const int r = (lane & 31) ^ c;  // the slot's row within the sub-tile (frag_offset's swizzle is its own inverse)
+    const long long vrow = (long long)tile * GEMM_MT + sub * 32 + r;
+    const int col = step * GEMM_KS + c * 8;
     const bool paired = a.x_dtype == 0;
     const long long src_row = paired ? (vrow >> 1) : vrow;
-    float v[4] = {0.f, 0.f, 0.f, 0.f};
-    if (src_row < a.m && col < a.k) {
+    float v[8];
+#pragma unroll
+    for (int e = 0; e < 8; e++) v[e] = 0.f;
+    if (src_row < a.m && col < a.k) {  // k is a multiple of 32, so a chunk of 8 is inside or outside as a whole
         if (a.x_dtype == 0) {
-            float4_t t = *(const float4_t *)((const float *)a.x + src_row * a.k + col);
-            v[0] = t[0]; v[1] = t[1]; v[2] = t[2]; v[3] = t[3];
-        } else {
-            uint2_t raw = *(const uint2_t *)((const uint16_t *)a.x + src_row * a.k + col);
+            const float4_t *p = (const float4_t *)((const float *)a.x + src_row * a.k + col);
+            float4_t t0 = p[0], t1 = p[1];
 #pragma unroll
             for (int e = 0; e < 4; e++) {
+                v[e] = t0[e];
+                v[4 + e] = t1[e];
+            }
+        } else {
+            uint4_t raw = *(const uint4_t *)((const uint16_t *)a.x + src_row * a.k + col);
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
                 uint32_t bits = (e & 1) ? (raw[e >> 1] >> 16) : (raw[e >> 1] & 0xFFFFu);
                 v[e] = a.x_dtype == 1 ? __builtin_bit_cast(float, bits << 16) : (float)__builtin_bit_cast(half_t, (uint16_t)bits);
             }
         }
     }
-    typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
-    half4_t h;
+    Frag f;
     float sum = 0.f;
 #pragma unroll
-    for (int e = 0; e < 4; e++) {
+    for (int e = 0; e < 8; e++) {
         half_t hi = (half_t)v[e];
         if (paired && (vrow & 1)) hi = (half_t)((v[e] - (float)hi) * GEMM_LO_SCALE);  // odd rows carry the residual
-        h[e] = hi;
+        f.h8[e] = hi;
         sum += (float)hi;
     }
-    *(half4_t *)(a.xh + vrow * a.k_pad + col) = h;
+    uint8_t *dst = (uint8_t *)a.xh + ((long long)tile * steps + step) * GEMM_STAGE_A + ((ks * 8 + sub) * 64 + lane) * 16;
+    *(uint4_t *)dst = f.u4;
     if (a.sxh) {
-        // block sum over 8 lanes, then split into hi + lo*2048 halfs
-        sum += __shfl_xor(sum, 1);
-        sum += __shfl_xor(sum, 2);
-        sum += __shfl_xor(sum, 4);
-        if ((lane & 7) == 0) {
-            half_t hi = (half_t)sum;
-            half_t lo = (half_t)((sum - (float)hi) * GEMM_LO_SCALE);
-            half_t *dst = a.sxh + (vrow * spans + span) * 16 + (lane >> 3);
-            dst[0] = hi;
-            dst[8] = lo;
+        sum += __shfl_xor(sum, 33);  // the slot holding the other 8 columns of this row's k-slice
+        if (h == 0) part[ks][r] = sum;
+        __syncthreads();
+        if (threadIdx.x < 64) {  // (row, 32-column block of the step) -> hi + lo*2048 halfs
+            const int rr = threadIdx.x & 31, blk = threadIdx.x >> 5;
+            const float s32 = part[2 * blk][rr] + part[2 * blk + 1][rr];
+            const half_t hi = (half_t)s32;
+            const half_t lo = (half_t)((s32 - (float)hi) * GEMM_LO_SCALE);
+            const long long row = (long long)tile * GEMM_MT + sub * 32 + rr;
+            half_t *d = a.sxh + (row * (a.k_pad / 256) + (step >> 2)) * 16 + (step & 3) * 2 + blk;
+            d[0] = hi;
+            d[8] = lo;
         }
     }
 }
 
 }  // namespace rlx
 
-extern "C" __global__ __launch_bounds__(512) void rlx_gemm_q4_k(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q4K>(a); }
-extern "C" __global__ __launch_bounds__(512) void rlx_gemm_q4_0(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q4_0>(a); }
-extern "C" __global__ __launch_bounds__(512) void rlx_gemm_q8_0(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q8_0>(a); }
+extern "C" __global__ __launch_bounds__(512) void rlx_gemm_q4_k(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q4K, 2, 2>(a); }
+extern "C" __global__ __launch_bounds__(512) void rlx_gemm_q4_0(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q4_0, 2, 2>(a); }
+extern "C" __global__ __launch_bounds__(512) void rlx_gemm_q8_0(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q8_0, 2, 2>(a); }
+extern "C" __global__ __launch_bounds__(512) void rlx_gemm64_q4_k(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q4K, 1, 1>(a); }
+extern "C" __global__ __launch_bounds__(512) void rlx_gemm64_q4_0(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q4_0, 1, 1>(a); }
+extern "C" __global__ __launch_bounds__(512) void rlx_gemm64_q8_0(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q8_0, 1, 1>(a); }
 extern "C" __global__ __launch_bounds__(256) void rlx_xprep(rlx::XPrepArgs a) { rlx::xprep_body(a); }

@@ -383,7 +383,13 @@ def test_graph_batches_independent_matmuls(oracle):
 
 @pytest.mark.parametrize("scheme", [Q4K, Q4_0, Q8_0])
 @pytest.mark.parametrize("m,n,k,x_dtype", [(64, 256, 512, DType.BF16), (300, 200, 768, DType.BF16),
-                                           (40, 128, 1024, DType.F32), (512, 384, 2048, DType.F16)])
+                                           (40, 128, 1024, DType.F32), (512, 384, 2048, DType.F16),
+                                           # the 64-row tile: one and two row groups, ragged N, split K, both edges
+                                           # of the switch to the 256-row tile (128 / 129 activation rows)
+                                           (17, 128, 512, DType.BF16), (100, 168, 1280, DType.F16),
+                                           (9, 64, 768, DType.F32), (33, 128, 8192, DType.BF16),
+                                           (128, 96, 256, DType.BF16), (129, 96, 256, DType.BF16),
+                                           (64, 80, 512, DType.F32), (65, 80, 512, DType.F32)])
 def test_gemm_small(oracle, scheme, m, n, k, x_dtype):
     check_matmul(oracle, scheme, n, k, m, x_dtype=x_dtype, seed=m + n)
 
