@@ -148,8 +148,10 @@ int rlx_mi355x_gguf_matmul_bt_batch(const void *const *xs_dev, int x_dtype, cons
  *   x_dev, out_dev : len f32 (may alias)
  *   codes_dev      : optional len int8, the integer codes clamp(round(x/s)) (NULL to skip)
  *   state_dev      : chan_dim f32; read for FIXED, read+written for EMA, ignored (may be NULL) for PER_BATCH
- *   scratch_dev    : chan_dim * 8 bytes of device scratch: per-channel maxima, then per-channel scales
+ *   scratch_dev    : rlx_mi355x_fake_quantize_scratch_bytes() bytes of device scratch, 16-byte aligned: per-channel
+ *                    maxima [chan_dim], per-channel scales [chan_dim], then partial maxima of the first pass
  * bits in {8,4,2} -> q_max {127,7,1}; anything else is RLX_ERR_UNSUPPORTED (the reference panics). */
+size_t rlx_mi355x_fake_quantize_scratch_bytes(int64_t len, int64_t chan_dim, int64_t inner);
 int rlx_mi355x_fake_quantize(const float *x_dev, float *out_dev, int8_t *codes_dev, int64_t len, int64_t chan_dim,
                              int64_t inner, int bits, int scale_mode, float ema_decay, float *state_dev,
                              int round_mode, void *scratch_dev, void *stream);

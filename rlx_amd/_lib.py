@@ -78,6 +78,7 @@ SIGNATURES = {
     "rlx_mi355x_gguf_matmul_bt": (_i, [_vp, _i, _vp, _vp, _i64, _vp, _sz, _vp]),
     "rlx_mi355x_gguf_matmul_workspace": (_sz, [_i, _i, _i64, _i64, _i64]),
     "rlx_mi355x_gguf_matmul_bt_batch": (_i, [_pvp, _i, _pvp, _pvp, _i, _i64, _vp, _sz, _vp]),
+    "rlx_mi355x_fake_quantize_scratch_bytes": (_sz, [_i64, _i64, _i64]),
     "rlx_mi355x_fake_quantize": (_i, [_vp, _vp, _vp, _i64, _i64, _i64, _i, _i, _f, _vp, _i, _vp, _vp]),
     "rlx_mi355x_quantize": (_i, [_i, _vp, _i64, _vp]),
     "rlx_mi355x_philox_u32": (None, [C.c_uint64, _vp, _i64]),

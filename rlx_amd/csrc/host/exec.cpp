@@ -354,7 +354,7 @@ rlx_exec *rlx_mi355x_compile(const rlx_graph_desc *g, const rlx_compile_opts *op
             nd.slot = take((size_t)nd.numel * dtype_size(nd.d.dtype));
         }
         if (nd.d.op_kind == RLX_OP_FAKE_QUANTIZE) {
-            nd.aux = take((size_t)nd.chan_dim * 8);
+            nd.aux = take(rlx_mi355x_fake_quantize_scratch_bytes(nd.numel, nd.chan_dim, nd.inner));
             nd.codes = take((size_t)nd.numel);
         }
         if (nd.d.op_kind == RLX_OP_DEQUANT_MATMUL && nd.m > 8)  // prefill workspace, sized for f32 activations

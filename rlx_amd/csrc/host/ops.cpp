@@ -46,6 +46,8 @@ struct FqArgs {
     long long len, chan_dim, inner;
     float q_max, decay;
     int scale_mode, round_mode, rows_per_block;
+    float *partial;
+    int parts;
 };
 
 struct GemmArgs {
@@ -310,6 +312,36 @@ int rlx_mi355x_gguf_matmul_bt(const void *x_dev, int x_dtype, const rlx_qweight 
     return rlx_mi355x_gguf_matmul_bt_batch(&x_dev, x_dtype, &w, &out_dev, 1, m, workspace, workspace_bytes, stream);
 }
 
+// Column layout (channels along the last axis, 16-byte aligned rows): pass A and pass B use their own row blocking.
+struct FqColPlan {
+    bool col;
+    unsigned gx, gy_absmax, gy_apply;
+    int rpb_absmax, rpb_apply;
+};
+static FqColPlan fq_col_plan(int64_t len, int64_t chan_dim, int64_t inner) {
+    FqColPlan p{};
+    p.col = inner == 1 && chan_dim >= 4 && chan_dim % 4 == 0 && len % chan_dim == 0 && len > 0;
+    if (!p.col) return p;
+    p.gx = (unsigned)((chan_dim / 4 + 255) / 256);
+    const int64_t rows = len / chan_dim;
+    auto block = [&](int64_t groups, int64_t min_rows, unsigned *gy, int *rpb) {
+        int64_t want = std::max<int64_t>(1, groups / p.gx);
+        int64_t r = std::max<int64_t>(min_rows, (rows + want - 1) / want);
+        *rpb = (int)r;
+        *gy = (unsigned)((rows + r - 1) / r);
+    };
+    block(1024, 16, &p.gy_absmax, &p.rpb_absmax);  // read only: a thousand workgroups keep enough loads in flight
+    block(2048, 16, &p.gy_apply, &p.rpb_apply);
+    return p;
+}
+
+size_t rlx_mi355x_fake_quantize_scratch_bytes(int64_t len, int64_t chan_dim, int64_t inner) {
+    if (chan_dim < 1) chan_dim = 1;
+    if (inner < 1) inner = 1;
+    const FqColPlan p = fq_col_plan(len, chan_dim, inner);
+    return (size_t)chan_dim * 8 + (p.col ? (size_t)p.gy_absmax * chan_dim * 4 : 0);
+}
+
 int rlx_mi355x_fake_quantize(const float *x_dev, float *out_dev, int8_t *codes_dev, int64_t len, int64_t chan_dim,
                              int64_t inner, int bits, int scale_mode, float ema_decay, float *state_dev,
                              int round_mode, void *scratch_dev, void *stream) {
@@ -337,38 +369,38 @@ int rlx_mi355x_fake_quantize(const float *x_dev, float *out_dev, int8_t *codes_d
     hipStream_t s = (hipStream_t)stream;
     uint32_t *max_bits = (uint32_t *)scratch_dev;
     float *scale = (float *)scratch_dev + chan_dim;
-    const bool col = inner == 1 && chan_dim >= 4 && chan_dim % 4 == 0 && len % chan_dim == 0 &&
-                     ((uintptr_t)x_dev % 16 == 0) && ((uintptr_t)out_dev % 16 == 0) &&
-                     (!codes_dev || (uintptr_t)codes_dev % 4 == 0);
+    const FqColPlan plan = fq_col_plan(len, chan_dim, inner);
+    // the scratch is sized for the column plan whether or not the pointers allow it, so alignment only picks kernels
+    const bool col = plan.col && ((uintptr_t)x_dev % 16 == 0) && ((uintptr_t)out_dev % 16 == 0) &&
+                     ((uintptr_t)scratch_dev % 16 == 0) && (!codes_dev || (uintptr_t)codes_dev % 4 == 0);
     FqArgs a{x_dev, out_dev, codes_dev, max_bits, scale, state_dev, len, chan_dim, inner, q_max, ema_decay,
-             scale_mode, round_mode, 0};
+             scale_mode, round_mode, 0, nullptr, 0};
     void *params[] = {&a};
-    unsigned gx_col = (unsigned)((chan_dim / 4 + 255) / 256), gy_col = 1;
-    if (col) {
-        int64_t rows = len / chan_dim;
-        int64_t want = std::max<int64_t>(1, 512 / gx_col);
-        int64_t rpb = std::max<int64_t>(16, (rows + want - 1) / want);
-        a.rows_per_block = (int)rpb;
-        gy_col = (unsigned)((rows + rpb - 1) / rpb);
-    }
     if (scale_mode != RLX_SCALE_FIXED) {
-        RLX_TRY(rlx_mi355x_memset_u32(max_bits, 0, (size_t)chan_dim, stream));
         if (col) {
-            RLX_TRY(launch(K_FQ_COL_ABSMAX, gx_col, gy_col, 256, 0, s, params));
-        } else if (inner >= 256 && len % inner == 0 && len / inner <= 0x7FFFFFFF) {
-            // one workgroup per contiguous run of `inner` elements, long runs split into parts of >= 16K elements
-            unsigned bx = inner >= 4096 ? 1024 : 256;
-            unsigned parts = (unsigned)std::min<int64_t>(1024, std::max<int64_t>(1, inner / 16384));
-            a.rows_per_block = (int)((inner + parts - 1) / parts);
-            RLX_TRY(launch(K_FQ_SEG_ABSMAX, (unsigned)(len / inner), parts, bx, 0, s, params));
+            a.partial = (float *)scratch_dev + 2 * chan_dim;
+            a.parts = (int)plan.gy_absmax;
+            a.rows_per_block = plan.rpb_absmax;
+            RLX_TRY(launch(K_FQ_COL_ABSMAX, plan.gx, plan.gy_absmax, 256, 0, s, params));
         } else {
-            int64_t threads = (len + 31) / 32;
-            RLX_TRY(launch(K_FQ_FLAT_ABSMAX, (unsigned)((threads + 255) / 256), 1, 256, 0, s, params));
+            RLX_TRY(rlx_mi355x_memset_u32(max_bits, 0, (size_t)chan_dim, stream));
+            if (inner >= 256 && len % inner == 0 && len / inner <= 0x7FFFFFFF) {
+                // one workgroup per contiguous run of `inner` elements, long runs split into parts of >= 16K elements
+                unsigned bx = inner >= 4096 ? 1024 : 256;
+                unsigned parts = (unsigned)std::min<int64_t>(1024, std::max<int64_t>(1, inner / 16384));
+                a.rows_per_block = (int)((inner + parts - 1) / parts);
+                RLX_TRY(launch(K_FQ_SEG_ABSMAX, (unsigned)(len / inner), parts, bx, 0, s, params));
+            } else {
+                int64_t threads = (len + 31) / 32;
+                RLX_TRY(launch(K_FQ_FLAT_ABSMAX, (unsigned)((threads + 255) / 256), 1, 256, 0, s, params));
+            }
         }
     }
-    RLX_TRY(launch(K_FQ_SCALE, (unsigned)((chan_dim + 255) / 256), 1, 256, 0, s, params));
+    if (a.partial) RLX_TRY(launch(K_FQ_SCALE_PARTS, (unsigned)((chan_dim + 63) / 64), 1, 1024, 0, s, params));
+    else RLX_TRY(launch(K_FQ_SCALE, (unsigned)((chan_dim + 255) / 256), 1, 256, 0, s, params));
     if (col) {
-        RLX_TRY(launch(K_FQ_COL_APPLY, gx_col, gy_col, 256, 0, s, params));
+        a.rows_per_block = plan.rpb_apply;
+        RLX_TRY(launch(K_FQ_COL_APPLY, plan.gx, plan.gy_apply, 256, 0, s, params));
     } else {
         bool v4 = inner % 4 == 0 && len % 4 == 0 && ((uintptr_t)x_dev % 16 == 0) && ((uintptr_t)out_dev % 16 == 0) &&
                   (!codes_dev || (uintptr_t)codes_dev % 4 == 0);

@@ -8,7 +8,8 @@
 //
 // x / s is a true IEEE division and the multiply is never fused (-ffp-contract=off), so out and the integer
 // codes are bit-identical to the scalar reference. Three data layouts get their own indexing:
-//   col     inner == 1 and chan_dim % 4 == 0 : a thread owns 4 adjacent channels and walks down the rows
+//   col     inner == 1 and chan_dim % 4 == 0 : a thread owns 4 adjacent channels and walks down the rows; pass A
+//           writes one row of maxima per row block (no atomics) and the scale kernel folds them
 //   seg     any inner: one workgroup per contiguous (outer, channel) run of `inner` elements (pass A only)
 //   flat    element-wise with the channel computed per element (pass B, and pass A for short runs)
 #include "common.h"
@@ -26,6 +27,8 @@ struct FqArgs {
     float q_max, decay;
     int scale_mode, round_mode;
     int rows_per_block;  // col kernels: rows per workgroup; seg kernel: elements per part
+    float *partial;      // col pass A: [parts][chan_dim] maxima per row block (no atomics, nothing to clear); else null
+    int parts;
 };
 
 __device__ __forceinline__ float fq_scale_from_max(float max_abs, float q_max) {
@@ -62,10 +65,7 @@ __device__ __forceinline__ void col_absmax(const FqArgs &a) {
         m2 = a2 > m2 ? a2 : m2;
         m3 = a3 > m3 ? a3 : m3;
     }
-    atomicMax(a.max_bits + c4 + 0, __builtin_bit_cast(uint32_t, m0));
-    atomicMax(a.max_bits + c4 + 1, __builtin_bit_cast(uint32_t, m1));
-    atomicMax(a.max_bits + c4 + 2, __builtin_bit_cast(uint32_t, m2));
-    atomicMax(a.max_bits + c4 + 3, __builtin_bit_cast(uint32_t, m3));
+    *(float4_t *)(a.partial + (long long)blockIdx.y * a.chan_dim + c4) = float4_t{m0, m1, m2, m3};
 }
 
 __device__ __forceinline__ void seg_absmax(const FqArgs &a) {
@@ -119,16 +119,15 @@ __device__ __forceinline__ void flat_absmax(const FqArgs &a) {
 
 // ---- scale --------------------------------------------------------------------------------------------
 
-__device__ __forceinline__ void make_scale(const FqArgs &a) {
-    long long c = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (c >= a.chan_dim) return;
+// s[c] from the channel's max|x| (PerBatch), blended into the state (EMA) or read from it (Fixed).
+__device__ __forceinline__ void scale_from_max(const FqArgs &a, long long c, float max_abs) {
     float s;
     if (a.scale_mode == 2) {  // Fixed
         float v = a.state[c];
         s = v > 1e-12f ? v : 1e-12f;
         if (v != v) s = 1e-12f;  // f32::max(NaN, 1e-12) = 1e-12
     } else {
-        float cur = fq_scale_from_max(__builtin_bit_cast(float, a.max_bits[c]), a.q_max);
+        float cur = fq_scale_from_max(max_abs, a.q_max);
         if (a.scale_mode == 1) {  // EMA: cold start when state <= 0
             float st = a.state[c];
             if (st <= 0.0f) {
@@ -144,6 +143,39 @@ __device__ __forceinline__ void make_scale(const FqArgs &a) {
         }
     }
     a.scale[c] = s;
+}
+
+__device__ __forceinline__ void make_scale(const FqArgs &a) {
+    long long c = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= a.chan_dim) return;
+    scale_from_max(a, c, a.scale_mode == 2 ? 0.f : __builtin_bit_cast(float, a.max_bits[c]));
+}
+
+// Column layout: fold the [parts][chan_dim] maxima of pass A. One workgroup of 1024 threads per 64 channels:
+// thread (channel t % 64, group t / 64) takes every 16th row of maxima, then the 16 groups meet in LDS.
+__device__ __forceinline__ void make_scale_parts(const FqArgs &a) {
+    __shared__ float group_max[16][64];
+    const int cl = threadIdx.x & 63, grp = threadIdx.x >> 6;
+    const long long c = (long long)blockIdx.x * 64 + cl;
+    float m = 0.f;
+    if (c < a.chan_dim) {
+#pragma unroll 4
+        for (int p = grp; p < a.parts; p += 16) {
+            float v = a.partial[(long long)p * a.chan_dim + c];  // never NaN: pass A's compare drops them
+            m = v > m ? v : m;
+        }
+    }
+    group_max[grp][cl] = m;
+    __syncthreads();
+    if (grp == 0 && c < a.chan_dim) {
+#pragma unroll
+        for (int g = 1; g < 16; g++) {
+            float v = group_max[g][cl];
+            m = v > m ? v : m;
+        }
+        a.max_bits[c] = __builtin_bit_cast(uint32_t, m);
+        scale_from_max(a, c, m);
+    }
 }
 
 // ---- pass B -------------------------------------------------------------------------------------------
@@ -219,6 +251,7 @@ extern "C" __global__ __launch_bounds__(256) void rlx_fq_col_absmax(rlx::FqArgs 
 extern "C" __global__ __launch_bounds__(1024) void rlx_fq_seg_absmax(rlx::FqArgs a) { rlx::seg_absmax(a); }
 extern "C" __global__ __launch_bounds__(256) void rlx_fq_flat_absmax(rlx::FqArgs a) { rlx::flat_absmax(a); }
 extern "C" __global__ __launch_bounds__(256) void rlx_fq_scale(rlx::FqArgs a) { rlx::make_scale(a); }
+extern "C" __global__ __launch_bounds__(1024) void rlx_fq_scale_parts(rlx::FqArgs a) { rlx::make_scale_parts(a); }
 extern "C" __global__ __launch_bounds__(256) void rlx_fq_col_apply(rlx::FqArgs a) { rlx::col_apply(a); }
 extern "C" __global__ __launch_bounds__(256) void rlx_fq_flat_apply(rlx::FqArgs a) { rlx::flat_apply(a); }
 extern "C" __global__ __launch_bounds__(256) void rlx_fq_flat4_apply(rlx::FqArgs a) { rlx::flat4_apply(a); }

@@ -187,12 +187,12 @@ def fake_quantize(x, shape, axis, bits, scale_mode=ScaleMode.PerBatch, decay=0.0
     xd = DeviceBuffer.from_numpy(x)
     od = DeviceBuffer(max(x.nbytes, 4))
     cd = DeviceBuffer(max(x.size, 4))
-    scratch = DeviceBuffer(chan_dim * 8)
+    scratch = DeviceBuffer(_lib.lib().rlx_mi355x_fake_quantize_scratch_bytes(x.size, chan_dim, inner))
     sd = DeviceBuffer.from_numpy(state) if state is not None else None
     _lib.check(_lib.lib().rlx_mi355x_fake_quantize(xd.ptr, od.ptr, cd.ptr, x.size, chan_dim, inner, bits, int(scale_mode),
                                                   decay, sd.ptr if sd else None, int(round_mode), scratch.ptr, None))
     sync()
     if sd is not None and scale_mode == ScaleMode.EMA:
         state[...] = sd.to_numpy(np.float32)
-    scales = scratch.to_numpy(np.float32)[chan_dim:]
+    scales = scratch.to_numpy(np.float32)[chan_dim:2 * chan_dim]
     return od.to_numpy(np.float32, x.size).reshape(shape), cd.to_numpy(np.int8, x.size).reshape(shape), scales
