@@ -79,6 +79,11 @@ static int launch_gemv(const void *const *xs, int xk, const rlx_qweight *const *
                        hipStream_t stream) {
     const int scheme = ws[0]->scheme;
     const Layout L = layout_of(scheme);
+    for (int i = 0; i < count; i++)
+        if ((uintptr_t)xs[i] % 16 != 0) {
+            set_error("gguf_matmul_bt: activations must be 16-byte aligned");
+            return RLX_ERR_INVALID;
+        }
     const int rv = xk == 0 ? 2 * m : m;
     const int ng = (rv + 3) / 4;
     const bool r2 = rv <= 2;

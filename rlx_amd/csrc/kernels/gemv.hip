@@ -8,6 +8,8 @@
 // except the activations, and f32 activations are carried as an exact hi + lo pair of halfs in two A rows.
 //
 // Work decomposition and the LDS protocol are described above gemv_body().
+#include <type_traits>
+
 #include "common.h"
 
 namespace rlx {
@@ -166,39 +168,65 @@ __device__ __forceinline__ void compute_unit(const UnitRegs<SCHEME> &w, const ha
 }
 
 // Convert one K chunk of the activations into LDS as halfs: f32 -> hi rows [0,m) + lo rows [m,2m); 16-bit -> rows [0,m).
-__device__ __forceinline__ void stage_x(const GemvArgs &a, const GemvSeg &sg, half_t *xs, int row_stride, int k0, int kc) {
+// Each thread issues up to eight independent loads before it converts the first one, so a chunk of many rows costs
+// one memory latency per eight groups of columns, not one per group.
+template <int XD>
+__device__ __forceinline__ void stage_x_typed(const GemvArgs &a, const GemvSeg &sg, half_t *xs, int row_stride, int k0, int kc) {
+    constexpr int U = 8;
+    constexpr int G = XD == X_F32 ? 4 : 8;  // columns per 16-byte load
+    typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
     const int tid = threadIdx.x, nt = blockDim.x;
-    const int q4 = kc >> 2;  // groups of 4 columns
-    for (int idx = tid; idx < a.m * q4; idx += nt) {
-        int row = idx / q4, c = (idx - row * q4) * 4;
-        int kk = k0 + c;
-        if (a.x_dtype == X_F32) {
-            float4_t v = {0.f, 0.f, 0.f, 0.f};
-            if (kk < sg.k) v = *(const float4_t *)((const float *)sg.x + (long long)row * sg.k + kk);
-            half4_t hi, lo;
+    const int groups = kc / G;  // kc is a multiple of 64
+    const int total = a.m * groups;
+    for (int idx0 = tid; idx0 < total; idx0 += nt * U) {
+        typedef typename std::conditional<XD == X_F32, float4_t, uint4_t>::type raw_t;  // 16 bytes either way
+        raw_t raw[U];
 #pragma unroll
-            for (int e = 0; e < 4; e++) {
-                hi[e] = (half_t)v[e];
-                // residual, scaled by 2^11 so it stays in the normal binary16 range; undone in the final sum
-                lo[e] = (half_t)((v[e] - (float)hi[e]) * LO_SCALE);
-            }
-            *(half4_t *)(xs + row * row_stride + c) = hi;
-            *(half4_t *)(xs + (a.m + row) * row_stride + c) = lo;
-        } else {
-            uint2_t raw = {0, 0};
-            if (kk < sg.k) raw = *(const uint2_t *)((const uint16_t *)sg.x + (long long)row * sg.k + kk);
-            if (a.x_dtype == X_BF16) {
-                half4_t h;
+        for (int u = 0; u < U; u++) {
+            const int idx = idx0 + u * nt;
+            const int row = idx / groups, c = (idx - row * groups) * G;
+            // k is a multiple of 32: a group is inside or outside as a whole
+            const bool inside = idx < total && k0 + c < sg.k;
+            const raw_t *src = (const raw_t *)((const uint8_t *)sg.x + ((long long)row * sg.k + k0 + c) * (XD == X_F32 ? 4 : 2));
+            raw_t v = {};
+            if (inside) v = *src;
+            raw[u] = v;
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int idx = idx0 + u * nt;
+            if (idx >= total) continue;
+            const int row = idx / groups, c = (idx - row * groups) * G;
+            if constexpr (XD == X_F32) {
+                half4_t hi, lo;
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
-                    uint32_t bits = ((e & 1) ? (raw[e >> 1] >> 16) : (raw[e >> 1] & 0xFFFFu)) << 16;
+                    const float v = raw[u][e];
+                    hi[e] = (half_t)v;
+                    // residual, scaled by 2^11 so it stays in the normal binary16 range; undone in the final sum
+                    lo[e] = (half_t)((v - (float)hi[e]) * LO_SCALE);
+                }
+                *(half4_t *)(xs + row * row_stride + c) = hi;
+                *(half4_t *)(xs + (a.m + row) * row_stride + c) = lo;
+            } else if constexpr (XD == X_BF16) {
+                half8_t h;
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    const uint32_t bits = ((e & 1) ? (raw[u][e >> 1] >> 16) : (raw[u][e >> 1] & 0xFFFFu)) << 16;
                     h[e] = (half_t)__builtin_bit_cast(float, bits);
                 }
-                raw = __builtin_bit_cast(uint2_t, h);
+                *(half8_t *)(xs + row * row_stride + c) = h;
+            } else {
+                *(uint4_t *)(xs + row * row_stride + c) = raw[u];
             }
-            *(uint2_t *)(xs + row * row_stride + c) = raw;
         }
     }
+}
+
+__device__ __forceinline__ void stage_x(const GemvArgs &a, const GemvSeg &sg, half_t *xs, int row_stride, int k0, int kc) {
+    if (a.x_dtype == X_F32) stage_x_typed<X_F32>(a, sg, xs, row_stride, k0, kc);
+    else if (a.x_dtype == X_BF16) stage_x_typed<X_BF16>(a, sg, xs, row_stride, k0, kc);
+    else stage_x_typed<X_F16>(a, sg, xs, row_stride, k0, kc);
 }
 
 // One workgroup = a contiguous run of row tiles of one weight segment x all of K.
