@@ -100,45 +100,65 @@ static int launch_gemv(const void *const *xs, int xk, const rlx_qweight *const *
         max_units = std::max(max_units, (int)ws[i]->dims.units);
         work += ws[i]->dims.row_tiles * ws[i]->dims.units;
     }
-    const int nwaves = std::max(1, std::min(std::min(16, std::max(1, env_waves)), max_units));
-    // Grid: about env_wgs_per_cu workgroups per CU, every one resident at once, each with the same number of
-    // (tile, unit) items: a segment with a longer K gets fewer row tiles per workgroup.
     const int cus = std::max(1, device_props().cu_count);
-    const long long target_items = std::max<long long>(1, (work + (long long)env_wgs_per_cu * cus - 1) / ((long long)env_wgs_per_cu * cus));
     const size_t slot_bytes = (size_t)ng * 256;
-    const int tpw_cap = (int)std::max<size_t>(1, (32 * 1024) / (nwaves * slot_bytes));
-    GemvArgs a{};
-    int wg = 0, max_tpw = 1;
-    for (int i = 0; i < count; i++) {
-        const WeightDims &D = ws[i]->dims;
-        int tpw = (int)std::max<long long>(1, (target_items + D.units / 2) / D.units);
-        tpw = std::min(tpw, tpw_cap);
-        max_tpw = std::max(max_tpw, tpw);
-        a.seg[i] = GemvSeg{ws[i]->dev, xs[i], outs[i], (int)D.n, (int)D.k, (int)D.row_tiles, (int)D.units, wg, tpw};
-        wg += (int)((D.row_tiles + tpw - 1) / tpw);
-    }
-    const size_t part_bytes = (size_t)max_tpw * nwaves * slot_bytes;
-    // LDS: partial sums + the staged activation chunk (rv rows of halfs, 16 B row padding) + Q4_K block sums.
-    // 80 KB keeps two workgroups per CU (160 KB LDS) and holds a 14336-wide f32 vector (hi + lo rows) in one chunk.
-    const size_t budget = 80 * 1024;
     auto stage_bytes = [&](int kcu) {
         size_t b = ((size_t)rv * ((size_t)kcu * L.unit_k + 8) * 2 + 15) & ~(size_t)15;
         if (scheme == SCHEME_Q4K) b += (size_t)kcu * (L.unit_k / 32) * 16 * 4;
         return b;
     };
-    int kcu = max_units;
-    while (kcu > 1 && part_bytes + stage_bytes(kcu) > budget) kcu--;
-    if (part_bytes + stage_bytes(kcu) > budget) {
+    // A launch shape: `wgs_per_cu` workgroups of `waves` waves per CU, every one resident at once, each with the same
+    // number of (tile, unit) items (a segment with a longer K gets fewer row tiles per workgroup), LDS split between
+    // the per-(tile, wave) partial sums and the staged activation chunk (rv rows of halfs, 16 B row padding, plus the
+    // Q4_K block sums).
+    struct Shape {
+        GemvArgs a;
+        int nwaves, wg, kcu;
+        size_t lds;
+        bool fits;
+    };
+    auto shape = [&](int waves, int wgs_per_cu, size_t budget) {
+        Shape sh{};
+        sh.nwaves = std::max(1, std::min(std::min(16, std::max(1, waves)), max_units));
+        const long long slots = (long long)std::max(1, wgs_per_cu) * cus;
+        const long long target_items = std::max<long long>(1, (work + slots - 1) / slots);
+        const int tpw_cap = (int)std::max<size_t>(1, (budget * 2 / 5) / (sh.nwaves * slot_bytes));
+        int max_tpw = 1;
+        for (int i = 0; i < count; i++) {
+            const WeightDims &D = ws[i]->dims;
+            int tpw = (int)std::max<long long>(1, (target_items + D.units / 2) / D.units);
+            tpw = std::min(tpw, tpw_cap);
+            max_tpw = std::max(max_tpw, tpw);
+            sh.a.seg[i] = GemvSeg{ws[i]->dev, xs[i], outs[i], (int)D.n, (int)D.k, (int)D.row_tiles, (int)D.units, sh.wg, tpw};
+            sh.wg += (int)((D.row_tiles + tpw - 1) / tpw);
+        }
+        const size_t part_bytes = (size_t)max_tpw * sh.nwaves * slot_bytes;
+        sh.kcu = max_units;
+        while (sh.kcu > 1 && part_bytes + stage_bytes(sh.kcu) > budget) sh.kcu--;
+        sh.fits = part_bytes + stage_bytes(sh.kcu) <= budget;
+        sh.lds = part_bytes + stage_bytes(sh.kcu);
+        sh.a.nseg = count;
+        sh.a.m = m;
+        sh.a.kc_units = sh.kcu;
+        sh.a.x_dtype = xk;
+        sh.a.max_tiles_per_wg = max_tpw;
+        return sh;
+    };
+    // Two workgroups of 8 waves per CU with 80 KB each: holds a 14336-wide f32 vector (hi + lo rows) in one chunk.
+    Shape sh = shape(env_waves, env_wgs_per_cu, (size_t)(env_wgs_per_cu <= 1 ? 156 : 80) * 1024);
+    // With four or more activation rows every workgroup restages all of x, and that traffic (workgroups x rows x K)
+    // rivals the weights: one workgroup of 16 waves per CU with the whole LDS halves it, provided a single round of
+    // workgroups still covers the matrix.
+    if (rv >= 4 && !getenv("RLX_GEMV_WGS_PER_CU")) {
+        Shape fat = shape(16, 1, (size_t)156 * 1024);
+        if (fat.fits && fat.wg <= cus) sh = fat;
+    }
+    if (!sh.fits) {
         set_error("gemv: one K unit of %d activation rows does not fit LDS", rv);
         return RLX_ERR_INVALID;
     }
-    a.nseg = count;
-    a.m = m;
-    a.kc_units = kcu;
-    a.x_dtype = xk;
-    a.max_tiles_per_wg = max_tpw;
-    void *params[] = {&a};
-    return launch(id, (unsigned)wg, 1, (unsigned)nwaves * 64, (unsigned)(part_bytes + stage_bytes(kcu)), stream, params);
+    void *params[] = {&sh.a};
+    return launch(id, (unsigned)sh.wg, 1, (unsigned)sh.nwaves * 64, (unsigned)sh.lds, stream, params);
 }
 
 struct GemmPlan {
