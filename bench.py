@@ -206,6 +206,8 @@ def main():
 
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(base, xs)
+        if args.extra:
+            result["extra"]["cpu_baselines"] = cpu_baselines_extra()
     print(json.dumps(result), flush=True)
 
 
@@ -404,6 +406,35 @@ def cpu_baseline(base, xs):
             "sample": f"{reps} pass(es) over the same seven Q4_0 projections of one layer, {spent:.1f} s, "
                       f"C restatement of rlx-cpu gguf_matmul_bt (scalar, single thread, as the reference runs it)",
             "host_cpus": os.cpu_count()}
+
+
+def cpu_baselines_extra():
+    """The reference CPU path (oracle restatement, scalar, one thread) on bounded samples of the other configs."""
+    import oracle
+    from rlx_amd import QuantScheme, ops
+
+    out = {}
+    # FakeQuantize [8192, 4096] per column, in full (two scalar passes over 33.5 M elements)
+    rows, cols = 8192, 4096
+    x = ops.philox_normal(9, rows * cols)
+    t0 = time.time()
+    oracle.fake_quantize(x, (rows, cols), 1, 8)
+    dt = time.time() - t0
+    out["fake_quantize_8192x4096_cols"] = {"s": round(dt, 3), "GB/s_1R1W": round(2 * rows * cols * 4 / dt / 1e9, 3), "cores": 1,
+                                           "kind": "port", "sample": "the whole tensor, one call"}
+    # Q4_K GEMM M = 512, 4096 -> 14336: a 1024-column slice of N, scaled (the loop is linear in N)
+    n, k, m, ncols = 14336, 4096, 512, 1024
+    w = (ops.philox_normal(41, ncols * k) * np.float32(0.02)).astype(np.float32)
+    packed = ops.quantize(QuantScheme.GgufQ4K, w)
+    xa = oracle.bf16_round(ops.philox_normal(31, m * k))
+    t0 = time.time()
+    oracle.gguf_matmul_bt(xa, packed, m, k, ncols, oracle.Q4K)
+    dt = time.time() - t0
+    tf = 2.0 * m * ncols * k / dt / 1e12
+    out["q4_k_gemm_m512_gate_up_4096x14336"] = {"TFLOP/s": round(tf, 6), "s_full_size_extrapolated": round(dt * n / ncols, 1),
+                                                "cores": 1, "kind": "port",
+                                                "sample": f"{ncols} of {n} output columns, {dt:.1f} s, scaled by {n // ncols}"}
+    return out
 
 
 if __name__ == "__main__":
