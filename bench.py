@@ -2,7 +2,7 @@
 """Headline benchmark: Q4_0 decode GEMV (batch 1) over the seven Llama-3-8B layer projections on one MI355X.
 
 A step is one pass over one layer's seven projections (q, k, v, o, gate, up, down): seven DequantMatMul nodes of one
-compiled graph, each with its own f32 activation vector as BASELINE's config states, which the backend issues as one
+compiled graph, each with its own f32 activation vector as the benchmark definition states, which the backend issues as one
 batched launch replayed as a hipGraph (`--wiring layer` orders them like a transformer layer instead: four dependent
 launches). The layers rotate through LAYERS distinct weight sets (~123 MB each), far
 more than the 256 MB of last-level cache, so every launch streams its weights from HBM. Inputs and weights are
@@ -29,13 +29,13 @@ CALIBRATION_COPY_BYTES = 256 << 20
 # each scaled by the same counter's reading for the copy kernel above); profiles/gemv_q4_0_llama8b_layer_traffic.txt.
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 124314627
 
-# (name, N, K) — BASELINE config 2
+# (name, N, K) — the Llama-3-8B layer projections of the headline workload
 LLAMA8B = [("q", 4096, 4096), ("k", 1024, 4096), ("v", 1024, 4096), ("o", 4096, 4096),
            ("gate", 14336, 4096), ("up", 14336, 4096), ("down", 4096, 14336)]
 
 
 # Which activations each projection reads ("@p" = the output of projection p). "independent" is the workload as
-# BASELINE states it: seven GEMVs, each with its own seeded f32 activation vector; nothing orders them, so the backend
+# the benchmark definition states it: seven GEMVs, each with its own seeded f32 activation vector; nothing orders them, so the backend
 # issues all seven as one batched launch. "layer" chains them the way a transformer layer's data flow does
 # (x -> q,k,v; q -> o; o -> gate,up; gate -> down; the attention / activation math in between is not part of this
 # path), which forces four dependent launches; it is reported under "extra" for comparison.
@@ -118,7 +118,7 @@ def main():
                          "cost more per launch than a plain launch on this runtime)")
     ap.add_argument("--calibration-copies", type=int, default=3,
                     help="untimed launches of the 256 MiB copy kernel before the run (counter calibration)")
-    ap.add_argument("--extra", action="store_true", help="also time the other BASELINE configs (reported under 'extra')")
+    ap.add_argument("--extra", action="store_true", help="also time the other benchmark configurations (reported under 'extra')")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1", file=sys.stderr)
@@ -225,7 +225,7 @@ def time_launches(ops, stream, fn, reps, warm):
 
 
 def extra_configs(rlx_amd, stream):
-    """Other BASELINE configs, each as back-to-back launches on rotating buffers (reported, not the headline)."""
+    """Other benchmark configurations, each as back-to-back launches on rotating buffers (reported, not the headline)."""
     from rlx_amd import DType, QuantScheme, ops
     L = rlx_amd._lib.lib()
     out = {}

@@ -136,7 +136,7 @@ def check_matmul(oracle, scheme, n, k, m, x_dtype=DType.F32, std=0.02, seed=0, c
 
 
 def test_config1_q8_0_gemv_4096(oracle):
-    # BASELINE config 1: W 4096x4096 ~N(0,0.02) Q8_0, x [1,4096] f32 ~N(0,1)
+    # benchmark configuration 1: W 4096x4096 ~N(0,0.02) Q8_0, x [1,4096] f32 ~N(0,1)
     got, x, packed, err = check_matmul(oracle, Q8_0, 4096, 4096, 1)
     cpu = oracle.gguf_matmul_bt(x, packed, 1, 4096, 4096, Q8_0)     # the reference CPU path, f32
     ref64 = oracle.gguf_matmul_f64(x, packed, 1, 4096, 4096, Q8_0)
@@ -201,7 +201,7 @@ def test_matmul_is_deterministic(oracle):
 
 
 def test_matmul_linearity_full_size(oracle):
-    # size-independent property at a BASELINE shape: W(x1 + 2 x2) = W x1 + 2 W x2 up to f32 rounding
+    # size-independent property at a benchmark shape: W(x1 + 2 x2) = W x1 + 2 W x2 up to f32 rounding
     n, k = 14336, 4096
     packed, _ = make_weights(Q4_0, n, k, seed=11)
     w = ops.QWeight(Q4_0, packed, n, k)
@@ -250,7 +250,7 @@ def heavy_tailed(rows, cols, seed):
 
 
 def test_config4_fq_columns_full_size(oracle):
-    # BASELINE config 4: [8192, 4096] f32, N(0,1) with 0.1% of entries x20; int8 per channel along the last axis
+    # benchmark configuration 4: [8192, 4096] f32, N(0,1) with 0.1% of entries x20; int8 per channel along the last axis
     x = heavy_tailed(8192, 4096, 21)
     for mode in (RoundMode.HalfAway, RoundMode.HalfEven):
         got, codes = check_fq(oracle, x, x.shape, 1, 8, round_mode=mode)
@@ -395,7 +395,7 @@ def test_gemm_small(oracle, scheme, m, n, k, x_dtype):
 
 
 def test_config3_q4k_gemm_m512_slices(oracle):
-    # BASELINE config 3 shapes at full size; the f64 oracle is run on column windows (it is O(m n k) scalar work)
+    # benchmark configuration 3 shapes at full size; the f64 oracle is run on column windows (it is O(m n k) scalar work)
     for n, k in [(14336, 4096), (4096, 14336)]:
         packed, _ = make_weights(Q4K, n, k, seed=n % 89)
         x = oracle.bf16_round(np.random.default_rng(n).standard_normal((512, k)).astype(np.float32))
@@ -413,7 +413,7 @@ def test_config3_q4k_gemm_m512_slices(oracle):
 
 
 def test_gemm_q4_0_70b_shape_bf16(oracle):
-    # BASELINE config 5, one projection at M = 64 and 256
+    # benchmark configuration 5, one projection at M = 64 and 256
     n, k = 1024, 8192
     packed, _ = make_weights(Q4_0, n, k, std=0.015, seed=77)
     w = ops.QWeight(Q4_0, packed, n, k)
