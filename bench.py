@@ -195,8 +195,20 @@ def main():
     }
 
     if args.extra:
+        # the same layer through the host-buffer boundary (ExecutableGraph::run: seven H2D copies, the launch, seven
+        # D2H copies, synchronous) - PCIe and call overhead included, reported beside the headline, never as `value`
+        ins = [(src, v) for src, v in {WIRING[args.wiring][n]: xs[n] for n, _, _ in LLAMA8B if xs[n] is not None}.items()]
+        for _ in range(3):
+            layers[0].run(ins)
+        t1 = time.time()
+        for i in range(50):
+            layers[i % len(layers)].run(ins)
+        host_ms = (time.time() - t1) / 50 * 1e3
         del layers
         result["extra"] = extra_configs(rlx_amd, stream)
+        result["extra"]["q4_0_gemv_llama8b_layer_host_boundary"] = {
+            "ms_per_call": round(host_ms, 4), "GB/s": round(layer_bytes / host_ms / 1e6, 1),
+            "note": "rlx_exec_run with host inputs and outputs (H2D + launch + D2H, synchronous)"}
         other = "layer" if args.wiring == "independent" else "independent"
         ms_o, lay_o, _ = time_layers(rlx_amd, ops, stream, base, other, args.layers, args.steps, args.warmup, args.graph)
         result["extra"][f"q4_0_gemv_llama8b_{other}_wiring"] = {
@@ -249,6 +261,11 @@ def extra_configs(rlx_amd, stream):
         b = gemv_bytes(n, k)
         out[f"q4_0_gemv_{name}"] = {"us": round(ms * 1e3, 3), "GB/s": round(b / ms / 1e6, 1),
                                     "frac_hbm": round(b / ms / 1e6 / HBM_PEAK_GBS, 4), "copies": copies}
+        if name == "k/v":  # the same projection when its 2.4 MB of weights stay cache-resident (one copy, back to back)
+            def fn_warm():
+                rlx_amd._lib.check(L.rlx_mi355x_gguf_matmul_bt(x.ptr, int(DType.F32), qws[0].ptr, y.ptr, 1, None, 0, stream))
+            msw = time_launches(ops, stream, fn_warm, 400, 50)
+            out["q4_0_gemv_k/v_warm"] = {"us": round(msw * 1e3, 3), "GB/s": round(b / msw / 1e6, 1)}
         for q in qws:
             q.free()
     # config 1: Q8_0 GEMV 4096x4096
