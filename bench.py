@@ -316,8 +316,37 @@ def extra_configs(rlx_amd, stream):
     for xd, od in sets:
         xd.free()
         od.free()
+    out.update(moe_config(rlx_amd, stream))
     out.update(gemm_configs(rlx_amd, stream))
     return out
+
+
+def moe_config(rlx_amd, stream):
+    """Mixture-of-experts decode (DequantGroupedMatMul): 8 experts of a 4096 -> 14336 Q4_0 projection, two routed rows per
+    call (top-2 of one token), the expert pair rotating so no slab is cache-resident when it is read."""
+    from rlx_amd import DType, QuantScheme, ops
+    L = rlx_amd._lib.lib()
+    n, k, experts = 14336, 4096, 8
+    w = (ops.philox_normal(61, 2048 * k) * np.float32(0.02)).astype(np.float32)
+    slab = ops.quantize(QuantScheme.GgufQ4_0, w).reshape(2048, -1)
+    one = np.concatenate([np.roll(slab, 17 * r, axis=0) for r in range(n // 2048)], axis=0)
+    packed = np.concatenate([np.roll(one, 5 * e, axis=0).reshape(-1) for e in range(experts)])
+    qw = ops.QWeight(QuantScheme.GgufQ4_0, packed, n, k, num_experts=experts)
+    x = ops.DeviceBuffer.from_numpy(np.tile(ops.philox_normal(62, k), 2))
+    y = ops.DeviceBuffer(2 * n * 4)
+    idxs = [ops.DeviceBuffer.from_numpy(np.array([2 * p, 2 * p + 1], np.float32)) for p in range(experts // 2)]
+    state = {"i": 0}
+
+    def fn():
+        idx = idxs[state["i"] % len(idxs)]
+        state["i"] += 1
+        rlx_amd._lib.check(L.rlx_mi355x_gguf_grouped_matmul_bt(x.ptr, int(DType.F32), qw.ptr, idx.ptr, y.ptr, 2, stream))
+
+    ms = time_launches(ops, stream, fn, 400, 40)
+    b = 2 * gemv_bytes(n, k)
+    qw.free()
+    return {"q4_0_moe_grouped_top2_of_8x14336x4096": {"us": round(ms * 1e3, 3), "GB/s": round(b / ms / 1e6, 1),
+                                                     "frac_hbm": round(b / ms / 1e6 / HBM_PEAK_GBS, 4)}}
 
 
 def f32_to_bf16_bits(x):

@@ -13,9 +13,10 @@ pub const RLX_OP_INPUT: u32 = 0;
 pub const RLX_OP_PARAM: u32 = 1;
 pub const RLX_OP_DEQUANT_MATMUL: u32 = 2;
 pub const RLX_OP_FAKE_QUANTIZE: u32 = 3;
+pub const RLX_OP_DEQUANT_GROUPED_MATMUL: u32 = 4;
 
 pub const RLX_MAX_RANK: usize = 6;
-pub const RLX_MAX_INPUTS: usize = 2;
+pub const RLX_MAX_INPUTS: usize = 3;
 
 #[repr(C)]
 #[derive(Clone, Copy)]

@@ -90,6 +90,10 @@ fn describe(node: &Node, name: &CString) -> ffi::rlx_node_desc {
             d.op_kind = ffi::RLX_OP_DEQUANT_MATMUL;
             d.scheme = *scheme as u32; // declaration order of QuantScheme (rlx-ir/src/quant.rs:39-79)
         }
+        Op::DequantGroupedMatMul { scheme } => {
+            d.op_kind = ffi::RLX_OP_DEQUANT_GROUPED_MATMUL; // inputs [x, packed expert stack, expert_idx]
+            d.scheme = *scheme as u32;
+        }
         Op::FakeQuantize { bits, axis, ste, scale_mode } => {
             d.op_kind = ffi::RLX_OP_FAKE_QUANTIZE;
             d.bits = *bits as u32;
@@ -136,7 +140,7 @@ impl Backend for Mi355xBackend {
     }
 
     fn supported_ops(&self) -> &'static [OpKind] {
-        &[OpKind::Input, OpKind::Param, OpKind::DequantMatMul, OpKind::FakeQuantize]
+        &[OpKind::Input, OpKind::Param, OpKind::DequantMatMul, OpKind::DequantGroupedMatMul, OpKind::FakeQuantize]
     }
 }
 

@@ -139,6 +139,18 @@ size_t rlx_mi355x_gguf_matmul_workspace(int scheme, int x_dtype, int64_t m, int6
  * outs_dev[i][m, n_i] = xs_dev[i][m, k_i] . W_i^T. No counterpart in the reference, which runs one thunk per node;
  * the graph level uses it to issue together every DequantMatMul whose inputs are ready at the same point of the
  * schedule (q/k/v and gate/up of a layer share their activations; independent projections need not). */
+/* A stack of `num_experts` [n, k] matrices, expert outermost, each slab in the GGUF layout of a standalone matrix
+ * (rlx-cpu/src/gguf_matmul.rs:98-100); every slab is repacked like a plain weight. */
+int rlx_mi355x_qweight_create_experts(int scheme, const void *gguf_bytes, size_t nbytes, int64_t n, int64_t k,
+                                      int64_t num_experts, rlx_qweight **out);
+int rlx_mi355x_qweight_create_experts_at(int scheme, const void *gguf_bytes, size_t nbytes, int64_t n, int64_t k,
+                                         int64_t num_experts, void *device_mem, rlx_qweight **out);
+/* rlx_cpu::gguf_matmul::gguf_grouped_matmul_bt (rlx-cpu/src/gguf_matmul.rs:101-139): out[i, :] = x[i, :] . W_e^T with
+ * e = (int)expert_idx_dev[i]. The reference sorts rows by expert and runs one matmul per expert; every output row
+ * depends on its own input row and slab only, so here each row is one segment of the decode kernel (eight rows per
+ * launch). An index outside [0, num_experts) is clamped to the stack (the reference debug-asserts). */
+int rlx_mi355x_gguf_grouped_matmul_bt(const void *x_dev, int x_dtype, const rlx_qweight *w, const float *expert_idx_dev,
+                                      float *out_dev, int64_t m, void *stream);
 int rlx_mi355x_gguf_matmul_bt_batch(const void *const *xs_dev, int x_dtype, const rlx_qweight *const *ws,
                                     float *const *outs_dev, int count, int64_t m, void *workspace, size_t workspace_bytes,
                                     void *stream);
@@ -179,11 +191,13 @@ typedef enum rlx_op_kind {
     RLX_OP_INPUT = 0,          /* OpKind::Input  */
     RLX_OP_PARAM = 1,          /* OpKind::Param  */
     RLX_OP_DEQUANT_MATMUL = 2, /* OpKind::DequantMatMul, Op::DequantMatMul{scheme} (rlx-ir/src/op.rs:736-752) */
-    RLX_OP_FAKE_QUANTIZE = 3   /* OpKind::FakeQuantize,  Op::FakeQuantize{bits,axis,ste,scale_mode} (op.rs:407-432) */
+    RLX_OP_FAKE_QUANTIZE = 3,  /* OpKind::FakeQuantize,  Op::FakeQuantize{bits,axis,ste,scale_mode} (op.rs:407-432) */
+    RLX_OP_DEQUANT_GROUPED_MATMUL = 4 /* OpKind::DequantGroupedMatMul, Op::DequantGroupedMatMul{scheme} (op.rs:862-871):
+                                       * inputs [x [m,k], packed expert stack, expert_idx [m] F32] -> [m,n] */
 } rlx_op_kind;
 
 #define RLX_MAX_RANK 6
-#define RLX_MAX_INPUTS 2
+#define RLX_MAX_INPUTS 3
 
 /* One rlx_ir::Node{id, op, inputs, shape, name} (rlx-ir/src/graph.rs:40-81); id = index in the array. */
 typedef struct rlx_node_desc {

@@ -49,6 +49,8 @@ def lib():
         L.orc_get_scale_min_k4.argtypes = [C.c_int, u8p, u8p, u8p]
         L.orc_dequant.restype = C.c_int
         L.orc_dequant.argtypes = [C.c_int, u8p, C.c_int64, C.c_int64, f32p]
+        L.orc_gguf_grouped_matmul_bt.restype = C.c_int
+        L.orc_gguf_grouped_matmul_bt.argtypes = [f32p, u8p, C.c_int64, f32p, f32p, C.c_int64, C.c_int64, C.c_int64, C.c_int64, C.c_int]
         L.orc_gguf_matmul_bt.restype = C.c_int
         L.orc_gguf_matmul_bt.argtypes = [f32p, u8p, C.c_int64, f32p, C.c_int64, C.c_int64, C.c_int64, C.c_int]
         L.orc_gguf_matmul_f64.restype = C.c_int
@@ -130,6 +132,32 @@ def gguf_matmul_bt(x, packed, m, k, n, scheme):
     if rc != 0:
         raise ValueError("gguf_matmul_bt: bad sizes")
     return out.reshape(m, n)
+
+
+def gguf_grouped_matmul_bt(x, packed, expert_idx, m, k, n, num_experts, scheme):
+    """The reference MoE path (rlx-cpu/src/gguf_matmul.rs:101-139): row i is multiplied by expert expert_idx[i]'s slab."""
+    x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1)
+    packed = np.ascontiguousarray(packed, dtype=np.uint8)
+    idx = np.ascontiguousarray(expert_idx, dtype=np.float32)
+    assert x.size == m * k and idx.size == m
+    out = np.empty(m * n, dtype=np.float32)
+    rc = lib().orc_gguf_grouped_matmul_bt(_p(x, C.c_float), _p(packed, C.c_uint8), packed.size, _p(idx, C.c_float),
+                                          _p(out, C.c_float), m, k, n, num_experts, scheme)
+    if rc != 0:
+        raise ValueError("gguf_grouped_matmul_bt: bad sizes" if rc == -1 else "gguf_grouped_matmul_bt: expert index out of range")
+    return out.reshape(m, n)
+
+
+def gguf_grouped_matmul_f64(x, packed, expert_idx, m, k, n, num_experts, scheme):
+    """f64-accumulated yardstick of the grouped matmul: one independent matmul per row."""
+    x = np.ascontiguousarray(x, dtype=np.float32).reshape(m, k)
+    packed = np.ascontiguousarray(packed, dtype=np.uint8)
+    slab = packed.size // num_experts
+    out = np.empty((m, n), dtype=np.float64)
+    for i in range(m):
+        e = int(expert_idx[i])
+        out[i] = gguf_matmul_f64(x[i], packed[e * slab:(e + 1) * slab], 1, k, n, scheme)[0]
+    return out
 
 
 def gguf_matmul_f64(x, packed, m, k, n, scheme, n0=0, n1=None):

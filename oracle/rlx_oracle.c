@@ -280,6 +280,53 @@ int orc_gguf_matmul_bt(const float *x, const uint8_t *w_bytes, int64_t w_nbytes,
     return 0;
 }
 
+/* rlx-cpu/src/gguf_matmul.rs:101-139 with grouped_moe_sort_plan (:178-206) and grouped_moe_unpermute_out (:208-219):
+ * rows are gathered per expert (stable order), each expert's slab multiplies its rows with orc_gguf_matmul_bt, and
+ * the packed result is scattered back. expert_idx holds float-encoded indices; an index outside [0, num_experts)
+ * returns -2 (the reference debug-asserts and then slices out of range). */
+int orc_gguf_grouped_matmul_bt(const float *x, const uint8_t *w_bytes, int64_t w_nbytes, const float *expert_idx, float *out,
+                               int64_t m, int64_t k, int64_t n, int64_t num_experts, int scheme) {
+    int be = orc_block_elems(scheme), bb = orc_block_bytes(scheme);
+    if (be == 0 || (k * n) % be != 0 || num_experts <= 0) return -1;
+    int64_t slab_bytes = (k * n) / be * bb;
+    if (w_nbytes != num_experts * slab_bytes) return -1;
+    int64_t *counts = (int64_t *)calloc((size_t)num_experts, sizeof(int64_t));
+    int64_t *offsets = (int64_t *)calloc((size_t)num_experts + 1, sizeof(int64_t));
+    int64_t *write_idx = (int64_t *)calloc((size_t)num_experts, sizeof(int64_t));
+    int64_t *original_pos = (int64_t *)calloc((size_t)(m > 0 ? m : 1), sizeof(int64_t));
+    float *packed_in = (float *)malloc(sizeof(float) * (size_t)(m * k > 0 ? m * k : 1));
+    float *packed_out = (float *)calloc((size_t)(m * n > 0 ? m * n : 1), sizeof(float));
+    int rc = 0;
+    for (int64_t i = 0; i < m; i++) {
+        int64_t e = (int64_t)expert_idx[i];
+        if (expert_idx[i] < 0.0f || e >= num_experts) { rc = -2; goto done; }
+        counts[e] += 1;
+    }
+    for (int64_t e = 0; e < num_experts; e++) offsets[e + 1] = offsets[e] + counts[e];
+    for (int64_t i = 0; i < m; i++) {
+        int64_t e = (int64_t)expert_idx[i];
+        int64_t dst_row = offsets[e] + write_idx[e];
+        memcpy(packed_in + dst_row * k, x + i * k, sizeof(float) * (size_t)k);
+        original_pos[dst_row] = i;
+        write_idx[e] += 1;
+    }
+    for (int64_t e = 0; e < num_experts; e++) {
+        int64_t count = offsets[e + 1] - offsets[e];
+        if (count == 0) continue;
+        int64_t in_start = offsets[e];
+        rc = orc_gguf_matmul_bt(packed_in + in_start * k, w_bytes + e * slab_bytes, slab_bytes, packed_out + in_start * n, count, k,
+                                n, scheme);
+        if (rc != 0) goto done;
+    }
+    for (int64_t pi = 0; pi < m; pi++) {
+        int64_t i = original_pos[pi];
+        memcpy(out + i * n, packed_out + pi * n, sizeof(float) * (size_t)n);
+    }
+done:
+    free(counts); free(offsets); free(write_idx); free(original_pos); free(packed_in); free(packed_out);
+    return rc;
+}
+
 /* Error yardstick: same decoded weights, products and sums in f64. Rows [n0, n1) only. */
 int orc_gguf_matmul_f64(const float *x, const uint8_t *w_bytes, int64_t w_nbytes, double *out, int64_t m, int64_t k,
                         int64_t n, int scheme, int64_t n0, int64_t n1) {

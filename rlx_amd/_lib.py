@@ -8,7 +8,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 SO_PATH = os.path.join(_HERE, "librlx_mi355x.so")
 
 RLX_MAX_RANK = 6
-RLX_MAX_INPUTS = 2
+RLX_MAX_INPUTS = 3
 
 
 class RlxError(RuntimeError):
@@ -78,6 +78,9 @@ SIGNATURES = {
     "rlx_mi355x_gguf_matmul_bt": (_i, [_vp, _i, _vp, _vp, _i64, _vp, _sz, _vp]),
     "rlx_mi355x_gguf_matmul_workspace": (_sz, [_i, _i, _i64, _i64, _i64]),
     "rlx_mi355x_gguf_matmul_bt_batch": (_i, [_pvp, _i, _pvp, _pvp, _i, _i64, _vp, _sz, _vp]),
+    "rlx_mi355x_qweight_create_experts": (_i, [_i, _vp, _sz, _i64, _i64, _i64, _pvp]),
+    "rlx_mi355x_qweight_create_experts_at": (_i, [_i, _vp, _sz, _i64, _i64, _i64, _vp, _pvp]),
+    "rlx_mi355x_gguf_grouped_matmul_bt": (_i, [_vp, _i, _vp, _vp, _vp, _i64, _vp]),
     "rlx_mi355x_fake_quantize_scratch_bytes": (_sz, [_i64, _i64, _i64]),
     "rlx_mi355x_fake_quantize": (_i, [_vp, _vp, _vp, _i64, _i64, _i64, _i, _i, _f, _vp, _i, _vp, _vp]),
     "rlx_mi355x_quantize": (_i, [_i, _vp, _i64, _vp]),

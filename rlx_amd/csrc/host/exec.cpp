@@ -21,6 +21,8 @@ extern "C" int rlx_mi355x_fake_quantize(const float *, float *, int8_t *, int64_
                                         void *, void *);
 extern "C" int rlx_mi355x_qweight_create_at(int, const void *, size_t, int64_t, int64_t, void *, rlx_qweight **);
 extern "C" void rlx_mi355x_qweight_destroy(rlx_qweight *);
+extern "C" int rlx_mi355x_qweight_create_experts_at(int, const void *, size_t, int64_t, int64_t, int64_t, void *, rlx_qweight **);
+extern "C" int rlx_mi355x_gguf_grouped_matmul_bt(const void *, int, const rlx_qweight *, const float *, float *, int64_t, void *);
 extern "C" int rlx_mi355x_gguf_matmul_bt_batch(const void *const *, int, const rlx_qweight *const *, float *const *, int, int64_t,
                                                void *, size_t, void *);
 
@@ -28,12 +30,14 @@ namespace {
 
 using namespace rlx;
 
-const uint32_t kSupportedOps[] = {RLX_OP_INPUT, RLX_OP_PARAM, RLX_OP_DEQUANT_MATMUL, RLX_OP_FAKE_QUANTIZE};
+const uint32_t kSupportedOps[] = {RLX_OP_INPUT, RLX_OP_PARAM, RLX_OP_DEQUANT_MATMUL, RLX_OP_FAKE_QUANTIZE,
+                                 RLX_OP_DEQUANT_GROUPED_MATMUL};
 const char *op_name(uint32_t k) {
     switch (k) {
     case RLX_OP_INPUT: return "Input";
     case RLX_OP_PARAM: return "Param";
     case RLX_OP_DEQUANT_MATMUL: return "DequantMatMul";
+    case RLX_OP_DEQUANT_GROUPED_MATMUL: return "DequantGroupedMatMul";
     case RLX_OP_FAKE_QUANTIZE: return "FakeQuantize";
     default: return "?";
     }
@@ -68,7 +72,7 @@ struct Node {
     // packed weight param
     bool is_packed = false;
     int scheme = 0;
-    int64_t w_n = 0, w_k = 0;
+    int64_t w_n = 0, w_k = 0, w_experts = 1;
     rlx_qweight *qw = nullptr;
 };
 
@@ -159,7 +163,7 @@ rlx_exec *rlx_mi355x_compile(const rlx_graph_desc *g, const rlx_compile_opts *op
     int n_bad = 0;
     for (uint32_t i = 0; i < g->n_nodes; i++) {
         uint32_t k = g->nodes[i].op_kind;
-        if (k > RLX_OP_FAKE_QUANTIZE) {
+        if (k > RLX_OP_DEQUANT_GROUPED_MATMUL) {
             n_bad++;
             bad += "\n  - node " + std::to_string(i) + ": op kind " + std::to_string(k);
         }
@@ -265,6 +269,51 @@ rlx_exec *rlx_mi355x_compile(const rlx_graph_desc *g, const rlx_compile_opts *op
             w.w_k = nd.k;
             break;
         }
+        case RLX_OP_DEQUANT_GROUPED_MATMUL: {  // [x [m,k], packed expert stack, expert_idx [m]] -> [m, n]
+            Layout L = layout_of((int)nd.d.scheme);
+            if (L.unit_k == 0) {
+                set_error("compile: node %u: DequantGroupedMatMul scheme %u is not claimed (GGUF Q4_K=5, Q4_0=11, Q8_0=12)", i,
+                          nd.d.scheme);
+                return nullptr;
+            }
+            if (nd.d.n_inputs != 3 || nd.d.rank == 0 || nd.d.dtype != RLX_F32) {
+                set_error("compile: node %u: DequantGroupedMatMul takes [x, packed_experts, expert_idx] and yields an F32 tensor", i);
+                return nullptr;
+            }
+            Node &x = e->nodes[nd.d.inputs[0]];
+            Node &w = e->nodes[nd.d.inputs[1]];
+            Node &idx = e->nodes[nd.d.inputs[2]];
+            nd.n = nd.d.dims[nd.d.rank - 1];
+            nd.m = nd.numel / std::max<int64_t>(nd.n, 1);
+            nd.k = x.numel / std::max<int64_t>(nd.m, 1);
+            if (nd.n <= 0 || nd.m <= 0 || nd.k <= 0 || nd.m * nd.k != x.numel || idx.numel != nd.m || idx.d.dtype != RLX_F32) {
+                set_error("compile: node %u: need x [m,k], expert_idx [m] F32 and out [m,n]; got x numel %lld, idx numel %lld, out numel %lld",
+                          i, (long long)x.numel, (long long)idx.numel, (long long)nd.numel);
+                return nullptr;
+            }
+            const int64_t slab = (nd.k * nd.n) % L.block_elems == 0 && nd.k % L.block_elems == 0
+                                     ? nd.k * nd.n / L.block_elems * L.block_bytes : -1;
+            if (w.d.op_kind != RLX_OP_PARAM || (w.d.dtype != RLX_U8 && w.d.dtype != RLX_I8) || slab <= 0 || w.numel < slab ||
+                w.numel % slab != 0) {
+                set_error("compile: node %u: packed experts must be a U8 param of E x %lld bytes ([n=%lld, k=%lld] per expert); got %lld",
+                          i, (long long)slab, (long long)nd.n, (long long)nd.k, (long long)w.numel);
+                return nullptr;
+            }
+            if (w.is_packed && (w.scheme != (int)nd.d.scheme || w.w_n != nd.n || w.w_k != nd.k)) {
+                set_error("compile: packed param '%s' is used with two different (scheme, n, k)", w.name.c_str());
+                return nullptr;
+            }
+            if (x.d.dtype != RLX_F32 && x.d.dtype != RLX_F16 && x.d.dtype != RLX_BF16) {
+                set_error("compile: node %u: activation dtype %u unsupported", i, x.d.dtype);
+                return nullptr;
+            }
+            w.is_packed = true;
+            w.scheme = (int)nd.d.scheme;
+            w.w_n = nd.n;
+            w.w_k = nd.k;
+            w.w_experts = w.numel / slab;
+            break;
+        }
         case RLX_OP_FAKE_QUANTIZE: {
             if (nd.d.bits != 8 && nd.d.bits != 4 && nd.d.bits != 2) {
                 set_error("FakeQuantize: unsupported bits %u", nd.d.bits);
@@ -318,7 +367,9 @@ rlx_exec *rlx_mi355x_compile(const rlx_graph_desc *g, const rlx_compile_opts *op
     std::vector<bool> grouped(e->nodes.size(), false);
     for (uint32_t i = 0; i < g->n_nodes; i++) {
         Node &nd = e->nodes[i];
-        if (grouped[i] || (nd.d.op_kind != RLX_OP_DEQUANT_MATMUL && nd.d.op_kind != RLX_OP_FAKE_QUANTIZE)) continue;
+        if (grouped[i] || (nd.d.op_kind != RLX_OP_DEQUANT_MATMUL && nd.d.op_kind != RLX_OP_FAKE_QUANTIZE &&
+                           nd.d.op_kind != RLX_OP_DEQUANT_GROUPED_MATMUL))
+            continue;
         std::vector<uint32_t> step{i};
         if (nd.d.op_kind == RLX_OP_DEQUANT_MATMUL) {
             const uint32_t xdt = e->nodes[nd.d.inputs[0]].d.dtype;
@@ -346,7 +397,7 @@ rlx_exec *rlx_mi355x_compile(const rlx_graph_desc *g, const rlx_compile_opts *op
     };
     for (Node &nd : e->nodes) {
         if (nd.is_packed) {
-            nd.slot = take((size_t)weight_dims(nd.scheme, nd.w_n, nd.w_k).bytes);  // device layout, resident
+            nd.slot = take((size_t)weight_dims(nd.scheme, nd.w_n, nd.w_k).bytes * (size_t)nd.w_experts);  // device layout, resident
         } else if (nd.d.op_kind == RLX_OP_INPUT) {
             nd.slot = take((size_t)nd.numel * 4);  // room for an f32 upload even when declared 16-bit
             nd.cur_dtype = nd.d.dtype;
@@ -397,6 +448,9 @@ int rlx_exec_set_param_typed(rlx_exec *e, const char *name, const void *data, si
                 rlx_mi355x_qweight_destroy(nd.qw);
                 nd.qw = nullptr;
             }
+            if (nd.w_experts > 1)
+                return rlx_mi355x_qweight_create_experts_at(nd.scheme, data, nbytes, nd.w_n, nd.w_k, nd.w_experts, e->ptr(nd.slot),
+                                                            &nd.qw);
             return rlx_mi355x_qweight_create_at(nd.scheme, data, nbytes, nd.w_n, nd.w_k, e->ptr(nd.slot), &nd.qw);
         }
         if (nbytes > nd.slot.size) {
@@ -468,7 +522,23 @@ int rlx_exec_write_input(rlx_exec *e, const char *name, const void *data, size_t
 static int enqueue_schedule(rlx_exec *e) {
     for (const std::vector<uint32_t> &step : e->steps) {
         Node &nd = e->nodes[step[0]];
-        if (nd.d.op_kind == RLX_OP_DEQUANT_MATMUL && nd.m > 8) {
+        if (nd.d.op_kind == RLX_OP_DEQUANT_GROUPED_MATMUL) {
+            Node &x = e->nodes[nd.d.inputs[0]];
+            Node &w = e->nodes[nd.d.inputs[1]];
+            Node &idx = e->nodes[nd.d.inputs[2]];
+            if (!w.qw) {
+                set_error("run: packed weight '%s' was never set (set_param_typed(.., U8))", w.name.c_str());
+                return RLX_ERR_INVALID;
+            }
+            uint32_t dt = x.d.op_kind == RLX_OP_INPUT ? x.cur_dtype : x.d.dtype;
+            uint32_t idt = idx.d.op_kind == RLX_OP_INPUT ? idx.cur_dtype : idx.d.dtype;
+            if (idt != RLX_F32) {
+                set_error("run: expert_idx of node %u must be written as F32", step[0]);
+                return RLX_ERR_INVALID;
+            }
+            RLX_TRY(rlx_mi355x_gguf_grouped_matmul_bt(e->ptr(x.slot), (int)dt, w.qw, (const float *)e->ptr(idx.slot),
+                                                      (float *)e->ptr(nd.slot), nd.m, e->stream));
+        } else if (nd.d.op_kind == RLX_OP_DEQUANT_MATMUL && nd.m > 8) {
             for (uint32_t id : step) {  // prefill: one GEMM per node, each with its own workspace slot
                 Node &mm = e->nodes[id];
                 Node &x = e->nodes[mm.d.inputs[0]];

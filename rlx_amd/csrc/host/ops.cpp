@@ -12,9 +12,10 @@ int repack_host(int scheme, const uint8_t *src, size_t nbytes, int64_t n, int64_
 
 struct rlx_qweight {
     int scheme;
-    rlx::WeightDims dims;
+    rlx::WeightDims dims;  // of one [n, k] matrix
     uint8_t *dev;
     bool owns;
+    int experts;           // matrices stacked dims.bytes apart (1 for a plain weight)
 };
 
 namespace rlx {
@@ -35,6 +36,9 @@ struct GemvSeg {
 struct GemvArgs {
     GemvSeg seg[GEMV_MAX_SEG];
     int nseg, m, kc_units, x_dtype, max_tiles_per_wg;
+    const float *expert_idx;
+    long long slab_bytes;
+    int num_experts;
 };
 struct FqArgs {
     const float *x;
@@ -76,7 +80,7 @@ static int x_kind(int x_dtype) {
 // One decode launch over `count` (<= GEMV_MAX_SEG) matmuls of one scheme, batch and activation dtype; each has
 // its own activations, K and N.
 static int launch_gemv(const void *const *xs, int xk, const rlx_qweight *const *ws, float *const *outs, int count, int m,
-                       hipStream_t stream) {
+                       hipStream_t stream, const float *expert_idx = nullptr) {
     const int scheme = ws[0]->scheme;
     const Layout L = layout_of(scheme);
     for (int i = 0; i < count; i++)
@@ -142,6 +146,9 @@ static int launch_gemv(const void *const *xs, int xk, const rlx_qweight *const *
         sh.a.kc_units = sh.kcu;
         sh.a.x_dtype = xk;
         sh.a.max_tiles_per_wg = max_tpw;
+        sh.a.expert_idx = expert_idx;
+        sh.a.slab_bytes = ws[0]->dims.bytes;
+        sh.a.num_experts = ws[0]->experts;
         return sh;
     };
     // Two workgroups of 8 waves per CU with 80 KB each: holds a 14336-wide f32 vector (hi + lo rows) in one chunk.
@@ -248,7 +255,7 @@ int rlx_mi355x_qweight_create_at(int scheme, const void *gguf_bytes, size_t nbyt
         set_error("qweight upload: %s", hipGetErrorString(e));
         return RLX_ERR_HIP;
     }
-    *out = new rlx_qweight{scheme, D, (uint8_t *)device_mem, owns};
+    *out = new rlx_qweight{scheme, D, (uint8_t *)device_mem, owns, 1};
     return RLX_OK;
 }
 
@@ -257,13 +264,48 @@ int rlx_mi355x_qweight_create(int scheme, const void *gguf_bytes, size_t nbytes,
     return rlx_mi355x_qweight_create_at(scheme, gguf_bytes, nbytes, n, k, nullptr, out);
 }
 
+int rlx_mi355x_qweight_create_experts_at(int scheme, const void *gguf_bytes, size_t nbytes, int64_t n, int64_t k,
+                                         int64_t num_experts, void *device_mem, rlx_qweight **out) {
+    using namespace rlx;
+    RLX_TRY(runtime_init());
+    WeightDims D = weight_dims(scheme, n, k);
+    if (D.bytes == 0) {
+        set_error("qweight: scheme %d is not a claimed GGUF scheme", scheme);
+        return RLX_ERR_UNSUPPORTED;
+    }
+    const int64_t slab = rlx_mi355x_bytes_for(scheme, n * k);
+    if (num_experts < 1 || num_experts > 0x7FFFFFFF || slab < 0 || nbytes != (size_t)(slab * num_experts)) {
+        set_error("qweight: got %zu bytes, %lld experts of [%lld x %lld] need %lld", nbytes, (long long)num_experts, (long long)n,
+                  (long long)k, (long long)(slab < 0 ? -1 : slab * num_experts));
+        return RLX_ERR_INVALID;
+    }
+    std::vector<uint8_t> staging((size_t)D.bytes * (size_t)num_experts);
+    for (int64_t e = 0; e < num_experts; e++)
+        RLX_TRY(repack_host(scheme, (const uint8_t *)gguf_bytes + e * slab, (size_t)slab, n, k, staging.data() + e * D.bytes));
+    bool owns = device_mem == nullptr;
+    if (owns) RLX_HIP(hipMalloc(&device_mem, staging.size()));
+    hipError_t err = hipMemcpy(device_mem, staging.data(), staging.size(), hipMemcpyHostToDevice);
+    if (err != hipSuccess) {
+        if (owns) (void)hipFree(device_mem);
+        set_error("qweight upload: %s", hipGetErrorString(err));
+        return RLX_ERR_HIP;
+    }
+    *out = new rlx_qweight{scheme, D, (uint8_t *)device_mem, owns, (int)num_experts};
+    return RLX_OK;
+}
+
+int rlx_mi355x_qweight_create_experts(int scheme, const void *gguf_bytes, size_t nbytes, int64_t n, int64_t k,
+                                      int64_t num_experts, rlx_qweight **out) {
+    return rlx_mi355x_qweight_create_experts_at(scheme, gguf_bytes, nbytes, n, k, num_experts, nullptr, out);
+}
+
 void rlx_mi355x_qweight_destroy(rlx_qweight *w) {
     if (!w) return;
     if (w->owns) (void)hipFree(w->dev);
     delete w;
 }
 
-size_t rlx_mi355x_qweight_device_bytes(const rlx_qweight *w) { return w ? (size_t)w->dims.bytes : 0; }
+size_t rlx_mi355x_qweight_device_bytes(const rlx_qweight *w) { return w ? (size_t)w->dims.bytes * (size_t)w->experts : 0; }
 
 int rlx_mi355x_dequant(const rlx_qweight *w, float *out_dev, void *stream) {
     using namespace rlx;
@@ -335,6 +377,37 @@ int rlx_mi355x_gguf_matmul_bt_batch(const void *const *xs_dev, int x_dtype, cons
 int rlx_mi355x_gguf_matmul_bt(const void *x_dev, int x_dtype, const rlx_qweight *w, float *out_dev, int64_t m,
                               void *workspace, size_t workspace_bytes, void *stream) {
     return rlx_mi355x_gguf_matmul_bt_batch(&x_dev, x_dtype, &w, &out_dev, 1, m, workspace, workspace_bytes, stream);
+}
+
+int rlx_mi355x_gguf_grouped_matmul_bt(const void *x_dev, int x_dtype, const rlx_qweight *w, const float *expert_idx_dev,
+                                      float *out_dev, int64_t m, void *stream) {
+    using namespace rlx;
+    if (!x_dev || !w || !expert_idx_dev || !out_dev || m <= 0) {
+        set_error("gguf_grouped_matmul_bt: null argument or m=%lld", (long long)m);
+        return RLX_ERR_INVALID;
+    }
+    const int xk = x_kind(x_dtype);
+    if (xk < 0) {
+        set_error("gguf_grouped_matmul_bt: activation dtype %d is not F32 / BF16 / F16", x_dtype);
+        return RLX_ERR_UNSUPPORTED;
+    }
+    RLX_TRY(runtime_init());
+    // Every token is its own one-row matmul against the slab its index names: up to eight tokens per launch, each
+    // a segment of the decode kernel. Tokens that share an expert stream its slab again (once from HBM, then from L2).
+    const size_t esz = xk == 0 ? 4 : 2;
+    for (int64_t t0 = 0; t0 < m; t0 += GEMV_MAX_SEG) {
+        const int c = (int)std::min<int64_t>(GEMV_MAX_SEG, m - t0);
+        const void *xs[GEMV_MAX_SEG];
+        const rlx_qweight *ws[GEMV_MAX_SEG];
+        float *outs[GEMV_MAX_SEG];
+        for (int i = 0; i < c; i++) {
+            xs[i] = (const uint8_t *)x_dev + (size_t)(t0 + i) * w->dims.k * esz;
+            ws[i] = w;
+            outs[i] = out_dev + (size_t)(t0 + i) * w->dims.n;
+        }
+        RLX_TRY(launch_gemv(xs, xk, ws, outs, c, 1, (hipStream_t)stream, expert_idx_dev + t0));
+    }
+    return RLX_OK;
 }
 
 // Column layout (channels along the last axis, 16-byte aligned rows): pass A and pass B use their own row blocking.

@@ -38,6 +38,11 @@ struct GemvArgs {
     int kc_units;      // most units staged in LDS at once
     int x_dtype;
     int max_tiles_per_wg;
+    // Mixture-of-experts routing (rlx-cpu/src/gguf_matmul.rs:101-139): when expert_idx is set, segment s is token s and
+    // reads the slab of expert (int)expert_idx[s] (clamped to the stack), slab_bytes apart in the device layout.
+    const float *expert_idx;
+    long long slab_bytes;
+    int num_experts;
 };
 
 constexpr int XS_PAD_HALFS = 8;      // 16 bytes of padding per LDS row: rows land in different bank groups
@@ -255,7 +260,12 @@ __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
 #pragma unroll
     for (int i = 1; i < GEMV_MAX_SEG; i++)
         if (i < a.nseg && (int)blockIdx.x >= a.seg[i].wg_begin) s = i;
-    const GemvSeg seg = a.seg[s];
+    GemvSeg seg = a.seg[s];
+    if (a.expert_idx) {
+        int e = (int)a.expert_idx[s];
+        e = e < 0 ? 0 : (e >= a.num_experts ? a.num_experts - 1 : e);
+        seg.w += (long long)e * a.slab_bytes;
+    }
     const int tile0 = ((int)blockIdx.x - seg.wg_begin) * seg.tiles_per_wg;
     const int ntiles = min(seg.tiles_per_wg, seg.row_tiles - tile0);
     const int kc_units = min(a.kc_units, seg.units);

@@ -64,6 +64,7 @@ class OpKind(enum.IntEnum):
     Param = 1
     DequantMatMul = 2
     FakeQuantize = 3
+    DequantGroupedMatMul = 4
 
 
 @dataclass(frozen=True)
@@ -101,6 +102,10 @@ class Op:
     @staticmethod
     def DequantMatMul(scheme):  # Op::DequantMatMul { scheme } (op.rs:736-752)
         return Op(OpKind.DequantMatMul, scheme=scheme)
+
+    @staticmethod
+    def DequantGroupedMatMul(scheme):  # Op::DequantGroupedMatMul { scheme } (op.rs:862-871)
+        return Op(OpKind.DequantGroupedMatMul, scheme=scheme)
 
     @staticmethod
     def FakeQuantize(bits, axis, ste=SteKind.Identity, scale_mode=ScaleMode.PerBatch, ema_decay=0.0):  # op.rs:407-432
@@ -143,6 +148,9 @@ class Graph:
 
     def dequant_matmul_packed(self, x, packed_w, scheme, shape):  # rlx-ir/src/ops/linalg.rs:78-91
         return self.add_node(Op.DequantMatMul(scheme), [x, packed_w], shape)
+
+    def dequant_grouped_matmul(self, x, packed_experts, expert_idx, scheme, shape):
+        return self.add_node(Op.DequantGroupedMatMul(scheme), [x, packed_experts, expert_idx], shape)
 
     def fake_quantize(self, x, bits, axis, scale_mode=ScaleMode.PerBatch, state=None, ema_decay=0.0):
         ins = [x] if state is None else [x, state]

@@ -121,11 +121,16 @@ def philox_normal(seed, n):
 class QWeight:
     """GGUF-packed [n, k] matrix resident in HBM in the device layout."""
 
-    def __init__(self, scheme, packed, n, k):
+    def __init__(self, scheme, packed, n, k, num_experts=1):
+        """`num_experts` > 1: `packed` is a stack of that many [n, k] slabs, expert outermost (MoE weights)."""
         packed = np.ascontiguousarray(packed, dtype=np.uint8)
-        self.scheme, self.n, self.k = QuantScheme(scheme), int(n), int(k)
+        self.scheme, self.n, self.k, self.num_experts = QuantScheme(scheme), int(n), int(k), int(num_experts)
         p = C.c_void_p()
-        _lib.check(_lib.lib().rlx_mi355x_qweight_create(int(scheme), packed.ctypes.data, packed.size, n, k, C.byref(p)))
+        if num_experts == 1:
+            _lib.check(_lib.lib().rlx_mi355x_qweight_create(int(scheme), packed.ctypes.data, packed.size, n, k, C.byref(p)))
+        else:
+            _lib.check(_lib.lib().rlx_mi355x_qweight_create_experts(int(scheme), packed.ctypes.data, packed.size, n, k,
+                                                                    num_experts, C.byref(p)))
         self.ptr = p.value
 
     def device_bytes(self):
@@ -172,6 +177,18 @@ def gguf_matmul_bt(x, w: QWeight, m, x_dtype=DType.F32):
     ws = gguf_matmul_bt_device(xd, x_dtype, w, od, m)
     sync()
     del ws
+    return od.to_numpy(np.float32).reshape(m, w.n)
+
+
+def gguf_grouped_matmul_bt(x, w: QWeight, expert_idx, x_dtype=DType.F32):
+    """Host convenience for the MoE matmul: out[i] = x[i] . W[expert_idx[i]]^T; x is [m, k], expert_idx [m]."""
+    idx = np.ascontiguousarray(expert_idx, dtype=np.float32)
+    m = idx.size
+    xd = DeviceBuffer.from_numpy(x)
+    idd = DeviceBuffer.from_numpy(idx)
+    od = DeviceBuffer(m * w.n * 4)
+    _lib.check(_lib.lib().rlx_mi355x_gguf_grouped_matmul_bt(xd.ptr, int(x_dtype), w.ptr, idd.ptr, od.ptr, m, None))
+    sync()
     return od.to_numpy(np.float32).reshape(m, w.n)
 
 

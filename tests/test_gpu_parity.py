@@ -432,3 +432,58 @@ def test_graph_prefill_through_session(oracle):
     x = np.random.default_rng(82).standard_normal((m, k)).astype(np.float32)
     got = run_dq(packed, Q4K, x, m, k, n)
     assert rel_err(got, oracle.gguf_matmul_f64(x, packed, m, k, n, Q4K)) <= TOL
+
+
+# ------------------------------------------------------------------ grouped (MoE) matmul
+
+@pytest.mark.parametrize("scheme", [Q4K, Q4_0, Q8_0])
+def test_grouped_matmul_reference_case_through_session(oracle, scheme):
+    # rlx-runtime/tests/dequant_grouped_matmul_gguf.rs:71-123 restated for the schemes on this path: k=256, n=4, m=5,
+    # three experts, non-contiguous expert ids, x[i] = 0.01 (i+1), compared per row with the reference CPU path
+    k, n, m, experts = 256, 4, 5, 3
+    packed = np.concatenate([make_weights(scheme, n, k, std=0.02 * (e + 1), seed=70 + e)[0] for e in range(experts)])
+    x = (0.01 * (np.arange(m * k, dtype=np.float32) + 1.0)).astype(np.float32)
+    idx = np.array([1.0, 0.0, 2.0, 1.0, 0.0], np.float32)
+    g = Graph.new("dq_grouped_matmul")
+    x_in = g.input("x", Shape.new([m, k], DType.F32))
+    w = g.param("w_packed", Shape.new([packed.size], DType.U8))
+    i_in = g.input("expert_idx", Shape.new([m], DType.F32))
+    y = g.add_node(Op.DequantGroupedMatMul(QuantScheme(scheme)), [x_in, w, i_in], Shape.new([m, n], DType.F32))
+    g.set_outputs([y])
+    c = Session.new(rlx_amd.Device.Mi355x).compile(g)
+    c.set_param_typed("w_packed", packed, DType.U8)
+    got = c.run([("x", x), ("expert_idx", idx)])[0].reshape(m, n)
+    want = oracle.gguf_grouped_matmul_bt(x, packed, idx, m, k, n, experts, scheme)
+    assert np.max(np.abs(got - want) / np.maximum(np.abs(want), 1.0)) < 1e-4
+    assert rel_err(got, oracle.gguf_grouped_matmul_f64(x, packed, idx, m, k, n, experts, scheme)) <= TOL
+
+
+@pytest.mark.parametrize("x_dtype", [DType.F32, DType.BF16])
+def test_grouped_matmul_many_tokens_and_experts(oracle, x_dtype):
+    # more rows than one launch carries (8), every expert used, one unused, a repeated expert, ragged n
+    rng = np.random.default_rng(12)
+    k, n, experts, m = 1024, 40, 6, 19
+    packed = np.concatenate([make_weights(Q4K, n, k, seed=90 + e)[0] for e in range(experts)])
+    w = ops.QWeight(QuantScheme.GgufQ4K, packed, n, k, num_experts=experts)
+    assert w.device_bytes() == experts * ops.QWeight(QuantScheme.GgufQ4K, packed[:packed.size // experts], n, k).device_bytes()
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    idx = rng.integers(0, experts - 1, m).astype(np.float32)  # expert 5 never picked
+    idx[0] = idx[1] = idx[9] = 3.0
+    if x_dtype == DType.BF16:
+        x = oracle.bf16_round(x)
+        got = ops.gguf_grouped_matmul_bt(f32_to_bf16_bits(x), w, idx, DType.BF16)
+    else:
+        got = ops.gguf_grouped_matmul_bt(x, w, idx)
+    assert rel_err(got, oracle.gguf_grouped_matmul_f64(x, packed, idx, m, k, n, experts, oracle.Q4K)) <= TOL
+    # routing is exact: rows sent to the same expert with the same input give identical outputs
+    x2 = x.copy()
+    x2[1] = x2[0]
+    got2 = ops.gguf_grouped_matmul_bt(f32_to_bf16_bits(x2), w, idx, DType.BF16) if x_dtype == DType.BF16 else \
+        ops.gguf_grouped_matmul_bt(x2, w, idx)
+    assert np.array_equal(got2[0], got2[1]) and np.array_equal(got2[0], got[0])
+    # an index past the stack is clamped to the last expert rather than read out of bounds
+    hi = ops.gguf_grouped_matmul_bt(f32_to_bf16_bits(x[:1]) if x_dtype == DType.BF16 else x[:1], w, np.array([99.0], np.float32),
+                                    x_dtype)
+    last = ops.gguf_grouped_matmul_bt(f32_to_bf16_bits(x[:1]) if x_dtype == DType.BF16 else x[:1], w,
+                                      np.array([experts - 1.0], np.float32), x_dtype)
+    assert np.array_equal(hi, last)

@@ -128,7 +128,7 @@ def compile_error(g):
 
 
 def test_supported_ops():
-    assert [int(k) for k in rlx_amd.supported_ops()] == [0, 1, 2, 3]
+    assert [int(k) for k in rlx_amd.supported_ops()] == [0, 1, 2, 3, 4]
 
 
 def test_compile_rejects_wrong_weight_size():
@@ -176,3 +176,21 @@ def test_compile_without_device_fails_loudly():
     assert "no HIP device" in msg or "gfx950" in msg
     with pytest.raises(rlx_amd.RlxError):
         ops.DeviceBuffer(16)
+
+
+def test_compile_rejects_bad_grouped_matmul():
+    from rlx_amd import DType, Graph, Op, Shape
+    m, k, n, experts = 5, 256, 4, 3
+    slab = k * n // 256 * 144
+
+    def graph(w_bytes, idx_len):
+        g = Graph.new("grouped")
+        x = g.input("x", Shape.new([m, k], DType.F32))
+        w = g.param("w_packed", Shape.new([w_bytes], DType.U8))
+        idx = g.input("expert_idx", Shape.new([idx_len], DType.F32))
+        y = g.add_node(Op.DequantGroupedMatMul(Q4K), [x, w, idx], Shape.new([m, n], DType.F32))
+        g.set_outputs([y])
+        return g
+
+    assert "packed experts must be a U8 param" in compile_error(graph(experts * slab + 7, m))
+    assert "expert_idx [m]" in compile_error(graph(experts * slab, m + 1))

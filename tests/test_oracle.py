@@ -3,6 +3,8 @@ independent restatements (numpy library casts, bit-field views, textbook f64 mat
 import numpy as np
 import pytest
 
+from helpers import random_blocks
+
 Q4K, Q4_0, Q8_0 = 5, 11, 12
 
 
@@ -411,3 +413,53 @@ def test_philox_stream_properties(oracle):
     # counter advances once per 4 outputs: stream = concatenated blocks of counters 0,1,2...
     blk1 = oracle.philox_block([1, 0, 0, 0], [7, 0], oracle.M0_REFERENCE)
     assert np.array_equal(oracle.philox_u32(7, 8)[4:], blk1)
+
+
+# ------------------------------------------------------------------ grouped (MoE) matmul
+
+def test_grouped_matmul_reference_case_shape(oracle):
+    # the case of rlx-runtime/tests/dequant_grouped_matmul_gguf.rs:71-123 (k=256, n=4, m=5, 3 experts with distinct
+    # scales, non-contiguous expert ids, x[i] = 0.01 (i+1)) restated for the schemes on this path; expected values come
+    # from the test's own per-row restatement: dequantize the row's slab, then a scalar f32 dot product per column
+    k, n, m, experts = 256, 4, 5, 3
+    x = (0.01 * (np.arange(m * k, dtype=np.float32) + 1.0)).astype(np.float32)
+    idx = np.array([1.0, 0.0, 2.0, 1.0, 0.0], np.float32)
+    for scheme, block_bytes, block in ((oracle.Q8_0, 34, 32), (oracle.Q4_0, 18, 32), (oracle.Q4K, 144, 256)):
+        slabs = []
+        for e, scale in enumerate((0.25, 0.5, 1.0)):
+            blocks = random_blocks(scheme, n, k, seed=40 + e)
+            blocks = blocks.reshape(-1, block_bytes).copy()
+            blocks[:, 0:2] = np.frombuffer(np.float16(scale).tobytes(), np.uint8)  # d of every block
+            slabs.append(blocks.reshape(-1))
+        packed = np.concatenate(slabs)
+        slab = packed.size // experts
+        got = oracle.gguf_grouped_matmul_bt(x, packed, idx, m, k, n, experts, scheme)
+        for row in range(m):
+            e = int(idx[row])
+            w_ref = oracle.dequant(scheme, packed[e * slab:(e + 1) * slab], k * n).reshape(n, k)
+            for c in range(n):
+                acc = np.float32(0.0)
+                for i in range(k):
+                    acc = np.float32(acc + np.float32(x[row * k + i] * w_ref[c, i]))
+                assert abs(got[row, c] - acc) / max(abs(acc), 1.0) < 1e-4
+
+
+def test_grouped_matmul_equals_independent_rows(oracle):
+    # every output row is the plain matmul of its input row with its expert's slab, bit for bit: the sort by expert
+    # and the scatter back move rows, they do not change any sum
+    rng = np.random.default_rng(9)
+    k, n, m, experts = 128, 24, 11, 4
+    packed = np.concatenate([random_blocks(oracle.Q4_0, n, k, seed=60 + e) for e in range(experts)])
+    slab = packed.size // experts
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    idx = rng.integers(0, experts, m).astype(np.float32)
+    idx[3] = 2.9  # float-encoded indices truncate (`as usize`)
+    got = oracle.gguf_grouped_matmul_bt(x, packed, idx, m, k, n, experts, oracle.Q4_0)
+    for i in range(m):
+        e = int(idx[i])
+        want = oracle.gguf_matmul_bt(x[i], packed[e * slab:(e + 1) * slab], 1, k, n, oracle.Q4_0)[0]
+        assert np.array_equal(got[i], want)
+    with pytest.raises(ValueError, match="out of range"):
+        oracle.gguf_grouped_matmul_bt(x, packed, np.full(m, float(experts), np.float32), m, k, n, experts, oracle.Q4_0)
+    with pytest.raises(ValueError, match="bad sizes"):
+        oracle.gguf_grouped_matmul_bt(x, packed[:-1], idx, m, k, n, experts, oracle.Q4_0)
