@@ -317,17 +317,16 @@ __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
         __syncthreads();
         if constexpr (SCHEME == SCHEME_Q4K) {
             const int nblk = nu * BLK_PER_UNIT;
-            for (int idx = tid; idx < nblk * 16; idx += blockDim.x) {
-                int blk = idx >> 4, i = idx & 15;
+            // rows >= rv of the [blk][16] table are never read: compute_unit only uses the rows its lane group owns
+            for (int idx = tid; idx < nblk * rv; idx += blockDim.x) {
+                const int blk = idx / rv, i = idx - blk * rv;
                 float sum = 0.f;
-                if (i < rv) {
 #pragma unroll
-                    for (int e4 = 0; e4 < 4; e4++) {
-                        Frag f;
-                        f.u4 = *(const uint4_t *)(xs + i * row_stride + blk * 32 + e4 * 8);
+                for (int e4 = 0; e4 < 4; e4++) {
+                    Frag f;
+                    f.u4 = *(const uint4_t *)(xs + i * row_stride + blk * 32 + e4 * 8);
 #pragma unroll
-                        for (int e = 0; e < 8; e++) sum += (float)f.h8[e];
-                    }
+                    for (int e = 0; e < 8; e++) sum += (float)f.h8[e];
                 }
                 sxs[blk * 16 + i] = sum;
             }
