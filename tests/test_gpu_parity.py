@@ -487,3 +487,39 @@ def test_grouped_matmul_many_tokens_and_experts(oracle, x_dtype):
     last = ops.gguf_grouped_matmul_bt(f32_to_bf16_bits(x[:1]) if x_dtype == DType.BF16 else x[:1], w,
                                       np.array([experts - 1.0], np.float32), x_dtype)
     assert np.array_equal(hi, last)
+
+
+def test_captured_graph_fq_prefill_and_grouped_replays(oracle):
+    # FakeQuantize -> split-K prefill GEMM (its output clear is a fill kernel, not a memset node) and an MoE matmul in
+    # one executable, captured into a hipGraph and replayed with fresh inputs; every replay is checked like the eager run
+    rows, k, n, experts = 64, 2048, 96, 3
+    packed, _ = make_weights(Q4K, n, k, seed=51)
+    stack = np.concatenate([make_weights(Q4_0, n, k, seed=52 + e)[0] for e in range(experts)])
+    g = Graph.new("captured")
+    xi = g.input("x", Shape.new([rows, k], DType.F32))
+    fq = g.add_node(Op.FakeQuantize(8, 1), [xi], Shape.new([rows, k], DType.F32))
+    w = g.param("w", Shape.new([len(packed)], DType.U8))
+    y = g.add_node(Op.DequantMatMul(QuantScheme.GgufQ4K), [fq, w], Shape.new([rows, n], DType.F32))
+    xt = g.input("tokens", Shape.new([4, k], DType.F32))
+    we = g.param("experts", Shape.new([len(stack)], DType.U8))
+    ei = g.input("expert_idx", Shape.new([4], DType.F32))
+    z = g.add_node(Op.DequantGroupedMatMul(QuantScheme.GgufQ4_0), [xt, we, ei], Shape.new([4, n], DType.F32))
+    g.set_outputs([y, z])
+    c = Session.new().compile(g)
+    c.set_param_typed("w", packed, DType.U8)
+    c.set_param_typed("experts", stack, DType.U8)
+    rng = np.random.default_rng(53)
+    for attempt in ("eager", "replay 1", "replay 2", "replay 3"):
+        x = heavy_tailed(rows, k, 54 + len(attempt)) * np.float32(1.0 + 0.25 * len(attempt))
+        tokens = rng.standard_normal((4, k)).astype(np.float32)
+        idx = rng.integers(0, experts, 4).astype(np.float32)
+        c.write_input("x", x)
+        c.write_input("tokens", tokens)
+        c.write_input("expert_idx", idx)
+        c.launch()
+        y_got, z_got = c.read_output(0).reshape(rows, n), c.read_output(1).reshape(4, n)
+        fq_ref, _, _ = oracle.fake_quantize(x, x.shape, 1, 8)
+        assert rel_err(y_got, oracle.gguf_matmul_f64(fq_ref, packed, rows, k, n, Q4K)) <= TOL, attempt
+        assert rel_err(z_got, oracle.gguf_grouped_matmul_f64(tokens, stack, idx, 4, k, n, experts, Q4_0)) <= TOL, attempt
+        if attempt == "eager":
+            c.capture()
