@@ -109,31 +109,33 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
     // Activations run AD steps ahead of their LDS store: two where registers allow (their loads come through L2 with
     // the whole workgroup's 32 KB per step behind them), one for Q4_K whose second accumulator set takes the room.
     constexpr int AD = K4 ? 1 : 2;
+    // Buffer loads: wave-uniform descriptor and scalar offset, constant per-lane offset, so a fetch costs no VALU.
+    // A wave that moves no activation chunk (64-row tile) gets an empty range: its loads return zeros without traffic.
+    const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)a_base, 0, a_mine ? 0x7FFFFFFF : 0, 0x00020000);
+    const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)b_tile, 0, 0x7FFFFFFF, 0x00020000);
+    auto ld128 = [&](__amdgpu_buffer_rsrc_t r, int voff, int soff) { return __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0); };
     auto fetch_a = [&](int step, int set) {
-        const uint8_t *p = a_base + (long long)step * GEMM_STAGE_A + a_src0;
-        if (a_mine) {
 #pragma unroll
-            for (int i = 0; i < 4; i++) a_reg[AD == 2 ? set : 0][i] = *(const uint4_t *)(p + i * 8192);
-        }
+        for (int i = 0; i < 4; i++) a_reg[AD == 2 ? set : 0][i] = ld128(a_rsrc, a_src0, step * GEMM_STAGE_A + i * 8192);
     };
     auto fetch_b = [&](int step, int q) {  // q = step & 3, compile-time at every call site
         if constexpr (K4) {  // dead tiles read tile 0 (valid memory) and are zeroed when stored
-            const uint8_t *unit = b_tile + (long long)(step >> 2) * L.unit_bytes;
-            if ((q & 1) == 0) b_q[(q >> 1) & 1] = *(const uint4_t *)(unit + (q >> 1) * 1024 + lane * 16);
-            if (q == 0) b_meta[0] = *(const uint4_t *)(unit + 2048 + b_n16 * 16);  // consumed one step later, before the next fetch
+            const int unit = (step >> 2) * L.unit_bytes;
+            if ((q & 1) == 0) b_q[(q >> 1) & 1] = ld128(b_rsrc, lane * 16, unit + (q >> 1) * 1024);
+            if (q == 0) b_meta[0] = ld128(b_rsrc, b_n16 * 16, unit + 2048);  // consumed one step later, before the next fetch
         } else if constexpr (SCHEME == SCHEME_Q4_0) {
-            const uint8_t *unit = b_tile + (long long)(step >> 1) * L.unit_bytes;
+            const int unit = (step >> 1) * L.unit_bytes;
             if ((q & 1) == 0) {
-                b_q[(q >> 1) & 1] = *(const uint4_t *)(unit + lane * 16);
-                uint2_t sc = *(const uint2_t *)(unit + 1024 + b_n16 * 8);
+                b_q[(q >> 1) & 1] = ld128(b_rsrc, lane * 16, unit);
+                uint2_t sc = __builtin_amdgcn_raw_buffer_load_b64(b_rsrc, b_n16 * 8, unit + 1024, 0);
                 b_meta[(q >> 1) & 1][0] = sc[0];
                 b_meta[(q >> 1) & 1][1] = sc[1];
             }
         } else {
-            const uint8_t *unit = b_tile + (long long)(step >> 1) * L.unit_bytes;
-            b_q[q & 1] = *(const uint4_t *)(unit + (q & 1) * 1024 + lane * 16);
+            const int unit = (step >> 1) * L.unit_bytes;
+            b_q[q & 1] = ld128(b_rsrc, lane * 16, unit + (q & 1) * 1024);
             if ((q & 1) == 0) {
-                uint2_t sc = *(const uint2_t *)(unit + 2048 + b_n16 * 8);
+                uint2_t sc = __builtin_amdgcn_raw_buffer_load_b64(b_rsrc, b_n16 * 8, unit + 2048, 0);
                 b_meta[(q >> 1) & 1][0] = sc[0];
                 b_meta[(q >> 1) & 1][1] = sc[1];
             }
@@ -154,18 +156,18 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
                 uint32_t mn[2];
                 const uint4_t &m4 = b_meta[0];
                 q4k_scales(m4[1], m4[2], m4[3], b_sc, mn);
+                b_sc[0] &= b_keep;  // a dead tile decodes to zeros
+                b_sc[1] &= b_keep;
             }
             unpack_q4_scaled(b_q[cp][t], splat_code_half(b_sc[q >> 1], t), f);
         } else {
-            const uint32_t dbits = (t & 1) ? (b_meta[cp][t >> 1] >> 16) : (b_meta[cp][t >> 1] & 0xFFFFu);
+            const uint32_t dbits = ((t & 1) ? (b_meta[cp][t >> 1] >> 16) : (b_meta[cp][t >> 1] & 0xFFFFu)) & b_keep;  // dead tile: d = 0
             const half2_t d2 = as_half2(dbits | (dbits << 16));
             if constexpr (SCHEME == SCHEME_Q4_0) unpack_q4<8>(b_q[cp][t], f);
             else unpack_q8(b_q[q & 1][2 * jl], b_q[q & 1][2 * jl + 1], f);
 #pragma unroll
             for (int e = 0; e < 4; e++) f.h2[e] = f.h2[e] * d2;
         }
-#pragma unroll
-        for (int e = 0; e < 4; e++) f.u[e] &= b_keep;
         *(uint4_t *)(stage + b_dst[jl]) = f.u4;
     };
 
@@ -200,129 +202,173 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
         a_rd[ks] = frag_offset(NSA, ks, wm * TI, lr, lh);
         b_rd[ks] = SA + frag_offset(4, ks, wn * TJ, lr, lh);
     }
-    Frag fa[2][TI], fb[2][TJ];  // [buffer][tile]
+    // Fragment buffers: a compute half starts with slices 0 .. PD-1 already in registers (read during the data half
+    // before it) and reads slice ks + PD under the MFMAs of slice ks.
+    constexpr int NB = K4 ? 2 : 4, PD = NB / 2;
+    Frag fa[NB][TI], fb[NB][TJ];  // [buffer][tile]
     auto load_frags = [&](const uint8_t *stage, int ks, int buf) {
 #pragma unroll
         for (int i = 0; i < TI; i++) fa[buf][i].u4 = *(const uint4_t *)(stage + a_rd[ks] + i * 1024);
 #pragma unroll
         for (int j = 0; j < TJ; j++) fb[buf][j].u4 = *(const uint4_t *)(stage + b_rd[ks] + j * 1024);
     };
+    auto preload = [&](const uint8_t *stage) {
+#pragma unroll
+        for (int ks = 0; ks < PD; ks++) load_frags(stage, ks, ks);
+    };
 
-    if (step0 < step1) {  // step0 is a multiple of 4
-        fetch_a(step0, 0);
-        fetch_b(step0, 0);
-        if (AD == 2) fetch_a(min(step0 + 1, step1 - 1), 1);
-        fetch_b(min(step0 + 1, step1 - 1), 1);
-        store_a2(smem, 0, 0);
-        store_a2(smem, 2, 0);
-        store_b1(step0, 0, 0, smem);
-        store_b1(step0, 0, 1, smem);
-    }
-    __syncthreads();
-    if (step0 < step1) load_frags(smem, 0, 0);
-    // Three LDS stages: step s reads stage s % 3 and fills stage (s + 1) % 3, whose last readers (step s - 2) all
-    // passed the barrier of step s - 1. The one barrier per step sits after the third k-slice, when this step's
-    // stores are long issued, and the last slice already reads the first fragments of the next step: no wave
-    // starts a step by waiting for LDS.
-    int rd_off = 0, wr_off = ST;  // wave-uniform
-
-    for (int sbase = step0; sbase < step1; sbase += 4) {
+    // ---- Q4_K: a 256-column super-block is complete: total += d * P - dmin * (mn . sx) ----------------------
+    auto load_sb_meta = [&](int sb) {  // this wave's rows: meta and activation block sums of the super-block
 #pragma unroll
-        for (int q = 0; q < 4; q++) {
-            const int step = sbase + q;
-            if (step < step1) {
-                const uint8_t *stage = smem + rd_off;
-                uint8_t *next = smem + wr_off;
-                // No branches inside a step: the last steps re-fetch / re-store the final step into a stage nobody
-                // reads again, so each k-slice group below is one scheduling region.
-                const int nstep = min(step + 1, step1 - 1);
-                fetch_a(AD == 2 ? min(step + 2, step1 - 1) : nstep, q & 1);
-                fetch_b(min(step + 2, step1 - 1), (q + 2) & 3);
-                if constexpr (K4) {
-                    if (q == 0) {  // this wave's rows: meta and activation block sums of the super-block, used at q == 3
-                        const int sb = step >> 2;
+        for (int j = 0; j < TJ; j++) w_meta[j] = *(const uint4_t *)(my_meta[j] + (long long)sb * L.unit_bytes);
 #pragma unroll
-                        for (int j = 0; j < TJ; j++) w_meta[j] = *(const uint4_t *)(my_meta[j] + (long long)sb * L.unit_bytes);
+        for (int i = 0; i < TI; i++) {
+            long long row = m_tile0 + (wm * TI + i) * 32 + lr;
+            fs[i].u4 = *(const uint4_t *)(a.sxh + (row * (a.k_pad / 256) + sb) * 16 + lh * 8);
+        }
+    };
+    auto scale_sb = [&]() {
 #pragma unroll
-                        for (int i = 0; i < TI; i++) {
-                            long long row = m_tile0 + (wm * TI + i) * 32 + lr;
-                            fs[i].u4 = *(const uint4_t *)(a.sxh + (row * (a.k_pad / 256) + sb) * 16 + lh * 8);
-                        }
-                    }
+        for (int j = 0; j < TJ; j++) {
+            const uint4_t meta = w_meta[j];
+            const float d = my_ok[j] ? half_bits_to_float(meta[0] & 0xFFFFu) : 0.f;
+            const float dmin = my_ok[j] ? half_bits_to_float(meta[0] >> 16) : 0.f;
+            uint32_t sc[2], mn[2];
+            q4k_scales(meta[1], meta[2], meta[3], sc, mn);
+            // B' fragment: half 0 holds mn_0..7, half 1 holds mn_0..7 / 2048 (pairs with the lo sums)
+            Frag fm;
+            const half2_t k1024 = {(half_t)1024.0f, (half_t)1024.0f};
+            const half2_t lo_scale = {(half_t)(1.0f / GEMM_LO_SCALE), (half_t)(1.0f / GEMM_LO_SCALE)};
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                uint32_t src = (e < 2) ? mn[0] : mn[1];
+                uint32_t sel = (e & 1) ? 0x04030402u : 0x04010400u;  // bytes (2,3) or (0,1) -> [b,0x64,b',0x64]
+                half2_t v = as_half2(__builtin_amdgcn_perm(0x64646464u, src, sel)) - k1024;
+                fm.h2[e] = lh ? v * lo_scale : v;
+            }
+#pragma unroll
+            for (int i = 0; i < TI; i++) {
+                float16_t qq = mfma32(fs[i], fm, zero16);
+#pragma unroll
+                for (int e = 0; e < 16; e++) {
+                    total[i][j][e] = __builtin_fmaf(d, part[i][j][e], total[i][j][e]);
+                    total[i][j][e] = __builtin_fmaf(-dmin, qq[e], total[i][j][e]);
                 }
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int ks = 0; ks < 4; ks++) {
-                    const int buf = ks & 1;
-                    if (ks < 3) load_frags(stage, ks + 1, buf ^ 1);
-                    else load_frags(next, 0, 0);  // after this step's barrier
-#pragma unroll
-                    for (int i = 0; i < TI; i++)
-#pragma unroll
-                        for (int j = 0; j < TJ; j++) {
-                            if constexpr (K4) {
-                                // the first slice of a super-block starts the partial product from zero
-                                part[i][j] = mfma32(fa[buf][i], fb[buf][j], (q == 0 && ks == 0) ? zero16 : part[i][j]);
-                            } else {
-                                total[i][j] = mfma32(fa[buf][i], fb[buf][j], total[i][j]);
-                            }
-                        }
-                    // weights first: the activations were fetched only at the top of this step
-                    if (ks == 0) store_b1(nstep, (q + 1) & 3, 0, next);
-                    if (ks == 1) store_b1(nstep, (q + 1) & 3, 1, next);
-                    if (ks == 2) {
-                        store_a2(next, 0, (q + 1) & 1);
-                        store_a2(next, 2, (q + 1) & 1);
-                    }
-                    // order inside the group: the LDS reads of the next slice, then MFMA / few VALU alternating
-                    __builtin_amdgcn_sched_group_barrier(0x100, TI + TJ, 0);
-#pragma unroll
-                    for (int r = 0; r < 4; r++) {
-                        if (r < TI * TJ) __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                        __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
-                        if (ks == 2) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
-                    }
-                    if (ks < 2) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
-                    __builtin_amdgcn_sched_barrier(0);
-                    if (ks == 2) __syncthreads();
-                }
-                if constexpr (K4) {
-                    if (q == 3) {  // a 256-column super-block is complete: total += d * P - dmin * (mn . sx)
-#pragma unroll
-                        for (int j = 0; j < TJ; j++) {
-                            const uint4_t meta = w_meta[j];
-                            const float d = my_ok[j] ? half_bits_to_float(meta[0] & 0xFFFFu) : 0.f;
-                            const float dmin = my_ok[j] ? half_bits_to_float(meta[0] >> 16) : 0.f;
-                            uint32_t sc[2], mn[2];
-                            q4k_scales(meta[1], meta[2], meta[3], sc, mn);
-                            // B' fragment: half 0 holds mn_0..7, half 1 holds mn_0..7 / 2048 (pairs with the lo sums)
-                            Frag fm;
-                            const half2_t k1024 = {(half_t)1024.0f, (half_t)1024.0f};
-                            const half2_t lo_scale = {(half_t)(1.0f / GEMM_LO_SCALE), (half_t)(1.0f / GEMM_LO_SCALE)};
-#pragma unroll
-                            for (int e = 0; e < 4; e++) {
-                                uint32_t src = (e < 2) ? mn[0] : mn[1];
-                                uint32_t sel = (e & 1) ? 0x04030402u : 0x04010400u;  // bytes (2,3) or (0,1) -> [b,0x64,b',0x64]
-                                half2_t v = as_half2(__builtin_amdgcn_perm(0x64646464u, src, sel)) - k1024;
-                                fm.h2[e] = lh ? v * lo_scale : v;
-                            }
-#pragma unroll
-                            for (int i = 0; i < TI; i++) {
-                                float16_t qq = mfma32(fs[i], fm, zero16);
-#pragma unroll
-                                for (int e = 0; e < 16; e++) {
-                                    total[i][j][e] = __builtin_fmaf(d, part[i][j][e], total[i][j][e]);
-                                    total[i][j][e] = __builtin_fmaf(-dmin, qq[e], total[i][j][e]);
-                                }
-                            }
-                        }
-                    }
-                }
-                rd_off = wr_off;
-                wr_off = wr_off == 2 * ST ? 0 : wr_off + ST;
             }
         }
+    };
+
+    // ---- the two halves of a step ------------------------------------------------------------------------
+    // compute: the sixteen (TI = TJ = 2) MFMAs of one 64-column step.
+    // It also issues, between the MFMAs, the global loads that refill the registers this wave's last data half emptied
+    // (step fstep, phase fq): activations of step fstep + AD and weights of step fstep + 1. Issuing a load can stall a
+    // wave for tens of cycles when the CU's vector-memory queue is full; here that time is MFMA shadow.
+    auto compute = [&](const uint8_t *stage, int q, int fstep, int fq) {
+        const int last = step1 - 1;
+        __builtin_amdgcn_s_setprio(2);
+#pragma unroll
+        for (int ks = 0; ks < 4; ks++) {
+            const int buf = ks % NB;
+            if (ks + PD < 4) load_frags(stage, ks + PD, (ks + PD) % NB);
+            if (ks == 0) fetch_a(min(fstep + AD, last), AD == 2 ? (fq & 1) : 0);
+            if (ks == 1) fetch_b(min(fstep + 1, last), (fq + 1) & 3);
+#pragma unroll
+            for (int i = 0; i < TI; i++)
+#pragma unroll
+                for (int j = 0; j < TJ; j++) {
+                    if constexpr (K4) {
+                        // the first slice of a super-block starts the partial product from zero
+                        part[i][j] = mfma32(fa[buf][i], fb[buf][j], (q == 0 && ks == 0) ? zero16 : part[i][j]);
+                    } else {
+                        total[i][j] = mfma32(fa[buf][i], fb[buf][j], total[i][j]);
+                    }
+                }
+            if (ks + PD < 4) __builtin_amdgcn_sched_group_barrier(0x100, TI + TJ, 0);
+#pragma unroll
+            for (int r = 0; r < TI * TJ; r++) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                if (ks < 2) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        __builtin_amdgcn_s_setprio(0);
+    };
+    // data: this wave's share of the stage of step `dstep` (phase dq = dstep % 4, compile-time): the activation chunks
+    // fetched AD steps ago and two decoded weight blocks; then the global loads that refill those registers.
+    auto data = [&](int dstep, int dq, uint8_t *stage) {
+        const int last = step1 - 1;
+        const int set = AD == 2 ? (dq & 1) : 0;
+        store_a2(stage, 0, set);
+        store_a2(stage, 2, set);
+        store_b1(min(dstep, last), dq, 0, stage);
+        store_b1(min(dstep, last), dq, 1, stage);
+    };
+
+    // Three LDS stages and two wave groups (waves 0-3 and 4-7: one wave of each on every SIMD). Step s is computed
+    // from stage s % 3 by group 0 in the first half of the iteration and by group 1 in the second; the other group
+    // spends that half decoding its share of a later step: group 1 of step s + 1, group 0 of step s + 2, so the stage
+    // either group computes from next is complete one barrier before it is needed and its first fragments are read
+    // ahead. A SIMD always has one wave issuing MFMAs back to back (raised priority) and one doing the VALU / LDS /
+    // global work, instead of two waves that contend for the same slots and then wait for each other.
+    const int grp = wave >> 2;  // wave-uniform
+    if (step0 < step1) {  // step0 is a multiple of 4
+        const int last = step1 - 1;
+        fetch_a(step0, 0);
+        fetch_b(step0, 0);
+        if (AD == 2) fetch_a(min(step0 + 1, last), 1);
+        data(step0, 0, smem);
+        fetch_a(min(step0 + AD, last), 0);
+        fetch_b(min(step0 + 1, last), 1);
+        if (grp == 0) data(step0 + 1, 1, smem + ST);
     }
+    __syncthreads();
+    // The two groups run separate copies of the loop (the branch is outside it), so the accumulators of each stay
+    // in place; the hardware barrier only counts arrivals, and both copies arrive twice per step.
+    auto run = [&](auto group) {
+        constexpr int GRP = decltype(group)::value;
+        int s0 = 0, s1 = ST, s2 = 2 * ST;  // stage of this step, the next, the one after
+        if constexpr (GRP == 0) {
+            if (step0 < step1) preload(smem);
+        }
+        for (int sbase = step0; sbase < step1; sbase += 4) {
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const int step = sbase + q;
+                if (step < step1) {
+                    if constexpr (GRP == 0) {
+                        compute(smem + s0, q, step + 1, (q + 1) & 3);
+                        __syncthreads();
+                        preload(smem + s1);
+                        data(step + 2, (q + 2) & 3, smem + s2);
+                        if constexpr (K4) {
+                            if (q == 1) load_sb_meta(step >> 2);
+                            if (q == 3) scale_sb();
+                        }
+                        __syncthreads();
+                    } else {
+                        preload(smem + s0);
+                        data(step + 1, (q + 1) & 3, smem + s1);
+                        if constexpr (K4) {
+                            if (q == 1) load_sb_meta(step >> 2);
+                            if (q == 0 && step > step0) scale_sb();  // the super-block finished in the last iteration
+                        }
+                        __syncthreads();
+                        compute(smem + s0, q, step + 1, (q + 1) & 3);
+                        __syncthreads();
+                    }
+                    const int t = s0;
+                    s0 = s1;
+                    s1 = s2;
+                    s2 = t;
+                }
+            }
+        }
+        if constexpr (K4 && GRP == 1) {
+            if (step0 < step1) scale_sb();
+        }
+    };
+    if (grp == 0) run(std::integral_constant<int, 0>{});
+    else run(std::integral_constant<int, 1>{});
 
     // ---- epilogue: register e of tile (i, j) is row 8 (e/4) + 4 lh + e%4, column lr ------------------------
 #pragma unroll
@@ -430,7 +476,7 @@ __device__ __forceinline__ void xprep_body(const XPrepArgs &a) {
 extern "C" __global__ __launch_bounds__(512) void rlx_gemm_q4_k(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q4K, 2, 2>(a); }
 extern "C" __global__ __launch_bounds__(512) void rlx_gemm_q4_0(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q4_0, 2, 2>(a); }
 extern "C" __global__ __launch_bounds__(512) void rlx_gemm_q8_0(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q8_0, 2, 2>(a); }
-extern "C" __global__ __launch_bounds__(512) void rlx_gemm64_q4_k(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q4K, 1, 1>(a); }
-extern "C" __global__ __launch_bounds__(512) void rlx_gemm64_q4_0(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q4_0, 1, 1>(a); }
-extern "C" __global__ __launch_bounds__(512) void rlx_gemm64_q8_0(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q8_0, 1, 1>(a); }
+extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64_q4_k(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q4K, 1, 1>(a); }
+extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64_q4_0(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q4_0, 1, 1>(a); }
+extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64_q8_0(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q8_0, 1, 1>(a); }
 extern "C" __global__ __launch_bounds__(256) void rlx_xprep(rlx::XPrepArgs a) { rlx::xprep_body(a); }
