@@ -31,7 +31,7 @@ struct GemvSeg {
     const uint8_t *w;
     const void *x;
     float *out;
-    int n, k, row_tiles, units, wg_begin, tiles_per_wg;
+    int n, k, row_tiles, units, wg_begin, tiles_per_wg, tile_stride;
 };
 struct GemvArgs {
     GemvSeg seg[GEMV_MAX_SEG];
@@ -133,8 +133,11 @@ static int launch_gemv(const void *const *xs, int xk, const rlx_qweight *const *
             int tpw = (int)std::max<long long>(1, (target_items + D.units / 2) / D.units);
             tpw = std::min(tpw, tpw_cap);
             max_tpw = std::max(max_tpw, tpw);
-            sh.a.seg[i] = GemvSeg{ws[i]->dev, xs[i], outs[i], (int)D.n, (int)D.k, (int)D.row_tiles, (int)D.units, sh.wg, tpw};
-            sh.wg += (int)((D.row_tiles + tpw - 1) / tpw);
+            const int seg_wgs = (int)((D.row_tiles + tpw - 1) / tpw);
+            static const bool contiguous = getenv("RLX_GEMV_CONTIGUOUS") != nullptr;
+            sh.a.seg[i] = GemvSeg{ws[i]->dev, xs[i], outs[i], (int)D.n, (int)D.k, (int)D.row_tiles, (int)D.units, sh.wg, tpw,
+                                  contiguous ? 1 : seg_wgs};
+            sh.wg += seg_wgs;
         }
         const size_t part_bytes = (size_t)max_tpw * sh.nwaves * slot_bytes;
         sh.kcu = max_units;

@@ -29,6 +29,7 @@ struct GemvSeg {
     int units;         // K units in its device layout
     int wg_begin;      // first workgroup of this segment
     int tiles_per_wg;  // row tiles per workgroup
+    int tile_stride;   // distance between a workgroup's tiles: 1 = a contiguous run, else the segment's workgroup count
 };
 
 struct GemvArgs {
@@ -58,8 +59,8 @@ struct UnitRegs<SCHEME_Q4_0> {
     uint2_t s;
     // `meta` is false for lanes whose accumulators hold no real row: they skip the scale load
     __device__ __forceinline__ void load(const uint8_t *unit, int l, int nrow, bool meta) {
-        q = *(const uint4_t *)(unit + l * 16);
-        if (meta) s = *(const uint2_t *)(unit + 1024 + nrow * 8);
+        q = __builtin_nontemporal_load((const uint4_t *)(unit + l * 16));
+        if (meta) s = __builtin_nontemporal_load((const uint2_t *)(unit + 1024 + nrow * 8));
     }
     __device__ __forceinline__ void clear() {
         q = uint4_t{0, 0, 0, 0};
@@ -71,9 +72,9 @@ struct UnitRegs<SCHEME_Q8_0> {
     uint4_t q0, q1;
     uint2_t s;
     __device__ __forceinline__ void load(const uint8_t *unit, int l, int nrow, bool meta) {
-        q0 = *(const uint4_t *)(unit + l * 16);
-        q1 = *(const uint4_t *)(unit + 1024 + l * 16);
-        if (meta) s = *(const uint2_t *)(unit + 2048 + nrow * 8);
+        q0 = __builtin_nontemporal_load((const uint4_t *)(unit + l * 16));
+        q1 = __builtin_nontemporal_load((const uint4_t *)(unit + 1024 + l * 16));
+        if (meta) s = __builtin_nontemporal_load((const uint2_t *)(unit + 2048 + nrow * 8));
     }
     __device__ __forceinline__ void clear() {
         q0 = q1 = uint4_t{0, 0, 0, 0};
@@ -84,9 +85,9 @@ template <>
 struct UnitRegs<SCHEME_Q4K> {
     uint4_t q0, q1, meta;
     __device__ __forceinline__ void load(const uint8_t *unit, int l, int nrow, bool want_meta) {
-        q0 = *(const uint4_t *)(unit + l * 16);
-        q1 = *(const uint4_t *)(unit + 1024 + l * 16);
-        if (want_meta) meta = *(const uint4_t *)(unit + 2048 + nrow * 16);
+        q0 = __builtin_nontemporal_load((const uint4_t *)(unit + l * 16));
+        q1 = __builtin_nontemporal_load((const uint4_t *)(unit + 1024 + l * 16));
+        if (want_meta) meta = __builtin_nontemporal_load((const uint4_t *)(unit + 2048 + nrow * 16));
     }
     __device__ __forceinline__ void clear() { q0 = q1 = meta = uint4_t{0, 0, 0, 0}; }  // d = dmin = 0
 };
@@ -266,8 +267,11 @@ __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
         e = e < 0 ? 0 : (e >= a.num_experts ? a.num_experts - 1 : e);
         seg.w += (long long)e * a.slab_bytes;
     }
-    const int tile0 = ((int)blockIdx.x - seg.wg_begin) * seg.tiles_per_wg;
-    const int ntiles = min(seg.tiles_per_wg, seg.row_tiles - tile0);
+    // Workgroup lw of a segment owns tiles tile0 + t * tstride: interleaved (tile0 = lw, tstride = workgroups of the
+    // segment), so at any moment the whole grid reads one moving window of the matrix rather than hundreds of streams.
+    const int tstride = seg.tile_stride;
+    const int tile0 = ((int)blockIdx.x - seg.wg_begin) * (tstride == 1 ? seg.tiles_per_wg : 1);
+    const int ntiles = tile0 < seg.row_tiles ? min(seg.tiles_per_wg, (seg.row_tiles - tile0 + tstride - 1) / tstride) : 0;
     const int kc_units = min(a.kc_units, seg.units);
 
     const int kc = kc_units * L.unit_k;
@@ -283,7 +287,7 @@ __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
     for (int i = tid; i < ntiles * nwaves * slot_floats; i += blockDim.x) part[i] = 0.f;
 
     const uint8_t *wbase = seg.w + (long long)tile0 * seg.units * L.unit_bytes;
-    const long long tile_bytes = (long long)seg.units * L.unit_bytes;
+    const long long tile_bytes = (long long)seg.units * L.unit_bytes * tstride;  // to this workgroup's next tile
 
     for (int u0 = 0; u0 < seg.units; u0 += kc_units) {
         const int nu = min(kc_units, seg.units - u0);  // units in this chunk
@@ -372,7 +376,7 @@ __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
             sum += slot[mr * 16];
             if (a.x_dtype == X_F32) sum += slot[(a.m + mr) * 16] * (1.0f / LO_SCALE);
         }
-        const int n_out = (tile0 + t) * 16 + col;
+        const int n_out = (tile0 + t * tstride) * 16 + col;
         if (n_out < seg.n) seg.out[(long long)mr * seg.n + n_out] = sum;
     }
 }
