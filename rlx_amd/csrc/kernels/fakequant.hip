@@ -58,7 +58,7 @@ __device__ __forceinline__ void col_absmax(const FqArgs &a) {
     const float *p = a.x + r0 * a.chan_dim + c4;
 #pragma unroll 8
     for (long long r = r0; r < r1; r++, p += a.chan_dim) {
-        float4_t v = *(const float4_t *)p;
+        float4_t v = *(const float4_t *)p;  // ordinary load: the apply pass finds most of x in the last-level cache
         float a0 = __builtin_fabsf(v[0]), a1 = __builtin_fabsf(v[1]), a2 = __builtin_fabsf(v[2]), a3 = __builtin_fabsf(v[3]);
         m0 = a0 > m0 ? a0 : m0;
         m1 = a1 > m1 ? a1 : m1;
@@ -193,14 +193,14 @@ __device__ __forceinline__ void col_apply(const FqArgs &a) {
     int8_t *cd = a.codes ? a.codes + base : nullptr;
 #pragma unroll 4
     for (long long r = r0; r < r1; r++, p += a.chan_dim, o += a.chan_dim) {
-        float4_t v = *(const float4_t *)p;
+        float4_t v = __builtin_nontemporal_load((const float4_t *)p);  // last use of x; out is not read back here
         float4_t q, y;
 #pragma unroll
         for (int e = 0; e < 4; e++) {
             q[e] = fq_code(v[e], s[e], a.q_max, a.round_mode);
             y[e] = q[e] * s[e];
         }
-        *(float4_t *)o = y;
+        __builtin_nontemporal_store(y, (float4_t *)o);
         if (cd) {
             uint32_t packed = (uint32_t)(uint8_t)fq_i8(q[0]) | ((uint32_t)(uint8_t)fq_i8(q[1]) << 8) |
                               ((uint32_t)(uint8_t)fq_i8(q[2]) << 16) | ((uint32_t)(uint8_t)fq_i8(q[3]) << 24);
@@ -230,13 +230,13 @@ __device__ __forceinline__ void flat4_apply(const FqArgs &a) {
         long long i = i4 * 4;
         long long c = a.chan_dim == 1 ? 0 : (i / a.inner) % a.chan_dim;
         float s = a.scale[c];
-        float4_t v = *(const float4_t *)(a.x + i), q, y;
+        float4_t v = __builtin_nontemporal_load((const float4_t *)(a.x + i)), q, y;
 #pragma unroll
         for (int e = 0; e < 4; e++) {
             q[e] = fq_code(v[e], s, a.q_max, a.round_mode);
             y[e] = q[e] * s;
         }
-        *(float4_t *)(a.out + i) = y;
+        __builtin_nontemporal_store(y, (float4_t *)(a.out + i));
         if (a.codes) {
             uint32_t packed = (uint32_t)(uint8_t)fq_i8(q[0]) | ((uint32_t)(uint8_t)fq_i8(q[1]) << 8) |
                               ((uint32_t)(uint8_t)fq_i8(q[2]) << 16) | ((uint32_t)(uint8_t)fq_i8(q[3]) << 24);
