@@ -300,7 +300,7 @@ __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
         UnitRegs<SCHEME> ring[DEPTH];
         auto prefetch = [&](UnitRegs<SCHEME> &slot) {
             if (pf_n < nitems) {
-                slot.load(pf_ptr, l, nrow, has_rows);
+                slot.load(pf_ptr, l, nrow, true);  // every lane loads its column's scales (lanes 16-63 repeat lanes 0-15)
                 pf_n++;
                 pf_u += nwaves;
                 pf_ptr += (long long)nwaves * L.unit_bytes;
