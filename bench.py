@@ -289,6 +289,31 @@ def extra_configs(rlx_amd, stream):
                                   "frac_hbm": round(b / ms / 1e6 / HBM_PEAK_GBS, 4)}
     for q in qws:
         q.free()
+    # a wide scheme: Q6_K gate/up projection [14336, 4096], resident as binary16 (117 MB per copy, four copies rotated)
+    n, k = 14336, 4096
+    rng = np.random.default_rng(5)
+    blocks = rng.integers(0, 256, (n * k // 256, 210), dtype=np.uint8)
+    blocks[:, 208:210] = np.full(n * k // 256, 5e-6, np.float16).view(np.uint8).reshape(-1, 2)  # weights of a few hundredths
+    copies = 4
+    qws = [ops.QWeight(QuantScheme.GgufQ6K, blocks.reshape(-1), n, k) for _ in range(copies)]
+    del blocks
+    x = ops.DeviceBuffer.from_numpy(ops.philox_normal(8, k))
+    y = ops.DeviceBuffer(n * 4)
+    state = {"i": 0}
+
+    def fn6():
+        q = qws[state["i"] % copies]
+        state["i"] += 1
+        rlx_amd._lib.check(L.rlx_mi355x_gguf_matmul_bt(x.ptr, int(DType.F32), q.ptr, y.ptr, 1, None, 0, stream))
+
+    ms = time_launches(ops, stream, fn6, 200, 20)
+    resident = qws[0].device_bytes() + 4 * k + 4 * n
+    out["q6_k_gemv_gate/up_resident_f16"] = {"us": round(ms * 1e3, 3), "GB/s_resident": round(resident / ms / 1e6, 1),
+                                             "frac_hbm_resident": round(resident / ms / 1e6 / HBM_PEAK_GBS, 4),
+                                             "GB/s_packed_equivalent": round((n * k // 256 * 210 + 4 * k + 4 * n) / ms / 1e6, 1),
+                                             "note": "wide schemes are decoded at upload and stream 2 bytes per weight with no decode arithmetic"}
+    for q in qws:
+        q.free()
     # config 4: FakeQuantize [8192, 4096], int8 per column, heavy-tailed input; three input / output sets in rotation
     # (3 x 268 MB) so that no launch finds its input in the 256 MB last-level cache
     rows, cols = 8192, 4096

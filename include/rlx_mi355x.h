@@ -44,10 +44,19 @@ typedef enum rlx_dtype {
     RLX_I32 = 6, RLX_I64 = 7, RLX_U8 = 8, RLX_U32 = 9, RLX_BOOL = 10, RLX_C64 = 11
 } rlx_dtype;
 
-/* rlx_ir::quant::QuantScheme, declaration order (rlx-ir/src/quant.rs:39-79). Only the three
- * GGUF schemes below are claimed; any other value is RLX_ERR_UNSUPPORTED. */
+/* rlx_ir::quant::QuantScheme, declaration order (rlx-ir/src/quant.rs:39-79). The eight GGUF schemes the reference's
+ * gguf_matmul_bt dispatches (rlx-cpu/src/gguf_matmul.rs:25-37) are claimed; any other value is RLX_ERR_UNSUPPORTED.
+ * Q4_K, Q4_0 and Q8_0 stay packed in HBM and have a bit-exact device decoder. The other five ("wide") are decoded once
+ * at upload with the reference's block decoder and kept as binary16 (2 bytes per weight): matmuls only, every decoded
+ * weight must fit binary16, and Q6_K scale bytes are read as the reference's block decoder reads them, unsigned
+ * (rlx-gguf/src/lib.rs:819-845), unless the environment variable RLX_Q6K_SIGNED_SCALES is set (ggml's reading). */
 typedef enum rlx_quant_scheme {
     RLX_SCHEME_GGUF_Q4K = 5,  /* 256 elems / 144 bytes */
+    RLX_SCHEME_GGUF_Q5K = 6,  /* 256 / 176, wide */
+    RLX_SCHEME_GGUF_Q6K = 7,  /* 256 / 210, wide */
+    RLX_SCHEME_GGUF_Q8K = 8,  /* 256 / 292, wide */
+    RLX_SCHEME_GGUF_Q2K = 9,  /* 256 / 84, wide (field order of rlx-gguf/src/lib.rs:857-886) */
+    RLX_SCHEME_GGUF_Q3K = 10, /* 256 / 110, wide (field order of rlx-gguf/src/lib.rs:889-930) */
     RLX_SCHEME_GGUF_Q4_0 = 11, /* 32 elems / 18 bytes  */
     RLX_SCHEME_GGUF_Q8_0 = 12  /* 32 elems / 34 bytes  */
 } rlx_quant_scheme;
@@ -95,8 +104,8 @@ int rlx_mi355x_event_elapsed_ms(void *start, void *stop, float *ms); /* synchron
  * Format constants (rlx-ir/src/quant.rs:138-183, rlx-gguf/src/lib.rs:377-419)
  * ---------------------------------------------------------------------------------------- */
 
-int rlx_mi355x_block_elems(int scheme);            /* QuantScheme::gguf_block_size(): 32 / 32 / 256, else 0 */
-int rlx_mi355x_block_bytes(int scheme);            /* QuantScheme::gguf_block_bytes(): 18 / 34 / 144, else 0 */
+int rlx_mi355x_block_elems(int scheme);            /* QuantScheme::gguf_block_size(): 32 (Q4_0, Q8_0) / 256 (K-quants), else 0 */
+int rlx_mi355x_block_bytes(int scheme);            /* QuantScheme::gguf_block_bytes(): 18 / 34 / 144 / 176 / 210 / 292 / 84 / 110, else 0 */
 int64_t rlx_mi355x_bytes_for(int scheme, int64_t n_elems); /* rlx_gguf bytes_for: -1 if n % block != 0 */
 
 /* ------------------------------------------------------------------------------------------
@@ -104,8 +113,8 @@ int64_t rlx_mi355x_bytes_for(int scheme, int64_t n_elems); /* rlx_gguf bytes_for
  * ---------------------------------------------------------------------------------------- */
 
 /* A GGUF-packed [n, k] matrix (row-major, blocks along k: rlx-cpu/src/gguf_matmul.rs:15-20) repacked once
- * into the device layout the kernels stream (same byte count per block; 16-row x 64/256-k units whose
- * 16-byte lane slots hold MFMA operand fragments). */
+ * into the device layout the kernels stream (same byte count per block; 16-row x 128/256-k units whose
+ * 16-byte lane slots hold MFMA operand fragments; wide schemes: binary16 fragments, 2 bytes per weight). */
 typedef struct rlx_qweight rlx_qweight;
 
 /* Repack `gguf_bytes` (host, exactly bytes_for(scheme, n*k) long) and upload. Where the reference memcpy's the
@@ -122,7 +131,8 @@ size_t rlx_mi355x_qweight_device_bytes_for(int scheme, int64_t n, int64_t k);
 int rlx_mi355x_repack_host(int scheme, const void *gguf_bytes, size_t nbytes, int64_t n, int64_t k, void *out);
 
 /* rlx_gguf::dequant_q8_0 / dequant_q4_0 / dequant_q4_k (rlx-gguf/src/lib.rs:600-633,974-1013) on the device:
- * out_dev[n*k] f32, row-major [n,k], bit-identical to the reference decoders. */
+ * out_dev[n*k] f32, row-major [n,k], bit-identical to the reference decoders. RLX_ERR_UNSUPPORTED for the wide
+ * schemes (the exact f32 decode is not kept on the device). */
 int rlx_mi355x_dequant(const rlx_qweight *w, float *out_dev, void *stream);
 
 /* rlx_cpu::gguf_matmul::gguf_matmul_bt (rlx-cpu/src/gguf_matmul.rs:40-95):

@@ -12,7 +12,7 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _SO = os.path.join(_HERE, "librlx_oracle.so")
 
-Q4K, Q4_0, Q8_0 = 5, 11, 12
+Q4K, Q5K, Q6K, Q8K, Q2K, Q3K, Q4_0, Q8_0 = 5, 6, 7, 8, 9, 10, 11, 12
 PER_BATCH, EMA, FIXED = 0, 1, 2
 HALF_AWAY, HALF_EVEN = 0, 1
 M0_REFERENCE = 0xD2561A75
@@ -49,6 +49,8 @@ def lib():
         L.orc_get_scale_min_k4.argtypes = [C.c_int, u8p, u8p, u8p]
         L.orc_dequant.restype = C.c_int
         L.orc_dequant.argtypes = [C.c_int, u8p, C.c_int64, C.c_int64, f32p]
+        L.orc_dequant_matmul_blocks.restype = C.c_int
+        L.orc_dequant_matmul_blocks.argtypes = [C.c_int, u8p, C.c_int64, C.c_int64, f32p]
         L.orc_gguf_grouped_matmul_bt.restype = C.c_int
         L.orc_gguf_grouped_matmul_bt.argtypes = [f32p, u8p, C.c_int64, f32p, f32p, C.c_int64, C.c_int64, C.c_int64, C.c_int64, C.c_int]
         L.orc_gguf_matmul_bt.restype = C.c_int
@@ -118,6 +120,17 @@ def dequant(scheme, packed, n):
     rc = lib().orc_dequant(scheme, _p(packed, C.c_uint8), packed.size, n, _p(out, C.c_float))
     if rc != 0:
         raise ValueError(f"dequant: bad size (scheme={scheme}, n={n}, bytes={packed.size})")
+    return out
+
+
+def dequant_matmul_blocks(scheme, packed, n):
+    """Decode with the per-block decoders the reference's matmul dispatches to (rlx-cpu/src/gguf_matmul.rs:25-37).
+    Same as `dequant` except for Q6_K, whose block decoder reads the scale bytes as unsigned."""
+    packed = np.ascontiguousarray(packed, dtype=np.uint8)
+    out = np.empty(n, dtype=np.float32)
+    rc = lib().orc_dequant_matmul_blocks(scheme, _p(packed, C.c_uint8), packed.size, n, _p(out, C.c_float))
+    if rc != 0:
+        raise ValueError(f"dequant_matmul_blocks: bad size (scheme={scheme}, n={n}, bytes={packed.size})")
     return out
 
 

@@ -13,6 +13,12 @@
  *   Q8_0 / Q4_0 / Q4_K    the reference's own known-answer blocks
  *                         (rlx-gguf/src/lib.rs:1187-1264) + independent numpy
  *                         bit-field restatements on random bytes
+ *   Q5_K                  reduces to the pinned Q4_K decoder when the fifth-bit plane is zero; a set bit adds exactly
+ *                         16 * d * sc at the position the format fixes (closed form), random bytes vs numpy
+ *   Q6_K / Q2_K / Q3_K / Q8_K  the reference's known-answer blocks (rlx-gguf/src/lib.rs:1266-1334) + one-hot
+ *                         position probes against the closed-form index map of each format + numpy on random bytes;
+ *                         Q6_K in both scale readings (block decoder unsigned, lib.rs:819-845; tensor decoder i8,
+ *                         lib.rs:1070-1112)
  *   gguf_matmul_bt        reference tests rlx-cpu/src/gguf_matmul.rs:238-277 and
  *                         rlx-runtime/tests/dequant_matmul_gguf.rs:176-308
  *                         (layout idx = j*k + p), f64 dense matmul (textbook)
@@ -40,7 +46,7 @@
 #define K_SCALE_SIZE 12
 
 /* scheme ids shared with include/rlx_mi355x.h (rlx-ir/src/quant.rs:39-79 order) */
-enum { ORC_Q4K = 5, ORC_Q4_0 = 11, ORC_Q8_0 = 12 };
+enum { ORC_Q4K = 5, ORC_Q5K = 6, ORC_Q6K = 7, ORC_Q8K = 8, ORC_Q2K = 9, ORC_Q3K = 10, ORC_Q4_0 = 11, ORC_Q8_0 = 12 };
 
 /* ---- half / bfloat16 -------------------------------------------------- */
 
@@ -123,7 +129,12 @@ float orc_bf16_to_f32(uint16_t h) {
 
 int orc_block_elems(int scheme) {
     switch (scheme) {
-    case ORC_Q4K: return QK_K;
+    case ORC_Q4K:
+    case ORC_Q5K:
+    case ORC_Q6K:
+    case ORC_Q8K:
+    case ORC_Q2K:
+    case ORC_Q3K: return QK_K;
     case ORC_Q4_0: return QK4_0;
     case ORC_Q8_0: return QK8_0;
     default: return 0;
@@ -133,6 +144,11 @@ int orc_block_elems(int scheme) {
 int orc_block_bytes(int scheme) {
     switch (scheme) {
     case ORC_Q4K: return 2 + 2 + K_SCALE_SIZE + QK_K / 2; /* 144 */
+    case ORC_Q5K: return 2 + 2 + K_SCALE_SIZE + QK_K / 8 + QK_K / 2; /* 176 */
+    case ORC_Q6K: return QK_K / 2 + QK_K / 4 + QK_K / 16 + 2;       /* 210 */
+    case ORC_Q8K: return 4 + QK_K + (QK_K / 16) * 2;                /* 292 */
+    case ORC_Q2K: return 2 + 2 + QK_K / 16 + QK_K / 4;              /* 84 */
+    case ORC_Q3K: return 2 + K_SCALE_SIZE + QK_K / 8 + QK_K / 4;    /* 110 */
     case ORC_Q4_0: return 2 + QK4_0 / 2;                  /* 18 */
     case ORC_Q8_0: return 2 + QK8_0;                      /* 34 */
     default: return 0;
@@ -211,18 +227,182 @@ void orc_dequant_q4_k_block(const uint8_t *block, float *out) {
     }
 }
 
+/* rlx-gguf/src/lib.rs:783-816 */
+void orc_dequant_q5_k_block(const uint8_t *block, float *out) {
+    float d = read_f16_le(block);
+    float dmin = read_f16_le(block + 2);
+    const uint8_t *scales = block + 4;
+    const uint8_t *qh = block + 4 + K_SCALE_SIZE;
+    const uint8_t *qs = block + 4 + K_SCALE_SIZE + QK_K / 8;
+    int is = 0, oi = 0;
+    uint8_t u1 = 1, u2 = 2;
+    for (int j = 0; j < 8; j += 2) {
+        uint8_t sc0, m0, sc1, m1;
+        orc_get_scale_min_k4(j, scales, &sc0, &m0);
+        orc_get_scale_min_k4(j + 1, scales, &sc1, &m1);
+        float d0 = d * (float)sc0;
+        float m0f = dmin * (float)m0;
+        float d1 = d * (float)sc1;
+        float m1f = dmin * (float)m1;
+        for (int l = 0; l < 32; l++) {
+            uint8_t lo = qs[is + l] & 0x0F;
+            uint8_t hi = (qh[l] & u1) ? 16 : 0;
+            float t = d0 * (float)(uint8_t)(lo + hi);
+            out[oi++] = t - m0f;
+        }
+        for (int l = 0; l < 32; l++) {
+            uint8_t lo = qs[is + l] >> 4;
+            uint8_t hi = (qh[l] & u2) ? 16 : 0;
+            float t = d1 * (float)(uint8_t)(lo + hi);
+            out[oi++] = t - m1f;
+        }
+        is += 32;
+        u1 <<= 2;
+        u2 <<= 2;
+    }
+}
+
+/* rlx-gguf/src/lib.rs:819-845 (signed_scales = 0): the block decoder the matmul calls converts the sixteen scale bytes
+ * as unsigned. rlx-gguf/src/lib.rs:1070-1112 (signed_scales = 1): the whole-tensor decoder reads them as i8. */
+void orc_dequant_q6_k_block(const uint8_t *block, float *out, int signed_scales) {
+    const int ql_len = QK_K / 2, qh_len = QK_K / 4, sc_len = QK_K / 16;
+    const uint8_t *ql = block, *qh = block + ql_len, *sc = block + ql_len + qh_len;
+    float d = read_f16_le(block + ql_len + qh_len + sc_len);
+    for (int h = 0; h < 2; h++) {
+        int dst_base = h * 128, ql_off = h * 64, qh_off_h = h * 32, sc_off = h * 8;
+        for (int l = 0; l < 32; l++) {
+            int is = l / 16;
+            uint8_t qh_b = qh[qh_off_h + l];
+            int32_t q1 = (int32_t)(uint8_t)((ql[ql_off + l] & 0x0F) | ((qh_b & 3) << 4)) - 32;
+            int32_t q2 = (int32_t)(uint8_t)((ql[ql_off + l + 32] & 0x0F) | (((qh_b >> 2) & 3) << 4)) - 32;
+            int32_t q3 = (int32_t)(uint8_t)((ql[ql_off + l] >> 4) | (((qh_b >> 4) & 3) << 4)) - 32;
+            int32_t q4 = (int32_t)(uint8_t)((ql[ql_off + l + 32] >> 4) | (((qh_b >> 6) & 3) << 4)) - 32;
+            float s1 = signed_scales ? (float)(int8_t)sc[sc_off + is] : (float)sc[sc_off + is];
+            float s2 = signed_scales ? (float)(int8_t)sc[sc_off + is + 2] : (float)sc[sc_off + is + 2];
+            float s3 = signed_scales ? (float)(int8_t)sc[sc_off + is + 4] : (float)sc[sc_off + is + 4];
+            float s4 = signed_scales ? (float)(int8_t)sc[sc_off + is + 6] : (float)sc[sc_off + is + 6];
+            float t1 = d * s1, t2 = d * s2, t3 = d * s3, t4 = d * s4;
+            out[dst_base + l] = t1 * (float)q1;
+            out[dst_base + l + 32] = t2 * (float)q2;
+            out[dst_base + l + 64] = t3 * (float)q3;
+            out[dst_base + l + 96] = t4 * (float)q4;
+        }
+    }
+}
+
+/* rlx-gguf/src/lib.rs:848-854 */
+void orc_dequant_q8_k_block(const uint8_t *block, float *out) {
+    float d;
+    memcpy(&d, block, 4);
+    const uint8_t *qs = block + 4;
+    for (int i = 0; i < QK_K; i++) out[i] = d * (float)(int8_t)qs[i];
+}
+
+/* rlx-gguf/src/lib.rs:857-886 */
+void orc_dequant_q2_k_block(const uint8_t *block, float *out) {
+    float d = read_f16_le(block);
+    float mn = read_f16_le(block + 2);
+    const uint8_t *q = block + 4 + QK_K / 16;
+    int is = 0, oi = 0;
+    for (int n = 0; n < QK_K / 128; n++) {
+        unsigned shift = 0;
+        for (int j = 0; j < 4; j++) {
+            uint8_t sc = block[4 + is];
+            is++;
+            float dl = d * (float)(sc & 0xF);
+            float ml = mn * (float)(sc >> 4);
+            for (int l = 0; l < 16; l++) {
+                float t = dl * (float)((q[l] >> shift) & 3);
+                out[oi++] = t - ml;
+            }
+            sc = block[4 + is];
+            is++;
+            dl = d * (float)(sc & 0xF);
+            ml = mn * (float)(sc >> 4);
+            for (int l = 0; l < 16; l++) {
+                float t = dl * (float)((q[l + 16] >> shift) & 3);
+                out[oi++] = t - ml;
+            }
+            shift += 2;
+        }
+        q += 32;
+    }
+}
+
+/* rlx-gguf/src/lib.rs:889-930 */
+void orc_dequant_q3_k_block(const uint8_t *block, float *out) {
+    const uint32_t KMASK1 = 0x03030303u, KMASK2 = 0x0f0f0f0fu;
+    float d_all = read_f16_le(block);
+    const uint8_t *hm = block + 2 + K_SCALE_SIZE;
+    const uint8_t *q = block + 2 + K_SCALE_SIZE + QK_K / 8;
+    uint32_t aux[4];
+    memcpy(&aux[0], block + 2, 4); /* little-endian host, as u32::from_le_bytes */
+    memcpy(&aux[1], block + 6, 4);
+    memcpy(&aux[2], block + 10, 4);
+    uint32_t tmp = aux[2];
+    aux[2] = ((aux[0] >> 4) & KMASK2) | (((tmp >> 4) & KMASK1) << 4);
+    aux[3] = ((aux[1] >> 4) & KMASK2) | (((tmp >> 6) & KMASK1) << 4);
+    aux[0] = (aux[0] & KMASK2) | ((tmp & KMASK1) << 4);
+    aux[1] = (aux[1] & KMASK2) | (((tmp >> 2) & KMASK1) << 4);
+    int8_t scales[16];
+    memcpy(scales, aux, 16);
+    int is = 0, oi = 0;
+    uint8_t m = 1;
+    for (int n = 0; n < QK_K / 128; n++) {
+        unsigned shift = 0;
+        for (int j = 0; j < 4; j++) {
+            float dl = d_all * (float)(int8_t)(scales[is] - 32);
+            is++;
+            for (int l = 0; l < 16; l++) {
+                int8_t h = (hm[l] & m) ? 0 : 4;
+                out[oi++] = dl * (float)(int8_t)((int8_t)((q[l] >> shift) & 3) - h);
+            }
+            dl = d_all * (float)(int8_t)(scales[is] - 32);
+            is++;
+            for (int l = 0; l < 16; l++) {
+                int8_t h = (hm[l + 16] & m) ? 0 : 4;
+                out[oi++] = dl * (float)(int8_t)((int8_t)((q[l + 16] >> shift) & 3) - h);
+            }
+            shift += 2;
+            m <<= 1;
+        }
+        q += 32;
+    }
+}
+
 /* rlx-cpu/src/gguf_matmul.rs:25-37 */
 static void dequant_block(int scheme, const uint8_t *block, float *out) {
     switch (scheme) {
     case ORC_Q4K: orc_dequant_q4_k_block(block, out); break;
+    case ORC_Q5K: orc_dequant_q5_k_block(block, out); break;
+    case ORC_Q6K: orc_dequant_q6_k_block(block, out, 0); break;
+    case ORC_Q8K: orc_dequant_q8_k_block(block, out); break;
+    case ORC_Q2K: orc_dequant_q2_k_block(block, out); break;
+    case ORC_Q3K: orc_dequant_q3_k_block(block, out); break;
     case ORC_Q4_0: orc_dequant_q4_0_block(block, out); break;
     case ORC_Q8_0: orc_dequant_q8_0_block(block, out); break;
     default: break;
     }
 }
 
-/* Whole-tensor forms (rlx-gguf/src/lib.rs:600-633, 974-1013). Returns 0, or -1 on a bad size. */
+/* Whole-tensor forms (rlx-gguf/src/lib.rs:600-633, 932-1145). Returns 0, or -1 on a bad size. */
 int orc_dequant(int scheme, const uint8_t *bytes, int64_t nbytes, int64_t n, float *out) {
+    int be = orc_block_elems(scheme), bb = orc_block_bytes(scheme);
+    if (be == 0 || n % be != 0) return -1;
+    int64_t nb = n / be;
+    if (nbytes != nb * bb) return -1;
+    float tmp[QK_K];
+    for (int64_t i = 0; i < nb; i++) {
+        if (scheme == ORC_Q6K) orc_dequant_q6_k_block(bytes + i * bb, tmp, 1); /* lib.rs:1070-1112 reads the scales as i8 */
+        else dequant_block(scheme, bytes + i * bb, tmp);
+        memcpy(out + i * be, tmp, (size_t)be * sizeof(float));
+    }
+    return 0;
+}
+
+/* The same, with the block decoders the matmul dispatches to (rlx-cpu/src/gguf_matmul.rs:25-37): differs from
+ * orc_dequant only for Q6_K (scale bytes read as unsigned). */
+int orc_dequant_matmul_blocks(int scheme, const uint8_t *bytes, int64_t nbytes, int64_t n, float *out) {
     int be = orc_block_elems(scheme), bb = orc_block_bytes(scheme);
     if (be == 0 || n % be != 0) return -1;
     int64_t nb = n / be;

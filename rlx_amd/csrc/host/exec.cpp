@@ -226,8 +226,8 @@ rlx_exec *rlx_mi355x_compile(const rlx_graph_desc *g, const rlx_compile_opts *op
             e->params[nd.name] = i;
             break;
         case RLX_OP_DEQUANT_MATMUL: {
-            if (layout_of((int)nd.d.scheme).unit_k == 0) {
-                set_error("compile: node %u: DequantMatMul scheme %u is not claimed (GGUF Q4_K=5, Q4_0=11, Q8_0=12)", i,
+            if (layout_of((int)nd.d.scheme).block_elems == 0) {
+                set_error("compile: node %u: DequantMatMul scheme %u is not claimed (GGUF Q4_K=5 .. Q3_K=10, Q4_0=11, Q8_0=12)", i,
                           nd.d.scheme);
                 return nullptr;
             }
@@ -271,8 +271,8 @@ rlx_exec *rlx_mi355x_compile(const rlx_graph_desc *g, const rlx_compile_opts *op
         }
         case RLX_OP_DEQUANT_GROUPED_MATMUL: {  // [x [m,k], packed expert stack, expert_idx [m]] -> [m, n]
             Layout L = layout_of((int)nd.d.scheme);
-            if (L.unit_k == 0) {
-                set_error("compile: node %u: DequantGroupedMatMul scheme %u is not claimed (GGUF Q4_K=5, Q4_0=11, Q8_0=12)", i,
+            if (L.block_elems == 0) {
+                set_error("compile: node %u: DequantGroupedMatMul scheme %u is not claimed (GGUF Q4_K=5 .. Q3_K=10, Q4_0=11, Q8_0=12)", i,
                           nd.d.scheme);
                 return nullptr;
             }

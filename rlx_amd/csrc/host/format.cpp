@@ -1,6 +1,7 @@
 // Host-side format code: GGUF block geometry, the one-time repack into the device layout, the encoders that
 // produce GGUF bytes from f32 (the reference has none: rlx-gguf is decode-only), and the reference's Philox stream.
 #include <cmath>
+#include <cstdlib>
 #include <cstring>
 #include <vector>
 
@@ -46,12 +47,151 @@ static inline float f16_bits_to_f32(uint16_t h) {
     return f;
 }
 
+// ---- block decoders of the wide schemes ------------------------------------------------------------------
+// Element-indexed restatements of the reference's super-block decoders, same f32 operation order, used once per weight
+// at upload. `i` is the element's position in the 256-element super-block.
+
+static inline void k4_scale_min(int j, const uint8_t *q, uint8_t *sc, uint8_t *mn) {  // rlx-gguf/src/lib.rs:743-751
+    if (j < 4) {
+        *sc = q[j] & 63;
+        *mn = q[j + 4] & 63;
+    } else {
+        *sc = (uint8_t)((q[j + 4] & 0x0F) | ((q[j - 4] >> 6) << 4));
+        *mn = (uint8_t)((q[j + 4] >> 4) | ((q[j] >> 6) << 4));
+    }
+}
+
+static inline float f16_at(const uint8_t *p) { return f16_bits_to_f32((uint16_t)(p[0] | (p[1] << 8))); }
+
+// Q5_K (lib.rs:783-816): d, dmin, 12 scale bytes, 32 bytes of fifth bits, 128 bytes of nibbles.
+static void decode_q5_k(const uint8_t *b, float *out) {
+    const float d = f16_at(b), dmin = f16_at(b + 2);
+    const uint8_t *scales = b + 4, *qh = b + 16, *qs = b + 48;
+    for (int j = 0; j < 8; j++) {
+        uint8_t sc, mn;
+        k4_scale_min(j, scales, &sc, &mn);
+        const float dj = d * (float)sc, mj = dmin * (float)mn;
+        for (int l = 0; l < 32; l++) {
+            const uint8_t byte = qs[32 * (j >> 1) + l];
+            const int lo = (j & 1) ? (byte >> 4) : (byte & 0x0F);
+            const int hi = (qh[l] >> j) & 1 ? 16 : 0;
+            out[32 * j + l] = dj * (float)(lo + hi) - mj;
+        }
+    }
+}
+
+// Q6_K (lib.rs:819-845): 128 bytes of low nibbles, 64 bytes of high bit pairs, 16 scale bytes, d. The reference's block
+// decoder, the one its matmul calls, converts the scale bytes as unsigned; its whole-tensor decoder (lib.rs:1070-1112)
+// and upstream ggml read them as signed. `signed_scales` selects the latter.
+static void decode_q6_k(const uint8_t *b, float *out, bool signed_scales) {
+    const uint8_t *ql = b, *qh = b + 128, *sc = b + 192;
+    const float d = f16_at(b + 208);
+    for (int i = 0; i < 256; i++) {
+        const int h = i >> 7, quarter = (i >> 5) & 3, l = i & 31;
+        const uint8_t lowbyte = ql[64 * h + 32 * (quarter & 1) + l];
+        const int low = (quarter >> 1) ? (lowbyte >> 4) : (lowbyte & 0x0F);
+        const int high = (qh[32 * h + l] >> (2 * quarter)) & 3;
+        const int q = (low | (high << 4)) - 32;
+        const uint8_t sbyte = sc[8 * h + 2 * quarter + (l >> 4)];
+        const float s = signed_scales ? (float)(int8_t)sbyte : (float)sbyte;
+        out[i] = d * s * (float)q;
+    }
+}
+
+// Q8_K (lib.rs:848-854): f32 d, 256 signed bytes (the 16 block sums that follow are not read).
+static void decode_q8_k(const uint8_t *b, float *out) {
+    float d;
+    memcpy(&d, b, 4);
+    for (int i = 0; i < 256; i++) out[i] = d * (float)(int8_t)b[4 + i];
+}
+
+// Q2_K in the reference's field order (lib.rs:857-886): d, min, 16 scale bytes (low nibble scale, high nibble min),
+// 64 bytes of 2-bit codes.
+static void decode_q2_k(const uint8_t *b, float *out) {
+    const float d = f16_at(b), mn = f16_at(b + 2);
+    const uint8_t *scales = b + 4, *q = b + 20;
+    for (int i = 0; i < 256; i++) {
+        const int h = i >> 7, pair = (i >> 5) & 3, l = i & 31;
+        const uint8_t sc = scales[8 * h + 2 * pair + (l >> 4)];
+        const float dl = d * (float)(sc & 0xF), ml = mn * (float)(sc >> 4);
+        out[i] = dl * (float)((q[32 * h + l] >> (2 * pair)) & 3) - ml;
+    }
+}
+
+// Q3_K in the reference's field order (lib.rs:889-930): d, 12 scale bytes, 32 bytes of high-bit mask, 64 bytes of 2-bit codes.
+static void decode_q3_k(const uint8_t *b, float *out) {
+    const float d_all = f16_at(b);
+    const uint8_t *s = b + 2, *hm = b + 14, *q = b + 46;
+    int scale[16];
+    for (int j = 0; j < 4; j++) {
+        scale[j] = (s[j] & 0xF) | ((s[8 + j] & 3) << 4);
+        scale[4 + j] = (s[4 + j] & 0xF) | (((s[8 + j] >> 2) & 3) << 4);
+        scale[8 + j] = (s[j] >> 4) | (((s[8 + j] >> 4) & 3) << 4);
+        scale[12 + j] = (s[4 + j] >> 4) | (((s[8 + j] >> 6) & 3) << 4);
+    }
+    for (int i = 0; i < 256; i++) {
+        const int h = i >> 7, pair = (i >> 5) & 3, l = i & 31;
+        const float dl = d_all * (float)(scale[8 * h + 2 * pair + (l >> 4)] - 32);
+        const int code = ((q[32 * h + l] >> (2 * pair)) & 3) - ((hm[l] >> (4 * h + pair)) & 1 ? 0 : 4);
+        out[i] = dl * (float)code;
+    }
+}
+
+static bool q6k_signed_scales() {
+    static const bool v = getenv("RLX_Q6K_SIGNED_SCALES") != nullptr;
+    return v;
+}
+
+static void decode_wide_block(int scheme, const uint8_t *b, float *out) {
+    switch (scheme) {
+    case SCHEME_Q5K: decode_q5_k(b, out); break;
+    case SCHEME_Q6K: decode_q6_k(b, out, q6k_signed_scales()); break;
+    case SCHEME_Q8K: decode_q8_k(b, out); break;
+    case SCHEME_Q2K: decode_q2_k(b, out); break;
+    default: decode_q3_k(b, out); break;
+    }
+}
+
+// Wide schemes: decode every super-block and store the weights as binary16 operand fragments.
+static int repack_wide(int scheme, const uint8_t *src, int64_t n, int64_t k, uint8_t *out) {
+    const Layout L = layout_of(scheme);
+    const WeightDims D = weight_dims(scheme, n, k);
+    const int64_t bpr = k / 256;
+    memset(out, 0, (size_t)D.bytes);
+    float vals[256];
+    for (int64_t r = 0; r < n; r++) {
+        const int64_t tile = r >> 4;
+        const int nrow = (int)(r & 15);
+        for (int64_t sb = 0; sb < bpr; sb++) {
+            decode_wide_block(scheme, src + (r * bpr + sb) * L.block_bytes, vals);
+            for (int blk = 0; blk < 8; blk++) {  // 32-column blocks of the super-block
+                const int64_t gblk = sb * 8 + blk, u = gblk >> 2;
+                uint8_t *unit = out + (tile * D.units + u) * L.unit_bytes + (gblk & 3) * 1024;
+                for (int g = 0; g < 4; g++) {
+                    uint16_t h8[8];
+                    for (int e = 0; e < 8; e++) {
+                        const float v = vals[32 * blk + 8 * g + e];
+                        h8[e] = f32_to_f16_bits(v);
+                        if ((h8[e] & 0x7FFFu) >= 0x7C00u && std::isfinite(v)) {
+                            set_error("repack: a decoded weight (%g, row %lld) exceeds the binary16 range the wide schemes are stored in",
+                                      (double)v, (long long)r);
+                            return RLX_ERR_UNSUPPORTED;
+                        }
+                    }
+                    memcpy(unit + (g * 16 + nrow) * 16, h8, 16);
+                }
+            }
+        }
+    }
+    return RLX_OK;
+}
+
 // ---- repack ---------------------------------------------------------------------------------------------
 
 int repack_host(int scheme, const uint8_t *src, size_t nbytes, int64_t n, int64_t k, uint8_t *out) {
     Layout L = layout_of(scheme);
-    if (L.unit_k == 0) {
-        set_error("repack: scheme %d is not a claimed GGUF scheme (Q4_K=5, Q4_0=11, Q8_0=12)", scheme);
+    if (L.unit_k == 0 || L.block_elems == 0) {
+        set_error("repack: scheme %d is not a claimed GGUF scheme (Q4_K=5, Q5_K=6, Q6_K=7, Q8_K=8, Q2_K=9, Q3_K=10, Q4_0=11, Q8_0=12)", scheme);
         return RLX_ERR_UNSUPPORTED;
     }
     if (n <= 0 || k <= 0 || k % L.block_elems != 0) {
@@ -65,6 +205,7 @@ int repack_host(int scheme, const uint8_t *src, size_t nbytes, int64_t n, int64_
                   (long long)(n * bpr * L.block_bytes));
         return RLX_ERR_INVALID;
     }
+    if (scheme_is_wide(scheme)) return repack_wide(scheme, src, n, k, out);
     WeightDims D = weight_dims(scheme, n, k);
     for (int64_t tile = 0; tile < D.row_tiles; tile++) {
         for (int64_t u = 0; u < D.units; u++) {
@@ -258,7 +399,7 @@ int rlx_mi355x_repack_host(int scheme, const void *gguf_bytes, size_t nbytes, in
 
 int rlx_mi355x_quantize(int scheme, const float *src, int64_t n_elems, void *out) {
     rlx::Layout L = rlx::layout_of(scheme);
-    if (L.block_elems == 0) {
+    if (L.block_elems == 0 || rlx::scheme_is_wide(scheme)) {
         rlx::set_error("quantize: scheme %d unsupported", scheme);
         return RLX_ERR_UNSUPPORTED;
     }

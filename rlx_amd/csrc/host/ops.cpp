@@ -91,9 +91,10 @@ static int launch_gemv(const void *const *xs, int xk, const rlx_qweight *const *
     const int rv = xk == 0 ? 2 * m : m;
     const int ng = (rv + 3) / 4;
     const bool r2 = rv <= 2;
-    KernelId id = scheme == SCHEME_Q4_0   ? (r2 ? K_GEMV_Q4_0_R2 : K_GEMV_Q4_0_R4)
-                  : scheme == SCHEME_Q8_0 ? (r2 ? K_GEMV_Q8_0_R2 : K_GEMV_Q8_0_R4)
-                                          : (r2 ? K_GEMV_Q4_K_R2 : K_GEMV_Q4_K_R4);
+    KernelId id = scheme == SCHEME_Q4_0     ? (r2 ? K_GEMV_Q4_0_R2 : K_GEMV_Q4_0_R4)
+                  : scheme == SCHEME_Q8_0   ? (r2 ? K_GEMV_Q8_0_R2 : K_GEMV_Q8_0_R4)
+                  : scheme_is_wide(scheme) ? (r2 ? K_GEMV_F16W_R2 : K_GEMV_F16W_R4)
+                                            : (r2 ? K_GEMV_Q4_K_R2 : K_GEMV_Q4_K_R4);
     static const int env_waves = getenv("RLX_GEMV_WAVES") ? atoi(getenv("RLX_GEMV_WAVES")) : 8;
     static const int env_depth = getenv("RLX_GEMV_DEPTH") ? atoi(getenv("RLX_GEMV_DEPTH")) : 4;
     static const int env_wgs_per_cu = getenv("RLX_GEMV_WGS_PER_CU") ? atoi(getenv("RLX_GEMV_WGS_PER_CU")) : 2;
@@ -226,9 +227,10 @@ static int launch_gemm(const void *x, int xk, const rlx_qweight *w, float *out, 
     GemmArgs a{w->dev, xh, sxh, out, (int)p.m_rows, (int)m, (int)w->dims.n, (int)p.k_pad, (int)w->dims.units,
                (int)w->dims.row_tiles, xk == 0 ? 1 : 0, units_per_split * steps_per_unit, split > 1 ? 1 : 0};
     void *params[] = {&a};
-    KernelId id = w->scheme == SCHEME_Q4K    ? (skinny ? K_GEMM64_Q4_K : K_GEMM_Q4_K)
-                  : w->scheme == SCHEME_Q4_0 ? (skinny ? K_GEMM64_Q4_0 : K_GEMM_Q4_0)
-                                             : (skinny ? K_GEMM64_Q8_0 : K_GEMM_Q8_0);
+    KernelId id = w->scheme == SCHEME_Q4K       ? (skinny ? K_GEMM64_Q4_K : K_GEMM_Q4_K)
+                  : w->scheme == SCHEME_Q4_0    ? (skinny ? K_GEMM64_Q4_0 : K_GEMM_Q4_0)
+                  : scheme_is_wide(w->scheme) ? (skinny ? K_GEMM64_F16W : K_GEMM_F16W)
+                                                : (skinny ? K_GEMM64_Q8_0 : K_GEMM_Q8_0);
     RLX_TRY(runtime_init());
     RLX_TRY(launch3(id, (unsigned)gx, (unsigned)gy, (unsigned)split, 512, skinny ? 3 * 24 * 1024 : 3 * 48 * 1024, stream, params));
     return RLX_OK;
@@ -244,7 +246,7 @@ int rlx_mi355x_qweight_create_at(int scheme, const void *gguf_bytes, size_t nbyt
     RLX_TRY(runtime_init());
     WeightDims D = weight_dims(scheme, n, k);
     std::vector<uint8_t> staging;
-    if (D.bytes == 0) {
+    if (D.bytes == 0 || layout_of(scheme).block_elems == 0) {
         set_error("qweight: scheme %d is not a claimed GGUF scheme", scheme);
         return RLX_ERR_UNSUPPORTED;
     }
@@ -272,7 +274,7 @@ int rlx_mi355x_qweight_create_experts_at(int scheme, const void *gguf_bytes, siz
     using namespace rlx;
     RLX_TRY(runtime_init());
     WeightDims D = weight_dims(scheme, n, k);
-    if (D.bytes == 0) {
+    if (D.bytes == 0 || layout_of(scheme).block_elems == 0) {
         set_error("qweight: scheme %d is not a claimed GGUF scheme", scheme);
         return RLX_ERR_UNSUPPORTED;
     }
@@ -315,6 +317,11 @@ int rlx_mi355x_dequant(const rlx_qweight *w, float *out_dev, void *stream) {
     if (!w || !out_dev) {
         set_error("dequant: null argument");
         return RLX_ERR_INVALID;
+    }
+    if (scheme_is_wide(w->scheme)) {
+        set_error("dequant: scheme %d is resident as binary16 (decoded at upload); the exact f32 decode is not kept on the device",
+                  w->scheme);
+        return RLX_ERR_UNSUPPORTED;
     }
     DequantArgs a{w->dev, out_dev, w->dims.n, w->dims.k, w->dims.units};
     void *params[] = {&a};

@@ -123,6 +123,10 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
             const int unit = (step >> 2) * L.unit_bytes;
             if ((q & 1) == 0) b_q[(q >> 1) & 1] = ld128(b_rsrc, lane * 16, unit + (q >> 1) * 1024);
             if (q == 0) b_meta[0] = ld128(b_rsrc, b_n16 * 16, unit + 2048);  // consumed one step later, before the next fetch
+        } else if constexpr (SCHEME == SCHEME_F16W) {  // two ready-made fragments per lane and step: b_q and b_meta hold them
+            const int unit = (step >> 1) * L.unit_bytes + (q & 1) * 2048;
+            b_q[q & 1] = ld128(b_rsrc, lane * 16, unit);
+            b_meta[q & 1] = ld128(b_rsrc, lane * 16, unit + 1024);
         } else if constexpr (SCHEME == SCHEME_Q4_0) {
             const int unit = (step >> 1) * L.unit_bytes;
             if ((q & 1) == 0) {
@@ -160,6 +164,10 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
                 b_sc[1] &= b_keep;
             }
             unpack_q4_scaled(b_q[cp][t], splat_code_half(b_sc[q >> 1], t), f);
+        } else if constexpr (SCHEME == SCHEME_F16W) {
+            f.u4 = jl ? b_meta[q & 1] : b_q[q & 1];
+#pragma unroll
+            for (int e = 0; e < 4; e++) f.u[e] &= b_keep;  // a dead tile stores zeros
         } else {
             const uint32_t dbits = ((t & 1) ? (b_meta[cp][t >> 1] >> 16) : (b_meta[cp][t >> 1] & 0xFFFFu)) & b_keep;  // dead tile: d = 0
             const half2_t d2 = as_half2(dbits | (dbits << 16));
@@ -476,6 +484,8 @@ __device__ __forceinline__ void xprep_body(const XPrepArgs &a) {
 extern "C" __global__ __launch_bounds__(512) void rlx_gemm_q4_k(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q4K, 2, 2>(a); }
 extern "C" __global__ __launch_bounds__(512) void rlx_gemm_q4_0(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q4_0, 2, 2>(a); }
 extern "C" __global__ __launch_bounds__(512) void rlx_gemm_q8_0(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q8_0, 2, 2>(a); }
+extern "C" __global__ __launch_bounds__(512) void rlx_gemm_f16w(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_F16W, 2, 2>(a); }
+extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64_f16w(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_F16W, 1, 1>(a); }
 extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64_q4_k(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q4K, 1, 1>(a); }
 extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64_q4_0(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q4_0, 1, 1>(a); }
 extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64_q8_0(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q8_0, 1, 1>(a); }

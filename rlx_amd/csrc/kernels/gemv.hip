@@ -92,6 +92,19 @@ struct UnitRegs<SCHEME_Q4K> {
     __device__ __forceinline__ void clear() { q0 = q1 = meta = uint4_t{0, 0, 0, 0}; }  // d = dmin = 0
 };
 
+template <>
+struct UnitRegs<SCHEME_F16W> {  // weights already stored as binary16 fragments: four 32-column blocks, no scales
+    uint4_t q[4];
+    __device__ __forceinline__ void load(const uint8_t *unit, int l, int, bool) {
+#pragma unroll
+        for (int t = 0; t < 4; t++) q[t] = __builtin_nontemporal_load((const uint4_t *)(unit + t * 1024 + l * 16));
+    }
+    __device__ __forceinline__ void clear() {
+#pragma unroll
+        for (int t = 0; t < 4; t++) q[t] = uint4_t{0, 0, 0, 0};
+    }
+};
+
 __device__ __forceinline__ float scale_of(uint2_t s, int t) {
     return half_bits_to_float((t & 1) ? (s[t >> 1] >> 16) : (s[t >> 1] & 0xFFFFu));
 }
@@ -125,6 +138,17 @@ __device__ __forceinline__ void compute_unit(const UnitRegs<SCHEME> &w, const ha
 #pragma unroll
             for (int r = 0; r < NREG; r++) acc[r] = __builtin_fmaf(d, blk[t][r], acc[r]);
         }
+    } else if constexpr (SCHEME == SCHEME_F16W) {
+        load_afrags<4>(xrow, live, ucol, a);
+        float4_t sum = zero;  // the matrix unit accumulates the four blocks; nothing to decode or scale
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            Frag b;
+            b.u4 = w.q[t];
+            sum = mfma16(a[t], b, sum);
+        }
+#pragma unroll
+        for (int r = 0; r < NREG; r++) acc[r] += sum[r];
     } else if constexpr (SCHEME == SCHEME_Q8_0) {
         Frag b[4];
         load_afrags<4>(xrow, live, ucol, a);
@@ -396,3 +420,5 @@ RLX_GEMV_INST(rlx_gemv_q8_0_r2, rlx::SCHEME_Q8_0, 2, 3)
 RLX_GEMV_INST(rlx_gemv_q8_0_r4, rlx::SCHEME_Q8_0, 4, 3)
 RLX_GEMV_INST(rlx_gemv_q4_k_r2, rlx::SCHEME_Q4K, 2, 3)
 RLX_GEMV_INST(rlx_gemv_q4_k_r4, rlx::SCHEME_Q4K, 4, 3)
+RLX_GEMV_INST(rlx_gemv_f16w_r2, rlx::SCHEME_F16W, 2, 2)
+RLX_GEMV_INST(rlx_gemv_f16w_r4, rlx::SCHEME_F16W, 4, 2)

@@ -20,6 +20,10 @@
 //          [2048,2176) f16 d[n][4]
 //   Q4_K : [0,2048)  two halves h: 16 B at 1024*h + 16*l = granules of sub-blocks 4h+0..3 of super-block u
 //          [2048,2304) per row n: 16 B = f16 d, f16 dmin, 12 scale bytes (verbatim from the GGUF block)
+//   Q5_K, Q6_K, Q8_K, Q2_K, Q3_K ("wide" schemes): the weights are decoded once, at upload, with the reference's block
+//          decoder and stored as binary16: [0,4096) four blocks t: 16 B at 1024*t + 16*l = the 8 halfs of granule
+//          (n, 4u+t, g), already an MFMA operand fragment. No scales. 2 bytes per weight resident instead of the
+//          packed 0.33-1.14, in exchange for kernels that do no decode arithmetic at all.
 // Units are stored [row_tile][unit] with the unit index (K direction) fastest.
 // N is padded to a multiple of 16 and K to a multiple of UNIT_K with zero-scale blocks.
 #pragma once
@@ -33,7 +37,17 @@
 
 namespace rlx {
 
-enum Scheme : int { SCHEME_Q4K = 5, SCHEME_Q4_0 = 11, SCHEME_Q8_0 = 12 };
+// Values of the reference's QuantScheme discriminants (rlx-ir/src/quant.rs:39-73); SCHEME_F16W is internal: the device
+// layout every wide scheme is stored in, and the template argument of the kernels that read it.
+enum Scheme : int {
+    SCHEME_Q4K = 5, SCHEME_Q5K = 6, SCHEME_Q6K = 7, SCHEME_Q8K = 8, SCHEME_Q2K = 9, SCHEME_Q3K = 10,
+    SCHEME_Q4_0 = 11, SCHEME_Q8_0 = 12, SCHEME_F16W = 100
+};
+
+RLX_HD constexpr bool scheme_is_wide(int scheme) {
+    return scheme == SCHEME_Q5K || scheme == SCHEME_Q6K || scheme == SCHEME_Q8K || scheme == SCHEME_Q2K ||
+           scheme == SCHEME_Q3K || scheme == SCHEME_F16W;
+}
 
 constexpr int TILE_ROWS = 16;
 
@@ -49,6 +63,12 @@ RLX_HD constexpr Layout layout_of(int scheme) {
     return scheme == SCHEME_Q4_0   ? Layout{128, 1152, 1024, 32, 18}
            : scheme == SCHEME_Q8_0 ? Layout{128, 2176, 2048, 32, 34}
            : scheme == SCHEME_Q4K  ? Layout{256, 2304, 2048, 256, 144}
+           : scheme == SCHEME_Q5K  ? Layout{128, 4096, 4096, 256, 176}
+           : scheme == SCHEME_Q6K  ? Layout{128, 4096, 4096, 256, 210}
+           : scheme == SCHEME_Q8K  ? Layout{128, 4096, 4096, 256, 292}
+           : scheme == SCHEME_Q2K  ? Layout{128, 4096, 4096, 256, 84}
+           : scheme == SCHEME_Q3K  ? Layout{128, 4096, 4096, 256, 110}
+           : scheme == SCHEME_F16W ? Layout{128, 4096, 4096, 0, 0}
                                    : Layout{0, 0, 0, 0, 0};
 }
 

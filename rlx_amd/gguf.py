@@ -229,16 +229,18 @@ class GgufFile:
         return np.frombuffer(self._data, dtype=np.uint8, count=nbytes, offset=t.offset)
 
     def qweight(self, name):
-        """Upload a 2-D Q8_0 / Q4_0 / Q4_K tensor as a resident `QWeight`. GGML shape order is innermost first, so a
-        weight used as y = x . W^T has shape [k, n]."""
+        """Upload a 2-D Q8_0 / Q4_0 / Q4_K / Q5_K / Q6_K / Q8_K tensor as a resident `QWeight`. GGML shape order is
+        innermost first, so a weight used as y = x . W^T has shape [k, n]. (Q2_K and Q3_K files are not mapped: the
+        reference's block decoders read those two in a field order that differs from ggml's on-disk blocks.)"""
         from . import ops
         from .ir import QuantScheme
         t = self.tensors.get(name)
         if t is None:
             raise GgufError(f"tensor not found: {name}")
-        schemes = {GgmlType.Q8_0: QuantScheme.GgufQ8_0, GgmlType.Q4_0: QuantScheme.GgufQ4_0, GgmlType.Q4K: QuantScheme.GgufQ4K}
+        schemes = {GgmlType.Q8_0: QuantScheme.GgufQ8_0, GgmlType.Q4_0: QuantScheme.GgufQ4_0, GgmlType.Q4K: QuantScheme.GgufQ4K,
+                   GgmlType.Q5K: QuantScheme.GgufQ5K, GgmlType.Q6K: QuantScheme.GgufQ6K, GgmlType.Q8K: QuantScheme.GgufQ8K}
         if t.dtype not in schemes or len(t.shape) != 2:
-            raise GgufError(f"tensor {name}: {t.dtype.name} with shape {t.shape} is not a 2-D Q8_0 / Q4_0 / Q4_K matrix")
+            raise GgufError(f"tensor {name}: {t.dtype.name} with shape {t.shape} is not a 2-D matrix of a claimed scheme")
         k, n = t.shape
         return ops.QWeight(schemes[t.dtype], np.ascontiguousarray(self.tensor_bytes(t)), n, k)
 

@@ -28,14 +28,16 @@ class QuantScheme(enum.IntEnum):  # rlx-ir/src/quant.rs:39-79 (declaration order
     GgufQ5K = 6
     GgufQ6K = 7
     GgufQ8K = 8
+    GgufQ2K = 9
+    GgufQ3K = 10
     GgufQ4_0 = 11
     GgufQ8_0 = 12
 
     def gguf_block_size(self):  # quant.rs:138-150
-        return {5: 256, 6: 256, 7: 256, 8: 256, 11: 32, 12: 32}[int(self)]
+        return {5: 256, 6: 256, 7: 256, 8: 256, 9: 256, 10: 256, 11: 32, 12: 32}[int(self)]
 
     def gguf_block_bytes(self):  # quant.rs:152-164
-        return {5: 144, 6: 176, 7: 210, 8: 292, 11: 18, 12: 34}[int(self)]
+        return {5: 144, 6: 176, 7: 210, 8: 292, 9: 84, 10: 110, 11: 18, 12: 34}[int(self)]
 
     def is_gguf(self):
         return True

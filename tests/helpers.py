@@ -1,8 +1,10 @@
 """Shared test helpers: seeded inputs, packed weights, a numpy reader of the device layout, error metrics."""
 import numpy as np
 
-Q4K, Q4_0, Q8_0 = 5, 11, 12
-SCHEME_NAMES = {Q4K: "q4_k", Q4_0: "q4_0", Q8_0: "q8_0"}
+Q4K, Q5K, Q6K, Q8K, Q2K, Q3K, Q4_0, Q8_0 = 5, 6, 7, 8, 9, 10, 11, 12
+WIDE = (Q5K, Q6K, Q8K, Q2K, Q3K)  # stored as binary16 on the device
+SCHEME_NAMES = {Q4K: "q4_k", Q5K: "q5_k", Q6K: "q6_k", Q8K: "q8_k", Q2K: "q2_k", Q3K: "q3_k", Q4_0: "q4_0", Q8_0: "q8_0"}
+BLOCK = {Q4_0: (32, 18), Q8_0: (32, 34), Q4K: (256, 144), Q5K: (256, 176), Q6K: (256, 210), Q8K: (256, 292), Q2K: (256, 84), Q3K: (256, 110)}
 NIB_POS = [0, 4, 1, 5, 2, 6, 3, 7]
 UNIT = {Q4_0: (128, 1152, 1024), Q8_0: (128, 2176, 2048), Q4K: (256, 2304, 2048)}
 
@@ -16,18 +18,22 @@ def make_weights(scheme, n, k, std=0.02, seed=0):
     return ops.quantize(scheme, w), w
 
 
-def random_blocks(scheme, n, k, seed=0):
-    """Arbitrary block bytes (every bit pattern in codes and 6-bit fields) with finite f16 scales."""
+def random_blocks(scheme, n, k, seed=0, d_std=0.02, dmin_std=0.01):
+    """Arbitrary block bytes (every bit pattern in codes and 6-bit fields) with finite f16 scales ~N(0, d_std)."""
     rng = np.random.default_rng(seed)
-    be, bb = {Q4_0: (32, 18), Q8_0: (32, 34), Q4K: (256, 144)}[scheme]
+    be, bb = BLOCK[scheme]
     nb = n * k // be
     p = rng.integers(0, 256, (nb, bb), dtype=np.uint8)
-    d = (rng.standard_normal(nb) * 0.02).astype(np.float16)
+    d = (rng.standard_normal(nb) * d_std).astype(np.float16)
     d[::11] = np.float16(3e-6)   # subnormal halfs
     d[::13] = np.float16(0.0)
-    p[:, 0:2] = d.view(np.uint8).reshape(nb, 2)
-    if scheme == Q4K:
-        dm = (np.abs(rng.standard_normal(nb)) * 0.01).astype(np.float16)
+    if scheme == Q8K:  # f32 super-block scale
+        p[:, 0:4] = d.astype(np.float32).view(np.uint8).reshape(nb, 4)
+        return p.reshape(-1)
+    d_off = 208 if scheme == Q6K else 0
+    p[:, d_off:d_off + 2] = d.view(np.uint8).reshape(nb, 2)
+    if scheme in (Q4K, Q5K, Q2K):  # second f16 field: the super-block minimum
+        dm = (np.abs(rng.standard_normal(nb)) * dmin_std).astype(np.float16)
         p[:, 2:4] = dm.view(np.uint8).reshape(nb, 2)
     return p.reshape(-1)
 

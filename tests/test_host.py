@@ -137,7 +137,8 @@ def test_compile_rejects_wrong_weight_size():
 
 def test_compile_rejects_unclaimed_scheme():
     g = dq_graph(1, 256, 1, Q4K)
-    g.nodes[2] = type(g.nodes[2])(2, Op.DequantMatMul(QuantScheme.GgufQ6K), g.nodes[2].inputs, g.nodes[2].shape)
+    # discriminant 13 = QuantScheme::Nvfp4Block (rlx-ir/src/quant.rs:74-78): not a GGUF block format
+    g.nodes[2] = type(g.nodes[2])(2, Op.DequantMatMul(13), g.nodes[2].inputs, g.nodes[2].shape)
     assert "not claimed" in compile_error(g)
 
 
