@@ -314,6 +314,45 @@ def extra_configs(rlx_amd, stream):
                                              "note": "wide schemes are decoded at upload and stream 2 bytes per weight with no decode arithmetic"}
     for q in qws:
         q.free()
+    # tied LM head: argmax over a Llama-3 vocabulary [128256, 4096] in Q4_K (295 MB, two copies rotated), logits never written
+    n, k = 128256, 4096
+    w = (ops.philox_normal(21, 4096 * k) * np.float32(0.02)).astype(np.float32)
+    slab = ops.quantize(QuantScheme.GgufQ4K, w).reshape(4096, -1)
+    packed = np.concatenate([slab] * 32, axis=0)[:n]
+    copies = 2
+    qws = [ops.QWeight(QuantScheme.GgufQ4K, np.roll(packed, 7 * i, axis=0).reshape(-1), n, k) for i in range(copies)]
+    del packed, slab, w
+    x = ops.DeviceBuffer.from_numpy(ops.philox_normal(8, k))
+    res = ops.DeviceBuffer(16)
+    rlx_amd._lib.check(L.rlx_mi355x_memset_u32(res.ptr, 0, 4, stream))  # the key scratch starts zero; every call leaves it zero
+    y = ops.DeviceBuffer(n * 4)
+    state = {"i": 0}
+
+    def fn_arg():
+        q = qws[state["i"] % copies]
+        state["i"] += 1
+        rlx_amd._lib.check(L.rlx_mi355x_gguf_tied_lm_argmax(x.ptr, int(DType.F32), q.ptr, res.ptr, res.ptr + 4, res.ptr + 8, stream))
+
+    def fn_logits():
+        q = qws[state["i"] % copies]
+        state["i"] += 1
+        rlx_amd._lib.check(L.rlx_mi355x_gguf_matmul_bt(x.ptr, int(DType.F32), q.ptr, y.ptr, 1, None, 0, stream))
+
+    def fn_logits_sep():  # the unfused sequence has at least one more small kernel (the argmax over the logits) after it
+        fn_logits()
+        rlx_amd._lib.check(L.rlx_mi355x_memset_u32(res.ptr, 0, 1, stream))
+
+    ms = time_launches(ops, stream, fn_arg, 100, 10)
+    ms_l = time_launches(ops, stream, fn_logits, 100, 10)
+    ms_s = time_launches(ops, stream, fn_logits_sep, 100, 10)
+    b = n * k // 256 * 144 + 4 * k
+    out["q4_k_tied_lm_argmax_128256x4096"] = {"us": round(ms * 1e3, 2), "GB/s": round(b / ms / 1e6, 1),
+                                             "frac_hbm": round(b / ms / 1e6 / HBM_PEAK_GBS, 4),
+                                             "us_plain_gemv_writing_logits_back_to_back": round(ms_l * 1e3, 2),
+                                             "us_plain_gemv_plus_one_small_kernel": round(ms_s * 1e3, 2),
+                                             "launches": "gemv (argmax epilogue) + finish"}
+    for q in qws:
+        q.free()
     # config 4: FakeQuantize [8192, 4096], int8 per column, heavy-tailed input; three input / output sets in rotation
     # (3 x 268 MB) so that no launch finds its input in the 256 MB last-level cache
     rows, cols = 8192, 4096

@@ -161,6 +161,14 @@ int rlx_mi355x_qweight_create_experts_at(int scheme, const void *gguf_bytes, siz
  * launch). An index outside [0, num_experts) is clamped to the stack (the reference debug-asserts). */
 int rlx_mi355x_gguf_grouped_matmul_bt(const void *x_dev, int x_dtype, const rlx_qweight *w, const float *expert_idx_dev,
                                       float *out_dev, int64_t m, void *stream);
+/* rlx_cpu::lm_head::gguf_tied_lm_argmax (rlx-cpu/src/lm_head.rs:223-248): the row of the packed [n_vocab, n_embd] matrix
+ * with the largest dot product against one hidden vector, and that dot product. The first maximum wins, a NaN never
+ * does, and (0, -inf) comes back when no row beats -inf, as in the reference's loop. The logits are never written: the
+ * decode kernel's workgroups merge (value, row) keys with a 64-bit atomic max into `key_scratch_dev` (8 bytes, 8-byte
+ * aligned, ZERO before the first call, e.g. rlx_mi355x_memset_u32; every call leaves it zero again), and a one-thread
+ * kernel writes *out_idx_dev / *out_val_dev. Calls that share a scratch must be ordered on one stream. */
+int rlx_mi355x_gguf_tied_lm_argmax(const void *hidden_dev, int x_dtype, const rlx_qweight *embed, uint32_t *out_idx_dev,
+                                   float *out_val_dev, void *key_scratch_dev, void *stream);
 int rlx_mi355x_gguf_matmul_bt_batch(const void *const *xs_dev, int x_dtype, const rlx_qweight *const *ws,
                                     float *const *outs_dev, int count, int64_t m, void *workspace, size_t workspace_bytes,
                                     void *stream);

@@ -51,6 +51,8 @@ def lib():
         L.orc_dequant.argtypes = [C.c_int, u8p, C.c_int64, C.c_int64, f32p]
         L.orc_dequant_matmul_blocks.restype = C.c_int
         L.orc_dequant_matmul_blocks.argtypes = [C.c_int, u8p, C.c_int64, C.c_int64, f32p]
+        L.orc_gguf_tied_lm_argmax.restype = C.c_int
+        L.orc_gguf_tied_lm_argmax.argtypes = [f32p, u8p, C.c_int64, C.c_int64, C.c_int64, C.c_int, u32p, f32p]
         L.orc_gguf_grouped_matmul_bt.restype = C.c_int
         L.orc_gguf_grouped_matmul_bt.argtypes = [f32p, u8p, C.c_int64, f32p, f32p, C.c_int64, C.c_int64, C.c_int64, C.c_int64, C.c_int]
         L.orc_gguf_matmul_bt.restype = C.c_int
@@ -145,6 +147,19 @@ def gguf_matmul_bt(x, packed, m, k, n, scheme):
     if rc != 0:
         raise ValueError("gguf_matmul_bt: bad sizes")
     return out.reshape(m, n)
+
+
+def gguf_tied_lm_argmax(hidden, packed, n_embd, n_vocab, scheme):
+    """rlx-cpu/src/lm_head.rs:223-248 -> (row, value)."""
+    hidden = np.ascontiguousarray(hidden, dtype=np.float32).reshape(-1)
+    packed = np.ascontiguousarray(packed, dtype=np.uint8)
+    assert hidden.size == n_embd
+    idx, val = C.c_uint32(), C.c_float()
+    rc = lib().orc_gguf_tied_lm_argmax(_p(hidden, C.c_float), _p(packed, C.c_uint8), packed.size, n_embd, n_vocab, scheme,
+                                       C.byref(idx), C.byref(val))
+    if rc != 0:
+        raise ValueError("gguf_tied_lm_argmax: bad sizes")
+    return idx.value, val.value
 
 
 def gguf_grouped_matmul_bt(x, packed, expert_idx, m, k, n, num_experts, scheme):

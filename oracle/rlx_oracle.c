@@ -22,6 +22,8 @@
  *   gguf_matmul_bt        reference tests rlx-cpu/src/gguf_matmul.rs:238-277 and
  *                         rlx-runtime/tests/dequant_matmul_gguf.rs:176-308
  *                         (layout idx = j*k + p), f64 dense matmul (textbook)
+ *   gguf_tied_lm_argmax   the reference's test (rlx-cpu/src/lm_head.rs:306-334: equals the argmax of gguf_matmul_bt's
+ *                         logits) + constructed ties, NaN and all -inf rows against the loop's stated rule
  *   fake_quantize         closed forms (channel max -> code +-q_max, all-zero
  *                         channel, constructed ties, NaN), shapes/inputs of
  *                         rlx-mlx/tests/autodiff_fakequant_parity.rs:189-308
@@ -412,6 +414,47 @@ int orc_dequant_matmul_blocks(int scheme, const uint8_t *bytes, int64_t nbytes, 
         dequant_block(scheme, bytes + i * bb, tmp);
         memcpy(out + i * be, tmp, (size_t)be * sizeof(float));
     }
+    return 0;
+}
+
+/* ---- tied LM head ------------------------------------------------------ */
+
+/* rlx-cpu/src/lm_head.rs:46-77: one row of the packed matrix against `hidden`, block by block, f32 accumulation. */
+static float row_dot_gguf(const float *hidden, const uint8_t *w_bytes, int64_t row, int64_t n_embd, int scheme) {
+    int64_t k = n_embd, row_start = row * k, row_end = row_start + k;
+    int be = orc_block_elems(scheme), bb = orc_block_bytes(scheme);
+    int64_t first_block = row_start / be, last_block = (row_end - 1) / be;
+    float block_f32[QK_K];
+    float dot = 0.0f;
+    for (int64_t bi = first_block; bi <= last_block; bi++) {
+        dequant_block(scheme, w_bytes + bi * bb, block_f32);
+        int64_t idx0 = bi * be;
+        for (int t = 0; t < be; t++) {
+            int64_t idx = idx0 + t;
+            if (idx < row_start || idx >= row_end) continue;
+            float prod = hidden[idx - row_start] * block_f32[t];
+            dot += prod;
+        }
+    }
+    return dot;
+}
+
+/* rlx-cpu/src/lm_head.rs:223-248: first row with the largest dot; starts from (0, -inf), replaced only on `>`. */
+int orc_gguf_tied_lm_argmax(const float *hidden, const uint8_t *w_bytes, int64_t w_nbytes, int64_t n_embd, int64_t n_vocab,
+                            int scheme, uint32_t *best_idx, float *best_val) {
+    int be = orc_block_elems(scheme), bb = orc_block_bytes(scheme);
+    if (be == 0 || (n_embd * n_vocab) % be != 0 || w_nbytes != (n_embd * n_vocab) / be * bb) return -1;
+    uint32_t bi = 0;
+    float bv = -INFINITY;
+    for (int64_t j = 0; j < n_vocab; j++) {
+        float dot = row_dot_gguf(hidden, w_bytes, j, n_embd, scheme);
+        if (dot > bv) {
+            bv = dot;
+            bi = (uint32_t)j;
+        }
+    }
+    *best_idx = bi;
+    *best_val = bv;
     return 0;
 }
 

@@ -39,6 +39,7 @@ struct GemvArgs {
     const float *expert_idx;
     long long slab_bytes;
     int num_experts;
+    unsigned long long *argmax_key;
 };
 struct FqArgs {
     const float *x;
@@ -80,7 +81,7 @@ static int x_kind(int x_dtype) {
 // One decode launch over `count` (<= GEMV_MAX_SEG) matmuls of one scheme, batch and activation dtype; each has
 // its own activations, K and N.
 static int launch_gemv(const void *const *xs, int xk, const rlx_qweight *const *ws, float *const *outs, int count, int m,
-                       hipStream_t stream, const float *expert_idx = nullptr) {
+                       hipStream_t stream, const float *expert_idx = nullptr, unsigned long long *argmax_key = nullptr) {
     const int scheme = ws[0]->scheme;
     const Layout L = layout_of(scheme);
     for (int i = 0; i < count; i++)
@@ -151,6 +152,7 @@ static int launch_gemv(const void *const *xs, int xk, const rlx_qweight *const *
         sh.a.x_dtype = xk;
         sh.a.max_tiles_per_wg = max_tpw;
         sh.a.expert_idx = expert_idx;
+        sh.a.argmax_key = argmax_key;
         sh.a.slab_bytes = ws[0]->dims.bytes;
         sh.a.num_experts = ws[0]->experts;
         return sh;
@@ -387,6 +389,30 @@ int rlx_mi355x_gguf_matmul_bt_batch(const void *const *xs_dev, int x_dtype, cons
 int rlx_mi355x_gguf_matmul_bt(const void *x_dev, int x_dtype, const rlx_qweight *w, float *out_dev, int64_t m,
                               void *workspace, size_t workspace_bytes, void *stream) {
     return rlx_mi355x_gguf_matmul_bt_batch(&x_dev, x_dtype, &w, &out_dev, 1, m, workspace, workspace_bytes, stream);
+}
+
+int rlx_mi355x_gguf_tied_lm_argmax(const void *hidden_dev, int x_dtype, const rlx_qweight *embed, uint32_t *out_idx_dev,
+                                   float *out_val_dev, void *key_scratch_dev, void *stream) {
+    using namespace rlx;
+    if (!hidden_dev || !embed || !out_idx_dev || !out_val_dev || !key_scratch_dev) {
+        set_error("gguf_tied_lm_argmax: null argument");
+        return RLX_ERR_INVALID;
+    }
+    int xk = x_kind(x_dtype);
+    if (xk < 0) {
+        set_error("gguf_tied_lm_argmax: hidden dtype %d is not F32 / BF16 / F16", x_dtype);
+        return RLX_ERR_UNSUPPORTED;
+    }
+    if ((uintptr_t)key_scratch_dev % 8 != 0) {
+        set_error("gguf_tied_lm_argmax: the 8-byte key scratch must be 8-byte aligned");
+        return RLX_ERR_INVALID;
+    }
+    const void *xs[1] = {hidden_dev};
+    const rlx_qweight *ws[1] = {embed};
+    float *outs[1] = {nullptr};
+    RLX_TRY(launch_gemv(xs, xk, ws, outs, 1, 1, (hipStream_t)stream, nullptr, (unsigned long long *)key_scratch_dev));
+    void *params[] = {&key_scratch_dev, &out_idx_dev, &out_val_dev};
+    return launch(K_ARGMAX_FINISH, 1, 1, 64, 0, (hipStream_t)stream, params);
 }
 
 int rlx_mi355x_gguf_grouped_matmul_bt(const void *x_dev, int x_dtype, const rlx_qweight *w, const float *expert_idx_dev,

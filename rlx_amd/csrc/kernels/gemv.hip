@@ -44,6 +44,10 @@ struct GemvArgs {
     const float *expert_idx;
     long long slab_bytes;
     int num_experts;
+    // Tied LM head (rlx-cpu/src/lm_head.rs:223-248): when set (m = 1, one segment), nothing is written to `out`; every
+    // workgroup folds its outputs into one 64-bit key (ordered value bits, then ~row so that the first maximum wins) and
+    // merges it with an atomic max.
+    unsigned long long *argmax_key;
 };
 
 constexpr int XS_PAD_HALFS = 8;      // 16 bytes of padding per LDS row: rows land in different bank groups
@@ -259,6 +263,33 @@ __device__ __forceinline__ void stage_x(const GemvArgs &a, const GemvSeg &sg, ha
     else stage_x_typed<X_F16>(a, sg, xs, row_stride, k0, kc);
 }
 
+// Key of (value, row) for the tied-LM-head argmax: float bits mapped to an order-preserving unsigned, then ~row, so the
+// maximum key is the largest value and, among equal values, the smallest row.
+__device__ __forceinline__ unsigned long long argmax_key_of(float v, uint32_t row) {
+    const uint32_t b = __builtin_bit_cast(uint32_t, v + 0.0f);  // -0 and +0 compare equal: one key for both
+    const uint32_t ordered = (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+    return ((unsigned long long)ordered << 32) | (uint32_t)~row;
+}
+
+// Decodes the merged key into {row, value}; an untouched key (every dot NaN or -inf lost to the start value) gives
+// row 0 and -inf, the reference's starting pair. Leaves the key zero for the next call.
+extern "C" __global__ void rlx_argmax_finish(unsigned long long *key, uint32_t *out_idx, float *out_val) {
+    if (threadIdx.x != 0 || blockIdx.x != 0) return;
+    const unsigned long long k = *key;
+    *key = 0;
+    const uint32_t ordered = (uint32_t)(k >> 32);
+    const uint32_t b = (ordered & 0x80000000u) ? (ordered & 0x7FFFFFFFu) : ~ordered;
+    const float v = __builtin_bit_cast(float, b);
+    const float ninf = -__builtin_inff();
+    if (k == 0 || !(v > ninf)) {
+        *out_idx = 0;
+        *out_val = ninf;
+    } else {
+        *out_idx = ~(uint32_t)k;
+        *out_val = v;
+    }
+}
+
 // One workgroup = a contiguous run of row tiles of one weight segment x all of K.
 //   * the activations are converted into LDS once per workgroup (per K chunk when they do not fit);
 //   * wave w walks the (tile, unit) items with unit = w, w + nwaves, ... of every tile in the run, keeping DEPTH
@@ -392,6 +423,7 @@ __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
 
     __syncthreads();
     // out[mr][tile*16 + col] = sum over waves of row mr (+ 2^-11 * row m+mr for f32 activations)
+    unsigned long long best = 0;  // below every key a real value produces
     for (int idx = tid; idx < ntiles * a.m * 16; idx += blockDim.x) {
         const int col = idx & 15, mr = (idx >> 4) % a.m, t = idx / (16 * a.m);
         float sum = 0.f;
@@ -401,7 +433,24 @@ __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
             if (a.x_dtype == X_F32) sum += slot[(a.m + mr) * 16] * (1.0f / LO_SCALE);
         }
         const int n_out = (tile0 + t * tstride) * 16 + col;
-        if (n_out < seg.n) seg.out[(long long)mr * seg.n + n_out] = sum;
+        if (n_out < seg.n) {
+            if (a.argmax_key) {
+                if (sum == sum) best = max(best, argmax_key_of(sum, (uint32_t)n_out));  // a NaN never wins (dot > best is false)
+            } else {
+                seg.out[(long long)mr * seg.n + n_out] = sum;
+            }
+        }
+    }
+    if (a.argmax_key) {
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            const unsigned long long other = __shfl_xor(best, off);
+            best = max(best, other);
+        }
+        // Atomics on one address are served one after another (~35 ns each): look first, and only workgroups that can
+        // still raise the key queue up for it.
+        if (l == 0 && best != 0 && best > __hip_atomic_load(a.argmax_key, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
+            atomicMax(a.argmax_key, best);
     }
 }
 

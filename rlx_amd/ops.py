@@ -192,6 +192,18 @@ def gguf_grouped_matmul_bt(x, w: QWeight, expert_idx, x_dtype=DType.F32):
     return od.to_numpy(np.float32).reshape(m, w.n)
 
 
+def gguf_tied_lm_argmax(hidden, embed: QWeight, x_dtype=DType.F32):
+    """Host convenience for the tied LM head (rlx-cpu/src/lm_head.rs:223-248): (row, value) of the largest logit of
+    hidden . embed^T without materialising the logits."""
+    hd = DeviceBuffer.from_numpy(hidden)
+    res = DeviceBuffer(16)  # [0:4) row, [4:8) value, [8:16) the key scratch (zero before the first call)
+    _lib.check(_lib.lib().rlx_mi355x_memset_u32(res.ptr, 0, 4, None))
+    _lib.check(_lib.lib().rlx_mi355x_gguf_tied_lm_argmax(hd.ptr, int(x_dtype), embed.ptr, res.ptr, res.ptr + 4, res.ptr + 8, None))
+    sync()
+    raw = res.to_numpy(np.uint32, 2)
+    return int(raw[0]), float(raw[1:2].view(np.float32)[0])
+
+
 def fake_quantize(x, shape, axis, bits, scale_mode=ScaleMode.PerBatch, decay=0.0, state=None,
                   round_mode=RoundMode.HalfAway):
     """Host convenience around rlx_mi355x_fake_quantize. Returns (out f32, codes i8, scales f32); EMA updates `state`."""
