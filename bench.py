@@ -261,6 +261,16 @@ def extra_configs(rlx_amd, stream):
         b = gemv_bytes(n, k)
         out[f"q4_0_gemv_{name}"] = {"us": round(ms * 1e3, 3), "GB/s": round(b / ms / 1e6, 1),
                                     "frac_hbm": round(b / ms / 1e6 / HBM_PEAK_GBS, 4), "copies": copies}
+        if name == "gate/up":  # both projections and the SwiGLU in one launch: silu(x . gate^T) * (x . up^T), 66 MB per call
+            def fn_sw():
+                i = state["i"] % (copies // 2)
+                state["i"] += 1
+                rlx_amd._lib.check(L.rlx_mi355x_gguf_matmul_swiglu(x.ptr, int(DType.F32), qws[2 * i].ptr, qws[2 * i + 1].ptr, y.ptr, 1, stream))
+            mss = time_launches(ops, stream, fn_sw, 400, 50)
+            bs = 2 * wbytes + 4 * k + 4 * n
+            out["q4_0_gemv_swiglu_gate+up"] = {"us": round(mss * 1e3, 3), "GB/s": round(bs / mss / 1e6, 1),
+                                               "frac_hbm": round(bs / mss / 1e6 / HBM_PEAK_GBS, 4),
+                                               "note": "one launch; neither projection is written out"}
         if name == "k/v":  # the same projection when its 2.4 MB of weights stay cache-resident (one copy, back to back)
             def fn_warm():
                 rlx_amd._lib.check(L.rlx_mi355x_gguf_matmul_bt(x.ptr, int(DType.F32), qws[0].ptr, y.ptr, 1, None, 0, stream))

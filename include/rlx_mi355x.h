@@ -161,6 +161,12 @@ int rlx_mi355x_qweight_create_experts_at(int scheme, const void *gguf_bytes, siz
  * launch). An index outside [0, num_experts) is clamped to the stack (the reference debug-asserts). */
 int rlx_mi355x_gguf_grouped_matmul_bt(const void *x_dev, int x_dtype, const rlx_qweight *w, const float *expert_idx_dev,
                                       float *out_dev, int64_t m, void *stream);
+/* Two DequantMatMuls feeding Op::FusedSwiGLU (rlx-ir/src/op.rs:1157-1172, executed at rlx-cpu/src/thunk.rs:10337-10366):
+ * out[m, n] = up * (gate / (1 + exp(-gate))) with up = x . W_up^T and gate = x . W_gate^T. Decode path only (m <= 8 f32,
+ * <= 16 bf16 / f16): every workgroup of the decode kernel runs its row tiles through both matrices and combines the two
+ * sums in its epilogue, so neither projection is written out. Both weights must share scheme, n and k. */
+int rlx_mi355x_gguf_matmul_swiglu(const void *x_dev, int x_dtype, const rlx_qweight *w_up, const rlx_qweight *w_gate,
+                                  float *out_dev, int64_t m, void *stream);
 /* rlx_cpu::lm_head::gguf_tied_lm_argmax (rlx-cpu/src/lm_head.rs:223-248): the row of the packed [n_vocab, n_embd] matrix
  * with the largest dot product against one hidden vector, and that dot product. The first maximum wins, a NaN never
  * does, and (0, -inf) comes back when no row beats -inf, as in the reference's loop. The logits are never written: the

@@ -51,6 +51,8 @@ def lib():
         L.orc_dequant.argtypes = [C.c_int, u8p, C.c_int64, C.c_int64, f32p]
         L.orc_dequant_matmul_blocks.restype = C.c_int
         L.orc_dequant_matmul_blocks.argtypes = [C.c_int, u8p, C.c_int64, C.c_int64, f32p]
+        L.orc_fused_swiglu.restype = None
+        L.orc_fused_swiglu.argtypes = [f32p, f32p, C.c_int64, C.c_int64, C.c_int]
         L.orc_gguf_tied_lm_argmax.restype = C.c_int
         L.orc_gguf_tied_lm_argmax.argtypes = [f32p, u8p, C.c_int64, C.c_int64, C.c_int64, C.c_int, u32p, f32p]
         L.orc_gguf_grouped_matmul_bt.restype = C.c_int
@@ -147,6 +149,15 @@ def gguf_matmul_bt(x, packed, m, k, n, scheme):
     if rc != 0:
         raise ValueError("gguf_matmul_bt: bad sizes")
     return out.reshape(m, n)
+
+
+def fused_swiglu(inp, n_half, gate_first=False):
+    """rlx-cpu/src/thunk.rs:10337-10366: rows [up | gate] (or [gate | up]) of 2 n -> rows of n, up * gate / (1 + exp(-gate))."""
+    inp = np.ascontiguousarray(inp, dtype=np.float32)
+    total = inp.size // 2
+    out = np.empty(total, dtype=np.float32)
+    lib().orc_fused_swiglu(_p(inp.reshape(-1), C.c_float), _p(out, C.c_float), n_half, total, int(gate_first))
+    return out.reshape(inp.shape[:-1] + (n_half,))
 
 
 def gguf_tied_lm_argmax(hidden, packed, n_embd, n_vocab, scheme):

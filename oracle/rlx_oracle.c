@@ -22,6 +22,8 @@
  *   gguf_matmul_bt        reference tests rlx-cpu/src/gguf_matmul.rs:238-277 and
  *                         rlx-runtime/tests/dequant_matmul_gguf.rs:176-308
  *                         (layout idx = j*k + p), f64 dense matmul (textbook)
+ *   fused_swiglu          closed forms (gate 0 -> 0, large gate -> up * gate, silu(g) - silu(-g) = g), numpy f64 within
+ *                         2 ulp; the last ulp follows the platform's expf like the reference's f32::exp (unpinned there)
  *   gguf_tied_lm_argmax   the reference's test (rlx-cpu/src/lm_head.rs:306-334: equals the argmax of gguf_matmul_bt's
  *                         logits) + constructed ties, NaN and all -inf rows against the loop's stated rule
  *   fake_quantize         closed forms (channel max -> code +-q_max, all-zero
@@ -415,6 +417,24 @@ int orc_dequant_matmul_blocks(int scheme, const uint8_t *bytes, int64_t nbytes, 
         memcpy(out + i * be, tmp, (size_t)be * sizeof(float));
     }
     return 0;
+}
+
+/* ---- FusedSwiGLU -------------------------------------------------------- */
+
+/* rlx-cpu/src/thunk.rs:10337-10366: input rows of 2 n values, output rows of n; up is the low half unless gate_first. */
+void orc_fused_swiglu(const float *inp, float *out, int64_t n_half, int64_t total, int gate_first) {
+    int64_t n = n_half, outer = total / n;
+    for (int64_t o = 0; o < outer; o++) {
+        const float *in_row = inp + o * 2 * n;
+        float *out_row = out + o * n;
+        for (int64_t i = 0; i < n; i++) {
+            float up = gate_first ? in_row[n + i] : in_row[i];
+            float gate = gate_first ? in_row[i] : in_row[n + i];
+            float den = 1.0f + expf(-gate);
+            float sg = gate / den;
+            out_row[i] = up * sg;
+        }
+    }
 }
 
 /* ---- tied LM head ------------------------------------------------------ */

@@ -32,6 +32,7 @@ struct GemvSeg {
     const void *x;
     float *out;
     int n, k, row_tiles, units, wg_begin, tiles_per_wg, tile_stride;
+    const uint8_t *w_pair;
 };
 struct GemvArgs {
     GemvSeg seg[GEMV_MAX_SEG];
@@ -81,7 +82,8 @@ static int x_kind(int x_dtype) {
 // One decode launch over `count` (<= GEMV_MAX_SEG) matmuls of one scheme, batch and activation dtype; each has
 // its own activations, K and N.
 static int launch_gemv(const void *const *xs, int xk, const rlx_qweight *const *ws, float *const *outs, int count, int m,
-                       hipStream_t stream, const float *expert_idx = nullptr, unsigned long long *argmax_key = nullptr) {
+                       hipStream_t stream, const float *expert_idx = nullptr, unsigned long long *argmax_key = nullptr,
+                       const rlx_qweight *const *pairs = nullptr) {
     const int scheme = ws[0]->scheme;
     const Layout L = layout_of(scheme);
     for (int i = 0; i < count; i++)
@@ -104,7 +106,7 @@ static int launch_gemv(const void *const *xs, int xk, const rlx_qweight *const *
     long long work = 0;  // (tile, unit) items in the launch
     for (int i = 0; i < count; i++) {
         max_units = std::max(max_units, (int)ws[i]->dims.units);
-        work += ws[i]->dims.row_tiles * ws[i]->dims.units;
+        work += ws[i]->dims.row_tiles * ws[i]->dims.units * (pairs ? 2 : 1);
     }
     const int cus = std::max(1, device_props().cu_count);
     const size_t slot_bytes = (size_t)ng * 256;
@@ -132,13 +134,14 @@ static int launch_gemv(const void *const *xs, int xk, const rlx_qweight *const *
         int max_tpw = 1;
         for (int i = 0; i < count; i++) {
             const WeightDims &D = ws[i]->dims;
-            int tpw = (int)std::max<long long>(1, (target_items + D.units / 2) / D.units);
-            tpw = std::min(tpw, tpw_cap);
-            max_tpw = std::max(max_tpw, tpw);
+            const int per_tile = pairs ? 2 : 1;  // partial-sum slots and K runs per row tile
+            int tpw = (int)std::max<long long>(1, (target_items + D.units * per_tile / 2) / (D.units * per_tile));
+            tpw = std::min(tpw, std::max(1, tpw_cap / per_tile));
+            max_tpw = std::max(max_tpw, tpw * per_tile);
             const int seg_wgs = (int)((D.row_tiles + tpw - 1) / tpw);
             static const bool contiguous = getenv("RLX_GEMV_CONTIGUOUS") != nullptr;
             sh.a.seg[i] = GemvSeg{ws[i]->dev, xs[i], outs[i], (int)D.n, (int)D.k, (int)D.row_tiles, (int)D.units, sh.wg, tpw,
-                                  contiguous ? 1 : seg_wgs};
+                                  contiguous ? 1 : seg_wgs, pairs ? pairs[i]->dev : nullptr};
             sh.wg += seg_wgs;
         }
         const size_t part_bytes = (size_t)max_tpw * sh.nwaves * slot_bytes;
@@ -389,6 +392,37 @@ int rlx_mi355x_gguf_matmul_bt_batch(const void *const *xs_dev, int x_dtype, cons
 int rlx_mi355x_gguf_matmul_bt(const void *x_dev, int x_dtype, const rlx_qweight *w, float *out_dev, int64_t m,
                               void *workspace, size_t workspace_bytes, void *stream) {
     return rlx_mi355x_gguf_matmul_bt_batch(&x_dev, x_dtype, &w, &out_dev, 1, m, workspace, workspace_bytes, stream);
+}
+
+int rlx_mi355x_gguf_matmul_swiglu(const void *x_dev, int x_dtype, const rlx_qweight *w_up, const rlx_qweight *w_gate,
+                                  float *out_dev, int64_t m, void *stream) {
+    using namespace rlx;
+    if (!x_dev || !w_up || !w_gate || !out_dev || m <= 0) {
+        set_error("gguf_matmul_swiglu: null argument or m <= 0");
+        return RLX_ERR_INVALID;
+    }
+    int xk = x_kind(x_dtype);
+    if (xk < 0) {
+        set_error("gguf_matmul_swiglu: activation dtype %d is not F32 / BF16 / F16", x_dtype);
+        return RLX_ERR_UNSUPPORTED;
+    }
+    const bool same_layout = w_up->scheme == w_gate->scheme ||
+                             (scheme_is_wide(w_up->scheme) && scheme_is_wide(w_gate->scheme));
+    if (!same_layout || w_up->dims.n != w_gate->dims.n || w_up->dims.k != w_gate->dims.k || w_up->experts != 1 ||
+        w_gate->experts != 1) {
+        set_error("gguf_matmul_swiglu: the up and gate projections must share scheme, n and k");
+        return RLX_ERR_INVALID;
+    }
+    if (m > (xk == 0 ? 8 : 16)) {
+        set_error("gguf_matmul_swiglu: the fused form covers the decode path (m <= %d for this dtype); run two matmuls above it",
+                  xk == 0 ? 8 : 16);
+        return RLX_ERR_UNSUPPORTED;
+    }
+    const void *xs[1] = {x_dev};
+    const rlx_qweight *ws[1] = {w_up};
+    const rlx_qweight *ps[1] = {w_gate};
+    float *outs[1] = {out_dev};
+    return launch_gemv(xs, xk, ws, outs, 1, (int)m, (hipStream_t)stream, nullptr, nullptr, ps);
 }
 
 int rlx_mi355x_gguf_tied_lm_argmax(const void *hidden_dev, int x_dtype, const rlx_qweight *embed, uint32_t *out_idx_dev,

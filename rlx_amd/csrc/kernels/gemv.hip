@@ -30,6 +30,9 @@ struct GemvSeg {
     int wg_begin;      // first workgroup of this segment
     int tiles_per_wg;  // row tiles per workgroup
     int tile_stride;   // distance between a workgroup's tiles: 1 = a contiguous run, else the segment's workgroup count
+    // SwiGLU pairing (rlx-cpu/src/thunk.rs:10337-10366): when set, `w` is the up projection and `w_pair` the gate projection
+    // of the same shape; a workgroup runs each of its tiles through both and writes up * gate / (1 + exp(-gate)).
+    const uint8_t *w_pair;
 };
 
 struct GemvArgs {
@@ -339,17 +342,22 @@ __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
     float *sxs = (float *)(smem + part_bytes + (((size_t)rv * row_stride * 2 + 15) & ~(size_t)15));  // [blk][16]
     const half_t *xrow = xs + min(nrow, rv - 1) * row_stride + g * 8;  // this lane's A row
 
-    for (int i = tid; i < ntiles * nwaves * slot_floats; i += blockDim.x) part[i] = 0.f;
+    for (int i = tid; i < (seg.w_pair ? 2 : 1) * ntiles * nwaves * slot_floats; i += blockDim.x) part[i] = 0.f;
 
-    const uint8_t *wbase = seg.w + (long long)tile0 * seg.units * L.unit_bytes;
+    // With a paired matrix every tile is walked twice, first in `w`, then in `w_pair`: virtual tile vt = 2 t + which.
+    const bool paired = seg.w_pair != nullptr;
+    const int nvt = paired ? 2 * ntiles : ntiles;
     const long long tile_bytes = (long long)seg.units * L.unit_bytes * tstride;  // to this workgroup's next tile
+    const uint8_t *wbase = seg.w + (long long)tile0 * seg.units * L.unit_bytes;
+    const uint8_t *wbase2 = paired ? seg.w_pair + (long long)tile0 * seg.units * L.unit_bytes : wbase;
+    auto vtile_ptr = [&](int vt) { return paired ? ((vt & 1) ? wbase2 : wbase) + (vt >> 1) * tile_bytes : wbase + vt * tile_bytes; };
 
     for (int u0 = 0; u0 < seg.units; u0 += kc_units) {
         const int nu = min(kc_units, seg.units - u0);  // units in this chunk
         // This wave's items: for each tile, units wave, wave + nwaves, ... < nu. Two cursors walk them: `pf_*` issues
         // loads DEPTH items ahead into a register ring, `cu_*` consumes.
         const int my_units = wave < nu ? (nu - wave + nwaves - 1) / nwaves : 0;
-        const int nitems = ntiles * my_units;
+        const int nitems = nvt * my_units;
         int pf_t = 0, pf_u = wave, pf_n = 0;
         const uint8_t *pf_ptr = wbase + (long long)(u0 + wave) * L.unit_bytes;
         UnitRegs<SCHEME> ring[DEPTH];
@@ -362,7 +370,7 @@ __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
                 if (pf_u >= nu) {
                     pf_t++;
                     pf_u = wave;
-                    pf_ptr = wbase + pf_t * tile_bytes + (long long)(u0 + wave) * L.unit_bytes;
+                    pf_ptr = vtile_ptr(pf_t) + (long long)(u0 + wave) * L.unit_bytes;
                 }
             }
         };
@@ -426,11 +434,21 @@ __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
     unsigned long long best = 0;  // below every key a real value produces
     for (int idx = tid; idx < ntiles * a.m * 16; idx += blockDim.x) {
         const int col = idx & 15, mr = (idx >> 4) % a.m, t = idx / (16 * a.m);
-        float sum = 0.f;
-        for (int wv = 0; wv < nwaves; wv++) {
-            const float *slot = part + ((size_t)t * nwaves + wv) * slot_floats + col;
-            sum += slot[mr * 16];
-            if (a.x_dtype == X_F32) sum += slot[(a.m + mr) * 16] * (1.0f / LO_SCALE);
+        auto tile_sum = [&](int vt) {
+            float sum = 0.f;
+            for (int wv = 0; wv < nwaves; wv++) {
+                const float *slot = part + ((size_t)vt * nwaves + wv) * slot_floats + col;
+                sum += slot[mr * 16];
+                if (a.x_dtype == X_F32) sum += slot[(a.m + mr) * 16] * (1.0f / LO_SCALE);
+            }
+            return sum;
+        };
+        float sum;
+        if (paired) {
+            const float up = tile_sum(2 * t), gate = tile_sum(2 * t + 1);
+            sum = up * (gate / (1.0f + expf(-gate)));
+        } else {
+            sum = tile_sum(t);
         }
         const int n_out = (tile0 + t * tstride) * 16 + col;
         if (n_out < seg.n) {

@@ -192,6 +192,15 @@ def gguf_grouped_matmul_bt(x, w: QWeight, expert_idx, x_dtype=DType.F32):
     return od.to_numpy(np.float32).reshape(m, w.n)
 
 
+def gguf_matmul_swiglu(x, w_up: QWeight, w_gate: QWeight, m, x_dtype=DType.F32):
+    """Host convenience: (x . W_up^T) * silu(x . W_gate^T) in one decode launch (Op::FusedSwiGLU over two DequantMatMuls)."""
+    xd = DeviceBuffer.from_numpy(x)
+    od = DeviceBuffer(m * w_up.n * 4)
+    _lib.check(_lib.lib().rlx_mi355x_gguf_matmul_swiglu(xd.ptr, int(x_dtype), w_up.ptr, w_gate.ptr, od.ptr, m, None))
+    sync()
+    return od.to_numpy(np.float32).reshape(m, w_up.n)
+
+
 def gguf_tied_lm_argmax(hidden, embed: QWeight, x_dtype=DType.F32):
     """Host convenience for the tied LM head (rlx-cpu/src/lm_head.rs:223-248): (row, value) of the largest logit of
     hidden . embed^T without materialising the logits."""
