@@ -94,10 +94,14 @@ static int launch_gemv(const void *const *xs, int xk, const rlx_qweight *const *
     const int rv = xk == 0 ? 2 * m : m;
     const int ng = (rv + 3) / 4;
     const bool r2 = rv <= 2;
-    KernelId id = scheme == SCHEME_Q4_0     ? (r2 ? K_GEMV_Q4_0_R2 : K_GEMV_Q4_0_R4)
-                  : scheme == SCHEME_Q8_0   ? (r2 ? K_GEMV_Q8_0_R2 : K_GEMV_Q8_0_R4)
-                  : scheme_is_wide(scheme) ? (r2 ? K_GEMV_F16W_R2 : K_GEMV_F16W_R4)
-                                            : (r2 ? K_GEMV_Q4_K_R2 : K_GEMV_Q4_K_R4);
+    // kernel = scheme family x {r2, r4, r2_argmax, r2_paired, r4_paired}
+    const int family = scheme == SCHEME_Q4_0 ? K_GEMV_Q4_0_R2 : scheme == SCHEME_Q8_0 ? K_GEMV_Q8_0_R2
+                       : scheme_is_wide(scheme) ? K_GEMV_F16W_R2 : K_GEMV_Q4_K_R2;
+    if (argmax_key && !r2) {
+        set_error("gemv: the argmax epilogue takes one activation row");
+        return RLX_ERR_INVALID;
+    }
+    KernelId id = (KernelId)(family + (argmax_key ? 2 : pairs ? (r2 ? 3 : 4) : (r2 ? 0 : 1)));
     static const int env_waves = getenv("RLX_GEMV_WAVES") ? atoi(getenv("RLX_GEMV_WAVES")) : 8;
     static const int env_depth = getenv("RLX_GEMV_DEPTH") ? atoi(getenv("RLX_GEMV_DEPTH")) : 4;
     static const int env_wgs_per_cu = getenv("RLX_GEMV_WGS_PER_CU") ? atoi(getenv("RLX_GEMV_WGS_PER_CU")) : 2;

@@ -301,7 +301,12 @@ extern "C" __global__ void rlx_argmax_finish(unsigned long long *key, uint32_t *
 //     very end, then the slots of all waves are added in a fixed order and written out (deterministic).
 // A launch can carry up to GEMV_MAX_SEG independent matmuls (each with its own activations, K and N): q/k/v and
 // gate/up of a layer, or every projection whose inputs are ready at the same point of the schedule.
-template <int SCHEME, int NREG, int DEPTH>
+// MODE picks the epilogue at compile time, so the plain kernel carries none of the others' code: GEMV_PLAIN writes
+// out; GEMV_ARGMAX merges (value, row) keys (tied LM head); GEMV_PAIRED runs every tile through `w` and `w_pair` and
+// writes the SwiGLU of the two sums.
+enum { GEMV_PLAIN = 0, GEMV_ARGMAX = 1, GEMV_PAIRED = 2 };
+
+template <int SCHEME, int NREG, int DEPTH, int MODE>
 __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
     constexpr Layout L = layout_of(SCHEME);
     constexpr int BLK_PER_UNIT = L.unit_k / 32;
@@ -342,10 +347,10 @@ __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
     float *sxs = (float *)(smem + part_bytes + (((size_t)rv * row_stride * 2 + 15) & ~(size_t)15));  // [blk][16]
     const half_t *xrow = xs + min(nrow, rv - 1) * row_stride + g * 8;  // this lane's A row
 
-    for (int i = tid; i < (seg.w_pair ? 2 : 1) * ntiles * nwaves * slot_floats; i += blockDim.x) part[i] = 0.f;
+    for (int i = tid; i < (MODE == GEMV_PAIRED ? 2 : 1) * ntiles * nwaves * slot_floats; i += blockDim.x) part[i] = 0.f;
 
     // With a paired matrix every tile is walked twice, first in `w`, then in `w_pair`: virtual tile vt = 2 t + which.
-    const bool paired = seg.w_pair != nullptr;
+    constexpr bool paired = MODE == GEMV_PAIRED;
     const int nvt = paired ? 2 * ntiles : ntiles;
     const long long tile_bytes = (long long)seg.units * L.unit_bytes * tstride;  // to this workgroup's next tile
     const uint8_t *wbase = seg.w + (long long)tile0 * seg.units * L.unit_bytes;
@@ -452,14 +457,14 @@ __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
         }
         const int n_out = (tile0 + t * tstride) * 16 + col;
         if (n_out < seg.n) {
-            if (a.argmax_key) {
+            if constexpr (MODE == GEMV_ARGMAX) {
                 if (sum == sum) best = max(best, argmax_key_of(sum, (uint32_t)n_out));  // a NaN never wins (dot > best is false)
             } else {
                 seg.out[(long long)mr * seg.n + n_out] = sum;
             }
         }
     }
-    if (a.argmax_key) {
+    if constexpr (MODE == GEMV_ARGMAX) {
 #pragma unroll
         for (int off = 32; off > 0; off >>= 1) {
             const unsigned long long other = __shfl_xor(best, off);
@@ -474,18 +479,20 @@ __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
 
 }  // namespace rlx
 
-#define RLX_GEMV_INST(name, SCHEME, NREG, DEPTH)                                                            \
+#define RLX_GEMV_INST(name, SCHEME, NREG, DEPTH, MODE)                                                      \
     extern "C" __global__ __launch_bounds__(1024) void name(rlx::GemvArgs a) {                               \
-        rlx::gemv_body<SCHEME, NREG, DEPTH>(a);                                                               \
+        rlx::gemv_body<SCHEME, NREG, DEPTH, MODE>(a);                                                         \
     }
-
 // NREG = 2: at most two virtual rows (m = 1 f32, or m <= 2 16-bit); NREG = 4 otherwise.
-RLX_GEMV_INST(rlx_gemv_q4_0_r2, rlx::SCHEME_Q4_0, 2, 4)
-RLX_GEMV_INST(rlx_gemv_q4_0_r2_d8, rlx::SCHEME_Q4_0, 2, 8)
-RLX_GEMV_INST(rlx_gemv_q4_0_r4, rlx::SCHEME_Q4_0, 4, 4)
-RLX_GEMV_INST(rlx_gemv_q8_0_r2, rlx::SCHEME_Q8_0, 2, 3)
-RLX_GEMV_INST(rlx_gemv_q8_0_r4, rlx::SCHEME_Q8_0, 4, 3)
-RLX_GEMV_INST(rlx_gemv_q4_k_r2, rlx::SCHEME_Q4K, 2, 3)
-RLX_GEMV_INST(rlx_gemv_q4_k_r4, rlx::SCHEME_Q4K, 4, 3)
-RLX_GEMV_INST(rlx_gemv_f16w_r2, rlx::SCHEME_F16W, 2, 2)
-RLX_GEMV_INST(rlx_gemv_f16w_r4, rlx::SCHEME_F16W, 4, 2)
+#define RLX_GEMV_SCHEME(tag, SCHEME, DEPTH)                                           \
+    RLX_GEMV_INST(rlx_gemv_##tag##_r2, SCHEME, 2, DEPTH, rlx::GEMV_PLAIN)             \
+    RLX_GEMV_INST(rlx_gemv_##tag##_r4, SCHEME, 4, DEPTH, rlx::GEMV_PLAIN)             \
+    RLX_GEMV_INST(rlx_gemv_##tag##_r2_argmax, SCHEME, 2, DEPTH, rlx::GEMV_ARGMAX)     \
+    RLX_GEMV_INST(rlx_gemv_##tag##_r2_paired, SCHEME, 2, DEPTH, rlx::GEMV_PAIRED)     \
+    RLX_GEMV_INST(rlx_gemv_##tag##_r4_paired, SCHEME, 4, DEPTH, rlx::GEMV_PAIRED)
+
+RLX_GEMV_SCHEME(q4_0, rlx::SCHEME_Q4_0, 4)
+RLX_GEMV_SCHEME(q8_0, rlx::SCHEME_Q8_0, 3)
+RLX_GEMV_SCHEME(q4_k, rlx::SCHEME_Q4K, 3)
+RLX_GEMV_SCHEME(f16w, rlx::SCHEME_F16W, 2)
+RLX_GEMV_INST(rlx_gemv_q4_0_r2_d8, rlx::SCHEME_Q4_0, 2, 8, rlx::GEMV_PLAIN)
