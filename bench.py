@@ -17,6 +17,8 @@ import os
 import sys
 import time
 
+import ctypes as C
+
 import numpy as np
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
@@ -277,6 +279,42 @@ def extra_configs(rlx_amd, stream):
             msw = time_launches(ops, stream, fn_warm, 400, 50)
             out["q4_0_gemv_k/v_warm"] = {"us": round(msw * 1e3, 3), "GB/s": round(b / msw / 1e6, 1)}
         for q in qws:
+            q.free()
+    # one Llama-3-8B layer the way a decode loop runs it: four launches that include both RMSNorms and the SwiGLU
+    # (norm + q,k,v | o | norm + gate,up + SwiGLU | down), five rotating weight sets (615 MB), f32 activations
+    shapes = [("q", 4096, 4096), ("k", 1024, 4096), ("v", 1024, 4096), ("o", 4096, 4096), ("gate", 14336, 4096),
+              ("up", 14336, 4096), ("down", 4096, 14336)]
+    base = {}
+    for name, n, k in shapes:
+        w = (ops.philox_normal(31 + len(base), n * k) * np.float32(0.02)).astype(np.float32)
+        base[name] = ops.quantize(QuantScheme.GgufQ4_0, w).reshape(n, -1)
+    sets = [{name: ops.QWeight(QuantScheme.GgufQ4_0, np.roll(base[name], 3 * i, axis=0).reshape(-1), n, k) for name, n, k in shapes}
+            for i in range(5)]
+    del base
+    x4 = ops.DeviceBuffer.from_numpy(ops.philox_normal(41, 4096))
+    x14 = ops.DeviceBuffer.from_numpy(ops.philox_normal(42, 14336))
+    gam = ops.DeviceBuffer.from_numpy(np.ones(4096, np.float32))
+    oq, ok_, ov, oo, oh, od = (ops.DeviceBuffer(4 * n) for n in (4096, 1024, 1024, 4096, 14336, 4096))
+    state = {"i": 0}
+
+    def fn_layer():
+        ws = sets[state["i"] % len(sets)]
+        state["i"] += 1
+        wp = (C.c_void_p * 3)(ws["q"].ptr, ws["k"].ptr, ws["v"].ptr)
+        op = (C.c_void_p * 3)(oq.ptr, ok_.ptr, ov.ptr)
+        chk = rlx_amd._lib.check
+        chk(L.rlx_mi355x_rmsnorm_gguf_matmul_bt_batch(x4.ptr, gam.ptr, None, 1e-5, wp, op, 3, 1, stream))
+        chk(L.rlx_mi355x_gguf_matmul_bt(x4.ptr, int(DType.F32), ws["o"].ptr, oo.ptr, 1, None, 0, stream))
+        chk(L.rlx_mi355x_rmsnorm_gguf_matmul_swiglu(x4.ptr, gam.ptr, None, 1e-5, ws["up"].ptr, ws["gate"].ptr, oh.ptr, 1, stream))
+        chk(L.rlx_mi355x_gguf_matmul_bt(x14.ptr, int(DType.F32), ws["down"].ptr, od.ptr, 1, None, 0, stream))
+
+    ms = time_launches(ops, stream, fn_layer, 300, 30)
+    lb = sum(n * k // 32 * 18 for _, n, k in shapes)
+    out["q4_0_llama8b_layer_with_norms_and_swiglu"] = {"us": round(ms * 1e3, 2), "GB/s": round(lb / ms / 1e6, 1),
+                                                       "frac_hbm": round(lb / ms / 1e6 / HBM_PEAK_GBS, 4), "launches_per_layer": 4,
+                                                       "note": "rmsnorm+qkv | o | rmsnorm+gate,up+swiglu | down; no other kernels needed between them"}
+    for ws in sets:
+        for q in ws.values():
             q.free()
     # config 1: Q8_0 GEMV 4096x4096
     n = k = 4096

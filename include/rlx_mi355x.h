@@ -167,6 +167,22 @@ int rlx_mi355x_gguf_grouped_matmul_bt(const void *x_dev, int x_dtype, const rlx_
  * sums in its epilogue, so neither projection is written out. Both weights must share scheme, n and k. */
 int rlx_mi355x_gguf_matmul_swiglu(const void *x_dev, int x_dtype, const rlx_qweight *w_up, const rlx_qweight *w_gate,
                                   float *out_dev, int64_t m, void *stream);
+/* Op::RmsNorm (executed at rlx-cpu/src/thunk.rs:8839-8869: y = x * (1 / sqrt(mean(x^2) + eps)) * gamma + beta, per row)
+ * feeding DequantMatMuls, fused into the decode kernel's activation staging: every workgroup sums the squares of the
+ * rows it multiplies and normalizes while it converts them, so the normalized vector never reaches memory and its launch
+ * is gone. f32 activations, m <= 8; `beta_dev` may be NULL (zeros); gamma / beta are [k] f32, 16-byte aligned.
+ *   ..._bt_batch: `count` matrices of one scheme and k over the same normalized x (q, k, v of a layer);
+ *   ..._swiglu:   the normalized x through up and gate, combined as in rlx_mi355x_gguf_matmul_swiglu;
+ *   ..._tied_lm_argmax: the final norm in front of the LM head argmax. */
+int rlx_mi355x_rmsnorm_gguf_matmul_bt_batch(const float *x_dev, const float *gamma_dev, const float *beta_dev, float eps,
+                                            const rlx_qweight *const *ws, float *const *outs_dev, int count, int64_t m,
+                                            void *stream);
+int rlx_mi355x_rmsnorm_gguf_matmul_swiglu(const float *x_dev, const float *gamma_dev, const float *beta_dev, float eps,
+                                          const rlx_qweight *w_up, const rlx_qweight *w_gate, float *out_dev, int64_t m,
+                                          void *stream);
+int rlx_mi355x_rmsnorm_gguf_tied_lm_argmax(const float *hidden_dev, const float *gamma_dev, const float *beta_dev, float eps,
+                                           const rlx_qweight *embed, uint32_t *out_idx_dev, float *out_val_dev,
+                                           void *key_scratch_dev, void *stream);
 /* rlx_cpu::lm_head::gguf_tied_lm_argmax (rlx-cpu/src/lm_head.rs:223-248): the row of the packed [n_vocab, n_embd] matrix
  * with the largest dot product against one hidden vector, and that dot product. The first maximum wins, a NaN never
  * does, and (0, -inf) comes back when no row beats -inf, as in the reference's loop. The logits are never written: the

@@ -51,6 +51,8 @@ def lib():
         L.orc_dequant.argtypes = [C.c_int, u8p, C.c_int64, C.c_int64, f32p]
         L.orc_dequant_matmul_blocks.restype = C.c_int
         L.orc_dequant_matmul_blocks.argtypes = [C.c_int, u8p, C.c_int64, C.c_int64, f32p]
+        L.orc_rms_norm.restype = None
+        L.orc_rms_norm.argtypes = [f32p, f32p, f32p, f32p, C.c_int64, C.c_int64, C.c_float]
         L.orc_fused_swiglu.restype = None
         L.orc_fused_swiglu.argtypes = [f32p, f32p, C.c_int64, C.c_int64, C.c_int]
         L.orc_gguf_tied_lm_argmax.restype = C.c_int
@@ -149,6 +151,18 @@ def gguf_matmul_bt(x, packed, m, k, n, scheme):
     if rc != 0:
         raise ValueError("gguf_matmul_bt: bad sizes")
     return out.reshape(m, n)
+
+
+def rms_norm(x, gamma, beta, eps):
+    """rlx-cpu/src/thunk.rs:8839-8869 over the last axis."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    h = x.shape[-1]
+    gamma = np.ascontiguousarray(gamma, dtype=np.float32)
+    beta = np.zeros(h, np.float32) if beta is None else np.ascontiguousarray(beta, dtype=np.float32)
+    out = np.empty_like(x)
+    lib().orc_rms_norm(_p(x.reshape(-1), C.c_float), _p(gamma, C.c_float), _p(beta, C.c_float), _p(out.reshape(-1), C.c_float),
+                       x.size // h, h, eps)
+    return out
 
 
 def fused_swiglu(inp, n_half, gate_first=False):

@@ -22,6 +22,8 @@
  *   gguf_matmul_bt        reference tests rlx-cpu/src/gguf_matmul.rs:238-277 and
  *                         rlx-runtime/tests/dequant_matmul_gguf.rs:176-308
  *                         (layout idx = j*k + p), f64 dense matmul (textbook)
+ *   rms_norm              closed forms (constant row -> +-gamma + beta up to eps, scale invariance, eps only on a zero row),
+ *                         numpy f64 within a few ulp
  *   fused_swiglu          closed forms (gate 0 -> 0, large gate -> up * gate, silu(g) - silu(-g) = g), numpy f64 within
  *                         2 ulp; the last ulp follows the platform's expf like the reference's f32::exp (unpinned there)
  *   gguf_tied_lm_argmax   the reference's test (rlx-cpu/src/lm_head.rs:306-334: equals the argmax of gguf_matmul_bt's
@@ -417,6 +419,29 @@ int orc_dequant_matmul_blocks(int scheme, const uint8_t *bytes, int64_t nbytes, 
         memcpy(out + i * be, tmp, (size_t)be * sizeof(float));
     }
     return 0;
+}
+
+/* ---- RmsNorm ------------------------------------------------------------ */
+
+/* rlx-cpu/src/thunk.rs:8839-8869 */
+void orc_rms_norm(const float *input, const float *gamma, const float *beta, float *output, int64_t rows, int64_t h, float eps) {
+    float inv_h = 1.0f / (float)h;
+    for (int64_t row = 0; row < rows; row++) {
+        const float *in_row = input + row * h;
+        float *out_row = output + row * h;
+        float sumsq = 0.0f;
+        for (int64_t i = 0; i < h; i++) {
+            float sq = in_row[i] * in_row[i];
+            sumsq += sq;
+        }
+        float mean = sumsq * inv_h;
+        float inv_rms = 1.0f / sqrtf(mean + eps);
+        for (int64_t i = 0; i < h; i++) {
+            float t = in_row[i] * inv_rms;
+            t = t * gamma[i];
+            out_row[i] = t + beta[i];
+        }
+    }
 }
 
 /* ---- FusedSwiGLU -------------------------------------------------------- */

@@ -41,6 +41,14 @@ struct GemvArgs {
     long long slab_bytes;
     int num_experts;
     unsigned long long *argmax_key;
+    const float *gamma;
+    const float *beta;
+    float eps;
+    int lds_bytes;
+};
+struct RmsNorm {  // RMSNorm prologue of a decode launch (f32 activations only)
+    const float *gamma, *beta;
+    float eps;
 };
 struct FqArgs {
     const float *x;
@@ -83,7 +91,7 @@ static int x_kind(int x_dtype) {
 // its own activations, K and N.
 static int launch_gemv(const void *const *xs, int xk, const rlx_qweight *const *ws, float *const *outs, int count, int m,
                        hipStream_t stream, const float *expert_idx = nullptr, unsigned long long *argmax_key = nullptr,
-                       const rlx_qweight *const *pairs = nullptr) {
+                       const rlx_qweight *const *pairs = nullptr, const RmsNorm *norm = nullptr) {
     const int scheme = ws[0]->scheme;
     const Layout L = layout_of(scheme);
     for (int i = 0; i < count; i++)
@@ -101,7 +109,12 @@ static int launch_gemv(const void *const *xs, int xk, const rlx_qweight *const *
         set_error("gemv: the argmax epilogue takes one activation row");
         return RLX_ERR_INVALID;
     }
-    KernelId id = (KernelId)(family + (argmax_key ? 2 : pairs ? (r2 ? 3 : 4) : (r2 ? 0 : 1)));
+    if (norm && xk != 0) {
+        set_error("gemv: the RMSNorm prologue takes f32 activations");
+        return RLX_ERR_UNSUPPORTED;
+    }
+    const int variant = argmax_key ? (norm ? 9 : 2) : pairs ? (norm ? (r2 ? 7 : 8) : (r2 ? 3 : 4)) : (norm ? (r2 ? 5 : 6) : (r2 ? 0 : 1));
+    KernelId id = (KernelId)(family + variant);
     static const int env_waves = getenv("RLX_GEMV_WAVES") ? atoi(getenv("RLX_GEMV_WAVES")) : 8;
     static const int env_depth = getenv("RLX_GEMV_DEPTH") ? atoi(getenv("RLX_GEMV_DEPTH")) : 4;
     static const int env_wgs_per_cu = getenv("RLX_GEMV_WGS_PER_CU") ? atoi(getenv("RLX_GEMV_WGS_PER_CU")) : 2;
@@ -150,9 +163,9 @@ static int launch_gemv(const void *const *xs, int xk, const rlx_qweight *const *
         }
         const size_t part_bytes = (size_t)max_tpw * sh.nwaves * slot_bytes;
         sh.kcu = max_units;
-        while (sh.kcu > 1 && part_bytes + stage_bytes(sh.kcu) > budget) sh.kcu--;
-        sh.fits = part_bytes + stage_bytes(sh.kcu) <= budget;
-        sh.lds = part_bytes + stage_bytes(sh.kcu);
+        while (sh.kcu > 1 && part_bytes + stage_bytes(sh.kcu) + 64 > budget) sh.kcu--;
+        sh.fits = part_bytes + stage_bytes(sh.kcu) + 64 <= budget;
+        sh.lds = part_bytes + stage_bytes(sh.kcu) + 64;  // the last 64 bytes: 1 / rms per activation row (RMSNorm prologue)
         sh.a.nseg = count;
         sh.a.m = m;
         sh.a.kc_units = sh.kcu;
@@ -160,6 +173,10 @@ static int launch_gemv(const void *const *xs, int xk, const rlx_qweight *const *
         sh.a.max_tiles_per_wg = max_tpw;
         sh.a.expert_idx = expert_idx;
         sh.a.argmax_key = argmax_key;
+        sh.a.gamma = norm ? norm->gamma : nullptr;
+        sh.a.beta = norm ? norm->beta : nullptr;
+        sh.a.eps = norm ? norm->eps : 0.f;
+        sh.a.lds_bytes = (int)sh.lds;
         sh.a.slab_bytes = ws[0]->dims.bytes;
         sh.a.num_experts = ws[0]->experts;
         return sh;
@@ -396,6 +413,94 @@ int rlx_mi355x_gguf_matmul_bt_batch(const void *const *xs_dev, int x_dtype, cons
 int rlx_mi355x_gguf_matmul_bt(const void *x_dev, int x_dtype, const rlx_qweight *w, float *out_dev, int64_t m,
                               void *workspace, size_t workspace_bytes, void *stream) {
     return rlx_mi355x_gguf_matmul_bt_batch(&x_dev, x_dtype, &w, &out_dev, 1, m, workspace, workspace_bytes, stream);
+}
+
+// Shared checks of the RMSNorm-prologue entry points: f32 activations, decode sizes, 16-byte aligned gamma / beta.
+static int check_norm(const char *who, const void *x_dev, const float *gamma_dev, const float *beta_dev, int64_t m) {
+    if (!x_dev || !gamma_dev || m <= 0) {
+        rlx::set_error("%s: null argument or m <= 0", who);
+        return RLX_ERR_INVALID;
+    }
+    if (m > 8) {
+        rlx::set_error("%s: the fused RMSNorm covers the decode path (m <= 8 f32 rows)", who);
+        return RLX_ERR_UNSUPPORTED;
+    }
+    if ((uintptr_t)gamma_dev % 16 != 0 || (uintptr_t)beta_dev % 16 != 0) {
+        rlx::set_error("%s: gamma and beta must be 16-byte aligned", who);
+        return RLX_ERR_INVALID;
+    }
+    return RLX_OK;
+}
+
+int rlx_mi355x_rmsnorm_gguf_matmul_bt_batch(const float *x_dev, const float *gamma_dev, const float *beta_dev, float eps,
+                                            const rlx_qweight *const *ws, float *const *outs_dev, int count, int64_t m,
+                                            void *stream) {
+    using namespace rlx;
+    RLX_TRY(check_norm("rmsnorm_gguf_matmul_bt_batch", x_dev, gamma_dev, beta_dev, m));
+    if (!ws || !outs_dev || count <= 0) {
+        set_error("rmsnorm_gguf_matmul_bt_batch: null argument or count <= 0");
+        return RLX_ERR_INVALID;
+    }
+    const RmsNorm norm{gamma_dev, beta_dev, eps};
+    for (int i0 = 0; i0 < count; i0 += GEMV_MAX_SEG) {
+        const int c = std::min(GEMV_MAX_SEG, count - i0);
+        const void *xs[GEMV_MAX_SEG];
+        for (int i = 0; i < c; i++) {
+            if (!ws[i0 + i] || !outs_dev[i0 + i] || ws[i0 + i]->experts != 1) {
+                set_error("rmsnorm_gguf_matmul_bt_batch: null weight / output or an expert stack at %d", i0 + i);
+                return RLX_ERR_INVALID;
+            }
+            const bool same = ws[i0 + i]->scheme == ws[i0]->scheme || (scheme_is_wide(ws[i0 + i]->scheme) && scheme_is_wide(ws[i0]->scheme));
+            if (!same || ws[i0 + i]->dims.k != ws[0]->dims.k) {
+                set_error("rmsnorm_gguf_matmul_bt_batch: the matrices share one normalized input, so one scheme and one k");
+                return RLX_ERR_INVALID;
+            }
+            xs[i] = x_dev;
+        }
+        RLX_TRY(launch_gemv(xs, 0, ws + i0, outs_dev + i0, c, (int)m, (hipStream_t)stream, nullptr, nullptr, nullptr, &norm));
+    }
+    return RLX_OK;
+}
+
+int rlx_mi355x_rmsnorm_gguf_matmul_swiglu(const float *x_dev, const float *gamma_dev, const float *beta_dev, float eps,
+                                          const rlx_qweight *w_up, const rlx_qweight *w_gate, float *out_dev, int64_t m,
+                                          void *stream) {
+    using namespace rlx;
+    RLX_TRY(check_norm("rmsnorm_gguf_matmul_swiglu", x_dev, gamma_dev, beta_dev, m));
+    if (!w_up || !w_gate || !out_dev) {
+        set_error("rmsnorm_gguf_matmul_swiglu: null argument");
+        return RLX_ERR_INVALID;
+    }
+    const bool same_layout = w_up->scheme == w_gate->scheme || (scheme_is_wide(w_up->scheme) && scheme_is_wide(w_gate->scheme));
+    if (!same_layout || w_up->dims.n != w_gate->dims.n || w_up->dims.k != w_gate->dims.k || w_up->experts != 1 ||
+        w_gate->experts != 1) {
+        set_error("rmsnorm_gguf_matmul_swiglu: the up and gate projections must share scheme, n and k");
+        return RLX_ERR_INVALID;
+    }
+    const RmsNorm norm{gamma_dev, beta_dev, eps};
+    const void *xs[1] = {x_dev};
+    const rlx_qweight *ws[1] = {w_up};
+    const rlx_qweight *ps[1] = {w_gate};
+    float *outs[1] = {out_dev};
+    return launch_gemv(xs, 0, ws, outs, 1, (int)m, (hipStream_t)stream, nullptr, nullptr, ps, &norm);
+}
+
+int rlx_mi355x_rmsnorm_gguf_tied_lm_argmax(const float *hidden_dev, const float *gamma_dev, const float *beta_dev, float eps,
+                                           const rlx_qweight *embed, uint32_t *out_idx_dev, float *out_val_dev,
+                                           void *key_scratch_dev, void *stream) {
+    using namespace rlx;
+    RLX_TRY(check_norm("rmsnorm_gguf_tied_lm_argmax", hidden_dev, gamma_dev, beta_dev, 1));
+    if (!embed || !out_idx_dev || !out_val_dev || !key_scratch_dev || (uintptr_t)key_scratch_dev % 8 != 0) {
+        set_error("rmsnorm_gguf_tied_lm_argmax: null argument or misaligned key scratch");
+        return RLX_ERR_INVALID;
+    }
+    const RmsNorm norm{gamma_dev, beta_dev, eps};
+    const void *xs[1] = {hidden_dev};
+    const rlx_qweight *ws[1] = {embed};
+    float *outs[1] = {nullptr};
+    RLX_TRY(launch_gemv(xs, 0, ws, outs, 1, 1, (hipStream_t)stream, nullptr, (unsigned long long *)key_scratch_dev, nullptr, &norm));
+    void *params[] = {&key_scratch_dev, &out_idx_dev, &out_val_dev};
+    return launch(K_ARGMAX_FINISH, 1, 1, 64, 0, (hipStream_t)stream, params);
 }
 
 int rlx_mi355x_gguf_matmul_swiglu(const void *x_dev, int x_dtype, const rlx_qweight *w_up, const rlx_qweight *w_gate,

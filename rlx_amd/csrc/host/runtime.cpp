@@ -27,9 +27,13 @@ static const char *const kKernelNames[K_COUNT] = {
     "rlx_fq_flat_apply", "rlx_fq_flat4_apply",
     "rlx_fill_u32", "rlx_copy_u128",
     "rlx_gemv_q4_0_r2", "rlx_gemv_q4_0_r4", "rlx_gemv_q4_0_r2_argmax", "rlx_gemv_q4_0_r2_paired", "rlx_gemv_q4_0_r4_paired",
+    "rlx_gemv_q4_0_r2_norm", "rlx_gemv_q4_0_r4_norm", "rlx_gemv_q4_0_r2_norm_paired", "rlx_gemv_q4_0_r4_norm_paired", "rlx_gemv_q4_0_r2_norm_argmax",
     "rlx_gemv_q8_0_r2", "rlx_gemv_q8_0_r4", "rlx_gemv_q8_0_r2_argmax", "rlx_gemv_q8_0_r2_paired", "rlx_gemv_q8_0_r4_paired",
+    "rlx_gemv_q8_0_r2_norm", "rlx_gemv_q8_0_r4_norm", "rlx_gemv_q8_0_r2_norm_paired", "rlx_gemv_q8_0_r4_norm_paired", "rlx_gemv_q8_0_r2_norm_argmax",
     "rlx_gemv_q4_k_r2", "rlx_gemv_q4_k_r4", "rlx_gemv_q4_k_r2_argmax", "rlx_gemv_q4_k_r2_paired", "rlx_gemv_q4_k_r4_paired",
+    "rlx_gemv_q4_k_r2_norm", "rlx_gemv_q4_k_r4_norm", "rlx_gemv_q4_k_r2_norm_paired", "rlx_gemv_q4_k_r4_norm_paired", "rlx_gemv_q4_k_r2_norm_argmax",
     "rlx_gemv_f16w_r2", "rlx_gemv_f16w_r4", "rlx_gemv_f16w_r2_argmax", "rlx_gemv_f16w_r2_paired", "rlx_gemv_f16w_r4_paired",
+    "rlx_gemv_f16w_r2_norm", "rlx_gemv_f16w_r4_norm", "rlx_gemv_f16w_r2_norm_paired", "rlx_gemv_f16w_r4_norm_paired", "rlx_gemv_f16w_r2_norm_argmax",
     "rlx_gemv_q4_0_r2_d8",
     "rlx_gemm_q4_k", "rlx_gemm_q4_0", "rlx_gemm_q8_0", "rlx_gemm64_q4_k", "rlx_gemm64_q4_0", "rlx_gemm64_q8_0", "rlx_gemm_f16w", "rlx_gemm64_f16w", "rlx_xprep", "rlx_argmax_finish",
 };

@@ -51,6 +51,12 @@ struct GemvArgs {
     // workgroup folds its outputs into one 64-bit key (ordered value bits, then ~row so that the first maximum wins) and
     // merges it with an atomic max.
     unsigned long long *argmax_key;
+    // RMSNorm prologue (rlx-cpu/src/thunk.rs:8839-8869) in the kernels built with GEMV_NORM: the f32 activations are
+    // x * (1 / sqrt(mean(x^2) + eps)) * gamma + beta (beta may be null) before they are split into halfs.
+    const float *gamma;
+    const float *beta;
+    float eps;
+    int lds_bytes;     // dynamic LDS of the launch
 };
 
 constexpr int XS_PAD_HALFS = 8;      // 16 bytes of padding per LDS row: rows land in different bank groups
@@ -207,8 +213,9 @@ __device__ __forceinline__ void compute_unit(const UnitRegs<SCHEME> &w, const ha
 // Convert one K chunk of the activations into LDS as halfs: f32 -> hi rows [0,m) + lo rows [m,2m); 16-bit -> rows [0,m).
 // Each thread issues up to eight independent loads before it converts the first one, so a chunk of many rows costs
 // one memory latency per eight groups of columns, not one per group.
-template <int XD>
-__device__ __forceinline__ void stage_x_typed(const GemvArgs &a, const GemvSeg &sg, half_t *xs, int row_stride, int k0, int kc) {
+template <int XD, bool NORM = false>
+__device__ __forceinline__ void stage_x_typed(const GemvArgs &a, const GemvSeg &sg, half_t *xs, int row_stride, int k0, int kc,
+                                              const float *inv_rms = nullptr) {
     constexpr int U = 8;
     constexpr int G = XD == X_F32 ? 4 : 8;  // columns per 16-byte load
     typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
@@ -236,9 +243,19 @@ __device__ __forceinline__ void stage_x_typed(const GemvArgs &a, const GemvSeg &
             const int row = idx / groups, c = (idx - row * groups) * G;
             if constexpr (XD == X_F32) {
                 half4_t hi, lo;
+                float4_t gm = {1.f, 1.f, 1.f, 1.f}, bt = {0.f, 0.f, 0.f, 0.f};
+                float scale = 1.f;
+                if constexpr (NORM) {
+                    scale = inv_rms[row];
+                    if (k0 + c < sg.k) {
+                        gm = *(const float4_t *)(a.gamma + k0 + c);
+                        if (a.beta) bt = *(const float4_t *)(a.beta + k0 + c);
+                    }
+                }
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
-                    const float v = raw[u][e];
+                    float v = raw[u][e];
+                    if constexpr (NORM) v = v * scale * gm[e] + bt[e];  // in_row[i] * inv_rms * gamma[i] + beta[i], unfused
                     hi[e] = (half_t)v;
                     // residual, scaled by 2^11 so it stays in the normal binary16 range; undone in the final sum
                     lo[e] = (half_t)((v - (float)hi[e]) * LO_SCALE);
@@ -304,7 +321,7 @@ extern "C" __global__ void rlx_argmax_finish(unsigned long long *key, uint32_t *
 // MODE picks the epilogue at compile time, so the plain kernel carries none of the others' code: GEMV_PLAIN writes
 // out; GEMV_ARGMAX merges (value, row) keys (tied LM head); GEMV_PAIRED runs every tile through `w` and `w_pair` and
 // writes the SwiGLU of the two sums.
-enum { GEMV_PLAIN = 0, GEMV_ARGMAX = 1, GEMV_PAIRED = 2 };
+enum { GEMV_PLAIN = 0, GEMV_ARGMAX = 1, GEMV_PAIRED = 2, GEMV_NORM = 4 };  // GEMV_NORM combines with the others
 
 template <int SCHEME, int NREG, int DEPTH, int MODE>
 __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
@@ -347,10 +364,27 @@ __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
     float *sxs = (float *)(smem + part_bytes + (((size_t)rv * row_stride * 2 + 15) & ~(size_t)15));  // [blk][16]
     const half_t *xrow = xs + min(nrow, rv - 1) * row_stride + g * 8;  // this lane's A row
 
-    for (int i = tid; i < (MODE == GEMV_PAIRED ? 2 : 1) * ntiles * nwaves * slot_floats; i += blockDim.x) part[i] = 0.f;
+    for (int i = tid; i < ((MODE & GEMV_PAIRED) ? 2 : 1) * ntiles * nwaves * slot_floats; i += blockDim.x) part[i] = 0.f;
+    // RMSNorm prologue: one wave per activation row sums the squares of the whole row (the sum is needed before any
+    // element can be scaled), 1 / sqrt(mean + eps) lands in the last 64 bytes of the workgroup's LDS.
+    float *inv_rms = (float *)(smem + a.lds_bytes - 64);
+    if constexpr ((MODE & GEMV_NORM) != 0) {
+        for (int row = wave; row < a.m; row += nwaves) {
+            const float *xr = (const float *)seg.x + (long long)row * seg.k;
+            float sq = 0.f;
+            for (int c = l * 4; c < seg.k; c += 256) {
+                const float4_t v = *(const float4_t *)(xr + c);
+                sq += v[0] * v[0] + v[1] * v[1] + v[2] * v[2] + v[3] * v[3];
+            }
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) sq += __shfl_xor(sq, off);
+            if (l == 0) inv_rms[row] = 1.0f / sqrtf(sq * (1.0f / (float)seg.k) + a.eps);
+        }
+        __syncthreads();
+    }
 
     // With a paired matrix every tile is walked twice, first in `w`, then in `w_pair`: virtual tile vt = 2 t + which.
-    constexpr bool paired = MODE == GEMV_PAIRED;
+    constexpr bool paired = (MODE & GEMV_PAIRED) != 0;
     const int nvt = paired ? 2 * ntiles : ntiles;
     const long long tile_bytes = (long long)seg.units * L.unit_bytes * tstride;  // to this workgroup's next tile
     const uint8_t *wbase = seg.w + (long long)tile0 * seg.units * L.unit_bytes;
@@ -385,7 +419,8 @@ __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
             prefetch(ring[d]);
         }
         if (u0 > 0) __syncthreads();  // previous chunk fully consumed
-        stage_x(a, seg, xs, row_stride, u0 * L.unit_k, nu * L.unit_k);
+        if constexpr ((MODE & GEMV_NORM) != 0) stage_x_typed<X_F32, true>(a, seg, xs, row_stride, u0 * L.unit_k, nu * L.unit_k, inv_rms);
+        else stage_x(a, seg, xs, row_stride, u0 * L.unit_k, nu * L.unit_k);
         __syncthreads();
         if constexpr (SCHEME == SCHEME_Q4K) {
             const int nblk = nu * BLK_PER_UNIT;
@@ -457,14 +492,14 @@ __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
         }
         const int n_out = (tile0 + t * tstride) * 16 + col;
         if (n_out < seg.n) {
-            if constexpr (MODE == GEMV_ARGMAX) {
+            if constexpr ((MODE & GEMV_ARGMAX) != 0) {
                 if (sum == sum) best = max(best, argmax_key_of(sum, (uint32_t)n_out));  // a NaN never wins (dot > best is false)
             } else {
                 seg.out[(long long)mr * seg.n + n_out] = sum;
             }
         }
     }
-    if constexpr (MODE == GEMV_ARGMAX) {
+    if constexpr ((MODE & GEMV_ARGMAX) != 0) {
 #pragma unroll
         for (int off = 32; off > 0; off >>= 1) {
             const unsigned long long other = __shfl_xor(best, off);
@@ -489,7 +524,12 @@ __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
     RLX_GEMV_INST(rlx_gemv_##tag##_r4, SCHEME, 4, DEPTH, rlx::GEMV_PLAIN)             \
     RLX_GEMV_INST(rlx_gemv_##tag##_r2_argmax, SCHEME, 2, DEPTH, rlx::GEMV_ARGMAX)     \
     RLX_GEMV_INST(rlx_gemv_##tag##_r2_paired, SCHEME, 2, DEPTH, rlx::GEMV_PAIRED)     \
-    RLX_GEMV_INST(rlx_gemv_##tag##_r4_paired, SCHEME, 4, DEPTH, rlx::GEMV_PAIRED)
+    RLX_GEMV_INST(rlx_gemv_##tag##_r4_paired, SCHEME, 4, DEPTH, rlx::GEMV_PAIRED)     \
+    RLX_GEMV_INST(rlx_gemv_##tag##_r2_norm, SCHEME, 2, DEPTH, rlx::GEMV_NORM)         \
+    RLX_GEMV_INST(rlx_gemv_##tag##_r4_norm, SCHEME, 4, DEPTH, rlx::GEMV_NORM)         \
+    RLX_GEMV_INST(rlx_gemv_##tag##_r2_norm_paired, SCHEME, 2, DEPTH, rlx::GEMV_NORM | rlx::GEMV_PAIRED) \
+    RLX_GEMV_INST(rlx_gemv_##tag##_r4_norm_paired, SCHEME, 4, DEPTH, rlx::GEMV_NORM | rlx::GEMV_PAIRED) \
+    RLX_GEMV_INST(rlx_gemv_##tag##_r2_norm_argmax, SCHEME, 2, DEPTH, rlx::GEMV_NORM | rlx::GEMV_ARGMAX)
 
 RLX_GEMV_SCHEME(q4_0, rlx::SCHEME_Q4_0, 4)
 RLX_GEMV_SCHEME(q8_0, rlx::SCHEME_Q8_0, 3)

@@ -201,6 +201,45 @@ def gguf_matmul_swiglu(x, w_up: QWeight, w_gate: QWeight, m, x_dtype=DType.F32):
     return od.to_numpy(np.float32).reshape(m, w_up.n)
 
 
+def _norm_bufs(gamma, beta):
+    g = DeviceBuffer.from_numpy(np.ascontiguousarray(gamma, dtype=np.float32))
+    b = DeviceBuffer.from_numpy(np.ascontiguousarray(beta, dtype=np.float32)) if beta is not None else None
+    return g, b
+
+
+def rmsnorm_gguf_matmul_bt_batch(x, gamma, beta, eps, ws, m):
+    """Host convenience: RMSNorm(x) . W_i^T for every W_i of `ws` in one decode launch per eight matrices."""
+    xd = DeviceBuffer.from_numpy(np.ascontiguousarray(x, dtype=np.float32))
+    g, b = _norm_bufs(gamma, beta)
+    outs = [DeviceBuffer(m * w.n * 4) for w in ws]
+    wp = (C.c_void_p * len(ws))(*[w.ptr for w in ws])
+    op = (C.c_void_p * len(ws))(*[o.ptr for o in outs])
+    _lib.check(_lib.lib().rlx_mi355x_rmsnorm_gguf_matmul_bt_batch(xd.ptr, g.ptr, b.ptr if b else None, eps, wp, op, len(ws), m, None))
+    sync()
+    return [o.to_numpy(np.float32).reshape(m, w.n) for o, w in zip(outs, ws)]
+
+
+def rmsnorm_gguf_matmul_swiglu(x, gamma, beta, eps, w_up: QWeight, w_gate: QWeight, m):
+    xd = DeviceBuffer.from_numpy(np.ascontiguousarray(x, dtype=np.float32))
+    g, b = _norm_bufs(gamma, beta)
+    od = DeviceBuffer(m * w_up.n * 4)
+    _lib.check(_lib.lib().rlx_mi355x_rmsnorm_gguf_matmul_swiglu(xd.ptr, g.ptr, b.ptr if b else None, eps, w_up.ptr, w_gate.ptr, od.ptr, m, None))
+    sync()
+    return od.to_numpy(np.float32).reshape(m, w_up.n)
+
+
+def rmsnorm_gguf_tied_lm_argmax(hidden, gamma, beta, eps, embed: QWeight):
+    hd = DeviceBuffer.from_numpy(np.ascontiguousarray(hidden, dtype=np.float32))
+    g, b = _norm_bufs(gamma, beta)
+    res = DeviceBuffer(16)
+    _lib.check(_lib.lib().rlx_mi355x_memset_u32(res.ptr, 0, 4, None))
+    _lib.check(_lib.lib().rlx_mi355x_rmsnorm_gguf_tied_lm_argmax(hd.ptr, g.ptr, b.ptr if b else None, eps, embed.ptr, res.ptr, res.ptr + 4,
+                                                                res.ptr + 8, None))
+    sync()
+    raw = res.to_numpy(np.uint32, 2)
+    return int(raw[0]), float(raw[1:2].view(np.float32)[0])
+
+
 def gguf_tied_lm_argmax(hidden, embed: QWeight, x_dtype=DType.F32):
     """Host convenience for the tied LM head (rlx-cpu/src/lm_head.rs:223-248): (row, value) of the largest logit of
     hidden . embed^T without materialising the logits."""
