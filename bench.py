@@ -337,31 +337,34 @@ def extra_configs(rlx_amd, stream):
                                   "frac_hbm": round(b / ms / 1e6 / HBM_PEAK_GBS, 4)}
     for q in qws:
         q.free()
-    # a wide scheme: Q6_K gate/up projection [14336, 4096], resident as binary16 (117 MB per copy, four copies rotated)
+    # the other K-quants on a gate/up projection [14336, 4096]: Q6_K has packed kernels (48 MB per copy); Q5_K stands for the
+    # schemes decoded at upload and resident as binary16 (117 MB per copy). Copies rotated so that nothing is cache-resident.
     n, k = 14336, 4096
     rng = np.random.default_rng(5)
-    blocks = rng.integers(0, 256, (n * k // 256, 210), dtype=np.uint8)
-    blocks[:, 208:210] = np.full(n * k // 256, 5e-6, np.float16).view(np.uint8).reshape(-1, 2)  # weights of a few hundredths
-    copies = 4
-    qws = [ops.QWeight(QuantScheme.GgufQ6K, blocks.reshape(-1), n, k) for _ in range(copies)]
-    del blocks
-    x = ops.DeviceBuffer.from_numpy(ops.philox_normal(8, k))
-    y = ops.DeviceBuffer(n * 4)
-    state = {"i": 0}
+    for tag, scheme, bb, d_off, copies in (("q6_k_gemv_gate/up", QuantScheme.GgufQ6K, 210, 208, 13),
+                                            ("q5_k_gemv_gate/up_resident_f16", QuantScheme.GgufQ5K, 176, 0, 5)):
+        blocks = rng.integers(0, 256, (n * k // 256, bb), dtype=np.uint8)
+        blocks[:, d_off:d_off + 2] = np.full(n * k // 256, 5e-6, np.float16).view(np.uint8).reshape(-1, 2)  # weights of a few hundredths
+        if scheme == QuantScheme.GgufQ5K:
+            blocks[:, 2:4] = np.full(n * k // 256, 2e-5, np.float16).view(np.uint8).reshape(-1, 2)
+        qws = [ops.QWeight(scheme, blocks.reshape(-1), n, k) for _ in range(copies)]
+        del blocks
+        x = ops.DeviceBuffer.from_numpy(ops.philox_normal(8, k))
+        y = ops.DeviceBuffer(n * 4)
+        state = {"i": 0}
 
-    def fn6():
-        q = qws[state["i"] % copies]
-        state["i"] += 1
-        rlx_amd._lib.check(L.rlx_mi355x_gguf_matmul_bt(x.ptr, int(DType.F32), q.ptr, y.ptr, 1, None, 0, stream))
+        def fn6():
+            q = qws[state["i"] % copies]
+            state["i"] += 1
+            rlx_amd._lib.check(L.rlx_mi355x_gguf_matmul_bt(x.ptr, int(DType.F32), q.ptr, y.ptr, 1, None, 0, stream))
 
-    ms = time_launches(ops, stream, fn6, 200, 20)
-    resident = qws[0].device_bytes() + 4 * k + 4 * n
-    out["q6_k_gemv_gate/up_resident_f16"] = {"us": round(ms * 1e3, 3), "GB/s_resident": round(resident / ms / 1e6, 1),
-                                             "frac_hbm_resident": round(resident / ms / 1e6 / HBM_PEAK_GBS, 4),
-                                             "GB/s_packed_equivalent": round((n * k // 256 * 210 + 4 * k + 4 * n) / ms / 1e6, 1),
-                                             "note": "wide schemes are decoded at upload and stream 2 bytes per weight with no decode arithmetic"}
-    for q in qws:
-        q.free()
+        ms = time_launches(ops, stream, fn6, 200, 20)
+        resident = qws[0].device_bytes() + 4 * k + 4 * n
+        out[tag] = {"us": round(ms * 1e3, 3), "resident_MB": round(qws[0].device_bytes() / 1e6, 1),
+                    "GB/s_resident": round(resident / ms / 1e6, 1), "frac_hbm_resident": round(resident / ms / 1e6 / HBM_PEAK_GBS, 4),
+                    "GB/s_packed_equivalent": round((n * k // 256 * bb + 4 * k + 4 * n) / ms / 1e6, 1)}
+        for q in qws:
+            q.free()
     # tied LM head: argmax over a Llama-3 vocabulary [128256, 4096] in Q4_K (295 MB, two copies rotated), logits never written
     n, k = 128256, 4096
     w = (ops.philox_normal(21, 4096 * k) * np.float32(0.02)).astype(np.float32)
@@ -512,6 +515,19 @@ def gemm_configs(rlx_amd, stream):
                                         "frac_mfma_f16": round(tf / MFMA_F16_PEAK_TFLOPS, 4)}
         for q in qw:
             q.free()
+
+    # Q6_K, M = 512, gate/up shape, bf16 activations (random code bytes, super-block scales of model-like magnitude)
+    n, k = 14336, 4096
+    blocks = np.random.default_rng(7).integers(0, 256, (n * k // 256, 210), dtype=np.uint8)
+    blocks[:, 208:210] = np.full(n * k // 256, 5e-6, np.float16).view(np.uint8).reshape(-1, 2)
+    qw = [ops.QWeight(QuantScheme.GgufQ6K, blocks.reshape(-1), n, k) for _ in range(2)]
+    del blocks
+    ms = run_matmul(qw, 512, k, DType.BF16, 100, 10)
+    tf = 2.0 * 512 * n * k / ms / 1e9
+    out["q6_k_gemm_m512_gate_up_4096x14336"] = {"us": round(ms * 1e3, 2), "TFLOP/s": round(tf, 1),
+                                                "frac_mfma_f16": round(tf / MFMA_F16_PEAK_TFLOPS, 4)}
+    for q in qw:
+        q.free()
 
     # config 4 (second half): the fake-quantized [8192, 4096] f32 tensor against a Q8_0 4096x4096 weight
     qw = [tiled_weight(ops, QuantScheme.GgufQ8_0, 4096, 4096, 45, 0.02)]

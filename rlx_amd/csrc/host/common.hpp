@@ -35,7 +35,7 @@ void clear_error();
     } while (0)
 
 enum KernelId : int {
-    K_DEQUANT_Q4_0, K_DEQUANT_Q8_0, K_DEQUANT_Q4_K,
+    K_DEQUANT_Q4_0, K_DEQUANT_Q8_0, K_DEQUANT_Q4_K, K_DEQUANT_Q6_K,
     K_FQ_COL_ABSMAX, K_FQ_SEG_ABSMAX, K_FQ_FLAT_ABSMAX, K_FQ_SCALE, K_FQ_SCALE_PARTS, K_FQ_COL_APPLY, K_FQ_FLAT_APPLY, K_FQ_FLAT4_APPLY,
     K_FILL_U32, K_COPY_U128,
     // decode GEMV: per scheme {r2, r4, r2_argmax, r2_paired, r4_paired, r2_norm, r4_norm, r2_norm_paired, r4_norm_paired,
@@ -48,10 +48,18 @@ enum KernelId : int {
     K_GEMV_Q4_K_R2_NORM, K_GEMV_Q4_K_R4_NORM, K_GEMV_Q4_K_R2_NORM_PAIRED, K_GEMV_Q4_K_R4_NORM_PAIRED, K_GEMV_Q4_K_R2_NORM_ARGMAX,
     K_GEMV_F16W_R2, K_GEMV_F16W_R4, K_GEMV_F16W_R2_ARGMAX, K_GEMV_F16W_R2_PAIRED, K_GEMV_F16W_R4_PAIRED,
     K_GEMV_F16W_R2_NORM, K_GEMV_F16W_R4_NORM, K_GEMV_F16W_R2_NORM_PAIRED, K_GEMV_F16W_R4_NORM_PAIRED, K_GEMV_F16W_R2_NORM_ARGMAX,
+    K_GEMV_Q6_K_R2, K_GEMV_Q6_K_R4, K_GEMV_Q6_K_R2_ARGMAX, K_GEMV_Q6_K_R2_PAIRED, K_GEMV_Q6_K_R4_PAIRED,
+    K_GEMV_Q6_K_R2_NORM, K_GEMV_Q6_K_R4_NORM, K_GEMV_Q6_K_R2_NORM_PAIRED, K_GEMV_Q6_K_R4_NORM_PAIRED, K_GEMV_Q6_K_R2_NORM_ARGMAX,
     K_GEMV_Q4_0_R2_D8,
-    K_GEMM_Q4_K, K_GEMM_Q4_0, K_GEMM_Q8_0, K_GEMM64_Q4_K, K_GEMM64_Q4_0, K_GEMM64_Q8_0, K_GEMM_F16W, K_GEMM64_F16W, K_XPREP, K_ARGMAX_FINISH,
+    K_GEMM_Q4_K, K_GEMM_Q4_0, K_GEMM_Q8_0, K_GEMM64_Q4_K, K_GEMM64_Q4_0, K_GEMM64_Q8_0, K_GEMM_F16W, K_GEMM64_F16W, K_GEMM_Q6_K, K_GEMM64_Q6_K, K_XPREP, K_ARGMAX_FINISH,
     K_COUNT
 };
+
+// Device layout a scheme is kept in: its packed layout (layout_of), or binary16 fragments for the wide schemes — Q5_K,
+// Q8_K, Q2_K, Q3_K always, Q6_K when RLX_Q6K_SIGNED_SCALES asks for ggml's signed reading of its scale bytes (the
+// packed Q6_K kernels read them unsigned, as the reference's matmul does).
+Layout host_layout(int scheme);
+inline bool is_wide(int scheme) { return layout_is_f16w(host_layout(scheme)); }
 
 // Loads the embedded code object on first use (device 0). RLX_OK or an error code with text.
 int runtime_init();

@@ -397,7 +397,7 @@ rlx_exec *rlx_mi355x_compile(const rlx_graph_desc *g, const rlx_compile_opts *op
     };
     for (Node &nd : e->nodes) {
         if (nd.is_packed) {
-            nd.slot = take((size_t)weight_dims(nd.scheme, nd.w_n, nd.w_k).bytes * (size_t)nd.w_experts);  // device layout, resident
+            nd.slot = take((size_t)weight_dims(host_layout(nd.scheme), nd.w_n, nd.w_k).bytes * (size_t)nd.w_experts);  // device layout, resident
         } else if (nd.d.op_kind == RLX_OP_INPUT) {
             nd.slot = take((size_t)nd.numel * 4);  // room for an f32 upload even when declared 16-bit
             nd.cur_dtype = nd.d.dtype;

@@ -137,6 +137,11 @@ static void decode_q3_k(const uint8_t *b, float *out) {
     }
 }
 
+Layout host_layout(int scheme) {
+    if (scheme == SCHEME_Q6K && getenv("RLX_Q6K_SIGNED_SCALES") != nullptr) return wide_layout_of(scheme);
+    return layout_of(scheme);
+}
+
 static bool q6k_signed_scales() {
     static const bool v = getenv("RLX_Q6K_SIGNED_SCALES") != nullptr;
     return v;
@@ -154,8 +159,8 @@ static void decode_wide_block(int scheme, const uint8_t *b, float *out) {
 
 // Wide schemes: decode every super-block and store the weights as binary16 operand fragments.
 static int repack_wide(int scheme, const uint8_t *src, int64_t n, int64_t k, uint8_t *out) {
-    const Layout L = layout_of(scheme);
-    const WeightDims D = weight_dims(scheme, n, k);
+    const Layout L = host_layout(scheme);
+    const WeightDims D = weight_dims(L, n, k);
     const int64_t bpr = k / 256;
     memset(out, 0, (size_t)D.bytes);
     float vals[256];
@@ -189,7 +194,7 @@ static int repack_wide(int scheme, const uint8_t *src, int64_t n, int64_t k, uin
 // ---- repack ---------------------------------------------------------------------------------------------
 
 int repack_host(int scheme, const uint8_t *src, size_t nbytes, int64_t n, int64_t k, uint8_t *out) {
-    Layout L = layout_of(scheme);
+    Layout L = host_layout(scheme);
     if (L.unit_k == 0 || L.block_elems == 0) {
         set_error("repack: scheme %d is not a claimed GGUF scheme (Q4_K=5, Q5_K=6, Q6_K=7, Q8_K=8, Q2_K=9, Q3_K=10, Q4_0=11, Q8_0=12)", scheme);
         return RLX_ERR_UNSUPPORTED;
@@ -205,8 +210,8 @@ int repack_host(int scheme, const uint8_t *src, size_t nbytes, int64_t n, int64_
                   (long long)(n * bpr * L.block_bytes));
         return RLX_ERR_INVALID;
     }
-    if (scheme_is_wide(scheme)) return repack_wide(scheme, src, n, k, out);
-    WeightDims D = weight_dims(scheme, n, k);
+    if (is_wide(scheme)) return repack_wide(scheme, src, n, k, out);
+    WeightDims D = weight_dims(L, n, k);
     for (int64_t tile = 0; tile < D.row_tiles; tile++) {
         for (int64_t u = 0; u < D.units; u++) {
             uint8_t *unit = out + (tile * D.units + u) * L.unit_bytes;
@@ -235,6 +240,37 @@ int repack_host(int scheme, const uint8_t *src, size_t nbytes, int64_t n, int64_
                             for (int e = 0; e < 8; e++) dst[e] = live ? (uint8_t)(b[2 + 8 * g + e] ^ 0x80u) : 0x80u;
                         }
                     }
+                } else if (scheme == SCHEME_Q6K) {  // one super-block per unit: low nibbles, high-bit words, scales, d
+                    const bool live = r < n && u < bpr;
+                    const uint8_t *b = live ? src + (r * bpr + u) * L.block_bytes : nullptr;
+                    if (g == 0) {
+                        if (live) {
+                            memcpy(unit + 3072 + nrow * 16, b + 192, 16);
+                            memcpy(unit + 3328 + nrow * 2, b + 208, 2);
+                        } else {
+                            memset(unit + 3072 + nrow * 16, 0, 16);
+                            memset(unit + 3328 + nrow * 2, 0, 2);
+                        }
+                    }
+                    uint32_t hw[4] = {0, 0, 0, 0};
+                    for (int j = 0; j < 8; j++) {
+                        uint32_t word = 0;
+                        for (int e = 0; e < 8; e++) {
+                            const int i = 32 * j + 8 * g + e;  // element of the super-block
+                            uint32_t code = 32;               // decodes to zero
+                            if (live) {
+                                const int h = i >> 7, quarter = (i >> 5) & 3, l5 = i & 31;
+                                const uint8_t lowbyte = b[64 * h + 32 * (quarter & 1) + l5];
+                                const uint32_t low = (quarter >> 1) ? (uint32_t)(lowbyte >> 4) : (uint32_t)(lowbyte & 0x0F);
+                                const uint32_t high = (uint32_t)(b[128 + 32 * h + l5] >> (2 * quarter)) & 3u;
+                                code = low | (high << 4);
+                            }
+                            word |= (code & 0xFu) << (4 * nib_pos(e));
+                            hw[(j >> 2) * 2 + ((j & 3) >> 1)] |= (code >> 4) << ((q6k_hi_pos(e) + ((j & 1) ? 8 : 0)) & 31);
+                        }
+                        memcpy(unit + (j >> 2) * 1024 + l * 16 + (j & 3) * 4, &word, 4);
+                    }
+                    memcpy(unit + 2048 + l * 16, hw, 16);
                 } else {  // Q4_K: one super-block per unit
                     const bool live = r < n && u < bpr;
                     const uint8_t *b = live ? src + (r * bpr + u) * L.block_bytes : nullptr;
@@ -390,7 +426,7 @@ int64_t rlx_mi355x_bytes_for(int scheme, int64_t n) {
 }
 
 size_t rlx_mi355x_qweight_device_bytes_for(int scheme, int64_t n, int64_t k) {
-    return (size_t)rlx::weight_dims(scheme, n, k).bytes;
+    return (size_t)rlx::weight_dims(rlx::host_layout(scheme), n, k).bytes;
 }
 
 int rlx_mi355x_repack_host(int scheme, const void *gguf_bytes, size_t nbytes, int64_t n, int64_t k, void *out) {
@@ -399,7 +435,7 @@ int rlx_mi355x_repack_host(int scheme, const void *gguf_bytes, size_t nbytes, in
 
 int rlx_mi355x_quantize(int scheme, const float *src, int64_t n_elems, void *out) {
     rlx::Layout L = rlx::layout_of(scheme);
-    if (L.block_elems == 0 || rlx::scheme_is_wide(scheme)) {
+    if (L.block_elems == 0 || (scheme != rlx::SCHEME_Q4K && scheme != rlx::SCHEME_Q4_0 && scheme != rlx::SCHEME_Q8_0)) {
         rlx::set_error("quantize: scheme %d unsupported", scheme);
         return RLX_ERR_UNSUPPORTED;
     }

@@ -12,6 +12,7 @@ int repack_host(int scheme, const uint8_t *src, size_t nbytes, int64_t n, int64_
 
 struct rlx_qweight {
     int scheme;
+    rlx::Layout layout;    // device layout it was repacked into (packed, or binary16 for the wide schemes)
     rlx::WeightDims dims;  // of one [n, k] matrix
     uint8_t *dev;
     bool owns;
@@ -93,7 +94,8 @@ static int launch_gemv(const void *const *xs, int xk, const rlx_qweight *const *
                        hipStream_t stream, const float *expert_idx = nullptr, unsigned long long *argmax_key = nullptr,
                        const rlx_qweight *const *pairs = nullptr, const RmsNorm *norm = nullptr) {
     const int scheme = ws[0]->scheme;
-    const Layout L = layout_of(scheme);
+    const Layout L = ws[0]->layout;
+    const bool wide = layout_is_f16w(L);
     for (int i = 0; i < count; i++)
         if ((uintptr_t)xs[i] % 16 != 0) {
             set_error("gguf_matmul_bt: activations must be 16-byte aligned");
@@ -103,8 +105,8 @@ static int launch_gemv(const void *const *xs, int xk, const rlx_qweight *const *
     const int ng = (rv + 3) / 4;
     const bool r2 = rv <= 2;
     // kernel = scheme family x {r2, r4, r2_argmax, r2_paired, r4_paired}
-    const int family = scheme == SCHEME_Q4_0 ? K_GEMV_Q4_0_R2 : scheme == SCHEME_Q8_0 ? K_GEMV_Q8_0_R2
-                       : scheme_is_wide(scheme) ? K_GEMV_F16W_R2 : K_GEMV_Q4_K_R2;
+    const int family = wide ? K_GEMV_F16W_R2 : scheme == SCHEME_Q4_0 ? K_GEMV_Q4_0_R2 : scheme == SCHEME_Q8_0 ? K_GEMV_Q8_0_R2
+                       : scheme == SCHEME_Q6K ? K_GEMV_Q6_K_R2 : K_GEMV_Q4_K_R2;
     if (argmax_key && !r2) {
         set_error("gemv: the argmax epilogue takes one activation row");
         return RLX_ERR_INVALID;
@@ -216,7 +218,7 @@ static GemmPlan gemm_plan(int scheme, int xk, int64_t m, int64_t k) {
 // accumulation into a zeroed output) only when the tile grid alone would leave most CUs idle.
 static int launch_gemm(const void *x, int xk, const rlx_qweight *w, float *out, int64_t m, void *workspace,
                        size_t workspace_bytes, hipStream_t stream) {
-    const Layout L = layout_of(w->scheme);
+    const Layout L = w->layout;
     const GemmPlan p = gemm_plan(w->scheme, xk, m, w->dims.k);
     if (!workspace || workspace_bytes < p.xh_bytes + p.sxh_bytes) {
         set_error("gguf_matmul_bt: m=%lld needs a %zu-byte workspace, got %zu", (long long)m, p.xh_bytes + p.sxh_bytes,
@@ -255,7 +257,8 @@ static int launch_gemm(const void *x, int xk, const rlx_qweight *w, float *out, 
     void *params[] = {&a};
     KernelId id = w->scheme == SCHEME_Q4K       ? (skinny ? K_GEMM64_Q4_K : K_GEMM_Q4_K)
                   : w->scheme == SCHEME_Q4_0    ? (skinny ? K_GEMM64_Q4_0 : K_GEMM_Q4_0)
-                  : scheme_is_wide(w->scheme) ? (skinny ? K_GEMM64_F16W : K_GEMM_F16W)
+                  : layout_is_f16w(L)           ? (skinny ? K_GEMM64_F16W : K_GEMM_F16W)
+                  : w->scheme == SCHEME_Q6K     ? (skinny ? K_GEMM64_Q6_K : K_GEMM_Q6_K)
                                                 : (skinny ? K_GEMM64_Q8_0 : K_GEMM_Q8_0);
     RLX_TRY(runtime_init());
     RLX_TRY(launch3(id, (unsigned)gx, (unsigned)gy, (unsigned)split, 512, skinny ? 3 * 24 * 1024 : 3 * 48 * 1024, stream, params));
@@ -270,9 +273,10 @@ int rlx_mi355x_qweight_create_at(int scheme, const void *gguf_bytes, size_t nbyt
                                  void *device_mem, rlx_qweight **out) {
     using namespace rlx;
     RLX_TRY(runtime_init());
-    WeightDims D = weight_dims(scheme, n, k);
+    const Layout HL = host_layout(scheme);
+    WeightDims D = weight_dims(HL, n, k);
     std::vector<uint8_t> staging;
-    if (D.bytes == 0 || layout_of(scheme).block_elems == 0) {
+    if (D.bytes == 0 || HL.block_elems == 0) {
         set_error("qweight: scheme %d is not a claimed GGUF scheme", scheme);
         return RLX_ERR_UNSUPPORTED;
     }
@@ -286,7 +290,7 @@ int rlx_mi355x_qweight_create_at(int scheme, const void *gguf_bytes, size_t nbyt
         set_error("qweight upload: %s", hipGetErrorString(e));
         return RLX_ERR_HIP;
     }
-    *out = new rlx_qweight{scheme, D, (uint8_t *)device_mem, owns, 1};
+    *out = new rlx_qweight{scheme, HL, D, (uint8_t *)device_mem, owns, 1};
     return RLX_OK;
 }
 
@@ -299,8 +303,9 @@ int rlx_mi355x_qweight_create_experts_at(int scheme, const void *gguf_bytes, siz
                                          int64_t num_experts, void *device_mem, rlx_qweight **out) {
     using namespace rlx;
     RLX_TRY(runtime_init());
-    WeightDims D = weight_dims(scheme, n, k);
-    if (D.bytes == 0 || layout_of(scheme).block_elems == 0) {
+    const Layout HL = host_layout(scheme);
+    WeightDims D = weight_dims(HL, n, k);
+    if (D.bytes == 0 || HL.block_elems == 0) {
         set_error("qweight: scheme %d is not a claimed GGUF scheme", scheme);
         return RLX_ERR_UNSUPPORTED;
     }
@@ -321,7 +326,7 @@ int rlx_mi355x_qweight_create_experts_at(int scheme, const void *gguf_bytes, siz
         set_error("qweight upload: %s", hipGetErrorString(err));
         return RLX_ERR_HIP;
     }
-    *out = new rlx_qweight{scheme, D, (uint8_t *)device_mem, owns, (int)num_experts};
+    *out = new rlx_qweight{scheme, HL, D, (uint8_t *)device_mem, owns, (int)num_experts};
     return RLX_OK;
 }
 
@@ -344,14 +349,15 @@ int rlx_mi355x_dequant(const rlx_qweight *w, float *out_dev, void *stream) {
         set_error("dequant: null argument");
         return RLX_ERR_INVALID;
     }
-    if (scheme_is_wide(w->scheme)) {
+    if (layout_is_f16w(w->layout)) {
         set_error("dequant: scheme %d is resident as binary16 (decoded at upload); the exact f32 decode is not kept on the device",
                   w->scheme);
         return RLX_ERR_UNSUPPORTED;
     }
     DequantArgs a{w->dev, out_dev, w->dims.n, w->dims.k, w->dims.units};
     void *params[] = {&a};
-    KernelId id = w->scheme == SCHEME_Q4_0 ? K_DEQUANT_Q4_0 : w->scheme == SCHEME_Q8_0 ? K_DEQUANT_Q8_0 : K_DEQUANT_Q4_K;
+    KernelId id = w->scheme == SCHEME_Q4_0 ? K_DEQUANT_Q4_0 : w->scheme == SCHEME_Q8_0 ? K_DEQUANT_Q8_0
+                  : w->scheme == SCHEME_Q6K ? K_DEQUANT_Q6_K : K_DEQUANT_Q4_K;
     return launch(id, (unsigned)w->dims.units, (unsigned)w->dims.row_tiles, 64, 0, (hipStream_t)stream, params);
 }
 
@@ -450,7 +456,7 @@ int rlx_mi355x_rmsnorm_gguf_matmul_bt_batch(const float *x_dev, const float *gam
                 set_error("rmsnorm_gguf_matmul_bt_batch: null weight / output or an expert stack at %d", i0 + i);
                 return RLX_ERR_INVALID;
             }
-            const bool same = ws[i0 + i]->scheme == ws[i0]->scheme || (scheme_is_wide(ws[i0 + i]->scheme) && scheme_is_wide(ws[i0]->scheme));
+            const bool same = ws[i0 + i]->scheme == ws[i0]->scheme || (layout_is_f16w(ws[i0 + i]->layout) && layout_is_f16w(ws[i0]->layout));
             if (!same || ws[i0 + i]->dims.k != ws[0]->dims.k) {
                 set_error("rmsnorm_gguf_matmul_bt_batch: the matrices share one normalized input, so one scheme and one k");
                 return RLX_ERR_INVALID;
@@ -471,7 +477,7 @@ int rlx_mi355x_rmsnorm_gguf_matmul_swiglu(const float *x_dev, const float *gamma
         set_error("rmsnorm_gguf_matmul_swiglu: null argument");
         return RLX_ERR_INVALID;
     }
-    const bool same_layout = w_up->scheme == w_gate->scheme || (scheme_is_wide(w_up->scheme) && scheme_is_wide(w_gate->scheme));
+    const bool same_layout = w_up->scheme == w_gate->scheme || (layout_is_f16w(w_up->layout) && layout_is_f16w(w_gate->layout));
     if (!same_layout || w_up->dims.n != w_gate->dims.n || w_up->dims.k != w_gate->dims.k || w_up->experts != 1 ||
         w_gate->experts != 1) {
         set_error("rmsnorm_gguf_matmul_swiglu: the up and gate projections must share scheme, n and k");
@@ -515,8 +521,7 @@ int rlx_mi355x_gguf_matmul_swiglu(const void *x_dev, int x_dtype, const rlx_qwei
         set_error("gguf_matmul_swiglu: activation dtype %d is not F32 / BF16 / F16", x_dtype);
         return RLX_ERR_UNSUPPORTED;
     }
-    const bool same_layout = w_up->scheme == w_gate->scheme ||
-                             (scheme_is_wide(w_up->scheme) && scheme_is_wide(w_gate->scheme));
+    const bool same_layout = w_up->scheme == w_gate->scheme || (layout_is_f16w(w_up->layout) && layout_is_f16w(w_gate->layout));
     if (!same_layout || w_up->dims.n != w_gate->dims.n || w_up->dims.k != w_gate->dims.k || w_up->experts != 1 ||
         w_gate->experts != 1) {
         set_error("gguf_matmul_swiglu: the up and gate projections must share scheme, n and k");

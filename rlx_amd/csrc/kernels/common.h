@@ -103,6 +103,31 @@ __device__ __forceinline__ void q4k_scales(uint32_t s0, uint32_t s1, uint32_t s2
     mn[1] = ((s2 >> 4) & 0x0F0F0F0Fu) | ((s1 >> 2) & 0x30303030u);
 }
 
+// Q6_K granule: code word w (eight low nibbles) and its high-bit word hx (the pair's word as stored for the even code
+// word, rotated right by 8 for the odd one) -> sc * (q - 32) as halfs in fragment order, sc given as a half2 splat of an
+// integer in [0, 255]. (q - 32) is exact; the product is exact up to 2048 and rounded to binary16 above (|.| <= 8160).
+__device__ __forceinline__ void unpack_q6_scaled(uint32_t w, uint32_t hx, half2_t sc, Frag &f) {
+    const half2_t off = {(half_t)(-1056.0f), (half_t)(-1056.0f)};   // 1024 + 32
+    const half2_t r16 = {(half_t)0.0625f, (half_t)0.0625f};
+    const half2_t m96 = {(half_t)(-96.0f), (half_t)(-96.0f)};        // (1024 + 16 q) / 16 - 96 = q - 32
+    const half2_t sc16 = sc * r16, neg96 = sc * m96;                 // both exact: sc has 8 bits
+    const uint32_t w2 = w >> 8, h2 = hx >> 2;
+    const uint32_t a0 = (hx & 0x00300030u) | and_or(w, 0x000F000Fu, MAGIC);   // 1024 + q
+    const uint32_t a1 = (hx & 0x03000300u) | and_or(w, 0x00F000F0u, MAGIC);   // 1024 + 16 q
+    const uint32_t a2 = (h2 & 0x00300030u) | and_or(w2, 0x000F000Fu, MAGIC);
+    const uint32_t a3 = (h2 & 0x03000300u) | and_or(w2, 0x00F000F0u, MAGIC);
+    f.h2[0] = (as_half2(a0) + off) * sc;
+    f.h2[1] = __builtin_elementwise_fma(as_half2(a1), sc16, neg96);
+    f.h2[2] = (as_half2(a2) + off) * sc;
+    f.h2[3] = __builtin_elementwise_fma(as_half2(a3), sc16, neg96);
+}
+
+// half2 splat of the integer byte b (0..255), exact: bytes [b, 0x64, b, 0x64] = 1024 + b, minus 1024
+__device__ __forceinline__ half2_t splat_ubyte_half(uint32_t b) {
+    const half2_t k1024 = {(half_t)1024.0f, (half_t)1024.0f};
+    return as_half2(MAGIC | b | (b << 16)) - k1024;
+}
+
 __device__ __forceinline__ float ubyte_to_float(uint32_t w, int byte) { return (float)((w >> (8 * byte)) & 0xFFu); }
 
 // D(16x16) += A(16x32) * B(32x16), halfs in, f32 accumulate. Lane l: A row / B column l & 15, k-slice 8*(l>>4)..+7;

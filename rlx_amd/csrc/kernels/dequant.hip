@@ -61,6 +61,30 @@ __device__ __forceinline__ void dequant_tile(const DequantArgs &a) {
                 store8(a.out, a.n, a.k, r, u * 128 + t * 32 + g * 8, v);
             }
         }
+    } else if constexpr (SCHEME == SCHEME_Q6K) {
+        // the block decoder the reference's matmul calls (rlx-gguf/src/lib.rs:819-845): (d * sc) * (q - 32), scale bytes unsigned
+        const uint4_t hw = *(const uint4_t *)(unit + 2048 + l * 16);
+        const uint4_t scales = *(const uint4_t *)(unit + 3072 + nrow * 16);
+        const float d = half_bits_to_float(*(const uint16_t *)(unit + 3328 + nrow * 2));
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const uint4_t q = *(const uint4_t *)(unit + h * 1024 + l * 16);
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                const int j = 4 * h + t;
+                uint32_t hx = hw[2 * h + (t >> 1)];
+                if (t & 1) hx = __builtin_amdgcn_alignbit(hx, hx, 8);
+                const int si = 2 * j + (g >> 1);
+                const float ds = d * ubyte_to_float(scales[si >> 2], si & 3);
+                float v[8];
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    const int code = (int)(((q[t] >> (4 * nib_pos(e))) & 0xFu) | (((hx >> q6k_hi_pos(e)) & 3u) << 4)) - 32;
+                    v[e] = ds * (float)code;
+                }
+                store8(a.out, a.n, a.k, r, u * 256 + j * 32 + g * 8, v);
+            }
+        }
     } else {
         uint4_t meta = *(const uint4_t *)(unit + 2048 + nrow * 16);
         float d = half_bits_to_float(meta[0] & 0xFFFFu);
@@ -92,3 +116,4 @@ __device__ __forceinline__ void dequant_tile(const DequantArgs &a) {
 extern "C" __global__ __launch_bounds__(64) void rlx_dequant_q4_0(rlx::DequantArgs a) { rlx::dequant_tile<rlx::SCHEME_Q4_0>(a); }
 extern "C" __global__ __launch_bounds__(64) void rlx_dequant_q8_0(rlx::DequantArgs a) { rlx::dequant_tile<rlx::SCHEME_Q8_0>(a); }
 extern "C" __global__ __launch_bounds__(64) void rlx_dequant_q4_k(rlx::DequantArgs a) { rlx::dequant_tile<rlx::SCHEME_Q4K>(a); }
+extern "C" __global__ __launch_bounds__(64) void rlx_dequant_q6_k(rlx::DequantArgs a) { rlx::dequant_tile<rlx::SCHEME_Q6K>(a); }

@@ -66,6 +66,10 @@ template <int SCHEME, int TI, int TJ>
 __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
     constexpr Layout L = layout_of(SCHEME);
     constexpr bool K4 = SCHEME == SCHEME_Q4K;
+    constexpr bool K6 = SCHEME == SCHEME_Q6K;
+    // Super-block schemes: B holds integers (Q4_K: sc * q, exact; Q6_K: sc * (q - 32), exact up to 2048), a second
+    // accumulator set collects one 256-column super-block and d (Q4_K: and dmin) is applied in f32 per super-block.
+    constexpr bool SB = K4 || K6;
     constexpr int WN = GEMM_NT / (32 * TJ), WM = 8 / WN, MT = WM * TI * 32;  // wave grid and rows per workgroup
     constexpr int NSA = MT / 32, SA = 4 * NSA * 1024, ST = SA + GEMM_STAGE_B;  // LDS stage: activations [4][NSA][1 KB], then weights
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -104,11 +108,12 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
     uint4_t a_reg[2][4];                                // activations of the next steps, [step parity] (Q4_K: one set)
     uint4_t b_q[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};      // [chunk parity] packed codes of a two-step chunk (Q8_0: [step parity])
     uint4_t b_meta[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};   // Q4_K: [0] = meta of the super-block decoded next; else [chunk parity] .x/.y = four f16 scales
+    uint2_t b_hw[2] = {{0, 0}, {0, 0}};                 // Q6_K: [chunk parity] high-bit words of the two code-word pairs of a half
     uint32_t b_sc[2] = {0, 0};                          // Q4_K: 6-bit scales of sub-blocks 0-3 / 4-7 being decoded
 
     // Activations run AD steps ahead of their LDS store: two where registers allow (their loads come through L2 with
     // the whole workgroup's 32 KB per step behind them), one for Q4_K whose second accumulator set takes the room.
-    constexpr int AD = K4 ? 1 : 2;
+    constexpr int AD = SB ? 1 : 2;
     // Buffer loads: wave-uniform descriptor and scalar offset, constant per-lane offset, so a fetch costs no VALU.
     // A wave that moves no activation chunk (64-row tile) gets an empty range: its loads return zeros without traffic.
     const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)a_base, 0, a_mine ? 0x7FFFFFFF : 0, 0x00020000);
@@ -123,6 +128,13 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
             const int unit = (step >> 2) * L.unit_bytes;
             if ((q & 1) == 0) b_q[(q >> 1) & 1] = ld128(b_rsrc, lane * 16, unit + (q >> 1) * 1024);
             if (q == 0) b_meta[0] = ld128(b_rsrc, b_n16 * 16, unit + 2048);  // consumed one step later, before the next fetch
+        } else if constexpr (K6) {  // codes and high-bit words of a half every second step, the row's 16 scale bytes per super-block
+            const int unit = (step >> 2) * L.unit_bytes;
+            if ((q & 1) == 0) {
+                b_q[(q >> 1) & 1] = ld128(b_rsrc, lane * 16, unit + (q >> 1) * 1024);
+                b_hw[(q >> 1) & 1] = __builtin_amdgcn_raw_buffer_load_b64(b_rsrc, lane * 16 + (q >> 1) * 8, unit + 2048, 0);
+            }
+            if (q == 0) b_meta[0] = ld128(b_rsrc, b_n16 * 16, unit + 3072);  // copied aside when the super-block's decode starts
         } else if constexpr (SCHEME == SCHEME_F16W) {  // two ready-made fragments per lane and step: b_q and b_meta hold them
             const int unit = (step >> 1) * L.unit_bytes + (q & 1) * 2048;
             b_q[q & 1] = ld128(b_rsrc, lane * 16, unit);
@@ -164,6 +176,16 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
                 b_sc[1] &= b_keep;
             }
             unpack_q4_scaled(b_q[cp][t], splat_code_half(b_sc[q >> 1], t), f);
+        } else if constexpr (K6) {
+            if (q == 0 && jl == 0) {  // this super-block's scales, out of the way of the next super-block's fetch
+#pragma unroll
+                for (int e = 0; e < 4; e++) b_meta[1][e] = b_meta[0][e] & b_keep;  // a dead tile decodes to zeros
+            }
+            uint32_t hx = b_hw[cp][t >> 1];
+            if (t & 1) hx = __builtin_amdgcn_alignbit(hx, hx, 8);
+            // block 2 q + jl of the super-block, this lane's 16-column half of it: scale byte 4 q + 2 jl + g / 2
+            const uint32_t scb = (b_meta[1][q] >> (16 * jl + 8 * (b_g >> 1))) & 0xFFu;
+            unpack_q6_scaled(b_q[cp][t], hx, splat_ubyte_half(scb), f);
         } else if constexpr (SCHEME == SCHEME_F16W) {
             f.u4 = jl ? b_meta[q & 1] : b_q[q & 1];
 #pragma unroll
@@ -198,7 +220,8 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
     for (int j = 0; j < TJ; j++) {
         my_row[j] = n_tile0 + (wn * TJ + j) * 32 + lr;
         my_ok[j] = (my_row[j] >> 4) < a.row_tiles;
-        my_meta[j] = a.w + (long long)(my_ok[j] ? (my_row[j] >> 4) : 0) * a.units * L.unit_bytes + 2048 + (my_row[j] & 15) * 16;
+        my_meta[j] = a.w + (long long)(my_ok[j] ? (my_row[j] >> 4) : 0) * a.units * L.unit_bytes +
+                     (K6 ? 3328 + (my_row[j] & 15) * 2 : 2048 + (my_row[j] & 15) * 16);  // Q6_K: the row's d; Q4_K: its 16 meta bytes
     }
     uint4_t w_meta[TJ];
     Frag fs[TI];
@@ -212,7 +235,7 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
     }
     // Fragment buffers: a compute half starts with slices 0 .. PD-1 already in registers (read during the data half
     // before it) and reads slice ks + PD under the MFMAs of slice ks.
-    constexpr int NB = K4 ? 2 : 4, PD = NB / 2;
+    constexpr int NB = SB ? 2 : 4, PD = NB / 2;
     Frag fa[NB][TI], fb[NB][TJ];  // [buffer][tile]
     auto load_frags = [&](const uint8_t *stage, int ks, int buf) {
 #pragma unroll
@@ -227,6 +250,11 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
 
     // ---- Q4_K: a 256-column super-block is complete: total += d * P - dmin * (mn . sx) ----------------------
     auto load_sb_meta = [&](int sb) {  // this wave's rows: meta and activation block sums of the super-block
+        if constexpr (K6) {
+#pragma unroll
+            for (int j = 0; j < TJ; j++) w_meta[j][0] = *(const uint16_t *)(my_meta[j] + (long long)sb * L.unit_bytes);
+            return;
+        }
 #pragma unroll
         for (int j = 0; j < TJ; j++) w_meta[j] = *(const uint4_t *)(my_meta[j] + (long long)sb * L.unit_bytes);
 #pragma unroll
@@ -236,6 +264,17 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
         }
     };
     auto scale_sb = [&]() {
+        if constexpr (K6) {  // total += d * P
+#pragma unroll
+            for (int j = 0; j < TJ; j++) {
+                const float d = my_ok[j] ? half_bits_to_float(w_meta[j][0] & 0xFFFFu) : 0.f;
+#pragma unroll
+                for (int i = 0; i < TI; i++)
+#pragma unroll
+                    for (int e = 0; e < 16; e++) total[i][j][e] = __builtin_fmaf(d, part[i][j][e], total[i][j][e]);
+            }
+            return;
+        }
 #pragma unroll
         for (int j = 0; j < TJ; j++) {
             const uint4_t meta = w_meta[j];
@@ -284,7 +323,7 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
             for (int i = 0; i < TI; i++)
 #pragma unroll
                 for (int j = 0; j < TJ; j++) {
-                    if constexpr (K4) {
+                    if constexpr (SB) {
                         // the first slice of a super-block starts the partial product from zero
                         part[i][j] = mfma32(fa[buf][i], fb[buf][j], (q == 0 && ks == 0) ? zero16 : part[i][j]);
                     } else {
@@ -348,7 +387,7 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
                         __syncthreads();
                         preload(smem + s1);
                         data(step + 2, (q + 2) & 3, smem + s2);
-                        if constexpr (K4) {
+                        if constexpr (SB) {
                             if (q == 1) load_sb_meta(step >> 2);
                             if (q == 3) scale_sb();
                         }
@@ -356,7 +395,7 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
                     } else {
                         preload(smem + s0);
                         data(step + 1, (q + 1) & 3, smem + s1);
-                        if constexpr (K4) {
+                        if constexpr (SB) {
                             if (q == 1) load_sb_meta(step >> 2);
                             if (q == 0 && step > step0) scale_sb();  // the super-block finished in the last iteration
                         }
@@ -371,7 +410,7 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
                 }
             }
         }
-        if constexpr (K4 && GRP == 1) {
+        if constexpr (SB && GRP == 1) {
             if (step0 < step1) scale_sb();
         }
     };
@@ -484,6 +523,8 @@ __device__ __forceinline__ void xprep_body(const XPrepArgs &a) {
 extern "C" __global__ __launch_bounds__(512) void rlx_gemm_q4_k(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q4K, 2, 2>(a); }
 extern "C" __global__ __launch_bounds__(512) void rlx_gemm_q4_0(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q4_0, 2, 2>(a); }
 extern "C" __global__ __launch_bounds__(512) void rlx_gemm_q8_0(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q8_0, 2, 2>(a); }
+extern "C" __global__ __launch_bounds__(512) void rlx_gemm_q6_k(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q6K, 2, 2>(a); }
+extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64_q6_k(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q6K, 1, 1>(a); }
 extern "C" __global__ __launch_bounds__(512) void rlx_gemm_f16w(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_F16W, 2, 2>(a); }
 extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64_f16w(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_F16W, 1, 1>(a); }
 extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64_q4_k(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q4K, 1, 1>(a); }

@@ -106,6 +106,23 @@ struct UnitRegs<SCHEME_Q4K> {
 };
 
 template <>
+struct UnitRegs<SCHEME_Q6K> {  // one super-block: low nibbles (two halves), high-bit words, the row's 16 scales, d
+    uint4_t q0, q1, hw, sc;
+    uint32_t d;
+    __device__ __forceinline__ void load(const uint8_t *unit, int l, int nrow, bool) {
+        q0 = __builtin_nontemporal_load((const uint4_t *)(unit + l * 16));
+        q1 = __builtin_nontemporal_load((const uint4_t *)(unit + 1024 + l * 16));
+        hw = __builtin_nontemporal_load((const uint4_t *)(unit + 2048 + l * 16));
+        sc = __builtin_nontemporal_load((const uint4_t *)(unit + 3072 + nrow * 16));
+        d = __builtin_nontemporal_load((const uint16_t *)(unit + 3328 + nrow * 2));
+    }
+    __device__ __forceinline__ void clear() {
+        q0 = q1 = hw = sc = uint4_t{0, 0, 0, 0};
+        d = 0;
+    }
+};
+
+template <>
 struct UnitRegs<SCHEME_F16W> {  // weights already stored as binary16 fragments: four 32-column blocks, no scales
     uint4_t q[4];
     __device__ __forceinline__ void load(const uint8_t *unit, int l, int, bool) {
@@ -151,6 +168,28 @@ __device__ __forceinline__ void compute_unit(const UnitRegs<SCHEME> &w, const ha
 #pragma unroll
             for (int r = 0; r < NREG; r++) acc[r] = __builtin_fmaf(d, blk[t][r], acc[r]);
         }
+    } else if constexpr (SCHEME == SCHEME_Q6K) {
+        // B = sc * (q - 32): the 16-column scale is folded into the fragment (a lane's 8 columns share one scale), the
+        // matrix unit accumulates the eight blocks of the super-block, d is applied once.
+        float4_t sum = zero;
+        const int gshift = 8 * (g >> 1);  // this lane's half of each 32-column block: scale byte 2 j or 2 j + 1
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            load_afrags<4>(xrow, live, ucol + h * 128, a);
+            const uint4_t &q = h ? w.q1 : w.q0;
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                uint32_t hx = w.hw[2 * h + (t >> 1)];
+                if (t & 1) hx = __builtin_amdgcn_alignbit(hx, hx, 8);
+                const uint32_t scb = (w.sc[2 * h + (t >> 1)] >> (16 * (t & 1) + gshift)) & 0xFFu;
+                Frag b;
+                unpack_q6_scaled(q[t], hx, splat_ubyte_half(scb), b);
+                sum = mfma16(a[t], b, sum);
+            }
+        }
+        const float d = half_bits_to_float(w.d);
+#pragma unroll
+        for (int r = 0; r < NREG; r++) acc[r] = __builtin_fmaf(d, sum[r], acc[r]);
     } else if constexpr (SCHEME == SCHEME_F16W) {
         load_afrags<4>(xrow, live, ucol, a);
         float4_t sum = zero;  // the matrix unit accumulates the four blocks; nothing to decode or scale
@@ -535,4 +574,5 @@ RLX_GEMV_SCHEME(q4_0, rlx::SCHEME_Q4_0, 4)
 RLX_GEMV_SCHEME(q8_0, rlx::SCHEME_Q8_0, 3)
 RLX_GEMV_SCHEME(q4_k, rlx::SCHEME_Q4K, 3)
 RLX_GEMV_SCHEME(f16w, rlx::SCHEME_F16W, 2)
+RLX_GEMV_SCHEME(q6_k, rlx::SCHEME_Q6K, 2)
 RLX_GEMV_INST(rlx_gemv_q4_0_r2_d8, rlx::SCHEME_Q4_0, 2, 8, rlx::GEMV_PLAIN)

@@ -20,7 +20,16 @@
 //          [2048,2176) f16 d[n][4]
 //   Q4_K : [0,2048)  two halves h: 16 B at 1024*h + 16*l = granules of sub-blocks 4h+0..3 of super-block u
 //          [2048,2304) per row n: 16 B = f16 d, f16 dmin, 12 scale bytes (verbatim from the GGUF block)
-//   Q5_K, Q6_K, Q8_K, Q2_K, Q3_K ("wide" schemes): the weights are decoded once, at upload, with the reference's block
+//   Q6_K : [0,2048)  low nibbles of the 6-bit codes, two halves h like Q4_K (word t of a slot = 32-column block 4h + t)
+//          [2048,3072) the two high bits of every code: 16 B at 2048 + 16*l = words hw[2h + j], one per pair of code
+//                   words (t = 2j, 2j + 1) of half h. In hw the field of element e of the even word sits at bit
+//                   Q6K_HI_POS[e]; the odd word's fields sit 8 bits further (mod 32), so `hw` serves the even word as
+//                   is and the odd word after a rotate by 8. The positions are those the f16 magic-number decode
+//                   needs: elements 0,1 / 4,5 (value 1024 + q) take their high bits at mantissa bits 4-5 / 20-21,
+//                   elements 2,3 / 6,7 (value 1024 + 16 q) at bits 8-9 / 24-25; elements 4-7 are stored 2 bits higher
+//                   and used after a shift by 2, like their nibbles after a shift by 8.
+//          [3072,3328) per row n: the 16 scale bytes verbatim          [3328,3360) f16 d[n]
+//   Q5_K, Q8_K, Q2_K, Q3_K, and Q6_K when its scales are to be read as signed ("wide" schemes): the weights are decoded once, at upload, with the reference's block
 //          decoder and stored as binary16: [0,4096) four blocks t: 16 B at 1024*t + 16*l = the 8 halfs of granule
 //          (n, 4u+t, g), already an MFMA operand fragment. No scales. 2 bytes per weight resident instead of the
 //          packed 0.33-1.14, in exchange for kernels that do no decode arithmetic at all.
@@ -44,10 +53,8 @@ enum Scheme : int {
     SCHEME_Q4_0 = 11, SCHEME_Q8_0 = 12, SCHEME_F16W = 100
 };
 
-RLX_HD constexpr bool scheme_is_wide(int scheme) {
-    return scheme == SCHEME_Q5K || scheme == SCHEME_Q6K || scheme == SCHEME_Q8K || scheme == SCHEME_Q2K ||
-           scheme == SCHEME_Q3K || scheme == SCHEME_F16W;
-}
+// low bit of the 2-bit high field of element e (even code word of a pair) inside a Q6_K high-bit word
+RLX_HD constexpr int q6k_hi_pos(int e) { return e == 0 ? 4 : e == 1 ? 20 : e == 2 ? 8 : e == 3 ? 24 : e == 4 ? 6 : e == 5 ? 22 : e == 6 ? 10 : 26; }
 
 constexpr int TILE_ROWS = 16;
 
@@ -64,13 +71,19 @@ RLX_HD constexpr Layout layout_of(int scheme) {
            : scheme == SCHEME_Q8_0 ? Layout{128, 2176, 2048, 32, 34}
            : scheme == SCHEME_Q4K  ? Layout{256, 2304, 2048, 256, 144}
            : scheme == SCHEME_Q5K  ? Layout{128, 4096, 4096, 256, 176}
-           : scheme == SCHEME_Q6K  ? Layout{128, 4096, 4096, 256, 210}
+           : scheme == SCHEME_Q6K  ? Layout{256, 3360, 3072, 256, 210}
            : scheme == SCHEME_Q8K  ? Layout{128, 4096, 4096, 256, 292}
            : scheme == SCHEME_Q2K  ? Layout{128, 4096, 4096, 256, 84}
            : scheme == SCHEME_Q3K  ? Layout{128, 4096, 4096, 256, 110}
            : scheme == SCHEME_F16W ? Layout{128, 4096, 4096, 0, 0}
                                    : Layout{0, 0, 0, 0, 0};
 }
+
+// The binary16 layout of a scheme kept wide: F16W geometry with the scheme's own GGUF block size.
+RLX_HD constexpr Layout wide_layout_of(int scheme) {
+    return Layout{128, 4096, 4096, layout_of(scheme).block_elems, layout_of(scheme).block_bytes};
+}
+RLX_HD constexpr bool layout_is_f16w(const Layout &L) { return L.unit_k == 128 && L.unit_bytes == 4096; }
 
 // nibble position of fragment element e inside a granule word
 RLX_HD constexpr int nib_pos(int e) { return ((e & 1) << 2) | (e >> 1); }
@@ -83,8 +96,7 @@ struct WeightDims {
     int64_t bytes;       // device bytes
 };
 
-RLX_HD inline WeightDims weight_dims(int scheme, int64_t n, int64_t k) {
-    Layout L = layout_of(scheme);
+RLX_HD inline WeightDims weight_dims(const Layout &L, int64_t n, int64_t k) {
     WeightDims d{};
     d.n = n;
     d.k = k;
@@ -96,5 +108,6 @@ RLX_HD inline WeightDims weight_dims(int scheme, int64_t n, int64_t k) {
     d.bytes = d.row_tiles * d.units * (int64_t)L.unit_bytes;
     return d;
 }
+RLX_HD inline WeightDims weight_dims(int scheme, int64_t n, int64_t k) { return weight_dims(layout_of(scheme), n, k); }
 
 }  // namespace rlx

@@ -2,11 +2,12 @@
 import numpy as np
 
 Q4K, Q5K, Q6K, Q8K, Q2K, Q3K, Q4_0, Q8_0 = 5, 6, 7, 8, 9, 10, 11, 12
-WIDE = (Q5K, Q6K, Q8K, Q2K, Q3K)  # stored as binary16 on the device
+WIDE = (Q5K, Q8K, Q2K, Q3K)  # stored as binary16 on the device (Q6_K too when RLX_Q6K_SIGNED_SCALES is set)
 SCHEME_NAMES = {Q4K: "q4_k", Q5K: "q5_k", Q6K: "q6_k", Q8K: "q8_k", Q2K: "q2_k", Q3K: "q3_k", Q4_0: "q4_0", Q8_0: "q8_0"}
 BLOCK = {Q4_0: (32, 18), Q8_0: (32, 34), Q4K: (256, 144), Q5K: (256, 176), Q6K: (256, 210), Q8K: (256, 292), Q2K: (256, 84), Q3K: (256, 110)}
 NIB_POS = [0, 4, 1, 5, 2, 6, 3, 7]
-UNIT = {Q4_0: (128, 1152, 1024), Q8_0: (128, 2176, 2048), Q4K: (256, 2304, 2048)}
+UNIT = {Q4_0: (128, 1152, 1024), Q8_0: (128, 2176, 2048), Q4K: (256, 2304, 2048), Q6K: (256, 3360, 3072)}
+Q6K_HI_POS = [4, 20, 8, 24, 6, 22, 10, 26]  # low bit of element e's 2-bit high field in the even word of a pair (csrc/layout.h)
 
 
 def make_weights(scheme, n, k, std=0.02, seed=0):
@@ -60,6 +61,21 @@ def decode_device_layout(scheme, dev, n, k):
                         code = b - 128
                     cols = np.arange(units) * unit_k + t * 32 + g * 8 + e
                     out[np.ix_(rows, cols)] = d * code.astype(np.float32)
+        elif scheme == Q6K:  # the matmul's reading: (d * sc) * (q - 32), scale bytes unsigned
+            d = dev[:, :, 3328 + nrow * 2: 3328 + nrow * 2 + 2].copy().view(np.float16).astype(np.float32).reshape(tiles, units)
+            scales = dev[:, :, 3072 + nrow * 16: 3072 + nrow * 16 + 16]
+            hw = dev[:, :, 2048 + l * 16: 2048 + l * 16 + 16].copy().view(np.uint32).reshape(tiles, units, 4)
+            for j in range(8):
+                off = (j >> 2) * 1024 + l * 16 + (j & 3) * 4
+                w = dev[:, :, off: off + 4].copy().view(np.uint32).reshape(tiles, units)
+                hx = hw[:, :, (j >> 2) * 2 + ((j & 3) >> 1)]
+                if j & 1:
+                    hx = (hx >> 8) | (hx << 24)
+                ds = (d * scales[:, :, 2 * j + (g >> 1)].astype(np.float32)).astype(np.float32)
+                for e in range(8):
+                    code = ((w >> (4 * NIB_POS[e])) & 0xF) | (((hx >> Q6K_HI_POS[e]) & 3) << 4)
+                    cols = np.arange(units) * unit_k + j * 32 + g * 8 + e
+                    out[np.ix_(rows, cols)] = (ds * (code.astype(np.int32) - 32).astype(np.float32)).astype(np.float32)
         else:
             meta = dev[:, :, qbytes + nrow * 16: qbytes + nrow * 16 + 16]
             d = meta[:, :, 0:2].copy().view(np.float16).astype(np.float32).reshape(tiles, units)

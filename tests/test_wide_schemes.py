@@ -1,5 +1,6 @@
 """Q5_K, Q6_K, Q8_K, Q2_K, Q3_K: the other five schemes the reference's gguf_matmul_bt dispatches
-(rlx-cpu/src/gguf_matmul.rs:25-37). Here they are decoded once at upload and kept as binary16 ("wide").
+(rlx-cpu/src/gguf_matmul.rs:25-37). Q6_K has packed kernels of its own; the other four (and Q6_K when its scale bytes are
+to be read as signed) are decoded once at upload and kept as binary16 ("wide").
 
 CPU part: pins the oracle's five block decoders (the reference's own known-answer blocks, closed-form position
 probes, reduction of Q5_K to the pinned Q4_K decoder, independent numpy bit-field decoders on random bytes), then
@@ -11,7 +12,9 @@ import pytest
 import oracle
 import rlx_amd
 from rlx_amd import DType, QuantScheme, ops
-from helpers import BLOCK, Q2K, Q3K, Q4K, Q5K, Q6K, Q8K, WIDE, random_blocks, rel_err
+from helpers import BLOCK, Q2K, Q3K, Q4K, Q5K, Q6K, Q8K, WIDE, decode_device_layout, random_blocks, rel_err
+
+FIVE = WIDE + (Q6K,)
 
 F16 = lambda v: np.frombuffer(np.float16(v).tobytes(), np.uint8)  # noqa: E731
 
@@ -190,7 +193,7 @@ def np_decode(scheme, blocks, signed_q6=True):
     return ((dj * q.astype(np.float32)).astype(np.float32) - mj).reshape(-1)
 
 
-@pytest.mark.parametrize("scheme", WIDE)
+@pytest.mark.parametrize("scheme", FIVE)
 def test_oracle_matches_numpy_bitfields(scheme):
     blocks = random_blocks(scheme, 6, 512, seed=20 + scheme)
     assert np.array_equal(oracle.dequant(scheme, blocks, 6 * 512), np_decode(scheme, blocks))
@@ -228,6 +231,16 @@ def test_repack_host_is_f16_of_the_matmul_decoder(scheme):
     assert np.array_equal(read_wide_layout(dev, n, k).view(np.uint16), want.view(np.uint16))
 
 
+def test_q6k_packed_layout_keeps_every_bit():
+    """The packed Q6_K device layout (same byte count as the GGUF blocks) read back with numpy by the rules of csrc/layout.h."""
+    n, k = 37, 768
+    blocks = random_blocks(Q6K, n, k, seed=47)
+    dev = ops.repack_host(Q6K, blocks, n, k)
+    assert dev.size == ((n + 15) // 16) * (k // 256) * 16 * 210
+    assert np.array_equal(decode_device_layout(Q6K, dev, n, k).view(np.uint32),
+                          oracle.dequant_matmul_blocks(Q6K, blocks, n * k).reshape(n, k).view(np.uint32))
+
+
 def test_repack_rejects_weights_beyond_binary16():
     blk = np.concatenate([np.frombuffer(np.float32(1e4).tobytes(), np.uint8), np.full(256, 100, np.uint8), np.zeros(32, np.uint8)])
     with pytest.raises(rlx_amd.RlxError, match="binary16"):
@@ -259,7 +272,7 @@ def run_wide(scheme, blocks, m, n, k, dtype):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("scheme", WIDE)
+@pytest.mark.parametrize("scheme", FIVE)
 @pytest.mark.parametrize("m,n,k,dtype", SHAPES)
 def test_wide_matmul_matches_f64_oracle(scheme, m, n, k, dtype):
     """Weights of model-like magnitude: the reference tests' bound, |delta| / max(|expected|, 1) <= 2e-3
@@ -271,7 +284,7 @@ def test_wide_matmul_matches_f64_oracle(scheme, m, n, k, dtype):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("scheme", WIDE)
+@pytest.mark.parametrize("scheme", FIVE)
 @pytest.mark.parametrize("m,n,k,dtype", [SHAPES[0], SHAPES[3]])
 def test_wide_matmul_error_is_the_binary16_rounding_of_the_weights(scheme, m, n, k, dtype):
     """Arbitrary scale bytes (weights up to tens, sums in the hundreds, heavy cancellation): the only error source is
@@ -321,6 +334,35 @@ def test_q6k_graph_runs_and_is_finite():
     out = exe.run([("x", xv)])[0]
     assert out.size == n and np.all(np.isfinite(out))
     assert rel_err(out, oracle.gguf_matmul_f64(xv, blk, 1, k, n, Q6K)) <= 2e-3
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("n,k", [(16, 256), (37, 768), (300, 4096)])
+def test_q6k_dequant_is_bit_exact(n, k):
+    """rlx_mi355x_dequant on the packed Q6_K layout = the block decoder the reference's matmul calls (lib.rs:819-845)."""
+    blocks = random_blocks(Q6K, n, k, seed=n + k)
+    qw = ops.QWeight(QuantScheme.GgufQ6K, blocks, n, k)
+    got = qw.dequant()
+    qw.free()
+    assert np.array_equal(got.reshape(-1).view(np.uint32), oracle.dequant_matmul_blocks(Q6K, blocks, n * k).view(np.uint32))
+
+
+@pytest.mark.gpu
+def test_q6k_signed_scales_on_request(monkeypatch):
+    """RLX_Q6K_SIGNED_SCALES (read at upload) selects ggml's reading of the scale bytes; the weight is then kept as binary16."""
+    n, k, m = 40, 512, 1
+    blocks = random_blocks(Q6K, n, k, seed=5, d_std=5e-6)
+    x = np.random.default_rng(6).standard_normal((m, k)).astype(np.float32)
+    monkeypatch.setenv("RLX_Q6K_SIGNED_SCALES", "1")
+    qw = ops.QWeight(QuantScheme.GgufQ6K, blocks, n, k)
+    assert qw.device_bytes() == 3 * (k // 128) * 4096
+    got = ops.gguf_matmul_bt(x, qw, m)
+    qw.free()
+    monkeypatch.delenv("RLX_Q6K_SIGNED_SCALES")
+    w_signed = oracle.dequant(Q6K, blocks, n * k).reshape(n, k).astype(np.float64)
+    assert rel_err(got, x.astype(np.float64) @ w_signed.T) <= 2e-3
+    w_unsigned = oracle.dequant_matmul_blocks(Q6K, blocks, n * k).reshape(n, k).astype(np.float64)
+    assert rel_err(got, x.astype(np.float64) @ w_unsigned.T) > 2e-3  # the two readings differ on random scale bytes
 
 
 @pytest.mark.gpu
