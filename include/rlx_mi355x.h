@@ -46,14 +46,14 @@ typedef enum rlx_dtype {
 
 /* rlx_ir::quant::QuantScheme, declaration order (rlx-ir/src/quant.rs:39-79). The eight GGUF schemes the reference's
  * gguf_matmul_bt dispatches (rlx-cpu/src/gguf_matmul.rs:25-37) are claimed; any other value is RLX_ERR_UNSUPPORTED.
- * Q4_K, Q6_K, Q4_0 and Q8_0 stay packed in HBM (same byte count as the GGUF blocks) and have a bit-exact device decoder.
- * Q6_K scale bytes are read as the reference's block decoder reads them, unsigned (rlx-gguf/src/lib.rs:819-845). The other
- * four ("wide") are decoded once at upload with the reference's block decoder and kept as binary16 (2 bytes per weight):
+ * Q4_K, Q5_K, Q6_K, Q4_0 and Q8_0 stay packed in HBM (same byte count as the GGUF blocks) and have a bit-exact device
+ * decoder. Q6_K scale bytes are read as the reference's block decoder reads them, unsigned (rlx-gguf/src/lib.rs:819-845).
+ * The other three ("wide") are decoded once at upload with the reference's block decoder and kept as binary16 (2 bytes per weight):
  * matmuls only, every decoded weight must fit binary16. With the environment variable RLX_Q6K_SIGNED_SCALES set when a
  * Q6_K weight is uploaded, its scales are read as signed (ggml's reading) and it is kept wide as well. */
 typedef enum rlx_quant_scheme {
     RLX_SCHEME_GGUF_Q4K = 5,  /* 256 elems / 144 bytes */
-    RLX_SCHEME_GGUF_Q5K = 6,  /* 256 / 176, wide */
+    RLX_SCHEME_GGUF_Q5K = 6,  /* 256 / 176 */
     RLX_SCHEME_GGUF_Q6K = 7,  /* 256 / 210 */
     RLX_SCHEME_GGUF_Q8K = 8,  /* 256 / 292, wide */
     RLX_SCHEME_GGUF_Q2K = 9,  /* 256 / 84, wide (field order of rlx-gguf/src/lib.rs:857-886) */
@@ -132,8 +132,8 @@ size_t rlx_mi355x_qweight_device_bytes_for(int scheme, int64_t n, int64_t k);
 int rlx_mi355x_repack_host(int scheme, const void *gguf_bytes, size_t nbytes, int64_t n, int64_t k, void *out);
 
 /* rlx_gguf::dequant_q8_0 / dequant_q4_0 / dequant_q4_k (rlx-gguf/src/lib.rs:600-633,974-1013) on the device:
- * out_dev[n*k] f32, row-major [n,k], bit-identical to the reference decoders (Q6_K: to dequant_q6_k_block, the one the
- * matmul calls). RLX_ERR_UNSUPPORTED for the wide schemes (the exact f32 decode is not kept on the device). */
+ * out_dev[n*k] f32, row-major [n,k], bit-identical to the reference decoders (also Q5_K; Q6_K: to dequant_q6_k_block, the
+ * one the matmul calls). RLX_ERR_UNSUPPORTED for the wide schemes (the exact f32 decode is not kept on the device). */
 int rlx_mi355x_dequant(const rlx_qweight *w, float *out_dev, void *stream);
 
 /* rlx_cpu::gguf_matmul::gguf_matmul_bt (rlx-cpu/src/gguf_matmul.rs:40-95):

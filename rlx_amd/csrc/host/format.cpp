@@ -240,6 +240,30 @@ int repack_host(int scheme, const uint8_t *src, size_t nbytes, int64_t n, int64_
                             for (int e = 0; e < 8; e++) dst[e] = live ? (uint8_t)(b[2 + 8 * g + e] ^ 0x80u) : 0x80u;
                         }
                     }
+                } else if (scheme == SCHEME_Q5K) {  // one super-block per unit: nibbles as Q4_K, fifth-bit words, 16 meta bytes
+                    const bool live = r < n && u < bpr;
+                    const uint8_t *b = live ? src + (r * bpr + u) * L.block_bytes : nullptr;
+                    if (g == 0) {
+                        if (live) memcpy(unit + 2560 + nrow * 16, b, 16);
+                        else memset(unit + 2560 + nrow * 16, 0, 16);
+                    }
+                    uint32_t hb[2] = {0, 0};
+                    for (int j = 0; j < 8; j++) {
+                        uint32_t word = 0;
+                        for (int e = 0; e < 8; e++) {
+                            const int l5 = 8 * g + e;  // element of sub-block j
+                            uint32_t nib = 0, bit = 0;
+                            if (live) {
+                                const uint8_t byte = b[48 + 32 * (j >> 1) + l5];
+                                nib = (j & 1) ? (uint32_t)(byte >> 4) : (uint32_t)(byte & 0x0F);
+                                bit = (uint32_t)(b[16 + l5] >> j) & 1u;
+                            }
+                            word |= nib << (4 * nib_pos(e));
+                            hb[j >> 2] |= bit << ((q5k_hi_pos(e) + q5k_rot(j & 3)) & 31);
+                        }
+                        memcpy(unit + (j >> 2) * 1024 + l * 16 + (j & 3) * 4, &word, 4);
+                    }
+                    memcpy(unit + 2048 + l * 8, hb, 8);
                 } else if (scheme == SCHEME_Q6K) {  // one super-block per unit: low nibbles, high-bit words, scales, d
                     const bool live = r < n && u < bpr;
                     const uint8_t *b = live ? src + (r * bpr + u) * L.block_bytes : nullptr;

@@ -106,7 +106,7 @@ static int launch_gemv(const void *const *xs, int xk, const rlx_qweight *const *
     const bool r2 = rv <= 2;
     // kernel = scheme family x {r2, r4, r2_argmax, r2_paired, r4_paired}
     const int family = wide ? K_GEMV_F16W_R2 : scheme == SCHEME_Q4_0 ? K_GEMV_Q4_0_R2 : scheme == SCHEME_Q8_0 ? K_GEMV_Q8_0_R2
-                       : scheme == SCHEME_Q6K ? K_GEMV_Q6_K_R2 : K_GEMV_Q4_K_R2;
+                       : scheme == SCHEME_Q6K ? K_GEMV_Q6_K_R2 : scheme == SCHEME_Q5K ? K_GEMV_Q5_K_R2 : K_GEMV_Q4_K_R2;
     if (argmax_key && !r2) {
         set_error("gemv: the argmax epilogue takes one activation row");
         return RLX_ERR_INVALID;
@@ -131,7 +131,7 @@ static int launch_gemv(const void *const *xs, int xk, const rlx_qweight *const *
     const size_t slot_bytes = (size_t)ng * 256;
     auto stage_bytes = [&](int kcu) {
         size_t b = ((size_t)rv * ((size_t)kcu * L.unit_k + 8) * 2 + 15) & ~(size_t)15;
-        if (scheme == SCHEME_Q4K) b += (size_t)kcu * (L.unit_k / 32) * 16 * 4;
+        if (scheme == SCHEME_Q4K || (scheme == SCHEME_Q5K && !wide)) b += (size_t)kcu * (L.unit_k / 32) * 16 * 4;  // block sums
         return b;
     };
     // A launch shape: `wgs_per_cu` workgroups of `waves` waves per CU, every one resident at once, each with the same
@@ -210,7 +210,7 @@ static GemmPlan gemm_plan(int scheme, int xk, int64_t m, int64_t k) {
     p.m_rows = (rv + 255) / 256 * 256;
     p.k_pad = (k + 255) / 256 * 256;
     p.xh_bytes = ((size_t)p.m_rows * p.k_pad * 2 + 255) & ~(size_t)255;
-    p.sxh_bytes = scheme == SCHEME_Q4K ? (size_t)p.m_rows * (p.k_pad / 256) * 32 : 0;
+    p.sxh_bytes = (scheme == SCHEME_Q4K || scheme == SCHEME_Q5K) ? (size_t)p.m_rows * (p.k_pad / 256) * 32 : 0;
     return p;
 }
 
@@ -259,6 +259,7 @@ static int launch_gemm(const void *x, int xk, const rlx_qweight *w, float *out, 
                   : w->scheme == SCHEME_Q4_0    ? (skinny ? K_GEMM64_Q4_0 : K_GEMM_Q4_0)
                   : layout_is_f16w(L)           ? (skinny ? K_GEMM64_F16W : K_GEMM_F16W)
                   : w->scheme == SCHEME_Q6K     ? (skinny ? K_GEMM64_Q6_K : K_GEMM_Q6_K)
+                  : w->scheme == SCHEME_Q5K     ? (skinny ? K_GEMM64_Q5_K : K_GEMM_Q5_K)
                                                 : (skinny ? K_GEMM64_Q8_0 : K_GEMM_Q8_0);
     RLX_TRY(runtime_init());
     RLX_TRY(launch3(id, (unsigned)gx, (unsigned)gy, (unsigned)split, 512, skinny ? 3 * 24 * 1024 : 3 * 48 * 1024, stream, params));
@@ -357,7 +358,7 @@ int rlx_mi355x_dequant(const rlx_qweight *w, float *out_dev, void *stream) {
     DequantArgs a{w->dev, out_dev, w->dims.n, w->dims.k, w->dims.units};
     void *params[] = {&a};
     KernelId id = w->scheme == SCHEME_Q4_0 ? K_DEQUANT_Q4_0 : w->scheme == SCHEME_Q8_0 ? K_DEQUANT_Q8_0
-                  : w->scheme == SCHEME_Q6K ? K_DEQUANT_Q6_K : K_DEQUANT_Q4_K;
+                  : w->scheme == SCHEME_Q6K ? K_DEQUANT_Q6_K : w->scheme == SCHEME_Q5K ? K_DEQUANT_Q5_K : K_DEQUANT_Q4_K;
     return launch(id, (unsigned)w->dims.units, (unsigned)w->dims.row_tiles, 64, 0, (hipStream_t)stream, params);
 }
 

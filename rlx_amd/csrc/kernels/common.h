@@ -79,6 +79,39 @@ __device__ __forceinline__ void unpack_q4_scaled(uint32_t w, half2_t sc, Frag &f
     f.h2[3] = __builtin_elementwise_fma(a3, sc16, neg_hi);
 }
 
+// Q5_K: the same two decoders with the fifth bits merged into the magic numbers first. hx is the half's high-bit word
+// rotated right by q5k_rot(t) for code word t (see layout.h); sc * q <= 63 * 31 stays exact in binary16.
+__device__ __forceinline__ void q5_magic(uint32_t w, uint32_t hx, uint32_t a[4]) {
+    const uint32_t w2 = w >> 8, h1 = hx >> 1;
+    a[0] = (hx & 0x00100010u) | and_or(w, 0x000F000Fu, MAGIC);   // 1024 + q
+    a[1] = (hx & 0x01000100u) | and_or(w, 0x00F000F0u, MAGIC);   // 1024 + 16 q
+    a[2] = (h1 & 0x00100010u) | and_or(w2, 0x000F000Fu, MAGIC);
+    a[3] = (h1 & 0x01000100u) | and_or(w2, 0x00F000F0u, MAGIC);
+}
+__device__ __forceinline__ void unpack_q5(uint32_t w, uint32_t hx, Frag &f) {  // q, exact
+    const half2_t sub_lo = {(half_t)(-1024.0f), (half_t)(-1024.0f)};
+    const half2_t mul_hi = {(half_t)0.0625f, (half_t)0.0625f};
+    const half2_t sub_hi = {(half_t)(-64.0f), (half_t)(-64.0f)};
+    uint32_t a[4];
+    q5_magic(w, hx, a);
+    f.h2[0] = as_half2(a[0]) + sub_lo;
+    f.h2[1] = __builtin_elementwise_fma(as_half2(a[1]), mul_hi, sub_hi);
+    f.h2[2] = as_half2(a[2]) + sub_lo;
+    f.h2[3] = __builtin_elementwise_fma(as_half2(a[3]), mul_hi, sub_hi);
+}
+__device__ __forceinline__ void unpack_q5_scaled(uint32_t w, uint32_t hx, half2_t sc, Frag &f) {  // sc * q, exact
+    const half2_t k1024 = {(half_t)1024.0f, (half_t)1024.0f};
+    const half2_t k64 = {(half_t)64.0f, (half_t)64.0f};
+    const half2_t r16 = {(half_t)0.0625f, (half_t)0.0625f};
+    const half2_t neg_lo = -(sc * k1024), neg_hi = -(sc * k64), sc16 = sc * r16;
+    uint32_t a[4];
+    q5_magic(w, hx, a);
+    f.h2[0] = __builtin_elementwise_fma(as_half2(a[0]), sc, neg_lo);
+    f.h2[1] = __builtin_elementwise_fma(as_half2(a[1]), sc16, neg_hi);
+    f.h2[2] = __builtin_elementwise_fma(as_half2(a[2]), sc, neg_lo);
+    f.h2[3] = __builtin_elementwise_fma(as_half2(a[3]), sc16, neg_hi);
+}
+
 // Q8_0 granule (two words of offset-binary bytes) -> signed codes as halfs, fragment order.
 __device__ __forceinline__ void unpack_q8(uint32_t w0, uint32_t w1, Frag &f) {
     const half2_t sub = {(half_t)(-1152.0f), (half_t)(-1152.0f)};  // 1024 + 128

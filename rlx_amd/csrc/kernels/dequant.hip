@@ -85,8 +85,11 @@ __device__ __forceinline__ void dequant_tile(const DequantArgs &a) {
                 store8(a.out, a.n, a.k, r, u * 256 + j * 32 + g * 8, v);
             }
         }
-    } else {
-        uint4_t meta = *(const uint4_t *)(unit + 2048 + nrow * 16);
+    } else {  // Q4_K and Q5_K (the same with a fifth bit per code)
+        constexpr bool K5 = SCHEME == SCHEME_Q5K;
+        uint4_t meta = *(const uint4_t *)(unit + (K5 ? 2560 : 2048) + nrow * 16);
+        uint2_t hb = {0, 0};
+        if constexpr (K5) hb = *(const uint2_t *)(unit + 2048 + l * 8);
         float d = half_bits_to_float(meta[0] & 0xFFFFu);
         float dmin = half_bits_to_float(meta[0] >> 16);
         uint32_t sc[2], mn[2];
@@ -99,9 +102,10 @@ __device__ __forceinline__ void dequant_tile(const DequantArgs &a) {
                 float dj = d * ubyte_to_float(sc[h], t);
                 float mj = dmin * ubyte_to_float(mn[h], t);
                 float v[8];
+                const uint32_t hx = __builtin_amdgcn_alignbit(hb[h], hb[h], q5k_rot(t));  // zero for Q4_K
 #pragma unroll
                 for (int e = 0; e < 8; e++) {
-                    float code = (float)((q[t] >> (4 * nib_pos(e))) & 0xFu);
+                    float code = (float)(((q[t] >> (4 * nib_pos(e))) & 0xFu) + 16u * ((hx >> q5k_hi_pos(e)) & 1u));
                     float prod = dj * code;
                     v[e] = prod - mj;
                 }
@@ -116,4 +120,5 @@ __device__ __forceinline__ void dequant_tile(const DequantArgs &a) {
 extern "C" __global__ __launch_bounds__(64) void rlx_dequant_q4_0(rlx::DequantArgs a) { rlx::dequant_tile<rlx::SCHEME_Q4_0>(a); }
 extern "C" __global__ __launch_bounds__(64) void rlx_dequant_q8_0(rlx::DequantArgs a) { rlx::dequant_tile<rlx::SCHEME_Q8_0>(a); }
 extern "C" __global__ __launch_bounds__(64) void rlx_dequant_q4_k(rlx::DequantArgs a) { rlx::dequant_tile<rlx::SCHEME_Q4K>(a); }
+extern "C" __global__ __launch_bounds__(64) void rlx_dequant_q5_k(rlx::DequantArgs a) { rlx::dequant_tile<rlx::SCHEME_Q5K>(a); }
 extern "C" __global__ __launch_bounds__(64) void rlx_dequant_q6_k(rlx::DequantArgs a) { rlx::dequant_tile<rlx::SCHEME_Q6K>(a); }

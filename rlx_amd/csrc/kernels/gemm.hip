@@ -65,8 +65,10 @@ __device__ __forceinline__ int frag_offset(int ns, int ks, int s, int r, int h) 
 template <int SCHEME, int TI, int TJ>
 __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
     constexpr Layout L = layout_of(SCHEME);
-    constexpr bool K4 = SCHEME == SCHEME_Q4K;
+    constexpr bool K5 = SCHEME == SCHEME_Q5K;                 // Q4_K with a fifth bit: every Q4_K branch below serves both
+    constexpr bool K4 = SCHEME == SCHEME_Q4K || K5;
     constexpr bool K6 = SCHEME == SCHEME_Q6K;
+    constexpr int META_OFF = K5 ? 2560 : 2048;                // the 16 meta bytes per row of a Q4_K / Q5_K unit
     // Super-block schemes: B holds integers (Q4_K: sc * q, exact; Q6_K: sc * (q - 32), exact up to 2048), a second
     // accumulator set collects one 256-column super-block and d (Q4_K: and dmin) is applied in f32 per super-block.
     constexpr bool SB = K4 || K6;
@@ -126,8 +128,12 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
     auto fetch_b = [&](int step, int q) {  // q = step & 3, compile-time at every call site
         if constexpr (K4) {  // dead tiles read tile 0 (valid memory) and are zeroed when stored
             const int unit = (step >> 2) * L.unit_bytes;
-            if ((q & 1) == 0) b_q[(q >> 1) & 1] = ld128(b_rsrc, lane * 16, unit + (q >> 1) * 1024);
-            if (q == 0) b_meta[0] = ld128(b_rsrc, b_n16 * 16, unit + 2048);  // consumed one step later, before the next fetch
+            if ((q & 1) == 0) {
+                b_q[(q >> 1) & 1] = ld128(b_rsrc, lane * 16, unit + (q >> 1) * 1024);
+                if constexpr (K5)  // the half's fifth-bit word
+                    b_hw[(q >> 1) & 1][0] = __builtin_amdgcn_raw_buffer_load_b32(b_rsrc, lane * 8 + (q >> 1) * 4, unit + 2048, 0);
+            }
+            if (q == 0) b_meta[0] = ld128(b_rsrc, b_n16 * 16, unit + META_OFF);  // consumed one step later, before the next fetch
         } else if constexpr (K6) {  // codes and high-bit words of a half every second step, the row's 16 scale bytes per super-block
             const int unit = (step >> 2) * L.unit_bytes;
             if ((q & 1) == 0) {
@@ -175,7 +181,10 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
                 b_sc[0] &= b_keep;  // a dead tile decodes to zeros
                 b_sc[1] &= b_keep;
             }
-            unpack_q4_scaled(b_q[cp][t], splat_code_half(b_sc[q >> 1], t), f);
+            if constexpr (K5)
+                unpack_q5_scaled(b_q[cp][t], __builtin_amdgcn_alignbit(b_hw[cp][0], b_hw[cp][0], q5k_rot(t)), splat_code_half(b_sc[q >> 1], t), f);
+            else
+                unpack_q4_scaled(b_q[cp][t], splat_code_half(b_sc[q >> 1], t), f);
         } else if constexpr (K6) {
             if (q == 0 && jl == 0) {  // this super-block's scales, out of the way of the next super-block's fetch
 #pragma unroll
@@ -221,7 +230,7 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
         my_row[j] = n_tile0 + (wn * TJ + j) * 32 + lr;
         my_ok[j] = (my_row[j] >> 4) < a.row_tiles;
         my_meta[j] = a.w + (long long)(my_ok[j] ? (my_row[j] >> 4) : 0) * a.units * L.unit_bytes +
-                     (K6 ? 3328 + (my_row[j] & 15) * 2 : 2048 + (my_row[j] & 15) * 16);  // Q6_K: the row's d; Q4_K: its 16 meta bytes
+                     (K6 ? 3328 + (my_row[j] & 15) * 2 : META_OFF + (my_row[j] & 15) * 16);  // Q6_K: the row's d; Q4_K / Q5_K: its 16 meta bytes
     }
     uint4_t w_meta[TJ];
     Frag fs[TI];
@@ -523,6 +532,8 @@ __device__ __forceinline__ void xprep_body(const XPrepArgs &a) {
 extern "C" __global__ __launch_bounds__(512) void rlx_gemm_q4_k(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q4K, 2, 2>(a); }
 extern "C" __global__ __launch_bounds__(512) void rlx_gemm_q4_0(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q4_0, 2, 2>(a); }
 extern "C" __global__ __launch_bounds__(512) void rlx_gemm_q8_0(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q8_0, 2, 2>(a); }
+extern "C" __global__ __launch_bounds__(512) void rlx_gemm_q5_k(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q5K, 2, 2>(a); }
+extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64_q5_k(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q5K, 1, 1>(a); }
 extern "C" __global__ __launch_bounds__(512) void rlx_gemm_q6_k(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q6K, 2, 2>(a); }
 extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64_q6_k(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q6K, 1, 1>(a); }
 extern "C" __global__ __launch_bounds__(512) void rlx_gemm_f16w(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_F16W, 2, 2>(a); }

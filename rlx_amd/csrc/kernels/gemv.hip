@@ -106,6 +106,22 @@ struct UnitRegs<SCHEME_Q4K> {
 };
 
 template <>
+struct UnitRegs<SCHEME_Q5K> {  // Q4_K plus the two fifth-bit words of the lane
+    uint4_t q0, q1, meta;
+    uint2_t hb;
+    __device__ __forceinline__ void load(const uint8_t *unit, int l, int nrow, bool) {
+        q0 = __builtin_nontemporal_load((const uint4_t *)(unit + l * 16));
+        q1 = __builtin_nontemporal_load((const uint4_t *)(unit + 1024 + l * 16));
+        hb = __builtin_nontemporal_load((const uint2_t *)(unit + 2048 + l * 8));
+        meta = __builtin_nontemporal_load((const uint4_t *)(unit + 2560 + nrow * 16));
+    }
+    __device__ __forceinline__ void clear() {
+        q0 = q1 = meta = uint4_t{0, 0, 0, 0};
+        hb = uint2_t{0, 0};
+    }
+};
+
+template <>
 struct UnitRegs<SCHEME_Q6K> {  // one super-block: low nibbles (two halves), high-bit words, the row's 16 scales, d
     uint4_t q0, q1, hw, sc;
     uint32_t d;
@@ -229,7 +245,10 @@ __device__ __forceinline__ void compute_unit(const UnitRegs<SCHEME> &w, const ha
             load_afrags<4>(xrow, live, ucol + h * 128, a);
             const uint4_t &q = h ? w.q1 : w.q0;
 #pragma unroll
-            for (int t = 0; t < 4; t++) unpack_q4<0>(q[t], b[t]);
+            for (int t = 0; t < 4; t++) {
+                if constexpr (SCHEME == SCHEME_Q5K) unpack_q5(q[t], __builtin_amdgcn_alignbit(w.hb[h], w.hb[h], q5k_rot(t)), b[t]);
+                else unpack_q4<0>(q[t], b[t]);
+            }
             float4_t blk[4];
 #pragma unroll
             for (int t = 0; t < 4; t++) blk[t] = mfma16(a[t], b[t], zero);
@@ -461,7 +480,7 @@ __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
         if constexpr ((MODE & GEMV_NORM) != 0) stage_x_typed<X_F32, true>(a, seg, xs, row_stride, u0 * L.unit_k, nu * L.unit_k, inv_rms);
         else stage_x(a, seg, xs, row_stride, u0 * L.unit_k, nu * L.unit_k);
         __syncthreads();
-        if constexpr (SCHEME == SCHEME_Q4K) {
+        if constexpr (SCHEME == SCHEME_Q4K || SCHEME == SCHEME_Q5K) {
             const int nblk = nu * BLK_PER_UNIT;
             // rows >= rv of the [blk][16] table are never read: compute_unit only uses the rows its lane group owns
             for (int idx = tid; idx < nblk * rv; idx += blockDim.x) {
@@ -575,4 +594,5 @@ RLX_GEMV_SCHEME(q8_0, rlx::SCHEME_Q8_0, 3)
 RLX_GEMV_SCHEME(q4_k, rlx::SCHEME_Q4K, 3)
 RLX_GEMV_SCHEME(f16w, rlx::SCHEME_F16W, 2)
 RLX_GEMV_SCHEME(q6_k, rlx::SCHEME_Q6K, 2)
+RLX_GEMV_SCHEME(q5_k, rlx::SCHEME_Q5K, 2)
 RLX_GEMV_INST(rlx_gemv_q4_0_r2_d8, rlx::SCHEME_Q4_0, 2, 8, rlx::GEMV_PLAIN)

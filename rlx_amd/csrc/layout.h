@@ -20,6 +20,11 @@
 //          [2048,2176) f16 d[n][4]
 //   Q4_K : [0,2048)  two halves h: 16 B at 1024*h + 16*l = granules of sub-blocks 4h+0..3 of super-block u
 //          [2048,2304) per row n: 16 B = f16 d, f16 dmin, 12 scale bytes (verbatim from the GGUF block)
+//   Q5_K : [0,2048)  the nibbles, as Q4_K          [2048,2560) the fifth bits: 8 B at 2048 + 8*l = words hb[h], one per half,
+//                   serving the half's four code words t after a rotate right by Q5K_ROT[t] = {0, 2, 8, 10}: element e of the
+//                   rotated word sits at bit Q5K_HI_POS[e] (elements 0,1 / 4,5 at mantissa bit 4 / 20 of 1024 + q, elements
+//                   2,3 / 6,7 at bit 8 / 24 of 1024 + 16 q, elements 4-7 one bit higher and used after a shift by 1)
+//          [2560,2816) per row n: 16 B = f16 d, f16 dmin, 12 scale bytes (verbatim, as Q4_K)
 //   Q6_K : [0,2048)  low nibbles of the 6-bit codes, two halves h like Q4_K (word t of a slot = 32-column block 4h + t)
 //          [2048,3072) the two high bits of every code: 16 B at 2048 + 16*l = words hw[2h + j], one per pair of code
 //                   words (t = 2j, 2j + 1) of half h. In hw the field of element e of the even word sits at bit
@@ -29,7 +34,7 @@
 //                   elements 2,3 / 6,7 (value 1024 + 16 q) at bits 8-9 / 24-25; elements 4-7 are stored 2 bits higher
 //                   and used after a shift by 2, like their nibbles after a shift by 8.
 //          [3072,3328) per row n: the 16 scale bytes verbatim          [3328,3360) f16 d[n]
-//   Q5_K, Q8_K, Q2_K, Q3_K, and Q6_K when its scales are to be read as signed ("wide" schemes): the weights are decoded once, at upload, with the reference's block
+//   Q8_K, Q2_K, Q3_K, and Q6_K when its scales are to be read as signed ("wide" schemes): the weights are decoded once, at upload, with the reference's block
 //          decoder and stored as binary16: [0,4096) four blocks t: 16 B at 1024*t + 16*l = the 8 halfs of granule
 //          (n, 4u+t, g), already an MFMA operand fragment. No scales. 2 bytes per weight resident instead of the
 //          packed 0.33-1.14, in exchange for kernels that do no decode arithmetic at all.
@@ -53,6 +58,9 @@ enum Scheme : int {
     SCHEME_Q4_0 = 11, SCHEME_Q8_0 = 12, SCHEME_F16W = 100
 };
 
+// fifth bit of element e inside a Q5_K high-bit word (after the rotate of its code word), and the rotates
+RLX_HD constexpr int q5k_hi_pos(int e) { return e == 0 ? 4 : e == 1 ? 20 : e == 2 ? 8 : e == 3 ? 24 : e == 4 ? 5 : e == 5 ? 21 : e == 6 ? 9 : 25; }
+RLX_HD constexpr int q5k_rot(int t) { return t == 0 ? 0 : t == 1 ? 2 : t == 2 ? 8 : 10; }
 // low bit of the 2-bit high field of element e (even code word of a pair) inside a Q6_K high-bit word
 RLX_HD constexpr int q6k_hi_pos(int e) { return e == 0 ? 4 : e == 1 ? 20 : e == 2 ? 8 : e == 3 ? 24 : e == 4 ? 6 : e == 5 ? 22 : e == 6 ? 10 : 26; }
 
@@ -70,7 +78,7 @@ RLX_HD constexpr Layout layout_of(int scheme) {
     return scheme == SCHEME_Q4_0   ? Layout{128, 1152, 1024, 32, 18}
            : scheme == SCHEME_Q8_0 ? Layout{128, 2176, 2048, 32, 34}
            : scheme == SCHEME_Q4K  ? Layout{256, 2304, 2048, 256, 144}
-           : scheme == SCHEME_Q5K  ? Layout{128, 4096, 4096, 256, 176}
+           : scheme == SCHEME_Q5K  ? Layout{256, 2816, 2560, 256, 176}
            : scheme == SCHEME_Q6K  ? Layout{256, 3360, 3072, 256, 210}
            : scheme == SCHEME_Q8K  ? Layout{128, 4096, 4096, 256, 292}
            : scheme == SCHEME_Q2K  ? Layout{128, 4096, 4096, 256, 84}

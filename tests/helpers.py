@@ -2,11 +2,13 @@
 import numpy as np
 
 Q4K, Q5K, Q6K, Q8K, Q2K, Q3K, Q4_0, Q8_0 = 5, 6, 7, 8, 9, 10, 11, 12
-WIDE = (Q5K, Q8K, Q2K, Q3K)  # stored as binary16 on the device (Q6_K too when RLX_Q6K_SIGNED_SCALES is set)
+WIDE = (Q8K, Q2K, Q3K)  # stored as binary16 on the device (Q6_K too when RLX_Q6K_SIGNED_SCALES is set)
 SCHEME_NAMES = {Q4K: "q4_k", Q5K: "q5_k", Q6K: "q6_k", Q8K: "q8_k", Q2K: "q2_k", Q3K: "q3_k", Q4_0: "q4_0", Q8_0: "q8_0"}
 BLOCK = {Q4_0: (32, 18), Q8_0: (32, 34), Q4K: (256, 144), Q5K: (256, 176), Q6K: (256, 210), Q8K: (256, 292), Q2K: (256, 84), Q3K: (256, 110)}
 NIB_POS = [0, 4, 1, 5, 2, 6, 3, 7]
-UNIT = {Q4_0: (128, 1152, 1024), Q8_0: (128, 2176, 2048), Q4K: (256, 2304, 2048), Q6K: (256, 3360, 3072)}
+UNIT = {Q4_0: (128, 1152, 1024), Q8_0: (128, 2176, 2048), Q4K: (256, 2304, 2048), Q5K: (256, 2816, 2560), Q6K: (256, 3360, 3072)}
+Q5K_HI_POS = [4, 20, 8, 24, 5, 21, 9, 25]  # fifth bit of element e in the half's word after its code word's rotate (csrc/layout.h)
+Q5K_ROT = [0, 2, 8, 10]
 Q6K_HI_POS = [4, 20, 8, 24, 6, 22, 10, 26]  # low bit of element e's 2-bit high field in the even word of a pair (csrc/layout.h)
 
 
@@ -91,8 +93,14 @@ def decode_device_layout(scheme, dev, n, k):
                 mj = (dmin * mn.astype(np.float32)).astype(np.float32)
                 off = (j >> 2) * 1024 + l * 16 + (j & 3) * 4
                 w = dev[:, :, off: off + 4].copy().view(np.uint32).reshape(tiles, units)
+                if scheme == Q5K:
+                    hb = dev[:, :, 2048 + l * 8 + 4 * (j >> 2): 2048 + l * 8 + 4 * (j >> 2) + 4].copy().view(np.uint32).reshape(tiles, units)
+                    rot = Q5K_ROT[j & 3]
+                    hx = (hb >> rot) | (hb << (32 - rot)) if rot else hb
                 for e in range(8):
                     code = ((w >> (4 * NIB_POS[e])) & 0xF).astype(np.float32)
+                    if scheme == Q5K:
+                        code = code + np.float32(16) * ((hx >> Q5K_HI_POS[e]) & 1).astype(np.float32)
                     cols = np.arange(units) * unit_k + j * 32 + g * 8 + e
                     out[np.ix_(rows, cols)] = ((dj * code).astype(np.float32) - mj).astype(np.float32)
     return out[:n, :k]

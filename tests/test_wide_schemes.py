@@ -1,6 +1,6 @@
 """Q5_K, Q6_K, Q8_K, Q2_K, Q3_K: the other five schemes the reference's gguf_matmul_bt dispatches
-(rlx-cpu/src/gguf_matmul.rs:25-37). Q6_K has packed kernels of its own; the other four (and Q6_K when its scale bytes are
-to be read as signed) are decoded once at upload and kept as binary16 ("wide").
+(rlx-cpu/src/gguf_matmul.rs:25-37). Q5_K and Q6_K have packed kernels of their own; the other three (and Q6_K when its
+scale bytes are to be read as signed) are decoded once at upload and kept as binary16 ("wide").
 
 CPU part: pins the oracle's five block decoders (the reference's own known-answer blocks, closed-form position
 probes, reduction of Q5_K to the pinned Q4_K decoder, independent numpy bit-field decoders on random bytes), then
@@ -14,7 +14,8 @@ import rlx_amd
 from rlx_amd import DType, QuantScheme, ops
 from helpers import BLOCK, Q2K, Q3K, Q4K, Q5K, Q6K, Q8K, WIDE, decode_device_layout, random_blocks, rel_err
 
-FIVE = WIDE + (Q6K,)
+FIVE = WIDE + (Q5K, Q6K)
+PACKED = (Q5K, Q6K)
 
 F16 = lambda v: np.frombuffer(np.float16(v).tobytes(), np.uint8)  # noqa: E731
 
@@ -231,14 +232,16 @@ def test_repack_host_is_f16_of_the_matmul_decoder(scheme):
     assert np.array_equal(read_wide_layout(dev, n, k).view(np.uint16), want.view(np.uint16))
 
 
-def test_q6k_packed_layout_keeps_every_bit():
-    """The packed Q6_K device layout (same byte count as the GGUF blocks) read back with numpy by the rules of csrc/layout.h."""
+@pytest.mark.parametrize("scheme", PACKED)
+def test_packed_layout_keeps_every_bit(scheme):
+    """The packed Q5_K / Q6_K device layouts (same byte count as the GGUF blocks) read back with numpy by the rules of
+    csrc/layout.h."""
     n, k = 37, 768
-    blocks = random_blocks(Q6K, n, k, seed=47)
-    dev = ops.repack_host(Q6K, blocks, n, k)
-    assert dev.size == ((n + 15) // 16) * (k // 256) * 16 * 210
-    assert np.array_equal(decode_device_layout(Q6K, dev, n, k).view(np.uint32),
-                          oracle.dequant_matmul_blocks(Q6K, blocks, n * k).reshape(n, k).view(np.uint32))
+    blocks = random_blocks(scheme, n, k, seed=47)
+    dev = ops.repack_host(scheme, blocks, n, k)
+    assert dev.size == ((n + 15) // 16) * (k // 256) * 16 * BLOCK[scheme][1]
+    assert np.array_equal(decode_device_layout(scheme, dev, n, k).view(np.uint32),
+                          oracle.dequant_matmul_blocks(scheme, blocks, n * k).reshape(n, k).view(np.uint32))
 
 
 def test_repack_rejects_weights_beyond_binary16():
@@ -337,14 +340,15 @@ def test_q6k_graph_runs_and_is_finite():
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("scheme", PACKED)
 @pytest.mark.parametrize("n,k", [(16, 256), (37, 768), (300, 4096)])
-def test_q6k_dequant_is_bit_exact(n, k):
-    """rlx_mi355x_dequant on the packed Q6_K layout = the block decoder the reference's matmul calls (lib.rs:819-845)."""
-    blocks = random_blocks(Q6K, n, k, seed=n + k)
-    qw = ops.QWeight(QuantScheme.GgufQ6K, blocks, n, k)
+def test_packed_dequant_is_bit_exact(scheme, n, k):
+    """rlx_mi355x_dequant on the packed layouts = the block decoders the reference's matmul calls (lib.rs:783-845)."""
+    blocks = random_blocks(scheme, n, k, seed=n + k)
+    qw = ops.QWeight(QuantScheme(scheme), blocks, n, k)
     got = qw.dequant()
     qw.free()
-    assert np.array_equal(got.reshape(-1).view(np.uint32), oracle.dequant_matmul_blocks(Q6K, blocks, n * k).view(np.uint32))
+    assert np.array_equal(got.reshape(-1).view(np.uint32), oracle.dequant_matmul_blocks(scheme, blocks, n * k).view(np.uint32))
 
 
 @pytest.mark.gpu
@@ -367,8 +371,8 @@ def test_q6k_signed_scales_on_request(monkeypatch):
 
 @pytest.mark.gpu
 def test_wide_dequant_is_refused():
-    blocks = random_blocks(Q5K, 16, 256, seed=1)
-    qw = ops.QWeight(QuantScheme.GgufQ5K, blocks, 16, 256)
+    blocks = random_blocks(Q8K, 16, 256, seed=1)
+    qw = ops.QWeight(QuantScheme.GgufQ8K, blocks, 16, 256)
     with pytest.raises(rlx_amd.RlxError, match="binary16"):
         qw.dequant()
     qw.free()
