@@ -29,7 +29,7 @@ MFMA_F16_PEAK_TFLOPS = 2500.0  # dense f16/bf16 MFMA peak
 CALIBRATION_COPY_BYTES = 256 << 20
 # HBM bytes per launch of the headline kernel (FETCH_SIZE + WRITE_SIZE of two rocprofv3 --pmc runs of this command,
 # each scaled by the same counter's reading for the copy kernel above); profiles/gemv_q4_0_llama8b_layer_traffic.txt.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 124315038
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 124300624
 
 # (name, N, K) — the Llama-3-8B layer projections of the headline workload
 LLAMA8B = [("q", 4096, 4096), ("k", 1024, 4096), ("v", 1024, 4096), ("o", 4096, 4096),
@@ -189,7 +189,7 @@ def main():
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4),
                      "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH if args.wiring == "independent" else None,
-                     "kernel": "rlx_gemv_q4_0_r2", "avg_launch_us": round(us_per_launch, 3),
+                     "kernel": "rlx_gemv_q4_0_u2_r2", "avg_launch_us": round(us_per_launch, 3),
                      "algorithmic_bytes_per_launch": layer_bytes // launches_per_step},
         "parity_max_rel_err": parity,
         "device": info,

@@ -118,9 +118,7 @@ static int launch_gemv(const void *const *xs, int xk, const rlx_qweight *const *
     const int variant = argmax_key ? (norm ? 9 : 2) : pairs ? (norm ? (r2 ? 7 : 8) : (r2 ? 3 : 4)) : (norm ? (r2 ? 5 : 6) : (r2 ? 0 : 1));
     KernelId id = (KernelId)(family + variant);
     static const int env_waves = getenv("RLX_GEMV_WAVES") ? atoi(getenv("RLX_GEMV_WAVES")) : 8;
-    static const int env_depth = getenv("RLX_GEMV_DEPTH") ? atoi(getenv("RLX_GEMV_DEPTH")) : 4;
     static const int env_wgs_per_cu = getenv("RLX_GEMV_WGS_PER_CU") ? atoi(getenv("RLX_GEMV_WGS_PER_CU")) : 2;
-    if (id == K_GEMV_Q4_0_R2 && env_depth == 8) id = K_GEMV_Q4_0_R2_D8;
     int max_units = 0;
     long long work = 0;  // (tile, unit) items in the launch
     for (int i = 0; i < count; i++) {
@@ -195,6 +193,14 @@ static int launch_gemv(const void *const *xs, int xk, const rlx_qweight *const *
     if (!sh.fits) {
         set_error("gemv: one K unit of %d activation rows does not fit LDS", rv);
         return RLX_ERR_INVALID;
+    }
+    // Two K units per loop item halve the per-item bookkeeping; every chunk of every segment must then hold an even
+    // number of units, and every wave still needs an item.
+    static const bool env_u1 = getenv("RLX_GEMV_UPI") && atoi(getenv("RLX_GEMV_UPI")) == 1;
+    if (family == K_GEMV_Q4_0_R2 && !env_u1 && sh.kcu % 2 == 0 && sh.nwaves * 2 <= max_units) {
+        bool even = true;
+        for (int i = 0; i < count; i++) even = even && ws[i]->dims.units % 2 == 0;
+        if (even) id = (KernelId)(K_GEMV_Q4_0_U2_R2 + variant);
     }
     void *params[] = {&sh.a};
     return launch(id, (unsigned)sh.wg, 1, (unsigned)sh.nwaves * 64, (unsigned)sh.lds, stream, params);

@@ -381,7 +381,7 @@ extern "C" __global__ void rlx_argmax_finish(unsigned long long *key, uint32_t *
 // writes the SwiGLU of the two sums.
 enum { GEMV_PLAIN = 0, GEMV_ARGMAX = 1, GEMV_PAIRED = 2, GEMV_NORM = 4 };  // GEMV_NORM combines with the others
 
-template <int SCHEME, int NREG, int DEPTH, int MODE>
+template <int SCHEME, int NREG, int DEPTH, int MODE, int UPI = 1>
 __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
     constexpr Layout L = layout_of(SCHEME);
     constexpr int BLK_PER_UNIT = L.unit_k / 32;
@@ -453,27 +453,35 @@ __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
         const int nu = min(kc_units, seg.units - u0);  // units in this chunk
         // This wave's items: for each tile, units wave, wave + nwaves, ... < nu. Two cursors walk them: `pf_*` issues
         // loads DEPTH items ahead into a register ring, `cu_*` consumes.
-        const int my_units = wave < nu ? (nu - wave + nwaves - 1) / nwaves : 0;
+        // An item is UPI consecutive units (the host picks UPI > 1 only when every chunk holds a multiple of UPI).
+        const int nug = nu / UPI;
+        const int my_units = wave < nug ? (nug - wave + nwaves - 1) / nwaves : 0;
         const int nitems = nvt * my_units;
         int pf_t = 0, pf_u = wave, pf_n = 0;
-        const uint8_t *pf_ptr = wbase + (long long)(u0 + wave) * L.unit_bytes;
-        UnitRegs<SCHEME> ring[DEPTH];
-        auto prefetch = [&](UnitRegs<SCHEME> &slot) {
+        const uint8_t *pf_ptr = wbase + (long long)(u0 + wave * UPI) * L.unit_bytes;
+        struct Item {
+            UnitRegs<SCHEME> u[UPI];
+        };
+        Item ring[DEPTH];
+        auto prefetch = [&](Item &slot) {
             if (pf_n < nitems) {
-                slot.load(pf_ptr, l, nrow, true);  // every lane loads its column's scales (lanes 16-63 repeat lanes 0-15)
+#pragma unroll
+                for (int p = 0; p < UPI; p++)  // every lane loads its column's scales (lanes 16-63 repeat lanes 0-15)
+                    slot.u[p].load(pf_ptr + p * L.unit_bytes, l, nrow, true);
                 pf_n++;
                 pf_u += nwaves;
-                pf_ptr += (long long)nwaves * L.unit_bytes;
-                if (pf_u >= nu) {
+                pf_ptr += (long long)nwaves * UPI * L.unit_bytes;
+                if (pf_u >= nug) {
                     pf_t++;
                     pf_u = wave;
-                    pf_ptr = vtile_ptr(pf_t) + (long long)(u0 + wave) * L.unit_bytes;
+                    pf_ptr = vtile_ptr(pf_t) + (long long)(u0 + wave * UPI) * L.unit_bytes;
                 }
             }
         };
 #pragma unroll
         for (int d = 0; d < DEPTH; d++) {
-            ring[d].clear();
+#pragma unroll
+            for (int p = 0; p < UPI; p++) ring[d].u[p].clear();
             prefetch(ring[d]);
         }
         if (u0 > 0) __syncthreads();  // previous chunk fully consumed
@@ -506,11 +514,14 @@ __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
 #pragma unroll
             for (int d = 0; d < DEPTH; d++) {
                 if (base + d < nitems) {
-                    UnitRegs<SCHEME> cur = ring[d];
+                    Item cur = ring[d];
                     prefetch(ring[d]);
-                    compute_unit<SCHEME, NREG>(cur, xrow, nrow < rv, afr, sxs, g, cu_u * L.unit_k, cu_u * BLK_PER_UNIT, acc);
+#pragma unroll
+                    for (int p = 0; p < UPI; p++)
+                        compute_unit<SCHEME, NREG>(cur.u[p], xrow, nrow < rv, afr, sxs, g, (cu_u * UPI + p) * L.unit_k,
+                                                   (cu_u * UPI + p) * BLK_PER_UNIT, acc);
                     cu_u += nwaves;
-                    if (cu_u >= nu) {  // last unit of this tile for this wave: bank the partial sums
+                    if (cu_u >= nug) {  // last unit of this tile for this wave: bank the partial sums
                         if (has_rows) {
                             float *slot = part + ((size_t)cu_t * nwaves + wave) * slot_floats + g * 64 + nrow;
 #pragma unroll
@@ -572,27 +583,29 @@ __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
 
 }  // namespace rlx
 
-#define RLX_GEMV_INST(name, SCHEME, NREG, DEPTH, MODE)                                                      \
+#define RLX_GEMV_INST(name, SCHEME, NREG, DEPTH, MODE, UPI)                                                 \
     extern "C" __global__ __launch_bounds__(1024) void name(rlx::GemvArgs a) {                               \
-        rlx::gemv_body<SCHEME, NREG, DEPTH, MODE>(a);                                                         \
+        rlx::gemv_body<SCHEME, NREG, DEPTH, MODE, UPI>(a);                                                    \
     }
 // NREG = 2: at most two virtual rows (m = 1 f32, or m <= 2 16-bit); NREG = 4 otherwise.
-#define RLX_GEMV_SCHEME(tag, SCHEME, DEPTH)                                           \
-    RLX_GEMV_INST(rlx_gemv_##tag##_r2, SCHEME, 2, DEPTH, rlx::GEMV_PLAIN)             \
-    RLX_GEMV_INST(rlx_gemv_##tag##_r4, SCHEME, 4, DEPTH, rlx::GEMV_PLAIN)             \
-    RLX_GEMV_INST(rlx_gemv_##tag##_r2_argmax, SCHEME, 2, DEPTH, rlx::GEMV_ARGMAX)     \
-    RLX_GEMV_INST(rlx_gemv_##tag##_r2_paired, SCHEME, 2, DEPTH, rlx::GEMV_PAIRED)     \
-    RLX_GEMV_INST(rlx_gemv_##tag##_r4_paired, SCHEME, 4, DEPTH, rlx::GEMV_PAIRED)     \
-    RLX_GEMV_INST(rlx_gemv_##tag##_r2_norm, SCHEME, 2, DEPTH, rlx::GEMV_NORM)         \
-    RLX_GEMV_INST(rlx_gemv_##tag##_r4_norm, SCHEME, 4, DEPTH, rlx::GEMV_NORM)         \
-    RLX_GEMV_INST(rlx_gemv_##tag##_r2_norm_paired, SCHEME, 2, DEPTH, rlx::GEMV_NORM | rlx::GEMV_PAIRED) \
-    RLX_GEMV_INST(rlx_gemv_##tag##_r4_norm_paired, SCHEME, 4, DEPTH, rlx::GEMV_NORM | rlx::GEMV_PAIRED) \
-    RLX_GEMV_INST(rlx_gemv_##tag##_r2_norm_argmax, SCHEME, 2, DEPTH, rlx::GEMV_NORM | rlx::GEMV_ARGMAX)
+#define RLX_GEMV_SCHEME(tag, SCHEME, DEPTH, UPI)                                                      \
+    RLX_GEMV_INST(rlx_gemv_##tag##_r2, SCHEME, 2, DEPTH, rlx::GEMV_PLAIN, UPI)                         \
+    RLX_GEMV_INST(rlx_gemv_##tag##_r4, SCHEME, 4, DEPTH, rlx::GEMV_PLAIN, UPI)                         \
+    RLX_GEMV_INST(rlx_gemv_##tag##_r2_argmax, SCHEME, 2, DEPTH, rlx::GEMV_ARGMAX, UPI)                 \
+    RLX_GEMV_INST(rlx_gemv_##tag##_r2_paired, SCHEME, 2, DEPTH, rlx::GEMV_PAIRED, UPI)                 \
+    RLX_GEMV_INST(rlx_gemv_##tag##_r4_paired, SCHEME, 4, DEPTH, rlx::GEMV_PAIRED, UPI)                 \
+    RLX_GEMV_INST(rlx_gemv_##tag##_r2_norm, SCHEME, 2, DEPTH, rlx::GEMV_NORM, UPI)                     \
+    RLX_GEMV_INST(rlx_gemv_##tag##_r4_norm, SCHEME, 4, DEPTH, rlx::GEMV_NORM, UPI)                     \
+    RLX_GEMV_INST(rlx_gemv_##tag##_r2_norm_paired, SCHEME, 2, DEPTH, rlx::GEMV_NORM | rlx::GEMV_PAIRED, UPI) \
+    RLX_GEMV_INST(rlx_gemv_##tag##_r4_norm_paired, SCHEME, 4, DEPTH, rlx::GEMV_NORM | rlx::GEMV_PAIRED, UPI) \
+    RLX_GEMV_INST(rlx_gemv_##tag##_r2_norm_argmax, SCHEME, 2, DEPTH, rlx::GEMV_NORM | rlx::GEMV_ARGMAX, UPI)
 
-RLX_GEMV_SCHEME(q4_0, rlx::SCHEME_Q4_0, 4)
-RLX_GEMV_SCHEME(q8_0, rlx::SCHEME_Q8_0, 3)
-RLX_GEMV_SCHEME(q4_k, rlx::SCHEME_Q4K, 3)
-RLX_GEMV_SCHEME(f16w, rlx::SCHEME_F16W, 2)
-RLX_GEMV_SCHEME(q6_k, rlx::SCHEME_Q6K, 2)
-RLX_GEMV_SCHEME(q5_k, rlx::SCHEME_Q5K, 2)
-RLX_GEMV_INST(rlx_gemv_q4_0_r2_d8, rlx::SCHEME_Q4_0, 2, 8, rlx::GEMV_PLAIN)
+RLX_GEMV_SCHEME(q4_0, rlx::SCHEME_Q4_0, 4, 1)
+RLX_GEMV_SCHEME(q8_0, rlx::SCHEME_Q8_0, 3, 1)
+RLX_GEMV_SCHEME(q4_k, rlx::SCHEME_Q4K, 3, 1)
+RLX_GEMV_SCHEME(f16w, rlx::SCHEME_F16W, 2, 1)
+RLX_GEMV_SCHEME(q6_k, rlx::SCHEME_Q6K, 2, 1)
+RLX_GEMV_SCHEME(q5_k, rlx::SCHEME_Q5K, 2, 1)
+// Two 128-column units per loop item: taken when every K run holds an even number of units. (Measured neutral to
+// slightly slower for Q8_0, whose unit is twice the bytes, so only Q4_0 has it.)
+RLX_GEMV_SCHEME(q4_0_u2, rlx::SCHEME_Q4_0, 2, 2)

@@ -176,6 +176,12 @@ def test_decode_ragged_shapes(oracle, scheme, n, k):
     check_matmul(oracle, scheme, n, k, 3, seed=n)
 
 
+@pytest.mark.parametrize("units", [17, 18, 31])
+def test_decode_q4_0_unit_pairing(oracle, units):
+    # an even unit count walks K two units per loop item (9 pairs over 8 waves here), an odd one a unit at a time
+    check_matmul(oracle, Q4_0, 40, 128 * units, 2, seed=units)
+
+
 def test_rows_just_past_the_decode_limit(oracle):
     check_matmul(oracle, Q4_0, 128, 256, 20, seed=4)           # f32: more than 8 rows -> prefill kernel
     check_matmul(oracle, Q4K, 64, 512, 37, x_dtype=DType.BF16, seed=5)  # more than 16 rows -> prefill kernel
