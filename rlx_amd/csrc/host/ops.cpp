@@ -46,6 +46,7 @@ struct GemvArgs {
     const float *beta;
     float eps;
     int lds_bytes;
+    int kw;
 };
 struct RmsNorm {  // RMSNorm prologue of a decode launch (f32 activations only)
     const float *gamma, *beta;
@@ -142,26 +143,37 @@ static int launch_gemv(const void *const *xs, int xk, const rlx_qweight *const *
         size_t lds;
         bool fits;
     };
-    auto shape = [&](int waves, int wgs_per_cu, size_t budget) {
+    auto shape = [&](int waves, int wgs_per_cu, size_t budget, int kw_req) {
         Shape sh{};
         sh.nwaves = std::max(1, std::min(std::min(16, std::max(1, waves)), max_units));
+        // kw waves share a tile (its K units alternate between them), nwaves / kw tiles run side by side
+        const int kw = (kw_req > 0 && kw_req < sh.nwaves && sh.nwaves % kw_req == 0) ? kw_req : sh.nwaves;
+        const int tw = sh.nwaves / kw;
         const long long slots = (long long)std::max(1, wgs_per_cu) * cus;
-        const long long target_items = std::max<long long>(1, (work + slots - 1) / slots);
-        const int tpw_cap = (int)std::max<size_t>(1, (budget * 2 / 5) / (sh.nwaves * slot_bytes));
+        const int tpw_cap = (int)std::max<size_t>(1, (tw > 1 ? budget / 2 : budget * 2 / 5) / (kw * slot_bytes));
         int max_tpw = 1;
-        for (int i = 0; i < count; i++) {
-            const WeightDims &D = ws[i]->dims;
-            const int per_tile = pairs ? 2 : 1;  // partial-sum slots and K runs per row tile
-            int tpw = (int)std::max<long long>(1, (target_items + D.units * per_tile / 2) / (D.units * per_tile));
-            tpw = std::min(tpw, std::max(1, tpw_cap / per_tile));
-            max_tpw = std::max(max_tpw, tpw * per_tile);
-            const int seg_wgs = (int)((D.row_tiles + tpw - 1) / tpw);
-            static const bool contiguous = getenv("RLX_GEMV_CONTIGUOUS") != nullptr;
-            sh.a.seg[i] = GemvSeg{ws[i]->dev, xs[i], outs[i], (int)D.n, (int)D.k, (int)D.row_tiles, (int)D.units, sh.wg, tpw,
-                                  contiguous ? 1 : seg_wgs, pairs ? pairs[i]->dev : nullptr};
-            sh.wg += seg_wgs;
+        // With tw > 1 a workgroup's tile count is rounded up to whole rounds of tw tiles; the per-workgroup target then
+        // grows until one round of workgroups covers the launch (a few stragglers in a second round would double it).
+        for (double grow = 1.0;; grow += 0.04) {
+            const long long target_items = std::max<long long>(1, (long long)((double)((work + slots - 1) / slots) * grow));
+            sh.wg = 0;
+            max_tpw = 1;
+            for (int i = 0; i < count; i++) {
+                const WeightDims &D = ws[i]->dims;
+                const int per_tile = pairs ? 2 : 1;  // partial-sum slots and K runs per row tile
+                int tpw = (int)std::max<long long>(1, (target_items + D.units * per_tile / 2) / (D.units * per_tile));
+                tpw = std::min((tpw + tw - 1) / tw * tw, std::max(1, tpw_cap / per_tile / tw * tw));
+                tpw = std::max(tpw, 1);
+                max_tpw = std::max(max_tpw, tpw * per_tile);
+                const int seg_wgs = (int)((D.row_tiles + tpw - 1) / tpw);
+                static const bool contiguous = getenv("RLX_GEMV_CONTIGUOUS") != nullptr;
+                sh.a.seg[i] = GemvSeg{ws[i]->dev, xs[i], outs[i], (int)D.n, (int)D.k, (int)D.row_tiles, (int)D.units, sh.wg, tpw,
+                                      contiguous ? 1 : seg_wgs, pairs ? pairs[i]->dev : nullptr};
+                sh.wg += seg_wgs;
+            }
+            if (tw == 1 || sh.wg <= slots || grow > 2.0) break;
         }
-        const size_t part_bytes = (size_t)max_tpw * sh.nwaves * slot_bytes;
+        const size_t part_bytes = (size_t)max_tpw * kw * slot_bytes;
         sh.kcu = max_units;
         while (sh.kcu > 1 && part_bytes + stage_bytes(sh.kcu) + 64 > budget) sh.kcu--;
         sh.fits = part_bytes + stage_bytes(sh.kcu) + 64 <= budget;
@@ -177,17 +189,33 @@ static int launch_gemv(const void *const *xs, int xk, const rlx_qweight *const *
         sh.a.beta = norm ? norm->beta : nullptr;
         sh.a.eps = norm ? norm->eps : 0.f;
         sh.a.lds_bytes = (int)sh.lds;
+        sh.a.kw = kw;
         sh.a.slab_bytes = ws[0]->dims.bytes;
         sh.a.num_experts = ws[0]->experts;
         return sh;
     };
     // Two workgroups of 8 waves per CU with 80 KB each: holds a 14336-wide f32 vector (hi + lo rows) in one chunk.
-    Shape sh = shape(env_waves, env_wgs_per_cu, (size_t)(env_wgs_per_cu <= 1 ? 156 : 80) * 1024);
+    Shape sh = shape(env_waves, env_wgs_per_cu, (size_t)(env_wgs_per_cu <= 1 ? 156 : 80) * 1024, 0);
     // With four or more activation rows every workgroup restages all of x, and that traffic (workgroups x rows x K)
     // rivals the weights: one workgroup of 16 waves per CU with the whole LDS halves it, provided a single round of
     // workgroups still covers the matrix.
     if (rv >= 4 && !getenv("RLX_GEMV_WGS_PER_CU")) {
-        Shape fat = shape(16, 1, (size_t)156 * 1024);
+        // From five rows on, the per-(tile, wave) partial-sum slots (256 B per four rows) are what limits the tiles of
+        // a workgroup: two waves per tile instead of sixteen, eight tiles side by side, keeps the slot area small
+        // enough that one workgroup per CU covers the launch and the activations are staged once per CU.
+        static const int env_kw = getenv("RLX_GEMV_KW") ? atoi(getenv("RLX_GEMV_KW")) : -1;
+        int kw = 0;
+        if (rv >= 5) {  // as many tiles side by side (at most eight) as the segment with the fewest tiles per workgroup has
+            double min_tpw = 1e30;
+            for (int i = 0; i < count; i++)
+                min_tpw = std::min(min_tpw, (double)work / cus / (double)(ws[i]->dims.units * (pairs ? 2 : 1)));
+            int tw = 8;
+            while (tw > 1 && tw > min_tpw * 1.2) tw /= 2;
+            kw = tw > 1 ? 16 / tw : 0;
+        }
+        if (env_kw >= 0) kw = env_kw;
+        Shape fat = shape(16, 1, (size_t)156 * 1024, kw);
+        if (kw && !(fat.fits && fat.wg <= cus)) fat = shape(16, 1, (size_t)156 * 1024, 0);
         if (fat.fits && fat.wg <= cus) sh = fat;
     }
     if (!sh.fits) {

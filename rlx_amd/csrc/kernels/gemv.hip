@@ -57,6 +57,7 @@ struct GemvArgs {
     const float *beta;
     float eps;
     int lds_bytes;     // dynamic LDS of the launch
+    int kw;            // waves that split the K units of one tile; divides the waves of a workgroup
 };
 
 constexpr int XS_PAD_HALFS = 8;      // 16 bytes of padding per LDS row: rows land in different bank groups
@@ -417,12 +418,16 @@ __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
     // LDS: [partial sums: tiles_per_wg x nwaves x (4 ng) x 16 f32][staged activations: rv rows][Q4_K block sums]
     const int slot_floats = ng * 64;
     float *part = (float *)smem;
-    const size_t part_bytes = (size_t)a.max_tiles_per_wg * nwaves * slot_floats * 4;
+    // kw waves split the K units of one tile, tw = nwaves / kw tiles are walked side by side (kw = nwaves: every wave
+    // on the same tile, the decode shape; a small kw keeps the partial-sum area small when the slots are large).
+    const int kw = a.kw, tw = nwaves / kw;
+    const int kl = __builtin_amdgcn_readfirstlane(wave % kw), tl = __builtin_amdgcn_readfirstlane(wave / kw);
+    const size_t part_bytes = (size_t)a.max_tiles_per_wg * kw * slot_floats * 4;
     half_t *xs = (half_t *)(smem + part_bytes);
     float *sxs = (float *)(smem + part_bytes + (((size_t)rv * row_stride * 2 + 15) & ~(size_t)15));  // [blk][16]
     const half_t *xrow = xs + min(nrow, rv - 1) * row_stride + g * 8;  // this lane's A row
 
-    for (int i = tid; i < ((MODE & GEMV_PAIRED) ? 2 : 1) * ntiles * nwaves * slot_floats; i += blockDim.x) part[i] = 0.f;
+    for (int i = tid; i < ((MODE & GEMV_PAIRED) ? 2 : 1) * ntiles * kw * slot_floats; i += blockDim.x) part[i] = 0.f;
     // RMSNorm prologue: one wave per activation row sums the squares of the whole row (the sum is needed before any
     // element can be scaled), 1 / sqrt(mean + eps) lands in the last 64 bytes of the workgroup's LDS.
     float *inv_rms = (float *)(smem + a.lds_bytes - 64);
@@ -455,10 +460,11 @@ __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
         // loads DEPTH items ahead into a register ring, `cu_*` consumes.
         // An item is UPI consecutive units (the host picks UPI > 1 only when every chunk holds a multiple of UPI).
         const int nug = nu / UPI;
-        const int my_units = wave < nug ? (nug - wave + nwaves - 1) / nwaves : 0;
-        const int nitems = nvt * my_units;
-        int pf_t = 0, pf_u = wave, pf_n = 0;
-        const uint8_t *pf_ptr = wbase + (long long)(u0 + wave * UPI) * L.unit_bytes;
+        const int my_units = kl < nug ? (nug - kl + kw - 1) / kw : 0;
+        const int my_tiles = tl < nvt ? (nvt - tl + tw - 1) / tw : 0;
+        const int nitems = my_tiles * my_units;
+        int pf_t = tl, pf_u = kl, pf_n = 0;
+        const uint8_t *pf_ptr = vtile_ptr(tl) + (long long)(u0 + kl * UPI) * L.unit_bytes;
         struct Item {
             UnitRegs<SCHEME> u[UPI];
         };
@@ -469,12 +475,12 @@ __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
                 for (int p = 0; p < UPI; p++)  // every lane loads its column's scales (lanes 16-63 repeat lanes 0-15)
                     slot.u[p].load(pf_ptr + p * L.unit_bytes, l, nrow, true);
                 pf_n++;
-                pf_u += nwaves;
-                pf_ptr += (long long)nwaves * UPI * L.unit_bytes;
+                pf_u += kw;
+                pf_ptr += (long long)kw * UPI * L.unit_bytes;
                 if (pf_u >= nug) {
-                    pf_t++;
-                    pf_u = wave;
-                    pf_ptr = vtile_ptr(pf_t) + (long long)(u0 + wave * UPI) * L.unit_bytes;
+                    pf_t += tw;
+                    pf_u = kl;
+                    pf_ptr = vtile_ptr(pf_t) + (long long)(u0 + kl * UPI) * L.unit_bytes;
                 }
             }
         };
@@ -509,7 +515,7 @@ __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
         Frag afr[4];
 #pragma unroll
         for (int t = 0; t < 4; t++) afr[t].u4 = uint4_t{0, 0, 0, 0};
-        int cu_t = 0, cu_u = wave;
+        int cu_t = tl, cu_u = kl;
         for (int base = 0; base < nitems; base += DEPTH) {
 #pragma unroll
             for (int d = 0; d < DEPTH; d++) {
@@ -520,18 +526,18 @@ __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
                     for (int p = 0; p < UPI; p++)
                         compute_unit<SCHEME, NREG>(cur.u[p], xrow, nrow < rv, afr, sxs, g, (cu_u * UPI + p) * L.unit_k,
                                                    (cu_u * UPI + p) * BLK_PER_UNIT, acc);
-                    cu_u += nwaves;
+                    cu_u += kw;
                     if (cu_u >= nug) {  // last unit of this tile for this wave: bank the partial sums
                         if (has_rows) {
-                            float *slot = part + ((size_t)cu_t * nwaves + wave) * slot_floats + g * 64 + nrow;
+                            float *slot = part + ((size_t)cu_t * kw + kl) * slot_floats + g * 64 + nrow;
 #pragma unroll
                             for (int r = 0; r < 4; r++) {
                                 if (r < NREG) slot[r * 16] += acc[r];
                                 acc[r] = 0.f;
                             }
                         }
-                        cu_t++;
-                        cu_u = wave;
+                        cu_t += tw;
+                        cu_u = kl;
                     }
                 }
             }
@@ -545,8 +551,8 @@ __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
         const int col = idx & 15, mr = (idx >> 4) % a.m, t = idx / (16 * a.m);
         auto tile_sum = [&](int vt) {
             float sum = 0.f;
-            for (int wv = 0; wv < nwaves; wv++) {
-                const float *slot = part + ((size_t)vt * nwaves + wv) * slot_floats + col;
+            for (int wv = 0; wv < kw; wv++) {
+                const float *slot = part + ((size_t)vt * kw + wv) * slot_floats + col;
                 sum += slot[mr * 16];
                 if (a.x_dtype == X_F32) sum += slot[(a.m + mr) * 16] * (1.0f / LO_SCALE);
             }

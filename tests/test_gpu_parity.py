@@ -182,6 +182,16 @@ def test_decode_q4_0_unit_pairing(oracle, units):
     check_matmul(oracle, Q4_0, 40, 128 * units, 2, seed=units)
 
 
+@pytest.mark.parametrize("scheme,m,x_dtype", [(Q4_0, 16, DType.BF16), (Q4_0, 5, DType.F32), (Q4K, 9, DType.BF16), (Q8_0, 12, DType.F16)])
+def test_decode_many_rows_wide_matrix(oracle, scheme, m, x_dtype):
+    # five or more activation rows over a matrix with thousands of row tiles: two waves per tile, eight tiles side by
+    # side per workgroup, K in LDS chunks; checked on a band of output columns at each end and in the middle
+    n, k = 28672, 2048
+    got, x, packed, _ = check_matmul(oracle, scheme, n, k, m, x_dtype=x_dtype, seed=m, cols=(0, 64))
+    for n0, n1 in ((14320, 14400), (28608, 28672)):
+        assert rel_err(got[:, n0:n1], oracle.gguf_matmul_f64(x, packed, m, k, n, scheme, n0, n1)) <= TOL
+
+
 def test_rows_just_past_the_decode_limit(oracle):
     check_matmul(oracle, Q4_0, 128, 256, 20, seed=4)           # f32: more than 8 rows -> prefill kernel
     check_matmul(oracle, Q4K, 64, 512, 37, x_dtype=DType.BF16, seed=5)  # more than 16 rows -> prefill kernel

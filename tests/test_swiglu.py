@@ -45,7 +45,7 @@ def bf16_bits(x):
 @pytest.mark.parametrize("scheme,m,n,k,dtype", [(Q4_0, 1, 14336, 4096, DType.F32), (Q4_0, 4, 200, 1024, DType.F32),
                                                  (Q8_0, 1, 1000, 512, DType.F32), (Q4K, 2, 530, 2048, DType.F32),
                                                  (Q4K, 16, 96, 1024, DType.BF16), (Q6K, 1, 160, 768, DType.F32),
-                                                 (Q4_0, 1, 48, 28672, DType.F32)])
+                                                 (Q4_0, 1, 48, 28672, DType.F32), (Q4_0, 8, 28672, 1024, DType.BF16)])
 def test_fused_swiglu_matches_two_matmuls_and_oracle(scheme, m, n, k, dtype):
     if scheme == Q6K:
         up_b, gate_b = (random_blocks(scheme, n, k, seed=s, d_std=5e-6) for s in (1, 2))
