@@ -369,12 +369,14 @@ extern "C" __global__ void rlx_argmax_finish(unsigned long long *key, uint32_t *
     }
 }
 
-// One workgroup = a contiguous run of row tiles of one weight segment x all of K.
+// One workgroup = a set of row tiles of one weight segment x all of K.
 //   * the activations are converted into LDS once per workgroup (per K chunk when they do not fit);
-//   * wave w walks the (tile, unit) items with unit = w, w + nwaves, ... of every tile in the run, keeping DEPTH
-//     units of weights in flight in registers, so the stream of 16-byte loads never drains between tiles;
+//   * the waves form nwaves / kw teams of kw waves; team t takes tiles t, t + teams, ... of the workgroup and its
+//     wave j walks the (tile, item) pairs with item = j, j + kw, ... of each (an item is UPI K units), keeping DEPTH
+//     items of weights in flight in registers, so the stream of 16-byte loads never drains between tiles. Decode
+//     (up to four activation rows) runs with kw = nwaves: every wave on the same tile;
 //   * at the end of each (tile, chunk) the wave adds its partial sums into its own LDS slot; one barrier at the
-//     very end, then the slots of all waves are added in a fixed order and written out (deterministic).
+//     very end, then the kw slots of a tile are added in a fixed order and written out (deterministic).
 // A launch can carry up to GEMV_MAX_SEG independent matmuls (each with its own activations, K and N): q/k/v and
 // gate/up of a layer, or every projection whose inputs are ready at the same point of the schedule.
 // MODE picks the epilogue at compile time, so the plain kernel carries none of the others' code: GEMV_PLAIN writes
