@@ -406,6 +406,19 @@ def extra_configs(rlx_amd, stream):
                                              "us_plain_gemv_writing_logits_back_to_back": round(ms_l * 1e3, 2),
                                              "us_plain_gemv_plus_one_small_kernel": round(ms_s * 1e3, 2),
                                              "launches": "gemv (argmax epilogue) + finish"}
+    for cap in (8, 40):
+        need = L.rlx_mi355x_tied_lm_topk_scratch_bytes(n, cap)
+        scratch, top = ops.DeviceBuffer(need), ops.DeviceBuffer(8 * cap)
+
+        def fn_topk():
+            q = qws[state["i"] % copies]
+            state["i"] += 1
+            rlx_amd._lib.check(L.rlx_mi355x_gguf_tied_lm_topk(x.ptr, int(DType.F32), q.ptr, cap, top.ptr, top.ptr + 4 * cap, scratch.ptr,
+                                                             need, stream))
+
+        ms_t = time_launches(ops, stream, fn_topk, 100, 10)
+        out[f"q4_k_tied_lm_top{cap}_128256x4096"] = {"us": round(ms_t * 1e3, 2), "GB/s": round(b / ms_t / 1e6, 1),
+                                                    "launches": "gemv (logits into scratch) + three selection passes, one wave per 1024 candidates"}
     for q in qws:
         q.free()
     # config 4: FakeQuantize [8192, 4096], int8 per column, heavy-tailed input; three input / output sets in rotation

@@ -192,6 +192,16 @@ int rlx_mi355x_rmsnorm_gguf_tied_lm_argmax(const float *hidden_dev, const float 
  * kernel writes *out_idx_dev / *out_val_dev. Calls that share a scratch must be ordered on one stream. */
 int rlx_mi355x_gguf_tied_lm_argmax(const void *hidden_dev, int x_dtype, const rlx_qweight *embed, uint32_t *out_idx_dev,
                                    float *out_val_dev, void *key_scratch_dev, void *stream);
+/* rlx_cpu::lm_head::gguf_tied_lm_topk (rlx-cpu/src/lm_head.rs:172-198, topk_from_scores :130-141): the `cap` rows with the
+ * largest dot products against one hidden vector as (row, value) pairs, largest first; cap is clamped to [1, n_vocab] as
+ * there. Among equal values the smaller row comes first (the reference's order among ties is whatever its unstable
+ * selection leaves); a NaN dot product is never listed, and where fewer than cap rows hold a number the tail is
+ * (0, -inf). The decode kernel writes the logits into the scratch; then one wave per 1024 candidates keeps its `cap`
+ * best, pass after pass (three for a 128k vocabulary), until a single wave writes the answer. cap <= 64, else
+ * RLX_ERR_UNSUPPORTED. The scratch (8-byte aligned, ..._scratch_bytes(n_vocab, cap) bytes) needs no initialisation. */
+size_t rlx_mi355x_tied_lm_topk_scratch_bytes(int64_t n_vocab, int cap);
+int rlx_mi355x_gguf_tied_lm_topk(const void *hidden_dev, int x_dtype, const rlx_qweight *embed, int cap, uint32_t *out_idx_dev,
+                                 float *out_val_dev, void *scratch_dev, size_t scratch_bytes, void *stream);
 int rlx_mi355x_gguf_matmul_bt_batch(const void *const *xs_dev, int x_dtype, const rlx_qweight *const *ws,
                                     float *const *outs_dev, int count, int64_t m, void *workspace, size_t workspace_bytes,
                                     void *stream);

@@ -57,6 +57,8 @@ def lib():
         L.orc_fused_swiglu.argtypes = [f32p, f32p, C.c_int64, C.c_int64, C.c_int]
         L.orc_gguf_tied_lm_argmax.restype = C.c_int
         L.orc_gguf_tied_lm_argmax.argtypes = [f32p, u8p, C.c_int64, C.c_int64, C.c_int64, C.c_int, u32p, f32p]
+        L.orc_gguf_tied_lm_topk.restype = C.c_int
+        L.orc_gguf_tied_lm_topk.argtypes = [f32p, u8p, C.c_int64, C.c_int64, C.c_int64, C.c_int, C.c_int, u32p, f32p]
         L.orc_gguf_grouped_matmul_bt.restype = C.c_int
         L.orc_gguf_grouped_matmul_bt.argtypes = [f32p, u8p, C.c_int64, f32p, f32p, C.c_int64, C.c_int64, C.c_int64, C.c_int64, C.c_int]
         L.orc_gguf_matmul_bt.restype = C.c_int
@@ -185,6 +187,20 @@ def gguf_tied_lm_argmax(hidden, packed, n_embd, n_vocab, scheme):
     if rc != 0:
         raise ValueError("gguf_tied_lm_argmax: bad sizes")
     return idx.value, val.value
+
+
+def gguf_tied_lm_topk(hidden, packed, n_embd, n_vocab, scheme, cap):
+    """rlx-cpu/src/lm_head.rs:172-198 -> (rows uint32[c], values float32[c]), largest first, ties by smaller row."""
+    hidden = np.ascontiguousarray(hidden, dtype=np.float32).reshape(-1)
+    packed = np.ascontiguousarray(packed, dtype=np.uint8)
+    assert hidden.size == n_embd
+    c = max(1, min(int(cap), int(n_vocab)))
+    idx, val = np.zeros(c, np.uint32), np.zeros(c, np.float32)
+    got = lib().orc_gguf_tied_lm_topk(_p(hidden, C.c_float), _p(packed, C.c_uint8), packed.size, n_embd, n_vocab, scheme, c,
+                                      _p(idx, C.c_uint32), _p(val, C.c_float))
+    if got < 0:
+        raise ValueError("gguf_tied_lm_topk: bad sizes")
+    return idx[:got], val[:got]
 
 
 def gguf_grouped_matmul_bt(x, packed, expert_idx, m, k, n, num_experts, scheme):

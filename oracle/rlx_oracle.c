@@ -503,6 +503,37 @@ int orc_gguf_tied_lm_argmax(const float *hidden, const uint8_t *w_bytes, int64_t
     return 0;
 }
 
+/* rlx-cpu/src/lm_head.rs:172-198 with topk_from_scores (:130-141): the cap largest (row, dot) pairs, largest first, cap
+ * clamped to [1, n_vocab]. The reference's early exit (row_dot_gguf_early_exit, :79-128) only drops rows whose bound
+ * says they cannot reach the current floor, so the answer is the top of the full score list; its order among equal
+ * scores is whatever select_nth_unstable leaves, here the smaller row comes first. NaN scores are left out (the
+ * reference's partial_cmp treats them as equal to anything). Returns the number of pairs written, or -1. */
+int orc_gguf_tied_lm_topk(const float *hidden, const uint8_t *w_bytes, int64_t w_nbytes, int64_t n_embd, int64_t n_vocab,
+                          int scheme, int cap, uint32_t *out_idx, float *out_val) {
+    int be = orc_block_elems(scheme), bb = orc_block_bytes(scheme);
+    if (be == 0 || (n_embd * n_vocab) % be != 0 || w_nbytes != (n_embd * n_vocab) / be * bb) return -1;
+    if (cap > n_vocab) cap = (int)n_vocab;
+    if (cap < 1) cap = 1;
+    int have = 0;
+    for (int64_t j = 0; j < n_vocab; j++) {
+        float dot = row_dot_gguf(hidden, w_bytes, j, n_embd, scheme);
+        if (dot != dot) continue;
+        /* insertion into the sorted list: after every entry with a value >= dot (earlier rows win ties) */
+        int pos = have;
+        while (pos > 0 && out_val[pos - 1] < dot) pos--;
+        if (pos >= cap) continue;
+        int last = have < cap ? have : cap - 1;
+        for (int i = last; i > pos; i--) {
+            out_val[i] = out_val[i - 1];
+            out_idx[i] = out_idx[i - 1];
+        }
+        out_val[pos] = dot;
+        out_idx[pos] = (uint32_t)j;
+        if (have < cap) have++;
+    }
+    return have;
+}
+
 /* ---- matmul ------------------------------------------------------------ */
 
 /* rlx-cpu/src/gguf_matmul.rs:40-95, loop for loop: out zeroed, then for each block in

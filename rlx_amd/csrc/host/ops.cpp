@@ -598,6 +598,78 @@ int rlx_mi355x_gguf_tied_lm_argmax(const void *hidden_dev, int x_dtype, const rl
     return launch(K_ARGMAX_FINISH, 1, 1, 64, 0, (hipStream_t)stream, params);
 }
 
+namespace rlx {
+struct TopkArgs {  // mirrors kernels/topk.hip
+    const float *vals;
+    const unsigned long long *keys_in;
+    int n, cap;
+    unsigned long long *keys_out;
+    uint32_t *out_idx;
+    float *out_val;
+};
+constexpr int64_t TOPK_GROUP = 1024;  // candidates one wave reduces to `cap`
+constexpr int TOPK_MAX_CAP = 64;
+static int64_t topk_groups(int64_t n) { return (n + TOPK_GROUP - 1) / TOPK_GROUP; }
+}  // namespace rlx
+
+size_t rlx_mi355x_tied_lm_topk_scratch_bytes(int64_t n_vocab, int cap) {
+    using namespace rlx;
+    if (n_vocab <= 0 || cap <= 0) return 0;
+    const int64_t c = std::min<int64_t>(std::min<int64_t>(cap, TOPK_MAX_CAP), n_vocab);
+    // the logits, then two key areas the passes alternate between (the first pass writes the largest)
+    const int64_t keys = topk_groups(n_vocab) * c;
+    return (size_t)((n_vocab * 4 + 7) / 8 * 8 + 2 * keys * 8);
+}
+
+int rlx_mi355x_gguf_tied_lm_topk(const void *hidden_dev, int x_dtype, const rlx_qweight *embed, int cap, uint32_t *out_idx_dev,
+                                 float *out_val_dev, void *scratch_dev, size_t scratch_bytes, void *stream) {
+    using namespace rlx;
+    if (!hidden_dev || !embed || !out_idx_dev || !out_val_dev || !scratch_dev) {
+        set_error("gguf_tied_lm_topk: null argument");
+        return RLX_ERR_INVALID;
+    }
+    const int xk = x_kind(x_dtype);
+    if (xk < 0) {
+        set_error("gguf_tied_lm_topk: hidden dtype %d is not F32 / BF16 / F16", x_dtype);
+        return RLX_ERR_UNSUPPORTED;
+    }
+    const int64_t n = embed->dims.n;
+    if (cap < 1) cap = 1;  // the reference's cap.min(n_vocab).max(1)
+    if (cap > n) cap = (int)n;
+    if (cap > TOPK_MAX_CAP) {
+        set_error("gguf_tied_lm_topk: cap %d is beyond the selection kernel (cap <= %d)", cap, TOPK_MAX_CAP);
+        return RLX_ERR_UNSUPPORTED;
+    }
+    if ((uintptr_t)scratch_dev % 8 != 0 || scratch_bytes < rlx_mi355x_tied_lm_topk_scratch_bytes(n, cap)) {
+        set_error("gguf_tied_lm_topk: scratch of %zu bytes (8-byte aligned) needed, got %zu", rlx_mi355x_tied_lm_topk_scratch_bytes(n, cap),
+                  scratch_bytes);
+        return RLX_ERR_INVALID;
+    }
+    float *logits = (float *)scratch_dev;
+    unsigned long long *keys[2];
+    keys[0] = (unsigned long long *)((uint8_t *)scratch_dev + (n * 4 + 7) / 8 * 8);
+    keys[1] = keys[0] + topk_groups(n) * cap;
+    const void *xs[1] = {hidden_dev};
+    const rlx_qweight *ws[1] = {embed};
+    float *outs[1] = {logits};
+    RLX_TRY(launch_gemv(xs, xk, ws, outs, 1, 1, (hipStream_t)stream));
+    // every pass: one wave per 1024 candidates keeps its cap best; the pass with a single wave writes the answer
+    int64_t count = n;
+    int side = 0;
+    for (bool first = true;; first = false) {
+        const int64_t groups = topk_groups(count);
+        const bool last = groups == 1;
+        TopkArgs p{first ? logits : nullptr, first ? nullptr : keys[side ^ 1], (int)count, cap, last ? nullptr : keys[side],
+                   last ? out_idx_dev : nullptr, last ? out_val_dev : nullptr};
+        void *params[] = {&p};
+        RLX_TRY(launch(K_TOPK_SELECT, (unsigned)groups, 1, 64, 0, (hipStream_t)stream, params));
+        if (last) break;
+        count = groups * cap;
+        side ^= 1;
+    }
+    return RLX_OK;
+}
+
 int rlx_mi355x_gguf_grouped_matmul_bt(const void *x_dev, int x_dtype, const rlx_qweight *w, const float *expert_idx_dev,
                                       float *out_dev, int64_t m, void *stream) {
     using namespace rlx;

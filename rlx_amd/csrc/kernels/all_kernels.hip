@@ -3,3 +3,4 @@
 #include "fakequant.hip"
 #include "gemm.hip"
 #include "gemv.hip"
+#include "topk.hip"

@@ -252,6 +252,20 @@ def gguf_tied_lm_argmax(hidden, embed: QWeight, x_dtype=DType.F32):
     return int(raw[0]), float(raw[1:2].view(np.float32)[0])
 
 
+def gguf_tied_lm_topk(hidden, embed: QWeight, cap, x_dtype=DType.F32):
+    """Host convenience for rlx_cpu::lm_head::gguf_tied_lm_topk (rlx-cpu/src/lm_head.rs:172-198): (rows uint32[c],
+    values float32[c]) of the c = clamp(cap, 1, n_vocab) largest logits of hidden . embed^T, largest first."""
+    c = max(1, min(int(cap), embed.n))
+    hd = DeviceBuffer.from_numpy(hidden)
+    need = _lib.lib().rlx_mi355x_tied_lm_topk_scratch_bytes(embed.n, c)
+    scratch, res = DeviceBuffer(max(need, 8)), DeviceBuffer(8 * c)
+    _lib.check(_lib.lib().rlx_mi355x_gguf_tied_lm_topk(hd.ptr, int(x_dtype), embed.ptr, int(cap), res.ptr, res.ptr + 4 * c, scratch.ptr,
+                                                      scratch.nbytes, None))
+    sync()
+    raw = res.to_numpy(np.uint32, 2 * c)
+    return raw[:c].copy(), raw[c:].view(np.float32).copy()
+
+
 def fake_quantize(x, shape, axis, bits, scale_mode=ScaleMode.PerBatch, decay=0.0, state=None,
                   round_mode=RoundMode.HalfAway):
     """Host convenience around rlx_mi355x_fake_quantize. Returns (out f32, codes i8, scales f32); EMA updates `state`."""
