@@ -378,8 +378,7 @@ def extra_configs(rlx_amd, stream):
     qws = [ops.QWeight(QuantScheme.GgufQ4K, np.roll(packed, 7 * i, axis=0).reshape(-1), n, k) for i in range(copies)]
     del packed, slab, w
     x = ops.DeviceBuffer.from_numpy(ops.philox_normal(8, k))
-    res = ops.DeviceBuffer(16)
-    rlx_amd._lib.check(L.rlx_mi355x_memset_u32(res.ptr, 0, 4, stream))  # the key scratch starts zero; every call leaves it zero
+    res = ops.DeviceBuffer(8 + L.rlx_mi355x_tied_lm_argmax_scratch_bytes())  # row, value, then the per-workgroup key scratch
     y = ops.DeviceBuffer(n * 4)
     state = {"i": 0}
 

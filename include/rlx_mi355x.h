@@ -186,10 +186,11 @@ int rlx_mi355x_rmsnorm_gguf_tied_lm_argmax(const float *hidden_dev, const float 
                                            void *key_scratch_dev, void *stream);
 /* rlx_cpu::lm_head::gguf_tied_lm_argmax (rlx-cpu/src/lm_head.rs:223-248): the row of the packed [n_vocab, n_embd] matrix
  * with the largest dot product against one hidden vector, and that dot product. The first maximum wins, a NaN never
- * does, and (0, -inf) comes back when no row beats -inf, as in the reference's loop. The logits are never written: the
- * decode kernel's workgroups merge (value, row) keys with a 64-bit atomic max into `key_scratch_dev` (8 bytes, 8-byte
- * aligned, ZERO before the first call, e.g. rlx_mi355x_memset_u32; every call leaves it zero again), and a one-thread
- * kernel writes *out_idx_dev / *out_val_dev. Calls that share a scratch must be ordered on one stream. */
+ * does, and (0, -inf) comes back when no row beats -inf, as in the reference's loop. The logits are never written: every
+ * workgroup of the decode kernel stores one (value, row) key into `key_scratch_dev` (8-byte aligned,
+ * rlx_mi355x_tied_lm_argmax_scratch_bytes() bytes, no initialisation needed) and a one-workgroup kernel takes their
+ * maximum and writes *out_idx_dev / *out_val_dev. Calls that share a scratch must be ordered on one stream. */
+size_t rlx_mi355x_tied_lm_argmax_scratch_bytes(void);
 int rlx_mi355x_gguf_tied_lm_argmax(const void *hidden_dev, int x_dtype, const rlx_qweight *embed, uint32_t *out_idx_dev,
                                    float *out_val_dev, void *key_scratch_dev, void *stream);
 /* rlx_cpu::lm_head::gguf_tied_lm_topk (rlx-cpu/src/lm_head.rs:172-198, topk_from_scores :130-141): the `cap` rows with the

@@ -91,9 +91,11 @@ static int x_kind(int x_dtype) {
 
 // One decode launch over `count` (<= GEMV_MAX_SEG) matmuls of one scheme, batch and activation dtype; each has
 // its own activations, K and N.
+constexpr int ARGMAX_MAX_WGS = 4096;  // keys in the tied-LM-head scratch: one per workgroup of the decode launch
+
 static int launch_gemv(const void *const *xs, int xk, const rlx_qweight *const *ws, float *const *outs, int count, int m,
                        hipStream_t stream, const float *expert_idx = nullptr, unsigned long long *argmax_key = nullptr,
-                       const rlx_qweight *const *pairs = nullptr, const RmsNorm *norm = nullptr) {
+                       const rlx_qweight *const *pairs = nullptr, const RmsNorm *norm = nullptr, int *wgs_out = nullptr) {
     const int scheme = ws[0]->scheme;
     const Layout L = ws[0]->layout;
     const bool wide = layout_is_f16w(L);
@@ -230,6 +232,11 @@ static int launch_gemv(const void *const *xs, int xk, const rlx_qweight *const *
         for (int i = 0; i < count; i++) even = even && ws[i]->dims.units % 2 == 0;
         if (even) id = (KernelId)(K_GEMV_Q4_0_U2_R2 + variant);
     }
+    if (argmax_key && sh.wg > ARGMAX_MAX_WGS) {
+        set_error("gemv: %d workgroups are more than the argmax key scratch holds (%d)", sh.wg, ARGMAX_MAX_WGS);
+        return RLX_ERR_UNSUPPORTED;
+    }
+    if (wgs_out) *wgs_out = sh.wg;
     void *params[] = {&sh.a};
     return launch(id, (unsigned)sh.wg, 1, (unsigned)sh.nwaves * 64, (unsigned)sh.lds, stream, params);
 }
@@ -539,9 +546,10 @@ int rlx_mi355x_rmsnorm_gguf_tied_lm_argmax(const float *hidden_dev, const float 
     const void *xs[1] = {hidden_dev};
     const rlx_qweight *ws[1] = {embed};
     float *outs[1] = {nullptr};
-    RLX_TRY(launch_gemv(xs, 0, ws, outs, 1, 1, (hipStream_t)stream, nullptr, (unsigned long long *)key_scratch_dev, nullptr, &norm));
-    void *params[] = {&key_scratch_dev, &out_idx_dev, &out_val_dev};
-    return launch(K_ARGMAX_FINISH, 1, 1, 64, 0, (hipStream_t)stream, params);
+    int wgs = 0;
+    RLX_TRY(launch_gemv(xs, 0, ws, outs, 1, 1, (hipStream_t)stream, nullptr, (unsigned long long *)key_scratch_dev, nullptr, &norm, &wgs));
+    void *params[] = {&key_scratch_dev, &wgs, &out_idx_dev, &out_val_dev};
+    return launch(K_ARGMAX_FINISH, 1, 1, 256, 0, (hipStream_t)stream, params);
 }
 
 int rlx_mi355x_gguf_matmul_swiglu(const void *x_dev, int x_dtype, const rlx_qweight *w_up, const rlx_qweight *w_gate,
@@ -587,15 +595,16 @@ int rlx_mi355x_gguf_tied_lm_argmax(const void *hidden_dev, int x_dtype, const rl
         return RLX_ERR_UNSUPPORTED;
     }
     if ((uintptr_t)key_scratch_dev % 8 != 0) {
-        set_error("gguf_tied_lm_argmax: the 8-byte key scratch must be 8-byte aligned");
+        set_error("gguf_tied_lm_argmax: the key scratch must be 8-byte aligned");
         return RLX_ERR_INVALID;
     }
     const void *xs[1] = {hidden_dev};
     const rlx_qweight *ws[1] = {embed};
     float *outs[1] = {nullptr};
-    RLX_TRY(launch_gemv(xs, xk, ws, outs, 1, 1, (hipStream_t)stream, nullptr, (unsigned long long *)key_scratch_dev));
-    void *params[] = {&key_scratch_dev, &out_idx_dev, &out_val_dev};
-    return launch(K_ARGMAX_FINISH, 1, 1, 64, 0, (hipStream_t)stream, params);
+    int wgs = 0;
+    RLX_TRY(launch_gemv(xs, xk, ws, outs, 1, 1, (hipStream_t)stream, nullptr, (unsigned long long *)key_scratch_dev, nullptr, nullptr, &wgs));
+    void *params[] = {&key_scratch_dev, &wgs, &out_idx_dev, &out_val_dev};
+    return launch(K_ARGMAX_FINISH, 1, 1, 256, 0, (hipStream_t)stream, params);
 }
 
 namespace rlx {
@@ -611,6 +620,8 @@ constexpr int64_t TOPK_GROUP = 1024;  // candidates one wave reduces to `cap`
 constexpr int TOPK_MAX_CAP = 64;
 static int64_t topk_groups(int64_t n) { return (n + TOPK_GROUP - 1) / TOPK_GROUP; }
 }  // namespace rlx
+
+size_t rlx_mi355x_tied_lm_argmax_scratch_bytes(void) { return (size_t)rlx::ARGMAX_MAX_WGS * 8; }
 
 size_t rlx_mi355x_tied_lm_topk_scratch_bytes(int64_t n_vocab, int cap) {
     using namespace rlx;

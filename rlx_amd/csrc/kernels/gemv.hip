@@ -49,7 +49,7 @@ struct GemvArgs {
     int num_experts;
     // Tied LM head (rlx-cpu/src/lm_head.rs:223-248): when set (m = 1, one segment), nothing is written to `out`; every
     // workgroup folds its outputs into one 64-bit key (ordered value bits, then ~row so that the first maximum wins) and
-    // merges it with an atomic max.
+    // stores it at argmax_key[workgroup].
     unsigned long long *argmax_key;
     // RMSNorm prologue (rlx-cpu/src/thunk.rs:8839-8869) in the kernels built with GEMV_NORM: the f32 activations are
     // x * (1 / sqrt(mean(x^2) + eps)) * gamma + beta (beta may be null) before they are split into halfs.
@@ -350,12 +350,19 @@ __device__ __forceinline__ unsigned long long argmax_key_of(float v, uint32_t ro
     return ((unsigned long long)ordered << 32) | (uint32_t)~row;
 }
 
-// Decodes the merged key into {row, value}; an untouched key (every dot NaN or -inf lost to the start value) gives
-// row 0 and -inf, the reference's starting pair. Leaves the key zero for the next call.
-extern "C" __global__ void rlx_argmax_finish(unsigned long long *key, uint32_t *out_idx, float *out_val) {
-    if (threadIdx.x != 0 || blockIdx.x != 0) return;
-    const unsigned long long k = *key;
-    *key = 0;
+// Maximum over the `count` workgroup keys, decoded into {row, value}; when no key was set (every dot NaN, or -inf that
+// lost to the start value) row 0 and -inf, the reference's starting pair.
+extern "C" __global__ __launch_bounds__(256) void rlx_argmax_finish(const unsigned long long *keys, int count, uint32_t *out_idx,
+                                                                    float *out_val) {
+    __shared__ unsigned long long wave_best[4];
+    unsigned long long k = 0;
+    for (int i = threadIdx.x; i < count; i += 256) k = max(k, keys[i]);
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) k = max(k, (unsigned long long)__shfl_xor(k, off));
+    if ((threadIdx.x & 63) == 0) wave_best[threadIdx.x >> 6] = k;
+    __syncthreads();
+    if (threadIdx.x != 0) return;
+    for (int w = 1; w < 4; w++) k = max(k, wave_best[w]);
     const uint32_t ordered = (uint32_t)(k >> 32);
     const uint32_t b = (ordered & 0x80000000u) ? (ordered & 0x7FFFFFFFu) : ~ordered;
     const float v = __builtin_bit_cast(float, b);
@@ -582,10 +589,17 @@ __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
             const unsigned long long other = __shfl_xor(best, off);
             best = max(best, other);
         }
-        // Atomics on one address are served one after another (~35 ns each): look first, and only workgroups that can
-        // still raise the key queue up for it.
-        if (l == 0 && best != 0 && best > __hip_atomic_load(a.argmax_key, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
-            atomicMax(a.argmax_key, best);
+        // One key per workgroup, stored plainly: the waves meet in LDS (the partial sums are spent), the finishing
+        // kernel takes the maximum over the workgroups. (Merging with atomics on one word costs ~35 ns per workgroup,
+        // served one after another, and they all arrive at the end of the launch.)
+        __syncthreads();
+        unsigned long long *wave_best = (unsigned long long *)smem;
+        if (l == 0) wave_best[wave] = best;
+        __syncthreads();
+        if (tid == 0) {
+            for (int wv = 1; wv < nwaves; wv++) best = max(best, wave_best[wv]);
+            a.argmax_key[blockIdx.x] = best;
+        }
     }
 }
 

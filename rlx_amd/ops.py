@@ -231,8 +231,7 @@ def rmsnorm_gguf_matmul_swiglu(x, gamma, beta, eps, w_up: QWeight, w_gate: QWeig
 def rmsnorm_gguf_tied_lm_argmax(hidden, gamma, beta, eps, embed: QWeight):
     hd = DeviceBuffer.from_numpy(np.ascontiguousarray(hidden, dtype=np.float32))
     g, b = _norm_bufs(gamma, beta)
-    res = DeviceBuffer(16)
-    _lib.check(_lib.lib().rlx_mi355x_memset_u32(res.ptr, 0, 4, None))
+    res = DeviceBuffer(8 + _lib.lib().rlx_mi355x_tied_lm_argmax_scratch_bytes())  # [0:4) row, [4:8) value, then the key scratch
     _lib.check(_lib.lib().rlx_mi355x_rmsnorm_gguf_tied_lm_argmax(hd.ptr, g.ptr, b.ptr if b else None, eps, embed.ptr, res.ptr, res.ptr + 4,
                                                                 res.ptr + 8, None))
     sync()
@@ -244,8 +243,7 @@ def gguf_tied_lm_argmax(hidden, embed: QWeight, x_dtype=DType.F32):
     """Host convenience for the tied LM head (rlx-cpu/src/lm_head.rs:223-248): (row, value) of the largest logit of
     hidden . embed^T without materialising the logits."""
     hd = DeviceBuffer.from_numpy(hidden)
-    res = DeviceBuffer(16)  # [0:4) row, [4:8) value, [8:16) the key scratch (zero before the first call)
-    _lib.check(_lib.lib().rlx_mi355x_memset_u32(res.ptr, 0, 4, None))
+    res = DeviceBuffer(8 + _lib.lib().rlx_mi355x_tied_lm_argmax_scratch_bytes())  # [0:4) row, [4:8) value, then the key scratch
     _lib.check(_lib.lib().rlx_mi355x_gguf_tied_lm_argmax(hd.ptr, int(x_dtype), embed.ptr, res.ptr, res.ptr + 4, res.ptr + 8, None))
     sync()
     raw = res.to_numpy(np.uint32, 2)
