@@ -257,8 +257,10 @@ static GemmPlan gemm_plan(int scheme, int xk, int64_t m, int64_t k) {
 
 // Prefill path: convert the activations once (xprep), then the MFMA GEMM; K is split across workgroups (atomic
 // accumulation into a zeroed output) only when the tile grid alone would leave most CUs idle.
+// `prepared`: the workspace already holds this x (same pointer, k, m, dtype, and the block sums if this scheme needs
+// them) from the previous matrix of a batch on the same stream, so the conversion pass is skipped.
 static int launch_gemm(const void *x, int xk, const rlx_qweight *w, float *out, int64_t m, void *workspace,
-                       size_t workspace_bytes, hipStream_t stream) {
+                       size_t workspace_bytes, hipStream_t stream, bool prepared = false) {
     const Layout L = w->layout;
     const GemmPlan p = gemm_plan(w->scheme, xk, m, w->dims.k);
     if (!workspace || workspace_bytes < p.xh_bytes + p.sxh_bytes) {
@@ -275,7 +277,7 @@ static int launch_gemm(const void *x, int xk, const rlx_qweight *w, float *out, 
     XPrepArgs xa{x, xh, sxh, (int)m, (int)w->dims.k, (int)p.k_pad, (int)p.m_rows, xk};
     void *xparams[] = {&xa};
     const long long xblocks = (p.m_rows / 256) * (p.k_pad / 64) * 8;  // (tile, step, 32-row sub-tile)
-    RLX_TRY(launch(K_XPREP, (unsigned)xblocks, 1, 256, 0, stream, xparams));
+    if (!prepared) RLX_TRY(launch(K_XPREP, (unsigned)xblocks, 1, 256, 0, stream, xparams));
 
     const int steps_per_unit = L.unit_k / 64;
     // Up to 128 activation rows run the 64-row tile (the weights are decoded once per 64 rows, but nothing is spent on
@@ -438,8 +440,21 @@ int rlx_mi355x_gguf_matmul_bt_batch(const void *const *xs_dev, int x_dtype, cons
     const int64_t cap = xk == 0 ? 8 : 16;  // activation rows one decode pass holds
     const size_t esz = xk == 0 ? 4 : 2;
     if (m > cap) {  // prefill: one GEMM per weight, sharing the workspace (same stream, so launches are ordered)
-        for (int i = 0; i < count; i++)
-            RLX_TRY(launch_gemm(xs_dev[i], xk, ws[i], outs_dev[i], m, workspace, workspace_bytes, (hipStream_t)stream));
+        // q, k, v (and gate, up) of a layer share their input: its f16 image in the workspace is made once. An image
+        // with block sums (Q4_K / Q5_K) also serves a scheme that does not read them, not the other way round.
+        const void *have_x = nullptr;
+        int64_t have_k = -1;
+        bool have_sums = false;
+        for (int i = 0; i < count; i++) {
+            const bool sums = gemm_plan(ws[i]->scheme, xk, m, ws[i]->dims.k).sxh_bytes != 0;
+            const bool prepared = xs_dev[i] == have_x && ws[i]->dims.k == have_k && (have_sums || !sums);
+            RLX_TRY(launch_gemm(xs_dev[i], xk, ws[i], outs_dev[i], m, workspace, workspace_bytes, (hipStream_t)stream, prepared));
+            if (!prepared) {
+                have_x = xs_dev[i];
+                have_k = ws[i]->dims.k;
+                have_sums = sums;
+            }
+        }
         return RLX_OK;
     }
     for (int64_t r0 = 0; r0 < m; r0 += cap) {

@@ -180,6 +180,26 @@ def gguf_matmul_bt(x, w: QWeight, m, x_dtype=DType.F32):
     return od.to_numpy(np.float32).reshape(m, w.n)
 
 
+def gguf_matmul_bt_batch(xs, ws, m, x_dtype=DType.F32):
+    """Host convenience for rlx_mi355x_gguf_matmul_bt_batch: outs[i] = xs[i] . ws[i]^T, all of one scheme, m and dtype.
+    Entries of `xs` that are the same array object share one device buffer (q, k, v of a layer), which lets the
+    prefill path convert that input once."""
+    bufs = {}
+    for x in xs:
+        if id(x) not in bufs:
+            bufs[id(x)] = DeviceBuffer.from_numpy(x)
+    outs = [DeviceBuffer(m * w.n * 4) for w in ws]
+    need = max(matmul_workspace_bytes(w, x_dtype, m) for w in ws)
+    workspace = DeviceBuffer(need) if need else None
+    n = len(ws)
+    xp = (C.c_void_p * n)(*[bufs[id(x)].ptr for x in xs])
+    wp = (C.c_void_p * n)(*[w.ptr for w in ws])
+    op = (C.c_void_p * n)(*[o.ptr for o in outs])
+    _lib.check(_lib.lib().rlx_mi355x_gguf_matmul_bt_batch(xp, int(x_dtype), wp, op, n, m, workspace.ptr if workspace else None, need, None))
+    sync()
+    return [o.to_numpy(np.float32).reshape(m, w.n) for o, w in zip(outs, ws)]
+
+
 def gguf_grouped_matmul_bt(x, w: QWeight, expert_idx, x_dtype=DType.F32):
     """Host convenience for the MoE matmul: out[i] = x[i] . W[expert_idx[i]]^T; x is [m, k], expert_idx [m]."""
     idx = np.ascontiguousarray(expert_idx, dtype=np.float32)

@@ -397,6 +397,34 @@ def test_graph_batches_independent_matmuls(oracle):
 
 # ------------------------------------------------------------------ prefill GEMM (m > 16)
 
+@pytest.mark.parametrize("scheme,m,x_dtype", [(Q4K, 40, DType.BF16), (Q4_0, 300, DType.F32), (Q8_0, 130, DType.F16)])
+def test_batched_prefill_shares_the_converted_input(oracle, scheme, m, x_dtype):
+    # q / k / v on one input, then a matrix with its own input and another k, then the first input again: the input's
+    # f16 image is made once per run of matrices that share it, and every output is that of the matmul issued on its own
+    say("batched prefill", SCHEME_NAMES[scheme], "m", m, x_dtype.name)
+    rng = np.random.default_rng(m)
+    shapes = [(256, 1024, 0), (64, 1024, 0), (48, 1024, 0), (96, 512, 1), (80, 1024, 0)]
+    xs_f32 = [rng.standard_normal((m, 1024)).astype(np.float32), rng.standard_normal((m, 512)).astype(np.float32)]
+    if x_dtype == DType.BF16:
+        xs_in = [f32_to_bf16_bits(oracle.bf16_round(x)) for x in xs_f32]
+    elif x_dtype == DType.F16:
+        xs_in = [x.astype(np.float16) for x in xs_f32]
+    else:
+        xs_in = xs_f32
+    packs = [make_weights(scheme, n, k, seed=80 + i)[0] for i, (n, k, _) in enumerate(shapes)]
+    ws = [ops.QWeight(scheme, p, n, k) for p, (n, k, _) in zip(packs, shapes)]
+    got = ops.gguf_matmul_bt_batch([xs_in[which] for _, _, which in shapes], ws, m, x_dtype)
+    for i, (n, k, which) in enumerate(shapes):
+        alone = ops.gguf_matmul_bt(xs_in[which], ws[i], m, x_dtype)
+        # small tile grids split K and add the slices with atomics, so two runs may differ in the order of f32 additions
+        assert rel_err(got[i], alone) <= 1e-5, i
+        x_ref = oracle.bf16_round(xs_f32[which]) if x_dtype == DType.BF16 else \
+            xs_f32[which].astype(np.float16).astype(np.float32) if x_dtype == DType.F16 else xs_f32[which]
+        assert rel_err(got[i], oracle.gguf_matmul_f64(x_ref, packs[i], m, k, n, scheme)) <= TOL, i
+    for w in ws:
+        w.free()
+
+
 @pytest.mark.parametrize("scheme", [Q4K, Q4_0, Q8_0])
 @pytest.mark.parametrize("m,n,k,x_dtype", [(64, 256, 512, DType.BF16), (300, 200, 768, DType.BF16),
                                            (40, 128, 1024, DType.F32), (512, 384, 2048, DType.F16),
