@@ -560,7 +560,7 @@ def gemm_configs(rlx_amd, stream):
     weights = {name: tiled_weight(ops, QuantScheme.GgufQ4_0, n, k, 50 + i, 0.015) for i, (name, n, k) in enumerate(shapes70)}
     wbytes = sum(n * k // 32 * 18 for _, n, k in shapes70)
     sweep = {}
-    for m in (1, 4, 16, 64, 256):
+    for m in (1, 4, 16, 32, 64, 256):  # 32: the largest batch the decode kernels take
         # one timed repetition = the seven projections in turn, so the 481 MB of weights go round the 256 MB last-level
         # cache and every launch reads its matrix from HBM
         bufs = {}
@@ -586,7 +586,7 @@ def gemm_configs(rlx_amd, stream):
         algo = wbytes + sum(2 * m * k + 4 * m * n for _, n, k in shapes70)
         sweep[f"M={m}"] = {"us_layer": round(total_ms * 1e3, 1), "GB/s": round(algo / total_ms / 1e6, 1),
                            "TFLOP/s": round(flops / total_ms / 1e9, 2),
-                           "path": "gemv" if m <= 16 else "gemm"}
+                           "path": "gemv" if m <= 32 else "gemm"}
     out["q4_0_batch_sweep_llama70b_layer"] = sweep
     for q in weights.values():
         q.free()

@@ -141,8 +141,8 @@ int rlx_mi355x_dequant(const rlx_qweight *w, float *out_dev, void *stream);
  * x_dev is [m,k] row-major of x_dtype in {RLX_F32, RLX_BF16, RLX_F16}; 16-bit activations stand for the values
  * the reference's typed boundary would widen to f32 (rlx-runtime/src/backend.rs:49-53). out_dev is f32.
  * `workspace` must hold rlx_mi355x_gguf_matmul_workspace() bytes (may be NULL when that is 0).
- * m <= 8 (f32 activations) or m <= 16 (bf16 / f16) runs the decode kernel (weights streamed once, MFMA 16x16x32);
- * larger m runs the prefill GEMM. */
+ * m <= 16 (f32 activations) or m <= 32 (bf16 / f16) runs the decode kernels (weights streamed once, MFMA 16x16x32, one
+ * or two groups of 16 rows per decoded weight fragment, an f32 row taking two); larger m runs the prefill GEMM. */
 int rlx_mi355x_gguf_matmul_bt(const void *x_dev, int x_dtype, const rlx_qweight *w, float *out_dev, int64_t m,
                               void *workspace, size_t workspace_bytes, void *stream);
 size_t rlx_mi355x_gguf_matmul_workspace(int scheme, int x_dtype, int64_t m, int64_t k, int64_t n);

@@ -91,6 +91,10 @@ static int x_kind(int x_dtype) {
 
 // One decode launch over `count` (<= GEMV_MAX_SEG) matmuls of one scheme, batch and activation dtype; each has
 // its own activations, K and N.
+// Rows one launch of the decode kernels takes: two groups of 16 MFMA rows, an f32 row being a hi and a lo row. Above
+// that the prefill GEMM runs (measured on a 70B layer at 32 bf16 rows: 205 us against 317).
+static int64_t decode_rows(int xk) { return xk == 0 ? 16 : 32; }
+
 constexpr int ARGMAX_MAX_WGS = 4096;  // keys in the tied-LM-head scratch: one per workgroup of the decode launch
 
 static int launch_gemv(const void *const *xs, int xk, const rlx_qweight *const *ws, float *const *outs, int count, int m,
@@ -107,6 +111,12 @@ static int launch_gemv(const void *const *xs, int xk, const rlx_qweight *const *
     const int rv = xk == 0 ? 2 * m : m;
     const int ng = (rv + 3) / 4;
     const bool r2 = rv <= 2;
+    // groups of 16 activation rows per weight fragment: 1 (the decode kernels) or 2 (plain epilogue only)
+    const int rg = rv <= 16 ? 1 : 2;
+    if (rv > 32 || (rg > 1 && (argmax_key || pairs || norm || expert_idx))) {
+        set_error("gemv: %d activation rows are beyond this kernel", rv);
+        return RLX_ERR_UNSUPPORTED;
+    }
     // kernel = scheme family x {r2, r4, r2_argmax, r2_paired, r4_paired}
     const int family = wide ? K_GEMV_F16W_R2 : scheme == SCHEME_Q4_0 ? K_GEMV_Q4_0_R2 : scheme == SCHEME_Q8_0 ? K_GEMV_Q8_0_R2
                        : scheme == SCHEME_Q6K ? K_GEMV_Q6_K_R2 : scheme == SCHEME_Q5K ? K_GEMV_Q5_K_R2 : K_GEMV_Q4_K_R2;
@@ -120,6 +130,7 @@ static int launch_gemv(const void *const *xs, int xk, const rlx_qweight *const *
     }
     const int variant = argmax_key ? (norm ? 9 : 2) : pairs ? (norm ? (r2 ? 7 : 8) : (r2 ? 3 : 4)) : (norm ? (r2 ? 5 : 6) : (r2 ? 0 : 1));
     KernelId id = (KernelId)(family + variant);
+    if (rg > 1) id = (KernelId)(K_GEMV_Q4_0_G2 + (family - K_GEMV_Q4_0_R2) / 10);
     static const int env_waves = getenv("RLX_GEMV_WAVES") ? atoi(getenv("RLX_GEMV_WAVES")) : 8;
     static const int env_wgs_per_cu = getenv("RLX_GEMV_WGS_PER_CU") ? atoi(getenv("RLX_GEMV_WGS_PER_CU")) : 2;
     int max_units = 0;
@@ -132,7 +143,7 @@ static int launch_gemv(const void *const *xs, int xk, const rlx_qweight *const *
     const size_t slot_bytes = (size_t)ng * 256;
     auto stage_bytes = [&](int kcu) {
         size_t b = ((size_t)rv * ((size_t)kcu * L.unit_k + 8) * 2 + 15) & ~(size_t)15;
-        if (scheme == SCHEME_Q4K || (scheme == SCHEME_Q5K && !wide)) b += (size_t)kcu * (L.unit_k / 32) * 16 * 4;  // block sums
+        if (scheme == SCHEME_Q4K || (scheme == SCHEME_Q5K && !wide)) b += (size_t)kcu * (L.unit_k / 32) * 16 * rg * 4;  // block sums
         return b;
     };
     // A launch shape: `wgs_per_cu` workgroups of `waves` waves per CU, every one resident at once, each with the same
@@ -152,7 +163,9 @@ static int launch_gemv(const void *const *xs, int xk, const rlx_qweight *const *
         const int kw = (kw_req > 0 && kw_req < sh.nwaves && sh.nwaves % kw_req == 0) ? kw_req : sh.nwaves;
         const int tw = sh.nwaves / kw;
         const long long slots = (long long)std::max(1, wgs_per_cu) * cus;
-        const int tpw_cap = (int)std::max<size_t>(1, (tw > 1 ? budget / 2 : budget * 2 / 5) / (kw * slot_bytes));
+        // share of the LDS for the partial sums; the rest stages activations
+        const size_t part_budget = tw > 1 ? budget / 2 : budget * 2 / 5;
+        const int tpw_cap = (int)std::max<size_t>(1, part_budget / (kw * slot_bytes));
         int max_tpw = 1;
         // With tw > 1 a workgroup's tile count is rounded up to whole rounds of tw tiles; the per-workgroup target then
         // grows until one round of workgroups covers the launch (a few stragglers in a second round would double it).
@@ -204,8 +217,11 @@ static int launch_gemv(const void *const *xs, int xk, const rlx_qweight *const *
     if (rv >= 4 && !getenv("RLX_GEMV_WGS_PER_CU")) {
         // From five rows on, the per-(tile, wave) partial-sum slots (256 B per four rows) are what limits the tiles of
         // a workgroup: two waves per tile instead of sixteen, eight tiles side by side, keeps the slot area small
-        // enough that one workgroup per CU covers the launch and the activations are staged once per CU.
+        // enough that one workgroup per CU covers the launch and the activations are staged once per CU. The kernels
+        // for more than 16 rows run eight waves per workgroup (their register budget), one wave per tile when the
+        // launch has the tiles for it.
         static const int env_kw = getenv("RLX_GEMV_KW") ? atoi(getenv("RLX_GEMV_KW")) : -1;
+        const int fat_waves = rg > 1 ? 8 : 16;
         int kw = 0;
         if (rv >= 5) {  // as many tiles side by side (at most eight) as the segment with the fewest tiles per workgroup has
             double min_tpw = 1e30;
@@ -213,12 +229,13 @@ static int launch_gemv(const void *const *xs, int xk, const rlx_qweight *const *
                 min_tpw = std::min(min_tpw, (double)work / cus / (double)(ws[i]->dims.units * (pairs ? 2 : 1)));
             int tw = 8;
             while (tw > 1 && tw > min_tpw * 1.2) tw /= 2;
-            kw = tw > 1 ? 16 / tw : 0;
+            kw = tw > 1 ? fat_waves / tw : 0;
         }
         if (env_kw >= 0) kw = env_kw;
-        Shape fat = shape(16, 1, (size_t)156 * 1024, kw);
-        if (kw && !(fat.fits && fat.wg <= cus)) fat = shape(16, 1, (size_t)156 * 1024, 0);
-        if (fat.fits && fat.wg <= cus) sh = fat;
+        Shape fat = shape(fat_waves, 1, (size_t)156 * 1024, kw);
+        if (kw && !(fat.fits && fat.wg <= cus) && rg == 1) fat = shape(fat_waves, 1, (size_t)156 * 1024, 0);
+        if (fat.fits && (fat.wg <= cus || rg > 1)) sh = fat;
+        else if (rg > 1) sh = shape(fat_waves, 1, (size_t)156 * 1024, 0);
     }
     if (!sh.fits) {
         set_error("gemv: one K unit of %d activation rows does not fit LDS", rv);
@@ -227,7 +244,7 @@ static int launch_gemv(const void *const *xs, int xk, const rlx_qweight *const *
     // Two K units per loop item halve the per-item bookkeeping; every chunk of every segment must then hold an even
     // number of units, and every wave still needs an item.
     static const bool env_u1 = getenv("RLX_GEMV_UPI") && atoi(getenv("RLX_GEMV_UPI")) == 1;
-    if (family == K_GEMV_Q4_0_R2 && !env_u1 && sh.kcu % 2 == 0 && sh.nwaves * 2 <= max_units) {
+    if (family == K_GEMV_Q4_0_R2 && rg == 1 && !env_u1 && sh.kcu % 2 == 0 && sh.nwaves * 2 <= max_units) {
         bool even = true;
         for (int i = 0; i < count; i++) even = even && ws[i]->dims.units % 2 == 0;
         if (even) id = (KernelId)(K_GEMV_Q4_0_U2_R2 + variant);
@@ -409,7 +426,7 @@ size_t rlx_mi355x_gguf_matmul_workspace(int scheme, int x_dtype, int64_t m, int6
     using namespace rlx;
     (void)n;
     int xk = x_kind(x_dtype);
-    if (xk < 0 || layout_of(scheme).unit_k == 0 || m <= (xk == 0 ? 8 : 16)) return 0;  // decode path: no workspace
+    if (xk < 0 || layout_of(scheme).unit_k == 0 || m <= decode_rows(xk)) return 0;  // decode path: no workspace
     GemmPlan p = gemm_plan(scheme, xk, m, k);
     return p.xh_bytes + p.sxh_bytes;
 }
@@ -437,7 +454,7 @@ int rlx_mi355x_gguf_matmul_bt_batch(const void *const *xs_dev, int x_dtype, cons
         set_error("gguf_matmul_bt: activation dtype %d unsupported (F32, BF16, F16 only)", x_dtype);
         return RLX_ERR_UNSUPPORTED;
     }
-    const int64_t cap = xk == 0 ? 8 : 16;  // activation rows one decode pass holds
+    const int64_t cap = decode_rows(xk);  // activation rows one pass of the decode kernels holds
     const size_t esz = xk == 0 ? 4 : 2;
     if (m > cap) {  // prefill: one GEMM per weight, sharing the workspace (same stream, so launches are ordered)
         // q, k, v (and gate, up) of a layer share their input: its f16 image in the workspace is made once. An image

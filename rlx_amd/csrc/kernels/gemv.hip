@@ -167,73 +167,84 @@ __device__ __forceinline__ void load_afrags(const half_t *xrow, bool live, int c
     }
 }
 
-template <int SCHEME, int NREG>
-__device__ __forceinline__ void compute_unit(const UnitRegs<SCHEME> &w, const half_t *xrow, bool live, Frag (&a)[4],
-                                             const float *sxs, int g, int ucol, int ublk, float acc[4]) {
+// One K unit of one 16-row weight tile against RG groups of 16 activation rows: the fragments are decoded once and
+// every group runs its own matrix instructions on them. xrow[rg] / live[rg]: the lane's row of group rg in LDS and
+// whether that row exists; acc[rg]: the four output rows 4 g + r of group rg this lane holds. SXS: row stride of the
+// Q4_K / Q5_K block-sum table (16 RG).
+template <int SCHEME, int NREG, int RG>
+__device__ __forceinline__ void compute_unit(const UnitRegs<SCHEME> &w, const half_t *const (&xrow)[RG], const bool (&live)[RG],
+                                             Frag (&a)[4], const float *sxs, int g, int ucol, int ublk, float (&acc)[RG][4]) {
     const float4_t zero = {0.f, 0.f, 0.f, 0.f};
-    if constexpr (SCHEME == SCHEME_Q4_0) {
+    constexpr int SXS = 16 * RG;
+    if constexpr (SCHEME == SCHEME_Q4_0 || SCHEME == SCHEME_Q8_0) {
         Frag b[4];
-        load_afrags<4>(xrow, live, ucol, a);
-#pragma unroll
-        for (int t = 0; t < 4; t++) unpack_q4<8>(w.q[t], b[t]);
-        float4_t blk[4];
-#pragma unroll
-        for (int t = 0; t < 4; t++) blk[t] = mfma16(a[t], b[t], zero);
+        if constexpr (RG == 1) load_afrags<4>(xrow[0], live[0], ucol, a);  // before the decode, so the reads are in flight under it
 #pragma unroll
         for (int t = 0; t < 4; t++) {
-            float d = scale_of(w.s, t);
+            if constexpr (SCHEME == SCHEME_Q4_0) {
+                unpack_q4<8>(w.q[t], b[t]);
+            } else {
+                const uint4_t &q = (t < 2) ? w.q0 : w.q1;
+                unpack_q8(q[2 * (t & 1)], q[2 * (t & 1) + 1], b[t]);
+            }
+        }
 #pragma unroll
-            for (int r = 0; r < NREG; r++) acc[r] = __builtin_fmaf(d, blk[t][r], acc[r]);
+        for (int rg = 0; rg < RG; rg++) {
+            if constexpr (RG > 1) load_afrags<4>(xrow[rg], live[rg], ucol, a);
+            float4_t blk[4];
+#pragma unroll
+            for (int t = 0; t < 4; t++) blk[t] = mfma16(a[t], b[t], zero);
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                float d = scale_of(w.s, t);
+#pragma unroll
+                for (int r = 0; r < NREG; r++) acc[rg][r] = __builtin_fmaf(d, blk[t][r], acc[rg][r]);
+            }
         }
     } else if constexpr (SCHEME == SCHEME_Q6K) {
         // B = sc * (q - 32): the 16-column scale is folded into the fragment (a lane's 8 columns share one scale), the
         // matrix unit accumulates the eight blocks of the super-block, d is applied once.
-        float4_t sum = zero;
+        float4_t sum[RG];
+#pragma unroll
+        for (int rg = 0; rg < RG; rg++) sum[rg] = zero;
         const int gshift = 8 * (g >> 1);  // this lane's half of each 32-column block: scale byte 2 j or 2 j + 1
 #pragma unroll
         for (int h = 0; h < 2; h++) {
-            load_afrags<4>(xrow, live, ucol + h * 128, a);
+            if constexpr (RG == 1) load_afrags<4>(xrow[0], live[0], ucol + h * 128, a);
             const uint4_t &q = h ? w.q1 : w.q0;
+            Frag b[4];
 #pragma unroll
             for (int t = 0; t < 4; t++) {
                 uint32_t hx = w.hw[2 * h + (t >> 1)];
                 if (t & 1) hx = __builtin_amdgcn_alignbit(hx, hx, 8);
                 const uint32_t scb = (w.sc[2 * h + (t >> 1)] >> (16 * (t & 1) + gshift)) & 0xFFu;
-                Frag b;
-                unpack_q6_scaled(q[t], hx, splat_ubyte_half(scb), b);
-                sum = mfma16(a[t], b, sum);
+                unpack_q6_scaled(q[t], hx, splat_ubyte_half(scb), b[t]);
+            }
+#pragma unroll
+            for (int rg = 0; rg < RG; rg++) {
+                if constexpr (RG > 1) load_afrags<4>(xrow[rg], live[rg], ucol + h * 128, a);
+#pragma unroll
+                for (int t = 0; t < 4; t++) sum[rg] = mfma16(a[t], b[t], sum[rg]);
             }
         }
         const float d = half_bits_to_float(w.d);
 #pragma unroll
-        for (int r = 0; r < NREG; r++) acc[r] = __builtin_fmaf(d, sum[r], acc[r]);
+        for (int rg = 0; rg < RG; rg++)
+#pragma unroll
+            for (int r = 0; r < NREG; r++) acc[rg][r] = __builtin_fmaf(d, sum[rg][r], acc[rg][r]);
     } else if constexpr (SCHEME == SCHEME_F16W) {
-        load_afrags<4>(xrow, live, ucol, a);
-        float4_t sum = zero;  // the matrix unit accumulates the four blocks; nothing to decode or scale
 #pragma unroll
-        for (int t = 0; t < 4; t++) {
-            Frag b;
-            b.u4 = w.q[t];
-            sum = mfma16(a[t], b, sum);
-        }
+        for (int rg = 0; rg < RG; rg++) {
+            load_afrags<4>(xrow[rg], live[rg], ucol, a);
+            float4_t sum = zero;  // the matrix unit accumulates the four blocks; nothing to decode or scale
 #pragma unroll
-        for (int r = 0; r < NREG; r++) acc[r] += sum[r];
-    } else if constexpr (SCHEME == SCHEME_Q8_0) {
-        Frag b[4];
-        load_afrags<4>(xrow, live, ucol, a);
+            for (int t = 0; t < 4; t++) {
+                Frag b;
+                b.u4 = w.q[t];
+                sum = mfma16(a[t], b, sum);
+            }
 #pragma unroll
-        for (int t = 0; t < 4; t++) {
-            const uint4_t &q = (t < 2) ? w.q0 : w.q1;
-            unpack_q8(q[2 * (t & 1)], q[2 * (t & 1) + 1], b[t]);
-        }
-        float4_t blk[4];
-#pragma unroll
-        for (int t = 0; t < 4; t++) blk[t] = mfma16(a[t], b[t], zero);
-#pragma unroll
-        for (int t = 0; t < 4; t++) {
-            float d = scale_of(w.s, t);
-#pragma unroll
-            for (int r = 0; r < NREG; r++) acc[r] = __builtin_fmaf(d, blk[t][r], acc[r]);
+            for (int r = 0; r < NREG; r++) acc[rg][r] += sum[r];
         }
     } else {
         float d = half_bits_to_float(w.meta[0] & 0xFFFFu);
@@ -243,26 +254,52 @@ __device__ __forceinline__ void compute_unit(const UnitRegs<SCHEME> &w, const ha
 #pragma unroll
         for (int h = 0; h < 2; h++) {
             Frag b[4];
-            load_afrags<4>(xrow, live, ucol + h * 128, a);
+            if constexpr (RG == 1) load_afrags<4>(xrow[0], live[0], ucol + h * 128, a);
             const uint4_t &q = h ? w.q1 : w.q0;
 #pragma unroll
             for (int t = 0; t < 4; t++) {
                 if constexpr (SCHEME == SCHEME_Q5K) unpack_q5(q[t], __builtin_amdgcn_alignbit(w.hb[h], w.hb[h], q5k_rot(t)), b[t]);
                 else unpack_q4<0>(q[t], b[t]);
             }
-            float4_t blk[4];
+            if constexpr (RG == 1) {
+                float4_t blk[4];
 #pragma unroll
-            for (int t = 0; t < 4; t++) blk[t] = mfma16(a[t], b[t], zero);
+                for (int t = 0; t < 4; t++) blk[t] = mfma16(a[t], b[t], zero);
 #pragma unroll
-            for (int t = 0; t < 4; t++) {
-                float dj = d * ubyte_to_float(sc[h], t);
-                float mj = dmin * ubyte_to_float(mn[h], t);
-                // sum of the activations of this 32-column block for the four output rows this lane holds
-                float4_t sx = *(const float4_t *)(sxs + (ublk + 4 * h + t) * 16 + 4 * g);
+                for (int t = 0; t < 4; t++) {
+                    float dj = d * ubyte_to_float(sc[h], t);
+                    float mj = dmin * ubyte_to_float(mn[h], t);
+                    // sum of the activations of this 32-column block for the four output rows this lane holds
+                    float4_t sx = *(const float4_t *)(sxs + (ublk + 4 * h + t) * SXS + 4 * g);
 #pragma unroll
-                for (int r = 0; r < NREG; r++) {
-                    acc[r] = __builtin_fmaf(dj, blk[t][r], acc[r]);
-                    acc[r] = __builtin_fmaf(-mj, sx[r], acc[r]);
+                    for (int r = 0; r < NREG; r++) {
+                        acc[0][r] = __builtin_fmaf(dj, blk[t][r], acc[0][r]);
+                        acc[0][r] = __builtin_fmaf(-mj, sx[r], acc[0][r]);
+                    }
+                }
+            } else {
+                // block by block, the groups side by side: only RG products are in flight at a time (all 8 RG of a unit
+                // at once is what the scheduler would pick, and more registers than a wave has)
+#pragma unroll
+                for (int t = 0; t < 4; t++) {
+                    const float dj = d * ubyte_to_float(sc[h], t);
+                    const float mj = dmin * ubyte_to_float(mn[h], t);
+                    float4_t blk[RG], sx[RG];
+#pragma unroll
+                    for (int rg = 0; rg < RG; rg++) {
+                        Frag af;
+                        af.u4 = *(const uint4_t *)(xrow[rg] + ucol + h * 128 + t * 32);
+                        blk[rg] = mfma16(af, b[t], zero);
+                        sx[rg] = *(const float4_t *)(sxs + (ublk + 4 * h + t) * SXS + 16 * rg + 4 * g);
+                    }
+#pragma unroll
+                    for (int rg = 0; rg < RG; rg++)
+#pragma unroll
+                        for (int r = 0; r < NREG; r++) {
+                            acc[rg][r] = __builtin_fmaf(dj, blk[rg][r], acc[rg][r]);
+                            acc[rg][r] = __builtin_fmaf(-mj, sx[rg][r], acc[rg][r]);
+                        }
+                    __builtin_amdgcn_sched_barrier(0);
                 }
             }
         }
@@ -391,7 +428,7 @@ extern "C" __global__ __launch_bounds__(256) void rlx_argmax_finish(const unsign
 // writes the SwiGLU of the two sums.
 enum { GEMV_PLAIN = 0, GEMV_ARGMAX = 1, GEMV_PAIRED = 2, GEMV_NORM = 4 };  // GEMV_NORM combines with the others
 
-template <int SCHEME, int NREG, int DEPTH, int MODE, int UPI = 1>
+template <int SCHEME, int NREG, int DEPTH, int MODE, int UPI = 1, int RG = 1>
 __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
     constexpr Layout L = layout_of(SCHEME);
     constexpr int BLK_PER_UNIT = L.unit_k / 32;
@@ -402,8 +439,7 @@ __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), nwaves = blockDim.x >> 6;
     const int nrow = l & 15, g = l >> 4;
     const int rv = (a.x_dtype == X_F32) ? 2 * a.m : a.m;  // virtual A rows
-    const int ng = (rv + 3) >> 2;                         // lane groups whose accumulators hold real rows
-    const bool has_rows = g < ng;
+    const int ng = (rv + 3) >> 2;                         // groups of four output rows that exist (16 RG at most)
 
     int s = 0;
 #pragma unroll
@@ -434,7 +470,16 @@ __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
     const size_t part_bytes = (size_t)a.max_tiles_per_wg * kw * slot_floats * 4;
     half_t *xs = (half_t *)(smem + part_bytes);
     float *sxs = (float *)(smem + part_bytes + (((size_t)rv * row_stride * 2 + 15) & ~(size_t)15));  // [blk][16]
-    const half_t *xrow = xs + min(nrow, rv - 1) * row_stride + g * 8;  // this lane's A row
+    const half_t *xrow[RG];  // this lane's A row in each group of 16 activation rows
+    bool live[RG];
+#pragma unroll
+    for (int rg = 0; rg < RG; rg++) {
+        xrow[rg] = xs + min(16 * rg + nrow, rv - 1) * row_stride + g * 8;
+        // With one group, lanes without a row skip their LDS reads (at one row that is 15 lanes of 16). With several,
+        // nearly every lane has a row and a lane past the end rereads the last row (its products are never read back):
+        // no branches in the inner loop.
+        live[rg] = RG > 1 || nrow < rv;
+    }
 
     for (int i = tid; i < ((MODE & GEMV_PAIRED) ? 2 : 1) * ntiles * kw * slot_floats; i += blockDim.x) part[i] = 0.f;
     // RMSNorm prologue: one wave per activation row sums the squares of the whole row (the sum is needed before any
@@ -505,7 +550,7 @@ __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
         __syncthreads();
         if constexpr (SCHEME == SCHEME_Q4K || SCHEME == SCHEME_Q5K) {
             const int nblk = nu * BLK_PER_UNIT;
-            // rows >= rv of the [blk][16] table are never read: compute_unit only uses the rows its lane group owns
+            // rows >= rv of the [blk][16 RG] table are never read: compute_unit only uses the rows its lane group owns
             for (int idx = tid; idx < nblk * rv; idx += blockDim.x) {
                 const int blk = idx / rv, i = idx - blk * rv;
                 float sum = 0.f;
@@ -516,11 +561,15 @@ __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
 #pragma unroll
                     for (int e = 0; e < 8; e++) sum += (float)f.h8[e];
                 }
-                sxs[blk * 16 + i] = sum;
+                sxs[blk * (16 * RG) + i] = sum;
             }
             __syncthreads();
         }
-        float acc[4] = {0.f, 0.f, 0.f, 0.f};
+        float acc[RG][4];
+#pragma unroll
+        for (int rg = 0; rg < RG; rg++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) acc[rg][r] = 0.f;
         Frag afr[4];
 #pragma unroll
         for (int t = 0; t < 4; t++) afr[t].u4 = uint4_t{0, 0, 0, 0};
@@ -533,16 +582,19 @@ __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
                     prefetch(ring[d]);
 #pragma unroll
                     for (int p = 0; p < UPI; p++)
-                        compute_unit<SCHEME, NREG>(cur.u[p], xrow, nrow < rv, afr, sxs, g, (cu_u * UPI + p) * L.unit_k,
-                                                   (cu_u * UPI + p) * BLK_PER_UNIT, acc);
+                        compute_unit<SCHEME, NREG, RG>(cur.u[p], xrow, live, afr, sxs, g, (cu_u * UPI + p) * L.unit_k,
+                                                       (cu_u * UPI + p) * BLK_PER_UNIT, acc);
                     cu_u += kw;
                     if (cu_u >= nug) {  // last unit of this tile for this wave: bank the partial sums
-                        if (has_rows) {
-                            float *slot = part + ((size_t)cu_t * kw + kl) * slot_floats + g * 64 + nrow;
 #pragma unroll
-                            for (int r = 0; r < 4; r++) {
-                                if (r < NREG) slot[r * 16] += acc[r];
-                                acc[r] = 0.f;
+                        for (int rg = 0; rg < RG; rg++) {
+                            if (4 * rg + g < ng) {  // this lane's four rows of the group exist
+                                float *slot = part + ((size_t)cu_t * kw + kl) * slot_floats + (4 * rg + g) * 64 + nrow;
+#pragma unroll
+                                for (int r = 0; r < 4; r++) {
+                                    if (r < NREG) slot[r * 16] += acc[rg][r];
+                                    acc[rg][r] = 0.f;
+                                }
                             }
                         }
                         cu_t += tw;
@@ -605,9 +657,10 @@ __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
 
 }  // namespace rlx
 
-#define RLX_GEMV_INST(name, SCHEME, NREG, DEPTH, MODE, UPI)                                                 \
-    extern "C" __global__ __launch_bounds__(1024) void name(rlx::GemvArgs a) {                               \
-        rlx::gemv_body<SCHEME, NREG, DEPTH, MODE, UPI>(a);                                                    \
+#define RLX_GEMV_INST(name, SCHEME, NREG, DEPTH, MODE, UPI) RLX_GEMV_INST_RG(name, SCHEME, NREG, DEPTH, MODE, UPI, 1, 1024)
+#define RLX_GEMV_INST_RG(name, SCHEME, NREG, DEPTH, MODE, UPI, RG, THREADS)                                 \
+    extern "C" __global__ __launch_bounds__(THREADS) void name(rlx::GemvArgs a) {                            \
+        rlx::gemv_body<SCHEME, NREG, DEPTH, MODE, UPI, RG>(a);                                                \
     }
 // NREG = 2: at most two virtual rows (m = 1 f32, or m <= 2 16-bit); NREG = 4 otherwise.
 #define RLX_GEMV_SCHEME(tag, SCHEME, DEPTH, UPI)                                                      \
@@ -631,3 +684,14 @@ RLX_GEMV_SCHEME(q5_k, rlx::SCHEME_Q5K, 2, 1)
 // Two 128-column units per loop item: taken when every K run holds an even number of units. (Measured neutral to
 // slightly slower for Q8_0, whose unit is twice the bytes, so only Q4_0 has it.)
 RLX_GEMV_SCHEME(q4_0_u2, rlx::SCHEME_Q4_0, 2, 2)
+// Two groups of 16 activation rows per weight fragment (17..32 rows): plain epilogue only, workgroups of eight waves
+// (sixteen measured 40 - 70 % slower: the activation chunk and the partial sums of twice the tiles no longer fit
+// side by side). Four groups were built and measured too: at 64 rows a tile's partial sums take 4 KB of LDS, which
+// leaves room for three K units of activations per chunk, and the prefill kernel is faster.
+#define RLX_GEMV_ROWGROUPS(tag, SCHEME, DEPTH) RLX_GEMV_INST_RG(rlx_gemv_##tag##_g2, SCHEME, 4, DEPTH, rlx::GEMV_PLAIN, 1, 2, 512)
+RLX_GEMV_ROWGROUPS(q4_0, rlx::SCHEME_Q4_0, 2)
+RLX_GEMV_ROWGROUPS(q8_0, rlx::SCHEME_Q8_0, 2)
+RLX_GEMV_ROWGROUPS(q4_k, rlx::SCHEME_Q4K, 2)
+RLX_GEMV_ROWGROUPS(f16w, rlx::SCHEME_F16W, 2)
+RLX_GEMV_ROWGROUPS(q6_k, rlx::SCHEME_Q6K, 2)
+RLX_GEMV_ROWGROUPS(q5_k, rlx::SCHEME_Q5K, 2)

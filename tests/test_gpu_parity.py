@@ -192,9 +192,23 @@ def test_decode_many_rows_wide_matrix(oracle, scheme, m, x_dtype):
         assert rel_err(got[:, n0:n1], oracle.gguf_matmul_f64(x, packed, m, k, n, scheme, n0, n1)) <= TOL
 
 
+@pytest.mark.parametrize("scheme,m,x_dtype", [(Q4_0, 17, DType.BF16), (Q4_0, 32, DType.BF16), (Q8_0, 16, DType.F32), (Q4K, 9, DType.F32),
+                                              (Q4K, 32, DType.F16), (Q4K, 24, DType.BF16), (Q8_0, 31, DType.BF16)])
+def test_decode_two_row_groups(oracle, scheme, m, x_dtype):
+    # 17..32 MFMA rows (an f32 row counts twice): the weight fragments are decoded once for two groups of 16 rows
+    check_matmul(oracle, scheme, 512, 2048, m, x_dtype=x_dtype, seed=m)
+    check_matmul(oracle, scheme, 50, 96 if scheme != Q4K else 768, m, x_dtype=x_dtype, seed=m + 1)  # ragged n and k
+
+
+def test_decode_two_row_groups_wide_matrix_and_long_k(oracle):
+    got, x, packed, _ = check_matmul(oracle, Q4_0, 28672, 2048, 24, x_dtype=DType.BF16, seed=3, cols=(0, 64))
+    assert rel_err(got[:, 28600:28672], oracle.gguf_matmul_f64(x, packed, 24, 2048, 28672, Q4_0, 28600, 28672)) <= TOL
+    check_matmul(oracle, Q4K, 48, 28672, 32, x_dtype=DType.BF16, std=0.015, seed=4)  # many K chunks
+
+
 def test_rows_just_past_the_decode_limit(oracle):
-    check_matmul(oracle, Q4_0, 128, 256, 20, seed=4)           # f32: more than 8 rows -> prefill kernel
-    check_matmul(oracle, Q4K, 64, 512, 37, x_dtype=DType.BF16, seed=5)  # more than 16 rows -> prefill kernel
+    check_matmul(oracle, Q4_0, 128, 256, 20, seed=4)           # f32: more than 16 rows -> prefill kernel
+    check_matmul(oracle, Q4K, 64, 512, 37, x_dtype=DType.BF16, seed=5)  # more than 32 rows -> prefill kernel
 
 
 def test_decode_large_k_is_chunked(oracle):

@@ -260,7 +260,7 @@ def bf16_bits(x):
 # super-block scales that give weights of a few hundredths, like a quantized model's, whatever the code bytes are
 MODEL_SCALE = {Q5K: (4e-5, 2e-5), Q6K: (5e-6, 0.0), Q8K: (2e-4, 0.0), Q2K: (5e-4, 1e-4), Q3K: (2e-4, 0.0)}
 SHAPES = [(1, 200, 1024, DType.F32), (4, 48, 2304, DType.F32), (16, 130, 512, DType.BF16), (64, 200, 1024, DType.BF16),
-          (300, 136, 768, DType.F32)]
+          (300, 136, 768, DType.F32), (27, 330, 2048, DType.BF16), (13, 72, 768, DType.F32)]  # the last two: 17..32 MFMA rows
 
 
 def run_wide(scheme, blocks, m, n, k, dtype):
