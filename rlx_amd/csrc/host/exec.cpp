@@ -408,7 +408,7 @@ rlx_exec *rlx_mi355x_compile(const rlx_graph_desc *g, const rlx_compile_opts *op
             nd.aux = take(rlx_mi355x_fake_quantize_scratch_bytes(nd.numel, nd.chan_dim, nd.inner));
             nd.codes = take((size_t)nd.numel);
         }
-        if (nd.d.op_kind == RLX_OP_DEQUANT_MATMUL && nd.m > 8)  // prefill workspace, sized for f32 activations
+        if (nd.d.op_kind == RLX_OP_DEQUANT_MATMUL && nd.m > 16)  // beyond the decode kernels for any input dtype: prefill workspace, sized for f32
             nd.aux = take(rlx_mi355x_gguf_matmul_workspace((int)nd.d.scheme, RLX_F32, nd.m, nd.k, nd.n));
     }
     e->arena_bytes = off;
@@ -538,7 +538,7 @@ static int enqueue_schedule(rlx_exec *e) {
             }
             RLX_TRY(rlx_mi355x_gguf_grouped_matmul_bt(e->ptr(x.slot), (int)dt, w.qw, (const float *)e->ptr(idx.slot),
                                                       (float *)e->ptr(nd.slot), nd.m, e->stream));
-        } else if (nd.d.op_kind == RLX_OP_DEQUANT_MATMUL && nd.m > 8) {
+        } else if (nd.d.op_kind == RLX_OP_DEQUANT_MATMUL && nd.m > 16) {
             for (uint32_t id : step) {  // prefill: one GEMM per node, each with its own workspace slot
                 Node &mm = e->nodes[id];
                 Node &x = e->nodes[mm.d.inputs[0]];

@@ -374,26 +374,27 @@ def test_graph_typed_bf16_input(oracle):
     assert rel_err(got, oracle.gguf_matmul_f64(x, packed, m, k, n, Q4K)) <= TOL
 
 
-def test_graph_batches_independent_matmuls(oracle):
+@pytest.mark.parametrize("m", [2, 12])
+def test_graph_batches_independent_matmuls(oracle, m):
     # q/k/v-style: three weights on one activation vector plus a fourth matmul with its own activations and a
     # different k: all four are ready at the same point of the schedule and go out as one batched launch; outputs
-    # must be those of four separate matmuls, eagerly and on every hipGraph replay.
+    # must be those of four separate matmuls, eagerly and on every hipGraph replay. m = 12 f32 rows: the two-group kernel.
     k, ns = 1024, [256, 64, 48]
     rng = np.random.default_rng(50)
-    x = rng.standard_normal((2, k)).astype(np.float32)
-    x2 = rng.standard_normal((2, 512)).astype(np.float32)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    x2 = rng.standard_normal((m, 512)).astype(np.float32)
     g = Graph.new("qkv")
-    xi = g.input("x", Shape.new([2, k], DType.F32))
-    xj = g.input("x2", Shape.new([2, 512], DType.F32))
+    xi = g.input("x", Shape.new([m, k], DType.F32))
+    xj = g.input("x2", Shape.new([m, 512], DType.F32))
     packs, outs = [], []
     for i, n in enumerate(ns):
         p, _ = make_weights(Q4_0, n, k, seed=60 + i)
         packs.append(p)
         w = g.param(f"w{i}", Shape.new([len(p)], DType.U8))
-        outs.append(g.add_node(Op.DequantMatMul(QuantScheme.GgufQ4_0), [xi, w], Shape.new([2, n], DType.F32)))
+        outs.append(g.add_node(Op.DequantMatMul(QuantScheme.GgufQ4_0), [xi, w], Shape.new([m, n], DType.F32)))
     p4, _ = make_weights(Q4_0, 32, 512, seed=70)
     w4 = g.param("w4", Shape.new([len(p4)], DType.U8))
-    outs.append(g.add_node(Op.DequantMatMul(QuantScheme.GgufQ4_0), [xj, w4], Shape.new([2, 32], DType.F32)))
+    outs.append(g.add_node(Op.DequantMatMul(QuantScheme.GgufQ4_0), [xj, w4], Shape.new([m, 32], DType.F32)))
     g.set_outputs(outs)
     c = Session.new().compile(g)
     for i, p in enumerate(packs):
@@ -402,8 +403,8 @@ def test_graph_batches_independent_matmuls(oracle):
     for attempt in ("eager", "hipGraph replay 1", "hipGraph replay 2"):
         got = c.run([("x", x), ("x2", x2)])
         for i, n in enumerate(ns):
-            assert rel_err(got[i].reshape(2, n), oracle.gguf_matmul_f64(x, packs[i], 2, k, n, Q4_0)) <= TOL, attempt
-        assert rel_err(got[3].reshape(2, 32), oracle.gguf_matmul_f64(x2, p4, 2, 512, 32, Q4_0)) <= TOL, attempt
+            assert rel_err(got[i].reshape(m, n), oracle.gguf_matmul_f64(x, packs[i], m, k, n, Q4_0)) <= TOL, attempt
+        assert rel_err(got[3].reshape(m, 32), oracle.gguf_matmul_f64(x2, p4, m, 512, 32, Q4_0)) <= TOL, attempt
         if attempt == "eager":
             c.capture()
         x = (x * np.float32(1.5)).astype(np.float32)  # new inputs each replay: the graph must read them afresh
