@@ -139,6 +139,12 @@ static int launch_gemv(const void *const *xs, int xk, const rlx_qweight *const *
         max_units = std::max(max_units, (int)ws[i]->dims.units);
         work += ws[i]->dims.row_tiles * ws[i]->dims.units * (pairs ? 2 : 1);
     }
+    // Segments with the longest K last (equal K keeps the caller's order, which the expert routing relies on: segment s
+    // is token s). Measured on the seven projections of a layer: 5185 GB/s with the 14336-wide down projection at the
+    // end of the workgroup order, 5050 with it at the front, whatever the order of the others.
+    int order[GEMV_MAX_SEG];
+    for (int i = 0; i < count; i++) order[i] = i;
+    std::stable_sort(order, order + count, [&](int a, int b) { return ws[a]->dims.units < ws[b]->dims.units; });
     const int cus = std::max(1, device_props().cu_count);
     const size_t slot_bytes = (size_t)ng * 256;
     auto stage_bytes = [&](int kcu) {
@@ -173,7 +179,8 @@ static int launch_gemv(const void *const *xs, int xk, const rlx_qweight *const *
             const long long target_items = std::max<long long>(1, (long long)((double)((work + slots - 1) / slots) * grow));
             sh.wg = 0;
             max_tpw = 1;
-            for (int i = 0; i < count; i++) {
+            for (int oi = 0; oi < count; oi++) {
+                const int i = order[oi];
                 const WeightDims &D = ws[i]->dims;
                 const int per_tile = pairs ? 2 : 1;  // partial-sum slots and K runs per row tile
                 int tpw = (int)std::max<long long>(1, (target_items + D.units * per_tile / 2) / (D.units * per_tile));
@@ -182,7 +189,7 @@ static int launch_gemv(const void *const *xs, int xk, const rlx_qweight *const *
                 max_tpw = std::max(max_tpw, tpw * per_tile);
                 const int seg_wgs = (int)((D.row_tiles + tpw - 1) / tpw);
                 static const bool contiguous = getenv("RLX_GEMV_CONTIGUOUS") != nullptr;
-                sh.a.seg[i] = GemvSeg{ws[i]->dev, xs[i], outs[i], (int)D.n, (int)D.k, (int)D.row_tiles, (int)D.units, sh.wg, tpw,
+                sh.a.seg[oi] = GemvSeg{ws[i]->dev, xs[i], outs[i], (int)D.n, (int)D.k, (int)D.row_tiles, (int)D.units, sh.wg, tpw,
                                       contiguous ? 1 : seg_wgs, pairs ? pairs[i]->dev : nullptr};
                 sh.wg += seg_wgs;
             }
