@@ -221,12 +221,14 @@ def test_q4k_gemv_llama_shape(oracle):
     check_matmul(oracle, Q4K, 4096, 4096, 1, seed=8)
 
 
-def test_matmul_is_deterministic(oracle):
+@pytest.mark.parametrize("m", [1, 12, 24])
+def test_matmul_is_deterministic(oracle, m):
+    # every decode shape (all waves on one tile; two waves per tile; two row groups) adds its partial sums in a fixed order
     packed, _ = make_weights(Q4_0, 1024, 4096, seed=9)
-    x = np.random.default_rng(9).standard_normal((1, 4096)).astype(np.float32)
+    x = f32_to_bf16_bits(np.random.default_rng(9).standard_normal((m, 4096)).astype(np.float32))
     w = ops.QWeight(Q4_0, packed, 1024, 4096)
-    a = ops.gguf_matmul_bt(x, w, 1)
-    b = ops.gguf_matmul_bt(x, w, 1)
+    a = ops.gguf_matmul_bt(x, w, m, DType.BF16)
+    b = ops.gguf_matmul_bt(x, w, m, DType.BF16)
     assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
 
 
