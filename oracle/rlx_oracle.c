@@ -28,6 +28,10 @@
  *                         2 ulp; the last ulp follows the platform's expf like the reference's f32::exp (unpinned there)
  *   gguf_tied_lm_argmax   the reference's test (rlx-cpu/src/lm_head.rs:306-334: equals the argmax of gguf_matmul_bt's
  *                         logits) + constructed ties, NaN and all -inf rows against the loop's stated rule
+ *   gguf_tied_lm_topk     the inputs of the reference's test (rlx-cpu/src/lm_head.rs:278-304) against a brute-force
+ *                         stable sort of all scores (values pinned; the rows among the tied scores follow the
+ *                         smaller-row rule stated here, the reference leaves their order to an unstable selection),
+ *                         random rows of three schemes against the same brute force, cap = 1 against the argmax
  *   fake_quantize         closed forms (channel max -> code +-q_max, all-zero
  *                         channel, constructed ties, NaN), shapes/inputs of
  *                         rlx-mlx/tests/autodiff_fakequant_parity.rs:189-308
