@@ -446,7 +446,7 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
                 if (orow < a.m_out) {
                     float *p = a.out + (long long)orow * a.n + col;
                     if (a.use_atomics) atomicAdd(p, v);
-                    else *p = v;
+                    else __builtin_nontemporal_store(v, p);  // written once, read by another kernel: keep it out of the way of the operands
                 }
             }
         }
