@@ -368,8 +368,11 @@ def test_graph_fq_then_q8_0_matmul(oracle):
     assert rel_err(y_got.reshape(rows, n), ref64) <= TOL
 
 
-def test_graph_typed_bf16_input(oracle):
-    m, k, n = 4, 512, 64
+@pytest.mark.parametrize("m", [4, 16, 24, 40])
+def test_graph_typed_bf16_input(oracle, m):
+    # 4 and 16 rows: the executor's batched decode branch; 24: its per-node branch, which lands on the two-group decode
+    # kernel for 16-bit inputs; 40: the prefill kernel with the node's workspace
+    k, n = 512, 64
     packed, _ = make_weights(Q4K, n, k, seed=43)
     x = oracle.bf16_round(np.random.default_rng(44).standard_normal((m, k)).astype(np.float32))
     got = run_dq(packed, Q4K, f32_to_bf16_bits(x), m, k, n, typed=DType.BF16)
