@@ -235,3 +235,22 @@ def test_topk_ties_nan_tail_and_limits_on_device():
     want_idx, want_val = full_sort_topk(logits, 64)
     assert np.array_equal(idx, want_idx) and np.array_equal(val, want_val)
     big.free()
+
+
+@pytest.mark.gpu
+def test_topk_and_argmax_at_llama3_vocabulary_size():
+    # [128256, 4096] Q4_K (295 MB): the size the LM-head figures are quoted on. Checked through properties that need no
+    # CPU matmul: the selection is bit-identical to a full sort of the logits the plain kernel writes, and the fused
+    # argmax agrees with its first entry.
+    n, k = 128256, 4096
+    slab = ops.quantize(QuantScheme.GgufQ4K, (ops.philox_normal(21, 2048 * k) * np.float32(0.02)).astype(np.float32)).reshape(2048, -1)
+    packed = np.concatenate([np.roll(slab, 3 * i, axis=0) for i in range(63)], axis=0)[:n]
+    w = ops.QWeight(QuantScheme.GgufQ4K, packed.reshape(-1), n, k)
+    hidden = ops.philox_normal(8, k)
+    logits = ops.gguf_matmul_bt(hidden.reshape(1, k), w, 1)[0]
+    for cap in (1, 40, 64):
+        idx, val = ops.gguf_tied_lm_topk(hidden, w, cap)
+        want_idx, want_val = full_sort_topk(logits, cap)
+        assert np.array_equal(idx, want_idx) and np.array_equal(val.view(np.uint32), want_val.view(np.uint32)), cap
+    assert ops.gguf_tied_lm_argmax(hidden, w) == (int(want_idx[0]), float(want_val[0]))
+    w.free()
