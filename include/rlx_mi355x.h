@@ -203,6 +203,11 @@ int rlx_mi355x_gguf_tied_lm_argmax(const void *hidden_dev, int x_dtype, const rl
 size_t rlx_mi355x_tied_lm_topk_scratch_bytes(int64_t n_vocab, int cap);
 int rlx_mi355x_gguf_tied_lm_topk(const void *hidden_dev, int x_dtype, const rlx_qweight *embed, int cap, uint32_t *out_idx_dev,
                                  float *out_val_dev, void *scratch_dev, size_t scratch_bytes, void *stream);
+/* The same with the final Op::RmsNorm fused into the logits kernel's activation staging (f32 hidden state), as in
+ * rlx_mi355x_rmsnorm_gguf_tied_lm_argmax. */
+int rlx_mi355x_rmsnorm_gguf_tied_lm_topk(const float *hidden_dev, const float *gamma_dev, const float *beta_dev, float eps,
+                                         const rlx_qweight *embed, int cap, uint32_t *out_idx_dev, float *out_val_dev,
+                                         void *scratch_dev, size_t scratch_bytes, void *stream);
 int rlx_mi355x_gguf_matmul_bt_batch(const void *const *xs_dev, int x_dtype, const rlx_qweight *const *ws,
                                     float *const *outs_dev, int count, int64_t m, void *workspace, size_t workspace_bytes,
                                     void *stream);

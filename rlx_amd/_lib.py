@@ -84,6 +84,7 @@ SIGNATURES = {
     "rlx_mi355x_gguf_tied_lm_argmax": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _vp]),
     "rlx_mi355x_gguf_tied_lm_topk": (_i, [_vp, _i, _vp, _i, _vp, _vp, _vp, C.c_size_t, _vp]),
     "rlx_mi355x_tied_lm_topk_scratch_bytes": (C.c_size_t, [C.c_int64, _i]),
+    "rlx_mi355x_rmsnorm_gguf_tied_lm_topk": (_i, [_vp, _vp, _vp, _f, _vp, _i, _vp, _vp, _vp, C.c_size_t, _vp]),
     "rlx_mi355x_tied_lm_argmax_scratch_bytes": (C.c_size_t, []),
     "rlx_mi355x_gguf_matmul_swiglu": (_i, [_vp, _i, _vp, _vp, _vp, _i64, _vp]),
     "rlx_mi355x_rmsnorm_gguf_matmul_bt_batch": (_i, [_vp, _vp, _vp, _f, _vp, _vp, _i, _i64, _vp]),

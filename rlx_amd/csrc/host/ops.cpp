@@ -671,27 +671,18 @@ size_t rlx_mi355x_tied_lm_topk_scratch_bytes(int64_t n_vocab, int cap) {
     return (size_t)((n_vocab * 4 + 7) / 8 * 8 + 2 * keys * 8);
 }
 
-int rlx_mi355x_gguf_tied_lm_topk(const void *hidden_dev, int x_dtype, const rlx_qweight *embed, int cap, uint32_t *out_idx_dev,
-                                 float *out_val_dev, void *scratch_dev, size_t scratch_bytes, void *stream) {
+static int tied_lm_topk(const char *who, const void *hidden_dev, int xk, const rlx::RmsNorm *norm, const rlx_qweight *embed, int cap,
+                        uint32_t *out_idx_dev, float *out_val_dev, void *scratch_dev, size_t scratch_bytes, void *stream) {
     using namespace rlx;
-    if (!hidden_dev || !embed || !out_idx_dev || !out_val_dev || !scratch_dev) {
-        set_error("gguf_tied_lm_topk: null argument");
-        return RLX_ERR_INVALID;
-    }
-    const int xk = x_kind(x_dtype);
-    if (xk < 0) {
-        set_error("gguf_tied_lm_topk: hidden dtype %d is not F32 / BF16 / F16", x_dtype);
-        return RLX_ERR_UNSUPPORTED;
-    }
     const int64_t n = embed->dims.n;
     if (cap < 1) cap = 1;  // the reference's cap.min(n_vocab).max(1)
     if (cap > n) cap = (int)n;
     if (cap > TOPK_MAX_CAP) {
-        set_error("gguf_tied_lm_topk: cap %d is beyond the selection kernel (cap <= %d)", cap, TOPK_MAX_CAP);
+        set_error("%s: cap %d is beyond the selection kernel (cap <= %d)", who, cap, TOPK_MAX_CAP);
         return RLX_ERR_UNSUPPORTED;
     }
     if ((uintptr_t)scratch_dev % 8 != 0 || scratch_bytes < rlx_mi355x_tied_lm_topk_scratch_bytes(n, cap)) {
-        set_error("gguf_tied_lm_topk: scratch of %zu bytes (8-byte aligned) needed, got %zu", rlx_mi355x_tied_lm_topk_scratch_bytes(n, cap),
+        set_error("%s: scratch of %zu bytes (8-byte aligned) needed, got %zu", who, rlx_mi355x_tied_lm_topk_scratch_bytes(n, cap),
                   scratch_bytes);
         return RLX_ERR_INVALID;
     }
@@ -702,7 +693,7 @@ int rlx_mi355x_gguf_tied_lm_topk(const void *hidden_dev, int x_dtype, const rlx_
     const void *xs[1] = {hidden_dev};
     const rlx_qweight *ws[1] = {embed};
     float *outs[1] = {logits};
-    RLX_TRY(launch_gemv(xs, xk, ws, outs, 1, 1, (hipStream_t)stream));
+    RLX_TRY(launch_gemv(xs, xk, ws, outs, 1, 1, (hipStream_t)stream, nullptr, nullptr, nullptr, norm));
     // every pass: one wave per 1024 candidates keeps its cap best; the pass with a single wave writes the answer
     int64_t count = n;
     int side = 0;
@@ -718,6 +709,35 @@ int rlx_mi355x_gguf_tied_lm_topk(const void *hidden_dev, int x_dtype, const rlx_
         side ^= 1;
     }
     return RLX_OK;
+}
+
+int rlx_mi355x_gguf_tied_lm_topk(const void *hidden_dev, int x_dtype, const rlx_qweight *embed, int cap, uint32_t *out_idx_dev,
+                                 float *out_val_dev, void *scratch_dev, size_t scratch_bytes, void *stream) {
+    using namespace rlx;
+    if (!hidden_dev || !embed || !out_idx_dev || !out_val_dev || !scratch_dev) {
+        set_error("gguf_tied_lm_topk: null argument");
+        return RLX_ERR_INVALID;
+    }
+    const int xk = x_kind(x_dtype);
+    if (xk < 0) {
+        set_error("gguf_tied_lm_topk: hidden dtype %d is not F32 / BF16 / F16", x_dtype);
+        return RLX_ERR_UNSUPPORTED;
+    }
+    return tied_lm_topk("gguf_tied_lm_topk", hidden_dev, xk, nullptr, embed, cap, out_idx_dev, out_val_dev, scratch_dev, scratch_bytes, stream);
+}
+
+int rlx_mi355x_rmsnorm_gguf_tied_lm_topk(const float *hidden_dev, const float *gamma_dev, const float *beta_dev, float eps,
+                                         const rlx_qweight *embed, int cap, uint32_t *out_idx_dev, float *out_val_dev,
+                                         void *scratch_dev, size_t scratch_bytes, void *stream) {
+    using namespace rlx;
+    RLX_TRY(check_norm("rmsnorm_gguf_tied_lm_topk", hidden_dev, gamma_dev, beta_dev, 1));
+    if (!embed || !out_idx_dev || !out_val_dev || !scratch_dev) {
+        set_error("rmsnorm_gguf_tied_lm_topk: null argument");
+        return RLX_ERR_INVALID;
+    }
+    const RmsNorm norm{gamma_dev, beta_dev, eps};
+    return tied_lm_topk("rmsnorm_gguf_tied_lm_topk", hidden_dev, 0, &norm, embed, cap, out_idx_dev, out_val_dev, scratch_dev, scratch_bytes,
+                        stream);
 }
 
 int rlx_mi355x_gguf_grouped_matmul_bt(const void *x_dev, int x_dtype, const rlx_qweight *w, const float *expert_idx_dev,

@@ -284,6 +284,20 @@ def gguf_tied_lm_topk(hidden, embed: QWeight, cap, x_dtype=DType.F32):
     return raw[:c].copy(), raw[c:].view(np.float32).copy()
 
 
+def rmsnorm_gguf_tied_lm_topk(hidden, gamma, beta, eps, embed: QWeight, cap):
+    """The final RmsNorm, the tied LM head and the top-`cap` selection: (rows, values), largest first."""
+    c = max(1, min(int(cap), embed.n))
+    hd = DeviceBuffer.from_numpy(np.ascontiguousarray(hidden, dtype=np.float32))
+    g, b = _norm_bufs(gamma, beta)
+    need = _lib.lib().rlx_mi355x_tied_lm_topk_scratch_bytes(embed.n, c)
+    scratch, res = DeviceBuffer(max(need, 8)), DeviceBuffer(8 * c)
+    _lib.check(_lib.lib().rlx_mi355x_rmsnorm_gguf_tied_lm_topk(hd.ptr, g.ptr, b.ptr if b else None, eps, embed.ptr, int(cap), res.ptr,
+                                                              res.ptr + 4 * c, scratch.ptr, scratch.nbytes, None))
+    sync()
+    raw = res.to_numpy(np.uint32, 2 * c)
+    return raw[:c].copy(), raw[c:].view(np.float32).copy()
+
+
 def fake_quantize(x, shape, axis, bits, scale_mode=ScaleMode.PerBatch, decay=0.0, state=None,
                   round_mode=RoundMode.HalfAway):
     """Host convenience around rlx_mi355x_fake_quantize. Returns (out f32, codes i8, scales f32); EMA updates `state`."""

@@ -77,6 +77,11 @@ def test_rmsnorm_swiglu_and_argmax():
     idx, val = ops.rmsnorm_gguf_tied_lm_argmax(x[0], gamma, None, 1e-6, w_up)
     logits = ops.gguf_matmul_bt(xn, w_up, 1)[0]
     assert idx == int(np.argmax(logits)) and abs(val - logits[idx]) <= 2e-5 * max(abs(logits[idx]), 1.0)
+    # top-k behind the same fused norm: its first entry is the argmax, its values are the (normalised) logits, in order
+    tidx, tval = ops.rmsnorm_gguf_tied_lm_topk(x[0], gamma, None, 1e-6, w_up, 12)
+    assert (int(tidx[0]), float(tval[0])) == (idx, val) and np.all(np.diff(tval) <= 0) and len(set(tidx.tolist())) == 12
+    assert np.all(np.abs(tval - logits[tidx]) <= 2e-5 * np.maximum(np.abs(logits[tidx]), 1.0))
+    assert tval[-1] >= np.sort(logits)[-12] - 2e-5
     w_up.free()
     w_gate.free()
 
