@@ -330,6 +330,28 @@ def test_fq_ema_and_fixed(oracle):
     check_fq(oracle, x, x.shape, 0, 8, ScaleMode.EMA, decay=0.9, state=np.zeros(512, np.float32))
 
 
+@pytest.mark.parametrize("rows,cols", [(1030, 2048), (37, 4096), (8192, 2048), (8193, 2048), (128, 2064), (2305, 6144)])
+def test_fq_column_shapes(oracle, rows, cols):
+    # column channels (the layout of the benchmark configuration) at ragged row counts: every rounding mode and
+    # width, int8 codes, NaN / zero / tiny channels, maxima at the corners of the tensor, and the EMA state update,
+    # all bit-exact against the oracle
+    say("fq columns", rows, cols)
+    x = heavy_tailed(rows, cols, rows + cols)
+    x[:, 5] = 0.0
+    x[rows // 2, 7] = np.nan
+    x[:, 16] = np.float32(1e-15)
+    x[rows - 1, cols - 1] = np.float32(-300.0)  # the last element of the tensor is its channel's maximum
+    x[0, 0] = np.float32(250.0)
+    for bits in (8, 4, 2):
+        check_fq(oracle, x, x.shape, 1, bits)
+    got, codes = check_fq(oracle, x, x.shape, 1, 8, round_mode=RoundMode.HalfEven)
+    assert codes[rows - 1, cols - 1] == -127 and codes[0, 0] == 127 and np.isnan(got[rows // 2, 7])
+    state = np.abs(np.random.default_rng(rows).standard_normal(cols)).astype(np.float32) * 0.05
+    state[::5] = 0.0
+    state[3] = -1.0
+    check_fq(oracle, x, x.shape, 1, 8, ScaleMode.EMA, decay=0.99, state=state)
+
+
 def test_fq_idempotent_full_size(oracle):
     # size-independent property: fake-quantizing an already fake-quantized tensor changes nothing
     x = heavy_tailed(8192, 4096, 36)
