@@ -66,12 +66,18 @@ struct FqArgs {
     int parts;
 };
 
-struct GemmArgs {
+constexpr int GEMM_MAX_SEG = 4;
+struct GemmSeg {
     const uint8_t *w;
+    float *out;
+    int n, row_tiles, tile_begin;
+};
+struct GemmArgs {
+    GemmSeg seg[GEMM_MAX_SEG];
+    int nseg;
     const void *xh;
     const void *sxh;
-    float *out;
-    int m_rows, m_out, n, k_pad, units, row_tiles, pair_rows, steps_per_split, use_atomics;
+    int m_rows, m_out, k_pad, units, pair_rows, steps_per_split, use_atomics;
 };
 struct XPrepArgs {
     const void *x;
@@ -279,14 +285,28 @@ static GemmPlan gemm_plan(int scheme, int xk, int64_t m, int64_t k) {
     return p;
 }
 
-// Prefill path: convert the activations once (xprep), then the MFMA GEMM; K is split across workgroups (atomic
-// accumulation into a zeroed output) only when the tile grid alone would leave most CUs idle.
+// Prefill path: convert the activations once (xprep), then the MFMA GEMM over `count` (<= GEMM_MAX_SEG) matrices of one
+// scheme and K that multiply the same x (q, k, v or gate, up of a layer): one launch, their tiles side by side, so
+// a small matrix fills the chip together with its neighbours instead of being cut into slivers of K on its own.
+// K is split across workgroups (atomic accumulation into zeroed outputs) only when the tile grid alone would leave
+// most CUs idle.
 // `prepared`: the workspace already holds this x (same pointer, k, m, dtype, and the block sums if this scheme needs
-// them) from the previous matrix of a batch on the same stream, so the conversion pass is skipped.
-static int launch_gemm(const void *x, int xk, const rlx_qweight *w, float *out, int64_t m, void *workspace,
-                       size_t workspace_bytes, hipStream_t stream, bool prepared = false) {
+// them) from the previous launch of a batch on the same stream, so the conversion pass is skipped.
+static int launch_gemm(const void *x, int xk, const rlx_qweight *const *ws, float *const *outs, int count, int64_t m,
+                       void *workspace, size_t workspace_bytes, hipStream_t stream, bool prepared = false) {
+    const rlx_qweight *w = ws[0];
     const Layout L = w->layout;
     const GemmPlan p = gemm_plan(w->scheme, xk, m, w->dims.k);
+    if (count < 1 || count > GEMM_MAX_SEG) {
+        set_error("gguf_matmul_bt: %d matrices in one prefill launch", count);
+        return RLX_ERR_INVALID;
+    }
+    for (int i = 1; i < count; i++)
+        if (ws[i]->scheme != w->scheme || ws[i]->dims.k != w->dims.k || ws[i]->dims.units != w->dims.units ||
+            ws[i]->layout.unit_bytes != L.unit_bytes) {
+            set_error("gguf_matmul_bt: matrices of one prefill launch differ in scheme or K");
+            return RLX_ERR_INVALID;
+        }
     if (!workspace || workspace_bytes < p.xh_bytes + p.sxh_bytes) {
         set_error("gguf_matmul_bt: m=%lld needs a %zu-byte workspace, got %zu", (long long)m, p.xh_bytes + p.sxh_bytes,
                   workspace_bytes);
@@ -308,19 +328,33 @@ static int launch_gemm(const void *x, int xk, const rlx_qweight *w, float *out, 
     // padding rows); beyond that the 256-row tile.
     const int64_t rv = xk == 0 ? 2 * m : m;
     const bool skinny = rv <= 128;
-    const int gx = (int)((w->dims.row_tiles * 16 + 127) / 128);
+    GemmArgs a{};
+    long long gx = 0;
+    for (int i = 0; i < count; i++) {
+        a.seg[i] = GemmSeg{ws[i]->dev, outs[i], (int)ws[i]->dims.n, (int)ws[i]->dims.row_tiles, (int)gx};
+        gx += (ws[i]->dims.row_tiles * 16 + 127) / 128;
+    }
+    a.nseg = count;
     const int gy = skinny ? (int)((rv + 63) / 64) : (int)(p.m_rows / 256);
     // workgroup slots to fill: one per CU for the 256-row tile (144 KB of LDS), two for the 64-row tile
     const long long slots = (long long)std::max(1, device_props().cu_count) * (skinny ? 2 : 1);
     int split = 1;
-    if ((long long)gx * gy * 5 < slots * 4) split = (int)std::min<long long>(w->dims.units, slots / ((long long)gx * gy));
+    if (gx * gy * 5 < slots * 4) split = (int)std::min<long long>(w->dims.units, slots / (gx * gy));
     split = std::max(1, split);
     int units_per_split = (int)((w->dims.units + split - 1) / split);
     if (steps_per_unit == 2) units_per_split = (units_per_split + 1) & ~1;  // keep every split a multiple of 4 steps
     split = (int)((w->dims.units + units_per_split - 1) / units_per_split);
-    if (split > 1) RLX_TRY(rlx_mi355x_memset_u32(out, 0, (size_t)m * w->dims.n, stream));
-    GemmArgs a{w->dev, xh, sxh, out, (int)p.m_rows, (int)m, (int)w->dims.n, (int)p.k_pad, (int)w->dims.units,
-               (int)w->dims.row_tiles, xk == 0 ? 1 : 0, units_per_split * steps_per_unit, split > 1 ? 1 : 0};
+    if (split > 1)
+        for (int i = 0; i < count; i++) RLX_TRY(rlx_mi355x_memset_u32(outs[i], 0, (size_t)m * ws[i]->dims.n, stream));
+    a.xh = xh;
+    a.sxh = sxh;
+    a.m_rows = (int)p.m_rows;
+    a.m_out = (int)m;
+    a.k_pad = (int)p.k_pad;
+    a.units = (int)w->dims.units;
+    a.pair_rows = xk == 0 ? 1 : 0;
+    a.steps_per_split = units_per_split * steps_per_unit;
+    a.use_atomics = split > 1 ? 1 : 0;
     void *params[] = {&a};
     KernelId id = w->scheme == SCHEME_Q4K       ? (skinny ? K_GEMM64_Q4_K : K_GEMM_Q4_K)
                   : w->scheme == SCHEME_Q4_0    ? (skinny ? K_GEMM64_Q4_0 : K_GEMM_Q4_0)
@@ -466,18 +500,24 @@ int rlx_mi355x_gguf_matmul_bt_batch(const void *const *xs_dev, int x_dtype, cons
     if (m > cap) {  // prefill: one GEMM per weight, sharing the workspace (same stream, so launches are ordered)
         // q, k, v (and gate, up) of a layer share their input: its f16 image in the workspace is made once. An image
         // with block sums (Q4_K / Q5_K) also serves a scheme that does not read them, not the other way round.
+        // Consecutive matrices with the same input and K go into one launch, up to GEMM_MAX_SEG at a time.
         const void *have_x = nullptr;
         int64_t have_k = -1;
         bool have_sums = false;
-        for (int i = 0; i < count; i++) {
+        for (int i = 0; i < count;) {
+            int c = 1;
+            while (i + c < count && c < GEMM_MAX_SEG && xs_dev[i + c] == xs_dev[i] && ws[i + c]->dims.k == ws[i]->dims.k &&
+                   ws[i + c]->layout.unit_bytes == ws[i]->layout.unit_bytes)
+                c++;
             const bool sums = gemm_plan(ws[i]->scheme, xk, m, ws[i]->dims.k).sxh_bytes != 0;
             const bool prepared = xs_dev[i] == have_x && ws[i]->dims.k == have_k && (have_sums || !sums);
-            RLX_TRY(launch_gemm(xs_dev[i], xk, ws[i], outs_dev[i], m, workspace, workspace_bytes, (hipStream_t)stream, prepared));
+            RLX_TRY(launch_gemm(xs_dev[i], xk, ws + i, outs_dev + i, c, m, workspace, workspace_bytes, (hipStream_t)stream, prepared));
             if (!prepared) {
                 have_x = xs_dev[i];
                 have_k = ws[i]->dims.k;
                 have_sums = sums;
             }
+            i += c;
         }
         return RLX_OK;
     }

@@ -19,17 +19,25 @@ constexpr int GEMM_STAGE_A = 4 * 8 * 1024, GEMM_STAGE_B = 4 * 4 * 1024;  // [k-s
 constexpr int GEMM_STAGE = GEMM_STAGE_A + GEMM_STAGE_B;
 constexpr float GEMM_LO_SCALE = 2048.0f;
 
-struct GemmArgs {
+// One launch multiplies one converted input by up to GEMM_MAX_SEG matrices of the same scheme and K (q, k, v or
+// gate, up of a layer): their 128-row tiles are laid side by side along grid.x.
+constexpr int GEMM_MAX_SEG = 4;
+struct GemmSeg {
     const uint8_t *w;
+    float *out;      // [m_out][n]
+    int n;           // logical output columns (rows of W)
+    int row_tiles;   // 16-row tiles of the device layout
+    int tile_begin;  // first blockIdx.x of this matrix
+};
+struct GemmArgs {
+    GemmSeg seg[GEMM_MAX_SEG];
+    int nseg;
     const half_t *xh;   // binary16 activations as LDS stage images: [m_rows / 256][k_pad / 64][32 KB] (see rlx_xprep)
     const half_t *sxh;  // Q4_K: [m_rows][k_pad / 256][16]: per 32-column block sums, 8 x hi then 8 x lo*2048
-    float *out;         // [m_out][n]
     int m_rows;         // rows of xh
     int m_out;          // logical output rows
-    int n;              // logical output columns (rows of W)
     int k_pad;          // padded K
     int units;          // K units of the device layout
-    int row_tiles;      // 16-row tiles of the device layout
     int pair_rows;      // 1: rows 2i, 2i+1 of xh are hi / lo*2048 of logical row i (f32 activations)
     int steps_per_split;  // 64-column steps per grid.z slice (a multiple of 4)
     int use_atomics;      // split K: accumulate into a zeroed `out` with atomic adds
@@ -80,7 +88,13 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WN, wn = wave % WN;
     const int lr = lane & 31, lh = lane >> 5;
-    const int n_tile0 = blockIdx.x * GEMM_NT, m_tile0 = blockIdx.y * MT;
+    int si = 0;  // which matrix of the launch: wave-uniform, so its fields are scalar loads
+#pragma unroll
+    for (int i = 1; i < GEMM_MAX_SEG; i++)
+        if (i < a.nseg && (int)blockIdx.x >= a.seg[i].tile_begin) si = i;
+    const GemmSeg sg = a.seg[si];
+    const int bx = (int)blockIdx.x - sg.tile_begin;
+    const int n_tile0 = bx * GEMM_NT, m_tile0 = blockIdx.y * MT;
     const int step0 = blockIdx.z * a.steps_per_split;
     const int total_steps = a.units * (L.unit_k / GEMM_KS);
     const int step1 = min(step0 + a.steps_per_split, total_steps);
@@ -94,9 +108,9 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
 
     // ---- B loader: thread -> lane slot (n16 = lane % 16, g = lane / 16) of 16-row tile `wave` ---------------
     const int b_n16 = lane & 15, b_g = lane >> 4;
-    const int b_t16 = blockIdx.x * (GEMM_NT / 16) + wave;
-    const bool b_live = b_t16 < a.row_tiles;
-    const uint8_t *b_tile = a.w + (long long)(b_live ? b_t16 : 0) * a.units * L.unit_bytes;
+    const int b_t16 = bx * (GEMM_NT / 16) + wave;
+    const bool b_live = b_t16 < sg.row_tiles;
+    const uint8_t *b_tile = sg.w + (long long)(b_live ? b_t16 : 0) * a.units * L.unit_bytes;
     const uint32_t b_keep = b_live ? 0xFFFFFFFFu : 0u;
     int b_dst[2];  // [block jl of the step]: k-slice 2 jl + g/2, half g%2
     {
@@ -228,8 +242,8 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
 #pragma unroll
     for (int j = 0; j < TJ; j++) {
         my_row[j] = n_tile0 + (wn * TJ + j) * 32 + lr;
-        my_ok[j] = (my_row[j] >> 4) < a.row_tiles;
-        my_meta[j] = a.w + (long long)(my_ok[j] ? (my_row[j] >> 4) : 0) * a.units * L.unit_bytes +
+        my_ok[j] = (my_row[j] >> 4) < sg.row_tiles;
+        my_meta[j] = sg.w + (long long)(my_ok[j] ? (my_row[j] >> 4) : 0) * a.units * L.unit_bytes +
                      (K6 ? 3328 + (my_row[j] & 15) * 2 : META_OFF + (my_row[j] & 15) * 16);  // Q6_K: the row's d; Q4_K / Q5_K: its 16 meta bytes
     }
     uint4_t w_meta[TJ];
@@ -432,7 +446,7 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
 #pragma unroll
         for (int j = 0; j < TJ; j++) {
             const int col = my_row[j];
-            if (col >= a.n) continue;
+            if (col >= sg.n) continue;
 #pragma unroll
             for (int e = 0; e < 16; e++) {
                 const int vrow = m_tile0 + (wm * TI + i) * 32 + 8 * (e >> 2) + 4 * lh + (e & 3);
@@ -444,7 +458,7 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
                     orow = vrow >> 1;
                 }
                 if (orow < a.m_out) {
-                    float *p = a.out + (long long)orow * a.n + col;
+                    float *p = sg.out + (long long)orow * sg.n + col;
                     if (a.use_atomics) atomicAdd(p, v);
                     else __builtin_nontemporal_store(v, p);  // written once, read by another kernel: keep it out of the way of the operands
                 }

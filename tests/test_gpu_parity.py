@@ -441,11 +441,12 @@ def test_graph_batches_independent_matmuls(oracle, m):
 
 @pytest.mark.parametrize("scheme,m,x_dtype", [(Q4K, 40, DType.BF16), (Q4_0, 300, DType.F32), (Q8_0, 130, DType.F16)])
 def test_batched_prefill_shares_the_converted_input(oracle, scheme, m, x_dtype):
-    # q / k / v on one input, then a matrix with its own input and another k, then the first input again: the input's
-    # f16 image is made once per run of matrices that share it, and every output is that of the matmul issued on its own
+    # five matrices on one input (q / k / v and more; ragged N among them), then a matrix with its own input and another
+    # k, then the first input again: the input's f16 image is made once per run of matrices that share it, a run goes
+    # out as launches of up to four matrices side by side, and every output is that of the matmul issued on its own
     say("batched prefill", SCHEME_NAMES[scheme], "m", m, x_dtype.name)
     rng = np.random.default_rng(m)
-    shapes = [(256, 1024, 0), (64, 1024, 0), (48, 1024, 0), (96, 512, 1), (80, 1024, 0)]
+    shapes = [(256, 1024, 0), (64, 1024, 0), (48, 1024, 0), (200, 1024, 0), (136, 1024, 0), (96, 512, 1), (80, 1024, 0)]
     xs_f32 = [rng.standard_normal((m, 1024)).astype(np.float32), rng.standard_normal((m, 512)).astype(np.float32)]
     if x_dtype == DType.BF16:
         xs_in = [f32_to_bf16_bits(oracle.bf16_round(x)) for x in xs_f32]
