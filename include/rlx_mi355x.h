@@ -149,7 +149,9 @@ size_t rlx_mi355x_gguf_matmul_workspace(int scheme, int x_dtype, int64_t m, int6
 /* `count` independent matmuls of one scheme, batch size m and activation dtype in one launch per eight of them:
  * outs_dev[i][m, n_i] = xs_dev[i][m, k_i] . W_i^T. No counterpart in the reference, which runs one thunk per node;
  * the graph level uses it to issue together every DequantMatMul whose inputs are ready at the same point of the
- * schedule (q/k/v and gate/up of a layer share their activations; independent projections need not). */
+ * schedule (q/k/v and gate/up of a layer share their activations; independent projections need not). Above the
+ * decode limit of m, consecutive entries with the same xs_dev[i] and k share one conversion of the input and one
+ * prefill launch per four of them; other entries get a launch of their own. */
 /* A stack of `num_experts` [n, k] matrices, expert outermost, each slab in the GGUF layout of a standalone matrix
  * (rlx-cpu/src/gguf_matmul.rs:98-100); every slab is repacked like a plain weight. */
 int rlx_mi355x_qweight_create_experts(int scheme, const void *gguf_bytes, size_t nbytes, int64_t n, int64_t k,
