@@ -529,6 +529,28 @@ def gemm_configs(rlx_amd, stream):
         tf = 2.0 * 512 * n * k / ms / 1e9
         out[f"q4_k_gemm_m512_{name}"] = {"us": round(ms * 1e3, 2), "TFLOP/s": round(tf, 1),
                                         "frac_mfma_f16": round(tf / MFMA_F16_PEAK_TFLOPS, 4)}
+        if n == 14336:
+            # gate and up as a layer issues them: two matrices on one input through the batched entry point, which
+            # converts the input once and lays their tiles side by side in one launch (448 tiles for 256 CUs)
+            xd = ops.DeviceBuffer.from_numpy(f32_to_bf16_bits(ops.philox_normal(31, 512 * k)))
+            ods = [ops.DeviceBuffer(512 * n * 4) for _ in range(2)]
+            need = ops.matmul_workspace_bytes(qw[0], DType.BF16, 512)
+            wsb = ops.DeviceBuffer(need)
+            C = rlx_amd._lib.C
+            xp = (C.c_void_p * 2)(xd.ptr, xd.ptr)
+            wp = (C.c_void_p * 2)(qw[0].ptr, qw[1].ptr)
+            op = (C.c_void_p * 2)(ods[0].ptr, ods[1].ptr)
+
+            def pair():
+                rlx_amd._lib.check(L.rlx_mi355x_gguf_matmul_bt_batch(xp, int(DType.BF16), wp, op, 2, 512, wsb.ptr, need, stream))
+
+            ms = time_launches(ops, stream, pair, 100, 10)
+            ops.sync(stream)
+            tf = 2 * 2.0 * 512 * n * k / ms / 1e9
+            out["q4_k_gemm_m512_gate+up_pair_one_launch"] = {"us": round(ms * 1e3, 2), "TFLOP/s": round(tf, 1),
+                                                             "frac_mfma_f16": round(tf / MFMA_F16_PEAK_TFLOPS, 4)}
+            for b in [xd, wsb] + ods:
+                b.free()
         for q in qw:
             q.free()
 
