@@ -294,13 +294,13 @@ static GemmPlan gemm_plan(int scheme, int xk, int64_t m, int64_t k) {
 // them) from the previous launch of a batch on the same stream, so the conversion pass is skipped.
 static int launch_gemm(const void *x, int xk, const rlx_qweight *const *ws, float *const *outs, int count, int64_t m,
                        void *workspace, size_t workspace_bytes, hipStream_t stream, bool prepared = false) {
-    const rlx_qweight *w = ws[0];
-    const Layout L = w->layout;
-    const GemmPlan p = gemm_plan(w->scheme, xk, m, w->dims.k);
     if (count < 1 || count > GEMM_MAX_SEG) {
         set_error("gguf_matmul_bt: %d matrices in one prefill launch", count);
         return RLX_ERR_INVALID;
     }
+    const rlx_qweight *w = ws[0];
+    const Layout L = w->layout;
+    const GemmPlan p = gemm_plan(w->scheme, xk, m, w->dims.k);
     for (int i = 1; i < count; i++)
         if (ws[i]->scheme != w->scheme || ws[i]->dims.k != w->dims.k || ws[i]->dims.units != w->dims.units ||
             ws[i]->layout.unit_bytes != L.unit_bytes) {
