@@ -525,7 +525,7 @@ def gemm_configs(rlx_amd, stream):
     # config 3: Q4_K, M = 512, bf16 activations
     for name, n, k in [("gate_up_4096x14336", 14336, 4096), ("down_14336x4096", 4096, 14336)]:
         qw = [tiled_weight(ops, QuantScheme.GgufQ4K, n, k, 41 + i, 0.02) for i in range(2)]
-        ms = run_matmul(qw, 512, k, DType.BF16, 100, 10)
+        ms = run_matmul(qw, 512, k, DType.BF16, 300, 100)
         tf = 2.0 * 512 * n * k / ms / 1e9
         out[f"q4_k_gemm_m512_{name}"] = {"us": round(ms * 1e3, 2), "TFLOP/s": round(tf, 1),
                                         "frac_mfma_f16": round(tf / MFMA_F16_PEAK_TFLOPS, 4)}
@@ -544,7 +544,7 @@ def gemm_configs(rlx_amd, stream):
             def pair():
                 rlx_amd._lib.check(L.rlx_mi355x_gguf_matmul_bt_batch(xp, int(DType.BF16), wp, op, 2, 512, wsb.ptr, need, stream))
 
-            ms = time_launches(ops, stream, pair, 100, 10)
+            ms = time_launches(ops, stream, pair, 200, 60)
             ops.sync(stream)
             tf = 2 * 2.0 * 512 * n * k / ms / 1e9
             out["q4_k_gemm_m512_gate+up_pair_one_launch"] = {"us": round(ms * 1e3, 2), "TFLOP/s": round(tf, 1),
@@ -560,7 +560,7 @@ def gemm_configs(rlx_amd, stream):
     blocks[:, 208:210] = np.full(n * k // 256, 5e-6, np.float16).view(np.uint8).reshape(-1, 2)
     qw = [ops.QWeight(QuantScheme.GgufQ6K, blocks.reshape(-1), n, k) for _ in range(2)]
     del blocks
-    ms = run_matmul(qw, 512, k, DType.BF16, 100, 10)
+    ms = run_matmul(qw, 512, k, DType.BF16, 300, 100)
     tf = 2.0 * 512 * n * k / ms / 1e9
     out["q6_k_gemm_m512_gate_up_4096x14336"] = {"us": round(ms * 1e3, 2), "TFLOP/s": round(tf, 1),
                                                 "frac_mfma_f16": round(tf / MFMA_F16_PEAK_TFLOPS, 4)}
