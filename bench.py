@@ -29,7 +29,7 @@ MFMA_F16_PEAK_TFLOPS = 2500.0  # dense f16/bf16 MFMA peak
 CALIBRATION_COPY_BYTES = 256 << 20
 # HBM bytes per launch of the headline kernel (FETCH_SIZE + WRITE_SIZE of two rocprofv3 --pmc runs of this command,
 # each scaled by the same counter's reading for the copy kernel above); profiles/gemv_q4_0_llama8b_layer_traffic.txt.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 124294239
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 124295417
 
 # (name, N, K) — the Llama-3-8B layer projections of the headline workload
 LLAMA8B = [("q", 4096, 4096), ("k", 1024, 4096), ("v", 1024, 4096), ("o", 4096, 4096),
