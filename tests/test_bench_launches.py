@@ -1,0 +1,174 @@
+"""GPU parity of the very launches bench.py times, at the benchmark's shapes, against the f64 oracle.
+
+* the seven Q4_0 projections of a Llama-3-8B layer as one executable (one batched decode launch; and the
+  transformer-ordered wiring, four dependent launches), f32 activations, every output compared in full;
+* `rlx_mi355x_gguf_matmul_bt_batch` over the seven Q4_0 projections of a Llama-3-70B layer, bf16 activations,
+  M in {1, 4, 16, 64, 256}: column windows at the start, middle and end of every output;
+* FakeQuantize [8192, 4096] feeding a Q8_0 4096 x 4096 matmul through one executable, at full size.
+
+Error norm: |delta| / max(|expected|, 1), as rlx-runtime/tests/dequant_matmul_gguf.rs:231-233; bound 2e-3."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import bench
+import rlx_amd
+from rlx_amd import DType, Graph, Op, QuantScheme, Session, Shape, ops
+from helpers import Q4_0, Q8_0, f32_to_bf16_bits, rel_err
+
+pytestmark = pytest.mark.gpu
+TOL = 2e-3
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+def tiled_packed(scheme, n, k, seed, std, slab_rows=1024):
+    """[n, k] GGUF bytes built from one seeded slab of rows rolled per repetition (a fresh draw's statistics at a
+    fraction of its host time); returned as an [n, bytes_per_row] array."""
+    rng = np.random.default_rng(seed)
+    rows = min(n, slab_rows)
+    slab = ops.quantize(scheme, (rng.standard_normal((rows, k)) * std).astype(np.float32)).reshape(rows, -1)
+    reps = (n + rows - 1) // rows
+    return np.ascontiguousarray(np.concatenate([np.roll(slab, 37 * r + 1, axis=0) for r in range(reps)], axis=0)[:n])
+
+
+# ------------------------------------------------------------------ Llama-3-8B layer, the headline launch
+
+@pytest.fixture(scope="module")
+def llama8b_weights():
+    return {name: tiled_packed(Q4_0, n, k, 100 + i, 0.02) for i, (name, n, k) in enumerate(bench.LLAMA8B)}
+
+
+@pytest.mark.parametrize("capture", [False, True])
+def test_llama8b_layer_one_batched_launch(oracle, llama8b_weights, capture):
+    # exactly what the headline times: the executable bench.build_layer_graph() describes, seven independent f32
+    # activation vectors, one rlx_exec_launch (optionally replayed as a hipGraph); all 47,104 outputs checked
+    c = Session.new(rlx_amd.Device.Mi355x).compile(bench.build_layer_graph(0, "independent"))
+    xs = {}
+    for i, (name, n, k) in enumerate(bench.LLAMA8B):
+        c.set_param_typed(f"w_{name}", llama8b_weights[name].reshape(-1), DType.U8)
+        xs[name] = np.random.default_rng(200 + i).standard_normal(k).astype(np.float32)
+        c.write_input(f"x_{name}", xs[name])
+    c.sync()
+    if capture:
+        c.capture()
+    for rep in range(2 if capture else 1):
+        c.launch()
+        for i, (name, n, k) in enumerate(bench.LLAMA8B):
+            got = c.read_output(i).reshape(1, n)
+            ref = oracle.gguf_matmul_f64(xs[name], llama8b_weights[name].reshape(-1), 1, k, n, Q4_0)
+            err = rel_err(got, ref)
+            say(f"   8B layer launch (capture={capture}, rep {rep}) {name}: max rel err {err:.3e}")
+            assert err <= TOL, name
+
+
+def test_llama8b_layer_dependent_wiring(oracle, llama8b_weights):
+    # the transformer-ordered wiring of the same layer (x -> q,k,v; q -> o; o -> gate,up; gate -> down): four
+    # dependent launches; each matmul is checked against the oracle applied to the activations the device fed it
+    c = Session.new(rlx_amd.Device.Mi355x).compile(bench.build_layer_graph(0, "layer"))
+    for name, n, k in bench.LLAMA8B:
+        c.set_param_typed(f"w_{name}", llama8b_weights[name].reshape(-1), DType.U8)
+    x = np.random.default_rng(300).standard_normal(4096).astype(np.float32)
+    c.write_input("x_attn", x)
+    c.launch()
+    outs = {name: c.read_output(i).reshape(1, n) for i, (name, n, k) in enumerate(bench.LLAMA8B)}
+    feeds = {"q": x, "k": x, "v": x, "o": outs["q"], "gate": outs["o"], "up": outs["o"], "down": outs["gate"]}
+    for name, n, k in bench.LLAMA8B:
+        ref = oracle.gguf_matmul_f64(feeds[name].reshape(-1), llama8b_weights[name].reshape(-1), 1, k, n, Q4_0)
+        err = rel_err(outs[name], ref)
+        say(f"   8B dependent wiring {name}: max rel err {err:.3e}")
+        assert err <= TOL, name
+
+
+# ------------------------------------------------------------------ Llama-3-70B layer, the batch sweep
+
+SHAPES70 = [("q", 8192, 8192), ("k", 1024, 8192), ("v", 1024, 8192), ("o", 8192, 8192),
+            ("gate", 28672, 8192), ("up", 28672, 8192), ("down", 8192, 28672)]
+
+
+@pytest.fixture(scope="module")
+def llama70b():
+    packed = {name: tiled_packed(Q4_0, n, k, 400 + i, 0.015) for i, (name, n, k) in enumerate(SHAPES70)}
+    weights = {name: ops.QWeight(QuantScheme.GgufQ4_0, packed[name].reshape(-1), n, k) for name, n, k in SHAPES70}
+    yield packed, weights
+    for w in weights.values():
+        w.free()
+
+
+@pytest.mark.parametrize("m", [1, 4, 16, 64, 256])
+def test_llama70b_layer_batch_sweep(oracle, llama70b, m):
+    # the call bench.py's sweep times: seven matrices, activations shared per K, one workspace; the decode path issues
+    # the seven as one launch, the prefill path shares the converted input between matrices on the same activations
+    packed, weights = llama70b
+    x_f32 = {k: oracle.bf16_round(np.random.default_rng(500 + m + k).standard_normal((m, k)).astype(np.float32))
+             for k in (8192, 28672)}
+    bufs = {k: ops.DeviceBuffer.from_numpy(f32_to_bf16_bits(v)) for k, v in x_f32.items()}
+    outs = {name: ops.DeviceBuffer(m * n * 4) for name, n, k in SHAPES70}
+    need = max(ops.matmul_workspace_bytes(weights[name], DType.BF16, m) for name, _, _ in SHAPES70)
+    ws = ops.DeviceBuffer(need) if need else None
+    xs_arr = (C.c_void_p * 7)(*[bufs[k].ptr for _, _, k in SHAPES70])
+    ws_arr = (C.c_void_p * 7)(*[weights[name].ptr for name, _, _ in SHAPES70])
+    out_arr = (C.c_void_p * 7)(*[outs[name].ptr for name, _, _ in SHAPES70])
+    L = rlx_amd._lib.lib()
+    for rep in range(2):  # the second call reuses the workspace the first one left behind
+        rlx_amd._lib.check(L.rlx_mi355x_gguf_matmul_bt_batch(xs_arr, int(DType.BF16), ws_arr, out_arr, 7, m,
+                                                             ws.ptr if ws else None, need, None))
+    ops.sync()
+    for name, n, k in SHAPES70:
+        got = outs[name].to_numpy(np.float32).reshape(m, n)
+        assert np.all(np.isfinite(got)), name
+        worst = 0.0
+        for n0 in (0, (n // 2 - 16) & ~7, n - 32):
+            ref = oracle.gguf_matmul_f64(x_f32[k], packed[name].reshape(-1), m, k, n, Q4_0, n0, n0 + 32)
+            worst = max(worst, rel_err(got[:, n0:n0 + 32], ref))
+        say(f"   70B sweep M={m} {name} [{n} x {k}]: max rel err over three 32-column windows {worst:.3e}")
+        assert worst <= TOL, name
+        if m <= 16:  # every output at once: sum over the columns of y against x . (sum of W rows)
+            wsum = np.zeros(k, np.float64)
+            flat = packed[name]
+            for r0 in range(0, n, 2048):
+                r1 = min(n, r0 + 2048)
+                wsum += oracle.dequant(Q4_0, flat[r0:r1].reshape(-1), (r1 - r0) * k).reshape(r1 - r0, k).astype(np.float64).sum(axis=0)
+            want = x_f32[k].astype(np.float64) @ wsum
+            scale = np.maximum(np.abs(want), np.sqrt(n) * 0.5)
+            assert np.max(np.abs(got.astype(np.float64).sum(axis=1) - want) / scale) < 2e-3, name
+    for b in list(bufs.values()) + list(outs.values()) + ([ws] if ws else []):
+        b.free()
+
+
+# ------------------------------------------------------------------ FakeQuantize -> Q8_0 GEMM at full size
+
+def test_config4_chain_full_size(oracle):
+    # benchmark configuration 4 as one executable: FakeQuantize [8192, 4096] (int8, per column) feeding a Q8_0
+    # DequantMatMul against a 4096 x 4096 weight. Codes bit-exact over all 33.5 M elements; y against the f64 oracle
+    # applied to the oracle's fake-quantized tensor, on column windows over all 8192 rows and on a band of rows over
+    # every column.
+    rows, k, n = 8192, 4096, 4096
+    rng = np.random.default_rng(61)
+    x = rng.standard_normal((rows, k)).astype(np.float32)
+    x[rng.random((rows, k)) < 0.001] *= np.float32(20.0)
+    packed = tiled_packed(Q8_0, n, k, 62, 0.02).reshape(-1)
+    g = Graph.new("cfg4_full")
+    xi = g.input("x", Shape.new([rows, k], DType.F32))
+    fq = g.add_node(Op.FakeQuantize(8, 1), [xi], Shape.new([rows, k], DType.F32))
+    w = g.param("w", Shape.new([len(packed)], DType.U8))
+    y = g.add_node(Op.DequantMatMul(QuantScheme.GgufQ8_0), [fq, w], Shape.new([rows, n], DType.F32))
+    g.set_outputs([y, fq])
+    c = Session.new().compile(g)
+    c.set_param_typed("w", packed, DType.U8)
+    y_got, fq_got = c.run([("x", x)])
+    y_got = y_got.reshape(rows, n)
+    fq_ref, codes_ref, _ = oracle.fake_quantize(x, x.shape, 1, 8)
+    assert np.array_equal(fq_got.reshape(rows, k).view(np.uint32), fq_ref.view(np.uint32))
+    assert np.array_equal(c.fq_codes(fq).reshape(rows, k), codes_ref)
+    for n0 in (0, 2040, n - 24):
+        err = rel_err(y_got[:, n0:n0 + 24], oracle.gguf_matmul_f64(fq_ref, packed, rows, k, n, Q8_0, n0, n0 + 24))
+        say(f"   config 4 chain, columns {n0}..{n0 + 24}, all rows: max rel err {err:.3e}")
+        assert err <= TOL
+    for r0 in (0, 4090, rows - 6):
+        err = rel_err(y_got[r0:r0 + 6], oracle.gguf_matmul_f64(fq_ref[r0:r0 + 6], packed, 6, k, n, Q8_0))
+        say(f"   config 4 chain, rows {r0}..{r0 + 6}, all columns: max rel err {err:.3e}")
+        assert err <= TOL
