@@ -69,7 +69,12 @@ def build_layer_graph(li, wiring):
     return g
 
 
-def time_layers(rlx_amd, ops, stream, base, wiring, n_layers, steps, warmup, use_graph):
+SETTLE_LAUNCHES = 400   # untimed layer passes in front of every timed GEMV region, whatever --warmup says: the
+                        # clocks of a fresh box need a few milliseconds of load before they stop moving
+GEMM_SETTLE_CALLS = 100  # the same for the prefill GEMM leg (each call is ~80 us)
+
+
+def time_layers(rlx_amd, ops, stream, base, wiring, n_layers, steps, warmup, use_graph, settle=SETTLE_LAUNCHES):
     """Build n_layers executables (distinct weight bytes), replay them round-robin, return (ms_per_step, layers, xs)."""
     from rlx_amd import DType, Session
 
@@ -96,11 +101,12 @@ def time_layers(rlx_amd, ops, stream, base, wiring, n_layers, steps, warmup, use
     def run_steps(count, offset=0):
         rlx_amd.launch_sequence([layers[(offset + i) % len(layers)] for i in range(count)])
 
-    run_steps(warmup)
+    run_steps(settle)
+    run_steps(warmup, settle)
     ops.sync(stream)
     ev0, ev1 = ops.Event(), ops.Event()
     ev0.record(stream)
-    run_steps(steps, warmup)
+    run_steps(steps, settle + warmup)
     ev1.record(stream)
     ms = ev0.elapsed_ms(ev1)
     ops.sync(stream)
@@ -196,6 +202,8 @@ def main():
         "setup_s": round(setup_s, 1),
     }
 
+    other = "layer" if args.wiring == "independent" else "independent"
+    host_ms = None
     if args.extra:
         # the same layer through the host-buffer boundary (ExecutableGraph::run: seven H2D copies, the launch, seven
         # D2H copies, synchronous) - PCIe and call overhead included, reported beside the headline, never as `value`
@@ -206,20 +214,38 @@ def main():
         for i in range(50):
             layers[i % len(layers)].run(ins)
         host_ms = (time.time() - t1) / 50 * 1e3
-        del layers
+    del layers
+    # the other wiring of the same layer, beside the headline: "layer" is what a decode loop gets (four launches, each
+    # waiting for the one before)
+    ms_o, lay_o, _ = time_layers(rlx_amd, ops, stream, base, other, args.layers, max(args.steps, 200), args.warmup, args.graph)
+    del lay_o
+    result["config"][f"wiring_{other}_ms"] = round(ms_o, 6)
+    result["config"][f"wiring_{other}_GB/s"] = round(layer_bytes / ms_o / 1e6, 1)
+    result["config"][f"wiring_{other}_launches_per_step"] = 1 if other == "independent" else 4
+    result["config"]["settle_launches"] = SETTLE_LAUNCHES
+
+    # ---- second half of the metric: Q4_K prefill GEMM, M = 512, on the Llama-3-8B MLP shapes (bf16 activations)
+    gemm = q4k_gemm_m512(rlx_amd, stream, reps=300)
+    g0 = gemm["gate_up_4096x14336"]
+    result["roofline"]["secondary"] = {
+        "bound": "mfma", "kernel": "rlx_gemm_q4_k", "achieved": g0["TFLOP/s"], "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
+        "frac": round(g0["TFLOP/s"] / MFMA_F16_PEAK_TFLOPS, 4), "flop_per_launch": g0["flop"], "avg_launch_us": g0["us"],
+        "includes": "the rlx_xprep launch that converts the bf16 activations (and, where K is split, the output clear)",
+        "workload": "Q4_K GEMM M=512, 4096 -> 14336 (gate / up), bf16 activations ~N(0,1), weights ~N(0,0.02), f32 out; "
+                    f"{GEMM_SETTLE_CALLS} untimed calls, then {g0['reps']} timed, two weight copies in rotation",
+        "down_14336x4096": {k: gemm["down_14336x4096"][k] for k in ("us", "TFLOP/s", "frac_mfma_f16")},
+        "gate+up_pair_one_call": {k: gemm["gate+up_pair"][k] for k in ("us", "TFLOP/s", "frac_mfma_f16")},
+    }
+
+    if args.extra:
         result["extra"] = extra_configs(rlx_amd, stream)
         result["extra"]["q4_0_gemv_llama8b_layer_host_boundary"] = {
             "ms_per_call": round(host_ms, 4), "GB/s": round(layer_bytes / host_ms / 1e6, 1),
             "note": "rlx_exec_run with host inputs and outputs (H2D + launch + D2H, synchronous)"}
-        other = "layer" if args.wiring == "independent" else "independent"
-        ms_o, lay_o, _ = time_layers(rlx_amd, ops, stream, base, other, args.layers, args.steps, args.warmup, args.graph)
-        result["extra"][f"q4_0_gemv_llama8b_{other}_wiring"] = {
-            "ms_per_step": round(ms_o, 6), "GB/s": round(layer_bytes / ms_o / 1e6, 1),
-            "launches_per_step": 1 if other == "independent" else 4}
-        del lay_o
 
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(base, xs)
+        result["cpu_baseline"]["secondary"] = cpu_baseline_q4k_gemm()
         if args.extra:
             result["extra"]["cpu_baselines"] = cpu_baselines_extra()
     print(json.dumps(result), flush=True)
@@ -497,6 +523,57 @@ def tiled_weight(ops, scheme, n, k, seed, sigma):
     return ops.QWeight(scheme, np.ascontiguousarray(packed).reshape(-1), n, k)
 
 
+def q4k_gemm_m512(rlx_amd, stream, reps=300):
+    """Benchmark configuration 3: Q4_K prefill GEMM, M = 512 bf16 activations, on the Llama-3-8B MLP shapes, through
+    rlx_mi355x_gguf_matmul_bt (one rlx_xprep launch + one GEMM launch per call). Two weight copies in rotation;
+    GEMM_SETTLE_CALLS untimed calls, then `reps` timed ones bracketed by HIP events on the launch stream. Also gate and
+    up as a layer issues them: two matrices on one input through the batched entry point (the input converted once)."""
+    from rlx_amd import DType, QuantScheme, ops
+    L = rlx_amd._lib.lib()
+    C_ = rlx_amd._lib.C
+    out = {}
+    m = 512
+    for name, n, k in [("gate_up_4096x14336", 14336, 4096), ("down_14336x4096", 4096, 14336)]:
+        qw = [tiled_weight(ops, QuantScheme.GgufQ4K, n, k, 41 + i, 0.02) for i in range(2)]
+        xd = ops.DeviceBuffer.from_numpy(f32_to_bf16_bits(ops.philox_normal(31, m * k)))
+        od = ops.DeviceBuffer(m * n * 4)
+        need = ops.matmul_workspace_bytes(qw[0], DType.BF16, m)
+        ws = ops.DeviceBuffer(need)
+        state = {"i": 0}
+
+        def fn():
+            q = qw[state["i"] & 1]
+            state["i"] += 1
+            rlx_amd._lib.check(L.rlx_mi355x_gguf_matmul_bt(xd.ptr, int(DType.BF16), q.ptr, od.ptr, m, ws.ptr, need, stream))
+
+        ms = time_launches(ops, stream, fn, reps, GEMM_SETTLE_CALLS)
+        ops.sync(stream)
+        flop = 2 * m * n * k
+        tf = flop / ms / 1e9
+        out[name] = {"us": round(ms * 1e3, 2), "TFLOP/s": round(tf, 1), "frac_mfma_f16": round(tf / MFMA_F16_PEAK_TFLOPS, 4),
+                     "flop": flop, "reps": reps}
+        if n == 14336:
+            ods = [od, ops.DeviceBuffer(m * n * 4)]
+            xp = (C_.c_void_p * 2)(xd.ptr, xd.ptr)
+            wp = (C_.c_void_p * 2)(qw[0].ptr, qw[1].ptr)
+            op = (C_.c_void_p * 2)(ods[0].ptr, ods[1].ptr)
+
+            def pair():
+                rlx_amd._lib.check(L.rlx_mi355x_gguf_matmul_bt_batch(xp, int(DType.BF16), wp, op, 2, m, ws.ptr, need, stream))
+
+            ms = time_launches(ops, stream, pair, reps // 2, GEMM_SETTLE_CALLS // 2)
+            ops.sync(stream)
+            tf = 2 * flop / ms / 1e9
+            out["gate+up_pair"] = {"us": round(ms * 1e3, 2), "TFLOP/s": round(tf, 1),
+                                   "frac_mfma_f16": round(tf / MFMA_F16_PEAK_TFLOPS, 4)}
+            ods[1].free()
+        for b in [xd, od, ws]:
+            b.free()
+        for q in qw:
+            q.free()
+    return out
+
+
 def gemm_configs(rlx_amd, stream):
     """Prefill GEMM and the batch sweep: Q4_K M=512 on the 8B MLP shapes, FakeQuantize -> Q8_0 GEMM, and the Q4_0
     M sweep over one Llama-3-70B layer. Times include the activation-preparation kernel the GEMM path launches."""
@@ -522,37 +599,7 @@ def gemm_configs(rlx_amd, stream):
         ops.sync(stream)
         return ms
 
-    # config 3: Q4_K, M = 512, bf16 activations
-    for name, n, k in [("gate_up_4096x14336", 14336, 4096), ("down_14336x4096", 4096, 14336)]:
-        qw = [tiled_weight(ops, QuantScheme.GgufQ4K, n, k, 41 + i, 0.02) for i in range(2)]
-        ms = run_matmul(qw, 512, k, DType.BF16, 300, 100)
-        tf = 2.0 * 512 * n * k / ms / 1e9
-        out[f"q4_k_gemm_m512_{name}"] = {"us": round(ms * 1e3, 2), "TFLOP/s": round(tf, 1),
-                                        "frac_mfma_f16": round(tf / MFMA_F16_PEAK_TFLOPS, 4)}
-        if n == 14336:
-            # gate and up as a layer issues them: two matrices on one input through the batched entry point, which
-            # converts the input once and lays their tiles side by side in one launch (448 tiles for 256 CUs)
-            xd = ops.DeviceBuffer.from_numpy(f32_to_bf16_bits(ops.philox_normal(31, 512 * k)))
-            ods = [ops.DeviceBuffer(512 * n * 4) for _ in range(2)]
-            need = ops.matmul_workspace_bytes(qw[0], DType.BF16, 512)
-            wsb = ops.DeviceBuffer(need)
-            C = rlx_amd._lib.C
-            xp = (C.c_void_p * 2)(xd.ptr, xd.ptr)
-            wp = (C.c_void_p * 2)(qw[0].ptr, qw[1].ptr)
-            op = (C.c_void_p * 2)(ods[0].ptr, ods[1].ptr)
-
-            def pair():
-                rlx_amd._lib.check(L.rlx_mi355x_gguf_matmul_bt_batch(xp, int(DType.BF16), wp, op, 2, 512, wsb.ptr, need, stream))
-
-            ms = time_launches(ops, stream, pair, 200, 60)
-            ops.sync(stream)
-            tf = 2 * 2.0 * 512 * n * k / ms / 1e9
-            out["q4_k_gemm_m512_gate+up_pair_one_launch"] = {"us": round(ms * 1e3, 2), "TFLOP/s": round(tf, 1),
-                                                             "frac_mfma_f16": round(tf / MFMA_F16_PEAK_TFLOPS, 4)}
-            for b in [xd, wsb] + ods:
-                b.free()
-        for q in qw:
-            q.free()
+    # config 3: Q4_K, M = 512, bf16 activations: in the default line (roofline.secondary), see q4k_gemm_m512()
 
     # Q6_K, M = 512, gate/up shape, bf16 activations (random code bytes, super-block scales of model-like magnitude)
     n, k = 14336, 4096
@@ -638,6 +685,26 @@ def cpu_baseline(base, xs):
             "host_cpus": os.cpu_count()}
 
 
+def cpu_baseline_q4k_gemm():
+    """The reference CPU path on the Q4_K GEMM M = 512, 4096 -> 14336: a 512-column slice of N (the scalar loop is
+    linear in N), one thread."""
+    import oracle
+    from rlx_amd import QuantScheme, ops
+
+    n, k, m, ncols = 14336, 4096, 512, 512
+    w = (ops.philox_normal(41, ncols * k) * np.float32(0.02)).astype(np.float32)
+    packed = ops.quantize(QuantScheme.GgufQ4K, w)
+    xa = oracle.bf16_round(ops.philox_normal(31, m * k))
+    t0 = time.time()
+    oracle.gguf_matmul_bt(xa, packed, m, k, ncols, oracle.Q4K)
+    dt = time.time() - t0
+    tf = 2.0 * m * ncols * k / dt / 1e12
+    return {"value": round(tf, 6), "unit": "TFLOP/s", "s_full_size_extrapolated": round(dt * n / ncols, 1),
+            "cores": 1, "kind": "port",
+            "sample": f"{ncols} of {n} output columns of the M=512 Q4_K GEMM, {dt:.1f} s, C restatement of rlx-cpu "
+                      f"gguf_matmul_bt (scalar, single thread); full size = this x {n // ncols}"}
+
+
 def cpu_baselines_extra():
     """The reference CPU path (oracle restatement, scalar, one thread) on bounded samples of the other configs."""
     import oracle
@@ -652,18 +719,7 @@ def cpu_baselines_extra():
     dt = time.time() - t0
     out["fake_quantize_8192x4096_cols"] = {"s": round(dt, 3), "GB/s_1R1W": round(2 * rows * cols * 4 / dt / 1e9, 3), "cores": 1,
                                            "kind": "port", "sample": "the whole tensor, one call"}
-    # Q4_K GEMM M = 512, 4096 -> 14336: a 1024-column slice of N, scaled (the loop is linear in N)
-    n, k, m, ncols = 14336, 4096, 512, 1024
-    w = (ops.philox_normal(41, ncols * k) * np.float32(0.02)).astype(np.float32)
-    packed = ops.quantize(QuantScheme.GgufQ4K, w)
-    xa = oracle.bf16_round(ops.philox_normal(31, m * k))
-    t0 = time.time()
-    oracle.gguf_matmul_bt(xa, packed, m, k, ncols, oracle.Q4K)
-    dt = time.time() - t0
-    tf = 2.0 * m * ncols * k / dt / 1e12
-    out["q4_k_gemm_m512_gate_up_4096x14336"] = {"TFLOP/s": round(tf, 6), "s_full_size_extrapolated": round(dt * n / ncols, 1),
-                                                "cores": 1, "kind": "port",
-                                                "sample": f"{ncols} of {n} output columns, {dt:.1f} s, scaled by {n // ncols}"}
+    out["q4_k_gemm_m512_gate_up_4096x14336"] = cpu_baseline_q4k_gemm()
     return out
 
 

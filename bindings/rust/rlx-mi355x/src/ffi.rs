@@ -1,4 +1,4 @@
-//! Raw declarations of `include/rlx_mi355x.h` (ABI version 1). Plain C types only.
+//! Raw declarations of `include/rlx_mi355x.h` (ABI version 2). Plain C types only.
 #![allow(non_camel_case_types)]
 
 use std::os::raw::{c_char, c_int, c_void};
@@ -8,12 +8,14 @@ pub const RLX_ERR_INVALID: c_int = -1;
 pub const RLX_ERR_UNSUPPORTED: c_int = -2;
 pub const RLX_ERR_HIP: c_int = -3;
 pub const RLX_ERR_NO_DEVICE: c_int = -4;
+pub const RLX_ERR_NO_MEMORY: c_int = -5;
 
 pub const RLX_OP_INPUT: u32 = 0;
 pub const RLX_OP_PARAM: u32 = 1;
 pub const RLX_OP_DEQUANT_MATMUL: u32 = 2;
 pub const RLX_OP_FAKE_QUANTIZE: u32 = 3;
 pub const RLX_OP_DEQUANT_GROUPED_MATMUL: u32 = 4;
+pub const RLX_OP_CONSTANT: u32 = 5;
 
 pub const RLX_MAX_RANK: usize = 6;
 pub const RLX_MAX_INPUTS: usize = 3;
@@ -34,6 +36,10 @@ pub struct rlx_node_desc {
     pub scale_mode: u32,
     pub ema_decay: f32,
     pub ste: u32,
+    pub eps: f32,
+    pub flags: u32,
+    pub const_data: *const c_void,
+    pub const_nbytes: u64,
 }
 
 #[repr(C)]
@@ -51,7 +57,9 @@ pub struct rlx_compile_opts {
     pub arena_alignment: u32,
     pub fq_round_mode: u32,
     pub verbose: u32,
-    pub reserved: [u32; 5],
+    pub fq_emit_codes: u32,
+    pub q6k_signed_scales: u32,
+    pub reserved: [u32; 3],
 }
 
 #[repr(C)]

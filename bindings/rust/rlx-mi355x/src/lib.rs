@@ -18,6 +18,8 @@ use std::ffi::{CStr, CString};
 use std::os::raw::c_void;
 
 use rlx_driver::Device;
+use rlx_ir::quant::QuantScheme;
+use rlx_ir::op::SteKind;
 use rlx_ir::{DType, Graph, Node, Op, OpKind, ScaleMode};
 use rlx_runtime::backend::{Backend, ExecutableGraph};
 use rlx_runtime::options::CompileOptions;
@@ -61,6 +63,33 @@ fn dtype_code(d: DType) -> u32 {
     }
 }
 
+/// `rlx_quant_scheme`: the position of the GGUF variants in `QuantScheme`'s declaration (rlx-ir/src/quant.rs:39-79).
+/// `QuantScheme` has data-carrying variants, so it cannot be cast with `as`; anything that is not a claimed GGUF scheme
+/// maps to a value the library refuses at compile ("scheme ... is not claimed").
+fn scheme_code(s: &QuantScheme) -> u32 {
+    match s {
+        QuantScheme::GgufQ4K => 5,
+        QuantScheme::GgufQ5K => 6,
+        QuantScheme::GgufQ6K => 7,
+        QuantScheme::GgufQ8K => 8,
+        QuantScheme::GgufQ2K => 9,
+        QuantScheme::GgufQ3K => 10,
+        QuantScheme::GgufQ4_0 => 11,
+        QuantScheme::GgufQ8_0 => 12,
+        _ => u32::MAX,
+    }
+}
+
+/// `SteKind` (rlx-ir/src/op.rs:121-127); carried for completeness, the forward pass does not read it.
+fn ste_code(s: &SteKind) -> u32 {
+    match s {
+        SteKind::Identity => 0,
+        SteKind::ClippedIdentity => 1,
+        SteKind::Tanh => 2,
+        SteKind::HardTanh => 3,
+    }
+}
+
 fn describe(node: &Node, name: &CString) -> ffi::rlx_node_desc {
     let mut d = ffi::rlx_node_desc {
         op_kind: u32::MAX, // anything the library does not claim; it answers with the legalize message
@@ -69,13 +98,17 @@ fn describe(node: &Node, name: &CString) -> ffi::rlx_node_desc {
         dims: [0; ffi::RLX_MAX_RANK],
         n_inputs: node.inputs.len().min(ffi::RLX_MAX_INPUTS) as u32,
         inputs: [0; ffi::RLX_MAX_INPUTS],
-        name: if node.name.is_some() { name.as_ptr() } else { std::ptr::null() },
+        name: if name.as_bytes().is_empty() { std::ptr::null() } else { name.as_ptr() },
         scheme: 0,
         bits: 0,
         axis: -1,
         scale_mode: 0,
         ema_decay: 0.0,
         ste: 0,
+        eps: 0.0,
+        flags: 0,
+        const_data: std::ptr::null(),
+        const_nbytes: 0,
     };
     assert!(node.shape.rank() <= ffi::RLX_MAX_RANK, "rlx-mi355x: rank above {}", ffi::RLX_MAX_RANK);
     for (i, dim) in node.shape.dims().iter().enumerate() {
@@ -87,19 +120,25 @@ fn describe(node: &Node, name: &CString) -> ffi::rlx_node_desc {
     match &node.op {
         Op::Input { .. } => d.op_kind = ffi::RLX_OP_INPUT,
         Op::Param { .. } => d.op_kind = ffi::RLX_OP_PARAM,
+        Op::Constant { data } => {
+            // the bytes are copied into the arena inside rlx_mi355x_compile; `graph` outlives that call
+            d.op_kind = ffi::RLX_OP_CONSTANT;
+            d.const_data = data.as_ptr() as *const c_void;
+            d.const_nbytes = data.len() as u64;
+        }
         Op::DequantMatMul { scheme } => {
             d.op_kind = ffi::RLX_OP_DEQUANT_MATMUL;
-            d.scheme = *scheme as u32; // declaration order of QuantScheme (rlx-ir/src/quant.rs:39-79)
+            d.scheme = scheme_code(scheme);
         }
         Op::DequantGroupedMatMul { scheme } => {
             d.op_kind = ffi::RLX_OP_DEQUANT_GROUPED_MATMUL; // inputs [x, packed expert stack, expert_idx]
-            d.scheme = *scheme as u32;
+            d.scheme = scheme_code(scheme);
         }
         Op::FakeQuantize { bits, axis, ste, scale_mode } => {
             d.op_kind = ffi::RLX_OP_FAKE_QUANTIZE;
-            d.bits = *bits as u32;
+            d.bits = u32::from(*bits);
             d.axis = axis.map_or(-1, |a| a as i32);
-            d.ste = *ste as u32;
+            d.ste = ste_code(ste);
             match scale_mode {
                 ScaleMode::PerBatch => d.scale_mode = 0,
                 ScaleMode::EMA { decay } => {
@@ -118,8 +157,16 @@ pub struct Mi355xBackend;
 
 impl Backend for Mi355xBackend {
     fn compile(&self, graph: Graph, options: &CompileOptions) -> Box<dyn ExecutableGraph> {
-        let names: Vec<CString> =
-            graph.nodes().iter().map(|n| CString::new(n.name.clone().unwrap_or_default()).unwrap()).collect();
+        // The name set_param / run look up is the one the op carries (`Op::Input { name }`, `Op::Param { name }`,
+        // rlx-ir/src/op.rs:359-367), which is what the reference's executables index by; `Node::name` is a debug label.
+        let names: Vec<CString> = graph
+            .nodes()
+            .iter()
+            .map(|n| match &n.op {
+                Op::Input { name } | Op::Param { name } => CString::new(name.clone()).unwrap(),
+                _ => CString::new(n.name.clone().unwrap_or_default()).unwrap(),
+            })
+            .collect();
         let nodes: Vec<ffi::rlx_node_desc> = graph.nodes().iter().zip(&names).map(|(n, nm)| describe(n, nm)).collect();
         let outputs: Vec<u32> = graph.outputs.iter().map(|id| id.0).collect();
         let gname = CString::new(graph.name.clone()).unwrap();
@@ -141,7 +188,7 @@ impl Backend for Mi355xBackend {
     }
 
     fn supported_ops(&self) -> &'static [OpKind] {
-        &[OpKind::Input, OpKind::Param, OpKind::DequantMatMul, OpKind::DequantGroupedMatMul, OpKind::FakeQuantize]
+        &[OpKind::Input, OpKind::Param, OpKind::Constant, OpKind::DequantMatMul, OpKind::DequantGroupedMatMul, OpKind::FakeQuantize]
     }
 }
 
@@ -212,7 +259,17 @@ impl ExecutableGraph for Mi355xExecutable {
             .collect()
     }
 
-    fn commit_no_wait(&mut self) {
+    /// Encode + commit without waiting (rlx-runtime/src/backend.rs:275-277): every input is written into its arena
+    /// slot on the executable's stream, then the schedule is enqueued behind those copies. Outputs of earlier
+    /// commits are overwritten by later ones, as the trait documents; `sync_pending` drains the stream.
+    fn commit_no_wait(&mut self, inputs: &[(&str, &[f32])]) {
+        for (name, data) in inputs {
+            let n = CString::new(*name).unwrap();
+            let rc = unsafe {
+                ffi::rlx_exec_write_input(self.e, n.as_ptr(), data.as_ptr() as *const c_void, data.len() * 4, dtype_code(DType::F32))
+            };
+            check(rc, "write_input");
+        }
         check(unsafe { ffi::rlx_exec_launch(self.e) }, "launch");
     }
 

@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define RLX_MI355X_ABI_VERSION 1
+#define RLX_MI355X_ABI_VERSION 2
 
 typedef enum rlx_status {
     RLX_OK = 0,
@@ -35,7 +35,8 @@ typedef enum rlx_status {
     RLX_ERR_INVALID = -1,      /* bad argument / shape / size */
     RLX_ERR_UNSUPPORTED = -2,  /* op, scheme or dtype this backend does not claim */
     RLX_ERR_HIP = -3,          /* a HIP call failed; text in last_error */
-    RLX_ERR_NO_DEVICE = -4     /* no gfx950 device / HIP runtime unusable */
+    RLX_ERR_NO_DEVICE = -4,    /* no gfx950 device / HIP runtime unusable */
+    RLX_ERR_NO_MEMORY = -5     /* host or device allocation failed */
 } rlx_status;
 
 /* rlx_ir::DType, declaration order (rlx-ir/src/dtype.rs:20-44). */
@@ -47,10 +48,10 @@ typedef enum rlx_dtype {
 /* rlx_ir::quant::QuantScheme, declaration order (rlx-ir/src/quant.rs:39-79). The eight GGUF schemes the reference's
  * gguf_matmul_bt dispatches (rlx-cpu/src/gguf_matmul.rs:25-37) are claimed; any other value is RLX_ERR_UNSUPPORTED.
  * Q4_K, Q5_K, Q6_K, Q4_0 and Q8_0 stay packed in HBM (same byte count as the GGUF blocks) and have a bit-exact device
- * decoder. Q6_K scale bytes are read as the reference's block decoder reads them, unsigned (rlx-gguf/src/lib.rs:819-845).
+ * decoder. Q6_K scale bytes are read as the reference's block decoder reads them, unsigned (rlx-gguf/src/lib.rs:819-845),
+ * unless the weight is created with RLX_QW_Q6K_SIGNED_SCALES (below).
  * The other three ("wide") are decoded once at upload with the reference's block decoder and kept as binary16 (2 bytes per weight):
- * matmuls only, every decoded weight must fit binary16. With the environment variable RLX_Q6K_SIGNED_SCALES set when a
- * Q6_K weight is uploaded, its scales are read as signed (ggml's reading) and it is kept wide as well. */
+ * matmuls only, every decoded weight must fit binary16. */
 typedef enum rlx_quant_scheme {
     RLX_SCHEME_GGUF_Q4K = 5,  /* 256 elems / 144 bytes */
     RLX_SCHEME_GGUF_Q5K = 6,  /* 256 / 176 */
@@ -118,6 +119,12 @@ int64_t rlx_mi355x_bytes_for(int scheme, int64_t n_elems); /* rlx_gguf bytes_for
  * 16-byte lane slots hold MFMA operand fragments; wide schemes: binary16 fragments, 2 bytes per weight). */
 typedef struct rlx_qweight rlx_qweight;
 
+/* Per-weight options. RLX_QW_Q6K_SIGNED_SCALES: read the sixteen scale bytes of a Q6_K super-block as signed, which is
+ * what ggml writes and what the reference's whole-tensor decoder reads (rlx-gguf/src/lib.rs:1070-1112); without it they
+ * are read as unsigned, as the block decoder the reference's matmul calls does (lib.rs:819-845). Both readings stay packed
+ * and use the same kernels. Fixed when the weight is created; ignored for other schemes. */
+typedef enum rlx_qweight_flags { RLX_QW_Q6K_SIGNED_SCALES = 1 } rlx_qweight_flags;
+
 /* Repack `gguf_bytes` (host, exactly bytes_for(scheme, n*k) long) and upload. Where the reference memcpy's the
  * bytes into the arena (`set_param_bytes`, rlx-runtime/src/backend.rs:1175-1187). */
 int rlx_mi355x_qweight_create(int scheme, const void *gguf_bytes, size_t nbytes, int64_t n, int64_t k,
@@ -125,15 +132,22 @@ int rlx_mi355x_qweight_create(int scheme, const void *gguf_bytes, size_t nbytes,
 /* Same, into caller-owned device memory of rlx_mi355x_qweight_device_bytes_for() bytes (256-byte aligned). */
 int rlx_mi355x_qweight_create_at(int scheme, const void *gguf_bytes, size_t nbytes, int64_t n, int64_t k,
                                  void *device_mem, rlx_qweight **out);
+/* The general form the four above forward to: `num_experts` stacked [n, k] matrices (1 = a plain weight), rlx_qweight_flags,
+ * and, when `device_mem` is given, the bytes available there (refused when the device layout needs more). Every argument
+ * is checked before anything is allocated; a failed allocation is RLX_ERR_NO_MEMORY, never an exception. */
+int rlx_mi355x_qweight_create_ex(int scheme, uint32_t flags, const void *gguf_bytes, size_t nbytes, int64_t n, int64_t k,
+                                 int64_t num_experts, void *device_mem, size_t device_capacity, rlx_qweight **out);
 void rlx_mi355x_qweight_destroy(rlx_qweight *w);
 size_t rlx_mi355x_qweight_device_bytes(const rlx_qweight *w);
 size_t rlx_mi355x_qweight_device_bytes_for(int scheme, int64_t n, int64_t k);
 /* Host-side repack only (no device): writes device-layout bytes to `out` (size from ..._device_bytes_for). */
 int rlx_mi355x_repack_host(int scheme, const void *gguf_bytes, size_t nbytes, int64_t n, int64_t k, void *out);
+int rlx_mi355x_repack_host_ex(int scheme, uint32_t flags, const void *gguf_bytes, size_t nbytes, int64_t n, int64_t k, void *out);
 
 /* rlx_gguf::dequant_q8_0 / dequant_q4_0 / dequant_q4_k (rlx-gguf/src/lib.rs:600-633,974-1013) on the device:
  * out_dev[n*k] f32, row-major [n,k], bit-identical to the reference decoders (also Q5_K; Q6_K: to dequant_q6_k_block, the
- * one the matmul calls). RLX_ERR_UNSUPPORTED for the wide schemes (the exact f32 decode is not kept on the device). */
+ * one the matmul calls, or to dequant_q6_k for a weight created with RLX_QW_Q6K_SIGNED_SCALES). RLX_ERR_UNSUPPORTED for the
+ * wide schemes (the exact f32 decode is not kept on the device). */
 int rlx_mi355x_dequant(const rlx_qweight *w, float *out_dev, void *stream);
 
 /* rlx_cpu::gguf_matmul::gguf_matmul_bt (rlx-cpu/src/gguf_matmul.rs:40-95):
@@ -251,8 +265,10 @@ typedef enum rlx_op_kind {
     RLX_OP_PARAM = 1,          /* OpKind::Param  */
     RLX_OP_DEQUANT_MATMUL = 2, /* OpKind::DequantMatMul, Op::DequantMatMul{scheme} (rlx-ir/src/op.rs:736-752) */
     RLX_OP_FAKE_QUANTIZE = 3,  /* OpKind::FakeQuantize,  Op::FakeQuantize{bits,axis,ste,scale_mode} (op.rs:407-432) */
-    RLX_OP_DEQUANT_GROUPED_MATMUL = 4 /* OpKind::DequantGroupedMatMul, Op::DequantGroupedMatMul{scheme} (op.rs:862-871):
-                                       * inputs [x [m,k], packed expert stack, expert_idx [m] F32] -> [m,n] */
+    RLX_OP_DEQUANT_GROUPED_MATMUL = 4, /* OpKind::DequantGroupedMatMul, Op::DequantGroupedMatMul{scheme} (op.rs:862-871):
+                                        * inputs [x [m,k], packed expert stack, expert_idx [m] F32] -> [m,n] */
+    RLX_OP_CONSTANT = 5        /* OpKind::Constant, Op::Constant{data} (op.rs:369-372): const_data / const_nbytes are copied
+                                * into the arena at compile; a U8 constant feeding a DequantMatMul is repacked there */
 } rlx_op_kind;
 
 #define RLX_MAX_RANK 6
@@ -275,6 +291,12 @@ typedef struct rlx_node_desc {
     uint32_t scale_mode;              /* rlx_scale_mode; EMA / FIXED take a second input: state [chan_dim] */
     float ema_decay;
     uint32_t ste;                     /* SteKind; forward-only backend: carried, not used */
+    /* reserved for op kinds with an epsilon / boolean attribute */
+    float eps;
+    uint32_t flags;
+    /* Constant: the embedded bytes (read during rlx_mi355x_compile only) */
+    const void *const_data;
+    uint64_t const_nbytes;
 } rlx_node_desc;
 
 typedef struct rlx_graph_desc {
@@ -290,12 +312,16 @@ typedef struct rlx_compile_opts {
     uint32_t arena_alignment; /* bytes, power of two; 0 = 256 */
     uint32_t fq_round_mode;   /* rlx_round_mode for every FakeQuantize node */
     uint32_t verbose;         /* RLX_VERBOSE-style plan dump to stderr */
-    uint32_t reserved[5];
+    uint32_t fq_emit_codes;   /* 1: every FakeQuantize node also keeps its int8 codes for rlx_exec_read_fq_codes (one more
+                               * byte per element written and resident); 0 (default): the codes are not materialised */
+    uint32_t q6k_signed_scales; /* 1: the Q6_K weights of this graph are read with RLX_QW_Q6K_SIGNED_SCALES (ggml's
+                                 * reading); 0 (default): unsigned, as the reference's matmul reads them */
+    uint32_t reserved[3];
 } rlx_compile_opts;
 
 typedef struct rlx_exec rlx_exec; /* Box<dyn ExecutableGraph>: Send, not Sync — one thread at a time */
 
-/* Backend::supported_ops(): the op kinds this backend lowers. Returns the count. */
+/* Backend::supported_ops(): the op kinds this backend lowers (rlx_op_kind values). Returns the count. */
 size_t rlx_mi355x_supported_ops(const uint32_t **kinds);
 
 /* Backend::compile(graph, options): validates (legalize: unsupported op / scheme / dtype -> NULL with the
@@ -303,6 +329,10 @@ size_t rlx_mi355x_supported_ops(const uint32_t **kinds);
  * (rlx-cpu/src/thunk.rs:3027-3043, 2567-2598), plans the arena and allocates it. NULL on failure. */
 rlx_exec *rlx_mi355x_compile(const rlx_graph_desc *graph, const rlx_compile_opts *opts);
 void rlx_exec_destroy(rlx_exec *e);
+/* The device-free part of compile: validation, lowering, schedule and memory plan (what rlx-compile's plan_memory
+ * does before a backend allocates, rlx-compile/src/memory.rs:386-470). Returns the arena size in bytes, or a negative
+ * rlx_status with the same error text compile would give; `buf` (may be NULL) receives the plan as text. Needs no GPU. */
+int64_t rlx_mi355x_plan(const rlx_graph_desc *graph, const rlx_compile_opts *opts, char *buf, size_t cap);
 
 /* ExecutableGraph::set_param(name, &[f32]). */
 int rlx_exec_set_param(rlx_exec *e, const char *name, const float *data, size_t n);
@@ -355,7 +385,8 @@ int rlx_mi355x_launch_sequence(rlx_exec *const *execs, size_t n);
  * including the persistent repacked-weight slots. Writes a short text table. */
 size_t rlx_exec_arena_bytes(const rlx_exec *e);
 int rlx_exec_describe_plan(const rlx_exec *e, char *buf, size_t cap);
-/* FakeQuantize node's integer codes from the last run (int8, len elements), by output index; for parity checks. */
+/* FakeQuantize node's integer codes from the last run (int8, len elements), by node id; for parity checks. Needs
+ * rlx_compile_opts.fq_emit_codes. */
 int rlx_exec_read_fq_codes(rlx_exec *e, uint32_t node_id, int8_t *codes, size_t n);
 
 #ifdef __cplusplus

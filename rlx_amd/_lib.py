@@ -22,7 +22,8 @@ class NodeDesc(C.Structure):
     _fields_ = [("op_kind", C.c_uint32), ("dtype", C.c_uint32), ("rank", C.c_uint32),
                 ("dims", C.c_int64 * RLX_MAX_RANK), ("n_inputs", C.c_uint32), ("inputs", C.c_uint32 * RLX_MAX_INPUTS),
                 ("name", C.c_char_p), ("scheme", C.c_uint32), ("bits", C.c_uint32), ("axis", C.c_int32),
-                ("scale_mode", C.c_uint32), ("ema_decay", C.c_float), ("ste", C.c_uint32)]
+                ("scale_mode", C.c_uint32), ("ema_decay", C.c_float), ("ste", C.c_uint32),
+                ("eps", C.c_float), ("flags", C.c_uint32), ("const_data", C.c_void_p), ("const_nbytes", C.c_uint64)]
 
 
 class GraphDesc(C.Structure):
@@ -32,7 +33,7 @@ class GraphDesc(C.Structure):
 
 class CompileOpts(C.Structure):
     _fields_ = [("arena_alignment", C.c_uint32), ("fq_round_mode", C.c_uint32), ("verbose", C.c_uint32),
-                ("reserved", C.c_uint32 * 5)]
+                ("fq_emit_codes", C.c_uint32), ("q6k_signed_scales", C.c_uint32), ("reserved", C.c_uint32 * 3)]
 
 
 class NamedBuf(C.Structure):
@@ -70,6 +71,8 @@ SIGNATURES = {
     "rlx_mi355x_bytes_for": (_i64, [_i, _i64]),
     "rlx_mi355x_qweight_create": (_i, [_i, _vp, _sz, _i64, _i64, _pvp]),
     "rlx_mi355x_qweight_create_at": (_i, [_i, _vp, _sz, _i64, _i64, _vp, _pvp]),
+    "rlx_mi355x_qweight_create_ex": (_i, [_i, _u32, _vp, _sz, _i64, _i64, _i64, _vp, _sz, _pvp]),
+    "rlx_mi355x_repack_host_ex": (_i, [_i, _u32, _vp, _sz, _i64, _i64, _vp]),
     "rlx_mi355x_qweight_destroy": (None, [_vp]),
     "rlx_mi355x_qweight_device_bytes": (_sz, [_vp]),
     "rlx_mi355x_qweight_device_bytes_for": (_sz, [_i, _i64, _i64]),
@@ -98,6 +101,7 @@ SIGNATURES = {
     "rlx_mi355x_philox_normal": (None, [C.c_uint64, _vp, _i64]),
     "rlx_mi355x_supported_ops": (_sz, [C.POINTER(C.POINTER(_u32))]),
     "rlx_mi355x_compile": (_vp, [C.POINTER(GraphDesc), C.POINTER(CompileOpts)]),
+    "rlx_mi355x_plan": (_i64, [C.POINTER(GraphDesc), C.POINTER(CompileOpts), C.c_char_p, _sz]),
     "rlx_exec_destroy": (None, [_vp]),
     "rlx_exec_set_param": (_i, [_vp, C.c_char_p, _vp, _sz]),
     "rlx_exec_set_param_typed": (_i, [_vp, C.c_char_p, _vp, _sz, _u32]),

@@ -19,9 +19,8 @@ extern "C" int rlx_mi355x_gguf_matmul_bt(const void *, int, const rlx_qweight *,
 extern "C" size_t rlx_mi355x_gguf_matmul_workspace(int, int, int64_t, int64_t, int64_t);
 extern "C" int rlx_mi355x_fake_quantize(const float *, float *, int8_t *, int64_t, int64_t, int64_t, int, int, float, float *, int,
                                         void *, void *);
-extern "C" int rlx_mi355x_qweight_create_at(int, const void *, size_t, int64_t, int64_t, void *, rlx_qweight **);
 extern "C" void rlx_mi355x_qweight_destroy(rlx_qweight *);
-extern "C" int rlx_mi355x_qweight_create_experts_at(int, const void *, size_t, int64_t, int64_t, int64_t, void *, rlx_qweight **);
+extern "C" int rlx_mi355x_qweight_create_ex(int, uint32_t, const void *, size_t, int64_t, int64_t, int64_t, void *, size_t, rlx_qweight **);
 extern "C" int rlx_mi355x_gguf_grouped_matmul_bt(const void *, int, const rlx_qweight *, const float *, float *, int64_t, void *);
 extern "C" int rlx_mi355x_gguf_matmul_bt_batch(const void *const *, int, const rlx_qweight *const *, float *const *, int, int64_t,
                                                void *, size_t, void *);
@@ -31,7 +30,8 @@ namespace {
 using namespace rlx;
 
 const uint32_t kSupportedOps[] = {RLX_OP_INPUT, RLX_OP_PARAM, RLX_OP_DEQUANT_MATMUL, RLX_OP_FAKE_QUANTIZE,
-                                 RLX_OP_DEQUANT_GROUPED_MATMUL};
+                                 RLX_OP_DEQUANT_GROUPED_MATMUL, RLX_OP_CONSTANT};
+constexpr uint32_t kMaxOpKind = RLX_OP_CONSTANT;
 const char *op_name(uint32_t k) {
     switch (k) {
     case RLX_OP_INPUT: return "Input";
@@ -39,6 +39,7 @@ const char *op_name(uint32_t k) {
     case RLX_OP_DEQUANT_MATMUL: return "DequantMatMul";
     case RLX_OP_DEQUANT_GROUPED_MATMUL: return "DequantGroupedMatMul";
     case RLX_OP_FAKE_QUANTIZE: return "FakeQuantize";
+    case RLX_OP_CONSTANT: return "Constant";
     default: return "?";
     }
 }
@@ -57,13 +58,16 @@ struct Slot {
     size_t offset = 0, size = 0;
 };
 
+// A value without producer inside the graph: lives in the arena for the executable's whole life.
+inline bool is_source(uint32_t kind) { return kind == RLX_OP_INPUT || kind == RLX_OP_PARAM || kind == RLX_OP_CONSTANT; }
+
 struct Node {
     rlx_node_desc d;
     std::string name;
     int64_t numel = 0;
     Slot slot;          // the node's value
-    Slot aux;           // FakeQuantize: maxima + scales; DequantMatMul: workspace
-    Slot codes;         // FakeQuantize: int8 codes
+    Slot aux;           // FakeQuantize: maxima + scales; first DequantMatMul of a prefill step: the step's workspace
+    Slot codes;         // FakeQuantize: int8 codes (only with rlx_compile_opts.fq_emit_codes)
     uint32_t cur_dtype = RLX_F32;  // dtype of the bytes currently in an Input slot
     // DequantMatMul
     int64_t m = 0, k = 0, n = 0;
@@ -74,6 +78,7 @@ struct Node {
     int scheme = 0;
     int64_t w_n = 0, w_k = 0, w_experts = 1;
     rlx_qweight *qw = nullptr;
+    uint32_t w_flags = 0;  // rlx_qweight_flags the weight is created with
 };
 
 // f32 <-> half / bfloat16 as the reference's typed boundary does (rlx-driver/src/arena.rs:69-119, `half` crate).
@@ -100,6 +105,8 @@ float bf16_to_f32(uint16_t h) {
 }
 
 }  // namespace
+
+extern "C" int rlx_exec_describe_plan(const rlx_exec *e, char *buf, size_t cap);
 
 struct rlx_exec {
     std::string name;
@@ -142,7 +149,10 @@ size_t rlx_mi355x_supported_ops(const uint32_t **kinds) {
     return sizeof kSupportedOps / sizeof kSupportedOps[0];
 }
 
-rlx_exec *rlx_mi355x_compile(const rlx_graph_desc *g, const rlx_compile_opts *opts) {
+}  // extern "C"
+
+// Everything of Backend::compile that needs no device: validation, lowering, schedule, memory plan.
+static std::unique_ptr<rlx_exec> plan_graph(const rlx_graph_desc *g, const rlx_compile_opts *opts) {
     clear_error();
     if (!g || !g->nodes || g->n_nodes == 0 || !g->outputs || g->n_outputs == 0) {
         set_error("compile: empty graph or no outputs");
@@ -163,7 +173,7 @@ rlx_exec *rlx_mi355x_compile(const rlx_graph_desc *g, const rlx_compile_opts *op
     int n_bad = 0;
     for (uint32_t i = 0; i < g->n_nodes; i++) {
         uint32_t k = g->nodes[i].op_kind;
-        if (k > RLX_OP_DEQUANT_GROUPED_MATMUL) {
+        if (k > kMaxOpKind) {
             n_bad++;
             bad += "\n  - node " + std::to_string(i) + ": op kind " + std::to_string(k);
         }
@@ -225,6 +235,13 @@ rlx_exec *rlx_mi355x_compile(const rlx_graph_desc *g, const rlx_compile_opts *op
         case RLX_OP_PARAM:
             e->params[nd.name] = i;
             break;
+        case RLX_OP_CONSTANT:
+            if (!nd.d.const_data || nd.d.const_nbytes != (uint64_t)nd.numel * dtype_size(nd.d.dtype)) {
+                set_error("compile: constant node %u carries %llu bytes, its shape needs %llu", i,
+                          (unsigned long long)nd.d.const_nbytes, (unsigned long long)nd.numel * dtype_size(nd.d.dtype));
+                return nullptr;
+            }
+            break;
         case RLX_OP_DEQUANT_MATMUL: {
             if (layout_of((int)nd.d.scheme).block_elems == 0) {
                 set_error("compile: node %u: DequantMatMul scheme %u is not claimed (GGUF Q4_K=5 .. Q3_K=10, Q4_0=11, Q8_0=12)", i,
@@ -248,9 +265,9 @@ rlx_exec *rlx_mi355x_compile(const rlx_graph_desc *g, const rlx_compile_opts *op
             }
             Layout L = layout_of((int)nd.d.scheme);
             int64_t want = (nd.k * nd.n) % L.block_elems == 0 ? nd.k * nd.n / L.block_elems * L.block_bytes : -1;
-            if (w.d.op_kind != RLX_OP_PARAM || (w.d.dtype != RLX_U8 && w.d.dtype != RLX_I8) || w.numel != want ||
-                nd.k % L.block_elems != 0) {
-                set_error("compile: node %u: packed weight must be a U8 param of %lld bytes ([n=%lld, k=%lld], k %% %d == 0); "
+            if ((w.d.op_kind != RLX_OP_PARAM && w.d.op_kind != RLX_OP_CONSTANT) || (w.d.dtype != RLX_U8 && w.d.dtype != RLX_I8) ||
+                w.numel != want || nd.k % L.block_elems != 0) {
+                set_error("compile: node %u: packed weight must be a U8 param or constant of %lld bytes ([n=%lld, k=%lld], k %% %d == 0); "
                           "got %lld elements of dtype %u",
                           i, (long long)want, (long long)nd.n, (long long)nd.k, L.block_elems, (long long)w.numel, w.d.dtype);
                 return nullptr;
@@ -293,8 +310,8 @@ rlx_exec *rlx_mi355x_compile(const rlx_graph_desc *g, const rlx_compile_opts *op
             }
             const int64_t slab = (nd.k * nd.n) % L.block_elems == 0 && nd.k % L.block_elems == 0
                                      ? nd.k * nd.n / L.block_elems * L.block_bytes : -1;
-            if (w.d.op_kind != RLX_OP_PARAM || (w.d.dtype != RLX_U8 && w.d.dtype != RLX_I8) || slab <= 0 || w.numel < slab ||
-                w.numel % slab != 0) {
+            if ((w.d.op_kind != RLX_OP_PARAM && w.d.op_kind != RLX_OP_CONSTANT) || (w.d.dtype != RLX_U8 && w.d.dtype != RLX_I8) ||
+                slab <= 0 || w.numel < slab || w.numel % slab != 0) {
                 set_error("compile: node %u: packed experts must be a U8 param of E x %lld bytes ([n=%lld, k=%lld] per expert); got %lld",
                           i, (long long)slab, (long long)nd.n, (long long)nd.k, (long long)w.numel);
                 return nullptr;
@@ -359,7 +376,7 @@ rlx_exec *rlx_mi355x_compile(const rlx_graph_desc *g, const rlx_compile_opts *op
     std::vector<int> depth(e->nodes.size(), 0);
     for (uint32_t i = 0; i < g->n_nodes; i++) {
         Node &nd = e->nodes[i];
-        if (nd.d.op_kind == RLX_OP_INPUT || nd.d.op_kind == RLX_OP_PARAM) continue;
+        if (is_source(nd.d.op_kind)) continue;
         int dmax = 0;
         for (uint32_t j = 0; j < nd.d.n_inputs; j++) dmax = std::max(dmax, depth[nd.d.inputs[j]]);
         depth[i] = dmax + 1;
@@ -377,7 +394,7 @@ rlx_exec *rlx_mi355x_compile(const rlx_graph_desc *g, const rlx_compile_opts *op
                 Node &o = e->nodes[j];
                 if (!grouped[j] && o.d.op_kind == RLX_OP_DEQUANT_MATMUL && depth[j] == depth[i] &&
                     o.d.scheme == nd.d.scheme && o.m == nd.m && e->nodes[o.d.inputs[0]].d.dtype == xdt &&
-                    (o.d.inputs[0] < i || e->nodes[o.d.inputs[0]].d.op_kind == RLX_OP_INPUT)) {
+                    (o.d.inputs[0] < i || is_source(e->nodes[o.d.inputs[0]].d.op_kind))) {
                     grouped[j] = true;
                     step.push_back(j);
                 }
@@ -386,33 +403,98 @@ rlx_exec *rlx_mi355x_compile(const rlx_graph_desc *g, const rlx_compile_opts *op
         e->steps.push_back(step);
     }
 
-    // Memory plan.
-    size_t off = 0;
-    auto take = [&](size_t bytes) {
+    // Memory plan: one arena. Sources (inputs, params, constants), graph outputs and requested FakeQuantize codes
+    // live for the whole run; every other buffer lives from the step that writes it to the last step that reads it
+    // (a prefill workspace: its own step only), and a buffer may take the bytes of one that is dead by then:
+    // greedy first fit in step order, the contract of rlx-compile's planner (rlx-compile/src/memory.rs:386-470).
+    // Steps run one after another on one stream, also inside a captured graph, so reuse needs no further ordering.
+    const int kForever = 1 << 30;
+    std::vector<int> step_of(e->nodes.size(), 0), last_use(e->nodes.size(), 0);
+    for (size_t si = 0; si < e->steps.size(); si++)
+        for (uint32_t id : e->steps[si]) step_of[id] = (int)si;
+    for (uint32_t i = 0; i < g->n_nodes; i++) {
+        const Node &nd = e->nodes[i];
+        last_use[i] = std::max(last_use[i], step_of[i]);
+        if (is_source(nd.d.op_kind)) continue;
+        for (uint32_t j = 0; j < nd.d.n_inputs; j++) last_use[nd.d.inputs[j]] = std::max(last_use[nd.d.inputs[j]], step_of[i]);
+    }
+    for (uint32_t id : e->outputs) last_use[id] = kForever;
+    struct Placed {
+        size_t off, size;
+        int birth, death;
+    };
+    std::vector<Placed> placed;
+    size_t arena_end = 0;
+    auto take = [&](size_t bytes, int birth, int death) {
+        const size_t size = (std::max<size_t>(bytes, 1) + align - 1) & ~(align - 1);
+        std::vector<size_t> cand{0};
+        for (const Placed &p : placed) cand.push_back(p.off + p.size);
+        std::sort(cand.begin(), cand.end());
+        size_t best = (size_t)-1;
+        for (size_t c : cand) {
+            bool clash = false;
+            for (const Placed &p : placed)
+                if (c < p.off + p.size && c + size > p.off && birth <= p.death && death >= p.birth) {
+                    clash = true;
+                    break;
+                }
+            if (!clash) {
+                best = c;
+                break;
+            }
+        }
+        placed.push_back(Placed{best, size, birth, death});
+        arena_end = std::max(arena_end, best + size);
         Slot s;
-        s.offset = off;
+        s.offset = best;
         s.size = bytes;
-        off = (off + std::max<size_t>(bytes, 1) + align - 1) & ~(align - 1);
         return s;
     };
-    for (Node &nd : e->nodes) {
+    const uint32_t wflags = e->opts.q6k_signed_scales ? (uint32_t)RLX_QW_Q6K_SIGNED_SCALES : 0u;
+    for (Node &nd : e->nodes) {  // whole-life buffers first, so the reusable ones pack above them
+        if (!is_source(nd.d.op_kind)) continue;
         if (nd.is_packed) {
-            nd.slot = take((size_t)weight_dims(host_layout(nd.scheme), nd.w_n, nd.w_k).bytes * (size_t)nd.w_experts);  // device layout, resident
+            nd.w_flags = nd.scheme == SCHEME_Q6K ? wflags : 0u;
+            nd.slot = take((size_t)weight_dims(host_layout(nd.scheme), nd.w_n, nd.w_k).bytes * (size_t)nd.w_experts, 0, kForever);  // device layout, resident
         } else if (nd.d.op_kind == RLX_OP_INPUT) {
-            nd.slot = take((size_t)nd.numel * 4);  // room for an f32 upload even when declared 16-bit
+            nd.slot = take((size_t)nd.numel * 4, 0, kForever);  // room for an f32 upload even when declared 16-bit
             nd.cur_dtype = nd.d.dtype;
         } else {
-            nd.slot = take((size_t)nd.numel * dtype_size(nd.d.dtype));
+            nd.slot = take((size_t)nd.numel * dtype_size(nd.d.dtype), 0, kForever);
         }
-        if (nd.d.op_kind == RLX_OP_FAKE_QUANTIZE) {
-            nd.aux = take(rlx_mi355x_fake_quantize_scratch_bytes(nd.numel, nd.chan_dim, nd.inner));
-            nd.codes = take((size_t)nd.numel);
-        }
-        if (nd.d.op_kind == RLX_OP_DEQUANT_MATMUL && nd.m > 16)  // beyond the decode kernels for any input dtype: prefill workspace, sized for f32
-            nd.aux = take(rlx_mi355x_gguf_matmul_workspace((int)nd.d.scheme, RLX_F32, nd.m, nd.k, nd.n));
     }
-    e->arena_bytes = off;
+    for (size_t si = 0; si < e->steps.size(); si++) {
+        const std::vector<uint32_t> &step = e->steps[si];
+        size_t step_ws = 0;
+        for (uint32_t id : step) {
+            Node &nd = e->nodes[id];
+            nd.slot = take((size_t)nd.numel * dtype_size(nd.d.dtype), (int)si, last_use[id]);
+            if (nd.d.op_kind == RLX_OP_FAKE_QUANTIZE) {
+                nd.aux = take(rlx_mi355x_fake_quantize_scratch_bytes(nd.numel, nd.chan_dim, nd.inner), (int)si, (int)si);
+                if (e->opts.fq_emit_codes) nd.codes = take((size_t)nd.numel, (int)si, kForever);
+            }
+            if (nd.d.op_kind == RLX_OP_DEQUANT_MATMUL && nd.m > 16)  // may run the prefill kernels (which one is decided by the input dtype at run time): sized for f32
+                step_ws = std::max(step_ws, rlx_mi355x_gguf_matmul_workspace((int)nd.d.scheme, RLX_F32, nd.m, nd.k, nd.n));
+        }
+        if (step_ws) e->nodes[step[0]].aux = take(step_ws, (int)si, (int)si);  // one workspace for the whole step
+    }
+    e->arena_bytes = arena_end;
+    return e;
+}
 
+extern "C" {
+
+int64_t rlx_mi355x_plan(const rlx_graph_desc *g, const rlx_compile_opts *opts, char *buf, size_t cap) {
+    std::unique_ptr<rlx_exec> e = plan_graph(g, opts);
+    if (!e) return RLX_ERR_INVALID;
+    if (buf && cap) RLX_TRY(rlx_exec_describe_plan(e.get(), buf, cap));
+    return (int64_t)e->arena_bytes;
+}
+
+rlx_exec *rlx_mi355x_compile(const rlx_graph_desc *g, const rlx_compile_opts *opts) {
+    std::unique_ptr<rlx_exec> e = plan_graph(g, opts);
+    if (!e) return nullptr;
+    const size_t off = e->arena_bytes;
     if (runtime_init() != RLX_OK) return nullptr;
     if (hipMalloc((void **)&e->arena, std::max<size_t>(off, 256)) != hipSuccess) {
         set_error("compile: hipMalloc(%zu) for the arena failed", off);
@@ -423,6 +505,18 @@ rlx_exec *rlx_mi355x_compile(const rlx_graph_desc *g, const rlx_compile_opts *op
         return nullptr;
     }
     e->stream = e->own_stream;
+    for (Node &nd : e->nodes) {  // constants: their bytes go in now; a packed one is repacked like a param at set_param_typed
+        if (nd.d.op_kind != RLX_OP_CONSTANT) continue;
+        if (nd.is_packed) {
+            if (rlx_mi355x_qweight_create_ex(nd.scheme, nd.w_flags, nd.d.const_data, (size_t)nd.d.const_nbytes, nd.w_n, nd.w_k, nd.w_experts,
+                                             e->ptr(nd.slot), nd.slot.size, &nd.qw) < 0)
+                return nullptr;
+        } else if (hipMemcpy(e->ptr(nd.slot), nd.d.const_data, (size_t)nd.d.const_nbytes, hipMemcpyHostToDevice) != hipSuccess) {
+            set_error("compile: upload of constant node failed");
+            return nullptr;
+        }
+        nd.d.const_data = nullptr;  // the caller's bytes are not referenced after compile
+    }
     if (e->opts.verbose) {
         char buf[4096];
         rlx_exec_describe_plan(e.get(), buf, sizeof buf);
@@ -448,10 +542,8 @@ int rlx_exec_set_param_typed(rlx_exec *e, const char *name, const void *data, si
                 rlx_mi355x_qweight_destroy(nd.qw);
                 nd.qw = nullptr;
             }
-            if (nd.w_experts > 1)
-                return rlx_mi355x_qweight_create_experts_at(nd.scheme, data, nbytes, nd.w_n, nd.w_k, nd.w_experts, e->ptr(nd.slot),
-                                                            &nd.qw);
-            return rlx_mi355x_qweight_create_at(nd.scheme, data, nbytes, nd.w_n, nd.w_k, e->ptr(nd.slot), &nd.qw);
+            return rlx_mi355x_qweight_create_ex(nd.scheme, nd.w_flags, data, nbytes, nd.w_n, nd.w_k, nd.w_experts, e->ptr(nd.slot),
+                                                nd.slot.size, &nd.qw);
         }
         if (nbytes > nd.slot.size) {
             set_error("set_param_typed: '%s' holds %zu bytes, got %zu", name, nd.slot.size, nbytes);
@@ -538,8 +630,29 @@ static int enqueue_schedule(rlx_exec *e) {
             }
             RLX_TRY(rlx_mi355x_gguf_grouped_matmul_bt(e->ptr(x.slot), (int)dt, w.qw, (const float *)e->ptr(idx.slot),
                                                       (float *)e->ptr(nd.slot), nd.m, e->stream));
-        } else if (nd.d.op_kind == RLX_OP_DEQUANT_MATMUL && nd.m > 16) {
-            for (uint32_t id : step) {  // prefill: one GEMM per node, each with its own workspace slot
+        } else if (nd.d.op_kind == RLX_OP_DEQUANT_MATMUL) {
+            // The whole step through the batched entry point: up to 16 / 32 rows it issues one decode launch per eight
+            // matrices; above that, matrices that share their input (q, k, v; gate, up) share one conversion of it and
+            // one prefill launch per four, all on the step's single workspace. Matrices on the same input are made
+            // neighbours first (stable, so the order among them is the graph's).
+            std::vector<uint32_t> order(step);
+            std::stable_sort(order.begin(), order.end(), [&](uint32_t a, uint32_t b) {
+                return e->nodes[a].d.inputs[0] < e->nodes[b].d.inputs[0];
+            });
+            std::vector<const rlx_qweight *> ws;
+            std::vector<float *> outs;
+            std::vector<const void *> xs;
+            uint32_t xdt = RLX_F32;
+            auto flush = [&]() -> int {
+                if (ws.empty()) return RLX_OK;
+                int rc = rlx_mi355x_gguf_matmul_bt_batch(xs.data(), (int)xdt, ws.data(), outs.data(), (int)ws.size(), nd.m,
+                                                         nd.aux.size ? e->ptr(nd.aux) : nullptr, nd.aux.size, e->stream);
+                ws.clear();
+                outs.clear();
+                xs.clear();
+                return rc;
+            };
+            for (uint32_t id : order) {
                 Node &mm = e->nodes[id];
                 Node &x = e->nodes[mm.d.inputs[0]];
                 Node &w = e->nodes[mm.d.inputs[1]];
@@ -548,37 +661,13 @@ static int enqueue_schedule(rlx_exec *e) {
                     return RLX_ERR_INVALID;
                 }
                 uint32_t dt = x.d.op_kind == RLX_OP_INPUT ? x.cur_dtype : x.d.dtype;
-                RLX_TRY(rlx_mi355x_gguf_matmul_bt(e->ptr(x.slot), (int)dt, w.qw, (float *)e->ptr(mm.slot), mm.m, e->ptr(mm.aux),
-                                                  mm.aux.size, e->stream));
-            }
-        } else if (nd.d.op_kind == RLX_OP_DEQUANT_MATMUL) {
-            std::vector<const rlx_qweight *> ws;
-            std::vector<float *> outs;
-            std::vector<const void *> xs;
-            uint32_t xdt = RLX_F32;
-            for (size_t si = 0; si < step.size(); si++) {
-                Node &mm = e->nodes[step[si]];
-                Node &x = e->nodes[mm.d.inputs[0]];
-                Node &w = e->nodes[mm.d.inputs[1]];
-                if (!w.qw) {
-                    set_error("run: packed weight '%s' was never set (set_param_typed(.., U8))", w.name.c_str());
-                    return RLX_ERR_INVALID;
-                }
-                uint32_t dt = x.d.op_kind == RLX_OP_INPUT ? x.cur_dtype : x.d.dtype;
-                if (si > 0 && dt != xdt) {  // inputs of one batch were written with different dtypes: flush and start anew
-                    RLX_TRY(rlx_mi355x_gguf_matmul_bt_batch(xs.data(), (int)xdt, ws.data(), outs.data(), (int)ws.size(), nd.m,
-                                                            nullptr, 0, e->stream));
-                    ws.clear();
-                    outs.clear();
-                    xs.clear();
-                }
+                if (!ws.empty() && dt != xdt) RLX_TRY(flush());  // inputs of one step were written with different dtypes
                 xdt = dt;
                 ws.push_back(w.qw);
                 outs.push_back((float *)e->ptr(mm.slot));
                 xs.push_back(e->ptr(x.slot));
             }
-            RLX_TRY(rlx_mi355x_gguf_matmul_bt_batch(xs.data(), (int)xdt, ws.data(), outs.data(), (int)ws.size(), nd.m, nullptr,
-                                                    0, e->stream));
+            RLX_TRY(flush());
         } else {
             Node &x = e->nodes[nd.d.inputs[0]];
             if (x.d.op_kind == RLX_OP_INPUT && x.cur_dtype != RLX_F32) {
@@ -587,7 +676,7 @@ static int enqueue_schedule(rlx_exec *e) {
             }
             float *state = nd.d.n_inputs == 2 ? (float *)e->ptr(e->nodes[nd.d.inputs[1]].slot) : nullptr;
             RLX_TRY(rlx_mi355x_fake_quantize((const float *)e->ptr(x.slot), (float *)e->ptr(nd.slot),
-                                             (int8_t *)e->ptr(nd.codes), nd.numel, nd.chan_dim, nd.inner, (int)nd.d.bits,
+                                             nd.codes.size ? (int8_t *)e->ptr(nd.codes) : nullptr, nd.numel, nd.chan_dim, nd.inner, (int)nd.d.bits,
                                              (int)nd.d.scale_mode, nd.d.ema_decay, state, (int)e->opts.fq_round_mode,
                                              e->ptr(nd.aux), e->stream));
         }
@@ -731,7 +820,9 @@ int rlx_exec_describe_plan(const rlx_exec *e, char *buf, size_t cap) {
         if (nd.is_packed) put(" [device layout, scheme %d, n=%lld k=%lld]", nd.scheme, (long long)nd.w_n, (long long)nd.w_k);
         if (nd.d.op_kind == RLX_OP_DEQUANT_MATMUL) put(" m=%lld k=%lld n=%lld", (long long)nd.m, (long long)nd.k, (long long)nd.n);
         if (nd.d.op_kind == RLX_OP_FAKE_QUANTIZE)
-            put(" chan_dim=%lld inner=%lld aux@%zu codes@%zu", (long long)nd.chan_dim, (long long)nd.inner, nd.aux.offset, nd.codes.offset);
+            put(" chan_dim=%lld inner=%lld aux@%zu codes@%zu+%zu", (long long)nd.chan_dim, (long long)nd.inner, nd.aux.offset, nd.codes.offset,
+                nd.codes.size);
+        if (nd.d.op_kind == RLX_OP_DEQUANT_MATMUL && nd.aux.size) put(" step workspace@%zu+%zu", nd.aux.offset, nd.aux.size);
         put("\n");
     }
     return RLX_OK;
@@ -743,6 +834,10 @@ int rlx_exec_read_fq_codes(rlx_exec *e, uint32_t node_id, int8_t *codes, size_t 
         return RLX_ERR_INVALID;
     }
     Node &nd = e->nodes[node_id];
+    if (nd.codes.size == 0) {
+        set_error("read_fq_codes: the executable was compiled without rlx_compile_opts.fq_emit_codes");
+        return RLX_ERR_INVALID;
+    }
     if (n != (size_t)nd.numel) {
         set_error("read_fq_codes: node has %lld elements, buffer %zu", (long long)nd.numel, n);
         return RLX_ERR_INVALID;

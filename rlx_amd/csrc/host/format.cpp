@@ -51,52 +51,7 @@ static inline float f16_bits_to_f32(uint16_t h) {
 // Element-indexed restatements of the reference's super-block decoders, same f32 operation order, used once per weight
 // at upload. `i` is the element's position in the 256-element super-block.
 
-static inline void k4_scale_min(int j, const uint8_t *q, uint8_t *sc, uint8_t *mn) {  // rlx-gguf/src/lib.rs:743-751
-    if (j < 4) {
-        *sc = q[j] & 63;
-        *mn = q[j + 4] & 63;
-    } else {
-        *sc = (uint8_t)((q[j + 4] & 0x0F) | ((q[j - 4] >> 6) << 4));
-        *mn = (uint8_t)((q[j + 4] >> 4) | ((q[j] >> 6) << 4));
-    }
-}
-
 static inline float f16_at(const uint8_t *p) { return f16_bits_to_f32((uint16_t)(p[0] | (p[1] << 8))); }
-
-// Q5_K (lib.rs:783-816): d, dmin, 12 scale bytes, 32 bytes of fifth bits, 128 bytes of nibbles.
-static void decode_q5_k(const uint8_t *b, float *out) {
-    const float d = f16_at(b), dmin = f16_at(b + 2);
-    const uint8_t *scales = b + 4, *qh = b + 16, *qs = b + 48;
-    for (int j = 0; j < 8; j++) {
-        uint8_t sc, mn;
-        k4_scale_min(j, scales, &sc, &mn);
-        const float dj = d * (float)sc, mj = dmin * (float)mn;
-        for (int l = 0; l < 32; l++) {
-            const uint8_t byte = qs[32 * (j >> 1) + l];
-            const int lo = (j & 1) ? (byte >> 4) : (byte & 0x0F);
-            const int hi = (qh[l] >> j) & 1 ? 16 : 0;
-            out[32 * j + l] = dj * (float)(lo + hi) - mj;
-        }
-    }
-}
-
-// Q6_K (lib.rs:819-845): 128 bytes of low nibbles, 64 bytes of high bit pairs, 16 scale bytes, d. The reference's block
-// decoder, the one its matmul calls, converts the scale bytes as unsigned; its whole-tensor decoder (lib.rs:1070-1112)
-// and upstream ggml read them as signed. `signed_scales` selects the latter.
-static void decode_q6_k(const uint8_t *b, float *out, bool signed_scales) {
-    const uint8_t *ql = b, *qh = b + 128, *sc = b + 192;
-    const float d = f16_at(b + 208);
-    for (int i = 0; i < 256; i++) {
-        const int h = i >> 7, quarter = (i >> 5) & 3, l = i & 31;
-        const uint8_t lowbyte = ql[64 * h + 32 * (quarter & 1) + l];
-        const int low = (quarter >> 1) ? (lowbyte >> 4) : (lowbyte & 0x0F);
-        const int high = (qh[32 * h + l] >> (2 * quarter)) & 3;
-        const int q = (low | (high << 4)) - 32;
-        const uint8_t sbyte = sc[8 * h + 2 * quarter + (l >> 4)];
-        const float s = signed_scales ? (float)(int8_t)sbyte : (float)sbyte;
-        out[i] = d * s * (float)q;
-    }
-}
 
 // Q8_K (lib.rs:848-854): f32 d, 256 signed bytes (the 16 block sums that follow are not read).
 static void decode_q8_k(const uint8_t *b, float *out) {
@@ -137,20 +92,10 @@ static void decode_q3_k(const uint8_t *b, float *out) {
     }
 }
 
-Layout host_layout(int scheme) {
-    if (scheme == SCHEME_Q6K && getenv("RLX_Q6K_SIGNED_SCALES") != nullptr) return wide_layout_of(scheme);
-    return layout_of(scheme);
-}
-
-static bool q6k_signed_scales() {
-    static const bool v = getenv("RLX_Q6K_SIGNED_SCALES") != nullptr;
-    return v;
-}
+Layout host_layout(int scheme) { return layout_of(scheme); }
 
 static void decode_wide_block(int scheme, const uint8_t *b, float *out) {
     switch (scheme) {
-    case SCHEME_Q5K: decode_q5_k(b, out); break;
-    case SCHEME_Q6K: decode_q6_k(b, out, q6k_signed_scales()); break;
     case SCHEME_Q8K: decode_q8_k(b, out); break;
     case SCHEME_Q2K: decode_q2_k(b, out); break;
     default: decode_q3_k(b, out); break;
@@ -193,8 +138,10 @@ static int repack_wide(int scheme, const uint8_t *src, int64_t n, int64_t k, uin
 
 // ---- repack ---------------------------------------------------------------------------------------------
 
-int repack_host(int scheme, const uint8_t *src, size_t nbytes, int64_t n, int64_t k, uint8_t *out) {
+int repack_host(int scheme, uint32_t flags, const uint8_t *src, size_t nbytes, int64_t n, int64_t k, uint8_t *out) {
     Layout L = host_layout(scheme);
+    // Q6_K scale bytes read as signed are stored XOR 0x80 (offset binary): the kernels subtract 128 from the byte
+    const uint8_t q6_flip = (flags & RLX_QW_Q6K_SIGNED_SCALES) ? 0x80u : 0u;
     if (L.unit_k == 0 || L.block_elems == 0) {
         set_error("repack: scheme %d is not a claimed GGUF scheme (Q4_K=5, Q5_K=6, Q6_K=7, Q8_K=8, Q2_K=9, Q3_K=10, Q4_0=11, Q8_0=12)", scheme);
         return RLX_ERR_UNSUPPORTED;
@@ -268,13 +215,9 @@ int repack_host(int scheme, const uint8_t *src, size_t nbytes, int64_t n, int64_
                     const bool live = r < n && u < bpr;
                     const uint8_t *b = live ? src + (r * bpr + u) * L.block_bytes : nullptr;
                     if (g == 0) {
-                        if (live) {
-                            memcpy(unit + 3072 + nrow * 16, b + 192, 16);
-                            memcpy(unit + 3328 + nrow * 2, b + 208, 2);
-                        } else {
-                            memset(unit + 3072 + nrow * 16, 0, 16);
-                            memset(unit + 3328 + nrow * 2, 0, 2);
-                        }
+                        for (int e = 0; e < 16; e++) unit[3072 + nrow * 16 + e] = (uint8_t)((live ? b[192 + e] : 0) ^ q6_flip);
+                        if (live) memcpy(unit + 3328 + nrow * 2, b + 208, 2);
+                        else memset(unit + 3328 + nrow * 2, 0, 2);
                     }
                     uint32_t hw[4] = {0, 0, 0, 0};
                     for (int j = 0; j < 8; j++) {
@@ -454,7 +397,10 @@ size_t rlx_mi355x_qweight_device_bytes_for(int scheme, int64_t n, int64_t k) {
 }
 
 int rlx_mi355x_repack_host(int scheme, const void *gguf_bytes, size_t nbytes, int64_t n, int64_t k, void *out) {
-    return rlx::repack_host(scheme, (const uint8_t *)gguf_bytes, nbytes, n, k, (uint8_t *)out);
+    return rlx::repack_host(scheme, 0, (const uint8_t *)gguf_bytes, nbytes, n, k, (uint8_t *)out);
+}
+int rlx_mi355x_repack_host_ex(int scheme, uint32_t flags, const void *gguf_bytes, size_t nbytes, int64_t n, int64_t k, void *out) {
+    return rlx::repack_host(scheme, flags, (const uint8_t *)gguf_bytes, nbytes, n, k, (uint8_t *)out);
 }
 
 int rlx_mi355x_quantize(int scheme, const float *src, int64_t n_elems, void *out) {

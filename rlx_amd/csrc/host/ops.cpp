@@ -6,8 +6,10 @@
 
 #include "common.hpp"
 
+#include <new>
+
 namespace rlx {
-int repack_host(int scheme, const uint8_t *src, size_t nbytes, int64_t n, int64_t k, uint8_t *out);
+int repack_host(int scheme, uint32_t flags, const uint8_t *src, size_t nbytes, int64_t n, int64_t k, uint8_t *out);
 }
 
 struct rlx_qweight {
@@ -17,6 +19,8 @@ struct rlx_qweight {
     uint8_t *dev;
     bool owns;
     int experts;           // matrices stacked dims.bytes apart (1 for a plain weight)
+    uint32_t flags;        // rlx_qweight_flags it was created with
+    int sc_off() const { return (flags & RLX_QW_Q6K_SIGNED_SCALES) ? 128 : 0; }
 };
 
 namespace rlx {
@@ -26,6 +30,7 @@ struct DequantArgs {
     const uint8_t *w;
     float *out;
     long long n, k, units;
+    int sc_off;
 };
 constexpr int GEMV_MAX_SEG = 8;
 struct GemvSeg {
@@ -47,6 +52,7 @@ struct GemvArgs {
     float eps;
     int lds_bytes;
     int kw;
+    int sc_off;
 };
 struct RmsNorm {  // RMSNorm prologue of a decode launch (f32 activations only)
     const float *gamma, *beta;
@@ -77,7 +83,7 @@ struct GemmArgs {
     int nseg;
     const void *xh;
     const void *sxh;
-    int m_rows, m_out, k_pad, units, pair_rows, steps_per_split, use_atomics;
+    int m_rows, m_out, k_pad, units, pair_rows, steps_per_split, use_atomics, sc_off;
 };
 struct XPrepArgs {
     const void *x;
@@ -109,11 +115,16 @@ static int launch_gemv(const void *const *xs, int xk, const rlx_qweight *const *
     const int scheme = ws[0]->scheme;
     const Layout L = ws[0]->layout;
     const bool wide = layout_is_f16w(L);
-    for (int i = 0; i < count; i++)
+    for (int i = 0; i < count; i++) {
         if ((uintptr_t)xs[i] % 16 != 0) {
             set_error("gguf_matmul_bt: activations must be 16-byte aligned");
             return RLX_ERR_INVALID;
         }
+        if (ws[i]->sc_off() != ws[0]->sc_off() || (pairs && pairs[i]->sc_off() != ws[0]->sc_off())) {
+            set_error("gguf_matmul_bt: the Q6_K weights of one launch must share one reading of their scale bytes");
+            return RLX_ERR_INVALID;
+        }
+    }
     const int rv = xk == 0 ? 2 * m : m;
     const int ng = (rv + 3) / 4;
     const bool r2 = rv <= 2;
@@ -220,6 +231,7 @@ static int launch_gemv(const void *const *xs, int xk, const rlx_qweight *const *
         sh.a.kw = kw;
         sh.a.slab_bytes = ws[0]->dims.bytes;
         sh.a.num_experts = ws[0]->experts;
+        sh.a.sc_off = ws[0]->sc_off();
         return sh;
     };
     // Two workgroups of 8 waves per CU with 80 KB each: holds a 14336-wide f32 vector (hi + lo rows) in one chunk.
@@ -303,7 +315,7 @@ static int launch_gemm(const void *x, int xk, const rlx_qweight *const *ws, floa
     const GemmPlan p = gemm_plan(w->scheme, xk, m, w->dims.k);
     for (int i = 1; i < count; i++)
         if (ws[i]->scheme != w->scheme || ws[i]->dims.k != w->dims.k || ws[i]->dims.units != w->dims.units ||
-            ws[i]->layout.unit_bytes != L.unit_bytes) {
+            ws[i]->layout.unit_bytes != L.unit_bytes || ws[i]->sc_off() != w->sc_off()) {
             set_error("gguf_matmul_bt: matrices of one prefill launch differ in scheme or K");
             return RLX_ERR_INVALID;
         }
@@ -355,6 +367,7 @@ static int launch_gemm(const void *x, int xk, const rlx_qweight *const *ws, floa
     a.pair_rows = xk == 0 ? 1 : 0;
     a.steps_per_split = units_per_split * steps_per_unit;
     a.use_atomics = split > 1 ? 1 : 0;
+    a.sc_off = w->sc_off();
     void *params[] = {&a};
     KernelId id = w->scheme == SCHEME_Q4K       ? (skinny ? K_GEMM64_Q4_K : K_GEMM_Q4_K)
                   : w->scheme == SCHEME_Q4_0    ? (skinny ? K_GEMM64_Q4_0 : K_GEMM_Q4_0)
@@ -371,70 +384,94 @@ static int launch_gemm(const void *x, int xk, const rlx_qweight *const *ws, floa
 
 extern "C" {
 
-int rlx_mi355x_qweight_create_at(int scheme, const void *gguf_bytes, size_t nbytes, int64_t n, int64_t k,
-                                 void *device_mem, rlx_qweight **out) {
+// One or `num_experts` [n, k] matrices: validate, repack on the host, upload into `device_mem` (or fresh memory).
+int rlx_mi355x_qweight_create_ex(int scheme, uint32_t flags, const void *gguf_bytes, size_t nbytes, int64_t n, int64_t k,
+                                 int64_t num_experts, void *device_mem, size_t device_capacity, rlx_qweight **out) {
     using namespace rlx;
-    RLX_TRY(runtime_init());
+    if (!gguf_bytes || !out) {
+        set_error("qweight: null argument");
+        return RLX_ERR_INVALID;
+    }
+    *out = nullptr;
     const Layout HL = host_layout(scheme);
-    WeightDims D = weight_dims(HL, n, k);
-    std::vector<uint8_t> staging;
-    if (D.bytes == 0 || HL.block_elems == 0) {
+    if (HL.unit_k == 0 || HL.block_elems == 0) {
         set_error("qweight: scheme %d is not a claimed GGUF scheme", scheme);
         return RLX_ERR_UNSUPPORTED;
     }
-    staging.resize((size_t)D.bytes);
-    RLX_TRY(repack_host(scheme, (const uint8_t *)gguf_bytes, nbytes, n, k, staging.data()));
-    bool owns = device_mem == nullptr;
-    if (owns) RLX_HIP(hipMalloc(&device_mem, (size_t)D.bytes));
-    hipError_t e = hipMemcpy(device_mem, staging.data(), (size_t)D.bytes, hipMemcpyHostToDevice);
-    if (e != hipSuccess) {
-        if (owns) (void)hipFree(device_mem);
-        set_error("qweight upload: %s", hipGetErrorString(e));
-        return RLX_ERR_HIP;
+    if (flags & ~(uint32_t)RLX_QW_Q6K_SIGNED_SCALES) {
+        set_error("qweight: unknown flags 0x%x", flags);
+        return RLX_ERR_INVALID;
     }
-    *out = new rlx_qweight{scheme, HL, D, (uint8_t *)device_mem, owns, 1};
+    if (n <= 0 || k <= 0 || k % HL.block_elems != 0 || num_experts < 1 || num_experts > 0x7FFFFFFF) {
+        set_error("qweight: need n > 0, k a positive multiple of %d and 1 <= experts; got n=%lld k=%lld experts=%lld", HL.block_elems,
+                  (long long)n, (long long)k, (long long)num_experts);
+        return RLX_ERR_INVALID;
+    }
+    const int64_t slab = rlx_mi355x_bytes_for(scheme, n * k);
+    if (slab < 0 || nbytes != (size_t)slab * (size_t)num_experts) {
+        set_error("qweight: got %zu bytes, %lld x [%lld x %lld] needs %lld", nbytes, (long long)num_experts, (long long)n, (long long)k,
+                  (long long)(slab < 0 ? -1 : slab * num_experts));
+        return RLX_ERR_INVALID;
+    }
+    const WeightDims D = weight_dims(HL, n, k);
+    const size_t total = (size_t)D.bytes * (size_t)num_experts;
+    if (device_mem && device_capacity < total) {
+        set_error("qweight: the device layout takes %zu bytes, the slot holds %zu", total, device_capacity);
+        return RLX_ERR_INVALID;
+    }
+    RLX_TRY(runtime_init());
+    bool owns = false;
+    rlx_qweight *qw = nullptr;
+    try {
+        std::vector<uint8_t> staging(total);
+        for (int64_t e = 0; e < num_experts; e++)
+            RLX_TRY(repack_host(scheme, flags, (const uint8_t *)gguf_bytes + e * slab, (size_t)slab, n, k, staging.data() + e * D.bytes));
+        qw = new rlx_qweight{scheme, HL, D, nullptr, false, (int)num_experts, flags};
+        if (!device_mem) {
+            hipError_t me = hipMalloc(&device_mem, total);
+            if (me != hipSuccess) {
+                delete qw;
+                set_error("qweight: hipMalloc(%zu) failed: %s", total, hipGetErrorString(me));
+                return me == hipErrorOutOfMemory ? RLX_ERR_NO_MEMORY : RLX_ERR_HIP;
+            }
+            owns = true;
+        }
+        hipError_t e = hipMemcpy(device_mem, staging.data(), total, hipMemcpyHostToDevice);
+        if (e != hipSuccess) {
+            if (owns) (void)hipFree(device_mem);
+            delete qw;
+            set_error("qweight upload: %s", hipGetErrorString(e));
+            return RLX_ERR_HIP;
+        }
+    } catch (const std::bad_alloc &) {
+        delete qw;
+        set_error("qweight: out of host memory staging %zu bytes", total);
+        return RLX_ERR_NO_MEMORY;
+    }
+    qw->dev = (uint8_t *)device_mem;
+    qw->owns = owns;
+    *out = qw;
     return RLX_OK;
+}
+
+int rlx_mi355x_qweight_create_at(int scheme, const void *gguf_bytes, size_t nbytes, int64_t n, int64_t k,
+                                 void *device_mem, rlx_qweight **out) {
+    return rlx_mi355x_qweight_create_ex(scheme, 0, gguf_bytes, nbytes, n, k, 1, device_mem, device_mem ? (size_t)-1 : 0, out);
 }
 
 int rlx_mi355x_qweight_create(int scheme, const void *gguf_bytes, size_t nbytes, int64_t n, int64_t k,
                               rlx_qweight **out) {
-    return rlx_mi355x_qweight_create_at(scheme, gguf_bytes, nbytes, n, k, nullptr, out);
+    return rlx_mi355x_qweight_create_ex(scheme, 0, gguf_bytes, nbytes, n, k, 1, nullptr, 0, out);
 }
 
 int rlx_mi355x_qweight_create_experts_at(int scheme, const void *gguf_bytes, size_t nbytes, int64_t n, int64_t k,
                                          int64_t num_experts, void *device_mem, rlx_qweight **out) {
-    using namespace rlx;
-    RLX_TRY(runtime_init());
-    const Layout HL = host_layout(scheme);
-    WeightDims D = weight_dims(HL, n, k);
-    if (D.bytes == 0 || HL.block_elems == 0) {
-        set_error("qweight: scheme %d is not a claimed GGUF scheme", scheme);
-        return RLX_ERR_UNSUPPORTED;
-    }
-    const int64_t slab = rlx_mi355x_bytes_for(scheme, n * k);
-    if (num_experts < 1 || num_experts > 0x7FFFFFFF || slab < 0 || nbytes != (size_t)(slab * num_experts)) {
-        set_error("qweight: got %zu bytes, %lld experts of [%lld x %lld] need %lld", nbytes, (long long)num_experts, (long long)n,
-                  (long long)k, (long long)(slab < 0 ? -1 : slab * num_experts));
-        return RLX_ERR_INVALID;
-    }
-    std::vector<uint8_t> staging((size_t)D.bytes * (size_t)num_experts);
-    for (int64_t e = 0; e < num_experts; e++)
-        RLX_TRY(repack_host(scheme, (const uint8_t *)gguf_bytes + e * slab, (size_t)slab, n, k, staging.data() + e * D.bytes));
-    bool owns = device_mem == nullptr;
-    if (owns) RLX_HIP(hipMalloc(&device_mem, staging.size()));
-    hipError_t err = hipMemcpy(device_mem, staging.data(), staging.size(), hipMemcpyHostToDevice);
-    if (err != hipSuccess) {
-        if (owns) (void)hipFree(device_mem);
-        set_error("qweight upload: %s", hipGetErrorString(err));
-        return RLX_ERR_HIP;
-    }
-    *out = new rlx_qweight{scheme, HL, D, (uint8_t *)device_mem, owns, (int)num_experts};
-    return RLX_OK;
+    return rlx_mi355x_qweight_create_ex(scheme, 0, gguf_bytes, nbytes, n, k, num_experts, device_mem, device_mem ? (size_t)-1 : 0, out);
 }
 
 int rlx_mi355x_qweight_create_experts(int scheme, const void *gguf_bytes, size_t nbytes, int64_t n, int64_t k,
                                       int64_t num_experts, rlx_qweight **out) {
-    return rlx_mi355x_qweight_create_experts_at(scheme, gguf_bytes, nbytes, n, k, num_experts, nullptr, out);
+    return rlx_mi355x_qweight_create_ex(scheme, 0, gguf_bytes, nbytes, n, k, num_experts, nullptr, 0, out);
 }
 
 void rlx_mi355x_qweight_destroy(rlx_qweight *w) {
@@ -456,7 +493,7 @@ int rlx_mi355x_dequant(const rlx_qweight *w, float *out_dev, void *stream) {
                   w->scheme);
         return RLX_ERR_UNSUPPORTED;
     }
-    DequantArgs a{w->dev, out_dev, w->dims.n, w->dims.k, w->dims.units};
+    DequantArgs a{w->dev, out_dev, w->dims.n, w->dims.k, w->dims.units, w->sc_off()};
     void *params[] = {&a};
     KernelId id = w->scheme == SCHEME_Q4_0 ? K_DEQUANT_Q4_0 : w->scheme == SCHEME_Q8_0 ? K_DEQUANT_Q8_0
                   : w->scheme == SCHEME_Q6K ? K_DEQUANT_Q6_K : w->scheme == SCHEME_Q5K ? K_DEQUANT_Q5_K : K_DEQUANT_Q4_K;
@@ -507,7 +544,7 @@ int rlx_mi355x_gguf_matmul_bt_batch(const void *const *xs_dev, int x_dtype, cons
         for (int i = 0; i < count;) {
             int c = 1;
             while (i + c < count && c < GEMM_MAX_SEG && xs_dev[i + c] == xs_dev[i] && ws[i + c]->dims.k == ws[i]->dims.k &&
-                   ws[i + c]->layout.unit_bytes == ws[i]->layout.unit_bytes)
+                   ws[i + c]->layout.unit_bytes == ws[i]->layout.unit_bytes && ws[i + c]->sc_off() == ws[i]->sc_off())
                 c++;
             const bool sums = gemm_plan(ws[i]->scheme, xk, m, ws[i]->dims.k).sxh_bytes != 0;
             const bool prepared = xs_dev[i] == have_x && ws[i]->dims.k == have_k && (have_sums || !sums);

@@ -138,7 +138,8 @@ __device__ __forceinline__ void q4k_scales(uint32_t s0, uint32_t s1, uint32_t s2
 
 // Q6_K granule: code word w (eight low nibbles) and its high-bit word hx (the pair's word as stored for the even code
 // word, rotated right by 8 for the odd one) -> sc * (q - 32) as halfs in fragment order, sc given as a half2 splat of an
-// integer in [0, 255]. (q - 32) is exact; the product is exact up to 2048 and rounded to binary16 above (|.| <= 8160).
+// integer in [-128, 255] (the scale byte read as unsigned or as signed). (q - 32) is exact; the product is exact up to 2048
+// and rounded to binary16 above (|.| <= 8160).
 __device__ __forceinline__ void unpack_q6_scaled(uint32_t w, uint32_t hx, half2_t sc, Frag &f) {
     const half2_t off = {(half_t)(-1056.0f), (half_t)(-1056.0f)};   // 1024 + 32
     const half2_t r16 = {(half_t)0.0625f, (half_t)0.0625f};
@@ -159,6 +160,12 @@ __device__ __forceinline__ void unpack_q6_scaled(uint32_t w, uint32_t hx, half2_
 __device__ __forceinline__ half2_t splat_ubyte_half(uint32_t b) {
     const half2_t k1024 = {(half_t)1024.0f, (half_t)1024.0f};
     return as_half2(MAGIC | b | (b << 16)) - k1024;
+}
+// The same minus `bias` = splat of 1024 + off: the byte read as b - off (off = 128 undoes an offset-binary store).
+__device__ __forceinline__ half2_t splat_ubyte_half(uint32_t b, half2_t bias) { return as_half2(MAGIC | b | (b << 16)) - bias; }
+__device__ __forceinline__ half2_t ubyte_bias(int off) {
+    const half_t v = (half_t)(float)(1024 + off);
+    return half2_t{v, v};
 }
 
 __device__ __forceinline__ float ubyte_to_float(uint32_t w, int byte) { return (float)((w >> (8 * byte)) & 0xFFu); }

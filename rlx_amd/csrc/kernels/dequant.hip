@@ -11,6 +11,7 @@ struct DequantArgs {
     float *out;
     long long n, k;
     long long units;
+    int sc_off;  // Q6_K: the stored scale byte stands for byte - sc_off (0: read as unsigned; 128: signed, stored XOR 0x80)
 };
 
 __device__ __forceinline__ void store8(float *out, long long n, long long k, long long r, long long c, const float v[8]) {
@@ -62,7 +63,8 @@ __device__ __forceinline__ void dequant_tile(const DequantArgs &a) {
             }
         }
     } else if constexpr (SCHEME == SCHEME_Q6K) {
-        // the block decoder the reference's matmul calls (rlx-gguf/src/lib.rs:819-845): (d * sc) * (q - 32), scale bytes unsigned
+        // (d * sc) * (q - 32): the block decoder the reference's matmul calls reads the scale bytes as unsigned
+        // (rlx-gguf/src/lib.rs:819-845), its tensor decoder and ggml as signed (lib.rs:1070-1112); a.sc_off picks
         const uint4_t hw = *(const uint4_t *)(unit + 2048 + l * 16);
         const uint4_t scales = *(const uint4_t *)(unit + 3072 + nrow * 16);
         const float d = half_bits_to_float(*(const uint16_t *)(unit + 3328 + nrow * 2));
@@ -75,7 +77,7 @@ __device__ __forceinline__ void dequant_tile(const DequantArgs &a) {
                 uint32_t hx = hw[2 * h + (t >> 1)];
                 if (t & 1) hx = __builtin_amdgcn_alignbit(hx, hx, 8);
                 const int si = 2 * j + (g >> 1);
-                const float ds = d * ubyte_to_float(scales[si >> 2], si & 3);
+                const float ds = d * (ubyte_to_float(scales[si >> 2], si & 3) - (float)a.sc_off);
                 float v[8];
 #pragma unroll
                 for (int e = 0; e < 8; e++) {

@@ -41,6 +41,7 @@ struct GemmArgs {
     int pair_rows;      // 1: rows 2i, 2i+1 of xh are hi / lo*2048 of logical row i (f32 activations)
     int steps_per_split;  // 64-column steps per grid.z slice (a multiple of 4)
     int use_atomics;      // split K: accumulate into a zeroed `out` with atomic adds
+    int sc_off;           // Q6_K: a stored scale byte stands for byte - sc_off (0 unsigned reading, 128 signed)
 };
 
 // half2 (v, v) with v = byte `byte` of word as an exact binary16 integer: bytes [b, 0x64, b, 0x64] = 1024 + b
@@ -112,6 +113,8 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
     const bool b_live = b_t16 < sg.row_tiles;
     const uint8_t *b_tile = sg.w + (long long)(b_live ? b_t16 : 0) * a.units * L.unit_bytes;
     const uint32_t b_keep = b_live ? 0xFFFFFFFFu : 0u;
+    const half2_t sc_bias = ubyte_bias(a.sc_off);                 // Q6_K scale bytes: value = byte - sc_off
+    const uint32_t sc_dead = (uint32_t)a.sc_off * 0x01010101u;    // the byte that reads as a zero scale
     int b_dst[2];  // [block jl of the step]: k-slice 2 jl + g/2, half g%2
     {
         const int row = wave * 16 + b_n16;
@@ -202,13 +205,13 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
         } else if constexpr (K6) {
             if (q == 0 && jl == 0) {  // this super-block's scales, out of the way of the next super-block's fetch
 #pragma unroll
-                for (int e = 0; e < 4; e++) b_meta[1][e] = b_meta[0][e] & b_keep;  // a dead tile decodes to zeros
+                for (int e = 0; e < 4; e++) b_meta[1][e] = (b_meta[0][e] & b_keep) | (~b_keep & sc_dead);  // a dead tile decodes to zeros
             }
             uint32_t hx = b_hw[cp][t >> 1];
             if (t & 1) hx = __builtin_amdgcn_alignbit(hx, hx, 8);
             // block 2 q + jl of the super-block, this lane's 16-column half of it: scale byte 4 q + 2 jl + g / 2
             const uint32_t scb = (b_meta[1][q] >> (16 * jl + 8 * (b_g >> 1))) & 0xFFu;
-            unpack_q6_scaled(b_q[cp][t], hx, splat_ubyte_half(scb), f);
+            unpack_q6_scaled(b_q[cp][t], hx, splat_ubyte_half(scb, sc_bias), f);
         } else if constexpr (SCHEME == SCHEME_F16W) {
             f.u4 = jl ? b_meta[q & 1] : b_q[q & 1];
 #pragma unroll

@@ -58,6 +58,7 @@ struct GemvArgs {
     float eps;
     int lds_bytes;     // dynamic LDS of the launch
     int kw;            // waves that split the K units of one tile; divides the waves of a workgroup
+    int sc_off;        // Q6_K: a stored scale byte stands for byte - sc_off (0 unsigned reading, 128 signed)
 };
 
 constexpr int XS_PAD_HALFS = 8;      // 16 bytes of padding per LDS row: rows land in different bank groups
@@ -173,7 +174,8 @@ __device__ __forceinline__ void load_afrags(const half_t *xrow, bool live, int c
 // Q4_K / Q5_K block-sum table (16 RG).
 template <int SCHEME, int NREG, int RG>
 __device__ __forceinline__ void compute_unit(const UnitRegs<SCHEME> &w, const half_t *const (&xrow)[RG], const bool (&live)[RG],
-                                             Frag (&a)[4], const float *sxs, int g, int ucol, int ublk, float (&acc)[RG][4]) {
+                                             Frag (&a)[4], const float *sxs, int g, int ucol, int ublk, float (&acc)[RG][4],
+                                             half2_t sc_bias) {
     const float4_t zero = {0.f, 0.f, 0.f, 0.f};
     constexpr int SXS = 16 * RG;
     if constexpr (SCHEME == SCHEME_Q4_0 || SCHEME == SCHEME_Q8_0) {
@@ -218,7 +220,7 @@ __device__ __forceinline__ void compute_unit(const UnitRegs<SCHEME> &w, const ha
                 uint32_t hx = w.hw[2 * h + (t >> 1)];
                 if (t & 1) hx = __builtin_amdgcn_alignbit(hx, hx, 8);
                 const uint32_t scb = (w.sc[2 * h + (t >> 1)] >> (16 * (t & 1) + gshift)) & 0xFFu;
-                unpack_q6_scaled(q[t], hx, splat_ubyte_half(scb), b[t]);
+                unpack_q6_scaled(q[t], hx, splat_ubyte_half(scb, sc_bias), b[t]);
             }
 #pragma unroll
             for (int rg = 0; rg < RG; rg++) {
@@ -440,6 +442,7 @@ __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
     const int nrow = l & 15, g = l >> 4;
     const int rv = (a.x_dtype == X_F32) ? 2 * a.m : a.m;  // virtual A rows
     const int ng = (rv + 3) >> 2;                         // groups of four output rows that exist (16 RG at most)
+    const half2_t sc_bias = ubyte_bias(a.sc_off);
 
     int s = 0;
 #pragma unroll
@@ -583,7 +586,7 @@ __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
 #pragma unroll
                     for (int p = 0; p < UPI; p++)
                         compute_unit<SCHEME, NREG, RG>(cur.u[p], xrow, live, afr, sxs, g, (cu_u * UPI + p) * L.unit_k,
-                                                       (cu_u * UPI + p) * BLK_PER_UNIT, acc);
+                                                       (cu_u * UPI + p) * BLK_PER_UNIT, acc, sc_bias);
                     cu_u += kw;
                     if (cu_u >= nug) {  // last unit of this tile for this wave: bank the partial sums
 #pragma unroll

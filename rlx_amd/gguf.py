@@ -228,10 +228,13 @@ class GgufFile:
             raise GgufError(f"tensor {t.name} extends past data segment ({end} > {len(self._data)})")
         return np.frombuffer(self._data, dtype=np.uint8, count=nbytes, offset=t.offset)
 
-    def qweight(self, name):
+    def qweight(self, name, q6k_signed_scales=True):
         """Upload a 2-D Q8_0 / Q4_0 / Q4_K / Q5_K / Q6_K / Q8_K tensor as a resident `QWeight`. GGML shape order is
         innermost first, so a weight used as y = x . W^T has shape [k, n]. (Q2_K and Q3_K files are not mapped: the
-        reference's block decoders read those two in a field order that differs from ggml's on-disk blocks.)"""
+        reference's block decoders read those two in a field order that differs from ggml's on-disk blocks.)
+        A Q6_K tensor of a file is read with signed scale bytes by default, which is how ggml writes them and how the
+        reference's own tensor decoder reads them (rlx-gguf/src/lib.rs:1070-1112); pass q6k_signed_scales=False for the
+        unsigned reading of the block decoder its matmul calls (lib.rs:819-845)."""
         from . import ops
         from .ir import QuantScheme
         t = self.tensors.get(name)
@@ -242,7 +245,8 @@ class GgufFile:
         if t.dtype not in schemes or len(t.shape) != 2:
             raise GgufError(f"tensor {name}: {t.dtype.name} with shape {t.shape} is not a 2-D matrix of a claimed scheme")
         k, n = t.shape
-        return ops.QWeight(schemes[t.dtype], np.ascontiguousarray(self.tensor_bytes(t)), n, k)
+        return ops.QWeight(schemes[t.dtype], np.ascontiguousarray(self.tensor_bytes(t)), n, k,
+                           q6k_signed_scales=q6k_signed_scales and t.dtype == GgmlType.Q6K)
 
 
 def write_gguf(path_or_file, tensors, metadata=None, version=3, alignment=None):

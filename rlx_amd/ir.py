@@ -67,6 +67,7 @@ class OpKind(enum.IntEnum):
     DequantMatMul = 2
     FakeQuantize = 3
     DequantGroupedMatMul = 4
+    Constant = 5
 
 
 @dataclass(frozen=True)
@@ -100,6 +101,7 @@ class Op:
     ste: SteKind = SteKind.Identity
     scale_mode: ScaleMode = ScaleMode.PerBatch
     ema_decay: float = 0.0
+    data: Optional[bytes] = None  # Op::Constant { data } (op.rs:369-372)
 
     @staticmethod
     def DequantMatMul(scheme):  # Op::DequantMatMul { scheme } (op.rs:736-752)
@@ -144,6 +146,11 @@ class Graph:
 
     def param(self, name, shape):
         return self._push(Op(OpKind.Param), [], shape, name)
+
+    def constant(self, data, shape):  # Op::Constant: bytes embedded in the graph
+        import numpy as np
+        raw = np.ascontiguousarray(data).tobytes()
+        return self._push(Op(OpKind.Constant, data=raw), [], shape)
 
     def add_node(self, op, inputs, shape):
         return self._push(op, inputs, shape)

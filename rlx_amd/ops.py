@@ -91,10 +91,13 @@ def quantize(scheme, x):
     return out
 
 
-def repack_host(scheme, packed, n, k):
+Q6K_SIGNED_SCALES = 1  # rlx_qweight_flags
+
+
+def repack_host(scheme, packed, n, k, flags=0):
     packed = np.ascontiguousarray(packed, dtype=np.uint8)
     out = np.empty(_lib.lib().rlx_mi355x_qweight_device_bytes_for(int(scheme), n, k), dtype=np.uint8)
-    _lib.check(_lib.lib().rlx_mi355x_repack_host(int(scheme), packed.ctypes.data, packed.size, n, k, out.ctypes.data))
+    _lib.check(_lib.lib().rlx_mi355x_repack_host_ex(int(scheme), flags, packed.ctypes.data, packed.size, n, k, out.ctypes.data))
     return out
 
 
@@ -121,16 +124,19 @@ def philox_normal(seed, n):
 class QWeight:
     """GGUF-packed [n, k] matrix resident in HBM in the device layout."""
 
-    def __init__(self, scheme, packed, n, k, num_experts=1):
-        """`num_experts` > 1: `packed` is a stack of that many [n, k] slabs, expert outermost (MoE weights)."""
+    def __init__(self, scheme, packed, n, k, num_experts=1, q6k_signed_scales=False):
+        """`num_experts` > 1: `packed` is a stack of that many [n, k] slabs, expert outermost (MoE weights).
+        `q6k_signed_scales`: read a Q6_K weight's scale bytes as signed (what ggml writes) instead of unsigned (what the
+        reference's matmul reads)."""
         packed = np.ascontiguousarray(packed, dtype=np.uint8)
         self.scheme, self.n, self.k, self.num_experts = QuantScheme(scheme), int(n), int(k), int(num_experts)
         p = C.c_void_p()
-        if num_experts == 1:
+        flags = Q6K_SIGNED_SCALES if q6k_signed_scales else 0
+        if num_experts == 1 and not flags:
             _lib.check(_lib.lib().rlx_mi355x_qweight_create(int(scheme), packed.ctypes.data, packed.size, n, k, C.byref(p)))
         else:
-            _lib.check(_lib.lib().rlx_mi355x_qweight_create_experts(int(scheme), packed.ctypes.data, packed.size, n, k,
-                                                                    num_experts, C.byref(p)))
+            _lib.check(_lib.lib().rlx_mi355x_qweight_create_ex(int(scheme), flags, packed.ctypes.data, packed.size, n, k,
+                                                               num_experts, None, 0, C.byref(p)))
         self.ptr = p.value
 
     def device_bytes(self):

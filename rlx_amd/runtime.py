@@ -47,6 +47,11 @@ def _graph_desc(graph: Graph):
         d.scale_mode = int(nd.op.scale_mode)
         d.ema_decay = nd.op.ema_decay
         d.ste = int(nd.op.ste)
+        if nd.op.data is not None:
+            buf = C.create_string_buffer(nd.op.data, len(nd.op.data))
+            keep.append(buf)
+            d.const_data = C.cast(buf, C.c_void_p)
+            d.const_nbytes = len(nd.op.data)
     outs = (C.c_uint32 * len(graph.outputs))(*graph.outputs)
     gname = graph.name.encode()
     keep += [nodes, outs, gname]
@@ -158,18 +163,37 @@ class CompiledGraph:
 class Session:
     """Session::new(device).compile(graph) (rlx-runtime/src/session.rs:42-136)."""
 
-    def __init__(self, device=Device.Mi355x, fq_round_mode=RoundMode.HalfAway, verbose=False):
+    def __init__(self, device=Device.Mi355x, fq_round_mode=RoundMode.HalfAway, verbose=False, fq_codes=False,
+                 q6k_signed_scales=False):
+        """fq_codes: keep every FakeQuantize node's int8 codes readable (CompiledGraph.fq_codes); q6k_signed_scales: read
+        the scale bytes of Q6_K weights as signed (ggml's reading) instead of the reference matmul's unsigned one."""
         self.device = device
         self.fq_round_mode = fq_round_mode
         self.verbose = verbose
+        self.fq_codes = fq_codes
+        self.q6k_signed_scales = q6k_signed_scales
 
     @staticmethod
     def new(device=Device.Mi355x):
         return Session(device)
 
+    def _opts(self):
+        return _lib.CompileOpts(0, int(self.fq_round_mode), int(self.verbose), int(self.fq_codes), int(self.q6k_signed_scales))
+
+    def plan(self, graph: Graph):
+        """(arena bytes, plan text) of `graph` without touching a device: validation, schedule and memory plan only."""
+        g, keep = _graph_desc(graph)
+        opts = self._opts()
+        buf = C.create_string_buffer(1 << 16)
+        n = _lib.lib().rlx_mi355x_plan(C.byref(g), C.byref(opts), buf, len(buf))
+        del keep
+        if n < 0:
+            raise _lib.RlxError(int(n), _lib.last_error())
+        return int(n), buf.value.decode()
+
     def compile(self, graph: Graph) -> CompiledGraph:
         g, keep = _graph_desc(graph)
-        opts = _lib.CompileOpts(0, int(self.fq_round_mode), int(self.verbose))
+        opts = self._opts()
         h = _lib.lib().rlx_mi355x_compile(C.byref(g), C.byref(opts))
         del keep
         if not h:

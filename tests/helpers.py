@@ -2,7 +2,7 @@
 import numpy as np
 
 Q4K, Q5K, Q6K, Q8K, Q2K, Q3K, Q4_0, Q8_0 = 5, 6, 7, 8, 9, 10, 11, 12
-WIDE = (Q8K, Q2K, Q3K)  # stored as binary16 on the device (Q6_K too when RLX_Q6K_SIGNED_SCALES is set)
+WIDE = (Q8K, Q2K, Q3K)  # decoded at upload and stored as binary16 on the device
 SCHEME_NAMES = {Q4K: "q4_k", Q5K: "q5_k", Q6K: "q6_k", Q8K: "q8_k", Q2K: "q2_k", Q3K: "q3_k", Q4_0: "q4_0", Q8_0: "q8_0"}
 BLOCK = {Q4_0: (32, 18), Q8_0: (32, 34), Q4K: (256, 144), Q5K: (256, 176), Q6K: (256, 210), Q8K: (256, 292), Q2K: (256, 84), Q3K: (256, 110)}
 NIB_POS = [0, 4, 1, 5, 2, 6, 3, 7]
@@ -41,8 +41,9 @@ def random_blocks(scheme, n, k, seed=0, d_std=0.02, dmin_std=0.01):
     return p.reshape(-1)
 
 
-def decode_device_layout(scheme, dev, n, k):
-    """Read the device layout back into f32 [n,k] following csrc/layout.h, with the reference's arithmetic."""
+def decode_device_layout(scheme, dev, n, k, q6k_sc_off=0):
+    """Read the device layout back into f32 [n,k] following csrc/layout.h, with the reference's arithmetic.
+    q6k_sc_off: a stored Q6_K scale byte stands for byte - q6k_sc_off (128 for a weight repacked with signed scales)."""
     unit_k, unit_bytes, qbytes = UNIT[scheme]
     tiles, units = (n + 15) // 16, (k + unit_k - 1) // unit_k
     dev = dev.reshape(tiles, units, unit_bytes)
@@ -63,7 +64,7 @@ def decode_device_layout(scheme, dev, n, k):
                         code = b - 128
                     cols = np.arange(units) * unit_k + t * 32 + g * 8 + e
                     out[np.ix_(rows, cols)] = d * code.astype(np.float32)
-        elif scheme == Q6K:  # the matmul's reading: (d * sc) * (q - 32), scale bytes unsigned
+        elif scheme == Q6K:  # (d * sc) * (q - 32)
             d = dev[:, :, 3328 + nrow * 2: 3328 + nrow * 2 + 2].copy().view(np.float16).astype(np.float32).reshape(tiles, units)
             scales = dev[:, :, 3072 + nrow * 16: 3072 + nrow * 16 + 16]
             hw = dev[:, :, 2048 + l * 16: 2048 + l * 16 + 16].copy().view(np.uint32).reshape(tiles, units, 4)
@@ -73,7 +74,7 @@ def decode_device_layout(scheme, dev, n, k):
                 hx = hw[:, :, (j >> 2) * 2 + ((j & 3) >> 1)]
                 if j & 1:
                     hx = (hx >> 8) | (hx << 24)
-                ds = (d * scales[:, :, 2 * j + (g >> 1)].astype(np.float32)).astype(np.float32)
+                ds = (d * (scales[:, :, 2 * j + (g >> 1)].astype(np.float32) - np.float32(q6k_sc_off))).astype(np.float32)
                 for e in range(8):
                     code = ((w >> (4 * NIB_POS[e])) & 0xF) | (((hx >> Q6K_HI_POS[e]) & 3) << 4)
                     cols = np.arange(units) * unit_k + j * 32 + g * 8 + e

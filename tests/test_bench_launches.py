@@ -157,7 +157,7 @@ def test_config4_chain_full_size(oracle):
     w = g.param("w", Shape.new([len(packed)], DType.U8))
     y = g.add_node(Op.DequantMatMul(QuantScheme.GgufQ8_0), [fq, w], Shape.new([rows, n], DType.F32))
     g.set_outputs([y, fq])
-    c = Session.new().compile(g)
+    c = Session(fq_codes=True).compile(g)
     c.set_param_typed("w", packed, DType.U8)
     y_got, fq_got = c.run([("x", x)])
     y_got = y_got.reshape(rows, n)

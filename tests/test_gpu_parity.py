@@ -379,7 +379,7 @@ def test_graph_fq_then_q8_0_matmul(oracle):
     w = g.param("w", Shape.new([len(packed)], DType.U8))
     y = g.add_node(Op.DequantMatMul(QuantScheme.GgufQ8_0), [fq, w], Shape.new([rows, n], DType.F32))
     g.set_outputs([y, fq])
-    c = Session.new().compile(g)
+    c = Session(fq_codes=True).compile(g)
     say(c.describe_plan())
     c.set_param_typed("w", packed, DType.U8)
     y_got, fq_got = c.run([("x", x)])
@@ -610,3 +610,91 @@ def test_captured_graph_fq_prefill_and_grouped_replays(oracle):
         assert rel_err(z_got, oracle.gguf_grouped_matmul_f64(tokens, stack, idx, 4, k, n, experts, Q4_0)) <= TOL, attempt
         if attempt == "eager":
             c.capture()
+
+
+# ------------------------------------------------------------------ graph level: constants, prefill steps, pipelined commits
+
+def test_graph_constant_nodes(oracle):
+    # Op::Constant (rlx-ir/src/op.rs:369-372): a constant FakeQuantize state and a packed weight embedded in the graph
+    rows, k, n = 8, 512, 48
+    packed, _ = make_weights(Q4_0, n, k, seed=91)
+    state = (np.float32(0.01) + np.float32(0.002) * np.arange(k, dtype=np.float32)).astype(np.float32)
+    x = np.random.default_rng(92).standard_normal((rows, k)).astype(np.float32)
+    g = Graph.new("consts")
+    xi = g.input("x", Shape.new([rows, k], DType.F32))
+    st = g.constant(state, Shape.new([k], DType.F32))
+    fq = g.add_node(Op.FakeQuantize(8, 1, scale_mode=ScaleMode.Fixed), [xi, st], Shape.new([rows, k], DType.F32))
+    w = g.constant(packed, Shape.new([len(packed)], DType.U8))
+    y = g.add_node(Op.DequantMatMul(QuantScheme.GgufQ4_0), [fq, w], Shape.new([rows, n], DType.F32))
+    g.set_outputs([y, fq])
+    c = Session.new().compile(g)
+    y_got, fq_got = c.run([("x", x)])
+    fq_ref, _, _ = oracle.fake_quantize(x, x.shape, 1, 8, int(ScaleMode.Fixed), 0.0, state.copy())
+    assert np.array_equal(fq_got.reshape(rows, k).view(np.uint32), fq_ref.view(np.uint32))
+    assert rel_err(y_got.reshape(rows, n), oracle.gguf_matmul_f64(fq_ref, packed, rows, k, n, Q4_0)) <= TOL
+
+
+@pytest.mark.parametrize("m,x_dtype", [(48, DType.F32), (200, DType.BF16), (24, DType.BF16)])
+def test_graph_prefill_step_shares_one_workspace(oracle, m, x_dtype):
+    # q / k / v on one input plus a matmul on another input, all ready at the same point of the schedule: the step goes
+    # through the batched entry point on a single workspace (the shared input converted once), eagerly and on every
+    # replay of the captured graph. 24 bf16 rows take the decode kernels from the same step.
+    k, ns = 1024, [256, 64, 80]
+    rng = np.random.default_rng(m)
+    g = Graph.new("prefill_qkv")
+    xi = g.input("x", Shape.new([m, k], x_dtype))
+    xj = g.input("x2", Shape.new([m, 512], x_dtype))
+    packs, outs = [], []
+    for i, n in enumerate(ns):
+        p, _ = make_weights(Q4K, n, k, seed=95 + i)
+        packs.append(p)
+        w = g.param(f"w{i}", Shape.new([len(p)], DType.U8))
+        outs.append(g.add_node(Op.DequantMatMul(QuantScheme.GgufQ4K), [xi, w], Shape.new([m, n], DType.F32)))
+    p4, _ = make_weights(Q4K, 32, 512, seed=99)
+    w4 = g.param("w4", Shape.new([len(p4)], DType.U8))
+    outs.append(g.add_node(Op.DequantMatMul(QuantScheme.GgufQ4K), [xj, w4], Shape.new([m, 32], DType.F32)))
+    g.set_outputs(outs)
+    c = Session.new().compile(g)
+    assert c.describe_plan().count("step workspace@") == 1
+    for i, p in enumerate(packs):
+        c.set_param_typed(f"w{i}", p, DType.U8)
+    c.set_param_typed("w4", p4, DType.U8)
+    for attempt in ("eager", "replay 1", "replay 2"):
+        x = rng.standard_normal((m, k)).astype(np.float32)
+        x2 = rng.standard_normal((m, 512)).astype(np.float32)
+        if x_dtype == DType.BF16:
+            x, x2 = oracle.bf16_round(x), oracle.bf16_round(x2)
+            c.write_input("x", f32_to_bf16_bits(x), DType.BF16)
+            c.write_input("x2", f32_to_bf16_bits(x2), DType.BF16)
+        else:
+            c.write_input("x", x)
+            c.write_input("x2", x2)
+        c.launch()
+        for i, n in enumerate(ns):
+            assert rel_err(c.read_output(i).reshape(m, n), oracle.gguf_matmul_f64(x, packs[i], m, k, n, Q4K)) <= TOL, (attempt, i)
+        assert rel_err(c.read_output(3).reshape(m, 32), oracle.gguf_matmul_f64(x2, p4, m, 512, 32, Q4K)) <= TOL, attempt
+        if attempt == "eager":
+            c.capture()
+
+
+def test_commit_no_wait_sequence(oracle):
+    # ExecutableGraph::commit_no_wait(inputs) / sync_pending (rlx-runtime/src/backend.rs:275-281) as a binding drives
+    # them: write each input, launch without waiting, again with new inputs, then one sync; the arena holds the
+    # outputs of the last commit (earlier ones are stomped, as the reference documents)
+    k, n = 512, 96
+    packed, _ = make_weights(Q8_0, n, k, seed=101)
+    g = Graph.new("pipelined")
+    xi = g.input("x", Shape.new([2, k], DType.F32))
+    w = g.param("w", Shape.new([len(packed)], DType.U8))
+    g.set_outputs([g.add_node(Op.DequantMatMul(QuantScheme.GgufQ8_0), [xi, w], Shape.new([2, n], DType.F32))])
+    c = Session.new().compile(g)
+    c.set_param_typed("w", packed, DType.U8)
+    rng = np.random.default_rng(102)
+    xs = [rng.standard_normal((2, k)).astype(np.float32) for _ in range(5)]
+    for x in xs:                     # commit_no_wait(&[("x", x)]) five times
+        c.write_input("x", x)
+        c.launch()
+    c.sync()                         # sync_pending()
+    got = c.read_output(0).reshape(2, n)
+    assert rel_err(got, oracle.gguf_matmul_f64(xs[-1], packed, 2, k, n, Q8_0)) <= TOL
+    assert rel_err(got, oracle.gguf_matmul_f64(xs[0], packed, 2, k, n, Q8_0)) > TOL

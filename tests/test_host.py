@@ -22,7 +22,7 @@ def test_header_symbols_all_exported():
     missing = [s for s in declared if not hasattr(L, s)]
     assert not missing, missing
     assert declared == set(rlx_amd._lib.SIGNATURES), declared ^ set(rlx_amd._lib.SIGNATURES)
-    assert L.rlx_mi355x_abi_version() == 1
+    assert L.rlx_mi355x_abi_version() == 2
     assert L.rlx_mi355x_device_name() == b"MI355X"
 
 
@@ -128,7 +128,80 @@ def compile_error(g):
 
 
 def test_supported_ops():
-    assert [int(k) for k in rlx_amd.supported_ops()] == [0, 1, 2, 3, 4]
+    assert [int(k) for k in rlx_amd.supported_ops()] == [0, 1, 2, 3, 4, 5]
+
+
+def test_qweight_create_validates_before_allocating():
+    # bad shapes, sizes and flags are refused with a message, before any host or device allocation (no GPU needed)
+    import ctypes as C
+    L = rlx_amd._lib.lib()
+    blob = np.zeros(18 * 8, np.uint8)
+    out = C.c_void_p()
+    for n, k, experts, flags, nbytes in [(-1, 256, 1, 0, blob.size), (0, 256, 1, 0, blob.size), (1, 0, 1, 0, blob.size),
+                                         (1, 100, 1, 0, blob.size), (1, 256, 0, 0, blob.size), (1, 256, 1, 8, blob.size),
+                                         (1, 256, 1, 0, blob.size - 1), (1, 256, 2, 0, blob.size)]:
+        rc = L.rlx_mi355x_qweight_create_ex(int(Q4_0), flags, blob.ctypes.data, nbytes, n, k, experts, None, 0, C.byref(out))
+        assert rc == -1 and not out.value, (n, k, experts, flags, nbytes, rlx_amd._lib.last_error())
+    assert L.rlx_mi355x_qweight_create_ex(3, 0, blob.ctypes.data, blob.size, 1, 256, 1, None, 0, C.byref(out)) == -2
+    # a caller-owned slot that is too small for the device layout is refused, not overrun
+    rc = L.rlx_mi355x_qweight_create_ex(int(Q4_0), 0, blob.ctypes.data, blob.size, 1, 256, 1, C.c_void_p(4096), 1000, C.byref(out))
+    assert rc == -1 and "slot holds 1000" in rlx_amd._lib.last_error()
+
+
+def test_plan_reuses_dead_slots():
+    # FakeQuantize -> matmul -> matmul: the second matmul's output may take the bytes of the fake-quantized tensor, which is
+    # dead by then, and a step's workspace lives for that step only (rlx-compile/src/memory.rs:386-470 is the contract)
+    g = Graph.new("chain")
+    x = g.input("x", Shape.new([64, 4096], DType.F32))
+    fq = g.add_node(Op.FakeQuantize(8, 1), [x], Shape.new([64, 4096], DType.F32))
+    w = g.param("w", Shape.new([4096 * 256 // 32 * 34], DType.U8))
+    y = g.add_node(Op.DequantMatMul(QuantScheme.GgufQ8_0), [fq, w], Shape.new([64, 256], DType.F32))
+    w2 = g.param("w2", Shape.new([256 * 128 // 32 * 34], DType.U8))
+    z = g.add_node(Op.DequantMatMul(QuantScheme.GgufQ8_0), [y, w2], Shape.new([64, 128], DType.F32))
+    g.set_outputs([z])
+    def slots_of(text):
+        return {int(line.split()[1]): (int(line.split("off=")[1].split()[0]), int(line.split("size=")[1].split()[0]))
+                for line in text.splitlines()[1:]}
+
+    total, text = Session().plan(g)
+    slots = slots_of(text)
+    assert slots[5][0] == slots[1][0]                      # z reuses the fake-quantized tensor's slot
+    bump = sum((sz + 255) // 256 * 256 for _, sz in slots.values())
+    assert total < bump + 2 * 1024 * 1024                  # less than one private slot per buffer plus both workspaces
+    live = [0, 2, 4]                                       # sources never share bytes with anything
+    for a in live:
+        for b, (ob, sb) in slots.items():
+            if a != b:
+                oa, sa = slots[a]
+                assert oa + sa <= ob or ob + sb <= oa, (a, b)
+    # with every intermediate an output nothing may be reused
+    g.set_outputs([z, y, fq])
+    total_all, text_all = Session().plan(g)
+    kept = slots_of(text_all)
+    for a in (1, 3, 5):
+        for b in (1, 3, 5):
+            if a < b:
+                assert kept[a][0] + kept[a][1] <= kept[b][0] or kept[b][0] + kept[b][1] <= kept[a][0], (a, b)
+    assert total_all >= total
+    # the integer codes are opt-in: one more resident byte per element
+    assert Session(fq_codes=True).plan(g)[0] >= total_all + 64 * 4096
+
+
+def test_plan_constant_nodes():
+    g = Graph.new("const")
+    x = g.input("x", Shape.new([4, 8], DType.F32))
+    st = g.constant(np.full(8, 0.05, np.float32), Shape.new([8], DType.F32))
+    q = g.add_node(Op.FakeQuantize(8, 1, scale_mode=ScaleMode.Fixed), [x, st], Shape.new([4, 8], DType.F32))
+    g.set_outputs([q])
+    total, text = Session().plan(g)
+    assert "Constant" in text and total >= 4 * 8 * 4 * 2 + 32
+    bad = Graph.new("const")
+    x = bad.input("x", Shape.new([4, 8], DType.F32))
+    st = bad.constant(np.full(7, 0.05, np.float32), Shape.new([8], DType.F32))
+    q = bad.add_node(Op.FakeQuantize(8, 1, scale_mode=ScaleMode.Fixed), [x, st], Shape.new([4, 8], DType.F32))
+    bad.set_outputs([q])
+    with pytest.raises(rlx_amd.RlxError, match="constant node"):
+        Session().plan(bad)
 
 
 def test_compile_rejects_wrong_weight_size():

@@ -1,6 +1,6 @@
 """Q5_K, Q6_K, Q8_K, Q2_K, Q3_K: the other five schemes the reference's gguf_matmul_bt dispatches
-(rlx-cpu/src/gguf_matmul.rs:25-37). Q5_K and Q6_K have packed kernels of their own; the other three (and Q6_K when its
-scale bytes are to be read as signed) are decoded once at upload and kept as binary16 ("wide").
+(rlx-cpu/src/gguf_matmul.rs:25-37). Q5_K and Q6_K have packed kernels of their own (Q6_K in both readings of its scale
+bytes); the other three are decoded once at upload and kept as binary16 ("wide").
 
 CPU part: pins the oracle's five block decoders (the reference's own known-answer blocks, closed-form position
 probes, reduction of Q5_K to the pinned Q4_K decoder, independent numpy bit-field decoders on random bytes), then
@@ -244,6 +244,18 @@ def test_packed_layout_keeps_every_bit(scheme):
                           oracle.dequant_matmul_blocks(scheme, blocks, n * k).reshape(n, k).view(np.uint32))
 
 
+def test_packed_q6k_layout_with_signed_scales():
+    """A Q6_K weight repacked for the signed reading (ggml's; the reference's tensor decoder, lib.rs:1070-1112) keeps the
+    same bytes except that its scale bytes are stored XOR 0x80 and read as byte - 128."""
+    n, k = 37, 768
+    blocks = random_blocks(Q6K, n, k, seed=48)
+    dev = ops.repack_host(Q6K, blocks, n, k, flags=ops.Q6K_SIGNED_SCALES)
+    plain = ops.repack_host(Q6K, blocks, n, k)
+    assert dev.size == plain.size and not np.array_equal(dev, plain)
+    assert np.array_equal(decode_device_layout(Q6K, dev, n, k, q6k_sc_off=128).view(np.uint32),
+                          oracle.dequant(Q6K, blocks, n * k).reshape(n, k).view(np.uint32))
+
+
 def test_repack_rejects_weights_beyond_binary16():
     blk = np.concatenate([np.frombuffer(np.float32(1e4).tobytes(), np.uint8), np.full(256, 100, np.uint8), np.zeros(32, np.uint8)])
     with pytest.raises(rlx_amd.RlxError, match="binary16"):
@@ -352,21 +364,53 @@ def test_packed_dequant_is_bit_exact(scheme, n, k):
 
 
 @pytest.mark.gpu
-def test_q6k_signed_scales_on_request(monkeypatch):
-    """RLX_Q6K_SIGNED_SCALES (read at upload) selects ggml's reading of the scale bytes; the weight is then kept as binary16."""
-    n, k, m = 40, 512, 1
+@pytest.mark.parametrize("m,x_dtype", [(1, DType.F32), (7, DType.BF16), (24, DType.BF16), (96, DType.BF16), (300, DType.F32)])
+def test_q6k_signed_scales_stay_packed(m, x_dtype):
+    """RLX_QW_Q6K_SIGNED_SCALES selects ggml's reading of the scale bytes: same packed bytes, same kernels; dequant is
+    bit-identical to the reference's tensor decoder and every matmul path (decode, two row groups, both prefill tiles)
+    follows it."""
+    n, k = 72, 1024
     blocks = random_blocks(Q6K, n, k, seed=5, d_std=5e-6)
     x = np.random.default_rng(6).standard_normal((m, k)).astype(np.float32)
-    monkeypatch.setenv("RLX_Q6K_SIGNED_SCALES", "1")
-    qw = ops.QWeight(QuantScheme.GgufQ6K, blocks, n, k)
-    assert qw.device_bytes() == 3 * (k // 128) * 4096
-    got = ops.gguf_matmul_bt(x, qw, m)
+    if x_dtype == DType.BF16:
+        x = oracle.bf16_round(x)
+    qw = ops.QWeight(QuantScheme.GgufQ6K, blocks, n, k, q6k_signed_scales=True)
+    assert qw.device_bytes() == 5 * (k // 256) * 3360
+    assert np.array_equal(qw.dequant().view(np.uint32), oracle.dequant(Q6K, blocks, n * k).reshape(n, k).view(np.uint32))
+    got = ops.gguf_matmul_bt(bf16_bits(x) if x_dtype == DType.BF16 else x, qw, m, x_dtype)
     qw.free()
-    monkeypatch.delenv("RLX_Q6K_SIGNED_SCALES")
     w_signed = oracle.dequant(Q6K, blocks, n * k).reshape(n, k).astype(np.float64)
     assert rel_err(got, x.astype(np.float64) @ w_signed.T) <= 2e-3
     w_unsigned = oracle.dequant_matmul_blocks(Q6K, blocks, n * k).reshape(n, k).astype(np.float64)
     assert rel_err(got, x.astype(np.float64) @ w_unsigned.T) > 2e-3  # the two readings differ on random scale bytes
+
+
+@pytest.mark.gpu
+def test_q6k_signed_scales_through_session_and_gguf_file(tmp_path):
+    """The graph level takes the reading from rlx_compile_opts.q6k_signed_scales; a Q6_K tensor of a GGUF file is read as
+    signed by default (that is how ggml writes it)."""
+    from rlx_amd import Graph, Op, Session, Shape, gguf
+    n, k, m = 48, 512, 3
+    blocks = random_blocks(Q6K, n, k, seed=7, d_std=5e-6)
+    x = np.random.default_rng(8).standard_normal((m, k)).astype(np.float32)
+    want = {True: x.astype(np.float64) @ oracle.dequant(Q6K, blocks, n * k).reshape(n, k).astype(np.float64).T,
+            False: x.astype(np.float64) @ oracle.dequant_matmul_blocks(Q6K, blocks, n * k).reshape(n, k).astype(np.float64).T}
+    for signed in (False, True):
+        g = Graph.new("q6k")
+        xi = g.input("x", Shape.new([m, k], DType.F32))
+        w = g.param("w", Shape.new([blocks.size], DType.U8))
+        g.set_outputs([g.add_node(Op.DequantMatMul(QuantScheme.GgufQ6K), [xi, w], Shape.new([m, n], DType.F32))])
+        c = Session(q6k_signed_scales=signed).compile(g)
+        c.set_param_typed("w", blocks, DType.U8)
+        assert rel_err(c.run([("x", x)])[0].reshape(m, n), want[signed]) <= 2e-3, signed
+    path = tmp_path / "q6k.gguf"
+    gguf.write_gguf(str(path), [("w", [k, n], gguf.GgmlType.Q6K, blocks.tobytes())])
+    f = gguf.GgufFile.from_path(str(path))
+    for signed in (True, False):
+        qw = f.qweight("w", q6k_signed_scales=signed)
+        assert rel_err(ops.gguf_matmul_bt(x, qw, m), want[signed]) <= 2e-3, signed
+        qw.free()
+    assert rel_err(ops.gguf_matmul_bt(x, f.qweight("w"), m), want[True]) <= 2e-3
 
 
 @pytest.mark.gpu
