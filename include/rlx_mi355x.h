@@ -241,6 +241,18 @@ int rlx_mi355x_fake_quantize(const float *x_dev, float *out_dev, int8_t *codes_d
                              int64_t inner, int bits, int scale_mode, float ema_decay, float *state_dev,
                              int round_mode, void *scratch_dev, void *stream);
 
+/* rlx_mi355x_fake_quantize for callers that cannot allocate (a stream capture in progress, tight serving loops,
+ * harnesses that forbid hipMalloc). No counterpart in the reference. Same arguments without `scratch_dev`: the scratch is
+ * a device array inside the library image, rlx_mi355x_fake_quantize_noalloc_max_scratch() = 8 MiB per GPU, held until
+ * the process ends. The call allocates nothing (no hipMalloc / hipFree, on any path) once the library is initialised
+ * (rlx_mi355x_is_available() does that). A shape whose rlx_mi355x_fake_quantize_scratch_bytes() exceeds the array is
+ * RLX_ERR_UNSUPPORTED ([8192, 4096] with 4096 channels needs 4.03 MiB). Every call on a GPU shares that GPU's array:
+ * calls that overlap in time on one GPU (two streams, two threads) race; calls ordered on one stream do not. */
+size_t rlx_mi355x_fake_quantize_noalloc_max_scratch(void);
+int rlx_mi355x_fake_quantize_noalloc(const float *x_dev, float *out_dev, int8_t *codes_dev, int64_t len, int64_t chan_dim,
+                                     int64_t inner, int bits, int scale_mode, float ema_decay, float *state_dev,
+                                     int round_mode, void *stream);
+
 /* ------------------------------------------------------------------------------------------
  * Host utilities that exist because the path needs inputs: the reference has no GGUF encoder
  * (rlx-gguf is decode-only) and seeds its tensors with Philox (rlx-ir/src/rng.rs:43-143).
