@@ -227,6 +227,16 @@ int rlx_mi355x_rmsnorm_gguf_tied_lm_topk(const float *hidden_dev, const float *g
 int rlx_mi355x_gguf_matmul_bt_batch(const void *const *xs_dev, int x_dtype, const rlx_qweight *const *ws,
                                     float *const *outs_dev, int count, int64_t m, void *workspace, size_t workspace_bytes,
                                     void *stream);
+/* The prefill path (m above the decode limit) in two calls, for a caller that multiplies one activation tensor by weights
+ * at several points of its schedule, or keeps the conversion out of a timed region. No counterpart in the reference
+ * (its thunk converts nothing). ..._prepare writes the binary16 image of x[m, k] (and, for Q4_K / Q5_K, its block
+ * sums) into `workspace` (rlx_mi355x_gguf_matmul_workspace(scheme, x_dtype, m, k, 0) bytes); ..._bt_prepared multiplies
+ * that image by `count` matrices, all with the k the image was made for: outs_dev[i][m, n_i]. An image made for Q4_K / Q5_K also
+ * serves the other schemes, not the other way round. */
+int rlx_mi355x_gguf_matmul_prepare(const void *x_dev, int x_dtype, int scheme, int64_t m, int64_t k, void *workspace,
+                                   size_t workspace_bytes, void *stream);
+int rlx_mi355x_gguf_matmul_bt_prepared(const void *workspace, size_t workspace_bytes, int x_dtype, const rlx_qweight *const *ws,
+                                       float *const *outs_dev, int count, int64_t m, void *stream);
 
 /* Thunk::FakeQuantize (rlx-cpu/src/thunk.rs:11159-11253) with the layout of quant_layout()
  * (thunk.rs:14163-14175): channel of flat element i is (i / inner) % chan_dim.

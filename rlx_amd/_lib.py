@@ -81,6 +81,8 @@ SIGNATURES = {
     "rlx_mi355x_gguf_matmul_bt": (_i, [_vp, _i, _vp, _vp, _i64, _vp, _sz, _vp]),
     "rlx_mi355x_gguf_matmul_workspace": (_sz, [_i, _i, _i64, _i64, _i64]),
     "rlx_mi355x_gguf_matmul_bt_batch": (_i, [_pvp, _i, _pvp, _pvp, _i, _i64, _vp, _sz, _vp]),
+    "rlx_mi355x_gguf_matmul_prepare": (_i, [_vp, _i, _i, _i64, _i64, _vp, _sz, _vp]),
+    "rlx_mi355x_gguf_matmul_bt_prepared": (_i, [_vp, _sz, _i, _pvp, _pvp, _i, _i64, _vp]),
     "rlx_mi355x_qweight_create_experts": (_i, [_i, _vp, _sz, _i64, _i64, _i64, _pvp]),
     "rlx_mi355x_qweight_create_experts_at": (_i, [_i, _vp, _sz, _i64, _i64, _i64, _vp, _pvp]),
     "rlx_mi355x_gguf_grouped_matmul_bt": (_i, [_vp, _i, _vp, _vp, _vp, _i64, _vp]),

@@ -59,9 +59,8 @@ enum KernelId : int {
     K_COUNT
 };
 
-// Device layout a scheme is kept in: its packed layout (layout_of), or binary16 fragments for the wide schemes — Q5_K,
-// Q8_K, Q2_K, Q3_K always, Q6_K when RLX_Q6K_SIGNED_SCALES asks for ggml's signed reading of its scale bytes (the
-// packed Q6_K kernels read them unsigned, as the reference's matmul does).
+// Device layout a scheme is kept in: its packed layout (layout_of), or binary16 fragments for the wide schemes (Q8_K,
+// Q2_K, Q3_K).
 Layout host_layout(int scheme);
 inline bool is_wide(int scheme) { return layout_is_f16w(host_layout(scheme)); }
 

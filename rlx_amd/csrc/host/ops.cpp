@@ -574,6 +574,55 @@ int rlx_mi355x_gguf_matmul_bt_batch(const void *const *xs_dev, int x_dtype, cons
     return RLX_OK;
 }
 
+// The two halves of the prefill path as calls of their own, for a caller that multiplies one activation tensor by several
+// weights at different points of its schedule (or wants the conversion outside a timed region): prepare converts x into
+// the workspace image once, prepared multiplies that image by up to four matrices of one scheme and K per launch.
+int rlx_mi355x_gguf_matmul_prepare(const void *x_dev, int x_dtype, int scheme, int64_t m, int64_t k, void *workspace,
+                                   size_t workspace_bytes, void *stream) {
+    using namespace rlx;
+    const int xk = x_kind(x_dtype);
+    const Layout L = layout_of(scheme);
+    if (!x_dev || xk < 0 || L.unit_k == 0 || m <= decode_rows(xk) || k <= 0 || k % 32 != 0) {
+        set_error("gguf_matmul_prepare: needs F32 / BF16 / F16 activations, a claimed scheme, k a multiple of 32 and m above the decode limit (%lld)",
+                  (long long)decode_rows(xk < 0 ? 0 : xk));
+        return RLX_ERR_INVALID;
+    }
+    const GemmPlan p = gemm_plan(scheme, xk, m, k);
+    if (!workspace || workspace_bytes < p.xh_bytes + p.sxh_bytes || (uintptr_t)workspace % 16 != 0 || (uintptr_t)x_dev % 16 != 0) {
+        set_error("gguf_matmul_prepare: a 16-byte aligned workspace of %zu bytes is needed, got %zu", p.xh_bytes + p.sxh_bytes, workspace_bytes);
+        return RLX_ERR_INVALID;
+    }
+    XPrepArgs xa{x_dev, workspace, p.sxh_bytes ? (uint8_t *)workspace + p.xh_bytes : nullptr, (int)m, (int)k, (int)p.k_pad, (int)p.m_rows, xk};
+    void *xparams[] = {&xa};
+    const long long xblocks = (p.m_rows / 256) * (p.k_pad / 64) * 8;
+    return launch(K_XPREP, (unsigned)xblocks, 1, 256, 0, (hipStream_t)stream, xparams);
+}
+
+int rlx_mi355x_gguf_matmul_bt_prepared(const void *workspace, size_t workspace_bytes, int x_dtype, const rlx_qweight *const *ws,
+                                       float *const *outs_dev, int count, int64_t m, void *stream) {
+    using namespace rlx;
+    const int xk = x_kind(x_dtype);
+    if (!workspace || !ws || !outs_dev || count <= 0 || xk < 0 || m <= decode_rows(xk)) {
+        set_error("gguf_matmul_bt_prepared: null argument, count=%d, or m=%lld within the decode limit", count, (long long)m);
+        return RLX_ERR_INVALID;
+    }
+    for (int i = 0; i < count; i++)
+        if (!ws[i] || !outs_dev[i]) {
+            set_error("gguf_matmul_bt_prepared: null weight / output %d", i);
+            return RLX_ERR_INVALID;
+        }
+    for (int i = 0; i < count;) {
+        int c = 1;
+        while (i + c < count && c < GEMM_MAX_SEG && ws[i + c]->scheme == ws[i]->scheme && ws[i + c]->dims.k == ws[i]->dims.k &&
+               ws[i + c]->sc_off() == ws[i]->sc_off())
+            c++;
+        // `workspace` is only read; the x pointer is not looked at when the image is already there
+        RLX_TRY(launch_gemm(workspace, xk, ws + i, outs_dev + i, c, m, const_cast<void *>(workspace), workspace_bytes, (hipStream_t)stream, true));
+        i += c;
+    }
+    return RLX_OK;
+}
+
 int rlx_mi355x_gguf_matmul_bt(const void *x_dev, int x_dtype, const rlx_qweight *w, float *out_dev, int64_t m,
                               void *workspace, size_t workspace_bytes, void *stream) {
     return rlx_mi355x_gguf_matmul_bt_batch(&x_dev, x_dtype, &w, &out_dev, 1, m, workspace, workspace_bytes, stream);

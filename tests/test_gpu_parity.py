@@ -698,3 +698,32 @@ def test_commit_no_wait_sequence(oracle):
     got = c.read_output(0).reshape(2, n)
     assert rel_err(got, oracle.gguf_matmul_f64(xs[-1], packed, 2, k, n, Q8_0)) <= TOL
     assert rel_err(got, oracle.gguf_matmul_f64(xs[0], packed, 2, k, n, Q8_0)) > TOL
+
+
+@pytest.mark.parametrize("scheme,x_dtype", [(Q4K, DType.BF16), (Q4_0, DType.F32)])
+def test_prefill_prepare_then_prepared(oracle, scheme, x_dtype):
+    # the prefill path in two calls: one conversion of x, then two launches over five matrices reading the same image;
+    # every output equals the one-call form bit for bit (the same kernels run on the same image)
+    import ctypes as C
+    m, k, ns = 200, 1024, [256, 64, 80, 128, 48]
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    xin = f32_to_bf16_bits(oracle.bf16_round(x)) if x_dtype == DType.BF16 else x
+    x_ref = oracle.bf16_round(x) if x_dtype == DType.BF16 else x
+    packs = [make_weights(scheme, n, k, seed=110 + i)[0] for i, n in enumerate(ns)]
+    ws = [ops.QWeight(scheme, p, n, k) for p, n in zip(packs, ns)]
+    L = rlx_amd._lib.lib()
+    need = ops.matmul_workspace_bytes(ws[0], x_dtype, m)
+    wsb, xd = ops.DeviceBuffer(need), ops.DeviceBuffer.from_numpy(xin)
+    outs = [ops.DeviceBuffer(m * n * 4) for n in ns]
+    rlx_amd._lib.check(L.rlx_mi355x_gguf_matmul_prepare(xd.ptr, int(x_dtype), int(scheme), m, k, wsb.ptr, need, None))
+    wp = (C.c_void_p * len(ns))(*[w.ptr for w in ws])
+    op = (C.c_void_p * len(ns))(*[o.ptr for o in outs])
+    rlx_amd._lib.check(L.rlx_mi355x_gguf_matmul_bt_prepared(wsb.ptr, need, int(x_dtype), wp, op, len(ns), m, None))
+    ops.sync()
+    for i, n in enumerate(ns):
+        got = outs[i].to_numpy(np.float32).reshape(m, n)
+        assert rel_err(got, oracle.gguf_matmul_f64(x_ref, packs[i], m, k, n, scheme)) <= TOL, i
+        assert rel_err(got, ops.gguf_matmul_bt(xin, ws[i], m, x_dtype)) <= 1e-5, i
+    with pytest.raises(rlx_amd.RlxError):  # decode sizes have no image to prepare
+        rlx_amd._lib.check(L.rlx_mi355x_gguf_matmul_prepare(xd.ptr, int(x_dtype), int(scheme), 4, k, wsb.ptr, need, None))
