@@ -84,12 +84,14 @@ struct GemmArgs {
     const void *xh;
     const void *sxh;
     int m_rows, m_out, k_pad, units, pair_rows, steps_per_split, use_atomics, sc_off;
+    const float *rowfac;
 };
 struct XPrepArgs {
     const void *x;
     void *xh;
     void *sxh;
     int m, k, k_pad, m_rows, x_dtype;
+    float *rowfac;
 };
 
 static int x_kind(int x_dtype) {
@@ -214,9 +216,12 @@ static int launch_gemv(const void *const *xs, int xk, const rlx_qweight *const *
         }
         const size_t part_bytes = (size_t)max_tpw * kw * slot_bytes;
         sh.kcu = max_units;
-        while (sh.kcu > 1 && part_bytes + stage_bytes(sh.kcu) + 64 > budget) sh.kcu--;
-        sh.fits = part_bytes + stage_bytes(sh.kcu) + 64 <= budget;
-        sh.lds = part_bytes + stage_bytes(sh.kcu) + 64;  // the last 64 bytes: 1 / rms per activation row (RMSNorm prologue)
+        // the last LDS_TAIL bytes: 1 / rms per activation row (RMSNorm prologue), the per-row factors of the binary16 range
+        // prescale and its bookkeeping (GEMV_LDS_TAIL in kernels/gemv.hip)
+        constexpr size_t LDS_TAIL = 640;
+        while (sh.kcu > 1 && part_bytes + stage_bytes(sh.kcu) + LDS_TAIL > budget) sh.kcu--;
+        sh.fits = part_bytes + stage_bytes(sh.kcu) + LDS_TAIL <= budget;
+        sh.lds = part_bytes + stage_bytes(sh.kcu) + LDS_TAIL;
         sh.a.nseg = count;
         sh.a.m = m;
         sh.a.kc_units = sh.kcu;
@@ -285,7 +290,8 @@ static int launch_gemv(const void *const *xs, int xk, const rlx_qweight *const *
 
 struct GemmPlan {
     int64_t m_rows, k_pad;
-    size_t xh_bytes, sxh_bytes;
+    size_t xh_bytes, sxh_bytes, fac_bytes;  // the image, the Q4_K / Q5_K block sums, the per-row prescale factors
+    size_t total() const { return xh_bytes + sxh_bytes + fac_bytes; }
 };
 static GemmPlan gemm_plan(int scheme, int xk, int64_t m, int64_t k) {
     GemmPlan p;
@@ -294,7 +300,20 @@ static GemmPlan gemm_plan(int scheme, int xk, int64_t m, int64_t k) {
     p.k_pad = (k + 255) / 256 * 256;
     p.xh_bytes = ((size_t)p.m_rows * p.k_pad * 2 + 255) & ~(size_t)255;
     p.sxh_bytes = (scheme == SCHEME_Q4K || scheme == SCHEME_Q5K) ? (size_t)p.m_rows * (p.k_pad / 256) * 32 : 0;
+    p.fac_bytes = ((size_t)m * 8 + 255) & ~(size_t)255;
     return p;
+}
+
+// The conversion of x [m, k] into the workspace: one look at every row for its prescale factor, then the image.
+static int launch_xprep(const void *x, int xk, int64_t m, int64_t k, const GemmPlan &p, void *workspace, hipStream_t stream) {
+    float *fac = (float *)workspace;
+    void *xh = (uint8_t *)workspace + p.fac_bytes;
+    void *sxh = p.sxh_bytes ? (uint8_t *)workspace + p.fac_bytes + p.xh_bytes : nullptr;
+    XPrepArgs xa{x, xh, sxh, (int)m, (int)k, (int)p.k_pad, (int)p.m_rows, xk, fac};
+    void *xparams[] = {&xa};
+    RLX_TRY(launch(K_XROWSCALE, (unsigned)((m + 3) / 4), 1, 256, 0, stream, xparams));
+    const long long xblocks = (p.m_rows / 256) * (p.k_pad / 64) * 8;  // (tile, step, 32-row sub-tile)
+    return launch(K_XPREP, (unsigned)xblocks, 1, 256, 0, stream, xparams);
 }
 
 // Prefill path: convert the activations once (xprep), then the MFMA GEMM over `count` (<= GEMM_MAX_SEG) matrices of one
@@ -319,21 +338,20 @@ static int launch_gemm(const void *x, int xk, const rlx_qweight *const *ws, floa
             set_error("gguf_matmul_bt: matrices of one prefill launch differ in scheme or K");
             return RLX_ERR_INVALID;
         }
-    if (!workspace || workspace_bytes < p.xh_bytes + p.sxh_bytes) {
-        set_error("gguf_matmul_bt: m=%lld needs a %zu-byte workspace, got %zu", (long long)m, p.xh_bytes + p.sxh_bytes,
-                  workspace_bytes);
+    if (!workspace || workspace_bytes < p.total()) {
+        set_error("gguf_matmul_bt: m=%lld needs a %zu-byte workspace, got %zu", (long long)m, p.total(), workspace_bytes);
         return RLX_ERR_INVALID;
     }
     if ((uintptr_t)workspace % 16 != 0 || (uintptr_t)x % 16 != 0) {
         set_error("gguf_matmul_bt: activations and workspace must be 16-byte aligned");
         return RLX_ERR_INVALID;
     }
-    void *xh = workspace;
-    void *sxh = p.sxh_bytes ? (uint8_t *)workspace + p.xh_bytes : nullptr;
-    XPrepArgs xa{x, xh, sxh, (int)m, (int)w->dims.k, (int)p.k_pad, (int)p.m_rows, xk};
-    void *xparams[] = {&xa};
-    const long long xblocks = (p.m_rows / 256) * (p.k_pad / 64) * 8;  // (tile, step, 32-row sub-tile)
-    if (!prepared) RLX_TRY(launch(K_XPREP, (unsigned)xblocks, 1, 256, 0, stream, xparams));
+    // workspace: [per-row prescale factors][binary16 image of x][block sums], so that an image made for a scheme with
+    // block sums is found at the same place by a scheme without
+    float *fac = (float *)workspace;
+    void *xh = (uint8_t *)workspace + p.fac_bytes;
+    void *sxh = p.sxh_bytes ? (uint8_t *)workspace + p.fac_bytes + p.xh_bytes : nullptr;
+    if (!prepared) RLX_TRY(launch_xprep(x, xk, m, w->dims.k, p, workspace, stream));
 
     const int steps_per_unit = L.unit_k / 64;
     // Up to 128 activation rows run the 64-row tile (the weights are decoded once per 64 rows, but nothing is spent on
@@ -368,6 +386,7 @@ static int launch_gemm(const void *x, int xk, const rlx_qweight *const *ws, floa
     a.steps_per_split = units_per_split * steps_per_unit;
     a.use_atomics = split > 1 ? 1 : 0;
     a.sc_off = w->sc_off();
+    a.rowfac = fac;
     void *params[] = {&a};
     KernelId id = w->scheme == SCHEME_Q4K       ? (skinny ? K_GEMM64_Q4_K : K_GEMM_Q4_K)
                   : w->scheme == SCHEME_Q4_0    ? (skinny ? K_GEMM64_Q4_0 : K_GEMM_Q4_0)
@@ -505,8 +524,7 @@ size_t rlx_mi355x_gguf_matmul_workspace(int scheme, int x_dtype, int64_t m, int6
     (void)n;
     int xk = x_kind(x_dtype);
     if (xk < 0 || layout_of(scheme).unit_k == 0 || m <= decode_rows(xk)) return 0;  // decode path: no workspace
-    GemmPlan p = gemm_plan(scheme, xk, m, k);
-    return p.xh_bytes + p.sxh_bytes;
+    return gemm_plan(scheme, xk, m, k).total();
 }
 
 int rlx_mi355x_gguf_matmul_bt_batch(const void *const *xs_dev, int x_dtype, const rlx_qweight *const *ws,
@@ -588,14 +606,11 @@ int rlx_mi355x_gguf_matmul_prepare(const void *x_dev, int x_dtype, int scheme, i
         return RLX_ERR_INVALID;
     }
     const GemmPlan p = gemm_plan(scheme, xk, m, k);
-    if (!workspace || workspace_bytes < p.xh_bytes + p.sxh_bytes || (uintptr_t)workspace % 16 != 0 || (uintptr_t)x_dev % 16 != 0) {
-        set_error("gguf_matmul_prepare: a 16-byte aligned workspace of %zu bytes is needed, got %zu", p.xh_bytes + p.sxh_bytes, workspace_bytes);
+    if (!workspace || workspace_bytes < p.total() || (uintptr_t)workspace % 16 != 0 || (uintptr_t)x_dev % 16 != 0) {
+        set_error("gguf_matmul_prepare: a 16-byte aligned workspace of %zu bytes is needed, got %zu", p.total(), workspace_bytes);
         return RLX_ERR_INVALID;
     }
-    XPrepArgs xa{x_dev, workspace, p.sxh_bytes ? (uint8_t *)workspace + p.xh_bytes : nullptr, (int)m, (int)k, (int)p.k_pad, (int)p.m_rows, xk};
-    void *xparams[] = {&xa};
-    const long long xblocks = (p.m_rows / 256) * (p.k_pad / 64) * 8;
-    return launch(K_XPREP, (unsigned)xblocks, 1, 256, 0, (hipStream_t)stream, xparams);
+    return launch_xprep(x_dev, xk, m, k, p, workspace, (hipStream_t)stream);
 }
 
 int rlx_mi355x_gguf_matmul_bt_prepared(const void *workspace, size_t workspace_bytes, int x_dtype, const rlx_qweight *const *ws,

@@ -42,6 +42,7 @@ struct GemmArgs {
     int steps_per_split;  // 64-column steps per grid.z slice (a multiple of 4)
     int use_atomics;      // split K: accumulate into a zeroed `out` with atomic adds
     int sc_off;           // Q6_K: a stored scale byte stands for byte - sc_off (0 unsigned reading, 128 signed)
+    const float *rowfac;  // [m_out][2]: the power of two row i of x was multiplied by when it was converted, and its inverse
 };
 
 // half2 (v, v) with v = byte `byte` of word as an exact binary16 integer: bytes [b, 0x64, b, 0x64] = 1024 + b
@@ -461,6 +462,7 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
                     orow = vrow >> 1;
                 }
                 if (orow < a.m_out) {
+                    v *= a.rowfac[2 * orow + 1];  // undo the row's prescale (1 for a row binary16 carries as it is)
                     float *p = sg.out + (long long)orow * sg.n + col;
                     if (a.use_atomics) atomicAdd(p, v);
                     else __builtin_nontemporal_store(v, p);  // written once, read by another kernel: keep it out of the way of the operands
@@ -479,7 +481,53 @@ struct XPrepArgs {
     half_t *sxh;  // may be null
     int m, k, k_pad, m_rows;
     int x_dtype;  // 0 f32 (rows become hi / lo*2048 pairs), 1 bf16, 2 f16
+    float *rowfac;  // [m][2] (forward factor, its inverse), written by rlx_xrowscale before rlx_xprep runs
 };
+
+// Activations travel as binary16, and so do the sums of 32 of them that the Q4_K / Q5_K min term needs. rlx_xrowscale
+// looks at every row of x once: a row with some |x| >= 2^10, or with no |x| >= 2^-8 at all, gets the power of two that
+// puts its largest value in [2^9, 2^10) (a sum of 32 such values stays below 2^15); every other row gets 1.
+// rlx_xprep multiplies by it while converting and the GEMM epilogue multiplies the finished sums by its inverse, both
+// exact, so the f32 range the reference computes in (rlx-cpu/src/gguf_matmul.rs:65-94) is kept. binary16 inputs are
+// carried as they are. One wave per row.
+__device__ __forceinline__ void xrowscale_body(const XPrepArgs &a) {
+    const int lane = threadIdx.x & 63;
+    const long long row = (long long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (row >= a.m) return;
+    float amax = 0.f;
+    if (a.x_dtype == 0) {
+        const float4_t *p = (const float4_t *)((const float *)a.x + row * a.k);
+        for (int c = lane; c < a.k / 4; c += 64) {
+            const float4_t v = p[c];
+#pragma unroll
+            for (int e = 0; e < 4; e++) amax = __builtin_fmaxf(amax, __builtin_fabsf(v[e]));  // a NaN is skipped
+        }
+    } else if (a.x_dtype == 1) {
+        const uint4_t *p = (const uint4_t *)((const uint16_t *)a.x + row * a.k);
+        for (int c = lane; c < a.k / 8; c += 64) {
+            const uint4_t raw = p[c];
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                amax = __builtin_fmaxf(amax, __builtin_fabsf(__builtin_bit_cast(float, raw[e] << 16)));
+                amax = __builtin_fmaxf(amax, __builtin_fabsf(__builtin_bit_cast(float, raw[e] & 0xFFFF0000u)));
+            }
+        }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) amax = __builtin_fmaxf(amax, __shfl_xor(amax, off));
+    if (lane == 0) {
+        float fwd = 1.f, back = 1.f;
+        const uint32_t mb = __builtin_bit_cast(uint32_t, amax);
+        if (a.x_dtype != 2 && mb != 0 && mb < 0x7F800000u && (amax >= 1024.0f || amax < 0.00390625f)) {
+            int e = (int)(mb >> 23) - 127;
+            e = e < -100 ? -100 : e;
+            fwd = __builtin_bit_cast(float, (uint32_t)(9 - e + 127) << 23);
+            back = __builtin_bit_cast(float, (uint32_t)(e - 9 + 127) << 23);
+        }
+        a.rowfac[2 * row] = fwd;
+        a.rowfac[2 * row + 1] = back;
+    }
+}
 
 // One workgroup of four waves per (tile, step, sub-tile); wave = k-slice, lane = slot of the 1 KB fragment block.
 __device__ __forceinline__ void xprep_body(const XPrepArgs &a) {
@@ -498,6 +546,7 @@ __device__ __forceinline__ void xprep_body(const XPrepArgs &a) {
     float v[8];
 #pragma unroll
     for (int e = 0; e < 8; e++) v[e] = 0.f;
+    const float fwd = src_row < a.m ? a.rowfac[2 * src_row] : 1.f;
     if (src_row < a.m && col < a.k) {  // k is a multiple of 32, so a chunk of 8 is inside or outside as a whole
         if (a.x_dtype == 0) {
             const float4_t *p = (const float4_t *)((const float *)a.x + src_row * a.k + col);
@@ -520,6 +569,7 @@ __device__ __forceinline__ void xprep_body(const XPrepArgs &a) {
     float sum = 0.f;
 #pragma unroll
     for (int e = 0; e < 8; e++) {
+        v[e] *= fwd;  // exact: a power of two
         half_t hi = (half_t)v[e];
         if (paired && (vrow & 1)) hi = (half_t)((v[e] - (float)hi) * GEMM_LO_SCALE);  // odd rows carry the residual
         f.h8[e] = hi;
@@ -559,3 +609,4 @@ extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64_q4_k(rlx::GemmAr
 extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64_q4_0(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q4_0, 1, 1>(a); }
 extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64_q8_0(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q8_0, 1, 1>(a); }
 extern "C" __global__ __launch_bounds__(256) void rlx_xprep(rlx::XPrepArgs a) { rlx::xprep_body(a); }
+extern "C" __global__ __launch_bounds__(256) void rlx_xrowscale(rlx::XPrepArgs a) { rlx::xrowscale_body(a); }

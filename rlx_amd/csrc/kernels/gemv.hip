@@ -63,6 +63,20 @@ struct GemvArgs {
 
 constexpr int XS_PAD_HALFS = 8;      // 16 bytes of padding per LDS row: rows land in different bank groups
 constexpr float LO_SCALE = 2048.0f;  // f32 activation x = hi + lo / LO_SCALE with hi, lo binary16
+
+// The last GEMV_LDS_TAIL bytes of a workgroup's LDS: [0,64) 1 / rms per activation row (RMSNorm prologue); then two
+// copies of GEMV_RANGE_AREA bytes, used by alternate K chunks (a wave that is still banking the sums of one chunk must
+// not see the next chunk's factors): [0,128) un-scale factor per virtual activation row (1 unless the row was
+// prescaled, below); [128,256) per logical row: bits of max |x| of the staged chunk, then reused for the forward
+// scale; [256,264) two row masks.
+//
+// Activations travel as binary16. A row whose values leave the range binary16 carries well - some |x| >= 2^15, or no
+// |x| >= 2^-8 at all - is multiplied by a power of two that puts its largest value in [2^14, 2^15) while it is staged,
+// and the partial sums of that row are multiplied back when they are banked: exact, so the f32 range of the reference
+// (rlx-cpu/src/gguf_matmul.rs:65-94 computes in f32 throughout) is kept. The check is two compares per 16-byte group in
+// the staging loop; the rescaling itself runs only in workgroups that saw such a row.
+constexpr int GEMV_RANGE_AREA = 272, GEMV_LDS_TAIL = 640;
+constexpr float X_BIG = 32768.0f, X_SMALL = 0.00390625f;
 typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 
 template <int SCHEME>
@@ -311,15 +325,19 @@ __device__ __forceinline__ void compute_unit(const UnitRegs<SCHEME> &w, const ha
 // Convert one K chunk of the activations into LDS as halfs: f32 -> hi rows [0,m) + lo rows [m,2m); 16-bit -> rows [0,m).
 // Each thread issues up to eight independent loads before it converts the first one, so a chunk of many rows costs
 // one memory latency per eight groups of columns, not one per group.
-template <int XD, bool NORM = false>
+// PASS 0: stage, and note in masks[0] / masks[1] the rows with some |x| >= X_BIG / some |x| >= X_SMALL; PASS 1: only find
+// the largest |x| of every row (rowmax, as bits); PASS 2: stage again with row r multiplied by fwd[r].
+template <int XD, bool NORM = false, int PASS = 0>
 __device__ __forceinline__ void stage_x_typed(const GemvArgs &a, const GemvSeg &sg, half_t *xs, int row_stride, int k0, int kc,
-                                              const float *inv_rms = nullptr) {
+                                              const float *inv_rms = nullptr, uint32_t *masks = nullptr, uint32_t *rowmax = nullptr,
+                                              const float *fwd = nullptr) {
     constexpr int U = 8;
     constexpr int G = XD == X_F32 ? 4 : 8;  // columns per 16-byte load
     typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
     const int tid = threadIdx.x, nt = blockDim.x;
     const int groups = kc / G;  // kc is a multiple of 64
     const int total = a.m * groups;
+    uint32_t big = 0, seen = 0;
     for (int idx0 = tid; idx0 < total; idx0 += nt * U) {
         typedef typename std::conditional<XD == X_F32, float4_t, uint4_t>::type raw_t;  // 16 bytes either way
         raw_t raw[U];
@@ -339,6 +357,8 @@ __device__ __forceinline__ void stage_x_typed(const GemvArgs &a, const GemvSeg &
             const int idx = idx0 + u * nt;
             if (idx >= total) continue;
             const int row = idx / groups, c = (idx - row * groups) * G;
+            float rowscale = 1.f;
+            if constexpr (PASS == 2) rowscale = fwd[row];
             if constexpr (XD == X_F32) {
                 half4_t hi, lo;
                 float4_t gm = {1.f, 1.f, 1.f, 1.f}, bt = {0.f, 0.f, 0.f, 0.f};
@@ -350,35 +370,117 @@ __device__ __forceinline__ void stage_x_typed(const GemvArgs &a, const GemvSeg &
                         if (a.beta) bt = *(const float4_t *)(a.beta + k0 + c);
                     }
                 }
+                float amax = 0.f;
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
                     float v = raw[u][e];
                     if constexpr (NORM) v = v * scale * gm[e] + bt[e];  // in_row[i] * inv_rms * gamma[i] + beta[i], unfused
+                    if constexpr (PASS != 2) amax = __builtin_fmaxf(amax, __builtin_fabsf(v));  // a NaN is skipped
+                    if constexpr (PASS == 2) v *= rowscale;
                     hi[e] = (half_t)v;
                     // residual, scaled by 2^11 so it stays in the normal binary16 range; undone in the final sum
                     lo[e] = (half_t)((v - (float)hi[e]) * LO_SCALE);
                 }
-                *(half4_t *)(xs + row * row_stride + c) = hi;
-                *(half4_t *)(xs + (a.m + row) * row_stride + c) = lo;
+                if constexpr (PASS == 0) {
+                    big |= (amax >= X_BIG ? 1u : 0u) << row;
+                    seen |= (amax >= X_SMALL ? 1u : 0u) << row;
+                }
+                if constexpr (PASS == 1) {
+                    atomicMax(rowmax + row, __builtin_bit_cast(uint32_t, amax));
+                } else {
+                    *(half4_t *)(xs + row * row_stride + c) = hi;
+                    *(half4_t *)(xs + (a.m + row) * row_stride + c) = lo;
+                }
             } else if constexpr (XD == X_BF16) {
                 half8_t h;
+                float amax = 0.f;
 #pragma unroll
                 for (int e = 0; e < 8; e++) {
                     const uint32_t bits = ((e & 1) ? (raw[u][e >> 1] >> 16) : (raw[u][e >> 1] & 0xFFFFu)) << 16;
-                    h[e] = (half_t)__builtin_bit_cast(float, bits);
+                    float v = __builtin_bit_cast(float, bits);
+                    if constexpr (PASS != 2) amax = __builtin_fmaxf(amax, __builtin_fabsf(v));
+                    if constexpr (PASS == 2) v *= rowscale;
+                    h[e] = (half_t)v;
                 }
-                *(half8_t *)(xs + row * row_stride + c) = h;
-            } else {
+                if constexpr (PASS == 0) {
+                    big |= (amax >= X_BIG ? 1u : 0u) << row;
+                    seen |= (amax >= X_SMALL ? 1u : 0u) << row;
+                }
+                if constexpr (PASS == 1) atomicMax(rowmax + row, __builtin_bit_cast(uint32_t, amax));
+                else *(half8_t *)(xs + row * row_stride + c) = h;
+            } else {  // binary16 activations are staged as they are: nothing to gain from a scale
                 *(uint4_t *)(xs + row * row_stride + c) = raw[u];
             }
         }
     }
+    if constexpr (PASS == 0 && XD != X_F16) {  // one LDS atomic per wave and mask, and only for masks that have a bit
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            big |= __shfl_xor(big, off);
+            seen |= __shfl_xor(seen, off);
+        }
+        if ((threadIdx.x & 63) == 0) {
+            if (big) atomicOr(masks, big);
+            if (seen) atomicOr(masks + 1, seen);
+        }
+    }
 }
 
-__device__ __forceinline__ void stage_x(const GemvArgs &a, const GemvSeg &sg, half_t *xs, int row_stride, int k0, int kc) {
-    if (a.x_dtype == X_F32) stage_x_typed<X_F32>(a, sg, xs, row_stride, k0, kc);
-    else if (a.x_dtype == X_BF16) stage_x_typed<X_BF16>(a, sg, xs, row_stride, k0, kc);
-    else stage_x_typed<X_F16>(a, sg, xs, row_stride, k0, kc);
+// Stage one K chunk of a segment's activations (two barriers), rescaling rows that binary16 would not carry (three
+// more passes, taken by the whole workgroup or not at all). tail = the workgroup's GEMV_LDS_TAIL bytes. On return
+// rsv[v] holds the factor the partial sums of virtual row v must be multiplied by.
+template <int XD, bool NORM>
+__device__ __forceinline__ void stage_chunk_typed(const GemvArgs &a, const GemvSeg &sg, half_t *xs, int row_stride, int k0, int kc,
+                                                  uint8_t *tail, int parity) {
+    const float *inv_rms = (const float *)tail;
+    uint8_t *area = tail + 64 + parity * GEMV_RANGE_AREA;
+    float *rsv = (float *)area;
+    uint32_t *rowmax = (uint32_t *)(area + 128);
+    uint32_t *masks = (uint32_t *)(area + 256);
+    const int tid = threadIdx.x;
+    if (tid < 32) rsv[tid] = 1.f;
+    if (tid < 2) masks[tid] = 0;
+    __syncthreads();  // also: the previous chunk is fully consumed
+    stage_x_typed<XD, NORM, 0>(a, sg, xs, row_stride, k0, kc, inv_rms, masks);
+    __syncthreads();
+    if constexpr (XD != X_F16) {
+        const uint32_t rows = a.m >= 32 ? 0xFFFFFFFFu : ((1u << a.m) - 1u);
+        const uint32_t need = (masks[0] | ~masks[1]) & rows;  // workgroup-uniform: read after the barrier
+        if (need) {
+            if (tid < 32) rowmax[tid] = 0;
+            __syncthreads();
+            stage_x_typed<XD, NORM, 1>(a, sg, xs, row_stride, k0, kc, inv_rms, nullptr, rowmax);
+            __syncthreads();
+            if (tid < a.m) {
+                const uint32_t mb = rowmax[tid];
+                float fwd = 1.f, back = 1.f;
+                if (((need >> tid) & 1u) && mb != 0 && mb < 0x7F800000u) {  // a zero row or one with an infinity stays as it is
+                    int e = (int)(mb >> 23) - 127;
+                    e = e < -100 ? -100 : e;
+                    fwd = __builtin_bit_cast(float, (uint32_t)(14 - e + 127) << 23);   // 2^(14 - e): largest value into [2^14, 2^15)
+                    back = __builtin_bit_cast(float, (uint32_t)(e - 14 + 127) << 23);
+                }
+                rsv[tid] = back;
+                if (XD == X_F32) rsv[a.m + tid] = back;
+                ((float *)rowmax)[tid] = fwd;
+            }
+            __syncthreads();
+            stage_x_typed<XD, NORM, 2>(a, sg, xs, row_stride, k0, kc, inv_rms, nullptr, nullptr, (const float *)rowmax);
+            __syncthreads();
+        }
+    }
+}
+
+template <bool NORM>
+__device__ __forceinline__ void stage_chunk(const GemvArgs &a, const GemvSeg &sg, half_t *xs, int row_stride, int k0, int kc, uint8_t *tail,
+                                            int parity) {
+    if constexpr (NORM) {
+        stage_chunk_typed<X_F32, true>(a, sg, xs, row_stride, k0, kc, tail, parity);
+    } else {
+        if (a.x_dtype == X_F32) stage_chunk_typed<X_F32, false>(a, sg, xs, row_stride, k0, kc, tail, parity);
+        else if (a.x_dtype == X_BF16) stage_chunk_typed<X_BF16, false>(a, sg, xs, row_stride, k0, kc, tail, parity);
+        else stage_chunk_typed<X_F16, false>(a, sg, xs, row_stride, k0, kc, tail, parity);
+    }
 }
 
 // Key of (value, row) for the tied-LM-head argmax: float bits mapped to an order-preserving unsigned, then ~row, so the
@@ -487,7 +589,8 @@ __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
     for (int i = tid; i < ((MODE & GEMV_PAIRED) ? 2 : 1) * ntiles * kw * slot_floats; i += blockDim.x) part[i] = 0.f;
     // RMSNorm prologue: one wave per activation row sums the squares of the whole row (the sum is needed before any
     // element can be scaled), 1 / sqrt(mean + eps) lands in the last 64 bytes of the workgroup's LDS.
-    float *inv_rms = (float *)(smem + a.lds_bytes - 64);
+    uint8_t *tail = smem + a.lds_bytes - GEMV_LDS_TAIL;
+    float *inv_rms = (float *)tail;
     if constexpr ((MODE & GEMV_NORM) != 0) {
         for (int row = wave; row < a.m; row += nwaves) {
             const float *xr = (const float *)seg.x + (long long)row * seg.k;
@@ -511,8 +614,10 @@ __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
     const uint8_t *wbase2 = paired ? seg.w_pair + (long long)tile0 * seg.units * L.unit_bytes : wbase;
     auto vtile_ptr = [&](int vt) { return paired ? ((vt & 1) ? wbase2 : wbase) + (vt >> 1) * tile_bytes : wbase + vt * tile_bytes; };
 
-    for (int u0 = 0; u0 < seg.units; u0 += kc_units) {
+    int parity = 0;
+    for (int u0 = 0; u0 < seg.units; u0 += kc_units, parity ^= 1) {
         const int nu = min(kc_units, seg.units - u0);  // units in this chunk
+        const float *rsv = (const float *)(tail + 64 + parity * GEMV_RANGE_AREA);
         // This wave's items: for each tile, units wave, wave + nwaves, ... < nu. Two cursors walk them: `pf_*` issues
         // loads DEPTH items ahead into a register ring, `cu_*` consumes.
         // An item is UPI consecutive units (the host picks UPI > 1 only when every chunk holds a multiple of UPI).
@@ -547,10 +652,7 @@ __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
             for (int p = 0; p < UPI; p++) ring[d].u[p].clear();
             prefetch(ring[d]);
         }
-        if (u0 > 0) __syncthreads();  // previous chunk fully consumed
-        if constexpr ((MODE & GEMV_NORM) != 0) stage_x_typed<X_F32, true>(a, seg, xs, row_stride, u0 * L.unit_k, nu * L.unit_k, inv_rms);
-        else stage_x(a, seg, xs, row_stride, u0 * L.unit_k, nu * L.unit_k);
-        __syncthreads();
+        stage_chunk<(MODE & GEMV_NORM) != 0>(a, seg, xs, row_stride, u0 * L.unit_k, nu * L.unit_k, tail, parity);
         if constexpr (SCHEME == SCHEME_Q4K || SCHEME == SCHEME_Q5K) {
             const int nblk = nu * BLK_PER_UNIT;
             // rows >= rv of the [blk][16 RG] table are never read: compute_unit only uses the rows its lane group owns
@@ -593,9 +695,10 @@ __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
                         for (int rg = 0; rg < RG; rg++) {
                             if (4 * rg + g < ng) {  // this lane's four rows of the group exist
                                 float *slot = part + ((size_t)cu_t * kw + kl) * slot_floats + (4 * rg + g) * 64 + nrow;
+                                const float4_t back = *(const float4_t *)(rsv + 16 * rg + 4 * g);  // 1 unless the row was prescaled
 #pragma unroll
                                 for (int r = 0; r < 4; r++) {
-                                    if (r < NREG) slot[r * 16] += acc[rg][r];
+                                    if (r < NREG) slot[r * 16] += acc[rg][r] * back[r];
                                     acc[rg][r] = 0.f;
                                 }
                             }

@@ -727,3 +727,65 @@ def test_prefill_prepare_then_prepared(oracle, scheme, x_dtype):
         assert rel_err(got, ops.gguf_matmul_bt(xin, ws[i], m, x_dtype)) <= 1e-5, i
     with pytest.raises(rlx_amd.RlxError):  # decode sizes have no image to prepare
         rlx_amd._lib.check(L.rlx_mi355x_gguf_matmul_prepare(xd.ptr, int(x_dtype), int(scheme), 4, k, wsb.ptr, need, None))
+
+
+# ------------------------------------------------------------------ activations beyond what binary16 carries
+
+@pytest.mark.parametrize("scheme,m,k,x_dtype", [(Q4_0, 1, 4096, DType.F32), (Q4K, 3, 1024, DType.F32), (Q8_0, 7, 512, DType.BF16),
+                                                (Q4_0, 12, 1024, DType.F32), (Q4K, 20, 1024, DType.BF16),    # two row groups
+                                                (Q4_0, 4, 28672, DType.F32),                                  # several K chunks
+                                                (Q4K, 40, 1024, DType.BF16), (Q4_0, 300, 512, DType.F32),    # both prefill tiles
+                                                (Q8_0, 200, 1024, DType.BF16), (Q4K, 130, 768, DType.F32)])
+def test_activation_rows_far_outside_binary16(oracle, scheme, m, k, x_dtype):
+    # The reference computes in f32 (rlx-cpu/src/gguf_matmul.rs:65-94); here activations travel as binary16, so rows whose
+    # values leave its range (|x| around 1e5 and beyond, or tiny) are prescaled by a power of two per row and the sums
+    # scaled back. Row i of x is N(0,1) times c_i; the result must match the f64 oracle to 2e-3 of max(|y|, c_i), the
+    # reference tests' norm applied to the unscaled problem. One row keeps c = 1, one row has a lone outlier late in K.
+    say("activation range", SCHEME_NAMES[scheme], m, k, x_dtype.name)
+    n = 96
+    packed, _ = make_weights(scheme, n, k, seed=m + k)
+    rng = np.random.default_rng(m * 7 + k)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    c = np.array([[1e5, 1e-6, 1.0, 3e7, 1e-9, 1e30, 2e-20][i % 7] for i in range(m)], np.float32)
+    x = (x * c[:, None]).astype(np.float32)
+    lone = m - 1
+    c[lone] = 1.0
+    x[lone] = rng.standard_normal(k).astype(np.float32)
+    x[lone, k - 5] = np.float32(3.0e5)          # in the last K chunk only
+    c[lone] = 3.0e5 / 4.0
+    if x_dtype == DType.BF16:
+        x = oracle.bf16_round(x)
+        xin = f32_to_bf16_bits(x)
+    else:
+        xin = x
+    w = ops.QWeight(scheme, packed, n, k)
+    got = ops.gguf_matmul_bt(xin, w, m, x_dtype)
+    w.free()
+    assert np.all(np.isfinite(got))
+    ref = oracle.gguf_matmul_f64(x, packed, m, k, n, scheme)
+    err = np.abs(got.astype(np.float64) - ref) / np.maximum(np.abs(ref), c[:, None].astype(np.float64))
+    say("   worst row errors:", np.max(err, axis=1)[:8])
+    assert float(np.max(err)) <= TOL
+
+
+def test_activation_range_through_fused_entry_points(oracle):
+    # the RMSNorm prologue normalizes before the range check; the SwiGLU epilogue and the MoE routing see rescaled rows
+    k, n = 1024, 64
+    rng = np.random.default_rng(77)
+    pu, _ = make_weights(Q4_0, n, k, seed=78)
+    pg, _ = make_weights(Q4_0, n, k, seed=79)
+    wu, wg = ops.QWeight(Q4_0, pu, n, k), ops.QWeight(Q4_0, pg, n, k)
+    x = (rng.standard_normal((2, k)) * np.array([[2e5], [1.0]])).astype(np.float32)
+    gamma = np.ones(k, np.float32)
+    got = ops.rmsnorm_gguf_matmul_bt_batch(x, gamma, None, 1e-5, [wu], 2)[0]
+    xn = oracle.rms_norm(x, gamma, np.zeros(k, np.float32), 1e-5)
+    assert rel_err(got, oracle.gguf_matmul_f64(xn, pu, 2, k, n, Q4_0)) <= TOL
+    big = (rng.standard_normal((2, k)) * 1e5).astype(np.float32)
+    plain = ops.gguf_matmul_bt(big, wu, 2)
+    ref = oracle.gguf_matmul_f64(big, pu, 2, k, n, Q4_0)
+    assert np.max(np.abs(plain - ref) / np.maximum(np.abs(ref), 1e5)) <= TOL
+    idx = np.array([0.0, 0.0], np.float32)
+    routed = ops.gguf_grouped_matmul_bt(big, wu, idx)
+    assert np.array_equal(routed.view(np.uint32), plain.view(np.uint32))
+    wu.free()
+    wg.free()
