@@ -637,6 +637,36 @@ def gemm_configs(rlx_amd, stream):
     out["q8_0_gemm_m8192_4096x4096_f32"] = {"us": round(ms * 1e3, 2), "TFLOP/s": round(tf, 1),
                                           "frac_mfma_f16": round(tf / MFMA_F16_PEAK_TFLOPS, 4),
                                           "note": "f32 activations run as hi + lo f16 rows: two MFMA rows per token"}
+    # the whole chain both ways: FakeQuantize writing f32 and the matmul converting it again, against FakeQuantize
+    # writing the matmul's operand image directly (no f32 tensor, no conversion pass)
+    rows, cols = 8192, 4096
+    xq = ops.philox_normal(9, rows * cols)
+    xq[ops.philox_uniform(19, rows * cols) < np.float32(0.001)] *= np.float32(20.0)
+    xd, fd, yd = ops.DeviceBuffer.from_numpy(xq), ops.DeviceBuffer(rows * cols * 4), ops.DeviceBuffer(rows * 4096 * 4)
+    scratch = ops.DeviceBuffer(L.rlx_mi355x_fake_quantize_scratch_bytes(rows * cols, cols, 1))
+    need = ops.matmul_workspace_bytes(qw[0], DType.F32, rows)
+    ws = ops.DeviceBuffer(need)
+    w_arr = (rlx_amd._lib.C.c_void_p * 1)(qw[0].ptr)
+    y_arr = (rlx_amd._lib.C.c_void_p * 1)(yd.ptr)
+
+    def chain_f32():
+        rlx_amd._lib.check(L.rlx_mi355x_fake_quantize(xd.ptr, fd.ptr, None, rows * cols, cols, 1, 8, 0, 0.0, None, 0, scratch.ptr, stream))
+        rlx_amd._lib.check(L.rlx_mi355x_gguf_matmul_bt(fd.ptr, int(DType.F32), qw[0].ptr, yd.ptr, rows, ws.ptr, need, stream))
+
+    def chain_image():
+        rlx_amd._lib.check(L.rlx_mi355x_fake_quantize_image(xd.ptr, None, None, rows, cols, 8, 0, 0.0, None, 0, scratch.ptr, ws.ptr, need, stream))
+        rlx_amd._lib.check(L.rlx_mi355x_gguf_matmul_bt_prepared(ws.ptr, need, int(DType.F32), w_arr, y_arr, 1, rows, stream))
+
+    def fq_image_only():
+        rlx_amd._lib.check(L.rlx_mi355x_fake_quantize_image(xd.ptr, None, None, rows, cols, 8, 0, 0.0, None, 0, scratch.ptr, ws.ptr, need, stream))
+
+    ms_a = time_launches(ops, stream, chain_f32, 30, 5)
+    ms_b = time_launches(ops, stream, chain_image, 30, 5)
+    ms_c = time_launches(ops, stream, fq_image_only, 60, 10)
+    out["fq_then_q8_0_gemm_8192x4096x4096"] = {
+        "us_fq_f32_then_matmul": round(ms_a * 1e3, 2), "us_fq_image_then_prepared_matmul": round(ms_b * 1e3, 2),
+        "us_fq_image_alone": round(ms_c * 1e3, 2),
+        "note": "the image holds hi + lo binary16 rows: one row alone was 2.8e-3 from the f64 result, above the 2e-3 bound"}
     qw[0].free()
 
     # config 5: Q4_0 batch sweep over the seven projections of one Llama-3-70B layer, bf16 activations

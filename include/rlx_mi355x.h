@@ -251,6 +251,18 @@ int rlx_mi355x_fake_quantize(const float *x_dev, float *out_dev, int8_t *codes_d
                              int64_t inner, int bits, int scale_mode, float ema_decay, float *state_dev,
                              int round_mode, void *scratch_dev, void *stream);
 
+/* FakeQuantize whose result feeds prefill matmuls (the benchmark's FakeQuantize -> Q8_0 GEMM chain): x is [m, k] with one
+ * channel per column (the layout of axis = last). Besides out_dev - which may be NULL here: the f32 tensor is then never
+ * written - the apply pass writes the binary16 image of the result into `workspace`, in the form
+ * rlx_mi355x_gguf_matmul_bt_prepared(workspace, .., RLX_F32, ..) reads (two binary16 rows per row, as for any f32
+ * activation), so the result needs no round trip through HBM as f32 and no conversion pass.
+ * workspace: rlx_mi355x_gguf_matmul_workspace(scheme, RLX_F32, m, k, 0) bytes of a scheme without block sums (any but
+ * Q4_K / Q5_K). k % 8 == 0. No counterpart in the reference, whose thunks exchange f32 tensors; the graph
+ * level uses it when every consumer of a FakeQuantize node is such a matmul. */
+int rlx_mi355x_fake_quantize_image(const float *x_dev, float *out_dev, int8_t *codes_dev, int64_t m, int64_t k, int bits,
+                                   int scale_mode, float ema_decay, float *state_dev, int round_mode, void *scratch_dev,
+                                   void *workspace, size_t workspace_bytes, void *stream);
+
 /* rlx_mi355x_fake_quantize for callers that cannot allocate (a stream capture in progress, tight serving loops,
  * harnesses that forbid hipMalloc). No counterpart in the reference. Same arguments without `scratch_dev`: the scratch is
  * a device array inside the library image, rlx_mi355x_fake_quantize_noalloc_max_scratch() = 8 MiB per GPU, held until

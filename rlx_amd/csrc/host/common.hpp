@@ -36,7 +36,7 @@ void clear_error();
 
 enum KernelId : int {
     K_DEQUANT_Q4_0, K_DEQUANT_Q8_0, K_DEQUANT_Q4_K, K_DEQUANT_Q6_K, K_DEQUANT_Q5_K,
-    K_FQ_COL_ABSMAX, K_FQ_SEG_ABSMAX, K_FQ_FLAT_ABSMAX, K_FQ_SCALE, K_FQ_SCALE_PARTS, K_FQ_COL_APPLY, K_FQ_FLAT_APPLY, K_FQ_FLAT4_APPLY,
+    K_FQ_COL_ABSMAX, K_FQ_SEG_ABSMAX, K_FQ_FLAT_ABSMAX, K_FQ_SCALE, K_FQ_SCALE_PARTS, K_FQ_COL_APPLY, K_FQ_COL_APPLY_IMG, K_FQ_FLAT_APPLY, K_FQ_FLAT4_APPLY,
     K_FILL_U32, K_COPY_U128,
     // decode GEMV: per scheme {r2, r4, r2_argmax, r2_paired, r4_paired, r2_norm, r4_norm, r2_norm_paired, r4_norm_paired,
     // r2_norm_argmax}, in this order (launch_gemv indexes into it)

@@ -24,6 +24,9 @@ extern "C" int rlx_mi355x_qweight_create_ex(int, uint32_t, const void *, size_t,
 extern "C" int rlx_mi355x_gguf_grouped_matmul_bt(const void *, int, const rlx_qweight *, const float *, float *, int64_t, void *);
 extern "C" int rlx_mi355x_gguf_matmul_bt_batch(const void *const *, int, const rlx_qweight *const *, float *const *, int, int64_t,
                                                void *, size_t, void *);
+extern "C" int rlx_mi355x_gguf_matmul_bt_prepared(const void *, size_t, int, const rlx_qweight *const *, float *const *, int, int64_t, void *);
+extern "C" int rlx_mi355x_fake_quantize_image(const float *, float *, int8_t *, int64_t, int64_t, int, int, float, float *, int, void *, void *,
+                                              size_t, void *);
 
 namespace {
 
@@ -79,6 +82,12 @@ struct Node {
     int64_t w_n = 0, w_k = 0, w_experts = 1;
     rlx_qweight *qw = nullptr;
     uint32_t w_flags = 0;  // rlx_qweight_flags the weight is created with
+    // FakeQuantize feeding prefill matmuls of one later step: its apply pass writes their binary16 image straight into
+    // that step's workspace (img_step = index of the step, -1 otherwise); the f32 tensor is written only when something
+    // else reads it (keep_f32). A DequantMatMul with x_image reads its activations from the step's workspace.
+    int img_step = -1;
+    bool keep_f32 = true;
+    bool x_image = false;  // (an f32 image: two binary16 rows per activation row)
 };
 
 // f32 <-> half / bfloat16 as the reference's typed boundary does (rlx-driver/src/arena.rs:69-119, `half` crate).
@@ -403,6 +412,43 @@ static std::unique_ptr<rlx_exec> plan_graph(const rlx_graph_desc *g, const rlx_c
         e->steps.push_back(step);
     }
 
+    // FakeQuantize -> prefill DequantMatMul: when every reader of a FakeQuantize result is a prefill matmul of one step
+    // (and of a scheme whose kernel needs no block sums), the apply pass writes the matmuls' binary16 image itself and
+    // the f32 tensor never goes through memory; when other readers exist both are written.
+    {
+        std::vector<int> step_idx(e->nodes.size(), -1);
+        for (size_t si = 0; si < e->steps.size(); si++)
+            for (uint32_t id : e->steps[si]) step_idx[id] = (int)si;
+        for (uint32_t f = 0; f < g->n_nodes; f++) {
+            Node &fq = e->nodes[f];
+            if (fq.d.op_kind != RLX_OP_FAKE_QUANTIZE || fq.inner != 1 || fq.chan_dim % 8 != 0 || fq.numel % fq.chan_dim != 0) continue;
+            int target = -1;
+            bool ok = true, other_reader = false;
+            std::vector<uint32_t> mms;
+            for (uint32_t j = f + 1; j < g->n_nodes && ok; j++) {
+                Node &o = e->nodes[j];
+                for (uint32_t t = 0; t < o.d.n_inputs; t++) {
+                    if (o.d.inputs[t] != f) continue;
+                    const bool as_x = o.d.op_kind == RLX_OP_DEQUANT_MATMUL && t == 0 && o.m > 16 && o.k == fq.chan_dim &&
+                                      o.d.scheme != SCHEME_Q4K && o.d.scheme != SCHEME_Q5K;
+                    if (!as_x) {
+                        other_reader = true;
+                    } else if (target >= 0 && step_idx[j] != target) {
+                        ok = false;  // matmuls of two different steps: each step has a workspace of its own
+                    } else {
+                        target = step_idx[j];
+                        mms.push_back(j);
+                    }
+                }
+            }
+            for (uint32_t id : e->outputs) other_reader = other_reader || id == f;
+            if (!ok || target < 0) continue;
+            fq.img_step = target;
+            fq.keep_f32 = other_reader;
+            for (uint32_t j : mms) e->nodes[j].x_image = true;
+        }
+    }
+
     // Memory plan: one arena. Sources (inputs, params, constants), graph outputs and requested FakeQuantize codes
     // live for the whole run; every other buffer lives from the step that writes it to the last step that reads it
     // (a prefill workspace: its own step only), and a buffer may take the bytes of one that is dead by then:
@@ -468,7 +514,8 @@ static std::unique_ptr<rlx_exec> plan_graph(const rlx_graph_desc *g, const rlx_c
         size_t step_ws = 0;
         for (uint32_t id : step) {
             Node &nd = e->nodes[id];
-            nd.slot = take((size_t)nd.numel * dtype_size(nd.d.dtype), (int)si, last_use[id]);
+            if (!(nd.img_step >= 0 && !nd.keep_f32))  // a FakeQuantize result that only travels as a prefill image has no slot
+                nd.slot = take((size_t)nd.numel * dtype_size(nd.d.dtype), (int)si, last_use[id]);
             if (nd.d.op_kind == RLX_OP_FAKE_QUANTIZE) {
                 nd.aux = take(rlx_mi355x_fake_quantize_scratch_bytes(nd.numel, nd.chan_dim, nd.inner), (int)si, (int)si);
                 if (e->opts.fq_emit_codes) nd.codes = take((size_t)nd.numel, (int)si, kForever);
@@ -476,7 +523,12 @@ static std::unique_ptr<rlx_exec> plan_graph(const rlx_graph_desc *g, const rlx_c
             if (nd.d.op_kind == RLX_OP_DEQUANT_MATMUL && nd.m > 16)  // may run the prefill kernels (which one is decided by the input dtype at run time): sized for f32
                 step_ws = std::max(step_ws, rlx_mi355x_gguf_matmul_workspace((int)nd.d.scheme, RLX_F32, nd.m, nd.k, nd.n));
         }
-        if (step_ws) e->nodes[step[0]].aux = take(step_ws, (int)si, (int)si);  // one workspace for the whole step
+        if (step_ws) {  // one workspace for the whole step; it is born earlier when a FakeQuantize writes the step's image into it
+            int birth = (int)si;
+            for (const Node &fq : e->nodes)
+                if (fq.img_step == (int)si) birth = std::min(birth, step_of[&fq - e->nodes.data()]);
+            e->nodes[step[0]].aux = take(step_ws, birth, (int)si);
+        }
     }
     e->arena_bytes = arena_end;
     return e;
@@ -639,6 +691,24 @@ static int enqueue_schedule(rlx_exec *e) {
             std::stable_sort(order.begin(), order.end(), [&](uint32_t a, uint32_t b) {
                 return e->nodes[a].d.inputs[0] < e->nodes[b].d.inputs[0];
             });
+            {  // matmuls whose activations a FakeQuantize left in the workspace as a binary16 image: first, while it is intact
+                std::vector<const rlx_qweight *> iw;
+                std::vector<float *> io;
+                for (uint32_t id : order) {
+                    Node &mm = e->nodes[id];
+                    if (!mm.x_image) continue;
+                    Node &w = e->nodes[mm.d.inputs[1]];
+                    if (!w.qw) {
+                        set_error("run: packed weight '%s' was never set (set_param_typed(.., U8))", w.name.c_str());
+                        return RLX_ERR_INVALID;
+                    }
+                    iw.push_back(w.qw);
+                    io.push_back((float *)e->ptr(mm.slot));
+                }
+                if (!iw.empty())
+                    RLX_TRY(rlx_mi355x_gguf_matmul_bt_prepared(e->ptr(nd.aux), nd.aux.size, RLX_F32, iw.data(), io.data(), (int)iw.size(), nd.m,
+                                                               e->stream));
+            }
             std::vector<const rlx_qweight *> ws;
             std::vector<float *> outs;
             std::vector<const void *> xs;
@@ -654,6 +724,7 @@ static int enqueue_schedule(rlx_exec *e) {
             };
             for (uint32_t id : order) {
                 Node &mm = e->nodes[id];
+                if (mm.x_image) continue;
                 Node &x = e->nodes[mm.d.inputs[0]];
                 Node &w = e->nodes[mm.d.inputs[1]];
                 if (!w.qw) {
@@ -675,6 +746,14 @@ static int enqueue_schedule(rlx_exec *e) {
                 return RLX_ERR_INVALID;
             }
             float *state = nd.d.n_inputs == 2 ? (float *)e->ptr(e->nodes[nd.d.inputs[1]].slot) : nullptr;
+            if (nd.img_step >= 0) {
+                const Slot &ws = e->nodes[e->steps[nd.img_step][0]].aux;
+                RLX_TRY(rlx_mi355x_fake_quantize_image((const float *)e->ptr(x.slot), nd.keep_f32 ? (float *)e->ptr(nd.slot) : nullptr,
+                                                       nd.codes.size ? (int8_t *)e->ptr(nd.codes) : nullptr, nd.numel / nd.chan_dim, nd.chan_dim,
+                                                       (int)nd.d.bits, (int)nd.d.scale_mode, nd.d.ema_decay, state, (int)e->opts.fq_round_mode,
+                                                       e->ptr(nd.aux), e->ptr(ws), ws.size, e->stream));
+                continue;
+            }
             RLX_TRY(rlx_mi355x_fake_quantize((const float *)e->ptr(x.slot), (float *)e->ptr(nd.slot),
                                              nd.codes.size ? (int8_t *)e->ptr(nd.codes) : nullptr, nd.numel, nd.chan_dim, nd.inner, (int)nd.d.bits,
                                              (int)nd.d.scale_mode, nd.d.ema_decay, state, (int)e->opts.fq_round_mode,
@@ -823,6 +902,8 @@ int rlx_exec_describe_plan(const rlx_exec *e, char *buf, size_t cap) {
             put(" chan_dim=%lld inner=%lld aux@%zu codes@%zu+%zu", (long long)nd.chan_dim, (long long)nd.inner, nd.aux.offset, nd.codes.offset,
                 nd.codes.size);
         if (nd.d.op_kind == RLX_OP_DEQUANT_MATMUL && nd.aux.size) put(" step workspace@%zu+%zu", nd.aux.offset, nd.aux.size);
+        if (nd.img_step >= 0) put(" -> prefill image of step %d%s", nd.img_step, nd.keep_f32 ? "" : " (f32 tensor not written)");
+        if (nd.x_image) put(" [x: binary16 image]");
         put("\n");
     }
     return RLX_OK;

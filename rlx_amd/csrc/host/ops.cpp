@@ -70,6 +70,9 @@ struct FqArgs {
     int scale_mode, round_mode, rows_per_block;
     float *partial;
     int parts;
+    void *img;
+    float *rowfac;
+    int k_pad, m_rows, write_out;
 };
 
 constexpr int GEMM_MAX_SEG = 4;
@@ -942,9 +945,11 @@ size_t rlx_mi355x_fake_quantize_scratch_bytes(int64_t len, int64_t chan_dim, int
     return (size_t)chan_dim * 8 + (p.col ? (size_t)p.gy_absmax * chan_dim * 4 : 0);
 }
 
-int rlx_mi355x_fake_quantize(const float *x_dev, float *out_dev, int8_t *codes_dev, int64_t len, int64_t chan_dim,
-                             int64_t inner, int bits, int scale_mode, float ema_decay, float *state_dev,
-                             int round_mode, void *scratch_dev, void *stream) {
+// img_ws != nullptr: column layout only; the apply pass also writes the prefill image of the result (and its per-row
+// factors) into img_ws, and skips the f32 tensor when out_dev is null.
+static int fake_quantize_impl(const float *x_dev, float *out_dev, int8_t *codes_dev, int64_t len, int64_t chan_dim,
+                              int64_t inner, int bits, int scale_mode, float ema_decay, float *state_dev,
+                              int round_mode, void *scratch_dev, void *stream, void *img_ws, size_t img_ws_bytes) {
     using namespace rlx;
     float q_max;
     switch (bits) {
@@ -957,7 +962,7 @@ int rlx_mi355x_fake_quantize(const float *x_dev, float *out_dev, int8_t *codes_d
     }
     if (chan_dim < 1) chan_dim = 1;
     if (inner < 1) inner = 1;
-    if (!x_dev || !out_dev || !scratch_dev || len < 0 || scale_mode < 0 || scale_mode > 2) {
+    if (!x_dev || (!out_dev && !img_ws) || !scratch_dev || len < 0 || scale_mode < 0 || scale_mode > 2) {
         set_error("FakeQuantize: null buffer, negative length or bad scale mode %d", scale_mode);
         return RLX_ERR_INVALID;
     }
@@ -972,9 +977,19 @@ int rlx_mi355x_fake_quantize(const float *x_dev, float *out_dev, int8_t *codes_d
     const FqColPlan plan = fq_col_plan(len, chan_dim, inner);
     // the scratch is sized for the column plan whether or not the pointers allow it, so alignment only picks kernels
     const bool col = plan.col && ((uintptr_t)x_dev % 16 == 0) && ((uintptr_t)out_dev % 16 == 0) &&
-                     ((uintptr_t)scratch_dev % 16 == 0) && (!codes_dev || (uintptr_t)codes_dev % 4 == 0);
+                     ((uintptr_t)scratch_dev % 16 == 0) && (!codes_dev || (uintptr_t)codes_dev % 8 == 0 || (!img_ws && (uintptr_t)codes_dev % 4 == 0));
     FqArgs a{x_dev, out_dev, codes_dev, max_bits, scale, state_dev, len, chan_dim, inner, q_max, ema_decay,
-             scale_mode, round_mode, 0, nullptr, 0};
+             scale_mode, round_mode, 0, nullptr, 0, nullptr, nullptr, 0, 0, 1};
+    GemmPlan ip{};
+    if (img_ws) {
+        const int64_t m = chan_dim > 0 ? len / chan_dim : 0;
+        ip = gemm_plan(SCHEME_Q8_0, 0, m, chan_dim);  // the image of an f32 tensor (hi / lo row pairs), no block sums
+        if (!col || chan_dim % 8 != 0 || (uintptr_t)img_ws % 16 != 0 || img_ws_bytes < ip.total()) {
+            set_error("FakeQuantize: the prefill image needs column channels in multiples of 8, 16-byte aligned buffers and %zu bytes of workspace",
+                      ip.total());
+            return RLX_ERR_INVALID;
+        }
+    }
     void *params[] = {&a};
     if (scale_mode != RLX_SCALE_FIXED) {
         if (col) {
@@ -998,7 +1013,17 @@ int rlx_mi355x_fake_quantize(const float *x_dev, float *out_dev, int8_t *codes_d
     }
     if (a.partial) RLX_TRY(launch(K_FQ_SCALE_PARTS, (unsigned)((chan_dim + 63) / 64), 1, 1024, 0, s, params));
     else RLX_TRY(launch(K_FQ_SCALE, (unsigned)((chan_dim + 255) / 256), 1, 256, 0, s, params));
-    if (col) {
+    if (img_ws) {
+        a.img = (uint8_t *)img_ws + ip.fac_bytes;
+        a.rowfac = (float *)img_ws;
+        a.k_pad = (int)ip.k_pad;
+        a.m_rows = (int)ip.m_rows;
+        a.write_out = out_dev ? 1 : 0;
+        const unsigned gx = (unsigned)((ip.k_pad + 255) / 256);
+        const int64_t want = std::max<int64_t>(1, 4096 / gx), lrows = ip.m_rows / 2;  // logical rows, padding included (a multiple of 128)
+        a.rows_per_block = (int)std::max<int64_t>(16, ((lrows + want - 1) / want + 15) / 16 * 16);
+        RLX_TRY(launch(K_FQ_COL_APPLY_IMG, gx, (unsigned)((lrows + a.rows_per_block - 1) / a.rows_per_block), 256, 0, s, params));
+    } else if (col) {
         a.rows_per_block = plan.rpb_apply;
         RLX_TRY(launch(K_FQ_COL_APPLY, plan.gx, plan.gy_apply, 256, 0, s, params));
     } else {
@@ -1009,6 +1034,24 @@ int rlx_mi355x_fake_quantize(const float *x_dev, float *out_dev, int8_t *codes_d
         RLX_TRY(launch(v4 ? K_FQ_FLAT4_APPLY : K_FQ_FLAT_APPLY, blocks, 1, 256, 0, s, params));
     }
     return RLX_OK;
+}
+
+int rlx_mi355x_fake_quantize(const float *x_dev, float *out_dev, int8_t *codes_dev, int64_t len, int64_t chan_dim,
+                             int64_t inner, int bits, int scale_mode, float ema_decay, float *state_dev,
+                             int round_mode, void *scratch_dev, void *stream) {
+    return fake_quantize_impl(x_dev, out_dev, codes_dev, len, chan_dim, inner, bits, scale_mode, ema_decay, state_dev, round_mode,
+                              scratch_dev, stream, nullptr, 0);
+}
+
+int rlx_mi355x_fake_quantize_image(const float *x_dev, float *out_dev, int8_t *codes_dev, int64_t m, int64_t k, int bits,
+                                   int scale_mode, float ema_decay, float *state_dev, int round_mode, void *scratch_dev,
+                                   void *workspace, size_t workspace_bytes, void *stream) {
+    if (!workspace || m <= 0 || k <= 0) {
+        rlx::set_error("fake_quantize_image: null workspace or empty tensor");
+        return RLX_ERR_INVALID;
+    }
+    return fake_quantize_impl(x_dev, out_dev, codes_dev, m * k, k, 1, bits, scale_mode, ema_decay, state_dev, round_mode, scratch_dev,
+                              stream, workspace, workspace_bytes);
 }
 
 }  // extern "C"

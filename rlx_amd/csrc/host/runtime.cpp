@@ -23,7 +23,7 @@ const char *last_error_cstr() { return g_error.c_str(); }
 
 static const char *const kKernelNames[K_COUNT] = {
     "rlx_dequant_q4_0", "rlx_dequant_q8_0", "rlx_dequant_q4_k", "rlx_dequant_q6_k", "rlx_dequant_q5_k",
-    "rlx_fq_col_absmax", "rlx_fq_seg_absmax", "rlx_fq_flat_absmax", "rlx_fq_scale", "rlx_fq_scale_parts", "rlx_fq_col_apply",
+    "rlx_fq_col_absmax", "rlx_fq_seg_absmax", "rlx_fq_flat_absmax", "rlx_fq_scale", "rlx_fq_scale_parts", "rlx_fq_col_apply", "rlx_fq_col_apply_img",
     "rlx_fq_flat_apply", "rlx_fq_flat4_apply",
     "rlx_fill_u32", "rlx_copy_u128",
     "rlx_gemv_q4_0_r2", "rlx_gemv_q4_0_r4", "rlx_gemv_q4_0_r2_argmax", "rlx_gemv_q4_0_r2_paired", "rlx_gemv_q4_0_r4_paired",

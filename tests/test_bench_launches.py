@@ -141,11 +141,13 @@ def test_llama70b_layer_batch_sweep(oracle, llama70b, m):
 
 # ------------------------------------------------------------------ FakeQuantize -> Q8_0 GEMM at full size
 
-def test_config4_chain_full_size(oracle):
+@pytest.mark.parametrize("fq_is_output", [True, False])
+def test_config4_chain_full_size(oracle, fq_is_output):
     # benchmark configuration 4 as one executable: FakeQuantize [8192, 4096] (int8, per column) feeding a Q8_0
-    # DequantMatMul against a 4096 x 4096 weight. Codes bit-exact over all 33.5 M elements; y against the f64 oracle
-    # applied to the oracle's fake-quantized tensor, on column windows over all 8192 rows and on a band of rows over
-    # every column.
+    # DequantMatMul against a 4096 x 4096 weight. The apply pass writes the matmul's binary16 image itself; with the
+    # fake-quantized tensor not an output, its f32 form never goes through memory. Codes bit-exact over all 33.5 M
+    # elements; y against the f64 oracle applied to the oracle's fake-quantized tensor, on column windows over all 8192
+    # rows and on a band of rows over every column.
     rows, k, n = 8192, 4096, 4096
     rng = np.random.default_rng(61)
     x = rng.standard_normal((rows, k)).astype(np.float32)
@@ -156,13 +158,16 @@ def test_config4_chain_full_size(oracle):
     fq = g.add_node(Op.FakeQuantize(8, 1), [xi], Shape.new([rows, k], DType.F32))
     w = g.param("w", Shape.new([len(packed)], DType.U8))
     y = g.add_node(Op.DequantMatMul(QuantScheme.GgufQ8_0), [fq, w], Shape.new([rows, n], DType.F32))
-    g.set_outputs([y, fq])
+    g.set_outputs([y, fq] if fq_is_output else [y])
     c = Session(fq_codes=True).compile(g)
+    plan = c.describe_plan()
+    assert "prefill image" in plan and ("f32 tensor not written" in plan) == (not fq_is_output)
     c.set_param_typed("w", packed, DType.U8)
-    y_got, fq_got = c.run([("x", x)])
-    y_got = y_got.reshape(rows, n)
+    outs = c.run([("x", x)])
+    y_got = outs[0].reshape(rows, n)
     fq_ref, codes_ref, _ = oracle.fake_quantize(x, x.shape, 1, 8)
-    assert np.array_equal(fq_got.reshape(rows, k).view(np.uint32), fq_ref.view(np.uint32))
+    if fq_is_output:
+        assert np.array_equal(outs[1].reshape(rows, k).view(np.uint32), fq_ref.view(np.uint32))
     assert np.array_equal(c.fq_codes(fq).reshape(rows, k), codes_ref)
     for n0 in (0, 2040, n - 24):
         err = rel_err(y_got[:, n0:n0 + 24], oracle.gguf_matmul_f64(fq_ref, packed, rows, k, n, Q8_0, n0, n0 + 24))
@@ -172,3 +177,33 @@ def test_config4_chain_full_size(oracle):
         err = rel_err(y_got[r0:r0 + 6], oracle.gguf_matmul_f64(fq_ref[r0:r0 + 6], packed, 6, k, n, Q8_0))
         say(f"   config 4 chain, rows {r0}..{r0 + 6}, all columns: max rel err {err:.3e}")
         assert err <= TOL
+
+
+def test_fq_image_chain_ragged_and_out_of_range(oracle):
+    # the same chain at a ragged shape (m not a multiple of 256, k not of 256, two matmuls on the fake-quantized tensor) and
+    # with inputs far outside binary16: the tensor-wide power of two keeps the image in range
+    rows, k, ns = 300, 1056, [96, 40]
+    rng = np.random.default_rng(63)
+    for scale in (1.0, 3.0e6, 1.0e-7):
+        x = (rng.standard_normal((rows, k)) * scale).astype(np.float32)
+        g = Graph.new("cfg4_ragged")
+        xi = g.input("x", Shape.new([rows, k], DType.F32))
+        fq = g.add_node(Op.FakeQuantize(8, 1), [xi], Shape.new([rows, k], DType.F32))
+        packs, outs = [], []
+        for i, n in enumerate(ns):
+            p = tiled_packed(Q4_0, n, k, 64 + i, 0.02).reshape(-1)
+            packs.append(p)
+            w = g.param(f"w{i}", Shape.new([len(p)], DType.U8))
+            outs.append(g.add_node(Op.DequantMatMul(QuantScheme.GgufQ4_0), [fq, w], Shape.new([rows, n], DType.F32)))
+        g.set_outputs(outs)
+        c = Session().compile(g)
+        assert c.describe_plan().count("[x: binary16 image]") == 2
+        for i, p in enumerate(packs):
+            c.set_param_typed(f"w{i}", p, DType.U8)
+        got = c.run([("x", x)])
+        fq_ref, _, _ = oracle.fake_quantize(x, x.shape, 1, 8)
+        for i, n in enumerate(ns):
+            ref = oracle.gguf_matmul_f64(fq_ref, packs[i], rows, k, n, Q4_0)
+            err = float(np.max(np.abs(got[i].reshape(rows, n) - ref) / np.maximum(np.abs(ref), scale)))
+            say(f"   fq image chain scale {scale:g} n={n}: max rel err {err:.3e}")
+            assert err <= TOL

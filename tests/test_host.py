@@ -149,8 +149,10 @@ def test_qweight_create_validates_before_allocating():
 
 
 def test_plan_reuses_dead_slots():
-    # FakeQuantize -> matmul -> matmul: the second matmul's output may take the bytes of the fake-quantized tensor, which is
-    # dead by then, and a step's workspace lives for that step only (rlx-compile/src/memory.rs:386-470 is the contract)
+    # FakeQuantize -> matmul -> matmul -> matmul: the third matmul's output may take the bytes of the first's, which is dead
+    # by then, and a step's workspace lives for that step only (rlx-compile/src/memory.rs:386-470 is the contract). The
+    # fake-quantized tensor itself is read by a prefill matmul only, so it is written as that step's operand image and has
+    # no f32 slot at all.
     g = Graph.new("chain")
     x = g.input("x", Shape.new([64, 4096], DType.F32))
     fq = g.add_node(Op.FakeQuantize(8, 1), [x], Shape.new([64, 4096], DType.F32))
@@ -158,31 +160,37 @@ def test_plan_reuses_dead_slots():
     y = g.add_node(Op.DequantMatMul(QuantScheme.GgufQ8_0), [fq, w], Shape.new([64, 256], DType.F32))
     w2 = g.param("w2", Shape.new([256 * 128 // 32 * 34], DType.U8))
     z = g.add_node(Op.DequantMatMul(QuantScheme.GgufQ8_0), [y, w2], Shape.new([64, 128], DType.F32))
-    g.set_outputs([z])
+    w3 = g.param("w3", Shape.new([128 * 64 // 32 * 34], DType.U8))
+    z2 = g.add_node(Op.DequantMatMul(QuantScheme.GgufQ8_0), [z, w3], Shape.new([64, 64], DType.F32))
+    g.set_outputs([z2])
     def slots_of(text):
         return {int(line.split()[1]): (int(line.split("off=")[1].split()[0]), int(line.split("size=")[1].split()[0]))
                 for line in text.splitlines()[1:]}
 
+    def disjoint(slots, a, b):
+        (oa, sa), (ob, sb) = slots[a], slots[b]
+        return sa == 0 or sb == 0 or oa + sa <= ob or ob + sb <= oa
+
     total, text = Session().plan(g)
     slots = slots_of(text)
-    assert slots[5][0] == slots[1][0]                      # z reuses the fake-quantized tensor's slot
+    assert slots[1][1] == 0 and "f32 tensor not written" in text.splitlines()[2]
+    assert slots[7][0] == slots[3][0]                      # z2 reuses y's slot
     bump = sum((sz + 255) // 256 * 256 for _, sz in slots.values())
-    assert total < bump + 2 * 1024 * 1024                  # less than one private slot per buffer plus both workspaces
-    live = [0, 2, 4]                                       # sources never share bytes with anything
-    for a in live:
-        for b, (ob, sb) in slots.items():
-            if a != b:
-                oa, sa = slots[a]
-                assert oa + sa <= ob or ob + sb <= oa, (a, b)
-    # with every intermediate an output nothing may be reused
-    g.set_outputs([z, y, fq])
+    assert total < bump + 3 * 1024 * 1024                  # less than one private slot per buffer plus the workspaces
+    for a in (0, 2, 4, 6):                                 # sources never share bytes with anything
+        for b in slots:
+            assert a == b or disjoint(slots, a, b), (a, b)
+    for a, b in ((3, 5), (5, 7)):                          # a matmul's input and output are live together
+        assert disjoint(slots, a, b), (a, b)
+    # with every intermediate an output nothing may be reused, and the fake-quantized tensor gets its f32 slot back
+    g.set_outputs([z2, z, y, fq])
     total_all, text_all = Session().plan(g)
     kept = slots_of(text_all)
-    for a in (1, 3, 5):
-        for b in (1, 3, 5):
-            if a < b:
-                assert kept[a][0] + kept[a][1] <= kept[b][0] or kept[b][0] + kept[b][1] <= kept[a][0], (a, b)
-    assert total_all >= total
+    assert kept[1][1] == 64 * 4096 * 4
+    for a in (1, 3, 5, 7):
+        for b in (1, 3, 5, 7):
+            assert a >= b or disjoint(kept, a, b), (a, b)
+    assert total_all >= total + 64 * 4096 * 4
     # the integer codes are opt-in: one more resident byte per element
     assert Session(fq_codes=True).plan(g)[0] >= total_all + 64 * 4096
 
