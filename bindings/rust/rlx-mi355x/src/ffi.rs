@@ -16,6 +16,9 @@ pub const RLX_OP_DEQUANT_MATMUL: u32 = 2;
 pub const RLX_OP_FAKE_QUANTIZE: u32 = 3;
 pub const RLX_OP_DEQUANT_GROUPED_MATMUL: u32 = 4;
 pub const RLX_OP_CONSTANT: u32 = 5;
+pub const RLX_OP_RMS_NORM: u32 = 6;
+pub const RLX_OP_FUSED_SWIGLU: u32 = 7;
+pub const RLX_NODE_FLAG_GATE_FIRST: u32 = 1;
 
 pub const RLX_MAX_RANK: usize = 6;
 pub const RLX_MAX_INPUTS: usize = 3;

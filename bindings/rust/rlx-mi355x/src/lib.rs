@@ -148,6 +148,16 @@ fn describe(node: &Node, name: &CString) -> ffi::rlx_node_desc {
                 ScaleMode::Fixed => d.scale_mode = 2,
             }
         }
+        // Over the last axis only, which is what the CPU backend's thunk computes whatever `axis` says
+        // (rlx-cpu/src/thunk.rs:2739-2751); another axis stays unclaimed and gets the legalize message.
+        Op::RmsNorm { axis, eps } if *axis == -1 || *axis as usize + 1 == node.shape.rank() => {
+            d.op_kind = ffi::RLX_OP_RMS_NORM; // inputs [x, gamma, beta]
+            d.eps = *eps;
+        }
+        Op::FusedSwiGLU { cast_to: None, gate_first } => {
+            d.op_kind = ffi::RLX_OP_FUSED_SWIGLU;
+            d.flags = if *gate_first { ffi::RLX_NODE_FLAG_GATE_FIRST } else { 0 };
+        }
         _ => {}
     }
     d
@@ -188,7 +198,10 @@ impl Backend for Mi355xBackend {
     }
 
     fn supported_ops(&self) -> &'static [OpKind] {
-        &[OpKind::Input, OpKind::Param, OpKind::Constant, OpKind::DequantMatMul, OpKind::DequantGroupedMatMul, OpKind::FakeQuantize]
+        &[
+            OpKind::Input, OpKind::Param, OpKind::Constant, OpKind::DequantMatMul, OpKind::DequantGroupedMatMul, OpKind::FakeQuantize,
+            OpKind::RmsNorm, OpKind::FusedSwiGLU,
+        ]
     }
 }
 

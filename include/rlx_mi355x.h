@@ -227,6 +227,20 @@ int rlx_mi355x_rmsnorm_gguf_tied_lm_topk(const float *hidden_dev, const float *g
 int rlx_mi355x_gguf_matmul_bt_batch(const void *const *xs_dev, int x_dtype, const rlx_qweight *const *ws,
                                     float *const *outs_dev, int count, int64_t m, void *workspace, size_t workspace_bytes,
                                     void *stream);
+/* Op::RmsNorm by itself (rlx-cpu/src/thunk.rs:8839-8869): out[rows, h] = x * (1 / sqrt(mean(x^2) + eps)) * gamma + beta per
+ * row; beta_dev may be NULL (zeros). One workgroup per row, one read and one write of the tensor. */
+int rlx_mi355x_rms_norm(const float *x_dev, const float *gamma_dev, const float *beta_dev, float eps, float *out_dev, int64_t rows,
+                        int64_t h, void *stream);
+/* Op::FusedSwiGLU by itself (rlx-cpu/src/thunk.rs:10337-10366): in[rows, 2 n_half] -> out[rows, n_half] =
+ * up * (gate / (1 + exp(-gate))), up in the low half and gate in the high half, the other way round with gate_first. */
+int rlx_mi355x_fused_swiglu(const float *in_dev, float *out_dev, int64_t rows, int64_t n_half, int gate_first, void *stream);
+/* A view of rows [row0, row0 + rows) of a plain weight as a weight of its own (the device layout is row tiles of 16, so
+ * row0 must be a multiple of 16 and the range must end on one or at the weight's last row). The view shares the parent's
+ * device memory, which must outlive it; release it with rlx_mi355x_qweight_destroy. No counterpart in the reference, whose
+ * concatenated up | gate projection is one DequantMatMul followed by Op::FusedSwiGLU; the executor uses views to run that
+ * pair through rlx_mi355x_gguf_matmul_swiglu. */
+int rlx_mi355x_qweight_rows(const rlx_qweight *w, int64_t row0, int64_t rows, rlx_qweight **out);
+
 /* The prefill path (m above the decode limit) in two calls, for a caller that multiplies one activation tensor by weights
  * at several points of its schedule, or keeps the conversion out of a timed region. No counterpart in the reference
  * (its thunk converts nothing). ..._prepare writes the binary16 image of x[m, k] (and, for Q4_K / Q5_K, its block
@@ -301,9 +315,16 @@ typedef enum rlx_op_kind {
     RLX_OP_FAKE_QUANTIZE = 3,  /* OpKind::FakeQuantize,  Op::FakeQuantize{bits,axis,ste,scale_mode} (op.rs:407-432) */
     RLX_OP_DEQUANT_GROUPED_MATMUL = 4, /* OpKind::DequantGroupedMatMul, Op::DequantGroupedMatMul{scheme} (op.rs:862-871):
                                         * inputs [x [m,k], packed expert stack, expert_idx [m] F32] -> [m,n] */
-    RLX_OP_CONSTANT = 5        /* OpKind::Constant, Op::Constant{data} (op.rs:369-372): const_data / const_nbytes are copied
+    RLX_OP_CONSTANT = 5,       /* OpKind::Constant, Op::Constant{data} (op.rs:369-372): const_data / const_nbytes are copied
                                 * into the arena at compile; a U8 constant feeding a DequantMatMul is repacked there */
+    RLX_OP_RMS_NORM = 6,       /* OpKind::RmsNorm, Op::RmsNorm{axis, eps} (op.rs:574-578), inputs [x, gamma, beta] over the
+                                * last axis as rlx-cpu lowers it (rlx-cpu/src/thunk.rs:2739-2751). In front of decode-size
+                                * DequantMatMuls it is folded into their activation staging; elsewhere a kernel of its own */
+    RLX_OP_FUSED_SWIGLU = 7    /* OpKind::FusedSwiGLU, Op::FusedSwiGLU{cast_to: None, gate_first} (op.rs:1157-1172): input
+                                * [.., 2n] -> [.., n]; flags bit 0 = gate_first. Behind a decode-size DequantMatMul that
+                                * nothing else reads, both halves of that matmul and the SwiGLU run as one launch */
 } rlx_op_kind;
+#define RLX_NODE_FLAG_GATE_FIRST 1u
 
 #define RLX_MAX_RANK 6
 #define RLX_MAX_INPUTS 3
@@ -325,9 +346,8 @@ typedef struct rlx_node_desc {
     uint32_t scale_mode;              /* rlx_scale_mode; EMA / FIXED take a second input: state [chan_dim] */
     float ema_decay;
     uint32_t ste;                     /* SteKind; forward-only backend: carried, not used */
-    /* reserved for op kinds with an epsilon / boolean attribute */
-    float eps;
-    uint32_t flags;
+    float eps;                        /* RmsNorm */
+    uint32_t flags;                   /* FusedSwiGLU: RLX_NODE_FLAG_GATE_FIRST */
     /* Constant: the embedded bytes (read during rlx_mi355x_compile only) */
     const void *const_data;
     uint64_t const_nbytes;

@@ -7,6 +7,7 @@
 // param owns a slot sized for the *device layout* of its weights, filled once by set_param_typed.
 #include <algorithm>
 #include <cstring>
+#include <functional>
 #include <map>
 #include <memory>
 #include <string>
@@ -25,6 +26,14 @@ extern "C" int rlx_mi355x_gguf_grouped_matmul_bt(const void *, int, const rlx_qw
 extern "C" int rlx_mi355x_gguf_matmul_bt_batch(const void *const *, int, const rlx_qweight *const *, float *const *, int, int64_t,
                                                void *, size_t, void *);
 extern "C" int rlx_mi355x_gguf_matmul_bt_prepared(const void *, size_t, int, const rlx_qweight *const *, float *const *, int, int64_t, void *);
+extern "C" int rlx_mi355x_rms_norm(const float *, const float *, const float *, float, float *, int64_t, int64_t, void *);
+extern "C" int rlx_mi355x_fused_swiglu(const float *, float *, int64_t, int64_t, int, void *);
+extern "C" int rlx_mi355x_qweight_rows(const rlx_qweight *, int64_t, int64_t, rlx_qweight **);
+extern "C" int rlx_mi355x_gguf_matmul_swiglu(const void *, int, const rlx_qweight *, const rlx_qweight *, float *, int64_t, void *);
+extern "C" int rlx_mi355x_rmsnorm_gguf_matmul_bt_batch(const float *, const float *, const float *, float, const rlx_qweight *const *,
+                                                       float *const *, int, int64_t, void *);
+extern "C" int rlx_mi355x_rmsnorm_gguf_matmul_swiglu(const float *, const float *, const float *, float, const rlx_qweight *,
+                                                     const rlx_qweight *, float *, int64_t, void *);
 extern "C" int rlx_mi355x_fake_quantize_image(const float *, float *, int8_t *, int64_t, int64_t, int, int, float, float *, int, void *, void *,
                                               size_t, void *);
 
@@ -33,8 +42,8 @@ namespace {
 using namespace rlx;
 
 const uint32_t kSupportedOps[] = {RLX_OP_INPUT, RLX_OP_PARAM, RLX_OP_DEQUANT_MATMUL, RLX_OP_FAKE_QUANTIZE,
-                                 RLX_OP_DEQUANT_GROUPED_MATMUL, RLX_OP_CONSTANT};
-constexpr uint32_t kMaxOpKind = RLX_OP_CONSTANT;
+                                 RLX_OP_DEQUANT_GROUPED_MATMUL, RLX_OP_CONSTANT, RLX_OP_RMS_NORM, RLX_OP_FUSED_SWIGLU};
+constexpr uint32_t kMaxOpKind = RLX_OP_FUSED_SWIGLU;
 const char *op_name(uint32_t k) {
     switch (k) {
     case RLX_OP_INPUT: return "Input";
@@ -43,6 +52,8 @@ const char *op_name(uint32_t k) {
     case RLX_OP_DEQUANT_GROUPED_MATMUL: return "DequantGroupedMatMul";
     case RLX_OP_FAKE_QUANTIZE: return "FakeQuantize";
     case RLX_OP_CONSTANT: return "Constant";
+    case RLX_OP_RMS_NORM: return "RmsNorm";
+    case RLX_OP_FUSED_SWIGLU: return "FusedSwiGLU";
     default: return "?";
     }
 }
@@ -88,6 +99,16 @@ struct Node {
     int img_step = -1;
     bool keep_f32 = true;
     bool x_image = false;  // (an f32 image: two binary16 rows per activation row)
+    // RmsNorm in front of decode-size DequantMatMuls only: the matmuls normalize while they stage their activations
+    // (norm_of = the RmsNorm node they read through) and the RmsNorm node has neither a launch nor a slot (folded).
+    // DequantMatMul [.., 2n] read by one FusedSwiGLU only, decode size: the SwiGLU node runs both halves of the weight
+    // and the combination as one launch (swiglu_mm = that matmul, which is folded too), on two row views of the weight.
+    int64_t h = 0;         // RmsNorm: row length; FusedSwiGLU: n_half
+    int norm_of = -1;
+    int swiglu_mm = -1;
+    bool folded = false;
+    rlx_qweight *view_lo = nullptr, *view_hi = nullptr;  // rows [0, n) and [n, 2n) of the folded matmul's weight
+    const rlx_qweight *view_parent = nullptr;
 };
 
 // f32 <-> half / bfloat16 as the reference's typed boundary does (rlx-driver/src/arena.rs:69-119, `half` crate).
@@ -136,8 +157,11 @@ struct rlx_exec {
     hipGraphExec_t graph_exec = nullptr;
 
     ~rlx_exec() {
-        for (auto &nd : nodes)
+        for (auto &nd : nodes) {
+            if (nd.view_lo) rlx_mi355x_qweight_destroy(nd.view_lo);
+            if (nd.view_hi) rlx_mi355x_qweight_destroy(nd.view_hi);
             if (nd.qw) rlx_mi355x_qweight_destroy(nd.qw);
+        }
         drop_graph();
         if (arena) (void)hipFree(arena);
         if (own_stream) (void)hipStreamDestroy(own_stream);
@@ -340,6 +364,36 @@ static std::unique_ptr<rlx_exec> plan_graph(const rlx_graph_desc *g, const rlx_c
             w.w_experts = w.numel / slab;
             break;
         }
+        case RLX_OP_RMS_NORM: {  // [x, gamma, beta] over the last axis (rlx-cpu/src/thunk.rs:2739-2751); beta may be left out
+            if ((nd.d.n_inputs != 3 && nd.d.n_inputs != 2) || nd.d.rank == 0 || nd.d.dtype != RLX_F32) {
+                set_error("compile: node %u: RmsNorm takes [x, gamma, beta] and yields an F32 tensor of rank >= 1", i);
+                return nullptr;
+            }
+            nd.h = nd.d.dims[nd.d.rank - 1];
+            const Node &x = e->nodes[nd.d.inputs[0]];
+            bool ok = nd.h > 0 && x.numel == nd.numel && x.d.dtype == RLX_F32;
+            for (uint32_t j = 1; j < nd.d.n_inputs; j++)
+                ok = ok && e->nodes[nd.d.inputs[j]].numel == nd.h && e->nodes[nd.d.inputs[j]].d.dtype == RLX_F32;
+            if (!ok) {
+                set_error("compile: node %u: RmsNorm needs F32 x with the output's element count and F32 gamma / beta of the last dim (%lld)", i,
+                          (long long)nd.h);
+                return nullptr;
+            }
+            break;
+        }
+        case RLX_OP_FUSED_SWIGLU: {  // [.., 2n] -> [.., n] (rlx-cpu/src/thunk.rs:3439-3453)
+            if (nd.d.n_inputs != 1 || nd.d.rank == 0 || nd.d.dtype != RLX_F32) {
+                set_error("compile: node %u: FusedSwiGLU takes one input and yields an F32 tensor of rank >= 1", i);
+                return nullptr;
+            }
+            nd.h = nd.d.dims[nd.d.rank - 1];
+            const Node &x = e->nodes[nd.d.inputs[0]];
+            if (nd.h <= 0 || x.numel != 2 * nd.numel || x.d.dtype != RLX_F32) {
+                set_error("compile: node %u: FusedSwiGLU needs an F32 input of twice the output's element count (cast_to is not claimed)", i);
+                return nullptr;
+            }
+            break;
+        }
         case RLX_OP_FAKE_QUANTIZE: {
             if (nd.d.bits != 8 && nd.d.bits != 4 && nd.d.bits != 2) {
                 set_error("FakeQuantize: unsupported bits %u", nd.d.bits);
@@ -381,6 +435,41 @@ static std::unique_ptr<rlx_exec> plan_graph(const rlx_graph_desc *g, const rlx_c
         }
     }
 
+    // RmsNorm / FusedSwiGLU around decode-size matmuls fold into the matmul launches.
+    {
+        auto is_output = [&](uint32_t id) { return std::find(e->outputs.begin(), e->outputs.end(), id) != e->outputs.end(); };
+        for (uint32_t r = 0; r < g->n_nodes; r++) {
+            Node &rn = e->nodes[r];
+            if (rn.d.op_kind != RLX_OP_RMS_NORM || rn.numel / rn.h > 8 || is_output(r)) continue;
+            bool ok = true;
+            std::vector<uint32_t> mms;
+            for (uint32_t j = r + 1; j < g->n_nodes && ok; j++) {
+                const Node &o = e->nodes[j];
+                for (uint32_t t = 0; t < o.d.n_inputs; t++) {
+                    if (o.d.inputs[t] != r) continue;
+                    if (o.d.op_kind == RLX_OP_DEQUANT_MATMUL && t == 0 && o.k == rn.h && o.m == rn.numel / rn.h) mms.push_back(j);
+                    else ok = false;
+                }
+            }
+            if (!ok || mms.empty()) continue;
+            rn.folded = true;
+            for (uint32_t j : mms) e->nodes[j].norm_of = (int)r;
+        }
+        for (uint32_t sidx = 0; sidx < g->n_nodes; sidx++) {
+            Node &sw = e->nodes[sidx];
+            if (sw.d.op_kind != RLX_OP_FUSED_SWIGLU) continue;
+            const uint32_t mi = sw.d.inputs[0];
+            Node &mm = e->nodes[mi];
+            if (mm.d.op_kind != RLX_OP_DEQUANT_MATMUL || mm.m > 8 || mm.n != 2 * sw.h || sw.h % TILE_ROWS != 0 || is_output(mi)) continue;
+            int readers = 0;
+            for (uint32_t j = mi + 1; j < g->n_nodes; j++)
+                for (uint32_t t = 0; t < e->nodes[j].d.n_inputs; t++) readers += e->nodes[j].d.inputs[t] == mi;
+            if (readers != 1) continue;
+            mm.folded = true;
+            sw.swiglu_mm = (int)mi;
+        }
+    }
+
     // depth[i] = longest chain of compute nodes below node i (inputs and params are depth 0)
     std::vector<int> depth(e->nodes.size(), 0);
     for (uint32_t i = 0; i < g->n_nodes; i++) {
@@ -393,15 +482,13 @@ static std::unique_ptr<rlx_exec> plan_graph(const rlx_graph_desc *g, const rlx_c
     std::vector<bool> grouped(e->nodes.size(), false);
     for (uint32_t i = 0; i < g->n_nodes; i++) {
         Node &nd = e->nodes[i];
-        if (grouped[i] || (nd.d.op_kind != RLX_OP_DEQUANT_MATMUL && nd.d.op_kind != RLX_OP_FAKE_QUANTIZE &&
-                           nd.d.op_kind != RLX_OP_DEQUANT_GROUPED_MATMUL))
-            continue;
+        if (grouped[i] || is_source(nd.d.op_kind) || nd.folded) continue;
         std::vector<uint32_t> step{i};
         if (nd.d.op_kind == RLX_OP_DEQUANT_MATMUL) {
             const uint32_t xdt = e->nodes[nd.d.inputs[0]].d.dtype;
             for (uint32_t j = i + 1; j < g->n_nodes; j++) {
                 Node &o = e->nodes[j];
-                if (!grouped[j] && o.d.op_kind == RLX_OP_DEQUANT_MATMUL && depth[j] == depth[i] &&
+                if (!grouped[j] && o.d.op_kind == RLX_OP_DEQUANT_MATMUL && depth[j] == depth[i] && !o.folded && o.norm_of == nd.norm_of &&
                     o.d.scheme == nd.d.scheme && o.m == nd.m && e->nodes[o.d.inputs[0]].d.dtype == xdt &&
                     (o.d.inputs[0] < i || is_source(e->nodes[o.d.inputs[0]].d.op_kind))) {
                     grouped[j] = true;
@@ -458,11 +545,18 @@ static std::unique_ptr<rlx_exec> plan_graph(const rlx_graph_desc *g, const rlx_c
     std::vector<int> step_of(e->nodes.size(), 0), last_use(e->nodes.size(), 0);
     for (size_t si = 0; si < e->steps.size(); si++)
         for (uint32_t id : e->steps[si]) step_of[id] = (int)si;
+    // a folded node runs inside the launch of its reader: what it reads must live until that reader's step
+    std::function<void(uint32_t, int)> reads = [&](uint32_t id, int step) {
+        last_use[id] = std::max(last_use[id], step);
+        const Node &src = e->nodes[id];
+        if (src.folded)
+            for (uint32_t j = 0; j < src.d.n_inputs; j++) reads(src.d.inputs[j], step);
+    };
     for (uint32_t i = 0; i < g->n_nodes; i++) {
         const Node &nd = e->nodes[i];
         last_use[i] = std::max(last_use[i], step_of[i]);
-        if (is_source(nd.d.op_kind)) continue;
-        for (uint32_t j = 0; j < nd.d.n_inputs; j++) last_use[nd.d.inputs[j]] = std::max(last_use[nd.d.inputs[j]], step_of[i]);
+        if (is_source(nd.d.op_kind) || nd.folded) continue;
+        for (uint32_t j = 0; j < nd.d.n_inputs; j++) reads(nd.d.inputs[j], step_of[i]);
     }
     for (uint32_t id : e->outputs) last_use[id] = kForever;
     struct Placed {
@@ -663,6 +757,18 @@ int rlx_exec_write_input(rlx_exec *e, const char *name, const void *data, size_t
     return RLX_OK;
 }
 
+// x, gamma and beta of an RmsNorm node must hold F32 when the launch is made (an Input may have been written as 16-bit).
+static int norm_operands(rlx_exec *e, const Node &rn, const char *what) {
+    for (uint32_t j = 0; j < rn.d.n_inputs; j++) {
+        const Node &in = e->nodes[rn.d.inputs[j]];
+        if (in.d.op_kind == RLX_OP_INPUT && in.cur_dtype != RLX_F32) {
+            set_error("run: %s input '%s' must be written as F32", what, in.name.c_str());
+            return RLX_ERR_INVALID;
+        }
+    }
+    return RLX_OK;
+}
+
 static int enqueue_schedule(rlx_exec *e) {
     for (const std::vector<uint32_t> &step : e->steps) {
         Node &nd = e->nodes[step[0]];
@@ -682,6 +788,66 @@ static int enqueue_schedule(rlx_exec *e) {
             }
             RLX_TRY(rlx_mi355x_gguf_grouped_matmul_bt(e->ptr(x.slot), (int)dt, w.qw, (const float *)e->ptr(idx.slot),
                                                       (float *)e->ptr(nd.slot), nd.m, e->stream));
+        } else if (nd.d.op_kind == RLX_OP_RMS_NORM) {
+            RLX_TRY(norm_operands(e, nd, "RmsNorm"));
+            const Node &x = e->nodes[nd.d.inputs[0]];
+            RLX_TRY(rlx_mi355x_rms_norm((const float *)e->ptr(x.slot), (const float *)e->ptr(e->nodes[nd.d.inputs[1]].slot),
+                                        nd.d.n_inputs > 2 ? (const float *)e->ptr(e->nodes[nd.d.inputs[2]].slot) : nullptr, nd.d.eps,
+                                        (float *)e->ptr(nd.slot), nd.numel / nd.h, nd.h, e->stream));
+        } else if (nd.d.op_kind == RLX_OP_FUSED_SWIGLU) {
+            const int gate_first = (nd.d.flags & RLX_NODE_FLAG_GATE_FIRST) ? 1 : 0;
+            if (nd.swiglu_mm < 0) {
+                RLX_TRY(rlx_mi355x_fused_swiglu((const float *)e->ptr(e->nodes[nd.d.inputs[0]].slot), (float *)e->ptr(nd.slot), nd.numel / nd.h,
+                                                nd.h, gate_first, e->stream));
+                continue;
+            }
+            Node &mm = e->nodes[nd.swiglu_mm];
+            Node &w = e->nodes[mm.d.inputs[1]];
+            if (!w.qw) {
+                set_error("run: packed weight '%s' was never set (set_param_typed(.., U8))", w.name.c_str());
+                return RLX_ERR_INVALID;
+            }
+            if (nd.view_parent != w.qw) {  // the weight was (re)loaded: cut its two halves again
+                if (nd.view_lo) rlx_mi355x_qweight_destroy(nd.view_lo);
+                if (nd.view_hi) rlx_mi355x_qweight_destroy(nd.view_hi);
+                nd.view_lo = nd.view_hi = nullptr;
+                nd.view_parent = nullptr;
+                RLX_TRY(rlx_mi355x_qweight_rows(w.qw, 0, nd.h, &nd.view_lo));
+                RLX_TRY(rlx_mi355x_qweight_rows(w.qw, nd.h, nd.h, &nd.view_hi));
+                nd.view_parent = w.qw;
+            }
+            const rlx_qweight *up = gate_first ? nd.view_hi : nd.view_lo, *gate = gate_first ? nd.view_lo : nd.view_hi;
+            if (mm.norm_of >= 0) {
+                Node &rn = e->nodes[mm.norm_of];
+                RLX_TRY(norm_operands(e, rn, "RmsNorm"));
+                RLX_TRY(rlx_mi355x_rmsnorm_gguf_matmul_swiglu((const float *)e->ptr(e->nodes[rn.d.inputs[0]].slot),
+                                                              (const float *)e->ptr(e->nodes[rn.d.inputs[1]].slot),
+                                                              rn.d.n_inputs > 2 ? (const float *)e->ptr(e->nodes[rn.d.inputs[2]].slot) : nullptr,
+                                                              rn.d.eps, up, gate, (float *)e->ptr(nd.slot), mm.m, e->stream));
+            } else {
+                Node &x = e->nodes[mm.d.inputs[0]];
+                const uint32_t dt = x.d.op_kind == RLX_OP_INPUT ? x.cur_dtype : x.d.dtype;
+                RLX_TRY(rlx_mi355x_gguf_matmul_swiglu(e->ptr(x.slot), (int)dt, up, gate, (float *)e->ptr(nd.slot), mm.m, e->stream));
+            }
+        } else if (nd.d.op_kind == RLX_OP_DEQUANT_MATMUL && nd.norm_of >= 0) {
+            // every matmul of the step reads through the same RmsNorm node: one launch per eight, normalizing as they stage x
+            Node &rn = e->nodes[nd.norm_of];
+            RLX_TRY(norm_operands(e, rn, "RmsNorm"));
+            std::vector<const rlx_qweight *> ws;
+            std::vector<float *> outs;
+            for (uint32_t id : step) {
+                Node &w = e->nodes[e->nodes[id].d.inputs[1]];
+                if (!w.qw) {
+                    set_error("run: packed weight '%s' was never set (set_param_typed(.., U8))", w.name.c_str());
+                    return RLX_ERR_INVALID;
+                }
+                ws.push_back(w.qw);
+                outs.push_back((float *)e->ptr(e->nodes[id].slot));
+            }
+            RLX_TRY(rlx_mi355x_rmsnorm_gguf_matmul_bt_batch((const float *)e->ptr(e->nodes[rn.d.inputs[0]].slot),
+                                                            (const float *)e->ptr(e->nodes[rn.d.inputs[1]].slot),
+                                                            rn.d.n_inputs > 2 ? (const float *)e->ptr(e->nodes[rn.d.inputs[2]].slot) : nullptr,
+                                                            rn.d.eps, ws.data(), outs.data(), (int)ws.size(), nd.m, e->stream));
         } else if (nd.d.op_kind == RLX_OP_DEQUANT_MATMUL) {
             // The whole step through the batched entry point: up to 16 / 32 rows it issues one decode launch per eight
             // matrices; above that, matrices that share their input (q, k, v; gate, up) share one conversion of it and
@@ -829,7 +995,7 @@ static int run_common(rlx_exec *e, const rlx_named_buf *inputs, size_t n_inputs,
     }
     int warn = RLX_OK;
     for (size_t i = 0; i < n_inputs; i++) {
-        int rc = rlx_exec_write_input(e, inputs[i].name, inputs[i].data, inputs[i].nbytes, typed ? inputs[i].dtype : RLX_F32);
+        int rc = rlx_exec_write_input(e, inputs[i].name, inputs[i].data, inputs[i].nbytes, typed ? inputs[i].dtype : (uint32_t)RLX_F32);
         if (rc < 0) return rc;
         if (rc > 0) warn = rc;
     }
@@ -904,6 +1070,10 @@ int rlx_exec_describe_plan(const rlx_exec *e, char *buf, size_t cap) {
         if (nd.d.op_kind == RLX_OP_DEQUANT_MATMUL && nd.aux.size) put(" step workspace@%zu+%zu", nd.aux.offset, nd.aux.size);
         if (nd.img_step >= 0) put(" -> prefill image of step %d%s", nd.img_step, nd.keep_f32 ? "" : " (f32 tensor not written)");
         if (nd.x_image) put(" [x: binary16 image]");
+        if (nd.d.op_kind == RLX_OP_RMS_NORM || nd.d.op_kind == RLX_OP_FUSED_SWIGLU) put(" h=%lld", (long long)nd.h);
+        if (nd.folded) put("%s", nd.d.op_kind == RLX_OP_RMS_NORM ? " (folded into the matmuls that read it)" : " (folded into the FusedSwiGLU that reads it)");
+        if (nd.norm_of >= 0) put(" [x: normalized while staged, RmsNorm node %d]", nd.norm_of);
+        if (nd.swiglu_mm >= 0) put(" [one launch with DequantMatMul node %d]", nd.swiglu_mm);
         put("\n");
     }
     return RLX_OK;

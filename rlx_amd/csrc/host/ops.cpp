@@ -765,6 +765,68 @@ int rlx_mi355x_gguf_matmul_swiglu(const void *x_dev, int x_dtype, const rlx_qwei
     return launch_gemv(xs, xk, ws, outs, 1, (int)m, (hipStream_t)stream, nullptr, nullptr, ps);
 }
 
+namespace rlx {
+struct RowOpArgs {  // mirrors kernels/rowops.hip
+    const float *x;
+    const float *gamma;
+    const float *beta;
+    float *out;
+    long long rows, h;
+    float eps;
+    int gate_first;
+    int vec4;
+};
+}  // namespace rlx
+
+int rlx_mi355x_rms_norm(const float *x_dev, const float *gamma_dev, const float *beta_dev, float eps, float *out_dev, int64_t rows,
+                        int64_t h, void *stream) {
+    using namespace rlx;
+    if (!x_dev || !gamma_dev || !out_dev || rows <= 0 || h <= 0) {
+        set_error("rms_norm: null argument, rows=%lld or h=%lld", (long long)rows, (long long)h);
+        return RLX_ERR_INVALID;
+    }
+    RowOpArgs a{x_dev, gamma_dev, beta_dev, out_dev, rows, h, eps, 0, 0};
+    a.vec4 = h % 4 == 0 && ((uintptr_t)x_dev | (uintptr_t)gamma_dev | (uintptr_t)beta_dev | (uintptr_t)out_dev) % 16 == 0;
+    void *params[] = {&a};
+    const unsigned bx = h >= 4096 ? 1024 : 256;
+    return launch(K_RMSNORM_ROWS, (unsigned)std::min<int64_t>(rows, 1 << 20), 1, bx, 0, (hipStream_t)stream, params);
+}
+
+int rlx_mi355x_fused_swiglu(const float *in_dev, float *out_dev, int64_t rows, int64_t n_half, int gate_first, void *stream) {
+    using namespace rlx;
+    if (!in_dev || !out_dev || rows <= 0 || n_half <= 0) {
+        set_error("fused_swiglu: null argument, rows=%lld or n_half=%lld", (long long)rows, (long long)n_half);
+        return RLX_ERR_INVALID;
+    }
+    RowOpArgs a{in_dev, nullptr, nullptr, out_dev, rows, n_half, 0.f, gate_first ? 1 : 0, 0};
+    a.vec4 = n_half % 4 == 0 && ((uintptr_t)in_dev | (uintptr_t)out_dev) % 16 == 0;
+    void *params[] = {&a};
+    const int64_t items = a.vec4 ? rows * n_half / 4 : rows * n_half;
+    const unsigned gx = (unsigned)std::min<int64_t>((items + 255) / 256, 16 * (int64_t)device_props().cu_count);
+    return launch(K_SWIGLU_ROWS, gx, 1, 256, 0, (hipStream_t)stream, params);
+}
+
+int rlx_mi355x_qweight_rows(const rlx_qweight *w, int64_t row0, int64_t rows, rlx_qweight **out) {
+    using namespace rlx;
+    if (out) *out = nullptr;
+    if (!w || !out || w->experts != 1 || row0 < 0 || rows <= 0 || row0 + rows > w->dims.n || row0 % TILE_ROWS != 0 ||
+        (rows % TILE_ROWS != 0 && row0 + rows != w->dims.n)) {
+        set_error("qweight_rows: rows [%lld, %lld) of a plain %lld-row weight must begin and end on a multiple of %d", (long long)row0,
+                  (long long)(row0 + rows), w ? (long long)w->dims.n : 0LL, TILE_ROWS);
+        return RLX_ERR_INVALID;
+    }
+    rlx_qweight *v = new (std::nothrow) rlx_qweight(*w);
+    if (!v) {
+        set_error("qweight_rows: out of host memory");
+        return RLX_ERR_NO_MEMORY;
+    }
+    v->dims = weight_dims(w->layout, rows, w->dims.k);
+    v->dev = w->dev + (row0 / TILE_ROWS) * w->dims.units * (int64_t)w->layout.unit_bytes;
+    v->owns = false;
+    *out = v;
+    return RLX_OK;
+}
+
 int rlx_mi355x_gguf_tied_lm_argmax(const void *hidden_dev, int x_dtype, const rlx_qweight *embed, uint32_t *out_idx_dev,
                                    float *out_val_dev, void *key_scratch_dev, void *stream) {
     using namespace rlx;

@@ -3,4 +3,5 @@
 #include "fakequant.hip"
 #include "gemm.hip"
 #include "gemv.hip"
+#include "rowops.hip"
 #include "topk.hip"

@@ -68,6 +68,8 @@ class OpKind(enum.IntEnum):
     FakeQuantize = 3
     DequantGroupedMatMul = 4
     Constant = 5
+    RmsNorm = 6
+    FusedSwiGLU = 7
 
 
 @dataclass(frozen=True)
@@ -102,6 +104,8 @@ class Op:
     scale_mode: ScaleMode = ScaleMode.PerBatch
     ema_decay: float = 0.0
     data: Optional[bytes] = None  # Op::Constant { data } (op.rs:369-372)
+    eps: float = 0.0              # Op::RmsNorm { axis, eps } (op.rs:574-578)
+    gate_first: bool = False      # Op::FusedSwiGLU { cast_to, gate_first } (op.rs:1157-1172)
 
     @staticmethod
     def DequantMatMul(scheme):  # Op::DequantMatMul { scheme } (op.rs:736-752)
@@ -114,6 +118,14 @@ class Op:
     @staticmethod
     def FakeQuantize(bits, axis, ste=SteKind.Identity, scale_mode=ScaleMode.PerBatch, ema_decay=0.0):  # op.rs:407-432
         return Op(OpKind.FakeQuantize, bits=bits, axis=axis, ste=ste, scale_mode=scale_mode, ema_decay=ema_decay)
+
+    @staticmethod
+    def RmsNorm(eps, axis=-1):  # inputs [x, gamma, beta]; normalizes the last axis (rlx-cpu/src/thunk.rs:2739-2751)
+        return Op(OpKind.RmsNorm, axis=axis, eps=eps)
+
+    @staticmethod
+    def FusedSwiGLU(gate_first=False):  # [.., 2n] -> [.., n]; cast_to is None
+        return Op(OpKind.FusedSwiGLU, gate_first=gate_first)
 
 
 @dataclass
@@ -165,6 +177,13 @@ class Graph:
         ins = [x] if state is None else [x, state]
         return self.add_node(Op.FakeQuantize(bits, axis, scale_mode=scale_mode, ema_decay=ema_decay), ins,
                              self.nodes[x].shape)
+
+    def rms_norm(self, x, gamma, beta, eps):
+        return self.add_node(Op.RmsNorm(eps), [x, gamma, beta], self.nodes[x].shape)
+
+    def fused_swiglu(self, cat, gate_first=False):
+        sh = self.nodes[cat].shape
+        return self.add_node(Op.FusedSwiGLU(gate_first), [cat], Shape(tuple(sh.dims[:-1]) + (sh.dims[-1] // 2,), sh.dtype))
 
     def set_outputs(self, outs):
         self.outputs = list(outs)

@@ -227,6 +227,27 @@ def gguf_matmul_swiglu(x, w_up: QWeight, w_gate: QWeight, m, x_dtype=DType.F32):
     return od.to_numpy(np.float32).reshape(m, w_up.n)
 
 
+def rms_norm(x, gamma, beta, eps):
+    """Host convenience: Op::RmsNorm over the last axis as a launch of its own."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    h = x.shape[-1]
+    xd, od = DeviceBuffer.from_numpy(x), DeviceBuffer(x.nbytes)
+    g, b = _norm_bufs(gamma, beta)
+    _lib.check(_lib.lib().rlx_mi355x_rms_norm(xd.ptr, g.ptr, b.ptr if b else None, eps, od.ptr, x.size // h, h, None))
+    sync()
+    return od.to_numpy(np.float32).reshape(x.shape)
+
+
+def fused_swiglu(inp, gate_first=False):
+    """Host convenience: Op::FusedSwiGLU over rows [up | gate] of 2 n -> rows of n."""
+    inp = np.ascontiguousarray(inp, dtype=np.float32)
+    n = inp.shape[-1] // 2
+    xd, od = DeviceBuffer.from_numpy(inp), DeviceBuffer(inp.nbytes // 2)
+    _lib.check(_lib.lib().rlx_mi355x_fused_swiglu(xd.ptr, od.ptr, inp.size // (2 * n), n, int(gate_first), None))
+    sync()
+    return od.to_numpy(np.float32).reshape(inp.shape[:-1] + (n,))
+
+
 def _norm_bufs(gamma, beta):
     g = DeviceBuffer.from_numpy(np.ascontiguousarray(gamma, dtype=np.float32))
     b = DeviceBuffer.from_numpy(np.ascontiguousarray(beta, dtype=np.float32)) if beta is not None else None

@@ -47,6 +47,8 @@ def _graph_desc(graph: Graph):
         d.scale_mode = int(nd.op.scale_mode)
         d.ema_decay = nd.op.ema_decay
         d.ste = int(nd.op.ste)
+        d.eps = nd.op.eps
+        d.flags = 1 if nd.op.gate_first else 0
         if nd.op.data is not None:
             buf = C.create_string_buffer(nd.op.data, len(nd.op.data))
             keep.append(buf)

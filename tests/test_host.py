@@ -128,7 +128,7 @@ def compile_error(g):
 
 
 def test_supported_ops():
-    assert [int(k) for k in rlx_amd.supported_ops()] == [0, 1, 2, 3, 4, 5]
+    assert [int(k) for k in rlx_amd.supported_ops()] == [0, 1, 2, 3, 4, 5, 6, 7]
 
 
 def test_qweight_create_validates_before_allocating():
@@ -193,6 +193,53 @@ def test_plan_reuses_dead_slots():
     assert total_all >= total + 64 * 4096 * 4
     # the integer codes are opt-in: one more resident byte per element
     assert Session(fq_codes=True).plan(g)[0] >= total_all + 64 * 4096
+
+
+def _llama_mlp_graph(m, k=256, n=512, norm_is_output=False):
+    # RmsNorm -> q, k; RmsNorm -> [up | gate] -> FusedSwiGLU -> down: the ops around the hot path as the reference's
+    # graphs hold them (rlx-ir/src/op.rs:574-578, 1157-1172)
+    g = Graph.new("mlp")
+    x = g.input("x", Shape.new([m, k], DType.F32))
+    gamma, beta = g.param("gamma", Shape.new([k], DType.F32)), g.param("beta", Shape.new([k], DType.F32))
+    xn = g.rms_norm(x, gamma, beta, 1e-5)
+    wq = g.param("wq", Shape.new([k * 128 // 32 * 18], DType.U8))
+    wk = g.param("wk", Shape.new([k * 64 // 32 * 18], DType.U8))
+    q = g.add_node(Op.DequantMatMul(QuantScheme.GgufQ4_0), [xn, wq], Shape.new([m, 128], DType.F32))
+    kk = g.add_node(Op.DequantMatMul(QuantScheme.GgufQ4_0), [xn, wk], Shape.new([m, 64], DType.F32))
+    wcat = g.param("wcat", Shape.new([k * 2 * n // 32 * 18], DType.U8))
+    cat = g.add_node(Op.DequantMatMul(QuantScheme.GgufQ4_0), [xn, wcat], Shape.new([m, 2 * n], DType.F32))
+    act = g.fused_swiglu(cat)
+    wd = g.param("wd", Shape.new([n * k // 32 * 18], DType.U8))
+    y = g.add_node(Op.DequantMatMul(QuantScheme.GgufQ4_0), [act, wd], Shape.new([m, k], DType.F32))
+    g.set_outputs([q, kk, y] + ([xn] if norm_is_output else []))
+    return g, dict(x=x, xn=xn, q=q, k=kk, cat=cat, act=act, y=y)
+
+
+def test_plan_folds_rmsnorm_and_swiglu_at_decode_sizes():
+    g, ids = _llama_mlp_graph(2)
+    lines = Session().plan(g)[1].splitlines()[1:]
+    line = {int(l.split()[1]): l for l in lines}
+    assert "folded into the matmuls" in line[ids["xn"]] and " size=0" in line[ids["xn"]]
+    assert f"RmsNorm node {ids['xn']}" in line[ids["q"]] and f"RmsNorm node {ids['xn']}" in line[ids["k"]]
+    assert "folded into the FusedSwiGLU" in line[ids["cat"]] and " size=0" in line[ids["cat"]]
+    assert f"one launch with DequantMatMul node {ids['cat']}" in line[ids["act"]]
+    # a normalized tensor that is an output, or a prefill batch, keeps every op a launch of its own
+    for gg in (_llama_mlp_graph(2, norm_is_output=True)[0], _llama_mlp_graph(64)[0]):
+        text = Session().plan(gg)[1]
+        assert "folded into the matmuls" not in text
+    assert "folded into the FusedSwiGLU" not in Session().plan(_llama_mlp_graph(64)[0])[1]
+
+
+def test_rmsnorm_and_swiglu_shape_errors():
+    g = Graph.new("bad")
+    x = g.input("x", Shape.new([2, 64], DType.F32))
+    gamma = g.param("gamma", Shape.new([32], DType.F32))
+    g.set_outputs([g.add_node(Op.RmsNorm(1e-5), [x, gamma, gamma], Shape.new([2, 64], DType.F32))])
+    assert "gamma / beta of the last dim (64)" in compile_error(g)
+    g = Graph.new("bad2")
+    x = g.input("x", Shape.new([2, 64], DType.F32))
+    g.set_outputs([g.add_node(Op.FusedSwiGLU(), [x], Shape.new([2, 64], DType.F32))])
+    assert "twice the output's element count" in compile_error(g)
 
 
 def test_plan_constant_nodes():
