@@ -503,9 +503,31 @@ def moe_config(rlx_amd, stream):
 
     ms = time_launches(ops, stream, fn, 400, 40)
     b = 2 * gemv_bytes(n, k)
+    out = {"q4_0_moe_grouped_top2_of_8x14336x4096": {"us": round(ms * 1e3, 3), "GB/s": round(b / ms / 1e6, 1),
+                                                    "frac_hbm": round(b / ms / 1e6 / HBM_PEAK_GBS, 4)}}
+    # the same stack at a prefill size: 512 tokens x top-2 = 1024 routed rows (bf16), sorted by expert on the device and
+    # multiplied in one prefill launch, against a launch per eight routed rows
+    m = 1024
+    xb = ops.DeviceBuffer.from_numpy(f32_to_bf16_bits(ops.philox_normal(63, m * k)))
+    yb = ops.DeviceBuffer(m * n * 4)
+    route = ops.DeviceBuffer.from_numpy(np.floor(ops.philox_uniform(64, m) * np.float32(experts)).astype(np.float32))
+    need = L.rlx_mi355x_gguf_grouped_matmul_workspace(int(QuantScheme.GgufQ4_0), int(DType.BF16), m, k, experts)
+    ws = ops.DeviceBuffer(need)
+
+    def fn_sorted():
+        rlx_amd._lib.check(L.rlx_mi355x_gguf_grouped_matmul_bt_ws(xb.ptr, int(DType.BF16), qw.ptr, route.ptr, yb.ptr, m, ws.ptr, need, stream))
+
+    def fn_rows():
+        rlx_amd._lib.check(L.rlx_mi355x_gguf_grouped_matmul_bt(xb.ptr, int(DType.BF16), qw.ptr, route.ptr, yb.ptr, m, stream))
+
+    ms_s = time_launches(ops, stream, fn_sorted, 40, 5)
+    ms_r = time_launches(ops, stream, fn_rows, 5, 1)
+    tf = 2.0 * m * n * k / ms_s / 1e9
+    out["q4_0_moe_grouped_1024_rows_of_8x14336x4096_bf16"] = {
+        "us_expert_sorted": round(ms_s * 1e3, 1), "TFLOP/s": round(tf, 1), "us_launch_per_eight_rows": round(ms_r * 1e3, 1),
+        "launches": "sort + row scales + image (gathered) + one prefill launch over 64-row tiles"}
     qw.free()
-    return {"q4_0_moe_grouped_top2_of_8x14336x4096": {"us": round(ms * 1e3, 3), "GB/s": round(b / ms / 1e6, 1),
-                                                     "frac_hbm": round(b / ms / 1e6 / HBM_PEAK_GBS, 4)}}
+    return out
 
 
 def f32_to_bf16_bits(x):

@@ -178,6 +178,16 @@ int rlx_mi355x_qweight_create_experts_at(int scheme, const void *gguf_bytes, siz
  * launch). An index outside [0, num_experts) is clamped to the stack (the reference debug-asserts). */
 int rlx_mi355x_gguf_grouped_matmul_bt(const void *x_dev, int x_dtype, const rlx_qweight *w, const float *expert_idx_dev,
                                       float *out_dev, int64_t m, void *stream);
+/* The same result for batches above the decode sizes (m > 16 f32 rows, > 32 bf16 / f16), the way the reference computes
+ * it (rlx-cpu/src/gguf_matmul.rs:101-139 over grouped_moe_sort_plan :178-207): tokens are put in expert order by a stable
+ * counting sort, here one workgroup on the device because expert_idx is device memory; the activations are converted
+ * into the prefill image in that order, every expert's run padded to a 64-row tile; one launch of the prefill kernel
+ * multiplies each tile by its expert's slab and writes the rows back to their tokens' places. Every expert's slab is read
+ * once per 64-row tile of its tokens instead of once per token. `workspace`: ..._grouped_matmul_workspace() bytes, 16-byte
+ * aligned; at decode sizes, or with more than 256 experts, that is 0 and the call is rlx_mi355x_gguf_grouped_matmul_bt. */
+size_t rlx_mi355x_gguf_grouped_matmul_workspace(int scheme, int x_dtype, int64_t m, int64_t k, int64_t num_experts);
+int rlx_mi355x_gguf_grouped_matmul_bt_ws(const void *x_dev, int x_dtype, const rlx_qweight *w, const float *expert_idx_dev,
+                                         float *out_dev, int64_t m, void *workspace, size_t workspace_bytes, void *stream);
 /* Two DequantMatMuls feeding Op::FusedSwiGLU (rlx-ir/src/op.rs:1157-1172, executed at rlx-cpu/src/thunk.rs:10337-10366):
  * out[m, n] = up * (gate / (1 + exp(-gate))) with up = x . W_up^T and gate = x . W_gate^T. Decode path only (m <= 8 f32,
  * <= 16 bf16 / f16): every workgroup of the decode kernel runs its row tiles through both matrices and combines the two

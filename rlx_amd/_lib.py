@@ -97,6 +97,8 @@ SIGNATURES = {
     "rlx_mi355x_rmsnorm_gguf_tied_lm_argmax": (_i, [_vp, _vp, _vp, _f, _vp, _vp, _vp, _vp, _vp]),
     "rlx_mi355x_fake_quantize_scratch_bytes": (_sz, [_i64, _i64, _i64]),
     "rlx_mi355x_fake_quantize": (_i, [_vp, _vp, _vp, _i64, _i64, _i64, _i, _i, _f, _vp, _i, _vp, _vp]),
+    "rlx_mi355x_gguf_grouped_matmul_workspace": (_sz, [_i, _i, _i64, _i64, _i64]),
+    "rlx_mi355x_gguf_grouped_matmul_bt_ws": (_i, [_vp, _i, _vp, _vp, _vp, _i64, _vp, _sz, _vp]),
     "rlx_mi355x_rms_norm": (_i, [_vp, _vp, _vp, _f, _vp, _i64, _i64, _vp]),
     "rlx_mi355x_fused_swiglu": (_i, [_vp, _vp, _i64, _i64, _i, _vp]),
     "rlx_mi355x_qweight_rows": (_i, [_vp, _i64, _i64, C.POINTER(_vp)]),

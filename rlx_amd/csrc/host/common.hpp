@@ -56,6 +56,7 @@ enum KernelId : int {
     K_GEMV_Q4_0_U2_R2_NORM, K_GEMV_Q4_0_U2_R4_NORM, K_GEMV_Q4_0_U2_R2_NORM_PAIRED, K_GEMV_Q4_0_U2_R4_NORM_PAIRED, K_GEMV_Q4_0_U2_R2_NORM_ARGMAX,
     K_GEMV_Q4_0_G2, K_GEMV_Q8_0_G2, K_GEMV_Q4_K_G2, K_GEMV_F16W_G2, K_GEMV_Q6_K_G2, K_GEMV_Q5_K_G2,
     K_GEMM_Q4_K, K_GEMM_Q4_0, K_GEMM_Q8_0, K_GEMM64_Q4_K, K_GEMM64_Q4_0, K_GEMM64_Q8_0, K_GEMM_F16W, K_GEMM64_F16W, K_GEMM_Q6_K, K_GEMM64_Q6_K, K_GEMM_Q5_K, K_GEMM64_Q5_K, K_XPREP, K_XROWSCALE, K_ARGMAX_FINISH, K_TOPK_SELECT, K_RMSNORM_ROWS, K_SWIGLU_ROWS,
+    K_GEMM64G_Q4_K, K_GEMM64G_Q4_0, K_GEMM64G_Q8_0, K_GEMM64G_Q5_K, K_GEMM64G_Q6_K, K_GEMM64G_F16W, K_MOE_SORT,
     K_COUNT
 };
 

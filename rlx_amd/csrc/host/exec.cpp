@@ -22,7 +22,8 @@ extern "C" int rlx_mi355x_fake_quantize(const float *, float *, int8_t *, int64_
                                         void *, void *);
 extern "C" void rlx_mi355x_qweight_destroy(rlx_qweight *);
 extern "C" int rlx_mi355x_qweight_create_ex(int, uint32_t, const void *, size_t, int64_t, int64_t, int64_t, void *, size_t, rlx_qweight **);
-extern "C" int rlx_mi355x_gguf_grouped_matmul_bt(const void *, int, const rlx_qweight *, const float *, float *, int64_t, void *);
+extern "C" int rlx_mi355x_gguf_grouped_matmul_bt_ws(const void *, int, const rlx_qweight *, const float *, float *, int64_t, void *, size_t, void *);
+extern "C" size_t rlx_mi355x_gguf_grouped_matmul_workspace(int, int, int64_t, int64_t, int64_t);
 extern "C" int rlx_mi355x_gguf_matmul_bt_batch(const void *const *, int, const rlx_qweight *const *, float *const *, int, int64_t,
                                                void *, size_t, void *);
 extern "C" int rlx_mi355x_gguf_matmul_bt_prepared(const void *, size_t, int, const rlx_qweight *const *, float *const *, int, int64_t, void *);
@@ -614,6 +615,10 @@ static std::unique_ptr<rlx_exec> plan_graph(const rlx_graph_desc *g, const rlx_c
                 nd.aux = take(rlx_mi355x_fake_quantize_scratch_bytes(nd.numel, nd.chan_dim, nd.inner), (int)si, (int)si);
                 if (e->opts.fq_emit_codes) nd.codes = take((size_t)nd.numel, (int)si, kForever);
             }
+            if (nd.d.op_kind == RLX_OP_DEQUANT_GROUPED_MATMUL) {  // above the decode sizes: the expert-sorted path's workspace (f32 is the larger)
+                const size_t need = rlx_mi355x_gguf_grouped_matmul_workspace((int)nd.d.scheme, RLX_F32, nd.m, nd.k, e->nodes[nd.d.inputs[1]].w_experts);
+                if (need) nd.aux = take(need, (int)si, (int)si);
+            }
             if (nd.d.op_kind == RLX_OP_DEQUANT_MATMUL && nd.m > 16)  // may run the prefill kernels (which one is decided by the input dtype at run time): sized for f32
                 step_ws = std::max(step_ws, rlx_mi355x_gguf_matmul_workspace((int)nd.d.scheme, RLX_F32, nd.m, nd.k, nd.n));
         }
@@ -786,8 +791,8 @@ static int enqueue_schedule(rlx_exec *e) {
                 set_error("run: expert_idx of node %u must be written as F32", step[0]);
                 return RLX_ERR_INVALID;
             }
-            RLX_TRY(rlx_mi355x_gguf_grouped_matmul_bt(e->ptr(x.slot), (int)dt, w.qw, (const float *)e->ptr(idx.slot),
-                                                      (float *)e->ptr(nd.slot), nd.m, e->stream));
+            RLX_TRY(rlx_mi355x_gguf_grouped_matmul_bt_ws(e->ptr(x.slot), (int)dt, w.qw, (const float *)e->ptr(idx.slot), (float *)e->ptr(nd.slot),
+                                                         nd.m, nd.aux.size ? e->ptr(nd.aux) : nullptr, nd.aux.size, e->stream));
         } else if (nd.d.op_kind == RLX_OP_RMS_NORM) {
             RLX_TRY(norm_operands(e, nd, "RmsNorm"));
             const Node &x = e->nodes[nd.d.inputs[0]];
@@ -1068,6 +1073,7 @@ int rlx_exec_describe_plan(const rlx_exec *e, char *buf, size_t cap) {
             put(" chan_dim=%lld inner=%lld aux@%zu codes@%zu+%zu", (long long)nd.chan_dim, (long long)nd.inner, nd.aux.offset, nd.codes.offset,
                 nd.codes.size);
         if (nd.d.op_kind == RLX_OP_DEQUANT_MATMUL && nd.aux.size) put(" step workspace@%zu+%zu", nd.aux.offset, nd.aux.size);
+        if (nd.d.op_kind == RLX_OP_DEQUANT_GROUPED_MATMUL && nd.aux.size) put(" expert-sorted, workspace@%zu+%zu", nd.aux.offset, nd.aux.size);
         if (nd.img_step >= 0) put(" -> prefill image of step %d%s", nd.img_step, nd.keep_f32 ? "" : " (f32 tensor not written)");
         if (nd.x_image) put(" [x: binary16 image]");
         if (nd.d.op_kind == RLX_OP_RMS_NORM || nd.d.op_kind == RLX_OP_FUSED_SWIGLU) put(" h=%lld", (long long)nd.h);

@@ -88,6 +88,9 @@ struct GemmArgs {
     const void *sxh;
     int m_rows, m_out, k_pad, units, pair_rows, steps_per_split, use_atomics, sc_off;
     const float *rowfac;
+    const int *tile_expert;
+    const int *perm;
+    long long slab_bytes;
 };
 struct XPrepArgs {
     const void *x;
@@ -95,6 +98,15 @@ struct XPrepArgs {
     void *sxh;
     int m, k, k_pad, m_rows, x_dtype;
     float *rowfac;
+    const int *perm;
+    int perm_len;
+};
+constexpr int MOE_MAX_EXPERTS = 256;
+struct MoeSortArgs {  // mirrors kernels/moe.hip
+    const float *expert_idx;
+    int m, num_experts, group_rows, perm_len;
+    int *perm;
+    int *tile_expert;
 };
 
 static int x_kind(int x_dtype) {
@@ -308,11 +320,13 @@ static GemmPlan gemm_plan(int scheme, int xk, int64_t m, int64_t k) {
 }
 
 // The conversion of x [m, k] into the workspace: one look at every row for its prescale factor, then the image.
-static int launch_xprep(const void *x, int xk, int64_t m, int64_t k, const GemmPlan &p, void *workspace, hipStream_t stream) {
+// With `perm` the image's row i is row perm[i] of x (tokens sorted by expert, padding rows -1), m still counting the rows of x.
+static int launch_xprep(const void *x, int xk, int64_t m, int64_t k, const GemmPlan &p, void *workspace, hipStream_t stream,
+                        const int *perm = nullptr, int perm_len = 0) {
     float *fac = (float *)workspace;
     void *xh = (uint8_t *)workspace + p.fac_bytes;
     void *sxh = p.sxh_bytes ? (uint8_t *)workspace + p.fac_bytes + p.xh_bytes : nullptr;
-    XPrepArgs xa{x, xh, sxh, (int)m, (int)k, (int)p.k_pad, (int)p.m_rows, xk, fac};
+    XPrepArgs xa{x, xh, sxh, (int)m, (int)k, (int)p.k_pad, (int)p.m_rows, xk, fac, perm, perm_len};
     void *xparams[] = {&xa};
     RLX_TRY(launch(K_XROWSCALE, (unsigned)((m + 3) / 4), 1, 256, 0, stream, xparams));
     const long long xblocks = (p.m_rows / 256) * (p.k_pad / 64) * 8;  // (tile, step, 32-row sub-tile)
@@ -944,6 +958,95 @@ int rlx_mi355x_rmsnorm_gguf_tied_lm_topk(const float *hidden_dev, const float *g
     const RmsNorm norm{gamma_dev, beta_dev, eps};
     return tied_lm_topk("rmsnorm_gguf_tied_lm_topk", hidden_dev, 0, &norm, embed, cap, out_idx_dev, out_val_dev, scratch_dev, scratch_bytes,
                         stream);
+}
+
+namespace rlx {
+// Sizes of the expert-sorted path: an expert's run of tokens is padded to one 64-row tile of the prefill image (64 tokens,
+// or 32 where an f32 token takes two image rows), so the sorted order holds at most m + experts * (group - 1) rows.
+struct MoePlan {
+    int group;        // tokens per tile
+    int64_t perm_len; // rows of the sorted, padded order
+    size_t head;      // bytes of perm + tile_expert in front of the GEMM workspace
+    GemmPlan gemm;
+    size_t total() const { return head + gemm.total(); }
+};
+static MoePlan moe_plan(int scheme, int xk, int64_t m, int64_t k, int64_t experts) {
+    MoePlan p;
+    p.group = xk == 0 ? 32 : 64;
+    p.perm_len = (m + experts * (p.group - 1) + p.group - 1) / p.group * p.group;
+    p.head = ((size_t)(p.perm_len + p.perm_len / p.group) * 4 + 255) & ~(size_t)255;
+    p.gemm = gemm_plan(scheme, xk, p.perm_len, k);
+    return p;
+}
+static bool moe_sorted_applies(int xk, int64_t m, int64_t experts) { return m > decode_rows(xk) && experts <= MOE_MAX_EXPERTS; }
+}  // namespace rlx
+
+size_t rlx_mi355x_gguf_grouped_matmul_workspace(int scheme, int x_dtype, int64_t m, int64_t k, int64_t num_experts) {
+    using namespace rlx;
+    const int xk = x_kind(x_dtype);
+    if (xk < 0 || layout_of(scheme).unit_k == 0 || m <= 0 || k <= 0 || num_experts < 1 || !moe_sorted_applies(xk, m, num_experts)) return 0;
+    return moe_plan(scheme, xk, m, k, num_experts).total();
+}
+
+int rlx_mi355x_gguf_grouped_matmul_bt_ws(const void *x_dev, int x_dtype, const rlx_qweight *w, const float *expert_idx_dev,
+                                         float *out_dev, int64_t m, void *workspace, size_t workspace_bytes, void *stream) {
+    using namespace rlx;
+    if (!x_dev || !w || !expert_idx_dev || !out_dev || m <= 0) {
+        set_error("gguf_grouped_matmul_bt: null argument or m=%lld", (long long)m);
+        return RLX_ERR_INVALID;
+    }
+    const int xk = x_kind(x_dtype);
+    if (xk < 0) {
+        set_error("gguf_grouped_matmul_bt: activation dtype %d is not F32 / BF16 / F16", x_dtype);
+        return RLX_ERR_UNSUPPORTED;
+    }
+    if (!moe_sorted_applies(xk, m, w->experts))  // decode sizes (or more experts than the sort kernel counts): a launch per eight tokens
+        return rlx_mi355x_gguf_grouped_matmul_bt(x_dev, x_dtype, w, expert_idx_dev, out_dev, m, stream);
+    const MoePlan p = moe_plan(w->scheme, xk, m, w->dims.k, w->experts);
+    if (!workspace || workspace_bytes < p.total() || (uintptr_t)workspace % 16 != 0 || (uintptr_t)x_dev % 16 != 0) {
+        set_error("gguf_grouped_matmul_bt: m=%lld over %d experts needs a 16-byte aligned workspace of %zu bytes, got %zu", (long long)m,
+                  w->experts, p.total(), workspace_bytes);
+        return RLX_ERR_INVALID;
+    }
+    if (p.gemm.m_rows > 0x7FFFFFFF || m > 0x7FFFFFFF / 2) {
+        set_error("gguf_grouped_matmul_bt: m=%lld is beyond the 32-bit row indices of the sorted path", (long long)m);
+        return RLX_ERR_UNSUPPORTED;
+    }
+    RLX_TRY(runtime_init());
+    hipStream_t s = (hipStream_t)stream;
+    int *perm = (int *)workspace, *tile_expert = perm + p.perm_len;
+    void *gws = (uint8_t *)workspace + p.head;
+    MoeSortArgs sa{expert_idx_dev, (int)m, w->experts, p.group, (int)p.perm_len, perm, tile_expert};
+    void *sparams[] = {&sa};
+    RLX_TRY(launch(K_MOE_SORT, 1, 1, 1024, 0, s, sparams));
+    RLX_TRY(launch_xprep(x_dev, xk, m, w->dims.k, p.gemm, gws, s, perm, (int)p.perm_len));
+    const Layout L = w->layout;
+    GemmArgs a{};
+    a.seg[0] = GemmSeg{w->dev, out_dev, (int)w->dims.n, (int)w->dims.row_tiles, 0};
+    a.nseg = 1;
+    a.xh = (uint8_t *)gws + p.gemm.fac_bytes;
+    a.sxh = p.gemm.sxh_bytes ? (uint8_t *)gws + p.gemm.fac_bytes + p.gemm.xh_bytes : nullptr;
+    a.m_rows = (int)p.gemm.m_rows;
+    a.m_out = (int)p.perm_len;  // bound of the sorted rows; every perm entry is a token below m <= perm_len
+    a.k_pad = (int)p.gemm.k_pad;
+    a.units = (int)w->dims.units;
+    a.pair_rows = xk == 0 ? 1 : 0;
+    a.steps_per_split = (int)w->dims.units * (L.unit_k / 64);
+    a.use_atomics = 0;
+    a.sc_off = w->sc_off();
+    a.rowfac = (const float *)gws;
+    a.tile_expert = tile_expert;
+    a.perm = perm;
+    a.slab_bytes = w->dims.bytes;
+    void *params[] = {&a};
+    const KernelId id = w->scheme == SCHEME_Q4K    ? K_GEMM64G_Q4_K
+                        : w->scheme == SCHEME_Q4_0 ? K_GEMM64G_Q4_0
+                        : layout_is_f16w(L)        ? K_GEMM64G_F16W
+                        : w->scheme == SCHEME_Q6K  ? K_GEMM64G_Q6_K
+                        : w->scheme == SCHEME_Q5K  ? K_GEMM64G_Q5_K
+                                                   : K_GEMM64G_Q8_0;
+    const unsigned gx = (unsigned)((w->dims.row_tiles * 16 + 127) / 128), gy = (unsigned)(p.perm_len / p.group);
+    return launch3(id, gx, gy, 1, 512, 3 * 24 * 1024, s, params);
 }
 
 int rlx_mi355x_gguf_grouped_matmul_bt(const void *x_dev, int x_dtype, const rlx_qweight *w, const float *expert_idx_dev,

@@ -3,5 +3,6 @@
 #include "fakequant.hip"
 #include "gemm.hip"
 #include "gemv.hip"
+#include "moe.hip"
 #include "rowops.hip"
 #include "topk.hip"

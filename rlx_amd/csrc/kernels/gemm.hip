@@ -43,6 +43,11 @@ struct GemmArgs {
     int use_atomics;      // split K: accumulate into a zeroed `out` with atomic adds
     int sc_off;           // Q6_K: a stored scale byte stands for byte - sc_off (0 unsigned reading, 128 signed)
     const float *rowfac;  // [m_out][2]: the power of two row i of x was multiplied by when it was converted, and its inverse
+    // Expert-sorted launch (rlx_gemm64g_*): the image rows are tokens sorted by expert, every 64-row tile inside one
+    // expert's run (see rlx_moe_sort); a tile multiplies the slab tile_expert names and writes row perm[.] of `out`.
+    const int *tile_expert;
+    const int *perm;
+    long long slab_bytes;
 };
 
 // half2 (v, v) with v = byte `byte` of word as an exact binary16 integer: bytes [b, 0x64, b, 0x64] = 1024 + b
@@ -72,7 +77,7 @@ __device__ __forceinline__ int frag_offset(int ns, int ks, int s, int r, int h) 
 // TI x TJ = MFMA tiles per wave: 2 x 2 is the prefill shape above; 1 x 1 puts the eight waves as 2 x 4 over a 64 x 128
 // tile for batches of a few dozen rows, where the job is to stream the weights and most of a 256-row tile would be
 // padding. Both read the same activation workspace (a 64-row tile is two 32-row sub-tiles of a 256-row image).
-template <int SCHEME, int TI, int TJ>
+template <int SCHEME, int TI, int TJ, bool GROUPED = false>
 __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
     constexpr Layout L = layout_of(SCHEME);
     constexpr bool K5 = SCHEME == SCHEME_Q5K;                 // Q4_K with a fifth bit: every Q4_K branch below serves both
@@ -87,6 +92,12 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
 
     const int tid = threadIdx.x, lane = tid & 63;
+    int expert = 0;
+    if constexpr (GROUPED) {
+        static_assert(TI == 1 && TJ == 1, "an expert's run is padded to the 64-row tile");
+        expert = a.tile_expert[blockIdx.y];  // workgroup-uniform
+        if (expert < 0) return;              // past the last run: nothing to do, and no barrier has been reached
+    }
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WN, wn = wave % WN;
     const int lr = lane & 31, lh = lane >> 5;
@@ -95,6 +106,7 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
     for (int i = 1; i < GEMM_MAX_SEG; i++)
         if (i < a.nseg && (int)blockIdx.x >= a.seg[i].tile_begin) si = i;
     const GemmSeg sg = a.seg[si];
+    const uint8_t *w_base = sg.w + (GROUPED ? (long long)expert * a.slab_bytes : 0LL);  // this launch's matrix, or the tile's expert slab
     const int bx = (int)blockIdx.x - sg.tile_begin;
     const int n_tile0 = bx * GEMM_NT, m_tile0 = blockIdx.y * MT;
     const int step0 = blockIdx.z * a.steps_per_split;
@@ -112,7 +124,7 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
     const int b_n16 = lane & 15, b_g = lane >> 4;
     const int b_t16 = bx * (GEMM_NT / 16) + wave;
     const bool b_live = b_t16 < sg.row_tiles;
-    const uint8_t *b_tile = sg.w + (long long)(b_live ? b_t16 : 0) * a.units * L.unit_bytes;
+    const uint8_t *b_tile = w_base + (long long)(b_live ? b_t16 : 0) * a.units * L.unit_bytes;
     const uint32_t b_keep = b_live ? 0xFFFFFFFFu : 0u;
     const half2_t sc_bias = ubyte_bias(a.sc_off);                 // Q6_K scale bytes: value = byte - sc_off
     const uint32_t sc_dead = (uint32_t)a.sc_off * 0x01010101u;    // the byte that reads as a zero scale
@@ -247,7 +259,7 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
     for (int j = 0; j < TJ; j++) {
         my_row[j] = n_tile0 + (wn * TJ + j) * 32 + lr;
         my_ok[j] = (my_row[j] >> 4) < sg.row_tiles;
-        my_meta[j] = sg.w + (long long)(my_ok[j] ? (my_row[j] >> 4) : 0) * a.units * L.unit_bytes +
+        my_meta[j] = w_base + (long long)(my_ok[j] ? (my_row[j] >> 4) : 0) * a.units * L.unit_bytes +
                      (K6 ? 3328 + (my_row[j] & 15) * 2 : META_OFF + (my_row[j] & 15) * 16);  // Q6_K: the row's d; Q4_K / Q5_K: its 16 meta bytes
     }
     uint4_t w_meta[TJ];
@@ -461,7 +473,8 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
                     v = v + total[i][j][e + 1] * (1.0f / GEMM_LO_SCALE);
                     orow = vrow >> 1;
                 }
-                if (orow < a.m_out) {
+                if constexpr (GROUPED) orow = orow < a.m_out ? a.perm[orow] : -1;  // the token this sorted row is (-1: padding)
+                if (orow >= 0 && orow < a.m_out) {
                     v *= a.rowfac[2 * orow + 1];  // undo the row's prescale (1 for a row binary16 carries as it is)
                     float *p = sg.out + (long long)orow * sg.n + col;
                     if (a.use_atomics) atomicAdd(p, v);
@@ -482,6 +495,8 @@ struct XPrepArgs {
     int m, k, k_pad, m_rows;
     int x_dtype;  // 0 f32 (rows become hi / lo*2048 pairs), 1 bf16, 2 f16
     float *rowfac;  // [m][2] (forward factor, its inverse), written by rlx_xrowscale before rlx_xprep runs
+    const int *perm;  // expert-sorted image: row i of the image is row perm[i] of x (-1: a padding row of zeros); else null
+    int perm_len;
 };
 
 // Activations travel as binary16, and so do the sums of 32 of them that the Q4_K / Q5_K min term needs. rlx_xrowscale
@@ -542,12 +557,14 @@ __device__ __forceinline__ void xprep_body(const XPrepArgs &a) {
     const long long vrow = (long long)tile * GEMM_MT + sub * 32 + r;
     const int col = step * GEMM_KS + c * 8;
     const bool paired = a.x_dtype == 0;
-    const long long src_row = paired ? (vrow >> 1) : vrow;
+    long long src_row = paired ? (vrow >> 1) : vrow;
+    if (a.perm) src_row = src_row < a.perm_len ? a.perm[src_row] : -1;
     float v[8];
 #pragma unroll
     for (int e = 0; e < 8; e++) v[e] = 0.f;
-    const float fwd = src_row < a.m ? a.rowfac[2 * src_row] : 1.f;
-    if (src_row < a.m && col < a.k) {  // k is a multiple of 32, so a chunk of 8 is inside or outside as a whole
+    const bool live_row = src_row >= 0 && src_row < a.m;
+    const float fwd = live_row ? a.rowfac[2 * src_row] : 1.f;
+    if (live_row && col < a.k) {  // k is a multiple of 32, so a chunk of 8 is inside or outside as a whole
         if (a.x_dtype == 0) {
             const float4_t *p = (const float4_t *)((const float *)a.x + src_row * a.k + col);
             float4_t t0 = p[0], t1 = p[1];
@@ -608,5 +625,11 @@ extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64_f16w(rlx::GemmAr
 extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64_q4_k(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q4K, 1, 1>(a); }
 extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64_q4_0(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q4_0, 1, 1>(a); }
 extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64_q8_0(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q8_0, 1, 1>(a); }
+extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64g_q4_k(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q4K, 1, 1, true>(a); }
+extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64g_q4_0(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q4_0, 1, 1, true>(a); }
+extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64g_q8_0(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q8_0, 1, 1, true>(a); }
+extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64g_q5_k(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q5K, 1, 1, true>(a); }
+extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64g_q6_k(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q6K, 1, 1, true>(a); }
+extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64g_f16w(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_F16W, 1, 1, true>(a); }
 extern "C" __global__ __launch_bounds__(256) void rlx_xprep(rlx::XPrepArgs a) { rlx::xprep_body(a); }
 extern "C" __global__ __launch_bounds__(256) void rlx_xrowscale(rlx::XPrepArgs a) { rlx::xrowscale_body(a); }

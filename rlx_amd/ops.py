@@ -206,14 +206,20 @@ def gguf_matmul_bt_batch(xs, ws, m, x_dtype=DType.F32):
     return [o.to_numpy(np.float32).reshape(m, w.n) for o, w in zip(outs, ws)]
 
 
-def gguf_grouped_matmul_bt(x, w: QWeight, expert_idx, x_dtype=DType.F32):
+def gguf_grouped_matmul_bt(x, w: QWeight, expert_idx, x_dtype=DType.F32, sorted_path=True):
     """Host convenience for the MoE matmul: out[i] = x[i] . W[expert_idx[i]]^T; x is [m, k], expert_idx [m]."""
     idx = np.ascontiguousarray(expert_idx, dtype=np.float32)
     m = idx.size
     xd = DeviceBuffer.from_numpy(x)
     idd = DeviceBuffer.from_numpy(idx)
     od = DeviceBuffer(m * w.n * 4)
-    _lib.check(_lib.lib().rlx_mi355x_gguf_grouped_matmul_bt(xd.ptr, int(x_dtype), w.ptr, idd.ptr, od.ptr, m, None))
+    L = _lib.lib()
+    need = L.rlx_mi355x_gguf_grouped_matmul_workspace(int(w.scheme), int(x_dtype), m, w.k, w.num_experts) if sorted_path else 0
+    if need:  # above the decode sizes: tokens sorted by expert, one prefill launch over the whole stack
+        ws = DeviceBuffer(need)
+        _lib.check(L.rlx_mi355x_gguf_grouped_matmul_bt_ws(xd.ptr, int(x_dtype), w.ptr, idd.ptr, od.ptr, m, ws.ptr, need, None))
+    else:
+        _lib.check(L.rlx_mi355x_gguf_grouped_matmul_bt(xd.ptr, int(x_dtype), w.ptr, idd.ptr, od.ptr, m, None))
     sync()
     return od.to_numpy(np.float32).reshape(m, w.n)
 
