@@ -203,17 +203,17 @@ def main():
     }
 
     other = "layer" if args.wiring == "independent" else "independent"
-    host_ms = None
-    if args.extra:
-        # the same layer through the host-buffer boundary (ExecutableGraph::run: seven H2D copies, the launch, seven
-        # D2H copies, synchronous) - PCIe and call overhead included, reported beside the headline, never as `value`
-        ins = [(src, v) for src, v in {WIRING[args.wiring][n]: xs[n] for n, _, _ in LLAMA8B if xs[n] is not None}.items()]
-        for _ in range(3):
-            layers[0].run(ins)
-        t1 = time.time()
-        for i in range(50):
-            layers[i % len(layers)].run(ins)
-        host_ms = (time.time() - t1) / 50 * 1e3
+    # the same layer through the host-buffer boundary (ExecutableGraph::run: the inputs up in one copy out of pinned
+    # memory, the launch, the outputs back in one copy, synchronous) - PCIe and call overhead included, reported beside
+    # the headline, never as `value`
+    ins = [(src, v) for src, v in {WIRING[args.wiring][n]: xs[n] for n, _, _ in LLAMA8B if xs[n] is not None}.items()]
+    for _ in range(5):
+        layers[0].run(ins)
+    t1 = time.time()
+    for i in range(100):
+        layers[i % len(layers)].run(ins)
+    host_ms = (time.time() - t1) / 100 * 1e3
+    result["config"]["host_boundary_ms_per_call"] = round(host_ms, 4)
     del layers
     # the other wiring of the same layer, beside the headline: "layer" is what a decode loop gets (four launches, each
     # waiting for the one before)
@@ -243,7 +243,7 @@ def main():
         result["extra"] = extra_configs(rlx_amd, stream)
         result["extra"]["q4_0_gemv_llama8b_layer_host_boundary"] = {
             "ms_per_call": round(host_ms, 4), "GB/s": round(layer_bytes / host_ms / 1e6, 1),
-            "note": "rlx_exec_run with host inputs and outputs (H2D + launch + D2H, synchronous)"}
+            "note": "rlx_exec_run with host inputs and outputs (H2D + launch + D2H, synchronous), called from Python"}
 
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(base, xs)

@@ -156,6 +156,12 @@ struct rlx_exec {
     hipStream_t own_stream = nullptr;  // created at compile time
     hipGraph_t graph = nullptr;
     hipGraphExec_t graph_exec = nullptr;
+    // Host boundary of run(): the Input slots are neighbours at the start of the arena and the output slots neighbours
+    // after the sources, so a call that brings every input moves each direction as one copy through pinned memory
+    // (a copy from pageable memory is staged by the runtime one buffer at a time).
+    size_t in_lo = 0, in_hi = 0, out_lo = 0, out_hi = 0;  // arena spans of all inputs / all outputs
+    uint8_t *stage = nullptr;                             // pinned: [in span][out span], allocated on the first run()
+    bool stage_tried = false;
 
     ~rlx_exec() {
         for (auto &nd : nodes) {
@@ -164,6 +170,7 @@ struct rlx_exec {
             if (nd.qw) rlx_mi355x_qweight_destroy(nd.qw);
         }
         drop_graph();
+        if (stage) (void)hipHostFree(stage);
         if (arena) (void)hipFree(arena);
         if (own_stream) (void)hipStreamDestroy(own_stream);
     }
@@ -592,24 +599,37 @@ static std::unique_ptr<rlx_exec> plan_graph(const rlx_graph_desc *g, const rlx_c
         return s;
     };
     const uint32_t wflags = e->opts.q6k_signed_scales ? (uint32_t)RLX_QW_Q6K_SIGNED_SCALES : 0u;
+    for (Node &nd : e->nodes)  // the inputs side by side at the start: one span for the host boundary to fill
+        if (nd.d.op_kind == RLX_OP_INPUT) {
+            nd.slot = take((size_t)nd.numel * 4, 0, kForever);  // room for an f32 upload even when declared 16-bit
+            nd.cur_dtype = nd.d.dtype;
+            e->in_hi = arena_end;
+        }
     for (Node &nd : e->nodes) {  // whole-life buffers first, so the reusable ones pack above them
-        if (!is_source(nd.d.op_kind)) continue;
+        if (!is_source(nd.d.op_kind) || nd.d.op_kind == RLX_OP_INPUT) continue;
         if (nd.is_packed) {
             nd.w_flags = nd.scheme == SCHEME_Q6K ? wflags : 0u;
             nd.slot = take((size_t)weight_dims(host_layout(nd.scheme), nd.w_n, nd.w_k).bytes * (size_t)nd.w_experts, 0, kForever);  // device layout, resident
-        } else if (nd.d.op_kind == RLX_OP_INPUT) {
-            nd.slot = take((size_t)nd.numel * 4, 0, kForever);  // room for an f32 upload even when declared 16-bit
-            nd.cur_dtype = nd.d.dtype;
         } else {
             nd.slot = take((size_t)nd.numel * dtype_size(nd.d.dtype), 0, kForever);
         }
+    }
+    // the outputs side by side next: they live to the end of the run anyway, and one span comes back in one copy
+    std::vector<bool> placed_early(e->nodes.size(), false);
+    e->out_lo = e->out_hi = arena_end;
+    for (uint32_t id : e->outputs) {
+        Node &nd = e->nodes[id];
+        if (is_source(nd.d.op_kind) || placed_early[id]) continue;
+        nd.slot = take((size_t)nd.numel * dtype_size(nd.d.dtype), 0, kForever);
+        placed_early[id] = true;
+        e->out_hi = arena_end;
     }
     for (size_t si = 0; si < e->steps.size(); si++) {
         const std::vector<uint32_t> &step = e->steps[si];
         size_t step_ws = 0;
         for (uint32_t id : step) {
             Node &nd = e->nodes[id];
-            if (!(nd.img_step >= 0 && !nd.keep_f32))  // a FakeQuantize result that only travels as a prefill image has no slot
+            if (!(nd.img_step >= 0 && !nd.keep_f32) && !placed_early[id])  // a FakeQuantize result that only travels as a prefill image has no slot
                 nd.slot = take((size_t)nd.numel * dtype_size(nd.d.dtype), (int)si, last_use[id]);
             if (nd.d.op_kind == RLX_OP_FAKE_QUANTIZE) {
                 nd.aux = take(rlx_mi355x_fake_quantize_scratch_bytes(nd.numel, nd.chan_dim, nd.inner), (int)si, (int)si);
@@ -739,26 +759,15 @@ int rlx_exec_set_param(rlx_exec *e, const char *name, const float *data, size_t 
     return rlx_exec_set_param_typed(e, name, data, n * 4, RLX_F32);
 }
 
+static int check_input(rlx_exec *e, const char *name, const void *data, size_t nbytes, uint32_t dtype, Node **node);
+
 int rlx_exec_write_input(rlx_exec *e, const char *name, const void *data, size_t nbytes, uint32_t dtype) {
-    if (!e || !name || !data) {
-        set_error("write_input: null argument");
-        return RLX_ERR_INVALID;
-    }
-    auto it = e->inputs.find(name);
-    if (it == e->inputs.end()) return RLX_WARN_UNKNOWN_NAME;
-    Node &nd = e->nodes[it->second];
-    size_t es = dtype == RLX_F32 ? 4 : (dtype == RLX_F16 || dtype == RLX_BF16) ? 2 : 0;
-    if (es == 0) {
-        set_error("run: input '%s' dtype %u unsupported (F32/F16/BF16 only)", name, dtype);
-        return RLX_ERR_UNSUPPORTED;
-    }
-    if (nbytes != (size_t)nd.numel * es) {
-        set_error("run: input '%s' needs %lld elements, got %zu bytes of dtype %u", name, (long long)nd.numel, nbytes, dtype);
-        return RLX_ERR_INVALID;
-    }
-    RLX_HIP(hipMemcpyAsync(e->ptr(nd.slot), data, nbytes, hipMemcpyHostToDevice, e->stream));
-    if (nd.cur_dtype != dtype) e->drop_graph();  // the captured launches were specialised on the old dtype
-    nd.cur_dtype = dtype;
+    Node *nd = nullptr;
+    const int rc = check_input(e, name, data, nbytes, dtype, &nd);
+    if (rc != RLX_OK) return rc;
+    RLX_HIP(hipMemcpyAsync(e->ptr(nd->slot), data, nbytes, hipMemcpyHostToDevice, e->stream));
+    if (nd->cur_dtype != dtype) e->drop_graph();  // the captured launches were specialised on the old dtype
+    nd->cur_dtype = dtype;
     return RLX_OK;
 }
 
@@ -991,6 +1000,30 @@ int rlx_exec_sync(rlx_exec *e) {
 
 void *rlx_exec_stream(rlx_exec *e) { return e ? e->stream : nullptr; }
 
+// Checks one named input of run() / write_input(); *node is set to its node, or the return is RLX_WARN_UNKNOWN_NAME.
+static int check_input(rlx_exec *e, const char *name, const void *data, size_t nbytes, uint32_t dtype, Node **node) {
+    if (!e || !name || !data) {
+        set_error("write_input: null argument");
+        return RLX_ERR_INVALID;
+    }
+    auto it = e->inputs.find(name);
+    if (it == e->inputs.end()) return RLX_WARN_UNKNOWN_NAME;
+    Node &nd = e->nodes[it->second];
+    size_t es = dtype == RLX_F32 ? 4 : (dtype == RLX_F16 || dtype == RLX_BF16) ? 2 : 0;
+    if (es == 0) {
+        set_error("run: input '%s' dtype %u unsupported (F32/F16/BF16 only)", name, dtype);
+        return RLX_ERR_UNSUPPORTED;
+    }
+    if (nbytes != (size_t)nd.numel * es) {
+        set_error("run: input '%s' needs %lld elements, got %zu bytes of dtype %u", name, (long long)nd.numel, nbytes, dtype);
+        return RLX_ERR_INVALID;
+    }
+    *node = &nd;
+    return RLX_OK;
+}
+
+constexpr size_t kStageCap = 16u << 20;  // beyond this a copy is long enough to hide how it is issued
+
 static int run_common(rlx_exec *e, const rlx_named_buf *inputs, size_t n_inputs, rlx_out_buf *outputs, size_t n_outputs,
                       bool typed) {
     clear_error();
@@ -998,17 +1031,45 @@ static int run_common(rlx_exec *e, const rlx_named_buf *inputs, size_t n_inputs,
         set_error("run: null argument");
         return RLX_ERR_INVALID;
     }
-    int warn = RLX_OK;
-    for (size_t i = 0; i < n_inputs; i++) {
-        int rc = rlx_exec_write_input(e, inputs[i].name, inputs[i].data, inputs[i].nbytes, typed ? inputs[i].dtype : (uint32_t)RLX_F32);
-        if (rc < 0) return rc;
-        if (rc > 0) warn = rc;
-    }
-    RLX_TRY(rlx_exec_launch(e));
     if (n_outputs > e->outputs.size()) {
         set_error("run: %zu output buffers for a graph with %zu outputs", n_outputs, e->outputs.size());
         return RLX_ERR_INVALID;
     }
+    const size_t in_span = e->in_hi - e->in_lo, out_span = e->out_hi - e->out_lo;
+    if (!e->stage_tried) {
+        e->stage_tried = true;
+        if (in_span + out_span > 0 && in_span + out_span <= kStageCap &&
+            hipHostMalloc((void **)&e->stage, in_span + out_span, hipHostMallocDefault) != hipSuccess) {
+            (void)hipGetLastError();
+            e->stage = nullptr;  // no pinned memory to be had: the copies go from the caller's buffers
+        }
+    }
+    int warn = RLX_OK;
+    // every input of the graph named exactly once -> one copy of the whole input span out of pinned memory
+    std::vector<Node *> in_nodes(n_inputs, nullptr);
+    size_t known = 0;
+    for (size_t i = 0; i < n_inputs; i++) {
+        int rc = check_input(e, inputs[i].name, inputs[i].data, inputs[i].nbytes, typed ? inputs[i].dtype : (uint32_t)RLX_F32, &in_nodes[i]);
+        if (rc < 0) return rc;
+        if (rc > 0) warn = rc;
+        else known++;
+    }
+    bool staged_in = e->stage && in_span > 0 && known == e->inputs.size();
+    for (size_t i = 0; i < n_inputs && staged_in; i++)
+        for (size_t j = 0; j < i; j++)
+            if (in_nodes[i] && in_nodes[i] == in_nodes[j]) staged_in = false;  // a name given twice: keep the caller's order of writes
+    for (size_t i = 0; i < n_inputs; i++) {
+        Node *nd = in_nodes[i];
+        if (!nd) continue;
+        const uint32_t dt = typed ? inputs[i].dtype : (uint32_t)RLX_F32;
+        if (staged_in) memcpy(e->stage + (nd->slot.offset - e->in_lo), inputs[i].data, inputs[i].nbytes);
+        else RLX_HIP(hipMemcpyAsync(e->ptr(nd->slot), inputs[i].data, inputs[i].nbytes, hipMemcpyHostToDevice, e->stream));
+        if (nd->cur_dtype != dt) e->drop_graph();  // the captured launches were specialised on the old dtype
+        nd->cur_dtype = dt;
+    }
+    if (staged_in) RLX_HIP(hipMemcpyAsync(e->arena + e->in_lo, e->stage, in_span, hipMemcpyHostToDevice, e->stream));
+    RLX_TRY(rlx_exec_launch(e));
+    bool staged_out = e->stage && out_span > 0;
     for (size_t i = 0; i < n_outputs; i++) {
         Node &nd = e->nodes[e->outputs[i]];
         size_t bytes = (size_t)nd.numel * dtype_size(nd.d.dtype);
@@ -1016,11 +1077,22 @@ static int run_common(rlx_exec *e, const rlx_named_buf *inputs, size_t n_inputs,
             set_error("run: output %zu needs %zu bytes, buffer has %zu", i, bytes, outputs[i].capacity);
             return RLX_ERR_INVALID;
         }
-        RLX_HIP(hipMemcpyAsync(outputs[i].data, e->ptr(nd.slot), bytes, hipMemcpyDeviceToHost, e->stream));
+        if (nd.slot.offset < e->out_lo || nd.slot.offset + bytes > e->out_hi) staged_out = false;  // an input handed back as output
+    }
+    if (staged_out) RLX_HIP(hipMemcpyAsync(e->stage + in_span, e->arena + e->out_lo, out_span, hipMemcpyDeviceToHost, e->stream));
+    for (size_t i = 0; i < n_outputs; i++) {
+        Node &nd = e->nodes[e->outputs[i]];
+        const size_t bytes = (size_t)nd.numel * dtype_size(nd.d.dtype);
+        if (!staged_out) RLX_HIP(hipMemcpyAsync(outputs[i].data, e->ptr(nd.slot), bytes, hipMemcpyDeviceToHost, e->stream));
         outputs[i].nbytes = bytes;
         outputs[i].dtype = nd.d.dtype;
     }
     RLX_HIP(hipStreamSynchronize(e->stream));
+    if (staged_out)
+        for (size_t i = 0; i < n_outputs; i++) {
+            const Node &nd = e->nodes[e->outputs[i]];
+            memcpy(outputs[i].data, e->stage + in_span + (nd.slot.offset - e->out_lo), outputs[i].nbytes);
+        }
     return warn;
 }
 

@@ -789,3 +789,35 @@ def test_activation_range_through_fused_entry_points(oracle):
     assert np.array_equal(routed.view(np.uint32), plain.view(np.uint32))
     wu.free()
     wg.free()
+
+
+def test_run_boundary_full_and_partial_inputs(oracle):
+    # run() with every input named moves each direction as one copy through pinned memory; with some inputs left out
+    # (their last contents stay, as in the reference's arena) or written on the device path in between it copies buffer by
+    # buffer. An input handed back as an output comes from its own slot. All three must agree with the oracle.
+    k, n = 256, 48
+    p1, p2 = make_weights(Q4_0, n, k, seed=201)[0], make_weights(Q4_0, n, k, seed=202)[0]
+    g = Graph.new("two_inputs")
+    x1, x2 = g.input("x1", Shape.new([2, k], DType.F32)), g.input("x2", Shape.new([2, k], DType.F32))
+    w1, w2 = g.param("w1", Shape.new([len(p1)], DType.U8)), g.param("w2", Shape.new([len(p2)], DType.U8))
+    y1 = g.add_node(Op.DequantMatMul(QuantScheme.GgufQ4_0), [x1, w1], Shape.new([2, n], DType.F32))
+    y2 = g.add_node(Op.DequantMatMul(QuantScheme.GgufQ4_0), [x2, w2], Shape.new([2, n], DType.F32))
+    g.set_outputs([y1, y2, x2])
+    c = Session.new().compile(g)
+    c.set_param_typed("w1", p1, DType.U8)
+    c.set_param_typed("w2", p2, DType.U8)
+    rng = np.random.default_rng(203)
+    a, b, b2, a2 = (rng.standard_normal((2, k)).astype(np.float32) for _ in range(4))
+
+    def check(outs, xa, xb, tag):
+        assert rel_err(outs[0].reshape(2, n), oracle.gguf_matmul_f64(xa, p1, 2, k, n, Q4_0)) <= TOL, tag
+        assert rel_err(outs[1].reshape(2, n), oracle.gguf_matmul_f64(xb, p2, 2, k, n, Q4_0)) <= TOL, tag
+        assert np.array_equal(outs[2].reshape(2, k), xb), tag
+
+    check(c.run([("x1", a), ("x2", b)]), a, b, "all inputs")
+    check(c.run([("x1", a2)]), a2, b, "x2 left as it was")
+    c.write_input("x2", b2)
+    check(c.run([("x1", a)]), a, b2, "x2 written on the device path")
+    check(c.run([("x2", b), ("x1", a2)]), a2, b, "all inputs again, other order")
+    bf = c.run_typed([("x1", f32_to_bf16_bits(oracle.bf16_round(a)), DType.BF16), ("x2", b, DType.F32)])
+    assert rel_err(bf[0][0].reshape(2, n), oracle.gguf_matmul_f64(oracle.bf16_round(a), p1, 2, k, n, Q4_0)) <= TOL

@@ -149,10 +149,10 @@ def test_qweight_create_validates_before_allocating():
 
 
 def test_plan_reuses_dead_slots():
-    # FakeQuantize -> matmul -> matmul -> matmul: the third matmul's output may take the bytes of the first's, which is dead
-    # by then, and a step's workspace lives for that step only (rlx-compile/src/memory.rs:386-470 is the contract). The
+    # FakeQuantize -> four matmuls in a chain: the third matmul's result may take the bytes of the first's, which is dead by
+    # then, and a step's workspace lives for that step only (rlx-compile/src/memory.rs:386-470 is the contract). The
     # fake-quantized tensor itself is read by a prefill matmul only, so it is written as that step's operand image and has
-    # no f32 slot at all.
+    # no f32 slot at all. Inputs sit side by side at the start of the arena and outputs side by side after the sources.
     g = Graph.new("chain")
     x = g.input("x", Shape.new([64, 4096], DType.F32))
     fq = g.add_node(Op.FakeQuantize(8, 1), [x], Shape.new([64, 4096], DType.F32))
@@ -162,7 +162,9 @@ def test_plan_reuses_dead_slots():
     z = g.add_node(Op.DequantMatMul(QuantScheme.GgufQ8_0), [y, w2], Shape.new([64, 128], DType.F32))
     w3 = g.param("w3", Shape.new([128 * 64 // 32 * 34], DType.U8))
     z2 = g.add_node(Op.DequantMatMul(QuantScheme.GgufQ8_0), [z, w3], Shape.new([64, 64], DType.F32))
-    g.set_outputs([z2])
+    w4 = g.param("w4", Shape.new([64 * 32 // 32 * 34], DType.U8))
+    z3 = g.add_node(Op.DequantMatMul(QuantScheme.GgufQ8_0), [z2, w4], Shape.new([64, 32], DType.F32))
+    g.set_outputs([z3])
     def slots_of(text):
         return {int(line.split()[1]): (int(line.split("off=")[1].split()[0]), int(line.split("size=")[1].split()[0]))
                 for line in text.splitlines()[1:]}
@@ -173,23 +175,25 @@ def test_plan_reuses_dead_slots():
 
     total, text = Session().plan(g)
     slots = slots_of(text)
-    assert slots[1][1] == 0 and "f32 tensor not written" in text.splitlines()[2]
-    assert slots[7][0] == slots[3][0]                      # z2 reuses y's slot
+    assert slots[x][0] == 0
+    assert slots[fq][1] == 0 and "f32 tensor not written" in text.splitlines()[1 + fq]
+    assert slots[z2][0] == slots[y][0]                     # z2 reuses y's slot
     bump = sum((sz + 255) // 256 * 256 for _, sz in slots.values())
-    assert total < bump + 3 * 1024 * 1024                  # less than one private slot per buffer plus the workspaces
-    for a in (0, 2, 4, 6):                                 # sources never share bytes with anything
+    assert total < bump + 4 * 1024 * 1024                  # less than one private slot per buffer plus the workspaces
+    for a in (x, w, w2, w3, w4, z3):                       # sources and outputs never share bytes with anything
         for b in slots:
             assert a == b or disjoint(slots, a, b), (a, b)
-    for a, b in ((3, 5), (5, 7)):                          # a matmul's input and output are live together
+    for a, b in ((y, z), (z, z2), (z2, z3)):               # a matmul's input and output are live together
         assert disjoint(slots, a, b), (a, b)
-    # with every intermediate an output nothing may be reused, and the fake-quantized tensor gets its f32 slot back
-    g.set_outputs([z2, z, y, fq])
+    # with every intermediate an output nothing may be reused, the fake-quantized tensor gets its f32 slot back, and the
+    # outputs form one span
+    g.set_outputs([z3, z2, z, y, fq])
     total_all, text_all = Session().plan(g)
     kept = slots_of(text_all)
-    assert kept[1][1] == 64 * 4096 * 4
-    for a in (1, 3, 5, 7):
-        for b in (1, 3, 5, 7):
-            assert a >= b or disjoint(kept, a, b), (a, b)
+    assert kept[fq][1] == 64 * 4096 * 4
+    outs = sorted((kept[i] for i in (z3, z2, z, y, fq)))
+    for (oa, sa), (ob, _) in zip(outs, outs[1:]):
+        assert oa + sa <= ob < oa + sa + 256                # neighbours up to the 256-byte alignment
     assert total_all >= total + 64 * 4096 * 4
     # the integer codes are opt-in: one more resident byte per element
     assert Session(fq_codes=True).plan(g)[0] >= total_all + 64 * 4096
