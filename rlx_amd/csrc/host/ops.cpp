@@ -233,7 +233,7 @@ static int launch_gemv(const void *const *xs, int xk, const rlx_qweight *const *
         sh.kcu = max_units;
         // the last LDS_TAIL bytes: 1 / rms per activation row (RMSNorm prologue), the per-row factors of the binary16 range
         // prescale and its bookkeeping (GEMV_LDS_TAIL in kernels/gemv.hip)
-        constexpr size_t LDS_TAIL = 640;
+        constexpr size_t LDS_TAIL = 448;
         while (sh.kcu > 1 && part_bytes + stage_bytes(sh.kcu) + LDS_TAIL > budget) sh.kcu--;
         sh.fits = part_bytes + stage_bytes(sh.kcu) + LDS_TAIL <= budget;
         sh.lds = part_bytes + stage_bytes(sh.kcu) + LDS_TAIL;

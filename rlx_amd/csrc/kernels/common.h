@@ -14,6 +14,7 @@ typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef float float4_t __attribute__((ext_vector_type(4)));
 typedef float float16_t __attribute__((ext_vector_type(16)));
 typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
+typedef float float2_t __attribute__((ext_vector_type(2)));
 typedef uint32_t uint2_t __attribute__((ext_vector_type(2)));
 
 union Frag {  // one MFMA A/B operand: 8 halfs = 4 dwords

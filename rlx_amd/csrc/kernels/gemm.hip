@@ -397,6 +397,19 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
     // ahead. A SIMD always has one wave issuing MFMAs back to back (raised priority) and one doing the VALU / LDS /
     // global work, instead of two waves that contend for the same slots and then wait for each other.
     const int grp = wave >> 2;  // wave-uniform
+    // The epilogue's per-row data, fetched now so its latency disappears behind the main loop: for output row t of this
+    // tile (two image rows each with f32 activations) the row of `out` it is written to (-1: none) and the factor that
+    // undoes the row's prescale.
+    __shared__ __attribute__((aligned(16))) int out_row_s[MT];
+    __shared__ __attribute__((aligned(16))) float out_fac_s[MT];
+    if (tid < MT) {
+        int orow = a.pair_rows ? (m_tile0 >> 1) + tid : m_tile0 + tid;
+        if (a.pair_rows && tid >= MT / 2) orow = -1;
+        if (orow >= a.m_out) orow = -1;
+        if constexpr (GROUPED) orow = orow >= 0 ? a.perm[orow] : -1;  // the token this sorted row is (-1: padding)
+        out_row_s[tid] = orow;
+        out_fac_s[tid] = orow >= 0 ? a.rowfac[2 * orow + 1] : 0.f;
+    }
     if (step0 < step1) {  // step0 is a multiple of 4
         const int last = step1 - 1;
         fetch_a(step0, 0);
@@ -457,31 +470,52 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
     else run(std::integral_constant<int, 1>{});
 
     // ---- epilogue: register e of tile (i, j) is row 8 (e/4) + 4 lh + e%4, column lr ------------------------
+    // The four rows of a register quad are neighbours, so their output rows and factors come as one 16-byte LDS read
+    // each (8 bytes with f32 activations, where two image rows make one output row), shared by the tiles j.
 #pragma unroll
-    for (int i = 0; i < TI; i++)
+    for (int i = 0; i < TI; i++) {
+        int orow[16];
+        float ofac[16];
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            const int t = (wm * TI + i) * 32 + 8 * q + 4 * lh;  // first row of the quad within the tile
+            if (a.pair_rows) {
+                const uint2_t r2 = *(const uint2_t *)(out_row_s + (t >> 1));
+                const float2_t f2 = *(const float2_t *)(out_fac_s + (t >> 1));
+                orow[4 * q] = (int)r2[0], orow[4 * q + 2] = (int)r2[1];
+                ofac[4 * q] = f2[0], ofac[4 * q + 2] = f2[1];
+                orow[4 * q + 1] = orow[4 * q + 3] = -1;
+                ofac[4 * q + 1] = ofac[4 * q + 3] = 0.f;
+            } else {
+                const uint4_t r4 = *(const uint4_t *)(out_row_s + t);
+                const float4_t f4 = *(const float4_t *)(out_fac_s + t);
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    orow[4 * q + r] = (int)r4[r];
+                    ofac[4 * q + r] = f4[r];
+                }
+            }
+        }
 #pragma unroll
         for (int j = 0; j < TJ; j++) {
             const int col = my_row[j];
             if (col >= sg.n) continue;
 #pragma unroll
             for (int e = 0; e < 16; e++) {
-                const int vrow = m_tile0 + (wm * TI + i) * 32 + 8 * (e >> 2) + 4 * lh + (e & 3);
                 float v = total[i][j][e];
-                int orow = vrow;
                 if (a.pair_rows) {
                     if (e & 1) continue;
                     v = v + total[i][j][e + 1] * (1.0f / GEMM_LO_SCALE);
-                    orow = vrow >> 1;
                 }
-                if constexpr (GROUPED) orow = orow < a.m_out ? a.perm[orow] : -1;  // the token this sorted row is (-1: padding)
-                if (orow >= 0 && orow < a.m_out) {
-                    v *= a.rowfac[2 * orow + 1];  // undo the row's prescale (1 for a row binary16 carries as it is)
-                    float *p = sg.out + (long long)orow * sg.n + col;
+                if (orow[e] >= 0) {
+                    v *= ofac[e];  // undo the row's prescale (1 for a row binary16 carries as it is)
+                    float *p = sg.out + (long long)orow[e] * sg.n + col;
                     if (a.use_atomics) atomicAdd(p, v);
                     else __builtin_nontemporal_store(v, p);  // written once, read by another kernel: keep it out of the way of the operands
                 }
             }
         }
+    }
 }
 
 // ---- activation preparation -------------------------------------------------------------------------

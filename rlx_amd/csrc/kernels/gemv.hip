@@ -7,7 +7,7 @@
 // per-block scale is applied to the block result in f32 (acc += d * blk), so nothing is rounded to 16 bits
 // except the activations, and f32 activations are carried as an exact hi + lo pair of halfs in two A rows.
 //
-// Work decomposition and the LDS protocol are described above gemv_body().
+// Work decomposition and the LDS protocol are described above gemv_pass().
 #include <type_traits>
 
 #include "common.h"
@@ -64,18 +64,21 @@ struct GemvArgs {
 constexpr int XS_PAD_HALFS = 8;      // 16 bytes of padding per LDS row: rows land in different bank groups
 constexpr float LO_SCALE = 2048.0f;  // f32 activation x = hi + lo / LO_SCALE with hi, lo binary16
 
-// The last GEMV_LDS_TAIL bytes of a workgroup's LDS: [0,64) 1 / rms per activation row (RMSNorm prologue); then two
-// copies of GEMV_RANGE_AREA bytes, used by alternate K chunks (a wave that is still banking the sums of one chunk must
-// not see the next chunk's factors): [0,128) un-scale factor per virtual activation row (1 unless the row was
-// prescaled, below); [128,256) per logical row: bits of max |x| of the staged chunk, then reused for the forward
-// scale; [256,264) two row masks.
+// The last GEMV_LDS_TAIL bytes of a workgroup's LDS: [0,64) 1 / rms per activation row (RMSNorm prologue); then
+// GEMV_RANGE_AREA bytes: [0,128) un-scale factor per virtual activation row and [128,256) per logical row the bits of
+// max |x| of the staged chunk, then the forward scale (both only in the slow pass, below); [256,384) two row masks per
+// wave (up to 16 waves), written once by every wave at the end of the common pass.
 //
 // Activations travel as binary16. A row whose values leave the range binary16 carries well - some |x| >= 2^15, or no
 // |x| >= 2^-8 at all - is multiplied by a power of two that puts its largest value in [2^14, 2^15) while it is staged,
 // and the partial sums of that row are multiplied back when they are banked: exact, so the f32 range of the reference
-// (rlx-cpu/src/gguf_matmul.rs:65-94 computes in f32 throughout) is kept. The check is two compares per 16-byte group in
-// the staging loop; the rescaling itself runs only in workgroups that saw such a row.
-constexpr int GEMV_RANGE_AREA = 272, GEMV_LDS_TAIL = 640;
+// (rlx-cpu/src/gguf_matmul.rs:65-94 computes in f32 throughout) is kept. A kernel is two passes over the workgroup's
+// share of the launch. The common pass stages without scaling and only notes, two compares per 16-byte group, which rows
+// are outside that range; when the workgroup is done it looks at the notes (after the barrier it needs anyway, with
+// nothing left in registers) and writes its outputs if there is no such row. Otherwise it writes nothing and the slow
+// pass does the same work again with the rescaling in its staging. The rescaling code sits in a part of the kernel the
+// common pass never enters; inside the common pass's staging it cost every launch registers, scalar spills and 0.5 us.
+constexpr int GEMV_RANGE_AREA = 384, GEMV_LDS_TAIL = 448;
 constexpr float X_BIG = 32768.0f, X_SMALL = 0.00390625f;
 typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 
@@ -325,8 +328,16 @@ __device__ __forceinline__ void compute_unit(const UnitRegs<SCHEME> &w, const ha
 // Convert one K chunk of the activations into LDS as halfs: f32 -> hi rows [0,m) + lo rows [m,2m); 16-bit -> rows [0,m).
 // Each thread issues up to eight independent loads before it converts the first one, so a chunk of many rows costs
 // one memory latency per eight groups of columns, not one per group.
-// PASS 0: stage, and note in masks[0] / masks[1] the rows with some |x| >= X_BIG / some |x| >= X_SMALL; PASS 1: only find
+// PASS 0: stage, and add to masks[0] / masks[1] (the calling wave's own) the rows with some |x| >= X_BIG / some |x| >= X_SMALL; PASS 1: only find
 // the largest |x| of every row (rowmax, as bits); PASS 2: stage again with row r multiplied by fwd[r].
+// Every wave of the launch runs PASS 0 at the same moment, before there is other work to hide it behind, so its VALU
+// count is launch latency: the largest |x| of a 16-byte group is one v_max3_f32 per two values, and with a single activation
+// row a running maximum is the whole note.
+__device__ __forceinline__ float max3_abs(float acc, float x, float y) {  // max(acc, |x|, |y|); a NaN operand is skipped
+    float r;
+    asm("v_max3_f32 %0, %1, |%2|, |%3|" : "=v"(r) : "v"(acc), "v"(x), "v"(y));
+    return r;
+}
 template <int XD, bool NORM = false, int PASS = 0>
 __device__ __forceinline__ void stage_x_typed(const GemvArgs &a, const GemvSeg &sg, half_t *xs, int row_stride, int k0, int kc,
                                               const float *inv_rms = nullptr, uint32_t *masks = nullptr, uint32_t *rowmax = nullptr,
@@ -338,25 +349,53 @@ __device__ __forceinline__ void stage_x_typed(const GemvArgs &a, const GemvSeg &
     const int groups = kc / G;  // kc is a multiple of 64
     const int total = a.m * groups;
     uint32_t big = 0, seen = 0;
+    float vmax = 0.f;  // the largest |x| this thread has seen: all the note there is to take with one activation row
+    const bool one_row = a.m == 1;  // (a variant of this function compiled for one row takes the kernels past 128 registers)
+    // group index -> (row, group within the row) without an integer division (20 instructions, some of them quarter
+    // rate, eight times over, in front of loads that every wave of the launch is waiting for): idx < 2^24 is exact in
+    // f32, the quotient estimate is off by at most one and is put right by one compare each way.
+    const float inv_groups = 1.0f / (float)groups;
+    const int lo_rows = a.m * row_stride;  // halfs from a hi row to its lo row
+    auto split = [&](int idx, int &row, int &cg) {
+        if (one_row) {
+            row = 0;
+            cg = idx;
+            return;
+        }
+        row = (int)((float)idx * inv_groups);
+        cg = idx - (int)__umul24((unsigned)row, (unsigned)groups);
+        if (cg < 0) {
+            row--;
+            cg += groups;
+        } else if (cg >= groups) {
+            row++;
+            cg -= groups;
+        }
+    };
     for (int idx0 = tid; idx0 < total; idx0 += nt * U) {
         typedef typename std::conditional<XD == X_F32, float4_t, uint4_t>::type raw_t;  // 16 bytes either way
         raw_t raw[U];
 #pragma unroll
         for (int u = 0; u < U; u++) {
             const int idx = idx0 + u * nt;
-            const int row = idx / groups, c = (idx - row * groups) * G;
-            // k is a multiple of 32: a group is inside or outside as a whole
-            const bool inside = idx < total && k0 + c < sg.k;
-            const raw_t *src = (const raw_t *)((const uint8_t *)sg.x + ((long long)row * sg.k + k0 + c) * (XD == X_F32 ? 4 : 2));
             raw_t v = {};
-            if (inside) v = *src;
+            if (idx < total) {  // a wave with no lane left skips the arithmetic too
+                int row, cg;
+                split(idx, row, cg);
+                const int c = cg * G;
+                // k is a multiple of 32: a group is inside or outside as a whole
+                const long long at = one_row ? (long long)(k0 + c) : (long long)row * sg.k + k0 + c;
+                if (k0 + c < sg.k) v = *(const raw_t *)((const uint8_t *)sg.x + at * (XD == X_F32 ? 4 : 2));
+            }
             raw[u] = v;
         }
 #pragma unroll
         for (int u = 0; u < U; u++) {
             const int idx = idx0 + u * nt;
             if (idx >= total) continue;
-            const int row = idx / groups, c = (idx - row * groups) * G;
+            int row, cg;
+            split(idx, row, cg);
+            const int c = cg * G;
             float rowscale = 1.f;
             if constexpr (PASS == 2) rowscale = fwd[row];
             if constexpr (XD == X_F32) {
@@ -370,26 +409,35 @@ __device__ __forceinline__ void stage_x_typed(const GemvArgs &a, const GemvSeg &
                         if (a.beta) bt = *(const float4_t *)(a.beta + k0 + c);
                     }
                 }
-                float amax = 0.f;
+                float amax = 0.f, prev = 0.f;
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
                     float v = raw[u][e];
                     if constexpr (NORM) v = v * scale * gm[e] + bt[e];  // in_row[i] * inv_rms * gamma[i] + beta[i], unfused
-                    if constexpr (PASS != 2) amax = __builtin_fmaxf(amax, __builtin_fabsf(v));  // a NaN is skipped
+                    if constexpr (PASS == 0) {
+                        if (e & 1) amax = max3_abs(amax, prev, v);
+                        else prev = v;
+                    }
+                    if constexpr (PASS == 1) amax = __builtin_fmaxf(amax, __builtin_fabsf(v));  // a NaN is skipped
                     if constexpr (PASS == 2) v *= rowscale;
                     hi[e] = (half_t)v;
                     // residual, scaled by 2^11 so it stays in the normal binary16 range; undone in the final sum
                     lo[e] = (half_t)((v - (float)hi[e]) * LO_SCALE);
                 }
                 if constexpr (PASS == 0) {
-                    big |= (amax >= X_BIG ? 1u : 0u) << row;
-                    seen |= (amax >= X_SMALL ? 1u : 0u) << row;
+                    if (one_row) {
+                        vmax = __builtin_fmaxf(vmax, amax);
+                    } else {
+                        big |= (amax >= X_BIG ? 1u : 0u) << row;
+                        seen |= (amax >= X_SMALL ? 1u : 0u) << row;
+                    }
                 }
                 if constexpr (PASS == 1) {
                     atomicMax(rowmax + row, __builtin_bit_cast(uint32_t, amax));
                 } else {
-                    *(half4_t *)(xs + row * row_stride + c) = hi;
-                    *(half4_t *)(xs + (a.m + row) * row_stride + c) = lo;
+                    half_t *dst = xs + (one_row ? c : (int)__umul24((unsigned)row, (unsigned)row_stride) + c);
+                    *(half4_t *)dst = hi;
+                    *(half4_t *)(dst + lo_rows) = lo;
                 }
             } else if constexpr (XD == X_BF16) {
                 half8_t h;
@@ -398,88 +446,99 @@ __device__ __forceinline__ void stage_x_typed(const GemvArgs &a, const GemvSeg &
                 for (int e = 0; e < 8; e++) {
                     const uint32_t bits = ((e & 1) ? (raw[u][e >> 1] >> 16) : (raw[u][e >> 1] & 0xFFFFu)) << 16;
                     float v = __builtin_bit_cast(float, bits);
-                    if constexpr (PASS != 2) amax = __builtin_fmaxf(amax, __builtin_fabsf(v));
+                    if constexpr (PASS == 1) amax = __builtin_fmaxf(amax, __builtin_fabsf(v));
                     if constexpr (PASS == 2) v *= rowscale;
                     h[e] = (half_t)v;
                 }
                 if constexpr (PASS == 0) {
-                    big |= (amax >= X_BIG ? 1u : 0u) << row;
-                    seen |= (amax >= X_SMALL ? 1u : 0u) << row;
+                    // a dword read as f32 is its upper bf16 value with up to 2^-8 added in magnitude: close enough for the thresholds
+#pragma unroll
+                    for (int d = 0; d < 4; d++)
+                        amax = max3_abs(amax, __builtin_bit_cast(float, raw[u][d]), __builtin_bit_cast(float, raw[u][d] << 16));
+                    if (one_row) {
+                        vmax = __builtin_fmaxf(vmax, amax);
+                    } else {
+                        big |= (amax >= X_BIG ? 1u : 0u) << row;
+                        seen |= (amax >= X_SMALL ? 1u : 0u) << row;
+                    }
                 }
                 if constexpr (PASS == 1) atomicMax(rowmax + row, __builtin_bit_cast(uint32_t, amax));
-                else *(half8_t *)(xs + row * row_stride + c) = h;
+                else *(half8_t *)(xs + (one_row ? c : (int)__umul24((unsigned)row, (unsigned)row_stride) + c)) = h;
             } else {  // binary16 activations are staged as they are: nothing to gain from a scale
-                *(uint4_t *)(xs + row * row_stride + c) = raw[u];
+                *(uint4_t *)(xs + (one_row ? c : (int)__umul24((unsigned)row, (unsigned)row_stride) + c)) = raw[u];
             }
         }
     }
-    if constexpr (PASS == 0 && XD != X_F16) {  // one LDS atomic per wave and mask, and only for masks that have a bit
-#pragma unroll
-        for (int off = 32; off > 0; off >>= 1) {
-            big |= __shfl_xor(big, off);
-            seen |= __shfl_xor(seen, off);
-        }
-        if ((threadIdx.x & 63) == 0) {
-            if (big) atomicOr(masks, big);
-            if (seen) atomicOr(masks + 1, seen);
+    if constexpr (PASS == 0 && XD != X_F16) {  // into the wave's two masks (wave-uniform: a vote per row is two scalar operations)
+        if (one_row) {
+            masks[0] |= __ballot(vmax >= X_BIG) != 0 ? 1u : 0u;
+            masks[1] |= __ballot(vmax >= X_SMALL) != 0 ? 1u : 0u;
+        } else {
+            for (int r = 0; r < a.m; r++) {
+                masks[0] |= (__ballot((big >> r) & 1u) != 0 ? 1u : 0u) << r;
+                masks[1] |= (__ballot((seen >> r) & 1u) != 0 ? 1u : 0u) << r;
+            }
         }
     }
 }
 
-// Stage one K chunk of a segment's activations (two barriers), rescaling rows that binary16 would not carry (three
-// more passes, taken by the whole workgroup or not at all). tail = the workgroup's GEMV_LDS_TAIL bytes. On return
-// rsv[v] holds the factor the partial sums of virtual row v must be multiplied by.
-template <int XD, bool NORM>
-__device__ __forceinline__ void stage_chunk_typed(const GemvArgs &a, const GemvSeg &sg, half_t *xs, int row_stride, int k0, int kc,
-                                                  uint8_t *tail, int parity) {
+// Common pass: stage one K chunk of a segment's activations (one barrier), noting rows outside the binary16 range in wm.
+template <bool NORM>
+__device__ __forceinline__ void stage_chunk(const GemvArgs &a, const GemvSeg &sg, half_t *xs, int row_stride, int k0, int kc, uint8_t *tail,
+                                            uint32_t *wm) {
     const float *inv_rms = (const float *)tail;
-    uint8_t *area = tail + 64 + parity * GEMV_RANGE_AREA;
-    float *rsv = (float *)area;
-    uint32_t *rowmax = (uint32_t *)(area + 128);
-    uint32_t *masks = (uint32_t *)(area + 256);
-    const int tid = threadIdx.x;
-    if (tid < 32) rsv[tid] = 1.f;
-    if (tid < 2) masks[tid] = 0;
-    __syncthreads();  // also: the previous chunk is fully consumed
-    stage_x_typed<XD, NORM, 0>(a, sg, xs, row_stride, k0, kc, inv_rms, masks);
-    __syncthreads();
-    if constexpr (XD != X_F16) {
-        const uint32_t rows = a.m >= 32 ? 0xFFFFFFFFu : ((1u << a.m) - 1u);
-        const uint32_t need = (masks[0] | ~masks[1]) & rows;  // workgroup-uniform: read after the barrier
-        if (need) {
-            if (tid < 32) rowmax[tid] = 0;
-            __syncthreads();
-            stage_x_typed<XD, NORM, 1>(a, sg, xs, row_stride, k0, kc, inv_rms, nullptr, rowmax);
-            __syncthreads();
-            if (tid < a.m) {
-                const uint32_t mb = rowmax[tid];
-                float fwd = 1.f, back = 1.f;
-                if (((need >> tid) & 1u) && mb != 0 && mb < 0x7F800000u) {  // a zero row or one with an infinity stays as it is
-                    int e = (int)(mb >> 23) - 127;
-                    e = e < -100 ? -100 : e;
-                    fwd = __builtin_bit_cast(float, (uint32_t)(14 - e + 127) << 23);   // 2^(14 - e): largest value into [2^14, 2^15)
-                    back = __builtin_bit_cast(float, (uint32_t)(e - 14 + 127) << 23);
-                }
-                rsv[tid] = back;
-                if (XD == X_F32) rsv[a.m + tid] = back;
-                ((float *)rowmax)[tid] = fwd;
-            }
-            __syncthreads();
-            stage_x_typed<XD, NORM, 2>(a, sg, xs, row_stride, k0, kc, inv_rms, nullptr, nullptr, (const float *)rowmax);
-            __syncthreads();
-        }
+    if constexpr (NORM) {
+        stage_x_typed<X_F32, true, 0>(a, sg, xs, row_stride, k0, kc, inv_rms, wm);
+    } else {
+        if (a.x_dtype == X_F32) stage_x_typed<X_F32, false, 0>(a, sg, xs, row_stride, k0, kc, inv_rms, wm);
+        else if (a.x_dtype == X_BF16) stage_x_typed<X_BF16, false, 0>(a, sg, xs, row_stride, k0, kc, inv_rms, wm);
+        else stage_x_typed<X_F16, false, 0>(a, sg, xs, row_stride, k0, kc, inv_rms, wm);
     }
+    __syncthreads();
+}
+
+// Slow pass: find every row's largest |x| in the chunk, stage the chunk with the rows that need it multiplied by a power
+// of two, and leave in rsv[v] the factor the partial sums of virtual row v must be multiplied by (four barriers).
+template <int XD, bool NORM>
+__device__ __forceinline__ void stage_chunk_rescaled(const GemvArgs &a, const GemvSeg &sg, half_t *xs, int row_stride, int k0, int kc,
+                                                     uint8_t *tail) {
+    const float *inv_rms = (const float *)tail;
+    float *rsv = (float *)(tail + 64);
+    uint32_t *rowmax = (uint32_t *)(tail + 64 + 128);
+    const int tid = threadIdx.x;
+    if (tid < 32) {
+        rowmax[tid] = 0;
+        rsv[tid] = 1.f;
+    }
+    __syncthreads();
+    stage_x_typed<XD, NORM, 1>(a, sg, xs, row_stride, k0, kc, inv_rms, nullptr, rowmax);
+    __syncthreads();
+    if (tid < a.m) {
+        const uint32_t mb = rowmax[tid];
+        const float amax = __builtin_bit_cast(float, mb);
+        float fwd = 1.f, back = 1.f;
+        if (mb != 0 && mb < 0x7F800000u && (amax >= X_BIG || amax < X_SMALL)) {  // a zero row or one with an infinity stays as it is
+            int e = (int)(mb >> 23) - 127;
+            e = e < -100 ? -100 : e;
+            fwd = __builtin_bit_cast(float, (uint32_t)(14 - e + 127) << 23);   // 2^(14 - e): largest value into [2^14, 2^15)
+            back = __builtin_bit_cast(float, (uint32_t)(e - 14 + 127) << 23);
+        }
+        rsv[tid] = back;
+        if (XD == X_F32) rsv[a.m + tid] = back;
+        ((float *)rowmax)[tid] = fwd;
+    }
+    __syncthreads();
+    stage_x_typed<XD, NORM, 2>(a, sg, xs, row_stride, k0, kc, inv_rms, nullptr, nullptr, (const float *)rowmax);
+    __syncthreads();
 }
 
 template <bool NORM>
-__device__ __forceinline__ void stage_chunk(const GemvArgs &a, const GemvSeg &sg, half_t *xs, int row_stride, int k0, int kc, uint8_t *tail,
-                                            int parity) {
+__device__ __forceinline__ void stage_chunk_slow(const GemvArgs &a, const GemvSeg &sg, half_t *xs, int row_stride, int k0, int kc, uint8_t *tail) {
     if constexpr (NORM) {
-        stage_chunk_typed<X_F32, true>(a, sg, xs, row_stride, k0, kc, tail, parity);
-    } else {
-        if (a.x_dtype == X_F32) stage_chunk_typed<X_F32, false>(a, sg, xs, row_stride, k0, kc, tail, parity);
-        else if (a.x_dtype == X_BF16) stage_chunk_typed<X_BF16, false>(a, sg, xs, row_stride, k0, kc, tail, parity);
-        else stage_chunk_typed<X_F16, false>(a, sg, xs, row_stride, k0, kc, tail, parity);
+        stage_chunk_rescaled<X_F32, true>(a, sg, xs, row_stride, k0, kc, tail);
+    } else {  // binary16 activations never get here: the common pass notes nothing for them
+        if (a.x_dtype == X_F32) stage_chunk_rescaled<X_F32, false>(a, sg, xs, row_stride, k0, kc, tail);
+        else stage_chunk_rescaled<X_BF16, false>(a, sg, xs, row_stride, k0, kc, tail);
     }
 }
 
@@ -532,8 +591,9 @@ extern "C" __global__ __launch_bounds__(256) void rlx_argmax_finish(const unsign
 // writes the SwiGLU of the two sums.
 enum { GEMV_PLAIN = 0, GEMV_ARGMAX = 1, GEMV_PAIRED = 2, GEMV_NORM = 4 };  // GEMV_NORM combines with the others
 
-template <int SCHEME, int NREG, int DEPTH, int MODE, int UPI = 1, int RG = 1>
-__device__ __forceinline__ void gemv_body(const GemvArgs &a) {
+// SLOW = false: the common pass; returns true, with nothing written, when some activation row needs the slow pass.
+template <int SCHEME, int NREG, int DEPTH, int MODE, int UPI, int RG, bool SLOW>
+__device__ __forceinline__ bool gemv_pass(const GemvArgs &a) {
     constexpr Layout L = layout_of(SCHEME);
     constexpr int BLK_PER_UNIT = L.unit_k / 32;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -614,10 +674,16 @@ __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
     const uint8_t *wbase2 = paired ? seg.w_pair + (long long)tile0 * seg.units * L.unit_bytes : wbase;
     auto vtile_ptr = [&](int vt) { return paired ? ((vt & 1) ? wbase2 : wbase) + (vt >> 1) * tile_bytes : wbase + vt * tile_bytes; };
 
-    int parity = 0;
-    for (int u0 = 0; u0 < seg.units; u0 += kc_units, parity ^= 1) {
+    const float *rsv = (const float *)(tail + 64);
+    uint32_t wm[2] = {0, a.x_dtype == X_F16 ? 0xFFFFFFFFu : 0u};  // this wave's notes: rows with a big value, rows with a value that is not tiny
+    uint32_t *notes = (uint32_t *)(tail + 64 + 256);               // the workgroup's: the waves' notes OR-ed together
+    if constexpr (!SLOW) {
+        if (tid == 0) notes[0] = notes[1] = 0;
+    }
+    for (int u0 = 0; u0 < seg.units; u0 += kc_units) {
         const int nu = min(kc_units, seg.units - u0);  // units in this chunk
-        const float *rsv = (const float *)(tail + 64 + parity * GEMV_RANGE_AREA);
+        if (u0 > 0) __syncthreads();  // every wave is done with the previous chunk: its activations, its factors
+        if constexpr (SLOW) stage_chunk_slow<(MODE & GEMV_NORM) != 0>(a, seg, xs, row_stride, u0 * L.unit_k, nu * L.unit_k, tail);
         // This wave's items: for each tile, units wave, wave + nwaves, ... < nu. Two cursors walk them: `pf_*` issues
         // loads DEPTH items ahead into a register ring, `cu_*` consumes.
         // An item is UPI consecutive units (the host picks UPI > 1 only when every chunk holds a multiple of UPI).
@@ -652,7 +718,13 @@ __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
             for (int p = 0; p < UPI; p++) ring[d].u[p].clear();
             prefetch(ring[d]);
         }
-        stage_chunk<(MODE & GEMV_NORM) != 0>(a, seg, xs, row_stride, u0 * L.unit_k, nu * L.unit_k, tail, parity);
+        if constexpr (!SLOW) {
+            stage_chunk<(MODE & GEMV_NORM) != 0>(a, seg, xs, row_stride, u0 * L.unit_k, nu * L.unit_k, tail, wm);
+            if (l == 0) {  // behind the barrier that also ordered the clearing of the notes; nothing waits for these
+                if (wm[0]) atomicOr(notes, wm[0]);
+                atomicOr(notes + 1, wm[1]);
+            }
+        }
         if constexpr (SCHEME == SCHEME_Q4K || SCHEME == SCHEME_Q5K) {
             const int nblk = nu * BLK_PER_UNIT;
             // rows >= rv of the [blk][16 RG] table are never read: compute_unit only uses the rows its lane group owns
@@ -695,10 +767,11 @@ __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
                         for (int rg = 0; rg < RG; rg++) {
                             if (4 * rg + g < ng) {  // this lane's four rows of the group exist
                                 float *slot = part + ((size_t)cu_t * kw + kl) * slot_floats + (4 * rg + g) * 64 + nrow;
-                                const float4_t back = *(const float4_t *)(rsv + 16 * rg + 4 * g);  // 1 unless the row was prescaled
+                                float4_t back = {1.f, 1.f, 1.f, 1.f};
+                                if constexpr (SLOW) back = *(const float4_t *)(rsv + 16 * rg + 4 * g);  // 1 unless the row was prescaled
 #pragma unroll
                                 for (int r = 0; r < 4; r++) {
-                                    if (r < NREG) slot[r * 16] += acc[rg][r] * back[r];
+                                    if (r < NREG) slot[r * 16] += SLOW ? acc[rg][r] * back[r] : acc[rg][r];
                                     acc[rg][r] = 0.f;
                                 }
                             }
@@ -712,6 +785,11 @@ __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
     }
 
     __syncthreads();
+    if constexpr (!SLOW) {  // did any wave note a row that binary16 does not carry? (one broadcast read, the same answer in every wave)
+        const uint2_t mk = *(const uint2_t *)notes;
+        const uint32_t rows = a.m >= 32 ? 0xFFFFFFFFu : ((1u << a.m) - 1u);
+        if (__builtin_amdgcn_readfirstlane((int)((mk[0] | ~mk[1]) & rows)) != 0) return true;
+    }
     // out[mr][tile*16 + col] = sum over waves of row mr (+ 2^-11 * row m+mr for f32 activations)
     unsigned long long best = 0;  // below every key a real value produces
     for (int idx = tid; idx < ntiles * a.m * 16; idx += blockDim.x) {
@@ -759,6 +837,7 @@ __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
             a.argmax_key[blockIdx.x] = best;
         }
     }
+    return false;
 }
 
 }  // namespace rlx
@@ -766,7 +845,10 @@ __device__ __forceinline__ void gemv_body(const GemvArgs &a) {
 #define RLX_GEMV_INST(name, SCHEME, NREG, DEPTH, MODE, UPI) RLX_GEMV_INST_RG(name, SCHEME, NREG, DEPTH, MODE, UPI, 1, 1024)
 #define RLX_GEMV_INST_RG(name, SCHEME, NREG, DEPTH, MODE, UPI, RG, THREADS)                                 \
     extern "C" __global__ __launch_bounds__(THREADS) void name(rlx::GemvArgs a) {                            \
-        rlx::gemv_body<SCHEME, NREG, DEPTH, MODE, UPI, RG>(a);                                                \
+        if (rlx::gemv_pass<SCHEME, NREG, DEPTH, MODE, UPI, RG, false>(a)) {                                  \
+            __syncthreads();                                                                                  \
+            rlx::gemv_pass<SCHEME, NREG, DEPTH, MODE, UPI, RG, true>(a);                                      \
+        }                                                                                                     \
     }
 // NREG = 2: at most two virtual rows (m = 1 f32, or m <= 2 16-bit); NREG = 4 otherwise.
 #define RLX_GEMV_SCHEME(tag, SCHEME, DEPTH, UPI)                                                      \
