@@ -543,25 +543,39 @@ __device__ __forceinline__ void xrowscale_body(const XPrepArgs &a) {
     const int lane = threadIdx.x & 63;
     const long long row = (long long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     if (row >= a.m) return;
+    // Eight 16-byte loads per lane are issued before the first is looked at: a row costs one memory latency per 8 KB, not
+    // one per KB (the kernel is a launch of its own in front of every prefill matmul, and nothing but latency).
     float amax = 0.f;
-    if (a.x_dtype == 0) {
-        const float4_t *p = (const float4_t *)((const float *)a.x + row * a.k);
-        for (int c = lane; c < a.k / 4; c += 64) {
-            const float4_t v = p[c];
+    auto scan = [&](auto as_f32) {  // as_f32(word, amax) folds the values of one 32-bit word into the maximum
+        const int esz = decltype(as_f32)::esz;
+        const int chunks = a.k * esz / 16;  // 16-byte chunks of the row (k is a multiple of 32)
+        const uint4_t *p = (const uint4_t *)((const uint8_t *)a.x + row * a.k * esz);
+        for (int c0 = lane; c0 < chunks; c0 += 64 * 8) {
+            uint4_t raw[8];
 #pragma unroll
-            for (int e = 0; e < 4; e++) amax = __builtin_fmaxf(amax, __builtin_fabsf(v[e]));  // a NaN is skipped
-        }
-    } else if (a.x_dtype == 1) {
-        const uint4_t *p = (const uint4_t *)((const uint16_t *)a.x + row * a.k);
-        for (int c = lane; c < a.k / 8; c += 64) {
-            const uint4_t raw = p[c];
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
-                amax = __builtin_fmaxf(amax, __builtin_fabsf(__builtin_bit_cast(float, raw[e] << 16)));
-                amax = __builtin_fmaxf(amax, __builtin_fabsf(__builtin_bit_cast(float, raw[e] & 0xFFFF0000u)));
+            for (int u = 0; u < 8; u++) {
+                raw[u] = uint4_t{0, 0, 0, 0};
+                if (c0 + 64 * u < chunks) raw[u] = p[c0 + 64 * u];
             }
+#pragma unroll
+            for (int u = 0; u < 8; u++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) amax = as_f32(raw[u][e], amax);
         }
-    }
+    };
+    struct F32Word {
+        enum { esz = 4 };
+        __device__ float operator()(uint32_t w, float m) const { return __builtin_fmaxf(m, __builtin_fabsf(__builtin_bit_cast(float, w))); }  // a NaN is skipped
+    };
+    struct Bf16Word {
+        enum { esz = 2 };
+        __device__ float operator()(uint32_t w, float m) const {
+            m = __builtin_fmaxf(m, __builtin_fabsf(__builtin_bit_cast(float, w << 16)));
+            return __builtin_fmaxf(m, __builtin_fabsf(__builtin_bit_cast(float, w & 0xFFFF0000u)));
+        }
+    };
+    if (a.x_dtype == 0) scan(F32Word{});
+    else if (a.x_dtype == 1) scan(Bf16Word{});  // binary16 rows are not looked at: they are carried as they are
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) amax = __builtin_fmaxf(amax, __shfl_xor(amax, off));
     if (lane == 0) {
