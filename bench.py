@@ -1,13 +1,22 @@
 #!/usr/bin/env python3
-"""Headline benchmark: Q4_0 decode GEMV (batch 1) over the seven Llama-3-8B layer projections on one MI355X.
+"""Headline benchmark: Q4_0 decode GEMV (batch 1) over the seven Llama-3-8B layer projections on one MI355X, with the
+second half of the metric (Q4_K prefill GEMM, M = 512) beside it.
 
 A step is one pass over one layer's seven projections (q, k, v, o, gate, up, down): seven DequantMatMul nodes of one
-compiled graph, each with its own f32 activation vector as the benchmark definition states, which the backend issues as one
-batched launch replayed as a hipGraph (`--wiring layer` orders them like a transformer layer instead: four dependent
-launches). The layers rotate through LAYERS distinct weight sets (~123 MB each), far
-more than the 256 MB of last-level cache, so every launch streams its weights from HBM. Inputs and weights are
-resident in HBM before the timed region. One JSON line is printed; `value` is algorithmic bytes per second
-(packed weights + f32 activations in + f32 outputs out), the figure the roofline fraction is taken from.
+compiled graph, each with its own f32 activation vector as the benchmark definition states, which the backend issues as
+one batched launch. The layers rotate through LAYERS distinct weight sets (~123 MB each), far more than the 256 MB of
+last-level cache, so every launch streams its weights from HBM. Inputs and weights are resident in HBM before the timed
+region, which is bracketed by HIP events on the launch stream after SETTLE_LAUNCHES untimed launches (the clocks of a
+fresh process take a few hundred launches to settle; a 20-step run then reads like a 2000-step one). One JSON line is
+printed; `value` is algorithmic bytes per second (packed weights + f32 activations in + f32 outputs out), the figure
+`roofline.frac` is taken from. Beside it in the same line:
+  config.wiring_layer_ms            the same layer in dependency order (x -> q,k,v; q -> o; o -> gate,up; gate -> down):
+                                    four dependent launches, what a decode loop gets;
+  config.host_boundary_ms_per_call  the layer through rlx_exec_run with host buffers (PCIe and call overhead included);
+  roofline.secondary                rlx_gemm_q4_k at M = 512 on 4096 -> 14336 (bf16 activations): the kernel's launches
+                                    alone between two events, the whole rlx_mi355x_gguf_matmul_bt call, the down
+                                    projection and the gate + up pair;
+  cpu_baseline[.secondary]          the oracle's C restatement of the reference's scalar CPU path on a bounded sample.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--no-cpu] [--extra]
 """
@@ -28,8 +37,9 @@ HBM_PEAK_GBS = 8000.0       # MI355X published HBM3E bandwidth
 MFMA_F16_PEAK_TFLOPS = 2500.0  # dense f16/bf16 MFMA peak
 CALIBRATION_COPY_BYTES = 256 << 20
 # HBM bytes per launch of the headline kernel (FETCH_SIZE + WRITE_SIZE of two rocprofv3 --pmc runs of this command,
-# each scaled by the same counter's reading for the copy kernel above); profiles/gemv_q4_0_llama8b_layer_traffic.txt.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 124295417
+# each scaled by the same counter's reading for the copy kernel above, the 478-workgroup dispatches of the kernel only);
+# profiles/gemv_q4_0_layer_and_gemm_q4_k_m512_traffic.txt.
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 124376267
 
 # (name, N, K) — the Llama-3-8B layer projections of the headline workload
 LLAMA8B = [("q", 4096, 4096), ("k", 1024, 4096), ("v", 1024, 4096), ("o", 4096, 4096),
@@ -40,7 +50,7 @@ LLAMA8B = [("q", 4096, 4096), ("k", 1024, 4096), ("v", 1024, 4096), ("o", 4096, 
 # the benchmark definition states it: seven GEMVs, each with its own seeded f32 activation vector; nothing orders them, so the backend
 # issues all seven as one batched launch. "layer" chains them the way a transformer layer's data flow does
 # (x -> q,k,v; q -> o; o -> gate,up; gate -> down; the attention / activation math in between is not part of this
-# path), which forces four dependent launches; it is reported under "extra" for comparison.
+# path), which forces four dependent launches; it is reported as config.wiring_layer_ms.
 WIRING = {
     "independent": {n: f"x_{n}" for n in ("q", "k", "v", "o", "gate", "up", "down")},
     "layer": {"q": "x_attn", "k": "x_attn", "v": "x_attn", "o": "@q", "gate": "@o", "up": "@o", "down": "@gate"},
