@@ -375,18 +375,23 @@ def extra_configs(rlx_amd, stream):
                                   "frac_hbm": round(b / ms / 1e6 / HBM_PEAK_GBS, 4)}
     for q in qws:
         q.free()
-    # the other K-quants on a gate/up projection [14336, 4096]: Q6_K and Q5_K have packed kernels (48 / 40 MB per copy); Q8_K
-    # stands for the schemes decoded at upload and resident as binary16 (117 MB per copy). Copies rotated: nothing cache-resident.
+    # the other K-quants on a gate/up projection [14336, 4096]: Q6_K, Q5_K and Q8_K have packed kernels (48 / 40 / 61 MB per
+    # copy); Q2_K stands for the schemes decoded at upload and resident as binary16 (117 MB per copy). Copies rotated: nothing
+    # cache-resident.
     n, k = 14336, 4096
     rng = np.random.default_rng(5)
     for tag, scheme, bb, d_off, copies in (("q6_k_gemv_gate/up", QuantScheme.GgufQ6K, 210, 208, 13),
                                             ("q5_k_gemv_gate/up", QuantScheme.GgufQ5K, 176, 0, 15),
-                                            ("q8_k_gemv_gate/up_resident_f16", QuantScheme.GgufQ8K, 292, 0, 5)):
+                                            ("q8_k_gemv_gate/up", QuantScheme.GgufQ8K, 292, 0, 10),
+                                            ("q2_k_gemv_gate/up_resident_f16", QuantScheme.GgufQ2K, 84, 0, 5)):
         blocks = rng.integers(0, 256, (n * k // 256, bb), dtype=np.uint8)
         if scheme == QuantScheme.GgufQ8K:
             blocks[:, 0:4] = np.full(n * k // 256, 2e-4, np.float32).view(np.uint8).reshape(-1, 4)
         else:  # weights of a few hundredths
-            blocks[:, d_off:d_off + 2] = np.full(n * k // 256, 5e-6 if scheme == QuantScheme.GgufQ6K else 4e-5, np.float16).view(np.uint8).reshape(-1, 2)
+            d16 = 5e-6 if scheme == QuantScheme.GgufQ6K else 5e-4 if scheme == QuantScheme.GgufQ2K else 4e-5
+            blocks[:, d_off:d_off + 2] = np.full(n * k // 256, d16, np.float16).view(np.uint8).reshape(-1, 2)
+        if scheme == QuantScheme.GgufQ2K:
+            blocks[:, 2:4] = np.full(n * k // 256, 1e-4, np.float16).view(np.uint8).reshape(-1, 2)
         if scheme == QuantScheme.GgufQ5K:
             blocks[:, 2:4] = np.full(n * k // 256, 2e-5, np.float16).view(np.uint8).reshape(-1, 2)
         qws = [ops.QWeight(scheme, blocks.reshape(-1), n, k) for _ in range(copies)]

@@ -47,16 +47,16 @@ typedef enum rlx_dtype {
 
 /* rlx_ir::quant::QuantScheme, declaration order (rlx-ir/src/quant.rs:39-79). The eight GGUF schemes the reference's
  * gguf_matmul_bt dispatches (rlx-cpu/src/gguf_matmul.rs:25-37) are claimed; any other value is RLX_ERR_UNSUPPORTED.
- * Q4_K, Q5_K, Q6_K, Q4_0 and Q8_0 stay packed in HBM (same byte count as the GGUF blocks) and have a bit-exact device
- * decoder. Q6_K scale bytes are read as the reference's block decoder reads them, unsigned (rlx-gguf/src/lib.rs:819-845),
+ * Q4_K, Q5_K, Q6_K, Q8_K, Q4_0 and Q8_0 stay packed in HBM (the byte count of the GGUF blocks; Q8_K without its 32 bytes
+ * of block sums per super-block, which no decoder reads) and have a bit-exact device decoder. Q6_K scale bytes are read as the reference's block decoder reads them, unsigned (rlx-gguf/src/lib.rs:819-845),
  * unless the weight is created with RLX_QW_Q6K_SIGNED_SCALES (below).
- * The other three ("wide") are decoded once at upload with the reference's block decoder and kept as binary16 (2 bytes per weight):
+ * The other two ("wide") are decoded once at upload with the reference's block decoder and kept as binary16 (2 bytes per weight):
  * matmuls only, every decoded weight must fit binary16. */
 typedef enum rlx_quant_scheme {
     RLX_SCHEME_GGUF_Q4K = 5,  /* 256 elems / 144 bytes */
     RLX_SCHEME_GGUF_Q5K = 6,  /* 256 / 176 */
     RLX_SCHEME_GGUF_Q6K = 7,  /* 256 / 210 */
-    RLX_SCHEME_GGUF_Q8K = 8,  /* 256 / 292, wide */
+    RLX_SCHEME_GGUF_Q8K = 8,  /* 256 / 292 */
     RLX_SCHEME_GGUF_Q2K = 9,  /* 256 / 84, wide (field order of rlx-gguf/src/lib.rs:857-886) */
     RLX_SCHEME_GGUF_Q3K = 10, /* 256 / 110, wide (field order of rlx-gguf/src/lib.rs:889-930) */
     RLX_SCHEME_GGUF_Q4_0 = 11, /* 32 elems / 18 bytes  */

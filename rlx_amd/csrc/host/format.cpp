@@ -53,13 +53,6 @@ static inline float f16_bits_to_f32(uint16_t h) {
 
 static inline float f16_at(const uint8_t *p) { return f16_bits_to_f32((uint16_t)(p[0] | (p[1] << 8))); }
 
-// Q8_K (lib.rs:848-854): f32 d, 256 signed bytes (the 16 block sums that follow are not read).
-static void decode_q8_k(const uint8_t *b, float *out) {
-    float d;
-    memcpy(&d, b, 4);
-    for (int i = 0; i < 256; i++) out[i] = d * (float)(int8_t)b[4 + i];
-}
-
 // Q2_K in the reference's field order (lib.rs:857-886): d, min, 16 scale bytes (low nibble scale, high nibble min),
 // 64 bytes of 2-bit codes.
 static void decode_q2_k(const uint8_t *b, float *out) {
@@ -96,7 +89,6 @@ Layout host_layout(int scheme) { return layout_of(scheme); }
 
 static void decode_wide_block(int scheme, const uint8_t *b, float *out) {
     switch (scheme) {
-    case SCHEME_Q8K: decode_q8_k(b, out); break;
     case SCHEME_Q2K: decode_q2_k(b, out); break;
     default: decode_q3_k(b, out); break;
     }
@@ -186,6 +178,17 @@ int repack_host(int scheme, uint32_t flags, const uint8_t *src, size_t nbytes, i
                             uint8_t *dst = unit + (t >> 1) * 1024 + l * 16 + (t & 1) * 8;
                             for (int e = 0; e < 8; e++) dst[e] = live ? (uint8_t)(b[2 + 8 * g + e] ^ 0x80u) : 0x80u;
                         }
+                    }
+                } else if (scheme == SCHEME_Q8K) {  // one super-block per unit: eight blocks of offset-binary bytes, f32 d
+                    const bool live = r < n && u < bpr;
+                    const uint8_t *b = live ? src + (r * bpr + u) * L.block_bytes : nullptr;
+                    if (g == 0) {
+                        if (live) memcpy(unit + 4096 + nrow * 4, b, 4);
+                        else memset(unit + 4096 + nrow * 4, 0, 4);
+                    }
+                    for (int j = 0; j < 8; j++) {
+                        uint8_t *dst = unit + (j >> 1) * 1024 + l * 16 + (j & 1) * 8;
+                        for (int e = 0; e < 8; e++) dst[e] = live ? (uint8_t)(b[4 + 32 * j + 8 * g + e] ^ 0x80u) : 0x80u;
                     }
                 } else if (scheme == SCHEME_Q5K) {  // one super-block per unit: nibbles as Q4_K, fifth-bit words, 16 meta bytes
                     const bool live = r < n && u < bpr;

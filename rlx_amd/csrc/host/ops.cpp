@@ -153,7 +153,8 @@ static int launch_gemv(const void *const *xs, int xk, const rlx_qweight *const *
     }
     // kernel = scheme family x {r2, r4, r2_argmax, r2_paired, r4_paired}
     const int family = wide ? K_GEMV_F16W_R2 : scheme == SCHEME_Q4_0 ? K_GEMV_Q4_0_R2 : scheme == SCHEME_Q8_0 ? K_GEMV_Q8_0_R2
-                       : scheme == SCHEME_Q6K ? K_GEMV_Q6_K_R2 : scheme == SCHEME_Q5K ? K_GEMV_Q5_K_R2 : K_GEMV_Q4_K_R2;
+                       : scheme == SCHEME_Q6K ? K_GEMV_Q6_K_R2 : scheme == SCHEME_Q5K ? K_GEMV_Q5_K_R2
+                       : scheme == SCHEME_Q8K ? K_GEMV_Q8_K_R2 : K_GEMV_Q4_K_R2;
     if (argmax_key && !r2) {
         set_error("gemv: the argmax epilogue takes one activation row");
         return RLX_ERR_INVALID;
@@ -410,6 +411,7 @@ static int launch_gemm(const void *x, int xk, const rlx_qweight *const *ws, floa
                   : layout_is_f16w(L)           ? (skinny ? K_GEMM64_F16W : K_GEMM_F16W)
                   : w->scheme == SCHEME_Q6K     ? (skinny ? K_GEMM64_Q6_K : K_GEMM_Q6_K)
                   : w->scheme == SCHEME_Q5K     ? (skinny ? K_GEMM64_Q5_K : K_GEMM_Q5_K)
+                  : w->scheme == SCHEME_Q8K     ? (skinny ? K_GEMM64_Q8_K : K_GEMM_Q8_K)
                                                 : (skinny ? K_GEMM64_Q8_0 : K_GEMM_Q8_0);
     RLX_TRY(runtime_init());
     RLX_TRY(launch3(id, (unsigned)gx, (unsigned)gy, (unsigned)split, 512, skinny ? 3 * 24 * 1024 : 3 * 48 * 1024, stream, params));
@@ -532,7 +534,8 @@ int rlx_mi355x_dequant(const rlx_qweight *w, float *out_dev, void *stream) {
     DequantArgs a{w->dev, out_dev, w->dims.n, w->dims.k, w->dims.units, w->sc_off()};
     void *params[] = {&a};
     KernelId id = w->scheme == SCHEME_Q4_0 ? K_DEQUANT_Q4_0 : w->scheme == SCHEME_Q8_0 ? K_DEQUANT_Q8_0
-                  : w->scheme == SCHEME_Q6K ? K_DEQUANT_Q6_K : w->scheme == SCHEME_Q5K ? K_DEQUANT_Q5_K : K_DEQUANT_Q4_K;
+                  : w->scheme == SCHEME_Q6K ? K_DEQUANT_Q6_K : w->scheme == SCHEME_Q5K ? K_DEQUANT_Q5_K
+                  : w->scheme == SCHEME_Q8K ? K_DEQUANT_Q8_K : K_DEQUANT_Q4_K;
     return launch(id, (unsigned)w->dims.units, (unsigned)w->dims.row_tiles, 64, 0, (hipStream_t)stream, params);
 }
 
@@ -1044,6 +1047,7 @@ int rlx_mi355x_gguf_grouped_matmul_bt_ws(const void *x_dev, int x_dtype, const r
                         : layout_is_f16w(L)        ? K_GEMM64G_F16W
                         : w->scheme == SCHEME_Q6K  ? K_GEMM64G_Q6_K
                         : w->scheme == SCHEME_Q5K  ? K_GEMM64G_Q5_K
+                        : w->scheme == SCHEME_Q8K  ? K_GEMM64G_Q8_K
                                                    : K_GEMM64G_Q8_0;
     const unsigned gx = (unsigned)((w->dims.row_tiles * 16 + 127) / 128), gy = (unsigned)(p.perm_len / p.group);
     return launch3(id, gx, gy, 1, 512, 3 * 24 * 1024, s, params);

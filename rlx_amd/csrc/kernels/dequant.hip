@@ -62,6 +62,23 @@ __device__ __forceinline__ void dequant_tile(const DequantArgs &a) {
                 store8(a.out, a.n, a.k, r, u * 128 + t * 32 + g * 8, v);
             }
         }
+    } else if constexpr (SCHEME == SCHEME_Q8K) {  // d * q with the super-block's f32 d (rlx-gguf/src/lib.rs:848-854)
+        const float d = *(const float *)(unit + 4096 + nrow * 4);
+#pragma unroll
+        for (int h = 0; h < 4; h++) {
+            const uint4_t q = *(const uint4_t *)(unit + h * 1024 + l * 16);
+#pragma unroll
+            for (int tt = 0; tt < 2; tt++) {
+                float v[8];
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    const uint32_t word = q[2 * tt + (e >> 2)];
+                    const int code = (int)((word >> (8 * (e & 3))) & 0xFFu) - 128;  // undo the offset-binary bias
+                    v[e] = d * (float)code;
+                }
+                store8(a.out, a.n, a.k, r, u * 256 + (2 * h + tt) * 32 + g * 8, v);
+            }
+        }
     } else if constexpr (SCHEME == SCHEME_Q6K) {
         // (d * sc) * (q - 32): the block decoder the reference's matmul calls reads the scale bytes as unsigned
         // (rlx-gguf/src/lib.rs:819-845), its tensor decoder and ggml as signed (lib.rs:1070-1112); a.sc_off picks
@@ -124,3 +141,4 @@ extern "C" __global__ __launch_bounds__(64) void rlx_dequant_q8_0(rlx::DequantAr
 extern "C" __global__ __launch_bounds__(64) void rlx_dequant_q4_k(rlx::DequantArgs a) { rlx::dequant_tile<rlx::SCHEME_Q4K>(a); }
 extern "C" __global__ __launch_bounds__(64) void rlx_dequant_q5_k(rlx::DequantArgs a) { rlx::dequant_tile<rlx::SCHEME_Q5K>(a); }
 extern "C" __global__ __launch_bounds__(64) void rlx_dequant_q6_k(rlx::DequantArgs a) { rlx::dequant_tile<rlx::SCHEME_Q6K>(a); }
+extern "C" __global__ __launch_bounds__(64) void rlx_dequant_q8_k(rlx::DequantArgs a) { rlx::dequant_tile<rlx::SCHEME_Q8K>(a); }

@@ -83,10 +83,11 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
     constexpr bool K5 = SCHEME == SCHEME_Q5K;                 // Q4_K with a fifth bit: every Q4_K branch below serves both
     constexpr bool K4 = SCHEME == SCHEME_Q4K || K5;
     constexpr bool K6 = SCHEME == SCHEME_Q6K;
+    constexpr bool K8 = SCHEME == SCHEME_Q8K;                 // exact int8 codes in B, the super-block's f32 d applied like Q6_K's
     constexpr int META_OFF = K5 ? 2560 : 2048;                // the 16 meta bytes per row of a Q4_K / Q5_K unit
     // Super-block schemes: B holds integers (Q4_K: sc * q, exact; Q6_K: sc * (q - 32), exact up to 2048), a second
     // accumulator set collects one 256-column super-block and d (Q4_K: and dmin) is applied in f32 per super-block.
-    constexpr bool SB = K4 || K6;
+    constexpr bool SB = K4 || K6 || K8;
     constexpr int WN = GEMM_NT / (32 * TJ), WM = 8 / WN, MT = WM * TI * 32;  // wave grid and rows per workgroup
     constexpr int NSA = MT / 32, SA = 4 * NSA * 1024, ST = SA + GEMM_STAGE_B;  // LDS stage: activations [4][NSA][1 KB], then weights
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -171,6 +172,8 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
                 b_hw[(q >> 1) & 1] = __builtin_amdgcn_raw_buffer_load_b64(b_rsrc, lane * 16 + (q >> 1) * 8, unit + 2048, 0);
             }
             if (q == 0) b_meta[0] = ld128(b_rsrc, b_n16 * 16, unit + 3072);  // copied aside when the super-block's decode starts
+        } else if constexpr (K8) {  // one quarter of the super-block (two 32-column blocks) per step
+            b_q[q & 1] = ld128(b_rsrc, lane * 16, (step >> 2) * L.unit_bytes + q * 1024);
         } else if constexpr (SCHEME == SCHEME_F16W) {  // two ready-made fragments per lane and step: b_q and b_meta hold them
             const int unit = (step >> 1) * L.unit_bytes + (q & 1) * 2048;
             b_q[q & 1] = ld128(b_rsrc, lane * 16, unit);
@@ -225,6 +228,10 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
             // block 2 q + jl of the super-block, this lane's 16-column half of it: scale byte 4 q + 2 jl + g / 2
             const uint32_t scb = (b_meta[1][q] >> (16 * jl + 8 * (b_g >> 1))) & 0xFFu;
             unpack_q6_scaled(b_q[cp][t], hx, splat_ubyte_half(scb, sc_bias), f);
+        } else if constexpr (K8) {
+            unpack_q8(b_q[q & 1][2 * jl], b_q[q & 1][2 * jl + 1], f);
+#pragma unroll
+            for (int e = 0; e < 4; e++) f.u[e] &= b_keep;  // a dead tile stores zeros
         } else if constexpr (SCHEME == SCHEME_F16W) {
             f.u4 = jl ? b_meta[q & 1] : b_q[q & 1];
 #pragma unroll
@@ -260,7 +267,7 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
         my_row[j] = n_tile0 + (wn * TJ + j) * 32 + lr;
         my_ok[j] = (my_row[j] >> 4) < sg.row_tiles;
         my_meta[j] = w_base + (long long)(my_ok[j] ? (my_row[j] >> 4) : 0) * a.units * L.unit_bytes +
-                     (K6 ? 3328 + (my_row[j] & 15) * 2 : META_OFF + (my_row[j] & 15) * 16);  // Q6_K: the row's d; Q4_K / Q5_K: its 16 meta bytes
+                     (K8 ? 4096 + (my_row[j] & 15) * 4 : K6 ? 3328 + (my_row[j] & 15) * 2 : META_OFF + (my_row[j] & 15) * 16);  // Q8_K / Q6_K: the row's d; Q4_K / Q5_K: its 16 meta bytes
     }
     uint4_t w_meta[TJ];
     Frag fs[TI];
@@ -294,6 +301,11 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
             for (int j = 0; j < TJ; j++) w_meta[j][0] = *(const uint16_t *)(my_meta[j] + (long long)sb * L.unit_bytes);
             return;
         }
+        if constexpr (K8) {
+#pragma unroll
+            for (int j = 0; j < TJ; j++) w_meta[j][0] = *(const uint32_t *)(my_meta[j] + (long long)sb * L.unit_bytes);
+            return;
+        }
 #pragma unroll
         for (int j = 0; j < TJ; j++) w_meta[j] = *(const uint4_t *)(my_meta[j] + (long long)sb * L.unit_bytes);
 #pragma unroll
@@ -303,10 +315,10 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
         }
     };
     auto scale_sb = [&]() {
-        if constexpr (K6) {  // total += d * P
+        if constexpr (K6 || K8) {  // total += d * P
 #pragma unroll
             for (int j = 0; j < TJ; j++) {
-                const float d = my_ok[j] ? half_bits_to_float(w_meta[j][0] & 0xFFFFu) : 0.f;
+                const float d = !my_ok[j] ? 0.f : K8 ? __builtin_bit_cast(float, w_meta[j][0]) : half_bits_to_float(w_meta[j][0] & 0xFFFFu);
 #pragma unroll
                 for (int i = 0; i < TI; i++)
 #pragma unroll
@@ -668,6 +680,9 @@ extern "C" __global__ __launch_bounds__(512) void rlx_gemm_q5_k(rlx::GemmArgs a)
 extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64_q5_k(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q5K, 1, 1>(a); }
 extern "C" __global__ __launch_bounds__(512) void rlx_gemm_q6_k(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q6K, 2, 2>(a); }
 extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64_q6_k(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q6K, 1, 1>(a); }
+extern "C" __global__ __launch_bounds__(512) void rlx_gemm_q8_k(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q8K, 2, 2>(a); }
+extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64_q8_k(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q8K, 1, 1>(a); }
+extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64g_q8_k(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q8K, 1, 1, true>(a); }
 extern "C" __global__ __launch_bounds__(512) void rlx_gemm_f16w(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_F16W, 2, 2>(a); }
 extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64_f16w(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_F16W, 1, 1>(a); }
 extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64_q4_k(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q4K, 1, 1>(a); }

@@ -158,6 +158,22 @@ struct UnitRegs<SCHEME_Q6K> {  // one super-block: low nibbles (two halves), hig
 };
 
 template <>
+struct UnitRegs<SCHEME_Q8K> {  // one super-block: four quarters of offset-binary bytes and the row's f32 d
+    uint4_t q[4];
+    uint32_t d;
+    __device__ __forceinline__ void load(const uint8_t *unit, int l, int nrow, bool) {
+#pragma unroll
+        for (int h = 0; h < 4; h++) q[h] = __builtin_nontemporal_load((const uint4_t *)(unit + h * 1024 + l * 16));
+        d = __builtin_nontemporal_load((const uint32_t *)(unit + 4096 + nrow * 4));
+    }
+    __device__ __forceinline__ void clear() {
+#pragma unroll
+        for (int h = 0; h < 4; h++) q[h] = uint4_t{0, 0, 0, 0};
+        d = 0;
+    }
+};
+
+template <>
 struct UnitRegs<SCHEME_F16W> {  // weights already stored as binary16 fragments: four 32-column blocks, no scales
     uint4_t q[4];
     __device__ __forceinline__ void load(const uint8_t *unit, int l, int, bool) {
@@ -247,6 +263,33 @@ __device__ __forceinline__ void compute_unit(const UnitRegs<SCHEME> &w, const ha
             }
         }
         const float d = half_bits_to_float(w.d);
+#pragma unroll
+        for (int rg = 0; rg < RG; rg++)
+#pragma unroll
+            for (int r = 0; r < NREG; r++) acc[rg][r] = __builtin_fmaf(d, sum[rg][r], acc[rg][r]);
+    } else if constexpr (SCHEME == SCHEME_Q8K) {
+        // B = q, an exact binary16 integer; the matrix unit accumulates the eight blocks of the super-block and the
+        // f32 d is applied once (the reference multiplies d into every weight: rlx-gguf/src/lib.rs:848-854)
+        float4_t sum[RG];
+#pragma unroll
+        for (int rg = 0; rg < RG; rg++) sum[rg] = zero;
+#pragma unroll
+        for (int h2 = 0; h2 < 2; h2++) {  // 128 columns at a time: quarters 2 h2 and 2 h2 + 1
+            if constexpr (RG == 1) load_afrags<4>(xrow[0], live[0], ucol + h2 * 128, a);
+            Frag b[4];
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                const uint4_t &q = w.q[2 * h2 + (t >> 1)];
+                unpack_q8(q[2 * (t & 1)], q[2 * (t & 1) + 1], b[t]);
+            }
+#pragma unroll
+            for (int rg = 0; rg < RG; rg++) {
+                if constexpr (RG > 1) load_afrags<4>(xrow[rg], live[rg], ucol + h2 * 128, a);
+#pragma unroll
+                for (int t = 0; t < 4; t++) sum[rg] = mfma16(a[t], b[t], sum[rg]);
+            }
+        }
+        const float d = __builtin_bit_cast(float, w.d);
 #pragma unroll
         for (int rg = 0; rg < RG; rg++)
 #pragma unroll
@@ -869,6 +912,7 @@ RLX_GEMV_SCHEME(q4_k, rlx::SCHEME_Q4K, 3, 1)
 RLX_GEMV_SCHEME(f16w, rlx::SCHEME_F16W, 2, 1)
 RLX_GEMV_SCHEME(q6_k, rlx::SCHEME_Q6K, 2, 1)
 RLX_GEMV_SCHEME(q5_k, rlx::SCHEME_Q5K, 2, 1)
+RLX_GEMV_SCHEME(q8_k, rlx::SCHEME_Q8K, 2, 1)
 // Two 128-column units per loop item: taken when every K run holds an even number of units. (Measured neutral to
 // slightly slower for Q8_0, whose unit is twice the bytes, so only Q4_0 has it.)
 RLX_GEMV_SCHEME(q4_0_u2, rlx::SCHEME_Q4_0, 2, 2)
@@ -884,3 +928,4 @@ RLX_GEMV_ROWGROUPS(q4_k, rlx::SCHEME_Q4K, 2)
 RLX_GEMV_ROWGROUPS(f16w, rlx::SCHEME_F16W, 2)
 RLX_GEMV_ROWGROUPS(q6_k, rlx::SCHEME_Q6K, 2)
 RLX_GEMV_ROWGROUPS(q5_k, rlx::SCHEME_Q5K, 2)
+RLX_GEMV_ROWGROUPS(q8_k, rlx::SCHEME_Q8K, 2)

@@ -34,7 +34,9 @@
 //                   elements 2,3 / 6,7 (value 1024 + 16 q) at bits 8-9 / 24-25; elements 4-7 are stored 2 bits higher
 //                   and used after a shift by 2, like their nibbles after a shift by 8.
 //          [3072,3328) per row n: the 16 scale bytes verbatim          [3328,3360) f16 d[n]
-//   Q8_K, Q2_K, Q3_K, and Q6_K when its scales are to be read as signed ("wide" schemes): the weights are decoded once, at upload, with the reference's block
+//   Q8_K : [0,4096)  four quarters h: 16 B at 1024*h + 16*l = granules of 32-column blocks 2h, 2h+1 of super-block u, bytes
+//                   XOR 0x80 as Q8_0          [4096,4160) f32 d[n] (the bsums of the GGUF block are not needed and not kept)
+//   Q2_K, Q3_K ("wide" schemes): the weights are decoded once, at upload, with the reference's block
 //          decoder and stored as binary16: [0,4096) four blocks t: 16 B at 1024*t + 16*l = the 8 halfs of granule
 //          (n, 4u+t, g), already an MFMA operand fragment. No scales. 2 bytes per weight resident instead of the
 //          packed 0.33-1.14, in exchange for kernels that do no decode arithmetic at all.
@@ -80,7 +82,7 @@ RLX_HD constexpr Layout layout_of(int scheme) {
            : scheme == SCHEME_Q4K  ? Layout{256, 2304, 2048, 256, 144}
            : scheme == SCHEME_Q5K  ? Layout{256, 2816, 2560, 256, 176}
            : scheme == SCHEME_Q6K  ? Layout{256, 3360, 3072, 256, 210}
-           : scheme == SCHEME_Q8K  ? Layout{128, 4096, 4096, 256, 292}
+           : scheme == SCHEME_Q8K  ? Layout{256, 4160, 4096, 256, 292}
            : scheme == SCHEME_Q2K  ? Layout{128, 4096, 4096, 256, 84}
            : scheme == SCHEME_Q3K  ? Layout{128, 4096, 4096, 256, 110}
            : scheme == SCHEME_F16W ? Layout{128, 4096, 4096, 0, 0}

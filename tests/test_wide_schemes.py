@@ -14,8 +14,8 @@ import rlx_amd
 from rlx_amd import DType, QuantScheme, ops
 from helpers import BLOCK, Q2K, Q3K, Q4K, Q5K, Q6K, Q8K, WIDE, decode_device_layout, random_blocks, rel_err
 
-FIVE = WIDE + (Q5K, Q6K)
-PACKED = (Q5K, Q6K)
+FIVE = WIDE + (Q5K, Q6K, Q8K)
+PACKED = (Q5K, Q6K, Q8K)
 
 F16 = lambda v: np.frombuffer(np.float16(v).tobytes(), np.uint8)  # noqa: E731
 
@@ -234,12 +234,12 @@ def test_repack_host_is_f16_of_the_matmul_decoder(scheme):
 
 @pytest.mark.parametrize("scheme", PACKED)
 def test_packed_layout_keeps_every_bit(scheme):
-    """The packed Q5_K / Q6_K device layouts (same byte count as the GGUF blocks) read back with numpy by the rules of
-    csrc/layout.h."""
+    """The packed Q5_K / Q6_K / Q8_K device layouts (the byte count of the GGUF blocks; Q8_K without the 32 bytes of block
+    sums per super-block, which no decoder reads) read back with numpy by the rules of csrc/layout.h."""
     n, k = 37, 768
     blocks = random_blocks(scheme, n, k, seed=47)
     dev = ops.repack_host(scheme, blocks, n, k)
-    assert dev.size == ((n + 15) // 16) * (k // 256) * 16 * BLOCK[scheme][1]
+    assert dev.size == ((n + 15) // 16) * (k // 256) * 16 * (BLOCK[scheme][1] - (32 if scheme == Q8K else 0))
     assert np.array_equal(decode_device_layout(scheme, dev, n, k).view(np.uint32),
                           oracle.dequant_matmul_blocks(scheme, blocks, n * k).reshape(n, k).view(np.uint32))
 
@@ -257,9 +257,13 @@ def test_packed_q6k_layout_with_signed_scales():
 
 
 def test_repack_rejects_weights_beyond_binary16():
-    blk = np.concatenate([np.frombuffer(np.float32(1e4).tobytes(), np.uint8), np.full(256, 100, np.uint8), np.zeros(32, np.uint8)])
+    # Q2_K: d = 60000, every scale nibble 15, every code 3 -> 2.7e6, past what the binary16 copy of a wide scheme holds
+    blk = np.concatenate([np.array([60000.0, 0.0], np.float16).view(np.uint8), np.full(16, 0x0F, np.uint8), np.full(64, 0xFF, np.uint8)])
     with pytest.raises(rlx_amd.RlxError, match="binary16"):
-        ops.repack_host(Q8K, blk, 1, 256)
+        ops.repack_host(Q2K, blk, 1, 256)
+    # Q8_K is packed: its f32 scale is kept as it is
+    big = np.concatenate([np.frombuffer(np.float32(1e4).tobytes(), np.uint8), np.full(256, 100, np.uint8), np.zeros(32, np.uint8)])
+    assert ops.repack_host(Q8K, big, 1, 256).size == 4160
 
 
 # ---- GPU ---------------------------------------------------------------------------------------------------------
@@ -415,15 +419,15 @@ def test_q6k_signed_scales_through_session_and_gguf_file(tmp_path):
 
 @pytest.mark.gpu
 def test_wide_dequant_is_refused():
-    blocks = random_blocks(Q8K, 16, 256, seed=1)
-    qw = ops.QWeight(QuantScheme.GgufQ8K, blocks, 16, 256)
+    blocks = random_blocks(Q2K, 16, 256, seed=1)
+    qw = ops.QWeight(QuantScheme.GgufQ2K, blocks, 16, 256)
     with pytest.raises(rlx_amd.RlxError, match="binary16"):
         qw.dequant()
     qw.free()
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("scheme", [Q6K, Q5K])
+@pytest.mark.parametrize("scheme", [Q6K, Q5K, Q8K])
 def test_wide_grouped_matmul(scheme):
     """Mixture-of-experts routing (rlx-cpu/src/gguf_matmul.rs:101-139) over a stack of wide-scheme slabs."""
     k, n, experts, m = 512, 24, 4, 11
