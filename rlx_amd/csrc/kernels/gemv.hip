@@ -369,13 +369,16 @@ __device__ __forceinline__ void compute_unit(const UnitRegs<SCHEME> &w, const ha
 }
 
 // Convert one K chunk of the activations into LDS as halfs: f32 -> hi rows [0,m) + lo rows [m,2m); 16-bit -> rows [0,m).
-// Each thread issues up to eight independent loads before it converts the first one, so a chunk of many rows costs
-// one memory latency per eight groups of columns, not one per group.
-// PASS 0: stage, and add to masks[0] / masks[1] (the calling wave's own) the rows with some |x| >= X_BIG / some |x| >= X_SMALL; PASS 1: only find
-// the largest |x| of every row (rowmax, as bits); PASS 2: stage again with row r multiplied by fwd[r].
+// The work is cut into (row, slice of the row's 16-byte groups) tasks, one wave per task: with fewer rows than waves a row
+// is shared by several waves, otherwise a wave takes whole rows in turn. A wave therefore works on one row at a time -
+// no index arithmetic per group, the row's LDS address and factors are scalars, and what the range check has to note
+// about a row is one running maximum per lane and two votes per task. Each lane issues up to eight independent loads
+// before it converts the first one, so a task costs one memory latency per eight wave-loads, not one per load.
+// PASS 0: stage, and add to masks[0] / masks[1] (the calling wave's own) the rows with some |x| >= X_BIG / some
+// |x| >= X_SMALL; PASS 1: only find the largest |x| of every row (rowmax, as bits); PASS 2: stage again with row r
+// multiplied by fwd[r].
 // Every wave of the launch runs PASS 0 at the same moment, before there is other work to hide it behind, so its VALU
-// count is launch latency: the largest |x| of a 16-byte group is one v_max3_f32 per two values, and with a single activation
-// row a running maximum is the whole note.
+// count is launch latency: the largest |x| costs one v_max3_f32 per two values.
 __device__ __forceinline__ float max3_abs(float acc, float x, float y) {  // max(acc, |x|, |y|); a NaN operand is skipped
     float r;
     asm("v_max3_f32 %0, %1, |%2|, |%3|" : "=v"(r) : "v"(acc), "v"(x), "v"(y));
@@ -387,139 +390,95 @@ __device__ __forceinline__ void stage_x_typed(const GemvArgs &a, const GemvSeg &
                                               const float *fwd = nullptr) {
     constexpr int U = 8;
     constexpr int G = XD == X_F32 ? 4 : 8;  // columns per 16-byte load
+    constexpr int ESZ = XD == X_F32 ? 4 : 2;
     typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
-    const int tid = threadIdx.x, nt = blockDim.x;
+    typedef typename std::conditional<XD == X_F32, float4_t, uint4_t>::type raw_t;  // 16 bytes either way
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), nwaves = (int)(blockDim.x >> 6);
     const int groups = kc / G;  // kc is a multiple of 64
-    const int total = a.m * groups;
-    uint32_t big = 0, seen = 0;
-    float vmax = 0.f;  // the largest |x| this thread has seen: all the note there is to take with one activation row
-    const bool one_row = a.m == 1;  // (a variant of this function compiled for one row takes the kernels past 128 registers)
-    // group index -> (row, group within the row) without an integer division (20 instructions, some of them quarter
-    // rate, eight times over, in front of loads that every wave of the launch is waiting for): idx < 2^24 is exact in
-    // f32, the quotient estimate is off by at most one and is put right by one compare each way.
-    const float inv_groups = 1.0f / (float)groups;
+    const int slices = a.m >= nwaves ? 1 : (nwaves + a.m - 1) / a.m;  // waves that share a row
+    const int gps = ((groups + slices - 1) / slices + 63) & ~63;      // groups per slice: whole wave-loads
+    const int tasks = a.m * slices;
     const int lo_rows = a.m * row_stride;  // halfs from a hi row to its lo row
-    auto split = [&](int idx, int &row, int &cg) {
-        if (one_row) {
-            row = 0;
-            cg = idx;
-            return;
-        }
-        row = (int)((float)idx * inv_groups);
-        cg = idx - (int)__umul24((unsigned)row, (unsigned)groups);
-        if (cg < 0) {
-            row--;
-            cg += groups;
-        } else if (cg >= groups) {
-            row++;
-            cg -= groups;
-        }
-    };
-    for (int idx0 = tid; idx0 < total; idx0 += nt * U) {
-        typedef typename std::conditional<XD == X_F32, float4_t, uint4_t>::type raw_t;  // 16 bytes either way
-        raw_t raw[U];
+    for (int t = wave; t < tasks; t += nwaves) {
+        const int row = t / slices, slice = t - row * slices;
+        const int g0 = slice * gps, g1 = min(groups, g0 + gps);
+        const uint8_t *src = (const uint8_t *)sg.x + ((long long)row * sg.k + k0) * ESZ;
+        half_t *dst = xs + row * row_stride;
+        float vmax = 0.f;  // the largest |x| this lane has seen in the row
+        float rowscale = 1.f, scale = 1.f;
+        if constexpr (PASS == 2) rowscale = fwd[row];
+        if constexpr (NORM) scale = inv_rms[row];
+        for (int cg0 = g0 + lane; cg0 < g1; cg0 += 64 * U) {
+            raw_t raw[U];
 #pragma unroll
-        for (int u = 0; u < U; u++) {
-            const int idx = idx0 + u * nt;
-            raw_t v = {};
-            if (idx < total) {  // a wave with no lane left skips the arithmetic too
-                int row, cg;
-                split(idx, row, cg);
-                const int c = cg * G;
+            for (int u = 0; u < U; u++) {
+                const int c = (cg0 + 64 * u) * G;
+                raw_t v = {};
                 // k is a multiple of 32: a group is inside or outside as a whole
-                const long long at = one_row ? (long long)(k0 + c) : (long long)row * sg.k + k0 + c;
-                if (k0 + c < sg.k) v = *(const raw_t *)((const uint8_t *)sg.x + at * (XD == X_F32 ? 4 : 2));
+                if (cg0 + 64 * u < g1 && k0 + c < sg.k) v = *(const raw_t *)(src + (long long)c * ESZ);
+                raw[u] = v;
             }
-            raw[u] = v;
-        }
 #pragma unroll
-        for (int u = 0; u < U; u++) {
-            const int idx = idx0 + u * nt;
-            if (idx >= total) continue;
-            int row, cg;
-            split(idx, row, cg);
-            const int c = cg * G;
-            float rowscale = 1.f;
-            if constexpr (PASS == 2) rowscale = fwd[row];
-            if constexpr (XD == X_F32) {
-                half4_t hi, lo;
-                float4_t gm = {1.f, 1.f, 1.f, 1.f}, bt = {0.f, 0.f, 0.f, 0.f};
-                float scale = 1.f;
-                if constexpr (NORM) {
-                    scale = inv_rms[row];
-                    if (k0 + c < sg.k) {
-                        gm = *(const float4_t *)(a.gamma + k0 + c);
-                        if (a.beta) bt = *(const float4_t *)(a.beta + k0 + c);
+            for (int u = 0; u < U; u++) {
+                const int c = (cg0 + 64 * u) * G;
+                if (cg0 + 64 * u >= g1) continue;
+                if constexpr (XD == X_F32) {
+                    half4_t hi, lo;
+                    float4_t gm = {1.f, 1.f, 1.f, 1.f}, bt = {0.f, 0.f, 0.f, 0.f};
+                    if constexpr (NORM) {
+                        if (k0 + c < sg.k) {
+                            gm = *(const float4_t *)(a.gamma + k0 + c);
+                            if (a.beta) bt = *(const float4_t *)(a.beta + k0 + c);
+                        }
                     }
-                }
-                float amax = 0.f, prev = 0.f;
+                    float prev = 0.f;
 #pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    float v = raw[u][e];
-                    if constexpr (NORM) v = v * scale * gm[e] + bt[e];  // in_row[i] * inv_rms * gamma[i] + beta[i], unfused
-                    if constexpr (PASS == 0) {
-                        if (e & 1) amax = max3_abs(amax, prev, v);
-                        else prev = v;
+                    for (int e = 0; e < 4; e++) {
+                        float v = raw[u][e];
+                        if constexpr (NORM) v = v * scale * gm[e] + bt[e];  // in_row[i] * inv_rms * gamma[i] + beta[i], unfused
+                        if constexpr (PASS != 2) {
+                            if (e & 1) vmax = max3_abs(vmax, prev, v);
+                            else prev = v;
+                        }
+                        if constexpr (PASS == 2) v *= rowscale;
+                        hi[e] = (half_t)v;
+                        // residual, scaled by 2^11 so it stays in the normal binary16 range; undone in the final sum
+                        lo[e] = (half_t)((v - (float)hi[e]) * LO_SCALE);
                     }
-                    if constexpr (PASS == 1) amax = __builtin_fmaxf(amax, __builtin_fabsf(v));  // a NaN is skipped
-                    if constexpr (PASS == 2) v *= rowscale;
-                    hi[e] = (half_t)v;
-                    // residual, scaled by 2^11 so it stays in the normal binary16 range; undone in the final sum
-                    lo[e] = (half_t)((v - (float)hi[e]) * LO_SCALE);
-                }
-                if constexpr (PASS == 0) {
-                    if (one_row) {
-                        vmax = __builtin_fmaxf(vmax, amax);
-                    } else {
-                        big |= (amax >= X_BIG ? 1u : 0u) << row;
-                        seen |= (amax >= X_SMALL ? 1u : 0u) << row;
+                    if constexpr (PASS != 1) {
+                        *(half4_t *)(dst + c) = hi;
+                        *(half4_t *)(dst + lo_rows + c) = lo;
                     }
-                }
-                if constexpr (PASS == 1) {
-                    atomicMax(rowmax + row, __builtin_bit_cast(uint32_t, amax));
-                } else {
-                    half_t *dst = xs + (one_row ? c : (int)__umul24((unsigned)row, (unsigned)row_stride) + c);
-                    *(half4_t *)dst = hi;
-                    *(half4_t *)(dst + lo_rows) = lo;
-                }
-            } else if constexpr (XD == X_BF16) {
-                half8_t h;
-                float amax = 0.f;
+                } else if constexpr (XD == X_BF16) {
+                    half8_t h;
+                    float prev = 0.f;
 #pragma unroll
-                for (int e = 0; e < 8; e++) {
-                    const uint32_t bits = ((e & 1) ? (raw[u][e >> 1] >> 16) : (raw[u][e >> 1] & 0xFFFFu)) << 16;
-                    float v = __builtin_bit_cast(float, bits);
-                    if constexpr (PASS == 1) amax = __builtin_fmaxf(amax, __builtin_fabsf(v));
-                    if constexpr (PASS == 2) v *= rowscale;
-                    h[e] = (half_t)v;
-                }
-                if constexpr (PASS == 0) {
-                    // a dword read as f32 is its upper bf16 value with up to 2^-8 added in magnitude: close enough for the thresholds
-#pragma unroll
-                    for (int d = 0; d < 4; d++)
-                        amax = max3_abs(amax, __builtin_bit_cast(float, raw[u][d]), __builtin_bit_cast(float, raw[u][d] << 16));
-                    if (one_row) {
-                        vmax = __builtin_fmaxf(vmax, amax);
-                    } else {
-                        big |= (amax >= X_BIG ? 1u : 0u) << row;
-                        seen |= (amax >= X_SMALL ? 1u : 0u) << row;
+                    for (int e = 0; e < 8; e++) {
+                        const uint32_t bits = ((e & 1) ? (raw[u][e >> 1] >> 16) : (raw[u][e >> 1] & 0xFFFFu)) << 16;
+                        float v = __builtin_bit_cast(float, bits);
+                        if constexpr (PASS != 2) {
+                            if (e & 1) vmax = max3_abs(vmax, prev, v);
+                            else prev = v;
+                        }
+                        if constexpr (PASS == 2) v *= rowscale;
+                        h[e] = (half_t)v;
                     }
+                    if constexpr (PASS != 1) *(half8_t *)(dst + c) = h;
+                } else {  // binary16 activations are staged as they are: nothing to gain from a scale
+                    *(uint4_t *)(dst + c) = raw[u];
                 }
-                if constexpr (PASS == 1) atomicMax(rowmax + row, __builtin_bit_cast(uint32_t, amax));
-                else *(half8_t *)(xs + (one_row ? c : (int)__umul24((unsigned)row, (unsigned)row_stride) + c)) = h;
-            } else {  // binary16 activations are staged as they are: nothing to gain from a scale
-                *(uint4_t *)(xs + (one_row ? c : (int)__umul24((unsigned)row, (unsigned)row_stride) + c)) = raw[u];
             }
         }
-    }
-    if constexpr (PASS == 0 && XD != X_F16) {  // into the wave's two masks (wave-uniform: a vote per row is two scalar operations)
-        if (one_row) {
-            masks[0] |= __ballot(vmax >= X_BIG) != 0 ? 1u : 0u;
-            masks[1] |= __ballot(vmax >= X_SMALL) != 0 ? 1u : 0u;
-        } else {
-            for (int r = 0; r < a.m; r++) {
-                masks[0] |= (__ballot((big >> r) & 1u) != 0 ? 1u : 0u) << r;
-                masks[1] |= (__ballot((seen >> r) & 1u) != 0 ? 1u : 0u) << r;
+        if constexpr (XD != X_F16) {
+            if constexpr (PASS == 0) {  // into the wave's two masks: one vote each per task
+                masks[0] |= (__ballot(vmax >= X_BIG) != 0 ? 1u : 0u) << row;
+                masks[1] |= (__ballot(vmax >= X_SMALL) != 0 ? 1u : 0u) << row;
+            }
+            if constexpr (PASS == 1) {
+#pragma unroll
+                for (int off = 32; off > 0; off >>= 1) vmax = __builtin_fmaxf(vmax, __shfl_xor(vmax, off));
+                if (lane == 0) atomicMax(rowmax + row, __builtin_bit_cast(uint32_t, vmax));
             }
         }
     }
