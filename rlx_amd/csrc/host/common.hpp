@@ -63,8 +63,8 @@ enum KernelId : int {
     K_COUNT
 };
 
-// Device layout a scheme is kept in: its packed layout (layout_of), or binary16 fragments for the wide schemes (Q8_K,
-// Q2_K, Q3_K).
+// Device layout a scheme is kept in: its packed layout (layout_of), or binary16 fragments for the wide schemes (Q2_K,
+// Q3_K).
 Layout host_layout(int scheme);
 inline bool is_wide(int scheme) { return layout_is_f16w(host_layout(scheme)); }
 
