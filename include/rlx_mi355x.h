@@ -58,7 +58,7 @@ typedef enum rlx_quant_scheme {
     RLX_SCHEME_GGUF_Q6K = 7,  /* 256 / 210 */
     RLX_SCHEME_GGUF_Q8K = 8,  /* 256 / 292 */
     RLX_SCHEME_GGUF_Q2K = 9,  /* 256 / 84, wide (field order of rlx-gguf/src/lib.rs:857-886) */
-    RLX_SCHEME_GGUF_Q3K = 10, /* 256 / 110, wide (field order of rlx-gguf/src/lib.rs:889-930) */
+    RLX_SCHEME_GGUF_Q3K = 10, /* 256 / 110 (field order of rlx-gguf/src/lib.rs:889-930); resident as Q6_K super-blocks of the same values */
     RLX_SCHEME_GGUF_Q4_0 = 11, /* 32 elems / 18 bytes  */
     RLX_SCHEME_GGUF_Q8_0 = 12  /* 32 elems / 34 bytes  */
 } rlx_quant_scheme;

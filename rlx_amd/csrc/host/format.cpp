@@ -66,33 +66,28 @@ static void decode_q2_k(const uint8_t *b, float *out) {
     }
 }
 
-// Q3_K in the reference's field order (lib.rs:889-930): d, 12 scale bytes, 32 bytes of high-bit mask, 64 bytes of 2-bit codes.
-static void decode_q3_k(const uint8_t *b, float *out) {
-    const float d_all = f16_at(b);
-    const uint8_t *s = b + 2, *hm = b + 14, *q = b + 46;
-    int scale[16];
+// Q3_K in the reference's field order (lib.rs:889-930): d, 12 scale bytes, 32 bytes of high-bit mask, 64 bytes of 2-bit
+// codes. The value of element i is d * (scale[i / 16] - 32) * code(i) with code in [-4, 3]: at most 20 significant bits, so
+// every product is exact in f32 in any order, and the super-block is the Q6_K super-block with codes code + 32 and signed
+// scale bytes scale - 32. These two read the fields a Q6_K unit needs.
+static void q3k_scales(const uint8_t *b, int scale[16]) {
+    const uint8_t *s = b + 2;
     for (int j = 0; j < 4; j++) {
         scale[j] = (s[j] & 0xF) | ((s[8 + j] & 3) << 4);
         scale[4 + j] = (s[4 + j] & 0xF) | (((s[8 + j] >> 2) & 3) << 4);
         scale[8 + j] = (s[j] >> 4) | (((s[8 + j] >> 4) & 3) << 4);
         scale[12 + j] = (s[4 + j] >> 4) | (((s[8 + j] >> 6) & 3) << 4);
     }
-    for (int i = 0; i < 256; i++) {
-        const int h = i >> 7, pair = (i >> 5) & 3, l = i & 31;
-        const float dl = d_all * (float)(scale[8 * h + 2 * pair + (l >> 4)] - 32);
-        const int code = ((q[32 * h + l] >> (2 * pair)) & 3) - ((hm[l] >> (4 * h + pair)) & 1 ? 0 : 4);
-        out[i] = dl * (float)code;
-    }
+}
+static inline int q3k_code(const uint8_t *b, int i) {
+    const uint8_t *hm = b + 14, *q = b + 46;
+    const int h = i >> 7, pair = (i >> 5) & 3, l = i & 31;
+    return ((q[32 * h + l] >> (2 * pair)) & 3) - ((hm[l] >> (4 * h + pair)) & 1 ? 0 : 4);
 }
 
 Layout host_layout(int scheme) { return layout_of(scheme); }
 
-static void decode_wide_block(int scheme, const uint8_t *b, float *out) {
-    switch (scheme) {
-    case SCHEME_Q2K: decode_q2_k(b, out); break;
-    default: decode_q3_k(b, out); break;
-    }
-}
+static void decode_wide_block(int, const uint8_t *b, float *out) { decode_q2_k(b, out); }
 
 // Wide schemes: decode every super-block and store the weights as binary16 operand fragments.
 static int repack_wide(int scheme, const uint8_t *src, int64_t n, int64_t k, uint8_t *out) {
@@ -214,12 +209,19 @@ int repack_host(int scheme, uint32_t flags, const uint8_t *src, size_t nbytes, i
                         memcpy(unit + (j >> 2) * 1024 + l * 16 + (j & 3) * 4, &word, 4);
                     }
                     memcpy(unit + 2048 + l * 8, hb, 8);
-                } else if (scheme == SCHEME_Q6K) {  // one super-block per unit: low nibbles, high-bit words, scales, d
-                    const bool live = r < n && u < bpr;
+                } else if (scheme == SCHEME_Q6K || scheme == SCHEME_Q3K) {
+                    // one super-block per unit: low nibbles, high-bit words, scales, d. A Q3_K super-block is stored as the
+                    // Q6_K super-block of the same values: codes + 32, scale bytes (scale - 32) XOR 0x80, the same d.
+                    const bool live = r < n && u < bpr, q3 = scheme == SCHEME_Q3K;
                     const uint8_t *b = live ? src + (r * bpr + u) * L.block_bytes : nullptr;
                     if (g == 0) {
-                        for (int e = 0; e < 16; e++) unit[3072 + nrow * 16 + e] = (uint8_t)((live ? b[192 + e] : 0) ^ q6_flip);
-                        if (live) memcpy(unit + 3328 + nrow * 2, b + 208, 2);
+                        int sc3[16];
+                        if (live && q3) q3k_scales(b, sc3);
+                        for (int e = 0; e < 16; e++) {
+                            const uint8_t byte = !live ? 0 : q3 ? (uint8_t)(int8_t)(sc3[e] - 32) : b[192 + e];
+                            unit[3072 + nrow * 16 + e] = (uint8_t)(byte ^ (q3 ? 0x80u : q6_flip));
+                        }
+                        if (live) memcpy(unit + 3328 + nrow * 2, q3 ? b : b + 208, 2);
                         else memset(unit + 3328 + nrow * 2, 0, 2);
                     }
                     uint32_t hw[4] = {0, 0, 0, 0};
@@ -228,7 +230,9 @@ int repack_host(int scheme, uint32_t flags, const uint8_t *src, size_t nbytes, i
                         for (int e = 0; e < 8; e++) {
                             const int i = 32 * j + 8 * g + e;  // element of the super-block
                             uint32_t code = 32;               // decodes to zero
-                            if (live) {
+                            if (live && q3) {
+                                code = (uint32_t)(q3k_code(b, i) + 32);
+                            } else if (live) {
                                 const int h = i >> 7, quarter = (i >> 5) & 3, l5 = i & 31;
                                 const uint8_t lowbyte = b[64 * h + 32 * (quarter & 1) + l5];
                                 const uint32_t low = (quarter >> 1) ? (uint32_t)(lowbyte >> 4) : (uint32_t)(lowbyte & 0x0F);

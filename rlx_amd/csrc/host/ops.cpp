@@ -464,7 +464,9 @@ int rlx_mi355x_qweight_create_ex(int scheme, uint32_t flags, const void *gguf_by
         std::vector<uint8_t> staging(total);
         for (int64_t e = 0; e < num_experts; e++)
             RLX_TRY(repack_host(scheme, flags, (const uint8_t *)gguf_bytes + e * slab, (size_t)slab, n, k, staging.data() + e * D.bytes));
-        qw = new rlx_qweight{scheme, HL, D, nullptr, false, (int)num_experts, flags};
+        // `scheme` of a weight names the kernels that read it: Q3_K units are Q6_K units with signed scale bytes
+        const uint32_t kflags = scheme == SCHEME_Q3K ? (uint32_t)RLX_QW_Q6K_SIGNED_SCALES : flags;
+        qw = new rlx_qweight{kernel_scheme(scheme), HL, D, nullptr, false, (int)num_experts, kflags};
         if (!device_mem) {
             hipError_t me = hipMalloc(&device_mem, total);
             if (me != hipSuccess) {

@@ -36,10 +36,12 @@
 //          [3072,3328) per row n: the 16 scale bytes verbatim          [3328,3360) f16 d[n]
 //   Q8_K : [0,4096)  four quarters h: 16 B at 1024*h + 16*l = granules of 32-column blocks 2h, 2h+1 of super-block u, bytes
 //                   XOR 0x80 as Q8_0          [4096,4160) f32 d[n] (the bsums of the GGUF block are not needed and not kept)
-//   Q2_K, Q3_K ("wide" schemes): the weights are decoded once, at upload, with the reference's block
+//   Q3_K : Q6_K units. A super-block's values d * (scale - 32) * code (code in [-4, 3]) are those of the Q6_K super-block
+//          with 6-bit codes code + 32, scale bytes scale - 32 (stored XOR 0x80, read as byte - 128) and the same d.
+//   Q2_K ("wide" scheme): the weights are decoded once, at upload, with the reference's block
 //          decoder and stored as binary16: [0,4096) four blocks t: 16 B at 1024*t + 16*l = the 8 halfs of granule
 //          (n, 4u+t, g), already an MFMA operand fragment. No scales. 2 bytes per weight resident instead of the
-//          packed 0.33-1.14, in exchange for kernels that do no decode arithmetic at all.
+//          packed 0.33, in exchange for kernels that do no decode arithmetic at all.
 // Units are stored [row_tile][unit] with the unit index (K direction) fastest.
 // N is padded to a multiple of 16 and K to a multiple of UNIT_K with zero-scale blocks.
 #pragma once
@@ -84,7 +86,7 @@ RLX_HD constexpr Layout layout_of(int scheme) {
            : scheme == SCHEME_Q6K  ? Layout{256, 3360, 3072, 256, 210}
            : scheme == SCHEME_Q8K  ? Layout{256, 4160, 4096, 256, 292}
            : scheme == SCHEME_Q2K  ? Layout{128, 4096, 4096, 256, 84}
-           : scheme == SCHEME_Q3K  ? Layout{128, 4096, 4096, 256, 110}
+           : scheme == SCHEME_Q3K  ? Layout{256, 3360, 3072, 256, 110}  // rewritten as Q6_K units
            : scheme == SCHEME_F16W ? Layout{128, 4096, 4096, 0, 0}
                                    : Layout{0, 0, 0, 0, 0};
 }
@@ -93,6 +95,9 @@ RLX_HD constexpr Layout layout_of(int scheme) {
 RLX_HD constexpr Layout wide_layout_of(int scheme) {
     return Layout{128, 4096, 4096, layout_of(scheme).block_elems, layout_of(scheme).block_bytes};
 }
+// The scheme whose kernels read a scheme's device units. A Q3_K super-block (3-bit codes in [-4, 3], 6-bit scales minus 32,
+// one d) is rewritten at upload, exactly, as the Q6_K super-block of the same values with signed scale bytes.
+RLX_HD constexpr int kernel_scheme(int scheme) { return scheme == SCHEME_Q3K ? SCHEME_Q6K : scheme; }
 RLX_HD constexpr bool layout_is_f16w(const Layout &L) { return L.unit_k == 128 && L.unit_bytes == 4096; }
 
 // nibble position of fragment element e inside a granule word

@@ -2,12 +2,12 @@
 import numpy as np
 
 Q4K, Q5K, Q6K, Q8K, Q2K, Q3K, Q4_0, Q8_0 = 5, 6, 7, 8, 9, 10, 11, 12
-WIDE = (Q2K, Q3K)  # decoded at upload and stored as binary16 on the device
+WIDE = (Q2K,)  # decoded at upload and stored as binary16 on the device
 SCHEME_NAMES = {Q4K: "q4_k", Q5K: "q5_k", Q6K: "q6_k", Q8K: "q8_k", Q2K: "q2_k", Q3K: "q3_k", Q4_0: "q4_0", Q8_0: "q8_0"}
 BLOCK = {Q4_0: (32, 18), Q8_0: (32, 34), Q4K: (256, 144), Q5K: (256, 176), Q6K: (256, 210), Q8K: (256, 292), Q2K: (256, 84), Q3K: (256, 110)}
 NIB_POS = [0, 4, 1, 5, 2, 6, 3, 7]
 UNIT = {Q4_0: (128, 1152, 1024), Q8_0: (128, 2176, 2048), Q4K: (256, 2304, 2048), Q5K: (256, 2816, 2560), Q6K: (256, 3360, 3072),
-        Q8K: (256, 4160, 4096)}
+        Q8K: (256, 4160, 4096), Q3K: (256, 3360, 3072)}  # Q3_K super-blocks are stored as Q6_K units with signed scale bytes
 Q5K_HI_POS = [4, 20, 8, 24, 5, 21, 9, 25]  # fifth bit of element e in the half's word after its code word's rotate (csrc/layout.h)
 Q5K_ROT = [0, 2, 8, 10]
 Q6K_HI_POS = [4, 20, 8, 24, 6, 22, 10, 26]  # low bit of element e's 2-bit high field in the even word of a pair (csrc/layout.h)
@@ -46,6 +46,8 @@ def decode_device_layout(scheme, dev, n, k, q6k_sc_off=0):
     """Read the device layout back into f32 [n,k] following csrc/layout.h, with the reference's arithmetic.
     q6k_sc_off: a stored Q6_K scale byte stands for byte - q6k_sc_off (128 for a weight repacked with signed scales)."""
     unit_k, unit_bytes, qbytes = UNIT[scheme]
+    if scheme == Q3K:
+        scheme, q6k_sc_off = Q6K, 128
     tiles, units = (n + 15) // 16, (k + unit_k - 1) // unit_k
     dev = dev.reshape(tiles, units, unit_bytes)
     out = np.zeros((tiles * 16, units * unit_k), np.float32)

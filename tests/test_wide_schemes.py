@@ -14,8 +14,8 @@ import rlx_amd
 from rlx_amd import DType, QuantScheme, ops
 from helpers import BLOCK, Q2K, Q3K, Q4K, Q5K, Q6K, Q8K, WIDE, decode_device_layout, random_blocks, rel_err
 
-FIVE = WIDE + (Q5K, Q6K, Q8K)
-PACKED = (Q5K, Q6K, Q8K)
+PACKED = (Q5K, Q6K, Q8K, Q3K)
+FIVE = WIDE + PACKED
 
 F16 = lambda v: np.frombuffer(np.float16(v).tobytes(), np.uint8)  # noqa: E731
 
@@ -235,11 +235,13 @@ def test_repack_host_is_f16_of_the_matmul_decoder(scheme):
 @pytest.mark.parametrize("scheme", PACKED)
 def test_packed_layout_keeps_every_bit(scheme):
     """The packed Q5_K / Q6_K / Q8_K device layouts (the byte count of the GGUF blocks; Q8_K without the 32 bytes of block
-    sums per super-block, which no decoder reads) read back with numpy by the rules of csrc/layout.h."""
+    sums per super-block, which no decoder reads) and Q3_K's (its super-blocks rewritten as Q6_K super-blocks of the same
+    values, 210 bytes each) read back with numpy by the rules of csrc/layout.h."""
     n, k = 37, 768
     blocks = random_blocks(scheme, n, k, seed=47)
     dev = ops.repack_host(scheme, blocks, n, k)
-    assert dev.size == ((n + 15) // 16) * (k // 256) * 16 * (BLOCK[scheme][1] - (32 if scheme == Q8K else 0))
+    per_block = 210 if scheme == Q3K else BLOCK[scheme][1] - (32 if scheme == Q8K else 0)
+    assert dev.size == ((n + 15) // 16) * (k // 256) * 16 * per_block
     assert np.array_equal(decode_device_layout(scheme, dev, n, k).view(np.uint32),
                           oracle.dequant_matmul_blocks(scheme, blocks, n * k).reshape(n, k).view(np.uint32))
 
