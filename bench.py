@@ -375,15 +375,15 @@ def extra_configs(rlx_amd, stream):
                                   "frac_hbm": round(b / ms / 1e6 / HBM_PEAK_GBS, 4)}
     for q in qws:
         q.free()
-    # the other K-quants on a gate/up projection [14336, 4096]: Q6_K, Q5_K and Q8_K have packed kernels (48 / 40 / 61 MB per
-    # copy); Q2_K stands for the schemes decoded at upload and resident as binary16 (117 MB per copy). Copies rotated: nothing
-    # cache-resident.
+    # the other K-quants on a gate/up projection [14336, 4096], all packed: Q6_K, Q5_K, Q8_K and Q2_K in kernels of their own
+    # (48 / 40 / 61 / 20 MB per copy), Q3_K as Q6_K super-blocks (48 MB). Copies rotated: nothing cache-resident.
     n, k = 14336, 4096
     rng = np.random.default_rng(5)
     for tag, scheme, bb, d_off, copies in (("q6_k_gemv_gate/up", QuantScheme.GgufQ6K, 210, 208, 13),
                                             ("q5_k_gemv_gate/up", QuantScheme.GgufQ5K, 176, 0, 15),
                                             ("q8_k_gemv_gate/up", QuantScheme.GgufQ8K, 292, 0, 10),
-                                            ("q2_k_gemv_gate/up_resident_f16", QuantScheme.GgufQ2K, 84, 0, 5)):
+                                            ("q2_k_gemv_gate/up", QuantScheme.GgufQ2K, 84, 0, 26),
+                                            ("q3_k_gemv_gate/up_as_q6_k_units", QuantScheme.GgufQ3K, 110, 0, 13)):
         blocks = rng.integers(0, 256, (n * k // 256, bb), dtype=np.uint8)
         if scheme == QuantScheme.GgufQ8K:
             blocks[:, 0:4] = np.full(n * k // 256, 2e-4, np.float32).view(np.uint8).reshape(-1, 4)

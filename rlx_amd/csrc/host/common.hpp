@@ -35,7 +35,7 @@ void clear_error();
     } while (0)
 
 enum KernelId : int {
-    K_DEQUANT_Q4_0, K_DEQUANT_Q8_0, K_DEQUANT_Q4_K, K_DEQUANT_Q6_K, K_DEQUANT_Q5_K, K_DEQUANT_Q8_K,
+    K_DEQUANT_Q4_0, K_DEQUANT_Q8_0, K_DEQUANT_Q4_K, K_DEQUANT_Q6_K, K_DEQUANT_Q5_K, K_DEQUANT_Q8_K, K_DEQUANT_Q2_K,
     K_FQ_COL_ABSMAX, K_FQ_SEG_ABSMAX, K_FQ_FLAT_ABSMAX, K_FQ_SCALE, K_FQ_SCALE_PARTS, K_FQ_COL_APPLY, K_FQ_COL_APPLY_IMG, K_FQ_FLAT_APPLY, K_FQ_FLAT4_APPLY,
     K_FILL_U32, K_COPY_U128,
     // decode GEMV: per scheme {r2, r4, r2_argmax, r2_paired, r4_paired, r2_norm, r4_norm, r2_norm_paired, r4_norm_paired,
@@ -54,12 +54,14 @@ enum KernelId : int {
     K_GEMV_Q5_K_R2_NORM, K_GEMV_Q5_K_R4_NORM, K_GEMV_Q5_K_R2_NORM_PAIRED, K_GEMV_Q5_K_R4_NORM_PAIRED, K_GEMV_Q5_K_R2_NORM_ARGMAX,
     K_GEMV_Q8_K_R2, K_GEMV_Q8_K_R4, K_GEMV_Q8_K_R2_ARGMAX, K_GEMV_Q8_K_R2_PAIRED, K_GEMV_Q8_K_R4_PAIRED,
     K_GEMV_Q8_K_R2_NORM, K_GEMV_Q8_K_R4_NORM, K_GEMV_Q8_K_R2_NORM_PAIRED, K_GEMV_Q8_K_R4_NORM_PAIRED, K_GEMV_Q8_K_R2_NORM_ARGMAX,
+    K_GEMV_Q2_K_R2, K_GEMV_Q2_K_R4, K_GEMV_Q2_K_R2_ARGMAX, K_GEMV_Q2_K_R2_PAIRED, K_GEMV_Q2_K_R4_PAIRED,
+    K_GEMV_Q2_K_R2_NORM, K_GEMV_Q2_K_R4_NORM, K_GEMV_Q2_K_R2_NORM_PAIRED, K_GEMV_Q2_K_R4_NORM_PAIRED, K_GEMV_Q2_K_R2_NORM_ARGMAX,
     K_GEMV_Q4_0_U2_R2, K_GEMV_Q4_0_U2_R4, K_GEMV_Q4_0_U2_R2_ARGMAX, K_GEMV_Q4_0_U2_R2_PAIRED, K_GEMV_Q4_0_U2_R4_PAIRED,
     K_GEMV_Q4_0_U2_R2_NORM, K_GEMV_Q4_0_U2_R4_NORM, K_GEMV_Q4_0_U2_R2_NORM_PAIRED, K_GEMV_Q4_0_U2_R4_NORM_PAIRED, K_GEMV_Q4_0_U2_R2_NORM_ARGMAX,
-    K_GEMV_Q4_0_G2, K_GEMV_Q8_0_G2, K_GEMV_Q4_K_G2, K_GEMV_F16W_G2, K_GEMV_Q6_K_G2, K_GEMV_Q5_K_G2, K_GEMV_Q8_K_G2,
+    K_GEMV_Q4_0_G2, K_GEMV_Q8_0_G2, K_GEMV_Q4_K_G2, K_GEMV_F16W_G2, K_GEMV_Q6_K_G2, K_GEMV_Q5_K_G2, K_GEMV_Q8_K_G2, K_GEMV_Q2_K_G2,
     K_GEMM_Q4_K, K_GEMM_Q4_0, K_GEMM_Q8_0, K_GEMM64_Q4_K, K_GEMM64_Q4_0, K_GEMM64_Q8_0, K_GEMM_F16W, K_GEMM64_F16W, K_GEMM_Q6_K, K_GEMM64_Q6_K, K_GEMM_Q5_K, K_GEMM64_Q5_K, K_XPREP, K_XROWSCALE, K_ARGMAX_FINISH, K_TOPK_SELECT, K_RMSNORM_ROWS, K_SWIGLU_ROWS,
     K_GEMM64G_Q4_K, K_GEMM64G_Q4_0, K_GEMM64G_Q8_0, K_GEMM64G_Q5_K, K_GEMM64G_Q6_K, K_GEMM64G_F16W, K_MOE_SORT,
-    K_GEMM_Q8_K, K_GEMM64_Q8_K, K_GEMM64G_Q8_K,
+    K_GEMM_Q8_K, K_GEMM64_Q8_K, K_GEMM64G_Q8_K, K_GEMM_Q2_K, K_GEMM64_Q2_K, K_GEMM64G_Q2_K,
     K_COUNT
 };
 

@@ -525,7 +525,7 @@ static std::unique_ptr<rlx_exec> plan_graph(const rlx_graph_desc *g, const rlx_c
                 for (uint32_t t = 0; t < o.d.n_inputs; t++) {
                     if (o.d.inputs[t] != f) continue;
                     const bool as_x = o.d.op_kind == RLX_OP_DEQUANT_MATMUL && t == 0 && o.m > 16 && o.k == fq.chan_dim &&
-                                      o.d.scheme != SCHEME_Q4K && o.d.scheme != SCHEME_Q5K;
+                                      act_sums_kind((int)o.d.scheme) == 0;
                     if (!as_x) {
                         other_reader = true;
                     } else if (target >= 0 && step_idx[j] != target) {

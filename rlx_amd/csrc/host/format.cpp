@@ -185,6 +185,28 @@ int repack_host(int scheme, uint32_t flags, const uint8_t *src, size_t nbytes, i
                         uint8_t *dst = unit + (j >> 1) * 1024 + l * 16 + (j & 1) * 8;
                         for (int e = 0; e < 8; e++) dst[e] = live ? (uint8_t)(b[4 + 32 * j + 8 * g + e] ^ 0x80u) : 0x80u;
                     }
+                } else if (scheme == SCHEME_Q2K) {  // one super-block per unit: 2-bit codes, 16 scale bytes, d and dmin
+                    // the reference's field order (lib.rs:857-886): d, dmin, 16 scale bytes, 64 bytes of codes
+                    const bool live = r < n && u < bpr;
+                    const uint8_t *b = live ? src + (r * bpr + u) * L.block_bytes : nullptr;
+                    if (g == 0) {
+                        if (live) {
+                            memcpy(unit + 1024 + nrow * 16, b + 4, 16);
+                            memcpy(unit + 1280 + nrow * 4, b, 4);
+                        } else {
+                            memset(unit + 1024 + nrow * 16, 0, 16);
+                            memset(unit + 1280 + nrow * 4, 0, 4);
+                        }
+                    }
+                    uint32_t words[4] = {0, 0, 0, 0};
+                    for (int j = 0; live && j < 8; j++)
+                        for (int e = 0; e < 8; e++) {
+                            const int i = 32 * j + 8 * g + e;  // element of the super-block
+                            const int h = i >> 7, pair = (i >> 5) & 3, l5 = i & 31;
+                            const uint32_t code = (uint32_t)(b[20 + 32 * h + l5] >> (2 * pair)) & 3u;
+                            words[j >> 1] |= code << (16 * (e & 1) + 8 * (j & 1) + 2 * (e >> 1));
+                        }
+                    memcpy(unit + l * 16, words, 16);
                 } else if (scheme == SCHEME_Q5K) {  // one super-block per unit: nibbles as Q4_K, fifth-bit words, 16 meta bytes
                     const bool live = r < n && u < bpr;
                     const uint8_t *b = live ? src + (r * bpr + u) * L.block_bytes : nullptr;

@@ -100,6 +100,7 @@ struct XPrepArgs {
     float *rowfac;
     const int *perm;
     int perm_len;
+    int sums16;
 };
 constexpr int MOE_MAX_EXPERTS = 256;
 struct MoeSortArgs {  // mirrors kernels/moe.hip
@@ -154,7 +155,7 @@ static int launch_gemv(const void *const *xs, int xk, const rlx_qweight *const *
     // kernel = scheme family x {r2, r4, r2_argmax, r2_paired, r4_paired}
     const int family = wide ? K_GEMV_F16W_R2 : scheme == SCHEME_Q4_0 ? K_GEMV_Q4_0_R2 : scheme == SCHEME_Q8_0 ? K_GEMV_Q8_0_R2
                        : scheme == SCHEME_Q6K ? K_GEMV_Q6_K_R2 : scheme == SCHEME_Q5K ? K_GEMV_Q5_K_R2
-                       : scheme == SCHEME_Q8K ? K_GEMV_Q8_K_R2 : K_GEMV_Q4_K_R2;
+                       : scheme == SCHEME_Q8K ? K_GEMV_Q8_K_R2 : scheme == SCHEME_Q2K ? K_GEMV_Q2_K_R2 : K_GEMV_Q4_K_R2;
     if (argmax_key && !r2) {
         set_error("gemv: the argmax epilogue takes one activation row");
         return RLX_ERR_INVALID;
@@ -306,7 +307,8 @@ static int launch_gemv(const void *const *xs, int xk, const rlx_qweight *const *
 
 struct GemmPlan {
     int64_t m_rows, k_pad;
-    size_t xh_bytes, sxh_bytes, fac_bytes;  // the image, the Q4_K / Q5_K block sums, the per-row prescale factors
+    size_t xh_bytes, sxh_bytes, fac_bytes;  // the image, the block sums (Q4_K / Q5_K per 32 columns, Q2_K per 16), the per-row prescale factors
+    int sums_kind;                          // act_sums_kind of the scheme the plan was made for
     size_t total() const { return xh_bytes + sxh_bytes + fac_bytes; }
 };
 static GemmPlan gemm_plan(int scheme, int xk, int64_t m, int64_t k) {
@@ -315,7 +317,8 @@ static GemmPlan gemm_plan(int scheme, int xk, int64_t m, int64_t k) {
     p.m_rows = (rv + 255) / 256 * 256;
     p.k_pad = (k + 255) / 256 * 256;
     p.xh_bytes = ((size_t)p.m_rows * p.k_pad * 2 + 255) & ~(size_t)255;
-    p.sxh_bytes = (scheme == SCHEME_Q4K || scheme == SCHEME_Q5K) ? (size_t)p.m_rows * (p.k_pad / 256) * 32 : 0;
+    p.sums_kind = act_sums_kind(scheme);
+    p.sxh_bytes = (size_t)p.m_rows * (p.k_pad / 256) * 32 * p.sums_kind;  // 16 or 32 halfs per row and super-block
     p.fac_bytes = ((size_t)m * 8 + 255) & ~(size_t)255;
     return p;
 }
@@ -327,7 +330,7 @@ static int launch_xprep(const void *x, int xk, int64_t m, int64_t k, const GemmP
     float *fac = (float *)workspace;
     void *xh = (uint8_t *)workspace + p.fac_bytes;
     void *sxh = p.sxh_bytes ? (uint8_t *)workspace + p.fac_bytes + p.xh_bytes : nullptr;
-    XPrepArgs xa{x, xh, sxh, (int)m, (int)k, (int)p.k_pad, (int)p.m_rows, xk, fac, perm, perm_len};
+    XPrepArgs xa{x, xh, sxh, (int)m, (int)k, (int)p.k_pad, (int)p.m_rows, xk, fac, perm, perm_len, p.sums_kind == 2};
     void *xparams[] = {&xa};
     RLX_TRY(launch(K_XROWSCALE, (unsigned)((m + 3) / 4), 1, 256, 0, stream, xparams));
     const long long xblocks = (p.m_rows / 256) * (p.k_pad / 64) * 8;  // (tile, step, 32-row sub-tile)
@@ -412,6 +415,7 @@ static int launch_gemm(const void *x, int xk, const rlx_qweight *const *ws, floa
                   : w->scheme == SCHEME_Q6K     ? (skinny ? K_GEMM64_Q6_K : K_GEMM_Q6_K)
                   : w->scheme == SCHEME_Q5K     ? (skinny ? K_GEMM64_Q5_K : K_GEMM_Q5_K)
                   : w->scheme == SCHEME_Q8K     ? (skinny ? K_GEMM64_Q8_K : K_GEMM_Q8_K)
+                  : w->scheme == SCHEME_Q2K     ? (skinny ? K_GEMM64_Q2_K : K_GEMM_Q2_K)
                                                 : (skinny ? K_GEMM64_Q8_0 : K_GEMM_Q8_0);
     RLX_TRY(runtime_init());
     RLX_TRY(launch3(id, (unsigned)gx, (unsigned)gy, (unsigned)split, 512, skinny ? 3 * 24 * 1024 : 3 * 48 * 1024, stream, params));
@@ -537,7 +541,7 @@ int rlx_mi355x_dequant(const rlx_qweight *w, float *out_dev, void *stream) {
     void *params[] = {&a};
     KernelId id = w->scheme == SCHEME_Q4_0 ? K_DEQUANT_Q4_0 : w->scheme == SCHEME_Q8_0 ? K_DEQUANT_Q8_0
                   : w->scheme == SCHEME_Q6K ? K_DEQUANT_Q6_K : w->scheme == SCHEME_Q5K ? K_DEQUANT_Q5_K
-                  : w->scheme == SCHEME_Q8K ? K_DEQUANT_Q8_K : K_DEQUANT_Q4_K;
+                  : w->scheme == SCHEME_Q8K ? K_DEQUANT_Q8_K : w->scheme == SCHEME_Q2K ? K_DEQUANT_Q2_K : K_DEQUANT_Q4_K;
     return launch(id, (unsigned)w->dims.units, (unsigned)w->dims.row_tiles, 64, 0, (hipStream_t)stream, params);
 }
 
@@ -576,18 +580,19 @@ int rlx_mi355x_gguf_matmul_bt_batch(const void *const *xs_dev, int x_dtype, cons
     const size_t esz = xk == 0 ? 4 : 2;
     if (m > cap) {  // prefill: one GEMM per weight, sharing the workspace (same stream, so launches are ordered)
         // q, k, v (and gate, up) of a layer share their input: its f16 image in the workspace is made once. An image
-        // with block sums (Q4_K / Q5_K) also serves a scheme that does not read them, not the other way round.
+        // with block sums (Q4_K / Q5_K: per 32 columns; Q2_K: per 16) also serves a scheme that reads none, not the
+        // other way round, and not a scheme that reads the other kind.
         // Consecutive matrices with the same input and K go into one launch, up to GEMM_MAX_SEG at a time.
         const void *have_x = nullptr;
         int64_t have_k = -1;
-        bool have_sums = false;
+        int have_sums = 0;
         for (int i = 0; i < count;) {
             int c = 1;
             while (i + c < count && c < GEMM_MAX_SEG && xs_dev[i + c] == xs_dev[i] && ws[i + c]->dims.k == ws[i]->dims.k &&
                    ws[i + c]->layout.unit_bytes == ws[i]->layout.unit_bytes && ws[i + c]->sc_off() == ws[i]->sc_off())
                 c++;
-            const bool sums = gemm_plan(ws[i]->scheme, xk, m, ws[i]->dims.k).sxh_bytes != 0;
-            const bool prepared = xs_dev[i] == have_x && ws[i]->dims.k == have_k && (have_sums || !sums);
+            const int sums = act_sums_kind(ws[i]->scheme);
+            const bool prepared = xs_dev[i] == have_x && ws[i]->dims.k == have_k && (sums == 0 || sums == have_sums);
             RLX_TRY(launch_gemm(xs_dev[i], xk, ws + i, outs_dev + i, c, m, workspace, workspace_bytes, (hipStream_t)stream, prepared));
             if (!prepared) {
                 have_x = xs_dev[i];
@@ -1050,6 +1055,7 @@ int rlx_mi355x_gguf_grouped_matmul_bt_ws(const void *x_dev, int x_dtype, const r
                         : w->scheme == SCHEME_Q6K  ? K_GEMM64G_Q6_K
                         : w->scheme == SCHEME_Q5K  ? K_GEMM64G_Q5_K
                         : w->scheme == SCHEME_Q8K  ? K_GEMM64G_Q8_K
+                        : w->scheme == SCHEME_Q2K  ? K_GEMM64G_Q2_K
                                                    : K_GEMM64G_Q8_0;
     const unsigned gx = (unsigned)((w->dims.row_tiles * 16 + 127) / 128), gy = (unsigned)(p.perm_len / p.group);
     return launch3(id, gx, gy, 1, 512, 3 * 24 * 1024, s, params);

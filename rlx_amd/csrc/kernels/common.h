@@ -157,6 +157,20 @@ __device__ __forceinline__ void unpack_q6_scaled(uint32_t w, uint32_t hx, half2_
     f.h2[3] = __builtin_elementwise_fma(as_half2(a3), sc16, neg96);
 }
 
+// Q2_K: byte BYTE (0 / 1) of each 16-bit half of `w` holds four 2-bit codes at bits 0-1, 2-3, 4-5, 6-7; element pair i of
+// the fragment is (low half, high half) at bits 2 i of that byte. ((w >> s) & 0x00030003) | magic is 1024 + q, and one fma
+// with sc and -1024 sc turns it into sc * q (sc <= 15, q <= 3: exact integers, rounded once from an exact value).
+template <int BYTE>
+__device__ __forceinline__ void unpack_q2_scaled(uint32_t w, half2_t sc, Frag &f) {
+    const half2_t m1024 = {(half_t)(-1024.0f), (half_t)(-1024.0f)};
+    const half2_t nsc = sc * m1024;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const uint32_t x = (8 * BYTE + 2 * i) ? (w >> (8 * BYTE + 2 * i)) : w;
+        f.h2[i] = __builtin_elementwise_fma(as_half2(and_or(x, 0x00030003u, MAGIC)), sc, nsc);
+    }
+}
+
 // half2 splat of the integer byte b (0..255), exact: bytes [b, 0x64, b, 0x64] = 1024 + b, minus 1024
 __device__ __forceinline__ half2_t splat_ubyte_half(uint32_t b) {
     const half2_t k1024 = {(half_t)1024.0f, (half_t)1024.0f};

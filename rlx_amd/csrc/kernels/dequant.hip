@@ -79,6 +79,25 @@ __device__ __forceinline__ void dequant_tile(const DequantArgs &a) {
                 store8(a.out, a.n, a.k, r, u * 256 + (2 * h + tt) * 32 + g * 8, v);
             }
         }
+    } else if constexpr (SCHEME == SCHEME_Q2K) {  // (d * sc) * q - dmin * m per 16-column sub-block (rlx-gguf/src/lib.rs:857-886)
+        const uint4_t q = *(const uint4_t *)(unit + l * 16);
+        const uint4_t scales = *(const uint4_t *)(unit + 1024 + nrow * 16);
+        const uint32_t dd = *(const uint32_t *)(unit + 1280 + nrow * 4);
+        const float d = half_bits_to_float(dd & 0xFFFFu), dmin = half_bits_to_float(dd >> 16);
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const int si = 2 * j + (g >> 1);
+            const uint32_t sb = (scales[si >> 2] >> (8 * (si & 3))) & 0xFFu;
+            const float dl = d * (float)(sb & 0xFu), ml = dmin * (float)(sb >> 4);
+            float v[8];
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const uint32_t code = (q[j >> 1] >> (16 * (e & 1) + 8 * (j & 1) + 2 * (e >> 1))) & 3u;
+                const float prod = dl * (float)code;
+                v[e] = prod - ml;
+            }
+            store8(a.out, a.n, a.k, r, u * 256 + j * 32 + g * 8, v);
+        }
     } else if constexpr (SCHEME == SCHEME_Q6K) {
         // (d * sc) * (q - 32): the block decoder the reference's matmul calls reads the scale bytes as unsigned
         // (rlx-gguf/src/lib.rs:819-845), its tensor decoder and ggml as signed (lib.rs:1070-1112); a.sc_off picks
@@ -142,3 +161,4 @@ extern "C" __global__ __launch_bounds__(64) void rlx_dequant_q4_k(rlx::DequantAr
 extern "C" __global__ __launch_bounds__(64) void rlx_dequant_q5_k(rlx::DequantArgs a) { rlx::dequant_tile<rlx::SCHEME_Q5K>(a); }
 extern "C" __global__ __launch_bounds__(64) void rlx_dequant_q6_k(rlx::DequantArgs a) { rlx::dequant_tile<rlx::SCHEME_Q6K>(a); }
 extern "C" __global__ __launch_bounds__(64) void rlx_dequant_q8_k(rlx::DequantArgs a) { rlx::dequant_tile<rlx::SCHEME_Q8K>(a); }
+extern "C" __global__ __launch_bounds__(64) void rlx_dequant_q2_k(rlx::DequantArgs a) { rlx::dequant_tile<rlx::SCHEME_Q2K>(a); }

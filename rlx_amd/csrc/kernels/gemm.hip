@@ -84,10 +84,11 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
     constexpr bool K4 = SCHEME == SCHEME_Q4K || K5;
     constexpr bool K6 = SCHEME == SCHEME_Q6K;
     constexpr bool K8 = SCHEME == SCHEME_Q8K;                 // exact int8 codes in B, the super-block's f32 d applied like Q6_K's
+    constexpr bool K2 = SCHEME == SCHEME_Q2K;                 // B = sc * q per 16-column sub-block like Q6_K, a dmin term like Q4_K's over 16 sub-blocks
     constexpr int META_OFF = K5 ? 2560 : 2048;                // the 16 meta bytes per row of a Q4_K / Q5_K unit
     // Super-block schemes: B holds integers (Q4_K: sc * q, exact; Q6_K: sc * (q - 32), exact up to 2048), a second
     // accumulator set collects one 256-column super-block and d (Q4_K: and dmin) is applied in f32 per super-block.
-    constexpr bool SB = K4 || K6 || K8;
+    constexpr bool SB = K4 || K6 || K8 || K2;
     constexpr int WN = GEMM_NT / (32 * TJ), WM = 8 / WN, MT = WM * TI * 32;  // wave grid and rows per workgroup
     constexpr int NSA = MT / 32, SA = 4 * NSA * 1024, ST = SA + GEMM_STAGE_B;  // LDS stage: activations [4][NSA][1 KB], then weights
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -172,6 +173,12 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
                 b_hw[(q >> 1) & 1] = __builtin_amdgcn_raw_buffer_load_b64(b_rsrc, lane * 16 + (q >> 1) * 8, unit + 2048, 0);
             }
             if (q == 0) b_meta[0] = ld128(b_rsrc, b_n16 * 16, unit + 3072);  // copied aside when the super-block's decode starts
+        } else if constexpr (K2) {  // the lane slot's codes of the whole super-block and the row's 16 scale bytes, once per super-block
+            if (q == 0) {
+                const int unit = (step >> 2) * L.unit_bytes;
+                b_q[0] = ld128(b_rsrc, lane * 16, unit);
+                b_meta[0] = ld128(b_rsrc, b_n16 * 16, unit + 1024);
+            }
         } else if constexpr (K8) {  // one quarter of the super-block (two 32-column blocks) per step
             b_q[q & 1] = ld128(b_rsrc, lane * 16, (step >> 2) * L.unit_bytes + q * 1024);
         } else if constexpr (SCHEME == SCHEME_F16W) {  // two ready-made fragments per lane and step: b_q and b_meta hold them
@@ -228,6 +235,17 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
             // block 2 q + jl of the super-block, this lane's 16-column half of it: scale byte 4 q + 2 jl + g / 2
             const uint32_t scb = (b_meta[1][q] >> (16 * jl + 8 * (b_g >> 1))) & 0xFFu;
             unpack_q6_scaled(b_q[cp][t], hx, splat_ubyte_half(scb, sc_bias), f);
+        } else if constexpr (K2) {
+            // The registers are used in place: the fetch of the next super-block is issued after the last block of this
+            // one has been decoded (either wave group: data of phase 3, then the fetch of phase 0, then data of phase 0).
+            if (q == 0 && jl == 0) {
+#pragma unroll
+                for (int e = 0; e < 4; e++) b_meta[0][e] &= b_keep;  // a dead tile decodes to zeros
+            }
+            // block 2 q + jl of the super-block, this lane's 16-column half of it: scale byte 4 q + 2 jl + g / 2
+            const uint32_t scb = (b_meta[0][q] >> (16 * jl + 8 * (b_g >> 1))) & 0x0Fu;
+            if (jl) unpack_q2_scaled<1>(b_q[0][q], splat_ubyte_half(scb), f);
+            else unpack_q2_scaled<0>(b_q[0][q], splat_ubyte_half(scb), f);
         } else if constexpr (K8) {
             unpack_q8(b_q[q & 1][2 * jl], b_q[q & 1][2 * jl + 1], f);
 #pragma unroll
@@ -267,10 +285,13 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
         my_row[j] = n_tile0 + (wn * TJ + j) * 32 + lr;
         my_ok[j] = (my_row[j] >> 4) < sg.row_tiles;
         my_meta[j] = w_base + (long long)(my_ok[j] ? (my_row[j] >> 4) : 0) * a.units * L.unit_bytes +
-                     (K8 ? 4096 + (my_row[j] & 15) * 4 : K6 ? 3328 + (my_row[j] & 15) * 2 : META_OFF + (my_row[j] & 15) * 16);  // Q8_K / Q6_K: the row's d; Q4_K / Q5_K: its 16 meta bytes
+                     (K8 ? 4096 + (my_row[j] & 15) * 4 : K6 ? 3328 + (my_row[j] & 15) * 2 : K2 ? 1024 + (my_row[j] & 15) * 16
+                                                                                        : META_OFF + (my_row[j] & 15) * 16);  // Q8_K / Q6_K: the row's d; Q4_K / Q5_K: its 16 meta bytes; Q2_K: its 16 scale bytes (d, dmin behind the tile's)
     }
     uint4_t w_meta[TJ];
+    uint32_t w_dd[TJ];   // Q2_K: the row's d and dmin
     Frag fs[TI];
+    int sb_now = 0;      // Q2_K: the super-block load_sb_meta was last called for
 #pragma unroll
     for (int j = 0; j < TJ; j++) w_meta[j] = uint4_t{0, 0, 0, 0};
     int a_rd[4], b_rd[4];  // per k-slice read offsets of this lane; + sub-tile * 1024
@@ -306,6 +327,24 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
             for (int j = 0; j < TJ; j++) w_meta[j][0] = *(const uint32_t *)(my_meta[j] + (long long)sb * L.unit_bytes);
             return;
         }
+        if constexpr (K2) {
+#pragma unroll
+            for (int j = 0; j < TJ; j++) {
+                // the eight scale bytes of sub-blocks 8 lh .. 8 lh + 7; 16 rows of 16 scale bytes, then 16 rows of (d, dmin):
+                // 256 - 12 (row & 15) bytes further on
+                const uint2_t sc8 = *(const uint2_t *)(my_meta[j] + (long long)sb * L.unit_bytes + lh * 8);
+                w_meta[j][0] = sc8[0];
+                w_meta[j][1] = sc8[1];
+                w_dd[j] = *(const uint32_t *)(my_meta[j] + (long long)sb * L.unit_bytes + 256 - 12 * (my_row[j] & 15));
+            }
+#pragma unroll
+            for (int i = 0; i < TI; i++) {  // sxh[row][super-block][32]: sixteen leading halves, sixteen residuals
+                long long row = m_tile0 + (wm * TI + i) * 32 + lr;
+                fs[i].u4 = *(const uint4_t *)(a.sxh + (row * (a.k_pad / 256) + sb) * 32 + lh * 8);
+            }
+            sb_now = sb;
+            return;
+        }
 #pragma unroll
         for (int j = 0; j < TJ; j++) w_meta[j] = *(const uint4_t *)(my_meta[j] + (long long)sb * L.unit_bytes);
 #pragma unroll
@@ -323,6 +362,43 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
                 for (int i = 0; i < TI; i++)
 #pragma unroll
                     for (int e = 0; e < 16; e++) total[i][j][e] = __builtin_fmaf(d, part[i][j][e], total[i][j][e]);
+            }
+            return;
+        }
+        if constexpr (K2) {  // total += d * P - dmin * (m . sx) over the sixteen sub-blocks: two matrix instructions of 16 k-slots
+            const half2_t k1024 = {(half_t)1024.0f, (half_t)1024.0f};
+            const half2_t lo_scale = {(half_t)(1.0f / GEMM_LO_SCALE), (half_t)(1.0f / GEMM_LO_SCALE)};
+            Frag fs_lo[TI];  // the residual halves of the sixteen sub-block sums (fs holds the leading halves)
+#pragma unroll
+            for (int j = 0; j < TJ; j++) {
+                const float d = my_ok[j] ? half_bits_to_float(w_dd[j] & 0xFFFFu) : 0.f;
+                const float dmin = my_ok[j] ? half_bits_to_float(w_dd[j] >> 16) : 0.f;
+                // B' fragment: k-slot 8 lh + e = min of sub-block 8 lh + e (the high nibble of its scale byte)
+                Frag fm, fm_lo;
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const uint32_t src = (w_meta[j][e >> 1] >> 4) & 0x0F0F0F0Fu;
+                    const uint32_t sel = (e & 1) ? 0x04030402u : 0x04010400u;  // bytes (2,3) or (0,1) -> [b,0x64,b',0x64]
+                    const half2_t v = as_half2(__builtin_amdgcn_perm(0x64646464u, src, sel)) - k1024;
+                    fm.h2[e] = v;
+                    fm_lo.h2[e] = v * lo_scale;
+                }
+#pragma unroll
+                for (int i = 0; i < TI; i++) {
+                    if (j == 0) {  // the residual halves are fetched here, not held since load_sb_meta: the d * P below covers the wait
+                        long long row = m_tile0 + (wm * TI + i) * 32 + lr;
+                        fs_lo[i].u4 = *(const uint4_t *)(a.sxh + (row * (a.k_pad / 256) + sb_now) * 32 + 16 + lh * 8);
+                    }
+#pragma unroll
+                    for (int e = 0; e < 16; e++) total[i][j][e] = __builtin_fmaf(d, part[i][j][e], total[i][j][e]);
+                }
+#pragma unroll
+                for (int i = 0; i < TI; i++) {
+                    float16_t qq = mfma32(fs[i], fm, zero16);
+                    qq = mfma32(fs_lo[i], fm_lo, qq);
+#pragma unroll
+                    for (int e = 0; e < 16; e++) total[i][j][e] = __builtin_fmaf(-dmin, qq[e], total[i][j][e]);
+                }
             }
             return;
         }
@@ -543,6 +619,7 @@ struct XPrepArgs {
     float *rowfac;  // [m][2] (forward factor, its inverse), written by rlx_xrowscale before rlx_xprep runs
     const int *perm;  // expert-sorted image: row i of the image is row perm[i] of x (-1: a padding row of zeros); else null
     int perm_len;
+    int sums16;       // sxh holds the sums of 16-column sub-blocks (Q2_K): sxh[row][k_pad / 256][32], leading halves then residuals
 };
 
 // Activations travel as binary16, and so do the sums of 32 of them that the Q4_K / Q5_K min term needs. rlx_xrowscale
@@ -658,7 +735,18 @@ __device__ __forceinline__ void xprep_body(const XPrepArgs &a) {
         sum += __shfl_xor(sum, 33);  // the slot holding the other 8 columns of this row's k-slice
         if (h == 0) part[ks][r] = sum;
         __syncthreads();
-        if (threadIdx.x < 64) {  // (row, 32-column block of the step) -> hi + lo*2048 halfs
+        if (a.sums16) {
+            if (threadIdx.x < 128) {  // (row, 16-column sub-block of the step) -> hi + lo*2048 halfs
+                const int rr = threadIdx.x & 31, sub16 = threadIdx.x >> 5;
+                const float s16 = part[sub16][rr];
+                const half_t hi = (half_t)s16;
+                const half_t lo = (half_t)((s16 - (float)hi) * GEMM_LO_SCALE);
+                const long long row = (long long)tile * GEMM_MT + sub * 32 + rr;
+                half_t *d = a.sxh + (row * (a.k_pad / 256) + (step >> 2)) * 32 + (step & 3) * 4 + sub16;
+                d[0] = hi;
+                d[16] = lo;
+            }
+        } else if (threadIdx.x < 64) {  // (row, 32-column block of the step) -> hi + lo*2048 halfs
             const int rr = threadIdx.x & 31, blk = threadIdx.x >> 5;
             const float s32 = part[2 * blk][rr] + part[2 * blk + 1][rr];
             const half_t hi = (half_t)s32;
@@ -678,6 +766,9 @@ extern "C" __global__ __launch_bounds__(512) void rlx_gemm_q4_0(rlx::GemmArgs a)
 extern "C" __global__ __launch_bounds__(512) void rlx_gemm_q8_0(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q8_0, 2, 2>(a); }
 extern "C" __global__ __launch_bounds__(512) void rlx_gemm_q5_k(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q5K, 2, 2>(a); }
 extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64_q5_k(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q5K, 1, 1>(a); }
+extern "C" __global__ __launch_bounds__(512) void rlx_gemm_q2_k(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q2K, 2, 2>(a); }
+extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64_q2_k(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q2K, 1, 1>(a); }
+extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64g_q2_k(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q2K, 1, 1, true>(a); }
 extern "C" __global__ __launch_bounds__(512) void rlx_gemm_q6_k(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q6K, 2, 2>(a); }
 extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64_q6_k(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q6K, 1, 1>(a); }
 extern "C" __global__ __launch_bounds__(512) void rlx_gemm_q8_k(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q8K, 2, 2>(a); }

@@ -174,6 +174,21 @@ struct UnitRegs<SCHEME_Q8K> {  // one super-block: four quarters of offset-binar
 };
 
 template <>
+struct UnitRegs<SCHEME_Q2K> {  // one super-block: the lane slot's 64 two-bit codes, the row's 16 scale bytes, d and dmin
+    uint4_t q, sc;
+    uint32_t dd;
+    __device__ __forceinline__ void load(const uint8_t *unit, int l, int nrow, bool) {
+        q = __builtin_nontemporal_load((const uint4_t *)(unit + l * 16));
+        sc = __builtin_nontemporal_load((const uint4_t *)(unit + 1024 + nrow * 16));
+        dd = __builtin_nontemporal_load((const uint32_t *)(unit + 1280 + nrow * 4));
+    }
+    __device__ __forceinline__ void clear() {
+        q = sc = uint4_t{0, 0, 0, 0};
+        dd = 0;
+    }
+};
+
+template <>
 struct UnitRegs<SCHEME_F16W> {  // weights already stored as binary16 fragments: four 32-column blocks, no scales
     uint4_t q[4];
     __device__ __forceinline__ void load(const uint8_t *unit, int l, int, bool) {
@@ -294,6 +309,46 @@ __device__ __forceinline__ void compute_unit(const UnitRegs<SCHEME> &w, const ha
         for (int rg = 0; rg < RG; rg++)
 #pragma unroll
             for (int r = 0; r < NREG; r++) acc[rg][r] = __builtin_fmaf(d, sum[rg][r], acc[rg][r]);
+    } else if constexpr (SCHEME == SCHEME_Q2K) {
+        // Two products per super-block, both of exact binary16 integers: P with B = sc * q (the 16-column scale folded into
+        // the fragment, as for Q6_K) and Q with B = m, the sub-block's min in all eight places, so that the matrix unit
+        // forms the sum of m times the activations of the sub-block; then acc += d * P - dmin * Q.
+        float4_t sum[RG], smin[RG];
+#pragma unroll
+        for (int rg = 0; rg < RG; rg++) sum[rg] = smin[rg] = zero;
+        const int gshift = 8 * (g >> 1);  // this lane's half of each 32-column block: scale byte 2 j or 2 j + 1
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            if constexpr (RG == 1) load_afrags<4>(xrow[0], live[0], ucol + h * 128, a);
+            Frag b[4], bm[4];
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                const uint32_t scb = (w.sc[2 * h + (t >> 1)] >> (16 * (t & 1) + gshift)) & 0xFFu;
+                const uint32_t wq = w.q[2 * h + (t >> 1)];
+                if (t & 1) unpack_q2_scaled<1>(wq, splat_ubyte_half(scb & 0xFu), b[t]);
+                else unpack_q2_scaled<0>(wq, splat_ubyte_half(scb & 0xFu), b[t]);
+                const half2_t m2 = splat_ubyte_half(scb >> 4);
+#pragma unroll
+                for (int e = 0; e < 4; e++) bm[t].h2[e] = m2;
+            }
+#pragma unroll
+            for (int rg = 0; rg < RG; rg++) {
+                if constexpr (RG > 1) load_afrags<4>(xrow[rg], live[rg], ucol + h * 128, a);
+#pragma unroll
+                for (int t = 0; t < 4; t++) {
+                    sum[rg] = mfma16(a[t], b[t], sum[rg]);
+                    smin[rg] = mfma16(a[t], bm[t], smin[rg]);
+                }
+            }
+        }
+        const float d = half_bits_to_float(w.dd & 0xFFFFu), dmin = half_bits_to_float(w.dd >> 16);
+#pragma unroll
+        for (int rg = 0; rg < RG; rg++)
+#pragma unroll
+            for (int r = 0; r < NREG; r++) {
+                acc[rg][r] = __builtin_fmaf(d, sum[rg][r], acc[rg][r]);
+                acc[rg][r] = __builtin_fmaf(-dmin, smin[rg][r], acc[rg][r]);
+            }
     } else if constexpr (SCHEME == SCHEME_F16W) {
 #pragma unroll
         for (int rg = 0; rg < RG; rg++) {
@@ -872,6 +927,7 @@ RLX_GEMV_SCHEME(f16w, rlx::SCHEME_F16W, 2, 1)
 RLX_GEMV_SCHEME(q6_k, rlx::SCHEME_Q6K, 2, 1)
 RLX_GEMV_SCHEME(q5_k, rlx::SCHEME_Q5K, 2, 1)
 RLX_GEMV_SCHEME(q8_k, rlx::SCHEME_Q8K, 2, 1)
+RLX_GEMV_SCHEME(q2_k, rlx::SCHEME_Q2K, 3, 1)
 // Two 128-column units per loop item: taken when every K run holds an even number of units. (Measured neutral to
 // slightly slower for Q8_0, whose unit is twice the bytes, so only Q4_0 has it.)
 RLX_GEMV_SCHEME(q4_0_u2, rlx::SCHEME_Q4_0, 2, 2)
@@ -888,3 +944,4 @@ RLX_GEMV_ROWGROUPS(f16w, rlx::SCHEME_F16W, 2)
 RLX_GEMV_ROWGROUPS(q6_k, rlx::SCHEME_Q6K, 2)
 RLX_GEMV_ROWGROUPS(q5_k, rlx::SCHEME_Q5K, 2)
 RLX_GEMV_ROWGROUPS(q8_k, rlx::SCHEME_Q8K, 2)
+RLX_GEMV_ROWGROUPS(q2_k, rlx::SCHEME_Q2K, 2)

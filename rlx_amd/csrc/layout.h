@@ -38,10 +38,14 @@
 //                   XOR 0x80 as Q8_0          [4096,4160) f32 d[n] (the bsums of the GGUF block are not needed and not kept)
 //   Q3_K : Q6_K units. A super-block's values d * (scale - 32) * code (code in [-4, 3]) are those of the Q6_K super-block
 //          with 6-bit codes code + 32, scale bytes scale - 32 (stored XOR 0x80, read as byte - 128) and the same d.
-//   Q2_K ("wide" scheme): the weights are decoded once, at upload, with the reference's block
-//          decoder and stored as binary16: [0,4096) four blocks t: 16 B at 1024*t + 16*l = the 8 halfs of granule
-//          (n, 4u+t, g), already an MFMA operand fragment. No scales. 2 bytes per weight resident instead of the
-//          packed 0.33, in exchange for kernels that do no decode arithmetic at all.
+//   Q2_K : [0,1024)  16 B at 16*l = the 2-bit codes of the lane slot's 8 columns in all eight 32-column blocks of
+//                   super-block u: word w serves blocks 2w (low byte of each 16-bit half) and 2w + 1 (high byte); in a
+//                   byte the codes of elements 2i (low half) / 2i + 1 (high half) sit at bits 2i
+//          [1024,1280) per row n: the 16 scale bytes verbatim (low nibble scale, high nibble min of a 16-column sub-block)
+//          [1280,1344) per row n: f16 d, f16 dmin
+//   F16W : weights stored as binary16 operand fragments (an internal layout no GGUF scheme uses any more; the kernels
+//          that read it are the identity-decode yardstick of the benchmark): [0,4096) four blocks t: 16 B at
+//          1024*t + 16*l = the 8 halfs of granule (n, 4u+t, g). No scales.
 // Units are stored [row_tile][unit] with the unit index (K direction) fastest.
 // N is padded to a multiple of 16 and K to a multiple of UNIT_K with zero-scale blocks.
 #pragma once
@@ -85,7 +89,7 @@ RLX_HD constexpr Layout layout_of(int scheme) {
            : scheme == SCHEME_Q5K  ? Layout{256, 2816, 2560, 256, 176}
            : scheme == SCHEME_Q6K  ? Layout{256, 3360, 3072, 256, 210}
            : scheme == SCHEME_Q8K  ? Layout{256, 4160, 4096, 256, 292}
-           : scheme == SCHEME_Q2K  ? Layout{128, 4096, 4096, 256, 84}
+           : scheme == SCHEME_Q2K  ? Layout{256, 1344, 1024, 256, 84}
            : scheme == SCHEME_Q3K  ? Layout{256, 3360, 3072, 256, 110}  // rewritten as Q6_K units
            : scheme == SCHEME_F16W ? Layout{128, 4096, 4096, 0, 0}
                                    : Layout{0, 0, 0, 0, 0};
@@ -98,6 +102,9 @@ RLX_HD constexpr Layout wide_layout_of(int scheme) {
 // The scheme whose kernels read a scheme's device units. A Q3_K super-block (3-bit codes in [-4, 3], 6-bit scales minus 32,
 // one d) is rewritten at upload, exactly, as the Q6_K super-block of the same values with signed scale bytes.
 RLX_HD constexpr int kernel_scheme(int scheme) { return scheme == SCHEME_Q3K ? SCHEME_Q6K : scheme; }
+// What a scheme's prefill kernel needs next to the activation image: 0 nothing, 1 the sums of every 32-column block
+// (Q4_K / Q5_K: the dmin term), 2 the sums of every 16-column sub-block (Q2_K).
+RLX_HD constexpr int act_sums_kind(int scheme) { return (scheme == SCHEME_Q4K || scheme == SCHEME_Q5K) ? 1 : scheme == SCHEME_Q2K ? 2 : 0; }
 RLX_HD constexpr bool layout_is_f16w(const Layout &L) { return L.unit_k == 128 && L.unit_bytes == 4096; }
 
 // nibble position of fragment element e inside a granule word

@@ -2,12 +2,12 @@
 import numpy as np
 
 Q4K, Q5K, Q6K, Q8K, Q2K, Q3K, Q4_0, Q8_0 = 5, 6, 7, 8, 9, 10, 11, 12
-WIDE = (Q2K,)  # decoded at upload and stored as binary16 on the device
 SCHEME_NAMES = {Q4K: "q4_k", Q5K: "q5_k", Q6K: "q6_k", Q8K: "q8_k", Q2K: "q2_k", Q3K: "q3_k", Q4_0: "q4_0", Q8_0: "q8_0"}
 BLOCK = {Q4_0: (32, 18), Q8_0: (32, 34), Q4K: (256, 144), Q5K: (256, 176), Q6K: (256, 210), Q8K: (256, 292), Q2K: (256, 84), Q3K: (256, 110)}
 NIB_POS = [0, 4, 1, 5, 2, 6, 3, 7]
 UNIT = {Q4_0: (128, 1152, 1024), Q8_0: (128, 2176, 2048), Q4K: (256, 2304, 2048), Q5K: (256, 2816, 2560), Q6K: (256, 3360, 3072),
-        Q8K: (256, 4160, 4096), Q3K: (256, 3360, 3072)}  # Q3_K super-blocks are stored as Q6_K units with signed scale bytes
+        Q8K: (256, 4160, 4096), Q2K: (256, 1344, 1024),
+        Q3K: (256, 3360, 3072)}  # Q3_K super-blocks are stored as Q6_K units with signed scale bytes
 Q5K_HI_POS = [4, 20, 8, 24, 5, 21, 9, 25]  # fifth bit of element e in the half's word after its code word's rotate (csrc/layout.h)
 Q5K_ROT = [0, 2, 8, 10]
 Q6K_HI_POS = [4, 20, 8, 24, 6, 22, 10, 26]  # low bit of element e's 2-bit high field in the even word of a pair (csrc/layout.h)
@@ -74,6 +74,18 @@ def decode_device_layout(scheme, dev, n, k, q6k_sc_off=0):
                     code = dev[:, :, (j >> 1) * 1024 + l * 16 + (j & 1) * 8 + e].astype(np.int32) - 128
                     cols = np.arange(units) * unit_k + j * 32 + g * 8 + e
                     out[np.ix_(rows, cols)] = d * code.astype(np.float32)
+        elif scheme == Q2K:  # (d * sc) * q - dmin * m: 2-bit codes, the row's 16 scale bytes, then d and dmin
+            dd = dev[:, :, 1280 + nrow * 4: 1280 + nrow * 4 + 4].copy().view(np.float16).astype(np.float32).reshape(tiles, units, 2)
+            scales = dev[:, :, 1024 + nrow * 16: 1024 + nrow * 16 + 16]
+            words = dev[:, :, l * 16: l * 16 + 16].copy().view(np.uint32).reshape(tiles, units, 4)
+            for j in range(8):
+                sb = scales[:, :, 2 * j + (g >> 1)]
+                dl = (dd[:, :, 0] * (sb & 0xF).astype(np.float32)).astype(np.float32)
+                ml = (dd[:, :, 1] * (sb >> 4).astype(np.float32)).astype(np.float32)
+                for e in range(8):
+                    code = (words[:, :, j >> 1] >> (16 * (e & 1) + 8 * (j & 1) + 2 * (e >> 1))) & 3
+                    cols = np.arange(units) * unit_k + j * 32 + g * 8 + e
+                    out[np.ix_(rows, cols)] = ((dl * code.astype(np.float32)).astype(np.float32) - ml).astype(np.float32)
         elif scheme == Q6K:  # (d * sc) * (q - 32)
             d = dev[:, :, 3328 + nrow * 2: 3328 + nrow * 2 + 2].copy().view(np.float16).astype(np.float32).reshape(tiles, units)
             scales = dev[:, :, 3072 + nrow * 16: 3072 + nrow * 16 + 16]

@@ -1,6 +1,6 @@
 """Q5_K, Q6_K, Q8_K, Q2_K, Q3_K: the other five schemes the reference's gguf_matmul_bt dispatches
-(rlx-cpu/src/gguf_matmul.rs:25-37). Q5_K and Q6_K have packed kernels of their own (Q6_K in both readings of its scale
-bytes); the other three are decoded once at upload and kept as binary16 ("wide").
+(rlx-cpu/src/gguf_matmul.rs:25-37). All five stay packed on the device: Q5_K, Q6_K (in both readings of its scale bytes),
+Q8_K and Q2_K in layouts and kernels of their own, Q3_K rewritten exactly as Q6_K super-blocks.
 
 CPU part: pins the oracle's five block decoders (the reference's own known-answer blocks, closed-form position
 probes, reduction of Q5_K to the pinned Q4_K decoder, independent numpy bit-field decoders on random bytes), then
@@ -12,10 +12,10 @@ import pytest
 import oracle
 import rlx_amd
 from rlx_amd import DType, QuantScheme, ops
-from helpers import BLOCK, Q2K, Q3K, Q4K, Q5K, Q6K, Q8K, WIDE, decode_device_layout, random_blocks, rel_err
+from helpers import BLOCK, Q2K, Q3K, Q4K, Q5K, Q6K, Q8K, decode_device_layout, random_blocks, rel_err
 
-PACKED = (Q5K, Q6K, Q8K, Q3K)
-FIVE = WIDE + PACKED
+PACKED = (Q5K, Q6K, Q8K, Q2K, Q3K)
+FIVE = PACKED
 
 F16 = lambda v: np.frombuffer(np.float16(v).tobytes(), np.uint8)  # noqa: E731
 
@@ -214,28 +214,10 @@ def test_block_geometry():
 
 # ---- the library's host repack ------------------------------------------------------------------------------------
 
-def read_wide_layout(dev, n, k):
-    """binary16 device layout -> [n, k] f16: unit (tile, u) holds four 1 KB blocks t; lane slot l = 16 g + row holds the
-    8 halfs of columns 128 u + 32 t + 8 g .. + 7."""
-    tiles, units = (n + 15) // 16, k // 128
-    a = dev.view(np.float16).reshape(tiles, units, 4, 4, 16, 8)  # tile, unit, t, g, row, e
-    return a.transpose(0, 4, 1, 2, 3, 5).reshape(tiles * 16, k)[:n]
-
-
-@pytest.mark.parametrize("scheme", WIDE)
-def test_repack_host_is_f16_of_the_matmul_decoder(scheme):
-    n, k = 21, 768
-    blocks = random_blocks(scheme, n, k, seed=40 + scheme)
-    dev = ops.repack_host(scheme, blocks, n, k)
-    assert dev.size == ((n + 15) // 16) * (k // 128) * 4096
-    want = oracle.dequant_matmul_blocks(scheme, blocks, n * k).reshape(n, k).astype(np.float16)
-    assert np.array_equal(read_wide_layout(dev, n, k).view(np.uint16), want.view(np.uint16))
-
-
 @pytest.mark.parametrize("scheme", PACKED)
 def test_packed_layout_keeps_every_bit(scheme):
-    """The packed Q5_K / Q6_K / Q8_K device layouts (the byte count of the GGUF blocks; Q8_K without the 32 bytes of block
-    sums per super-block, which no decoder reads) and Q3_K's (its super-blocks rewritten as Q6_K super-blocks of the same
+    """The packed Q5_K / Q6_K / Q8_K / Q2_K device layouts (the byte count of the GGUF blocks; Q8_K without the 32 bytes of
+    block sums per super-block, which no decoder reads) and Q3_K's (its super-blocks rewritten as Q6_K super-blocks of the same
     values, 210 bytes each) read back with numpy by the rules of csrc/layout.h."""
     n, k = 37, 768
     blocks = random_blocks(scheme, n, k, seed=47)
@@ -258,12 +240,13 @@ def test_packed_q6k_layout_with_signed_scales():
                           oracle.dequant(Q6K, blocks, n * k).reshape(n, k).view(np.uint32))
 
 
-def test_repack_rejects_weights_beyond_binary16():
-    # Q2_K: d = 60000, every scale nibble 15, every code 3 -> 2.7e6, past what the binary16 copy of a wide scheme holds
+def test_repack_keeps_scales_of_any_magnitude():
+    # Q2_K: d = 60000, every scale nibble 15, every code 3 -> weights of 2.7e6: the packed layout keeps d as it is
     blk = np.concatenate([np.array([60000.0, 0.0], np.float16).view(np.uint8), np.full(16, 0x0F, np.uint8), np.full(64, 0xFF, np.uint8)])
-    with pytest.raises(rlx_amd.RlxError, match="binary16"):
-        ops.repack_host(Q2K, blk, 1, 256)
-    # Q8_K is packed: its f32 scale is kept as it is
+    dev = ops.repack_host(Q2K, blk, 1, 256)
+    assert dev.size == 1344
+    assert np.all(decode_device_layout(Q2K, dev, 1, 256) == np.float32(60000.0 * 15 * 3))
+    # Q8_K: the f32 scale is kept as it is
     big = np.concatenate([np.frombuffer(np.float32(1e4).tobytes(), np.uint8), np.full(256, 100, np.uint8), np.zeros(32, np.uint8)])
     assert ops.repack_host(Q8K, big, 1, 256).size == 4160
 
@@ -420,19 +403,11 @@ def test_q6k_signed_scales_through_session_and_gguf_file(tmp_path):
 
 
 @pytest.mark.gpu
-def test_wide_dequant_is_refused():
-    blocks = random_blocks(Q2K, 16, 256, seed=1)
-    qw = ops.QWeight(QuantScheme.GgufQ2K, blocks, 16, 256)
-    with pytest.raises(rlx_amd.RlxError, match="binary16"):
-        qw.dequant()
-    qw.free()
-
-
-@pytest.mark.gpu
-@pytest.mark.parametrize("scheme", [Q6K, Q5K, Q8K])
-def test_wide_grouped_matmul(scheme):
-    """Mixture-of-experts routing (rlx-cpu/src/gguf_matmul.rs:101-139) over a stack of wide-scheme slabs."""
-    k, n, experts, m = 512, 24, 4, 11
+@pytest.mark.parametrize("scheme", [Q6K, Q5K, Q8K, Q2K, Q3K])
+@pytest.mark.parametrize("m", [11, 90])  # per-token decode launches; tokens sorted by expert and one prefill launch
+def test_wide_grouped_matmul(scheme, m):
+    """Mixture-of-experts routing (rlx-cpu/src/gguf_matmul.rs:101-139) over a stack of K-quant slabs."""
+    k, n, experts = 512, 24, 4
     d_std, dmin_std = MODEL_SCALE[scheme]
     packed = np.concatenate([random_blocks(scheme, n, k, seed=100 + e, d_std=d_std, dmin_std=dmin_std) for e in range(experts)])
     rng = np.random.default_rng(3)
