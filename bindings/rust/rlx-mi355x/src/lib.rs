@@ -1,5 +1,5 @@
-//! `Device::Mi355x` backend: `Op::DequantMatMul` over GGUF weights (Q8_0 / Q4_0 / Q4_K / Q5_K / Q6_K packed in HBM;
-//! Q8_K packed without its block sums; Q2_K / Q3_K decoded at upload and resident as binary16) and `Op::FakeQuantize`,
+//! `Device::Mi355x` backend: `Op::DequantMatMul` over GGUF weights (all eight schemes packed in HBM: Q8_K without its
+//! block sums, Q3_K rewritten as Q6_K super-blocks of the same values) and `Op::FakeQuantize`,
 //! executed by hand-written gfx950 kernels in `librlx_mi355x.so`.
 //!
 //! ```ignore

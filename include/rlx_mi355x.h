@@ -47,17 +47,17 @@ typedef enum rlx_dtype {
 
 /* rlx_ir::quant::QuantScheme, declaration order (rlx-ir/src/quant.rs:39-79). The eight GGUF schemes the reference's
  * gguf_matmul_bt dispatches (rlx-cpu/src/gguf_matmul.rs:25-37) are claimed; any other value is RLX_ERR_UNSUPPORTED.
- * Q4_K, Q5_K, Q6_K, Q8_K, Q4_0 and Q8_0 stay packed in HBM (the byte count of the GGUF blocks; Q8_K without its 32 bytes
- * of block sums per super-block, which no decoder reads) and have a bit-exact device decoder. Q6_K scale bytes are read as the reference's block decoder reads them, unsigned (rlx-gguf/src/lib.rs:819-845),
- * unless the weight is created with RLX_QW_Q6K_SIGNED_SCALES (below).
- * The other two ("wide") are decoded once at upload with the reference's block decoder and kept as binary16 (2 bytes per weight):
- * matmuls only, every decoded weight must fit binary16. */
+ * All eight stay packed in HBM and have a bit-exact device decoder: Q4_K, Q5_K, Q6_K, Q2_K, Q4_0 and Q8_0 in the byte
+ * count of their GGUF blocks, Q8_K without its 32 bytes of block sums per super-block (no decoder reads them), Q3_K
+ * rewritten exactly as Q6_K super-blocks of the same values (210 bytes each). Q6_K scale bytes are read as the
+ * reference's block decoder reads them, unsigned (rlx-gguf/src/lib.rs:819-845), unless the weight is created with
+ * RLX_QW_Q6K_SIGNED_SCALES (below). */
 typedef enum rlx_quant_scheme {
     RLX_SCHEME_GGUF_Q4K = 5,  /* 256 elems / 144 bytes */
     RLX_SCHEME_GGUF_Q5K = 6,  /* 256 / 176 */
     RLX_SCHEME_GGUF_Q6K = 7,  /* 256 / 210 */
     RLX_SCHEME_GGUF_Q8K = 8,  /* 256 / 292 */
-    RLX_SCHEME_GGUF_Q2K = 9,  /* 256 / 84, wide (field order of rlx-gguf/src/lib.rs:857-886) */
+    RLX_SCHEME_GGUF_Q2K = 9,  /* 256 / 84 (field order of rlx-gguf/src/lib.rs:857-886) */
     RLX_SCHEME_GGUF_Q3K = 10, /* 256 / 110 (field order of rlx-gguf/src/lib.rs:889-930); resident as Q6_K super-blocks of the same values */
     RLX_SCHEME_GGUF_Q4_0 = 11, /* 32 elems / 18 bytes  */
     RLX_SCHEME_GGUF_Q8_0 = 12  /* 32 elems / 34 bytes  */
@@ -116,7 +116,7 @@ int64_t rlx_mi355x_bytes_for(int scheme, int64_t n_elems); /* rlx_gguf bytes_for
 
 /* A GGUF-packed [n, k] matrix (row-major, blocks along k: rlx-cpu/src/gguf_matmul.rs:15-20) repacked once
  * into the device layout the kernels stream (same byte count per block; 16-row x 128/256-k units whose
- * 16-byte lane slots hold MFMA operand fragments; wide schemes: binary16 fragments, 2 bytes per weight). */
+ * 16-byte lane slots hold what one lane of an MFMA operand fragment is decoded from). */
 typedef struct rlx_qweight rlx_qweight;
 
 /* Per-weight options. RLX_QW_Q6K_SIGNED_SCALES: read the sixteen scale bytes of a Q6_K super-block as signed, which is
@@ -146,8 +146,8 @@ int rlx_mi355x_repack_host_ex(int scheme, uint32_t flags, const void *gguf_bytes
 
 /* rlx_gguf::dequant_q8_0 / dequant_q4_0 / dequant_q4_k (rlx-gguf/src/lib.rs:600-633,974-1013) on the device:
  * out_dev[n*k] f32, row-major [n,k], bit-identical to the reference decoders (also Q5_K; Q6_K: to dequant_q6_k_block, the
- * one the matmul calls, or to dequant_q6_k for a weight created with RLX_QW_Q6K_SIGNED_SCALES). RLX_ERR_UNSUPPORTED for the
- * wide schemes (the exact f32 decode is not kept on the device). */
+ * one the matmul calls, or to dequant_q6_k for a weight created with RLX_QW_Q6K_SIGNED_SCALES; Q8_K, Q2_K, Q3_K: to the
+ * block decoders of rlx-gguf/src/lib.rs:848-930). */
 int rlx_mi355x_dequant(const rlx_qweight *w, float *out_dev, void *stream);
 
 /* rlx_cpu::gguf_matmul::gguf_matmul_bt (rlx-cpu/src/gguf_matmul.rs:40-95):

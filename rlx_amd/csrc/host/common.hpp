@@ -46,8 +46,6 @@ enum KernelId : int {
     K_GEMV_Q8_0_R2_NORM, K_GEMV_Q8_0_R4_NORM, K_GEMV_Q8_0_R2_NORM_PAIRED, K_GEMV_Q8_0_R4_NORM_PAIRED, K_GEMV_Q8_0_R2_NORM_ARGMAX,
     K_GEMV_Q4_K_R2, K_GEMV_Q4_K_R4, K_GEMV_Q4_K_R2_ARGMAX, K_GEMV_Q4_K_R2_PAIRED, K_GEMV_Q4_K_R4_PAIRED,
     K_GEMV_Q4_K_R2_NORM, K_GEMV_Q4_K_R4_NORM, K_GEMV_Q4_K_R2_NORM_PAIRED, K_GEMV_Q4_K_R4_NORM_PAIRED, K_GEMV_Q4_K_R2_NORM_ARGMAX,
-    K_GEMV_F16W_R2, K_GEMV_F16W_R4, K_GEMV_F16W_R2_ARGMAX, K_GEMV_F16W_R2_PAIRED, K_GEMV_F16W_R4_PAIRED,
-    K_GEMV_F16W_R2_NORM, K_GEMV_F16W_R4_NORM, K_GEMV_F16W_R2_NORM_PAIRED, K_GEMV_F16W_R4_NORM_PAIRED, K_GEMV_F16W_R2_NORM_ARGMAX,
     K_GEMV_Q6_K_R2, K_GEMV_Q6_K_R4, K_GEMV_Q6_K_R2_ARGMAX, K_GEMV_Q6_K_R2_PAIRED, K_GEMV_Q6_K_R4_PAIRED,
     K_GEMV_Q6_K_R2_NORM, K_GEMV_Q6_K_R4_NORM, K_GEMV_Q6_K_R2_NORM_PAIRED, K_GEMV_Q6_K_R4_NORM_PAIRED, K_GEMV_Q6_K_R2_NORM_ARGMAX,
     K_GEMV_Q5_K_R2, K_GEMV_Q5_K_R4, K_GEMV_Q5_K_R2_ARGMAX, K_GEMV_Q5_K_R2_PAIRED, K_GEMV_Q5_K_R4_PAIRED,
@@ -58,17 +56,12 @@ enum KernelId : int {
     K_GEMV_Q2_K_R2_NORM, K_GEMV_Q2_K_R4_NORM, K_GEMV_Q2_K_R2_NORM_PAIRED, K_GEMV_Q2_K_R4_NORM_PAIRED, K_GEMV_Q2_K_R2_NORM_ARGMAX,
     K_GEMV_Q4_0_U2_R2, K_GEMV_Q4_0_U2_R4, K_GEMV_Q4_0_U2_R2_ARGMAX, K_GEMV_Q4_0_U2_R2_PAIRED, K_GEMV_Q4_0_U2_R4_PAIRED,
     K_GEMV_Q4_0_U2_R2_NORM, K_GEMV_Q4_0_U2_R4_NORM, K_GEMV_Q4_0_U2_R2_NORM_PAIRED, K_GEMV_Q4_0_U2_R4_NORM_PAIRED, K_GEMV_Q4_0_U2_R2_NORM_ARGMAX,
-    K_GEMV_Q4_0_G2, K_GEMV_Q8_0_G2, K_GEMV_Q4_K_G2, K_GEMV_F16W_G2, K_GEMV_Q6_K_G2, K_GEMV_Q5_K_G2, K_GEMV_Q8_K_G2, K_GEMV_Q2_K_G2,
-    K_GEMM_Q4_K, K_GEMM_Q4_0, K_GEMM_Q8_0, K_GEMM64_Q4_K, K_GEMM64_Q4_0, K_GEMM64_Q8_0, K_GEMM_F16W, K_GEMM64_F16W, K_GEMM_Q6_K, K_GEMM64_Q6_K, K_GEMM_Q5_K, K_GEMM64_Q5_K, K_XPREP, K_XROWSCALE, K_ARGMAX_FINISH, K_TOPK_SELECT, K_RMSNORM_ROWS, K_SWIGLU_ROWS,
-    K_GEMM64G_Q4_K, K_GEMM64G_Q4_0, K_GEMM64G_Q8_0, K_GEMM64G_Q5_K, K_GEMM64G_Q6_K, K_GEMM64G_F16W, K_MOE_SORT,
+    K_GEMV_Q4_0_G2, K_GEMV_Q8_0_G2, K_GEMV_Q4_K_G2, K_GEMV_Q6_K_G2, K_GEMV_Q5_K_G2, K_GEMV_Q8_K_G2, K_GEMV_Q2_K_G2,
+    K_GEMM_Q4_K, K_GEMM_Q4_0, K_GEMM_Q8_0, K_GEMM64_Q4_K, K_GEMM64_Q4_0, K_GEMM64_Q8_0, K_GEMM_Q6_K, K_GEMM64_Q6_K, K_GEMM_Q5_K, K_GEMM64_Q5_K, K_XPREP, K_XROWSCALE, K_ARGMAX_FINISH, K_TOPK_SELECT, K_RMSNORM_ROWS, K_SWIGLU_ROWS,
+    K_GEMM64G_Q4_K, K_GEMM64G_Q4_0, K_GEMM64G_Q8_0, K_GEMM64G_Q5_K, K_GEMM64G_Q6_K, K_MOE_SORT,
     K_GEMM_Q8_K, K_GEMM64_Q8_K, K_GEMM64G_Q8_K, K_GEMM_Q2_K, K_GEMM64_Q2_K, K_GEMM64G_Q2_K,
     K_COUNT
 };
-
-// Device layout a scheme is kept in: its packed layout (layout_of), or binary16 fragments for the wide schemes (Q2_K,
-// Q3_K).
-Layout host_layout(int scheme);
-inline bool is_wide(int scheme) { return layout_is_f16w(host_layout(scheme)); }
 
 // Loads the embedded code object on first use (device 0). RLX_OK or an error code with text.
 int runtime_init();

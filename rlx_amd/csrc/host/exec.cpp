@@ -609,7 +609,7 @@ static std::unique_ptr<rlx_exec> plan_graph(const rlx_graph_desc *g, const rlx_c
         if (!is_source(nd.d.op_kind) || nd.d.op_kind == RLX_OP_INPUT) continue;
         if (nd.is_packed) {
             nd.w_flags = nd.scheme == SCHEME_Q6K ? wflags : 0u;
-            nd.slot = take((size_t)weight_dims(host_layout(nd.scheme), nd.w_n, nd.w_k).bytes * (size_t)nd.w_experts, 0, kForever);  // device layout, resident
+            nd.slot = take((size_t)weight_dims(layout_of(nd.scheme), nd.w_n, nd.w_k).bytes * (size_t)nd.w_experts, 0, kForever);  // device layout, resident
         } else {
             nd.slot = take((size_t)nd.numel * dtype_size(nd.d.dtype), 0, kForever);
         }

@@ -47,24 +47,7 @@ static inline float f16_bits_to_f32(uint16_t h) {
     return f;
 }
 
-// ---- block decoders of the wide schemes ------------------------------------------------------------------
-// Element-indexed restatements of the reference's super-block decoders, same f32 operation order, used once per weight
-// at upload. `i` is the element's position in the 256-element super-block.
-
-static inline float f16_at(const uint8_t *p) { return f16_bits_to_f32((uint16_t)(p[0] | (p[1] << 8))); }
-
-// Q2_K in the reference's field order (lib.rs:857-886): d, min, 16 scale bytes (low nibble scale, high nibble min),
-// 64 bytes of 2-bit codes.
-static void decode_q2_k(const uint8_t *b, float *out) {
-    const float d = f16_at(b), mn = f16_at(b + 2);
-    const uint8_t *scales = b + 4, *q = b + 20;
-    for (int i = 0; i < 256; i++) {
-        const int h = i >> 7, pair = (i >> 5) & 3, l = i & 31;
-        const uint8_t sc = scales[8 * h + 2 * pair + (l >> 4)];
-        const float dl = d * (float)(sc & 0xF), ml = mn * (float)(sc >> 4);
-        out[i] = dl * (float)((q[32 * h + l] >> (2 * pair)) & 3) - ml;
-    }
-}
+// ---- Q3_K fields ----------------------------------------------------------------------------------------
 
 // Q3_K in the reference's field order (lib.rs:889-930): d, 12 scale bytes, 32 bytes of high-bit mask, 64 bytes of 2-bit
 // codes. The value of element i is d * (scale[i / 16] - 32) * code(i) with code in [-4, 3]: at most 20 significant bits, so
@@ -85,48 +68,10 @@ static inline int q3k_code(const uint8_t *b, int i) {
     return ((q[32 * h + l] >> (2 * pair)) & 3) - ((hm[l] >> (4 * h + pair)) & 1 ? 0 : 4);
 }
 
-Layout host_layout(int scheme) { return layout_of(scheme); }
-
-static void decode_wide_block(int, const uint8_t *b, float *out) { decode_q2_k(b, out); }
-
-// Wide schemes: decode every super-block and store the weights as binary16 operand fragments.
-static int repack_wide(int scheme, const uint8_t *src, int64_t n, int64_t k, uint8_t *out) {
-    const Layout L = host_layout(scheme);
-    const WeightDims D = weight_dims(L, n, k);
-    const int64_t bpr = k / 256;
-    memset(out, 0, (size_t)D.bytes);
-    float vals[256];
-    for (int64_t r = 0; r < n; r++) {
-        const int64_t tile = r >> 4;
-        const int nrow = (int)(r & 15);
-        for (int64_t sb = 0; sb < bpr; sb++) {
-            decode_wide_block(scheme, src + (r * bpr + sb) * L.block_bytes, vals);
-            for (int blk = 0; blk < 8; blk++) {  // 32-column blocks of the super-block
-                const int64_t gblk = sb * 8 + blk, u = gblk >> 2;
-                uint8_t *unit = out + (tile * D.units + u) * L.unit_bytes + (gblk & 3) * 1024;
-                for (int g = 0; g < 4; g++) {
-                    uint16_t h8[8];
-                    for (int e = 0; e < 8; e++) {
-                        const float v = vals[32 * blk + 8 * g + e];
-                        h8[e] = f32_to_f16_bits(v);
-                        if ((h8[e] & 0x7FFFu) >= 0x7C00u && std::isfinite(v)) {
-                            set_error("repack: a decoded weight (%g, row %lld) exceeds the binary16 range the wide schemes are stored in",
-                                      (double)v, (long long)r);
-                            return RLX_ERR_UNSUPPORTED;
-                        }
-                    }
-                    memcpy(unit + (g * 16 + nrow) * 16, h8, 16);
-                }
-            }
-        }
-    }
-    return RLX_OK;
-}
-
 // ---- repack ---------------------------------------------------------------------------------------------
 
 int repack_host(int scheme, uint32_t flags, const uint8_t *src, size_t nbytes, int64_t n, int64_t k, uint8_t *out) {
-    Layout L = host_layout(scheme);
+    Layout L = layout_of(scheme);
     // Q6_K scale bytes read as signed are stored XOR 0x80 (offset binary): the kernels subtract 128 from the byte
     const uint8_t q6_flip = (flags & RLX_QW_Q6K_SIGNED_SCALES) ? 0x80u : 0u;
     if (L.unit_k == 0 || L.block_elems == 0) {
@@ -144,7 +89,6 @@ int repack_host(int scheme, uint32_t flags, const uint8_t *src, size_t nbytes, i
                   (long long)(n * bpr * L.block_bytes));
         return RLX_ERR_INVALID;
     }
-    if (is_wide(scheme)) return repack_wide(scheme, src, n, k, out);
     WeightDims D = weight_dims(L, n, k);
     for (int64_t tile = 0; tile < D.row_tiles; tile++) {
         for (int64_t u = 0; u < D.units; u++) {
@@ -422,7 +366,7 @@ int64_t rlx_mi355x_bytes_for(int scheme, int64_t n) {
 }
 
 size_t rlx_mi355x_qweight_device_bytes_for(int scheme, int64_t n, int64_t k) {
-    return (size_t)rlx::weight_dims(rlx::host_layout(scheme), n, k).bytes;
+    return (size_t)rlx::weight_dims(rlx::layout_of(scheme), n, k).bytes;
 }
 
 int rlx_mi355x_repack_host(int scheme, const void *gguf_bytes, size_t nbytes, int64_t n, int64_t k, void *out) {

@@ -14,7 +14,7 @@ int repack_host(int scheme, uint32_t flags, const uint8_t *src, size_t nbytes, i
 
 struct rlx_qweight {
     int scheme;
-    rlx::Layout layout;    // device layout it was repacked into (packed, or binary16 for the wide schemes)
+    rlx::Layout layout;    // device layout it was repacked into
     rlx::WeightDims dims;  // of one [n, k] matrix
     uint8_t *dev;
     bool owns;
@@ -132,7 +132,6 @@ static int launch_gemv(const void *const *xs, int xk, const rlx_qweight *const *
                        const rlx_qweight *const *pairs = nullptr, const RmsNorm *norm = nullptr, int *wgs_out = nullptr) {
     const int scheme = ws[0]->scheme;
     const Layout L = ws[0]->layout;
-    const bool wide = layout_is_f16w(L);
     for (int i = 0; i < count; i++) {
         if ((uintptr_t)xs[i] % 16 != 0) {
             set_error("gguf_matmul_bt: activations must be 16-byte aligned");
@@ -153,7 +152,7 @@ static int launch_gemv(const void *const *xs, int xk, const rlx_qweight *const *
         return RLX_ERR_UNSUPPORTED;
     }
     // kernel = scheme family x {r2, r4, r2_argmax, r2_paired, r4_paired}
-    const int family = wide ? K_GEMV_F16W_R2 : scheme == SCHEME_Q4_0 ? K_GEMV_Q4_0_R2 : scheme == SCHEME_Q8_0 ? K_GEMV_Q8_0_R2
+    const int family = scheme == SCHEME_Q4_0 ? K_GEMV_Q4_0_R2 : scheme == SCHEME_Q8_0 ? K_GEMV_Q8_0_R2
                        : scheme == SCHEME_Q6K ? K_GEMV_Q6_K_R2 : scheme == SCHEME_Q5K ? K_GEMV_Q5_K_R2
                        : scheme == SCHEME_Q8K ? K_GEMV_Q8_K_R2 : scheme == SCHEME_Q2K ? K_GEMV_Q2_K_R2 : K_GEMV_Q4_K_R2;
     if (argmax_key && !r2) {
@@ -185,7 +184,7 @@ static int launch_gemv(const void *const *xs, int xk, const rlx_qweight *const *
     const size_t slot_bytes = (size_t)ng * 256;
     auto stage_bytes = [&](int kcu) {
         size_t b = ((size_t)rv * ((size_t)kcu * L.unit_k + 8) * 2 + 15) & ~(size_t)15;
-        if (scheme == SCHEME_Q4K || (scheme == SCHEME_Q5K && !wide)) b += (size_t)kcu * (L.unit_k / 32) * 16 * rg * 4;  // block sums
+        if (scheme == SCHEME_Q4K || scheme == SCHEME_Q5K) b += (size_t)kcu * (L.unit_k / 32) * 16 * rg * 4;  // block sums
         return b;
     };
     // A launch shape: `wgs_per_cu` workgroups of `waves` waves per CU, every one resident at once, each with the same
@@ -411,7 +410,6 @@ static int launch_gemm(const void *x, int xk, const rlx_qweight *const *ws, floa
     void *params[] = {&a};
     KernelId id = w->scheme == SCHEME_Q4K       ? (skinny ? K_GEMM64_Q4_K : K_GEMM_Q4_K)
                   : w->scheme == SCHEME_Q4_0    ? (skinny ? K_GEMM64_Q4_0 : K_GEMM_Q4_0)
-                  : layout_is_f16w(L)           ? (skinny ? K_GEMM64_F16W : K_GEMM_F16W)
                   : w->scheme == SCHEME_Q6K     ? (skinny ? K_GEMM64_Q6_K : K_GEMM_Q6_K)
                   : w->scheme == SCHEME_Q5K     ? (skinny ? K_GEMM64_Q5_K : K_GEMM_Q5_K)
                   : w->scheme == SCHEME_Q8K     ? (skinny ? K_GEMM64_Q8_K : K_GEMM_Q8_K)
@@ -435,7 +433,7 @@ int rlx_mi355x_qweight_create_ex(int scheme, uint32_t flags, const void *gguf_by
         return RLX_ERR_INVALID;
     }
     *out = nullptr;
-    const Layout HL = host_layout(scheme);
+    const Layout HL = layout_of(scheme);
     if (HL.unit_k == 0 || HL.block_elems == 0) {
         set_error("qweight: scheme %d is not a claimed GGUF scheme", scheme);
         return RLX_ERR_UNSUPPORTED;
@@ -531,11 +529,6 @@ int rlx_mi355x_dequant(const rlx_qweight *w, float *out_dev, void *stream) {
     if (!w || !out_dev) {
         set_error("dequant: null argument");
         return RLX_ERR_INVALID;
-    }
-    if (layout_is_f16w(w->layout)) {
-        set_error("dequant: scheme %d is resident as binary16 (decoded at upload); the exact f32 decode is not kept on the device",
-                  w->scheme);
-        return RLX_ERR_UNSUPPORTED;
     }
     DequantArgs a{w->dev, out_dev, w->dims.n, w->dims.k, w->dims.units, w->sc_off()};
     void *params[] = {&a};
@@ -705,7 +698,7 @@ int rlx_mi355x_rmsnorm_gguf_matmul_bt_batch(const float *x_dev, const float *gam
                 set_error("rmsnorm_gguf_matmul_bt_batch: null weight / output or an expert stack at %d", i0 + i);
                 return RLX_ERR_INVALID;
             }
-            const bool same = ws[i0 + i]->scheme == ws[i0]->scheme || (layout_is_f16w(ws[i0 + i]->layout) && layout_is_f16w(ws[i0]->layout));
+            const bool same = ws[i0 + i]->scheme == ws[i0]->scheme;
             if (!same || ws[i0 + i]->dims.k != ws[0]->dims.k) {
                 set_error("rmsnorm_gguf_matmul_bt_batch: the matrices share one normalized input, so one scheme and one k");
                 return RLX_ERR_INVALID;
@@ -726,7 +719,7 @@ int rlx_mi355x_rmsnorm_gguf_matmul_swiglu(const float *x_dev, const float *gamma
         set_error("rmsnorm_gguf_matmul_swiglu: null argument");
         return RLX_ERR_INVALID;
     }
-    const bool same_layout = w_up->scheme == w_gate->scheme || (layout_is_f16w(w_up->layout) && layout_is_f16w(w_gate->layout));
+    const bool same_layout = w_up->scheme == w_gate->scheme;
     if (!same_layout || w_up->dims.n != w_gate->dims.n || w_up->dims.k != w_gate->dims.k || w_up->experts != 1 ||
         w_gate->experts != 1) {
         set_error("rmsnorm_gguf_matmul_swiglu: the up and gate projections must share scheme, n and k");
@@ -771,7 +764,7 @@ int rlx_mi355x_gguf_matmul_swiglu(const void *x_dev, int x_dtype, const rlx_qwei
         set_error("gguf_matmul_swiglu: activation dtype %d is not F32 / BF16 / F16", x_dtype);
         return RLX_ERR_UNSUPPORTED;
     }
-    const bool same_layout = w_up->scheme == w_gate->scheme || (layout_is_f16w(w_up->layout) && layout_is_f16w(w_gate->layout));
+    const bool same_layout = w_up->scheme == w_gate->scheme;
     if (!same_layout || w_up->dims.n != w_gate->dims.n || w_up->dims.k != w_gate->dims.k || w_up->experts != 1 ||
         w_gate->experts != 1) {
         set_error("gguf_matmul_swiglu: the up and gate projections must share scheme, n and k");
@@ -1051,7 +1044,6 @@ int rlx_mi355x_gguf_grouped_matmul_bt_ws(const void *x_dev, int x_dtype, const r
     void *params[] = {&a};
     const KernelId id = w->scheme == SCHEME_Q4K    ? K_GEMM64G_Q4_K
                         : w->scheme == SCHEME_Q4_0 ? K_GEMM64G_Q4_0
-                        : layout_is_f16w(L)        ? K_GEMM64G_F16W
                         : w->scheme == SCHEME_Q6K  ? K_GEMM64G_Q6_K
                         : w->scheme == SCHEME_Q5K  ? K_GEMM64G_Q5_K
                         : w->scheme == SCHEME_Q8K  ? K_GEMM64G_Q8_K

@@ -32,8 +32,6 @@ static const char *const kKernelNames[K_COUNT] = {
     "rlx_gemv_q8_0_r2_norm", "rlx_gemv_q8_0_r4_norm", "rlx_gemv_q8_0_r2_norm_paired", "rlx_gemv_q8_0_r4_norm_paired", "rlx_gemv_q8_0_r2_norm_argmax",
     "rlx_gemv_q4_k_r2", "rlx_gemv_q4_k_r4", "rlx_gemv_q4_k_r2_argmax", "rlx_gemv_q4_k_r2_paired", "rlx_gemv_q4_k_r4_paired",
     "rlx_gemv_q4_k_r2_norm", "rlx_gemv_q4_k_r4_norm", "rlx_gemv_q4_k_r2_norm_paired", "rlx_gemv_q4_k_r4_norm_paired", "rlx_gemv_q4_k_r2_norm_argmax",
-    "rlx_gemv_f16w_r2", "rlx_gemv_f16w_r4", "rlx_gemv_f16w_r2_argmax", "rlx_gemv_f16w_r2_paired", "rlx_gemv_f16w_r4_paired",
-    "rlx_gemv_f16w_r2_norm", "rlx_gemv_f16w_r4_norm", "rlx_gemv_f16w_r2_norm_paired", "rlx_gemv_f16w_r4_norm_paired", "rlx_gemv_f16w_r2_norm_argmax",
     "rlx_gemv_q6_k_r2", "rlx_gemv_q6_k_r4", "rlx_gemv_q6_k_r2_argmax", "rlx_gemv_q6_k_r2_paired", "rlx_gemv_q6_k_r4_paired",
     "rlx_gemv_q6_k_r2_norm", "rlx_gemv_q6_k_r4_norm", "rlx_gemv_q6_k_r2_norm_paired", "rlx_gemv_q6_k_r4_norm_paired", "rlx_gemv_q6_k_r2_norm_argmax",
     "rlx_gemv_q5_k_r2", "rlx_gemv_q5_k_r4", "rlx_gemv_q5_k_r2_argmax", "rlx_gemv_q5_k_r2_paired", "rlx_gemv_q5_k_r4_paired",
@@ -44,9 +42,9 @@ static const char *const kKernelNames[K_COUNT] = {
     "rlx_gemv_q2_k_r2_norm", "rlx_gemv_q2_k_r4_norm", "rlx_gemv_q2_k_r2_norm_paired", "rlx_gemv_q2_k_r4_norm_paired", "rlx_gemv_q2_k_r2_norm_argmax",
     "rlx_gemv_q4_0_u2_r2", "rlx_gemv_q4_0_u2_r4", "rlx_gemv_q4_0_u2_r2_argmax", "rlx_gemv_q4_0_u2_r2_paired", "rlx_gemv_q4_0_u2_r4_paired",
     "rlx_gemv_q4_0_u2_r2_norm", "rlx_gemv_q4_0_u2_r4_norm", "rlx_gemv_q4_0_u2_r2_norm_paired", "rlx_gemv_q4_0_u2_r4_norm_paired", "rlx_gemv_q4_0_u2_r2_norm_argmax",
-    "rlx_gemv_q4_0_g2", "rlx_gemv_q8_0_g2", "rlx_gemv_q4_k_g2", "rlx_gemv_f16w_g2", "rlx_gemv_q6_k_g2", "rlx_gemv_q5_k_g2", "rlx_gemv_q8_k_g2", "rlx_gemv_q2_k_g2",
-    "rlx_gemm_q4_k", "rlx_gemm_q4_0", "rlx_gemm_q8_0", "rlx_gemm64_q4_k", "rlx_gemm64_q4_0", "rlx_gemm64_q8_0", "rlx_gemm_f16w", "rlx_gemm64_f16w", "rlx_gemm_q6_k", "rlx_gemm64_q6_k", "rlx_gemm_q5_k", "rlx_gemm64_q5_k", "rlx_xprep", "rlx_xrowscale", "rlx_argmax_finish", "rlx_topk_select", "rlx_rmsnorm_rows", "rlx_swiglu_rows",
-    "rlx_gemm64g_q4_k", "rlx_gemm64g_q4_0", "rlx_gemm64g_q8_0", "rlx_gemm64g_q5_k", "rlx_gemm64g_q6_k", "rlx_gemm64g_f16w", "rlx_moe_sort",
+    "rlx_gemv_q4_0_g2", "rlx_gemv_q8_0_g2", "rlx_gemv_q4_k_g2", "rlx_gemv_q6_k_g2", "rlx_gemv_q5_k_g2", "rlx_gemv_q8_k_g2", "rlx_gemv_q2_k_g2",
+    "rlx_gemm_q4_k", "rlx_gemm_q4_0", "rlx_gemm_q8_0", "rlx_gemm64_q4_k", "rlx_gemm64_q4_0", "rlx_gemm64_q8_0", "rlx_gemm_q6_k", "rlx_gemm64_q6_k", "rlx_gemm_q5_k", "rlx_gemm64_q5_k", "rlx_xprep", "rlx_xrowscale", "rlx_argmax_finish", "rlx_topk_select", "rlx_rmsnorm_rows", "rlx_swiglu_rows",
+    "rlx_gemm64g_q4_k", "rlx_gemm64g_q4_0", "rlx_gemm64g_q8_0", "rlx_gemm64g_q5_k", "rlx_gemm64g_q6_k", "rlx_moe_sort",
     "rlx_gemm_q8_k", "rlx_gemm64_q8_k", "rlx_gemm64g_q8_k", "rlx_gemm_q2_k", "rlx_gemm64_q2_k", "rlx_gemm64g_q2_k",
 };
 

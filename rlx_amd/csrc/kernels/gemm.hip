@@ -181,10 +181,6 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
             }
         } else if constexpr (K8) {  // one quarter of the super-block (two 32-column blocks) per step
             b_q[q & 1] = ld128(b_rsrc, lane * 16, (step >> 2) * L.unit_bytes + q * 1024);
-        } else if constexpr (SCHEME == SCHEME_F16W) {  // two ready-made fragments per lane and step: b_q and b_meta hold them
-            const int unit = (step >> 1) * L.unit_bytes + (q & 1) * 2048;
-            b_q[q & 1] = ld128(b_rsrc, lane * 16, unit);
-            b_meta[q & 1] = ld128(b_rsrc, lane * 16, unit + 1024);
         } else if constexpr (SCHEME == SCHEME_Q4_0) {
             const int unit = (step >> 1) * L.unit_bytes;
             if ((q & 1) == 0) {
@@ -248,10 +244,6 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
             else unpack_q2_scaled<0>(b_q[0][q], splat_ubyte_half(scb), f);
         } else if constexpr (K8) {
             unpack_q8(b_q[q & 1][2 * jl], b_q[q & 1][2 * jl + 1], f);
-#pragma unroll
-            for (int e = 0; e < 4; e++) f.u[e] &= b_keep;  // a dead tile stores zeros
-        } else if constexpr (SCHEME == SCHEME_F16W) {
-            f.u4 = jl ? b_meta[q & 1] : b_q[q & 1];
 #pragma unroll
             for (int e = 0; e < 4; e++) f.u[e] &= b_keep;  // a dead tile stores zeros
         } else {
@@ -774,8 +766,6 @@ extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64_q6_k(rlx::GemmAr
 extern "C" __global__ __launch_bounds__(512) void rlx_gemm_q8_k(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q8K, 2, 2>(a); }
 extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64_q8_k(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q8K, 1, 1>(a); }
 extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64g_q8_k(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q8K, 1, 1, true>(a); }
-extern "C" __global__ __launch_bounds__(512) void rlx_gemm_f16w(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_F16W, 2, 2>(a); }
-extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64_f16w(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_F16W, 1, 1>(a); }
 extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64_q4_k(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q4K, 1, 1>(a); }
 extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64_q4_0(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q4_0, 1, 1>(a); }
 extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64_q8_0(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q8_0, 1, 1>(a); }
@@ -784,6 +774,5 @@ extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64g_q4_0(rlx::GemmA
 extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64g_q8_0(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q8_0, 1, 1, true>(a); }
 extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64g_q5_k(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q5K, 1, 1, true>(a); }
 extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64g_q6_k(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q6K, 1, 1, true>(a); }
-extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64g_f16w(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_F16W, 1, 1, true>(a); }
 extern "C" __global__ __launch_bounds__(256) void rlx_xprep(rlx::XPrepArgs a) { rlx::xprep_body(a); }
 extern "C" __global__ __launch_bounds__(256) void rlx_xrowscale(rlx::XPrepArgs a) { rlx::xrowscale_body(a); }

@@ -188,19 +188,6 @@ struct UnitRegs<SCHEME_Q2K> {  // one super-block: the lane slot's 64 two-bit co
     }
 };
 
-template <>
-struct UnitRegs<SCHEME_F16W> {  // weights already stored as binary16 fragments: four 32-column blocks, no scales
-    uint4_t q[4];
-    __device__ __forceinline__ void load(const uint8_t *unit, int l, int, bool) {
-#pragma unroll
-        for (int t = 0; t < 4; t++) q[t] = __builtin_nontemporal_load((const uint4_t *)(unit + t * 1024 + l * 16));
-    }
-    __device__ __forceinline__ void clear() {
-#pragma unroll
-        for (int t = 0; t < 4; t++) q[t] = uint4_t{0, 0, 0, 0};
-    }
-};
-
 __device__ __forceinline__ float scale_of(uint2_t s, int t) {
     return half_bits_to_float((t & 1) ? (s[t >> 1] >> 16) : (s[t >> 1] & 0xFFFFu));
 }
@@ -349,20 +336,6 @@ __device__ __forceinline__ void compute_unit(const UnitRegs<SCHEME> &w, const ha
                 acc[rg][r] = __builtin_fmaf(d, sum[rg][r], acc[rg][r]);
                 acc[rg][r] = __builtin_fmaf(-dmin, smin[rg][r], acc[rg][r]);
             }
-    } else if constexpr (SCHEME == SCHEME_F16W) {
-#pragma unroll
-        for (int rg = 0; rg < RG; rg++) {
-            load_afrags<4>(xrow[rg], live[rg], ucol, a);
-            float4_t sum = zero;  // the matrix unit accumulates the four blocks; nothing to decode or scale
-#pragma unroll
-            for (int t = 0; t < 4; t++) {
-                Frag b;
-                b.u4 = w.q[t];
-                sum = mfma16(a[t], b, sum);
-            }
-#pragma unroll
-            for (int r = 0; r < NREG; r++) acc[rg][r] += sum[r];
-        }
     } else {
         float d = half_bits_to_float(w.meta[0] & 0xFFFFu);
         float dmin = half_bits_to_float(w.meta[0] >> 16);
@@ -923,7 +896,6 @@ __device__ __forceinline__ bool gemv_pass(const GemvArgs &a) {
 RLX_GEMV_SCHEME(q4_0, rlx::SCHEME_Q4_0, 4, 1)
 RLX_GEMV_SCHEME(q8_0, rlx::SCHEME_Q8_0, 3, 1)
 RLX_GEMV_SCHEME(q4_k, rlx::SCHEME_Q4K, 3, 1)
-RLX_GEMV_SCHEME(f16w, rlx::SCHEME_F16W, 2, 1)
 RLX_GEMV_SCHEME(q6_k, rlx::SCHEME_Q6K, 2, 1)
 RLX_GEMV_SCHEME(q5_k, rlx::SCHEME_Q5K, 2, 1)
 RLX_GEMV_SCHEME(q8_k, rlx::SCHEME_Q8K, 2, 1)
@@ -940,7 +912,6 @@ RLX_GEMV_SCHEME(q4_0_u2, rlx::SCHEME_Q4_0, 2, 2)
 RLX_GEMV_ROWGROUPS(q4_0, rlx::SCHEME_Q4_0, 2)
 RLX_GEMV_ROWGROUPS(q8_0, rlx::SCHEME_Q8_0, 2)
 RLX_GEMV_ROWGROUPS(q4_k, rlx::SCHEME_Q4K, 2)
-RLX_GEMV_ROWGROUPS(f16w, rlx::SCHEME_F16W, 2)
 RLX_GEMV_ROWGROUPS(q6_k, rlx::SCHEME_Q6K, 2)
 RLX_GEMV_ROWGROUPS(q5_k, rlx::SCHEME_Q5K, 2)
 RLX_GEMV_ROWGROUPS(q8_k, rlx::SCHEME_Q8K, 2)

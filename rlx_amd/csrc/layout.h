@@ -43,9 +43,6 @@
 //                   byte the codes of elements 2i (low half) / 2i + 1 (high half) sit at bits 2i
 //          [1024,1280) per row n: the 16 scale bytes verbatim (low nibble scale, high nibble min of a 16-column sub-block)
 //          [1280,1344) per row n: f16 d, f16 dmin
-//   F16W : weights stored as binary16 operand fragments (an internal layout no GGUF scheme uses any more; the kernels
-//          that read it are the identity-decode yardstick of the benchmark): [0,4096) four blocks t: 16 B at
-//          1024*t + 16*l = the 8 halfs of granule (n, 4u+t, g). No scales.
 // Units are stored [row_tile][unit] with the unit index (K direction) fastest.
 // N is padded to a multiple of 16 and K to a multiple of UNIT_K with zero-scale blocks.
 #pragma once
@@ -59,11 +56,10 @@
 
 namespace rlx {
 
-// Values of the reference's QuantScheme discriminants (rlx-ir/src/quant.rs:39-73); SCHEME_F16W is internal: the device
-// layout every wide scheme is stored in, and the template argument of the kernels that read it.
+// Values of the reference's QuantScheme discriminants (rlx-ir/src/quant.rs:39-73).
 enum Scheme : int {
     SCHEME_Q4K = 5, SCHEME_Q5K = 6, SCHEME_Q6K = 7, SCHEME_Q8K = 8, SCHEME_Q2K = 9, SCHEME_Q3K = 10,
-    SCHEME_Q4_0 = 11, SCHEME_Q8_0 = 12, SCHEME_F16W = 100
+    SCHEME_Q4_0 = 11, SCHEME_Q8_0 = 12
 };
 
 // fifth bit of element e inside a Q5_K high-bit word (after the rotate of its code word), and the rotates
@@ -91,21 +87,15 @@ RLX_HD constexpr Layout layout_of(int scheme) {
            : scheme == SCHEME_Q8K  ? Layout{256, 4160, 4096, 256, 292}
            : scheme == SCHEME_Q2K  ? Layout{256, 1344, 1024, 256, 84}
            : scheme == SCHEME_Q3K  ? Layout{256, 3360, 3072, 256, 110}  // rewritten as Q6_K units
-           : scheme == SCHEME_F16W ? Layout{128, 4096, 4096, 0, 0}
                                    : Layout{0, 0, 0, 0, 0};
 }
 
-// The binary16 layout of a scheme kept wide: F16W geometry with the scheme's own GGUF block size.
-RLX_HD constexpr Layout wide_layout_of(int scheme) {
-    return Layout{128, 4096, 4096, layout_of(scheme).block_elems, layout_of(scheme).block_bytes};
-}
 // The scheme whose kernels read a scheme's device units. A Q3_K super-block (3-bit codes in [-4, 3], 6-bit scales minus 32,
 // one d) is rewritten at upload, exactly, as the Q6_K super-block of the same values with signed scale bytes.
 RLX_HD constexpr int kernel_scheme(int scheme) { return scheme == SCHEME_Q3K ? SCHEME_Q6K : scheme; }
 // What a scheme's prefill kernel needs next to the activation image: 0 nothing, 1 the sums of every 32-column block
 // (Q4_K / Q5_K: the dmin term), 2 the sums of every 16-column sub-block (Q2_K).
 RLX_HD constexpr int act_sums_kind(int scheme) { return (scheme == SCHEME_Q4K || scheme == SCHEME_Q5K) ? 1 : scheme == SCHEME_Q2K ? 2 : 0; }
-RLX_HD constexpr bool layout_is_f16w(const Layout &L) { return L.unit_k == 128 && L.unit_bytes == 4096; }
 
 // nibble position of fragment element e inside a granule word
 RLX_HD constexpr int nib_pos(int e) { return ((e & 1) << 2) | (e >> 1); }
