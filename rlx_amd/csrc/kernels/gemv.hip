@@ -899,7 +899,7 @@ RLX_GEMV_SCHEME(q4_k, rlx::SCHEME_Q4K, 3, 1)
 RLX_GEMV_SCHEME(q6_k, rlx::SCHEME_Q6K, 2, 1)
 RLX_GEMV_SCHEME(q5_k, rlx::SCHEME_Q5K, 2, 1)
 RLX_GEMV_SCHEME(q8_k, rlx::SCHEME_Q8K, 2, 1)
-RLX_GEMV_SCHEME(q2_k, rlx::SCHEME_Q2K, 3, 1)
+RLX_GEMV_SCHEME(q2_k, rlx::SCHEME_Q2K, 2, 1)
 // Two 128-column units per loop item: taken when every K run holds an even number of units. (Measured neutral to
 // slightly slower for Q8_0, whose unit is twice the bytes, so only Q4_0 has it.)
 RLX_GEMV_SCHEME(q4_0_u2, rlx::SCHEME_Q4_0, 2, 2)
