@@ -264,7 +264,7 @@ SHAPES = [(1, 200, 1024, DType.F32), (4, 48, 2304, DType.F32), (16, 130, 512, DT
           (300, 136, 768, DType.F32), (27, 330, 2048, DType.BF16), (13, 72, 768, DType.F32)]  # the last two: 17..32 MFMA rows
 
 
-def run_wide(scheme, blocks, m, n, k, dtype):
+def run_matmul(scheme, blocks, m, n, k, dtype):
     rng = np.random.default_rng(m * 7 + n)
     x = rng.standard_normal((m, k)).astype(np.float32)
     if dtype == DType.BF16:
@@ -278,23 +278,25 @@ def run_wide(scheme, blocks, m, n, k, dtype):
 @pytest.mark.gpu
 @pytest.mark.parametrize("scheme", FIVE)
 @pytest.mark.parametrize("m,n,k,dtype", SHAPES)
-def test_wide_matmul_matches_f64_oracle(scheme, m, n, k, dtype):
+def test_k_quant_matmul_matches_f64_oracle(scheme, m, n, k, dtype):
     """Weights of model-like magnitude: the reference tests' bound, |delta| / max(|expected|, 1) <= 2e-3
     (rlx-runtime/tests/dequant_matmul_gguf.rs:231-233)."""
     d_std, dmin_std = MODEL_SCALE[scheme]
     blocks = random_blocks(scheme, n, k, seed=60 + scheme, d_std=d_std, dmin_std=dmin_std)
-    x, got = run_wide(scheme, blocks, m, n, k, dtype)
+    x, got = run_matmul(scheme, blocks, m, n, k, dtype)
     assert rel_err(got, oracle.gguf_matmul_f64(x, blocks, m, k, n, scheme)) <= 2e-3
 
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("scheme", FIVE)
 @pytest.mark.parametrize("m,n,k,dtype", [SHAPES[0], SHAPES[3]])
-def test_wide_matmul_error_is_the_binary16_rounding_of_the_weights(scheme, m, n, k, dtype):
-    """Arbitrary scale bytes (weights up to tens, sums in the hundreds, heavy cancellation): the only error source is
-    storing each decoded weight as binary16, so |delta_j| <= 2^-11 sum_p |w_jp x_p| (plus the f32 accumulation)."""
+def test_k_quant_matmul_error_is_below_a_binary16_rounding_of_the_weights(scheme, m, n, k, dtype):
+    """Arbitrary scale bytes (weights up to tens, sums in the hundreds, heavy cancellation), where the bound on
+    |delta| / max(|y|, 1) says little: the error stays below what rounding every decoded weight to binary16 would give,
+    |delta_j| <= 2^-11 sum_p |w_jp x_p| (plus the f32 accumulation). The packed kernels keep the weights exact except Q6_K
+    products sc * (q - 32) above 2048, which are rounded to binary16."""
     blocks = random_blocks(scheme, n, k, seed=80 + scheme)
-    x, got = run_wide(scheme, blocks, m, n, k, dtype)
+    x, got = run_matmul(scheme, blocks, m, n, k, dtype)
     w = oracle.dequant_matmul_blocks(scheme, blocks, n * k).reshape(n, k).astype(np.float64)
     want = oracle.gguf_matmul_f64(x, blocks, m, k, n, scheme)
     bound = (np.abs(x.astype(np.float64)) @ np.abs(w).T) * (2.0 ** -11 + 2.0 ** -20) + 1e-6
@@ -405,7 +407,7 @@ def test_q6k_signed_scales_through_session_and_gguf_file(tmp_path):
 @pytest.mark.gpu
 @pytest.mark.parametrize("scheme", [Q6K, Q5K, Q8K, Q2K, Q3K])
 @pytest.mark.parametrize("m", [11, 90])  # per-token decode launches; tokens sorted by expert and one prefill launch
-def test_wide_grouped_matmul(scheme, m):
+def test_k_quant_grouped_matmul(scheme, m):
     """Mixture-of-experts routing (rlx-cpu/src/gguf_matmul.rs:101-139) over a stack of K-quant slabs."""
     k, n, experts = 512, 24, 4
     d_std, dmin_std = MODEL_SCALE[scheme]
