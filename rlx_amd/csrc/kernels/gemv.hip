@@ -893,26 +893,31 @@ __device__ __forceinline__ bool gemv_pass(const GemvArgs &a) {
     RLX_GEMV_INST(rlx_gemv_##tag##_r4_norm_paired, SCHEME, 4, DEPTH, rlx::GEMV_NORM | rlx::GEMV_PAIRED, UPI) \
     RLX_GEMV_INST(rlx_gemv_##tag##_r2_norm_argmax, SCHEME, 2, DEPTH, rlx::GEMV_NORM | rlx::GEMV_ARGMAX, UPI)
 
-RLX_GEMV_SCHEME(q4_0, rlx::SCHEME_Q4_0, 4, 1)
-RLX_GEMV_SCHEME(q8_0, rlx::SCHEME_Q8_0, 3, 1)
-RLX_GEMV_SCHEME(q4_k, rlx::SCHEME_Q4K, 3, 1)
-RLX_GEMV_SCHEME(q6_k, rlx::SCHEME_Q6K, 2, 1)
-RLX_GEMV_SCHEME(q5_k, rlx::SCHEME_Q5K, 2, 1)
-RLX_GEMV_SCHEME(q8_k, rlx::SCHEME_Q8K, 2, 1)
-RLX_GEMV_SCHEME(q2_k, rlx::SCHEME_Q2K, 2, 1)
+// DEPTH = loop items a wave keeps in flight. One or two is what the memory system likes: with sixteen waves per CU a
+// deeper ring only queues requests (a read-only probe of this access pattern: 19.8 us for 123 MB with two units in flight
+// per wave, 21.5 with four, 22.7 with eight), and the kernels measured 4 - 11 % faster at one row and up to sixteen rows when
+// the rings went from 2 - 4 items to 1 - 2 (Q8_0, whose unit is 2 KB, is indifferent).
+RLX_GEMV_SCHEME(q4_0, rlx::SCHEME_Q4_0, 2, 1)
+RLX_GEMV_SCHEME(q8_0, rlx::SCHEME_Q8_0, 2, 1)
+RLX_GEMV_SCHEME(q4_k, rlx::SCHEME_Q4K, 1, 1)
+RLX_GEMV_SCHEME(q6_k, rlx::SCHEME_Q6K, 1, 1)
+RLX_GEMV_SCHEME(q5_k, rlx::SCHEME_Q5K, 1, 1)
+RLX_GEMV_SCHEME(q8_k, rlx::SCHEME_Q8K, 1, 1)
+RLX_GEMV_SCHEME(q2_k, rlx::SCHEME_Q2K, 1, 1)
 // Two 128-column units per loop item: taken when every K run holds an even number of units. (Measured neutral to
 // slightly slower for Q8_0, whose unit is twice the bytes, so only Q4_0 has it.)
-RLX_GEMV_SCHEME(q4_0_u2, rlx::SCHEME_Q4_0, 2, 2)
+RLX_GEMV_SCHEME(q4_0_u2, rlx::SCHEME_Q4_0, 1, 2)
 // Two groups of 16 activation rows per weight fragment (17..32 rows): plain epilogue only, workgroups of eight waves
 // (sixteen measured 40 - 70 % slower: the activation chunk and the partial sums of twice the tiles no longer fit
 // side by side). Four groups were built and measured too, with 24 tiles per workgroup (4 KB of partial sums per tile
 // leave LDS for three K units of activations per chunk) and with one tile per wave: 493 and 462 us at 64 rows on a
 // 70B layer against 343 for the prefill kernel.
+// Ring depth: the K-quants measured 3 - 6 % faster with one item in flight, Q4_0 and Q8_0 4 % faster with two.
 #define RLX_GEMV_ROWGROUPS(tag, SCHEME, DEPTH) RLX_GEMV_INST_RG(rlx_gemv_##tag##_g2, SCHEME, 4, DEPTH, rlx::GEMV_PLAIN, 1, 2, 512)
 RLX_GEMV_ROWGROUPS(q4_0, rlx::SCHEME_Q4_0, 2)
 RLX_GEMV_ROWGROUPS(q8_0, rlx::SCHEME_Q8_0, 2)
-RLX_GEMV_ROWGROUPS(q4_k, rlx::SCHEME_Q4K, 2)
-RLX_GEMV_ROWGROUPS(q6_k, rlx::SCHEME_Q6K, 2)
-RLX_GEMV_ROWGROUPS(q5_k, rlx::SCHEME_Q5K, 2)
-RLX_GEMV_ROWGROUPS(q8_k, rlx::SCHEME_Q8K, 2)
-RLX_GEMV_ROWGROUPS(q2_k, rlx::SCHEME_Q2K, 2)
+RLX_GEMV_ROWGROUPS(q4_k, rlx::SCHEME_Q4K, 1)
+RLX_GEMV_ROWGROUPS(q6_k, rlx::SCHEME_Q6K, 1)
+RLX_GEMV_ROWGROUPS(q5_k, rlx::SCHEME_Q5K, 1)
+RLX_GEMV_ROWGROUPS(q8_k, rlx::SCHEME_Q8K, 1)
+RLX_GEMV_ROWGROUPS(q2_k, rlx::SCHEME_Q2K, 1)
