@@ -261,7 +261,8 @@ def bf16_bits(x):
 # super-block scales that give weights of a few hundredths, like a quantized model's, whatever the code bytes are
 MODEL_SCALE = {Q5K: (4e-5, 2e-5), Q6K: (5e-6, 0.0), Q8K: (2e-4, 0.0), Q2K: (5e-4, 1e-4), Q3K: (2e-4, 0.0)}
 SHAPES = [(1, 200, 1024, DType.F32), (4, 48, 2304, DType.F32), (16, 130, 512, DType.BF16), (64, 200, 1024, DType.BF16),
-          (300, 136, 768, DType.F32), (27, 330, 2048, DType.BF16), (13, 72, 768, DType.F32)]  # the last two: 17..32 MFMA rows
+          (300, 136, 768, DType.F32), (27, 330, 2048, DType.BF16), (13, 72, 768, DType.F32),  # the last two: 17..32 MFMA rows
+          (40, 48, 4096, DType.BF16)]  # sixteen super-blocks per row, K split across workgroups
 
 
 def run_matmul(scheme, blocks, m, n, k, dtype):
@@ -321,6 +322,34 @@ def test_q8k_layout_for_n_gt_1():
     assert rel_err(got, x.astype(np.float64) @ w.astype(np.float64).T) <= 2e-3
     assert np.allclose(got, oracle.gguf_matmul_bt(x, packed, m, k, n, Q8K), rtol=2e-3, atol=2e-3)
     qw.free()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("m", [3, 70])  # decode launch; prefill launch(es) on the step's one workspace
+def test_graph_step_mixes_k_quants_on_one_input(m):
+    """Four matmuls of one step read the same activations with four schemes: Q4_K wants 32-column activation sums next to
+    the prefill image, Q2_K 16-column ones, Q3_K (Q6_K units) and Q8_K none. Each must get the image it needs out of the
+    step's single workspace."""
+    from rlx_amd import Graph, Session, Shape
+    k = 512
+    schemes = [(Q4K, 40), (Q2K, 24), (Q3K, 56), (Q8K, 16), (Q2K, 33), (Q4K, 17)]
+    g = Graph.new("mixed")
+    x = g.input("x", Shape.new([m, k], DType.F32))
+    packed, outs = [], []
+    for i, (scheme, n) in enumerate(schemes):
+        d_std, dmin_std = MODEL_SCALE.get(scheme, (4e-5, 2e-5))
+        blocks = random_blocks(scheme, n, k, seed=200 + i, d_std=d_std, dmin_std=dmin_std)
+        packed.append(blocks)
+        w = g.param(f"w{i}", Shape.new([blocks.size], DType.U8))
+        outs.append(g.dequant_matmul_packed(x, w, QuantScheme(scheme), Shape.new([m, n], DType.F32)))
+    g.set_outputs(outs)
+    exe = Session.new().compile(g)
+    for i, blocks in enumerate(packed):
+        exe.set_param_typed(f"w{i}", blocks, DType.U8)
+    xv = np.random.default_rng(m).standard_normal((m, k)).astype(np.float32)
+    got = exe.run([("x", xv)])
+    for (scheme, n), blocks, y in zip(schemes, packed, got):
+        assert rel_err(y.reshape(m, n), oracle.gguf_matmul_f64(xv, blocks, m, k, n, scheme)) <= 2e-3, (scheme, n)
 
 
 @pytest.mark.gpu
