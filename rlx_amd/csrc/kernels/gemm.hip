@@ -549,7 +549,54 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
     if (grp == 0) run(std::integral_constant<int, 0>{});
     else run(std::integral_constant<int, 1>{});
 
-    // ---- epilogue: register e of tile (i, j) is row 8 (e/4) + 4 lh + e%4, column lr ------------------------
+    // ---- epilogue ------------------------------------------------------------------------------------------
+    // Register e of tile (i, j) is row 8 (e/4) + 4 lh + e%4, column lr. Written straight from the registers a wave stores
+    // 128 contiguous bytes per output row and instruction, 64 instructions per 64 x 64 wave tile, and the store issue is
+    // what the end of the kernel waits for (every workgroup of the launch finishes at the same time). When the output
+    // rows can take 16-byte stores the wave turns its tile around through LDS instead (the stages are free by now):
+    // 32 image rows at a time, every lane then owns four consecutive columns of a row and a store instruction covers four
+    // whole rows of the wave tile.
+    if (!a.use_atomics && (sg.n & 3) == 0) {
+        constexpr int STRIDE = TJ * 32 + 8;  // floats per row: lanes 32-63 (four rows further) land 32 banks away
+        __syncthreads();                     // the last stage has been read by every wave
+        float *tile = (float *)smem + wave * (32 * STRIDE);
+        const int out_base = a.pair_rows ? wm * TI * 16 : wm * TI * 32;  // first entry of this wave in out_row_s / out_fac_s
+        constexpr int LPR = TJ * 8, RPI = 64 / LPR;  // lanes per row of the wave tile (four columns each), rows per instruction
+        const int c4 = (lane % LPR) * 4, col = n_tile0 + wn * TJ * 32 + c4;
+#pragma unroll
+        for (int i = 0; i < TI; i++) {
+#pragma unroll
+            for (int j = 0; j < TJ; j++)
+#pragma unroll
+                for (int e = 0; e < 16; e++) {
+                    int row = 8 * (e >> 2) + 4 * lh + (e & 3);
+                    float v = total[i][j][e];
+                    if (a.pair_rows) {
+                        if (e & 1) continue;
+                        v = v + total[i][j][e + 1] * (1.0f / GEMM_LO_SCALE);
+                        row >>= 1;
+                    }
+                    tile[row * STRIDE + j * 32 + lr] = v;
+                }
+            const int rows = a.pair_rows ? 16 : 32;  // output rows of this pass
+#pragma unroll
+            for (int it = 0; it < 32 / RPI; it++) {
+                const int r = it * RPI + lane / LPR;
+                if (it * RPI >= rows) break;  // wave-uniform: with paired rows the tile holds half as many
+                const int slot = out_base + i * rows + r;
+                const int orow = out_row_s[slot];
+                const float fac = out_fac_s[slot];
+                float4_t v = *(const float4_t *)(tile + r * STRIDE + c4);
+                if (orow >= 0 && col < sg.n) {
+#pragma unroll
+                    for (int q = 0; q < 4; q++) v[q] *= fac;  // undo the row's prescale
+                    __builtin_nontemporal_store(v, (float4_t *)(sg.out + (long long)orow * sg.n + col));
+                }
+            }
+        }
+        return;
+    }
+    // Otherwise (K split across workgroups, or a row length that is no multiple of four):
     // The four rows of a register quad are neighbours, so their output rows and factors come as one 16-byte LDS read
     // each (8 bytes with f32 activations, where two image rows make one output row), shared by the tiles j.
 #pragma unroll
