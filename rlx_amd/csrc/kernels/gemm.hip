@@ -556,7 +556,7 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
     // rows can take 16-byte stores the wave turns its tile around through LDS instead (the stages are free by now):
     // 32 image rows at a time, every lane then owns four consecutive columns of a row and a store instruction covers four
     // whole rows of the wave tile.
-    if (!a.use_atomics && (sg.n & 3) == 0) {
+    if (!a.use_atomics && (sg.n & 3) == 0 && ((uintptr_t)sg.out & 15) == 0) {
         constexpr int STRIDE = TJ * 32 + 8;  // floats per row: lanes 32-63 (four rows further) land 32 banks away
         __syncthreads();                     // the last stage has been read by every wave
         float *tile = (float *)smem + wave * (32 * STRIDE);

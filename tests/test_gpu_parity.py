@@ -729,6 +729,27 @@ def test_prefill_prepare_then_prepared(oracle, scheme, x_dtype):
         rlx_amd._lib.check(L.rlx_mi355x_gguf_matmul_prepare(xd.ptr, int(x_dtype), int(scheme), 4, k, wsb.ptr, need, None))
 
 
+@pytest.mark.parametrize("scheme,m,n,x_dtype", [(Q4_0, 40, 64, DType.BF16), (Q4K, 300, 128, DType.F32), (Q8_0, 64, 132, DType.BF16)])
+def test_prefill_output_that_is_only_4_byte_aligned(oracle, scheme, m, n, x_dtype):
+    # the prefill epilogue stores 16 bytes per lane when the output rows allow it; an output pointer that is only a
+    # multiple of four bytes takes the element-wise stores and must give the same numbers
+    k = 512
+    rng = np.random.default_rng(m + n)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    xin = f32_to_bf16_bits(oracle.bf16_round(x)) if x_dtype == DType.BF16 else x
+    packed = make_weights(scheme, n, k, seed=77)[0]
+    w = ops.QWeight(scheme, packed, n, k)
+    L = rlx_amd._lib.lib()
+    need = ops.matmul_workspace_bytes(w, x_dtype, m)
+    wsb, xd = ops.DeviceBuffer(need), ops.DeviceBuffer.from_numpy(xin)
+    out = ops.DeviceBuffer(m * n * 4 + 16)
+    rlx_amd._lib.check(L.rlx_mi355x_gguf_matmul_bt(xd.ptr, int(x_dtype), w.ptr, out.ptr + 4, m, wsb.ptr, need, None))
+    ops.sync()
+    got = out.to_numpy(np.float32)[1:1 + m * n].reshape(m, n)
+    assert np.array_equal(got.view(np.uint32), ops.gguf_matmul_bt(xin, w, m, x_dtype).view(np.uint32))
+    w.free()
+
+
 # ------------------------------------------------------------------ activations beyond what binary16 carries
 
 @pytest.mark.parametrize("scheme,m,k,x_dtype", [(Q4_0, 1, 4096, DType.F32), (Q4K, 3, 1024, DType.F32), (Q8_0, 7, 512, DType.BF16),
