@@ -39,7 +39,7 @@ CALIBRATION_COPY_BYTES = 256 << 20
 # HBM bytes per launch of the headline kernel (FETCH_SIZE + WRITE_SIZE of two rocprofv3 --pmc runs of this command,
 # each scaled by the same counter's reading for the copy kernel above, the 478-workgroup dispatches of the kernel only);
 # profiles/gemv_q4_0_layer_and_gemm_q4_k_m512_traffic.txt.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 124286348
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 124285646
 
 # (name, N, K) — the Llama-3-8B layer projections of the headline workload
 LLAMA8B = [("q", 4096, 4096), ("k", 1024, 4096), ("v", 1024, 4096), ("o", 4096, 4096),
