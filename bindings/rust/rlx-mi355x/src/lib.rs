@@ -19,8 +19,8 @@ use std::os::raw::c_void;
 
 use rlx_driver::Device;
 use rlx_ir::quant::QuantScheme;
-use rlx_ir::op::SteKind;
-use rlx_ir::{DType, Graph, Node, Op, OpKind, ScaleMode};
+use rlx_ir::op::{ScaleMode, SteKind};
+use rlx_ir::{DType, Graph, Node, Op, OpKind};
 use rlx_runtime::backend::{Backend, ExecutableGraph};
 use rlx_runtime::options::CompileOptions;
 use rlx_runtime::registry::register_backend;

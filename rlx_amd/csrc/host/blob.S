@@ -1,10 +1,17 @@
-/* The gfx950 code object, embedded verbatim; loaded with hipModuleLoadData at first use. */
+/* The gfx950 code objects, one per kernel source, embedded verbatim; loaded with hipModuleLoadData at first use. */
     .section .rodata
+.macro blob name
     .balign 4096
-    .global rlx_kernels_blob
-    .global rlx_kernels_blob_end
-rlx_kernels_blob:
-    .incbin "build/rlx_kernels.co"
-rlx_kernels_blob_end:
+    .global rlx_blob_\name
+rlx_blob_\name:
+    .incbin "build/\name\().co"
     .byte 0
+.endm
+    blob dequant
+    blob fakequant
+    blob gemm
+    blob gemv
+    blob moe
+    blob rowops
+    blob topk
     .section .note.GNU-stack,"",@progbits

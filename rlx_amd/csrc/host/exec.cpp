@@ -514,6 +514,9 @@ static std::unique_ptr<rlx_exec> plan_graph(const rlx_graph_desc *g, const rlx_c
         std::vector<int> step_idx(e->nodes.size(), -1);
         for (size_t si = 0; si < e->steps.size(); si++)
             for (uint32_t id : e->steps[si]) step_idx[id] = (int)si;
+        // A step has one workspace, so one image: the first FakeQuantize that targets a step owns it, a later one (matmuls
+        // of equal depth on another FakeQuantize result share the step) keeps its f32 tensor and goes through the conversion.
+        std::vector<bool> has_image(e->steps.size(), false);
         for (uint32_t f = 0; f < g->n_nodes; f++) {
             Node &fq = e->nodes[f];
             if (fq.d.op_kind != RLX_OP_FAKE_QUANTIZE || fq.inner != 1 || fq.chan_dim % 8 != 0 || fq.numel % fq.chan_dim != 0) continue;
@@ -537,7 +540,8 @@ static std::unique_ptr<rlx_exec> plan_graph(const rlx_graph_desc *g, const rlx_c
                 }
             }
             for (uint32_t id : e->outputs) other_reader = other_reader || id == f;
-            if (!ok || target < 0) continue;
+            if (!ok || target < 0 || has_image[target]) continue;
+            has_image[target] = true;
             fq.img_step = target;
             fq.keep_f32 = other_reader;
             for (uint32_t j : mms) e->nodes[j].x_image = true;
@@ -635,8 +639,13 @@ static std::unique_ptr<rlx_exec> plan_graph(const rlx_graph_desc *g, const rlx_c
                 nd.aux = take(rlx_mi355x_fake_quantize_scratch_bytes(nd.numel, nd.chan_dim, nd.inner), (int)si, (int)si);
                 if (e->opts.fq_emit_codes) nd.codes = take((size_t)nd.numel, (int)si, kForever);
             }
-            if (nd.d.op_kind == RLX_OP_DEQUANT_GROUPED_MATMUL) {  // above the decode sizes: the expert-sorted path's workspace (f32 is the larger)
-                const size_t need = rlx_mi355x_gguf_grouped_matmul_workspace((int)nd.d.scheme, RLX_F32, nd.m, nd.k, e->nodes[nd.d.inputs[1]].w_experts);
+            if (nd.d.op_kind == RLX_OP_DEQUANT_GROUPED_MATMUL) {
+                // Above the decode sizes: the expert-sorted path's workspace. The input's dtype is known when it is written, so
+                // the slot covers both widths: f32 rows are twice as wide, 16-bit rows pad every expert's run to 64 rows
+                // instead of 32, and with more experts than rows the padding decides.
+                const int64_t ne = e->nodes[nd.d.inputs[1]].w_experts;
+                const size_t need = std::max(rlx_mi355x_gguf_grouped_matmul_workspace((int)nd.d.scheme, RLX_F32, nd.m, nd.k, ne),
+                                             rlx_mi355x_gguf_grouped_matmul_workspace((int)nd.d.scheme, RLX_BF16, nd.m, nd.k, ne));
                 if (need) nd.aux = take(need, (int)si, (int)si);
             }
             if (nd.d.op_kind == RLX_OP_DEQUANT_MATMUL && nd.m > 16)  // may run the prefill kernels (which one is decided by the input dtype at run time): sized for f32

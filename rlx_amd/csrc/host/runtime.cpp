@@ -3,10 +3,12 @@
 #include <cstring>
 #include <mutex>
 
-extern "C" const unsigned char rlx_kernels_blob[];
-extern "C" const unsigned char rlx_kernels_blob_end[];
+extern "C" const unsigned char rlx_blob_dequant[], rlx_blob_fakequant[], rlx_blob_gemm[], rlx_blob_gemv[], rlx_blob_moe[], rlx_blob_rowops[],
+    rlx_blob_topk[];
 
 namespace rlx {
+
+int static_scratch_ptr(void **ptr);  // host/static_scratch.hip
 
 static thread_local std::string g_error;
 
@@ -51,7 +53,10 @@ static const char *const kKernelNames[K_COUNT] = {
 static std::once_flag g_once;
 static int g_init_rc = RLX_ERR_NO_DEVICE;
 static std::string g_init_error;
-static hipModule_t g_module;
+static const unsigned char *const kBlobs[] = {rlx_blob_dequant, rlx_blob_fakequant, rlx_blob_gemm, rlx_blob_gemv,
+                                              rlx_blob_moe,     rlx_blob_rowops,    rlx_blob_topk};
+constexpr int kModules = (int)(sizeof kBlobs / sizeof kBlobs[0]);
+static hipModule_t g_module[kModules];
 static hipFunction_t g_fn[K_COUNT];
 static DeviceProps g_props;
 
@@ -75,14 +80,20 @@ static int do_init() {
     g_props.lds_per_block = p.sharedMemPerBlock;
     snprintf(g_props.arch, sizeof g_props.arch, "%s", p.gcnArchName);
     snprintf(g_props.name, sizeof g_props.name, "%s", p.name);
-    RLX_HIP(hipModuleLoadData(&g_module, rlx_kernels_blob));
+    for (int m = 0; m < kModules; m++) RLX_HIP(hipModuleLoadData(&g_module[m], kBlobs[m]));
     for (int i = 0; i < K_COUNT; i++) {
-        hipError_t fe = hipModuleGetFunction(&g_fn[i], g_module, kKernelNames[i]);
+        hipError_t fe = hipErrorNotFound;  // a kernel lives in exactly one of the code objects
+        for (int m = 0; m < kModules && fe != hipSuccess; m++) fe = hipModuleGetFunction(&g_fn[i], g_module[m], kKernelNames[i]);
+        (void)hipGetLastError();
         if (fe != hipSuccess) {
             set_error("hipModuleGetFunction(%s): %s", kKernelNames[i], hipGetErrorString(fe));
             return RLX_ERR_HIP;
         }
     }
+    // The array behind rlx_mi355x_fake_quantize_noalloc: looking its address up loads the code object that holds it, which
+    // allocates; done here, once, so that the entry point itself only reads the cached pointer.
+    void *scratch = nullptr;
+    RLX_TRY(static_scratch_ptr(&scratch));
     return RLX_OK;
 }
 

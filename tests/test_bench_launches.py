@@ -179,6 +179,38 @@ def test_config4_chain_full_size(oracle, fq_is_output):
         assert err <= TOL
 
 
+def test_two_fake_quantize_producers_in_one_step(oracle):
+    # Two FakeQuantize nodes of equal depth, each feeding a prefill matmul of the same scheme: the matmuls land in one step,
+    # whose single workspace can hold one operand image. The first producer writes the image; the second keeps its f32
+    # tensor, and both results must be those of their own input (different K, so a mix-up cannot pass).
+    rows, ka, kb, n = 300, 512, 1024, 96
+    rng = np.random.default_rng(65)
+    xa = rng.standard_normal((rows, ka)).astype(np.float32)
+    xb = (rng.standard_normal((rows, kb)) * 3.0).astype(np.float32)
+    pa = tiled_packed(Q8_0, n, ka, 66, 0.02).reshape(-1)
+    pb = tiled_packed(Q8_0, n, kb, 67, 0.02).reshape(-1)
+    g = Graph.new("two_fq")
+    ia = g.input("xa", Shape.new([rows, ka], DType.F32))
+    ib = g.input("xb", Shape.new([rows, kb], DType.F32))
+    fa = g.add_node(Op.FakeQuantize(8, 1), [ia], Shape.new([rows, ka], DType.F32))
+    fb = g.add_node(Op.FakeQuantize(8, 1), [ib], Shape.new([rows, kb], DType.F32))
+    wa = g.param("wa", Shape.new([len(pa)], DType.U8))
+    wb = g.param("wb", Shape.new([len(pb)], DType.U8))
+    ya = g.add_node(Op.DequantMatMul(QuantScheme.GgufQ8_0), [fa, wa], Shape.new([rows, n], DType.F32))
+    yb = g.add_node(Op.DequantMatMul(QuantScheme.GgufQ8_0), [fb, wb], Shape.new([rows, n], DType.F32))
+    g.set_outputs([ya, yb])
+    c = Session().compile(g)
+    assert c.describe_plan().count("-> prefill image") == 1
+    c.set_param_typed("wa", pa, DType.U8)
+    c.set_param_typed("wb", pb, DType.U8)
+    got = c.run([("xa", xa), ("xb", xb)])
+    for name, y, x, p, k in (("a", got[0], xa, pa, ka), ("b", got[1], xb, pb, kb)):
+        fq_ref, _, _ = oracle.fake_quantize(x, x.shape, 1, 8)
+        err = rel_err(y.reshape(rows, n), oracle.gguf_matmul_f64(fq_ref, p, rows, k, n, Q8_0))
+        say(f"   two FakeQuantize producers, matmul {name}: max rel err {err:.3e}")
+        assert err <= TOL
+
+
 def test_fq_image_chain_ragged_and_out_of_range(oracle):
     # the same chain at a ragged shape (m not a multiple of 256, k not of 256, two matmuls on the fake-quantized tensor) and
     # with inputs far outside binary16: the tensor-wide power of two keeps the image in range

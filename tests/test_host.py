@@ -199,6 +199,50 @@ def test_plan_reuses_dead_slots():
     assert Session(fq_codes=True).plan(g)[0] >= total_all + 64 * 4096
 
 
+def _two_fq_graph(rows=64, ka=256, kb=512, n=32):
+    # two FakeQuantize nodes of equal depth, each feeding a prefill matmul: the matmuls share one step and one workspace
+    g = Graph.new("two_fq")
+    xa = g.input("xa", Shape.new([rows, ka], DType.F32))
+    xb = g.input("xb", Shape.new([rows, kb], DType.F32))
+    fa = g.add_node(Op.FakeQuantize(8, 1), [xa], Shape.new([rows, ka], DType.F32))
+    fb = g.add_node(Op.FakeQuantize(8, 1), [xb], Shape.new([rows, kb], DType.F32))
+    w1 = g.param("w1", Shape.new([n * ka // 32 * 34], DType.U8))
+    w2 = g.param("w2", Shape.new([n * kb // 32 * 34], DType.U8))
+    y1 = g.add_node(Op.DequantMatMul(QuantScheme.GgufQ8_0), [fa, w1], Shape.new([rows, n], DType.F32))
+    y2 = g.add_node(Op.DequantMatMul(QuantScheme.GgufQ8_0), [fb, w2], Shape.new([rows, n], DType.F32))
+    g.set_outputs([y1, y2])
+    return g, dict(fa=fa, fb=fb, y1=y1, y2=y2)
+
+
+def test_plan_gives_a_step_workspace_one_image_owner():
+    # The workspace of a step holds one operand image. The first FakeQuantize that feeds the step writes it; a second
+    # one keeps its f32 tensor and its matmul converts that tensor like any other input.
+    g, ids = _two_fq_graph()
+    lines = Session().plan(g)[1].splitlines()[1:]
+    assert "-> prefill image" in lines[ids["fa"]] and "[x: binary16 image]" in lines[ids["y1"]]
+    assert "-> prefill image" not in lines[ids["fb"]] and "[x: binary16 image]" not in lines[ids["y2"]]
+    assert int(lines[ids["fb"]].split("size=")[1].split()[0]) == 64 * 512 * 4   # the second result has its f32 slot
+    assert int(lines[ids["fa"]].split("size=")[1].split()[0]) == 0
+
+
+def test_plan_grouped_matmul_workspace_covers_both_input_widths():
+    # more experts than rows: 16-bit rows pad each expert's run to 64 rows, f32 rows to 32, so the 16-bit workspace is
+    # the larger one; the slot must hold either, since the input's dtype is only known when it is written
+    L = rlx_amd._lib.lib()
+    m, k, n, experts = 40, 4096, 32, 64
+    g = Graph.new("moe_ws")
+    x = g.input("x", Shape.new([m, k], DType.F32))
+    w = g.param("w", Shape.new([experts * n * k // 32 * 18], DType.U8))
+    idx = g.input("idx", Shape.new([m], DType.F32))
+    y = g.add_node(Op.DequantGroupedMatMul(QuantScheme.GgufQ4_0), [x, w, idx], Shape.new([m, n], DType.F32))
+    g.set_outputs([y])
+    f32 = L.rlx_mi355x_gguf_grouped_matmul_workspace(int(Q4_0), int(DType.F32), m, k, experts)
+    b16 = L.rlx_mi355x_gguf_grouped_matmul_workspace(int(Q4_0), int(DType.BF16), m, k, experts)
+    assert b16 > f32 > 0
+    line = Session().plan(g)[1].splitlines()[1 + y]
+    assert int(line.split("workspace@")[1].split("+")[1].split()[0]) >= b16
+
+
 def _llama_mlp_graph(m, k=256, n=512, norm_is_output=False):
     # RmsNorm -> q, k; RmsNorm -> [up | gate] -> FusedSwiGLU -> down: the ops around the hot path as the reference's
     # graphs hold them (rlx-ir/src/op.rs:574-578, 1157-1172)

@@ -98,6 +98,29 @@ def test_sorted_grouped_matmul_through_session_and_replays(oracle):
             c.capture()
 
 
+def test_sorted_grouped_matmul_through_session_bf16_more_experts_than_rows(oracle):
+    # 16-bit rows pad every expert's run to 64 rows (f32: 32), so with more experts than rows the bf16 workspace is the
+    # larger one; the executable's slot has to hold it although the input is declared F32 and written as BF16
+    m, k, n, experts = 40, 512, 32, 64
+    packed = stack(Q4_0, n, k, experts, seed=360)
+    g = Graph.new("moe_prefill_bf16")
+    x_in = g.input("x", Shape.new([m, k], DType.F32))
+    w = g.param("w_packed", Shape.new([packed.size], DType.U8))
+    i_in = g.input("expert_idx", Shape.new([m], DType.F32))
+    g.set_outputs([g.add_node(Op.DequantGroupedMatMul(QuantScheme.GgufQ4_0), [x_in, w, i_in], Shape.new([m, n], DType.F32))])
+    c = Session.new().compile(g)
+    c.set_param_typed("w_packed", packed, DType.U8)
+    rng = np.random.default_rng(10)
+    x = oracle.bf16_round(rng.standard_normal((m, k)).astype(np.float32))
+    idx = rng.integers(0, experts, m).astype(np.float32)
+    for dt, xin in ((DType.BF16, f32_to_bf16_bits(x)), (DType.F32, x)):
+        c.write_input("x", xin, dt)
+        c.write_input("expert_idx", idx)
+        c.launch()
+        got = c.read_output(0).reshape(m, n)
+        assert rel_err(got, oracle.gguf_grouped_matmul_f64(x, packed, idx, m, k, n, experts, Q4_0)) <= TOL, dt
+
+
 def test_grouped_workspace_is_zero_where_the_decode_path_runs():
     L = rlx_amd._lib.lib()
     assert L.rlx_mi355x_gguf_grouped_matmul_workspace(int(Q4_0), int(DType.F32), 16, 256, 8) == 0

@@ -61,6 +61,41 @@ def test_noalloc_matches_scratch_variant(first, second, scale_mode):
                 assert np.array_equal(got[2].view(np.uint32), want[2].view(np.uint32))
 
 
+def test_noalloc_inside_a_stream_capture_replays_like_the_scratch_variant():
+    # What the entry point is for: once the library is initialised (is_available() resolves the scratch array's address), a
+    # call made while a stream capture is in progress records kernels only. The capture is done here with the HIP
+    # runtime the library links, the graph is replayed three times with new input in between, and every replay is compared
+    # with an eager call of the scratch-argument entry point on the same input.
+    assert rlx_amd.is_available(), rlx_amd._lib.last_error()
+    L = rlx_amd._lib.lib()
+    hip = C.CDLL("libamdhip64.so")  # the copy the library already loaded
+    rows, chan = 1024, 768
+    n = rows * chan
+    rng = np.random.default_rng(11)
+    xd, od, cd = ops.DeviceBuffer(n * 4), ops.DeviceBuffer(n * 4), ops.DeviceBuffer(n)
+    stream = C.c_void_p()
+    rlx_amd._lib.check(L.rlx_mi355x_stream_create(C.byref(stream)))
+    graph, gexec = C.c_void_p(), C.c_void_p()
+    assert hip.hipStreamBeginCapture(stream, 1) == 0  # hipStreamCaptureModeThreadLocal
+    rc = L.rlx_mi355x_fake_quantize_noalloc(xd.ptr, od.ptr, cd.ptr, n, chan, 1, 8, 0, 0.0, None, 0, stream)
+    assert hip.hipStreamEndCapture(stream, C.byref(graph)) == 0
+    rlx_amd._lib.check(rc)
+    assert hip.hipGraphInstantiate(C.byref(gexec), graph, None, None, C.c_size_t(0)) == 0
+    scratch = ops.DeviceBuffer(L.rlx_mi355x_fake_quantize_scratch_bytes(n, chan, 1))
+    for replay in range(3):
+        x = (rng.standard_normal(n) * (1.0 + replay)).astype(np.float32)
+        x[::811] *= np.float32(20.0)
+        rlx_amd._lib.check(L.rlx_mi355x_memcpy_h2d(xd.ptr, x.ctypes.data, x.nbytes))
+        assert hip.hipGraphLaunch(gexec, stream) == 0
+        ops.sync(stream)
+        got_out, got_codes = od.to_numpy(np.float32), cd.to_numpy(np.int8)
+        want = _run("scratch", x, chan, 1, 8, 0, None, 0, scratch)
+        assert np.array_equal(got_out.view(np.uint32), want[0].view(np.uint32)), replay
+        assert np.array_equal(got_codes, want[1]), replay
+    assert hip.hipGraphExecDestroy(gexec) == 0 and hip.hipGraphDestroy(graph) == 0
+    rlx_amd._lib.check(L.rlx_mi355x_stream_destroy(stream))
+
+
 def test_noalloc_rejects_shapes_beyond_its_scratch():
     L = rlx_amd._lib.lib()
     cap = L.rlx_mi355x_fake_quantize_noalloc_max_scratch()
