@@ -682,7 +682,8 @@ def gemm_configs(rlx_amd, stream):
     xq[ops.philox_uniform(19, rows * cols) < np.float32(0.001)] *= np.float32(20.0)
     xd, fd, yd = ops.DeviceBuffer.from_numpy(xq), ops.DeviceBuffer(rows * cols * 4), ops.DeviceBuffer(rows * 4096 * 4)
     scratch = ops.DeviceBuffer(L.rlx_mi355x_fake_quantize_scratch_bytes(rows * cols, cols, 1))
-    need = ops.matmul_workspace_bytes(qw[0], DType.F32, rows)
+    need = max(ops.matmul_workspace_bytes(qw[0], DType.F32, rows),
+               L.rlx_mi355x_gguf_matmul_workspace(int(QuantScheme.GgufQ8_0), int(DType.I8), rows, cols, 4096))
     ws = ops.DeviceBuffer(need)
     w_arr = (rlx_amd._lib.C.c_void_p * 1)(qw[0].ptr)
     y_arr = (rlx_amd._lib.C.c_void_p * 1)(yd.ptr)
@@ -693,7 +694,7 @@ def gemm_configs(rlx_amd, stream):
 
     def chain_image():
         rlx_amd._lib.check(L.rlx_mi355x_fake_quantize_image(xd.ptr, None, None, rows, cols, 8, 0, 0.0, None, 0, scratch.ptr, ws.ptr, need, stream))
-        rlx_amd._lib.check(L.rlx_mi355x_gguf_matmul_bt_prepared(ws.ptr, need, int(DType.F32), w_arr, y_arr, 1, rows, stream))
+        rlx_amd._lib.check(L.rlx_mi355x_gguf_matmul_bt_prepared(ws.ptr, need, int(DType.I8), w_arr, y_arr, 1, rows, stream))
 
     def fq_image_only():
         rlx_amd._lib.check(L.rlx_mi355x_fake_quantize_image(xd.ptr, None, None, rows, cols, 8, 0, 0.0, None, 0, scratch.ptr, ws.ptr, need, stream))
@@ -704,7 +705,7 @@ def gemm_configs(rlx_amd, stream):
     out["fq_then_q8_0_gemm_8192x4096x4096"] = {
         "us_fq_f32_then_matmul": round(ms_a * 1e3, 2), "us_fq_image_then_prepared_matmul": round(ms_b * 1e3, 2),
         "us_fq_image_alone": round(ms_c * 1e3, 2),
-        "note": "the image holds hi + lo binary16 rows: one row alone was 2.8e-3 from the f64 result, above the 2e-3 bound"}
+        "note": "the image holds the integer codes (exact in binary16, one row per token); the column scales are multiplied into the weights"}
     qw[0].free()
 
     # config 5: Q4_0 batch sweep over the seven projections of one Llama-3-70B layer, bf16 activations

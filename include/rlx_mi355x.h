@@ -256,7 +256,8 @@ int rlx_mi355x_qweight_rows(const rlx_qweight *w, int64_t row0, int64_t rows, rl
  * (its thunk converts nothing). ..._prepare writes the binary16 image of x[m, k] (and, for Q4_K / Q5_K, its block
  * sums) into `workspace` (rlx_mi355x_gguf_matmul_workspace(scheme, x_dtype, m, k, 0) bytes); ..._bt_prepared multiplies
  * that image by `count` matrices, all with the k the image was made for: outs_dev[i][m, n_i]. An image made for Q4_K / Q5_K also
- * serves the other schemes, not the other way round. */
+ * serves the other schemes, not the other way round. x_dtype = RLX_I8 names the code image rlx_mi355x_fake_quantize_image
+ * leaves (see there). */
 int rlx_mi355x_gguf_matmul_prepare(const void *x_dev, int x_dtype, int scheme, int64_t m, int64_t k, void *workspace,
                                    size_t workspace_bytes, void *stream);
 int rlx_mi355x_gguf_matmul_bt_prepared(const void *workspace, size_t workspace_bytes, int x_dtype, const rlx_qweight *const *ws,
@@ -276,13 +277,16 @@ int rlx_mi355x_fake_quantize(const float *x_dev, float *out_dev, int8_t *codes_d
                              int round_mode, void *scratch_dev, void *stream);
 
 /* FakeQuantize whose result feeds prefill matmuls (the benchmark's FakeQuantize -> Q8_0 GEMM chain): x is [m, k] with one
- * channel per column (the layout of axis = last). Besides out_dev - which may be NULL here: the f32 tensor is then never
- * written - the apply pass writes the binary16 image of the result into `workspace`, in the form
- * rlx_mi355x_gguf_matmul_bt_prepared(workspace, .., RLX_F32, ..) reads (two binary16 rows per row, as for any f32
- * activation), so the result needs no round trip through HBM as f32 and no conversion pass.
- * workspace: rlx_mi355x_gguf_matmul_workspace(scheme, RLX_F32, m, k, 0) bytes of a scheme without block sums (any but
- * Q4_K / Q5_K). k % 8 == 0. No counterpart in the reference, whose thunks exchange f32 tensors; the graph
- * level uses it when every consumer of a FakeQuantize node is such a matmul. */
+ * channel per column (the layout of axis = last). The result is q[i][c] * s[c] with integer codes |q| <= 127, so the
+ * product with W^T is sum_c q[i][c] * (s[c] * W[j][c]): besides out_dev - which may be NULL here: the f32 tensor is then
+ * never written - the apply pass writes into `workspace` an operand image of the codes (exact in binary16, one row per
+ * row of x) and the column scales, and rlx_mi355x_gguf_matmul_bt_prepared(workspace, .., RLX_I8, ..) multiplies that image
+ * by weights of any scheme, scaling each matrix by s[c] into ready binary16 operands first (one rounding of
+ * W[j][c] * s[c] computed in f32; the reference rounds q * s to f32, rlx-cpu/src/thunk.rs:11242-11251, then accumulates
+ * in f32, rlx-cpu/src/gguf_matmul.rs:81-94). workspace: rlx_mi355x_gguf_matmul_workspace(scheme, RLX_I8, m, k, n) bytes
+ * with n the widest matrix it will be multiplied by (n = 0: what this call alone writes). k % 8 == 0. No counterpart in
+ * the reference, whose thunks exchange f32 tensors; the graph level uses it when prefill matmuls of one step read a
+ * FakeQuantize node. */
 int rlx_mi355x_fake_quantize_image(const float *x_dev, float *out_dev, int8_t *codes_dev, int64_t m, int64_t k, int bits,
                                    int scale_mode, float ema_decay, float *state_dev, int round_mode, void *scratch_dev,
                                    void *workspace, size_t workspace_bytes, void *stream);

@@ -507,9 +507,10 @@ static std::unique_ptr<rlx_exec> plan_graph(const rlx_graph_desc *g, const rlx_c
         e->steps.push_back(step);
     }
 
-    // FakeQuantize -> prefill DequantMatMul: when every reader of a FakeQuantize result is a prefill matmul of one step
-    // (and of a scheme whose kernel needs no block sums), the apply pass writes the matmuls' binary16 image itself and
-    // the f32 tensor never goes through memory; when other readers exist both are written.
+    // FakeQuantize -> prefill DequantMatMul: a FakeQuantize result with column channels is codes times column scales, so
+    // when prefill matmuls of one step read it, the apply pass writes their operand image itself - the integer codes as
+    // binary16, with the scales left for the matmul to multiply into its weights - and the f32 tensor goes through memory
+    // only when something else reads it as well.
     {
         std::vector<int> step_idx(e->nodes.size(), -1);
         for (size_t si = 0; si < e->steps.size(); si++)
@@ -527,8 +528,7 @@ static std::unique_ptr<rlx_exec> plan_graph(const rlx_graph_desc *g, const rlx_c
                 Node &o = e->nodes[j];
                 for (uint32_t t = 0; t < o.d.n_inputs; t++) {
                     if (o.d.inputs[t] != f) continue;
-                    const bool as_x = o.d.op_kind == RLX_OP_DEQUANT_MATMUL && t == 0 && o.m > 16 && o.k == fq.chan_dim &&
-                                      act_sums_kind((int)o.d.scheme) == 0;
+                    const bool as_x = o.d.op_kind == RLX_OP_DEQUANT_MATMUL && t == 0 && o.m > 16 && o.k == fq.chan_dim;
                     if (!as_x) {
                         other_reader = true;
                     } else if (target >= 0 && step_idx[j] != target) {
@@ -650,6 +650,8 @@ static std::unique_ptr<rlx_exec> plan_graph(const rlx_graph_desc *g, const rlx_c
             }
             if (nd.d.op_kind == RLX_OP_DEQUANT_MATMUL && nd.m > 16)  // may run the prefill kernels (which one is decided by the input dtype at run time): sized for f32
                 step_ws = std::max(step_ws, rlx_mi355x_gguf_matmul_workspace((int)nd.d.scheme, RLX_F32, nd.m, nd.k, nd.n));
+            if (nd.x_image)  // the code image a FakeQuantize writes, and this matrix scaled by its column scales
+                step_ws = std::max(step_ws, rlx_mi355x_gguf_matmul_workspace((int)nd.d.scheme, RLX_I8, nd.m, nd.k, nd.n));
         }
         if (step_ws) {  // one workspace for the whole step; it is born earlier when a FakeQuantize writes the step's image into it
             int birth = (int)si;
@@ -880,7 +882,7 @@ static int enqueue_schedule(rlx_exec *e) {
             std::stable_sort(order.begin(), order.end(), [&](uint32_t a, uint32_t b) {
                 return e->nodes[a].d.inputs[0] < e->nodes[b].d.inputs[0];
             });
-            {  // matmuls whose activations a FakeQuantize left in the workspace as a binary16 image: first, while it is intact
+            {  // matmuls whose activations a FakeQuantize left in the workspace as a code image: first, while it is intact
                 std::vector<const rlx_qweight *> iw;
                 std::vector<float *> io;
                 for (uint32_t id : order) {
@@ -895,7 +897,7 @@ static int enqueue_schedule(rlx_exec *e) {
                     io.push_back((float *)e->ptr(mm.slot));
                 }
                 if (!iw.empty())
-                    RLX_TRY(rlx_mi355x_gguf_matmul_bt_prepared(e->ptr(nd.aux), nd.aux.size, RLX_F32, iw.data(), io.data(), (int)iw.size(), nd.m,
+                    RLX_TRY(rlx_mi355x_gguf_matmul_bt_prepared(e->ptr(nd.aux), nd.aux.size, RLX_I8, iw.data(), io.data(), (int)iw.size(), nd.m,
                                                                e->stream));
             }
             std::vector<const rlx_qweight *> ws;
@@ -1156,7 +1158,7 @@ int rlx_exec_describe_plan(const rlx_exec *e, char *buf, size_t cap) {
         if (nd.d.op_kind == RLX_OP_DEQUANT_MATMUL && nd.aux.size) put(" step workspace@%zu+%zu", nd.aux.offset, nd.aux.size);
         if (nd.d.op_kind == RLX_OP_DEQUANT_GROUPED_MATMUL && nd.aux.size) put(" expert-sorted, workspace@%zu+%zu", nd.aux.offset, nd.aux.size);
         if (nd.img_step >= 0) put(" -> prefill image of step %d%s", nd.img_step, nd.keep_f32 ? "" : " (f32 tensor not written)");
-        if (nd.x_image) put(" [x: binary16 image]");
+        if (nd.x_image) put(" [x: code image]");
         if (nd.d.op_kind == RLX_OP_RMS_NORM || nd.d.op_kind == RLX_OP_FUSED_SWIGLU) put(" h=%lld", (long long)nd.h);
         if (nd.folded) put("%s", nd.d.op_kind == RLX_OP_RMS_NORM ? " (folded into the matmuls that read it)" : " (folded into the FusedSwiGLU that reads it)");
         if (nd.norm_of >= 0) put(" [x: normalized while staged, RmsNorm node %d]", nd.norm_of);

@@ -73,6 +73,15 @@ struct FqArgs {
     void *img;
     float *rowfac;
     int k_pad, m_rows, write_out;
+    float *colscale;
+};
+struct WScaleArgs {  // mirrors kernels/dequant.hip
+    const uint8_t *w;
+    void *wimg;
+    const float *cs;
+    const float *rowfac;
+    long long row_tiles, units;
+    int k_pad, sc_off;
 };
 
 constexpr int GEMM_MAX_SEG = 4;
@@ -110,6 +119,9 @@ struct MoeSortArgs {  // mirrors kernels/moe.hip
     int *tile_expert;
 };
 
+// Kinds of activation operand: 0 f32, 1 bf16, 2 f16 tensors; XK_CODES: the workspace image a FakeQuantize left
+// (rlx_mi355x_fake_quantize_image: integer codes as binary16 plus the column scales), named RLX_I8 at the boundary.
+constexpr int XK_CODES = 3;
 static int x_kind(int x_dtype) {
     switch (x_dtype) {
     case RLX_F32: return 0;
@@ -304,21 +316,28 @@ static int launch_gemv(const void *const *xs, int xk, const rlx_qweight *const *
     return launch(id, (unsigned)sh.wg, 1, (unsigned)sh.nwaves * 64, (unsigned)sh.lds, stream, params);
 }
 
+// Workspace of a prefill matmul: [per-row factors][column scales][image of x][block sums][image of the scaled weights].
+// The second and the last exist only for a FakeQuantize code image (XK_CODES), whose matmul runs on ready binary16
+// weights W * diag(s) (n is the widest matrix multiplied from the image, one at a time).
 struct GemmPlan {
     int64_t m_rows, k_pad;
     size_t xh_bytes, sxh_bytes, fac_bytes;  // the image, the block sums (Q4_K / Q5_K per 32 columns, Q2_K per 16), the per-row prescale factors
+    size_t cs_bytes, wimg_bytes;
     int sums_kind;                          // act_sums_kind of the scheme the plan was made for
-    size_t total() const { return xh_bytes + sxh_bytes + fac_bytes; }
+    size_t image_end() const { return fac_bytes + cs_bytes + xh_bytes + sxh_bytes; }
+    size_t total() const { return image_end() + wimg_bytes; }
 };
-static GemmPlan gemm_plan(int scheme, int xk, int64_t m, int64_t k) {
+static GemmPlan gemm_plan(int scheme, int xk, int64_t m, int64_t k, int64_t n = 0) {
     GemmPlan p;
     const int64_t rv = xk == 0 ? 2 * m : m;
     p.m_rows = (rv + 255) / 256 * 256;
     p.k_pad = (k + 255) / 256 * 256;
     p.xh_bytes = ((size_t)p.m_rows * p.k_pad * 2 + 255) & ~(size_t)255;
-    p.sums_kind = act_sums_kind(scheme);
+    p.sums_kind = xk == XK_CODES ? 0 : act_sums_kind(scheme);
     p.sxh_bytes = (size_t)p.m_rows * (p.k_pad / 256) * 32 * p.sums_kind;  // 16 or 32 halfs per row and super-block
     p.fac_bytes = ((size_t)m * 8 + 255) & ~(size_t)255;
+    p.cs_bytes = xk == XK_CODES ? (size_t)p.k_pad * 4 : 0;
+    p.wimg_bytes = xk == XK_CODES ? (size_t)((n + 127) / 128 * 128) * p.k_pad * 2 : 0;
     return p;
 }
 
@@ -328,7 +347,7 @@ static int launch_xprep(const void *x, int xk, int64_t m, int64_t k, const GemmP
                         const int *perm = nullptr, int perm_len = 0) {
     float *fac = (float *)workspace;
     void *xh = (uint8_t *)workspace + p.fac_bytes;
-    void *sxh = p.sxh_bytes ? (uint8_t *)workspace + p.fac_bytes + p.xh_bytes : nullptr;
+    void *sxh = p.sxh_bytes ? (uint8_t *)workspace + p.fac_bytes + p.cs_bytes + p.xh_bytes : nullptr;
     XPrepArgs xa{x, xh, sxh, (int)m, (int)k, (int)p.k_pad, (int)p.m_rows, xk, fac, perm, perm_len, p.sums_kind == 2};
     void *xparams[] = {&xa};
     RLX_TRY(launch(K_XROWSCALE, (unsigned)((m + 3) / 4), 1, 256, 0, stream, xparams));
@@ -345,13 +364,14 @@ static int launch_xprep(const void *x, int xk, int64_t m, int64_t k, const GemmP
 // them) from the previous launch of a batch on the same stream, so the conversion pass is skipped.
 static int launch_gemm(const void *x, int xk, const rlx_qweight *const *ws, float *const *outs, int count, int64_t m,
                        void *workspace, size_t workspace_bytes, hipStream_t stream, bool prepared = false) {
-    if (count < 1 || count > GEMM_MAX_SEG) {
+    if (count < 1 || count > GEMM_MAX_SEG || (xk == XK_CODES && count != 1)) {
         set_error("gguf_matmul_bt: %d matrices in one prefill launch", count);
         return RLX_ERR_INVALID;
     }
     const rlx_qweight *w = ws[0];
-    const Layout L = w->layout;
-    const GemmPlan p = gemm_plan(w->scheme, xk, m, w->dims.k);
+    const bool codes = xk == XK_CODES;  // the workspace holds a FakeQuantize code image; the weights are scaled into it first
+    const Layout L = codes ? Layout{64, 0, 0, 0, 0} : w->layout;
+    const GemmPlan p = gemm_plan(w->scheme, xk, m, w->dims.k, w->dims.n);
     for (int i = 1; i < count; i++)
         if (ws[i]->scheme != w->scheme || ws[i]->dims.k != w->dims.k || ws[i]->dims.units != w->dims.units ||
             ws[i]->layout.unit_bytes != L.unit_bytes || ws[i]->sc_off() != w->sc_off()) {
@@ -369,9 +389,24 @@ static int launch_gemm(const void *x, int xk, const rlx_qweight *const *ws, floa
     // workspace: [per-row prescale factors][binary16 image of x][block sums], so that an image made for a scheme with
     // block sums is found at the same place by a scheme without
     float *fac = (float *)workspace;
-    void *xh = (uint8_t *)workspace + p.fac_bytes;
-    void *sxh = p.sxh_bytes ? (uint8_t *)workspace + p.fac_bytes + p.xh_bytes : nullptr;
-    if (!prepared) RLX_TRY(launch_xprep(x, xk, m, w->dims.k, p, workspace, stream));
+    void *xh = (uint8_t *)workspace + p.fac_bytes + p.cs_bytes;
+    void *sxh = p.sxh_bytes ? (uint8_t *)workspace + p.fac_bytes + p.cs_bytes + p.xh_bytes : nullptr;
+    uint8_t *wimg = (uint8_t *)workspace + p.image_end();
+    if (codes) {  // B = fl16(W * diag(s) / S) as stage images; fac holds (1 / S, S) for every row
+        WScaleArgs wa{w->dev, wimg, (const float *)((uint8_t *)workspace + p.fac_bytes), fac, w->dims.row_tiles, w->dims.units, (int)p.k_pad, w->sc_off()};
+        void *wparams[] = {&wa};
+        const KernelId wid = w->scheme == SCHEME_Q4K    ? K_WSCALE_Q4_K
+                             : w->scheme == SCHEME_Q4_0 ? K_WSCALE_Q4_0
+                             : w->scheme == SCHEME_Q6K  ? K_WSCALE_Q6_K
+                             : w->scheme == SCHEME_Q5K  ? K_WSCALE_Q5_K
+                             : w->scheme == SCHEME_Q8K  ? K_WSCALE_Q8_K
+                             : w->scheme == SCHEME_Q2K  ? K_WSCALE_Q2_K
+                                                        : K_WSCALE_Q8_0;
+        RLX_TRY(launch(wid, (unsigned)(p.k_pad / w->layout.unit_k), (unsigned)((w->dims.n + 127) / 128 * 8), 64, 0, stream, wparams));
+    } else if (!prepared) {
+        RLX_TRY(launch_xprep(x, xk, m, w->dims.k, p, workspace, stream));
+    }
+    const int64_t k_units = codes ? p.k_pad / 64 : w->dims.units;  // K units of the operand the kernel reads
 
     const int steps_per_unit = L.unit_k / 64;
     // Up to 128 activation rows run the 64-row tile (the weights are decoded once per 64 rows, but nothing is spent on
@@ -381,7 +416,7 @@ static int launch_gemm(const void *x, int xk, const rlx_qweight *const *ws, floa
     GemmArgs a{};
     long long gx = 0;
     for (int i = 0; i < count; i++) {
-        a.seg[i] = GemmSeg{ws[i]->dev, outs[i], (int)ws[i]->dims.n, (int)ws[i]->dims.row_tiles, (int)gx};
+        a.seg[i] = GemmSeg{codes ? wimg : ws[i]->dev, outs[i], (int)ws[i]->dims.n, (int)ws[i]->dims.row_tiles, (int)gx};
         gx += (ws[i]->dims.row_tiles * 16 + 127) / 128;
     }
     a.nseg = count;
@@ -389,11 +424,12 @@ static int launch_gemm(const void *x, int xk, const rlx_qweight *const *ws, floa
     // workgroup slots to fill: one per CU for the 256-row tile (144 KB of LDS), two for the 64-row tile
     const long long slots = (long long)std::max(1, device_props().cu_count) * (skinny ? 2 : 1);
     int split = 1;
-    if (gx * gy * 5 < slots * 4) split = (int)std::min<long long>(w->dims.units, slots / (gx * gy));
+    if (gx * gy * 5 < slots * 4) split = (int)std::min<long long>(k_units, slots / (gx * gy));
     split = std::max(1, split);
-    int units_per_split = (int)((w->dims.units + split - 1) / split);
-    if (steps_per_unit == 2) units_per_split = (units_per_split + 1) & ~1;  // keep every split a multiple of 4 steps
-    split = (int)((w->dims.units + units_per_split - 1) / units_per_split);
+    int units_per_split = (int)((k_units + split - 1) / split);
+    const int upq = 4 / steps_per_unit;  // units in four steps: every split is a multiple of that
+    if (upq > 1) units_per_split = (units_per_split + upq - 1) / upq * upq;
+    split = (int)((k_units + units_per_split - 1) / units_per_split);
     if (split > 1)
         for (int i = 0; i < count; i++) RLX_TRY(rlx_mi355x_memset_u32(outs[i], 0, (size_t)m * ws[i]->dims.n, stream));
     a.xh = xh;
@@ -401,14 +437,15 @@ static int launch_gemm(const void *x, int xk, const rlx_qweight *const *ws, floa
     a.m_rows = (int)p.m_rows;
     a.m_out = (int)m;
     a.k_pad = (int)p.k_pad;
-    a.units = (int)w->dims.units;
+    a.units = (int)k_units;
     a.pair_rows = xk == 0 ? 1 : 0;
     a.steps_per_split = units_per_split * steps_per_unit;
     a.use_atomics = split > 1 ? 1 : 0;
     a.sc_off = w->sc_off();
     a.rowfac = fac;
     void *params[] = {&a};
-    KernelId id = w->scheme == SCHEME_Q4K       ? (skinny ? K_GEMM64_Q4_K : K_GEMM_Q4_K)
+    KernelId id = codes                         ? (skinny ? K_GEMM64_F16W : K_GEMM_F16W)
+                  : w->scheme == SCHEME_Q4K     ? (skinny ? K_GEMM64_Q4_K : K_GEMM_Q4_K)
                   : w->scheme == SCHEME_Q4_0    ? (skinny ? K_GEMM64_Q4_0 : K_GEMM_Q4_0)
                   : w->scheme == SCHEME_Q6K     ? (skinny ? K_GEMM64_Q6_K : K_GEMM_Q6_K)
                   : w->scheme == SCHEME_Q5K     ? (skinny ? K_GEMM64_Q5_K : K_GEMM_Q5_K)
@@ -540,7 +577,8 @@ int rlx_mi355x_dequant(const rlx_qweight *w, float *out_dev, void *stream) {
 
 size_t rlx_mi355x_gguf_matmul_workspace(int scheme, int x_dtype, int64_t m, int64_t k, int64_t n) {
     using namespace rlx;
-    (void)n;
+    if (x_dtype == RLX_I8)  // a FakeQuantize code image and the scaled weights of the widest matrix it is multiplied by
+        return layout_of(scheme).unit_k == 0 || m <= 0 || k <= 0 || n <= 0 ? 0 : gemm_plan(scheme, XK_CODES, m, k, n).total();
     int xk = x_kind(x_dtype);
     if (xk < 0 || layout_of(scheme).unit_k == 0 || m <= decode_rows(xk)) return 0;  // decode path: no workspace
     return gemm_plan(scheme, xk, m, k).total();
@@ -636,8 +674,8 @@ int rlx_mi355x_gguf_matmul_prepare(const void *x_dev, int x_dtype, int scheme, i
 int rlx_mi355x_gguf_matmul_bt_prepared(const void *workspace, size_t workspace_bytes, int x_dtype, const rlx_qweight *const *ws,
                                        float *const *outs_dev, int count, int64_t m, void *stream) {
     using namespace rlx;
-    const int xk = x_kind(x_dtype);
-    if (!workspace || !ws || !outs_dev || count <= 0 || xk < 0 || m <= decode_rows(xk)) {
+    const int xk = x_dtype == RLX_I8 ? XK_CODES : x_kind(x_dtype);
+    if (!workspace || !ws || !outs_dev || count <= 0 || xk < 0 || m <= (xk == XK_CODES ? 0 : decode_rows(xk))) {
         set_error("gguf_matmul_bt_prepared: null argument, count=%d, or m=%lld within the decode limit", count, (long long)m);
         return RLX_ERR_INVALID;
     }
@@ -646,6 +684,11 @@ int rlx_mi355x_gguf_matmul_bt_prepared(const void *workspace, size_t workspace_b
             set_error("gguf_matmul_bt_prepared: null weight / output %d", i);
             return RLX_ERR_INVALID;
         }
+    if (xk == XK_CODES) {  // one matrix at a time: each is scaled into the workspace's weight image first
+        for (int i = 0; i < count; i++)
+            RLX_TRY(launch_gemm(workspace, xk, ws + i, outs_dev + i, 1, m, const_cast<void *>(workspace), workspace_bytes, (hipStream_t)stream, true));
+        return RLX_OK;
+    }
     for (int i = 0; i < count;) {
         int c = 1;
         while (i + c < count && c < GEMM_MAX_SEG && ws[i + c]->scheme == ws[i]->scheme && ws[i + c]->dims.k == ws[i]->dims.k &&
@@ -1148,14 +1191,14 @@ static int fake_quantize_impl(const float *x_dev, float *out_dev, int8_t *codes_
     const bool col = plan.col && ((uintptr_t)x_dev % 16 == 0) && ((uintptr_t)out_dev % 16 == 0) &&
                      ((uintptr_t)scratch_dev % 16 == 0) && (!codes_dev || (uintptr_t)codes_dev % 8 == 0 || (!img_ws && (uintptr_t)codes_dev % 4 == 0));
     FqArgs a{x_dev, out_dev, codes_dev, max_bits, scale, state_dev, len, chan_dim, inner, q_max, ema_decay,
-             scale_mode, round_mode, 0, nullptr, 0, nullptr, nullptr, 0, 0, 1};
+             scale_mode, round_mode, 0, nullptr, 0, nullptr, nullptr, 0, 0, 1, nullptr};
     GemmPlan ip{};
     if (img_ws) {
         const int64_t m = chan_dim > 0 ? len / chan_dim : 0;
-        ip = gemm_plan(SCHEME_Q8_0, 0, m, chan_dim);  // the image of an f32 tensor (hi / lo row pairs), no block sums
-        if (!col || chan_dim % 8 != 0 || (uintptr_t)img_ws % 16 != 0 || img_ws_bytes < ip.total()) {
+        ip = gemm_plan(SCHEME_Q8_0, XK_CODES, m, chan_dim);  // one image row of integer codes per row, plus the column scales
+        if (!col || chan_dim % 8 != 0 || (uintptr_t)img_ws % 16 != 0 || img_ws_bytes < ip.image_end()) {
             set_error("FakeQuantize: the prefill image needs column channels in multiples of 8, 16-byte aligned buffers and %zu bytes of workspace",
-                      ip.total());
+                      ip.image_end());
             return RLX_ERR_INVALID;
         }
     }
@@ -1183,14 +1226,15 @@ static int fake_quantize_impl(const float *x_dev, float *out_dev, int8_t *codes_
     if (a.partial) RLX_TRY(launch(K_FQ_SCALE_PARTS, (unsigned)((chan_dim + 63) / 64), 1, 1024, 0, s, params));
     else RLX_TRY(launch(K_FQ_SCALE, (unsigned)((chan_dim + 255) / 256), 1, 256, 0, s, params));
     if (img_ws) {
-        a.img = (uint8_t *)img_ws + ip.fac_bytes;
+        a.img = (uint8_t *)img_ws + ip.fac_bytes + ip.cs_bytes;
         a.rowfac = (float *)img_ws;
+        a.colscale = (float *)((uint8_t *)img_ws + ip.fac_bytes);
         a.k_pad = (int)ip.k_pad;
         a.m_rows = (int)ip.m_rows;
         a.write_out = out_dev ? 1 : 0;
         const unsigned gx = (unsigned)((ip.k_pad + 255) / 256);
-        const int64_t want = std::max<int64_t>(1, 4096 / gx), lrows = ip.m_rows / 2;  // logical rows, padding included (a multiple of 128)
-        a.rows_per_block = (int)std::max<int64_t>(16, ((lrows + want - 1) / want + 15) / 16 * 16);
+        const int64_t want = std::max<int64_t>(1, 4096 / gx), lrows = ip.m_rows;  // image rows, padding included (a multiple of 256)
+        a.rows_per_block = (int)std::max<int64_t>(32, ((lrows + want - 1) / want + 31) / 32 * 32);
         RLX_TRY(launch(K_FQ_COL_APPLY_IMG, gx, (unsigned)((lrows + a.rows_per_block - 1) / a.rows_per_block), 256, 0, s, params));
     } else if (col) {
         a.rows_per_block = plan.rpb_apply;

@@ -29,11 +29,12 @@ struct FqArgs {
     int rows_per_block;  // col kernels: rows per workgroup; seg kernel: elements per part
     float *partial;      // col pass A: [parts][chan_dim] maxima per row block (no atomics, nothing to clear); else null
     int parts;
-    // rlx_fq_col_apply_img only: the binary16 image a prefill matmul reads (kernels/gemm.hip, rlx_xprep's format)
+    // rlx_fq_col_apply_img only: the binary16 image of the integer codes a prefill matmul reads (kernels/gemm.hip, rlx_xprep's format)
     void *img;           // [m_rows / 256][k_pad / 64][32 KB]
-    float *rowfac;       // [rows][2]: the power of two every row was multiplied by, and its inverse
+    float *rowfac;       // [rows][2]: (inv, S), see col_apply_img
     int k_pad, m_rows;
     int write_out;       // 0: only the image (and the codes, if wanted) is written
+    float *colscale;     // rlx_fq_col_apply_img only: [k_pad] copy of the column scales for the weight-scaling pass
 };
 
 __device__ __forceinline__ float fq_scale_from_max(float max_abs, float q_max) {
@@ -215,19 +216,19 @@ __device__ __forceinline__ void col_apply(const FqArgs &a) {
     }
 }
 
-// Pass B for a FakeQuantize whose result feeds prefill matmuls of the same executable: besides (or instead of) the f32
-// tensor it writes the binary16 image those matmuls read, in the LDS-stage order rlx_xprep produces (one 32 KB block per
-// 256-row tile and 64-column step; slot of row r, 8-column chunk c: k-slice c / 2, half c % 2, lane ((r ^ c) & 31) + 32
-// (c % 2)), so the f32 tensor need not make a round trip through HBM and a conversion kernel. As for any f32 activation,
-// logical row i becomes image rows 2 i (the value rounded to binary16) and 2 i + 1 (the residual times 2048): a single
-// binary16 row was measured at 2.8e-3 of the f64 result on the benchmark's heavy-tailed [8192, 4096] case, above the
-// 2e-3 bound. One power of two for the whole tensor (from the largest column scale) keeps the values inside the
-// binary16 range; the matmul epilogue undoes it. blockIdx.x covers 256 channels, blockIdx.y rows_per_block (a multiple
-// of 16) logical rows up to m_rows / 2 (the padding of the image is written as zeros).
+// Pass B for a FakeQuantize whose result feeds prefill matmuls: besides (or instead of) the f32 tensor it writes what those
+// matmuls read. The result is q[i][c] * s[c] with small integer codes, so the matmul is run on the codes, which binary16
+// holds exactly, with s[c] multiplied into the weights (rlx_wscale_* in kernels/dequant.hip). Written here:
+//   img      the codes as binary16 in the LDS-stage order of the prefill kernel, one image row per logical row (one 32 KB
+//            block per 256-row tile and 64-column step; slot of row r, 8-column chunk c: k-slice c / 2, half c % 2,
+//            lane ((r ^ c) & 31) + 32 (c % 2)); padding rows and columns are zeros
+//   colscale s[c] for c < k_pad (zeros past the channels)
+//   rowfac   for every row (inv, S): S the power of two with max s[c] / S in [1, 2); the weights are scaled by s[c] * inv
+//            and the matmul epilogue multiplies by S
+// blockIdx.x covers 256 channels, blockIdx.y rows_per_block (a multiple of 32) rows up to m_rows.
 __device__ __forceinline__ void col_apply_img(const FqArgs &a) {
     __shared__ float wave_max[4];
     const int tid = threadIdx.x;
-    // the largest column scale -> largest possible |out| = q_max * s_max -> the tensor's power of two
     float smax = 0.f;
     for (long long c = tid; c < a.chan_dim; c += blockDim.x) {
         const float v = a.scale[c];
@@ -242,64 +243,67 @@ __device__ __forceinline__ void col_apply_img(const FqArgs &a) {
     __syncthreads();
     smax = wave_max[0];
     for (int w = 1; w < (int)(blockDim.x >> 6); w++) smax = wave_max[w] > smax ? wave_max[w] : smax;
-    const float amax = smax * a.q_max;
-    float fwd = 1.f, back = 1.f;
-    const uint32_t mb = __builtin_bit_cast(uint32_t, amax);
-    if (mb != 0 && mb < 0x7F800000u && (amax >= 1024.0f || amax < 0.00390625f)) {
+    float inv = 1.f, big = 1.f;
+    const uint32_t mb = __builtin_bit_cast(uint32_t, smax);
+    if (mb >= 0x00800000u && mb < 0x7F800000u) {  // a normal number: its exponent
         int e = (int)(mb >> 23) - 127;
-        e = e < -100 ? -100 : e;
-        fwd = __builtin_bit_cast(float, (uint32_t)(9 - e + 127) << 23);
-        back = __builtin_bit_cast(float, (uint32_t)(e - 9 + 127) << 23);
+        e = e < -100 ? -100 : e > 100 ? 100 : e;
+        inv = __builtin_bit_cast(float, (uint32_t)(127 - e) << 23);
+        big = __builtin_bit_cast(float, (uint32_t)(127 + e) << 23);
     }
     const long long rows = a.len / a.chan_dim;
     long long r0 = (long long)blockIdx.y * a.rows_per_block, r1 = r0 + a.rows_per_block;
-    if (r1 > a.m_rows / 2) r1 = a.m_rows / 2;  // m_rows counts image rows: two per logical row
+    if (r1 > a.m_rows) r1 = a.m_rows;
     if (blockIdx.x == 0)
         for (long long r = r0 + tid; r < r1 && r < rows; r += blockDim.x) {
-            a.rowfac[2 * r] = fwd;
-            a.rowfac[2 * r + 1] = back;
+            a.rowfac[2 * r] = inv;
+            a.rowfac[2 * r + 1] = big;
         }
-    // A workgroup walks tiles of 16 logical rows x 256 channels. Lanes run along the channels for the loads (1 KB of a
-    // row per half wave); the 32 x 256 binary16 tile is put together in LDS in image order and leaves as sixteen
-    // contiguous 1 KB blocks (one per 16-channel slice), a full wave store each.
+    // A workgroup walks tiles of 32 rows x 256 channels. Lanes run along the channels for the loads (1 KB of a row per
+    // half wave); the 32 x 256 binary16 tile is put together in LDS in image order and leaves as sixteen contiguous 1 KB
+    // blocks (one per 16-channel slice), a full wave store each.
     __shared__ uint4_t tile_img[1024];  // [step in tile 0..3][ks 0..3][slot 0..63]
     const int cc = tid & 31, rl = tid >> 5;
     const long long c8 = ((long long)blockIdx.x * 32 + cc) * 8;
     const bool live_col = c8 < a.chan_dim;  // chan_dim is a multiple of 8: a chunk is inside or outside as a whole
-    float4_t s0 = {1.f, 1.f, 1.f, 1.f}, s1 = s0;
+    float4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = s0;
     if (live_col) {
         s0 = *(const float4_t *)(a.scale + c8);
         s1 = *(const float4_t *)(a.scale + c8 + 4);
     }
+    if (blockIdx.y == 0 && rl == 0 && c8 < a.k_pad) {
+        *(float4_t *)(a.colscale + c8) = s0;
+        *(float4_t *)(a.colscale + c8 + 4) = s1;
+    }
     const int steps = a.k_pad / 64;
     const int c = cc & 7, ks = c >> 1, h = c & 1;
     uint4_t *lds_col = tile_img + ((cc >> 3) * 4 + ks) * 64 + 32 * h;
-    for (long long t0 = r0; t0 < r1; t0 += 16) {
+    for (long long t0 = r0; t0 < r1; t0 += 32) {
 #pragma unroll
-        for (int pass = 0; pass < 2; pass++) {
+        for (int pass = 0; pass < 4; pass++) {
             const int lr = rl + 8 * pass;
             const long long r = t0 + lr;
-            Frag fh, fl;
-            fh.u4 = uint4_t{0, 0, 0, 0};
-            fl.u4 = uint4_t{0, 0, 0, 0};
+            Frag fq;
+            fq.u4 = uint4_t{0, 0, 0, 0};
             if (live_col && r < rows) {
                 const long long at = r * a.chan_dim + c8;
                 const float4_t v0 = __builtin_nontemporal_load((const float4_t *)(a.x + at));
                 const float4_t v1 = __builtin_nontemporal_load((const float4_t *)(a.x + at + 4));
-                float4_t q0, q1, y0, y1;
+                float4_t q0, q1;
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
                     q0[e] = fq_code(v0[e], s0[e], a.q_max, a.round_mode);
                     q1[e] = fq_code(v1[e], s1[e], a.q_max, a.round_mode);
-                    y0[e] = q0[e] * s0[e];
-                    y1[e] = q1[e] * s1[e];
-                    const float u0 = y0[e] * fwd, u1 = y1[e] * fwd;
-                    fh.h8[e] = (half_t)u0;
-                    fh.h8[4 + e] = (half_t)u1;
-                    fl.h8[e] = (half_t)((u0 - (float)fh.h8[e]) * 2048.0f);
-                    fl.h8[4 + e] = (half_t)((u1 - (float)fh.h8[4 + e]) * 2048.0f);
+                    fq.h8[e] = (half_t)q0[e];  // |q| <= 127: exact
+                    fq.h8[4 + e] = (half_t)q1[e];
                 }
                 if (a.write_out) {
+                    float4_t y0, y1;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        y0[e] = q0[e] * s0[e];
+                        y1[e] = q1[e] * s1[e];
+                    }
                     __builtin_nontemporal_store(y0, (float4_t *)(a.out + at));
                     __builtin_nontemporal_store(y1, (float4_t *)(a.out + at + 4));
                 }
@@ -312,14 +316,11 @@ __device__ __forceinline__ void col_apply_img(const FqArgs &a) {
                     *(uint2_t *)(a.codes + at) = packed;
                 }
             }
-            const int rr = 2 * lr;  // image rows 2 r (hi) and 2 r + 1 (lo) of this 32-row sub-tile
-            lds_col[(rr ^ c) & 31] = fh.u4;
-            lds_col[((rr + 1) ^ c) & 31] = fl.u4;
+            lds_col[(lr ^ c) & 31] = fq.u4;
         }
         __syncthreads();
-        const long long vr = 2 * t0;
-        const long long tile = vr >> 8;
-        const int sub = (int)(vr & 255) >> 5;
+        const long long tile = t0 >> 8;
+        const int sub = (int)(t0 & 255) >> 5;
 #pragma unroll
         for (int p = 0; p < 4; p++) {
             const int blk = p * 4 + (tid >> 6), lane = tid & 63;

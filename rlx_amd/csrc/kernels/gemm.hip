@@ -79,7 +79,10 @@ __device__ __forceinline__ int frag_offset(int ns, int ks, int s, int r, int h) 
 // padding. Both read the same activation workspace (a 64-row tile is two 32-row sub-tiles of a 256-row image).
 template <int SCHEME, int TI, int TJ, bool GROUPED = false>
 __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
-    constexpr Layout L = layout_of(SCHEME);
+    // IMG: the weights arrive as ready binary16 images of the LDS stage (one 16 KB block per 128-row tile and 64-column
+    // step, see rlx_wscale_*), so a "unit" is one step and the data half moves 16-byte chunks unchanged.
+    constexpr bool IMG = SCHEME == SCHEME_F16W;
+    constexpr Layout L = IMG ? Layout{GEMM_KS, GEMM_STAGE_B / 8, 0, 0, 0} : layout_of(SCHEME);
     constexpr bool K5 = SCHEME == SCHEME_Q5K;                 // Q4_K with a fifth bit: every Q4_K branch below serves both
     constexpr bool K4 = SCHEME == SCHEME_Q4K || K5;
     constexpr bool K6 = SCHEME == SCHEME_Q6K;
@@ -126,7 +129,8 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
     const int b_n16 = lane & 15, b_g = lane >> 4;
     const int b_t16 = bx * (GEMM_NT / 16) + wave;
     const bool b_live = b_t16 < sg.row_tiles;
-    const uint8_t *b_tile = w_base + (long long)(b_live ? b_t16 : 0) * a.units * L.unit_bytes;
+    const uint8_t *b_tile = IMG ? w_base + (long long)bx * a.units * GEMM_STAGE_B  // this tile's run of stage images
+                                : w_base + (long long)(b_live ? b_t16 : 0) * a.units * L.unit_bytes;
     const uint32_t b_keep = b_live ? 0xFFFFFFFFu : 0u;
     const half2_t sc_bias = ubyte_bias(a.sc_off);                 // Q6_K scale bytes: value = byte - sc_off
     const uint32_t sc_dead = (uint32_t)a.sc_off * 0x01010101u;    // the byte that reads as a zero scale
@@ -144,6 +148,7 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
     uint4_t b_meta[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};   // Q4_K: [0] = meta of the super-block decoded next; else [chunk parity] .x/.y = four f16 scales
     uint2_t b_hw[2] = {{0, 0}, {0, 0}};                 // Q6_K: [chunk parity] high-bit words of the two code-word pairs of a half
     uint32_t b_sc[2] = {0, 0};                          // Q4_K: 6-bit scales of sub-blocks 0-3 / 4-7 being decoded
+    uint4_t b_img[2][2] = {{{0, 0, 0, 0}, {0, 0, 0, 0}}, {{0, 0, 0, 0}, {0, 0, 0, 0}}};  // IMG: [step parity] chunks tid and tid + 512 of a stage image
 
     // Activations run AD steps ahead of their LDS store: two where registers allow (their loads come through L2 with
     // the whole workgroup's 32 KB per step behind them), one for Q4_K whose second accumulator set takes the room.
@@ -158,7 +163,10 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
         for (int i = 0; i < 4; i++) a_reg[AD == 2 ? set : 0][i] = ld128(a_rsrc, a_src0, step * GEMM_STAGE_A + i * 8192);
     };
     auto fetch_b = [&](int step, int q) {  // q = step & 3, compile-time at every call site
-        if constexpr (K4) {  // dead tiles read tile 0 (valid memory) and are zeroed when stored
+        if constexpr (IMG) {
+            b_img[q & 1][0] = ld128(b_rsrc, tid * 16, step * GEMM_STAGE_B);
+            b_img[q & 1][1] = ld128(b_rsrc, tid * 16, step * GEMM_STAGE_B + 8192);
+        } else if constexpr (K4) {  // dead tiles read tile 0 (valid memory) and are zeroed when stored
             const int unit = (step >> 2) * L.unit_bytes;
             if ((q & 1) == 0) {
                 b_q[(q >> 1) & 1] = ld128(b_rsrc, lane * 16, unit + (q >> 1) * 1024);
@@ -209,6 +217,10 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
         const int cp = (q >> 1) & 1;
         const int t = 2 * (q & 1) + jl;
         Frag f;
+        if constexpr (IMG) {
+            *(uint4_t *)(stage + SA + tid * 16 + jl * 8192) = b_img[q & 1][jl];
+            return;
+        }
         if constexpr (K4) {
             if (q == 0 && jl == 0) {
                 uint32_t mn[2];
@@ -821,5 +833,7 @@ extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64g_q4_0(rlx::GemmA
 extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64g_q8_0(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q8_0, 1, 1, true>(a); }
 extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64g_q5_k(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q5K, 1, 1, true>(a); }
 extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64g_q6_k(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q6K, 1, 1, true>(a); }
+extern "C" __global__ __launch_bounds__(512) void rlx_gemm_f16w(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_F16W, 2, 2>(a); }
+extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64_f16w(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_F16W, 1, 1>(a); }
 extern "C" __global__ __launch_bounds__(256) void rlx_xprep(rlx::XPrepArgs a) { rlx::xprep_body(a); }
 extern "C" __global__ __launch_bounds__(256) void rlx_xrowscale(rlx::XPrepArgs a) { rlx::xrowscale_body(a); }

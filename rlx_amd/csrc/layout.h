@@ -62,6 +62,10 @@ enum Scheme : int {
     SCHEME_Q4_0 = 11, SCHEME_Q8_0 = 12
 };
 
+// Not a GGUF scheme: ready binary16 operand images of the prefill kernel (weights already multiplied by per-column
+// scales, see rlx_wscale_* in kernels/dequant.hip). Never the scheme of a weight; names the prefill instantiation only.
+constexpr int SCHEME_F16W = 100;
+
 // fifth bit of element e inside a Q5_K high-bit word (after the rotate of its code word), and the rotates
 RLX_HD constexpr int q5k_hi_pos(int e) { return e == 0 ? 4 : e == 1 ? 20 : e == 2 ? 8 : e == 3 ? 24 : e == 4 ? 5 : e == 5 ? 21 : e == 6 ? 9 : 25; }
 RLX_HD constexpr int q5k_rot(int t) { return t == 0 ? 0 : t == 1 ? 2 : t == 2 ? 8 : 10; }

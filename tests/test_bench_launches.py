@@ -229,7 +229,7 @@ def test_fq_image_chain_ragged_and_out_of_range(oracle):
             outs.append(g.add_node(Op.DequantMatMul(QuantScheme.GgufQ4_0), [fq, w], Shape.new([rows, n], DType.F32)))
         g.set_outputs(outs)
         c = Session().compile(g)
-        assert c.describe_plan().count("[x: binary16 image]") == 2
+        assert c.describe_plan().count("[x: code image]") == 2
         for i, p in enumerate(packs):
             c.set_param_typed(f"w{i}", p, DType.U8)
         got = c.run([("x", x)])
