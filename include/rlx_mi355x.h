@@ -154,7 +154,11 @@ int rlx_mi355x_dequant(const rlx_qweight *w, float *out_dev, void *stream);
  *   out[m, n] = x[m, k] . W^T, W = decoded [n, k]; out is overwritten (the reference zero-fills first).
  * x_dev is [m,k] row-major of x_dtype in {RLX_F32, RLX_BF16, RLX_F16}; 16-bit activations stand for the values
  * the reference's typed boundary would widen to f32 (rlx-runtime/src/backend.rs:49-53). out_dev is f32.
- * `workspace` must hold rlx_mi355x_gguf_matmul_workspace() bytes (may be NULL when that is 0).
+ * `workspace` must hold rlx_mi355x_gguf_matmul_workspace() bytes (may be NULL when that is 0): the converted
+ * activations and, where the output tiles alone would leave most of the chip idle and K is cut across workgroups, the
+ * partial results of the K slices, which a reduce launch adds in ascending K (the order the reference walks a row in), so
+ * results are the same bits on every run. A workspace that holds only the activations (n = 0 in the size call) is
+ * accepted: K is then cut in fewer slices or not at all.
  * m <= 16 (f32 activations) or m <= 32 (bf16 / f16) runs the decode kernels (weights streamed once, MFMA 16x16x32, one
  * or two groups of 16 rows per decoded weight fragment, an f32 row taking two); larger m runs the prefill GEMM. */
 int rlx_mi355x_gguf_matmul_bt(const void *x_dev, int x_dtype, const rlx_qweight *w, float *out_dev, int64_t m,
@@ -281,9 +285,10 @@ int rlx_mi355x_fake_quantize(const float *x_dev, float *out_dev, int8_t *codes_d
  * product with W^T is sum_c q[i][c] * (s[c] * W[j][c]): besides out_dev - which may be NULL here: the f32 tensor is then
  * never written - the apply pass writes into `workspace` an operand image of the codes (exact in binary16, one row per
  * row of x) and the column scales, and rlx_mi355x_gguf_matmul_bt_prepared(workspace, .., RLX_I8, ..) multiplies that image
- * by weights of any scheme, scaling each matrix by s[c] into ready binary16 operands first (one rounding of
- * W[j][c] * s[c] computed in f32; the reference rounds q * s to f32, rlx-cpu/src/thunk.rs:11242-11251, then accumulates
- * in f32, rlx-cpu/src/gguf_matmul.rs:81-94). workspace: rlx_mi355x_gguf_matmul_workspace(scheme, RLX_I8, m, k, n) bytes
+ * by Q4_0 / Q8_0 weights, scaling each matrix by s[c] into ready binary16 operands first (one rounding of
+ * W[j][c] * s[c] computed in f32, where the plain prefill kernels of these two schemes round d * code; the reference
+ * rounds q * s to f32, rlx-cpu/src/thunk.rs:11242-11251, then accumulates in f32, rlx-cpu/src/gguf_matmul.rs:81-94).
+ * Other schemes are RLX_ERR_UNSUPPORTED there: their prefill operands are exact integers, and they take the f32 tensor. workspace: rlx_mi355x_gguf_matmul_workspace(scheme, RLX_I8, m, k, n) bytes
  * with n the widest matrix it will be multiplied by (n = 0: what this call alone writes). k % 8 == 0. No counterpart in
  * the reference, whose thunks exchange f32 tensors; the graph level uses it when prefill matmuls of one step read a
  * FakeQuantize node. */

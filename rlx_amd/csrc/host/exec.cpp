@@ -528,7 +528,10 @@ static std::unique_ptr<rlx_exec> plan_graph(const rlx_graph_desc *g, const rlx_c
                 Node &o = e->nodes[j];
                 for (uint32_t t = 0; t < o.d.n_inputs; t++) {
                     if (o.d.inputs[t] != f) continue;
-                    const bool as_x = o.d.op_kind == RLX_OP_DEQUANT_MATMUL && t == 0 && o.m > 16 && o.k == fq.chan_dim;
+                    // Q4_0 / Q8_0 only: their prefill kernels round d * code to binary16 anyway, so scaled binary16 weights
+                    // lose nothing; the K-quants multiply exact integers and keep the f32 route
+                    const bool as_x = o.d.op_kind == RLX_OP_DEQUANT_MATMUL && t == 0 && o.m > 16 && o.k == fq.chan_dim &&
+                                      (o.d.scheme == SCHEME_Q4_0 || o.d.scheme == SCHEME_Q8_0);
                     if (!as_x) {
                         other_reader = true;
                     } else if (target >= 0 && step_idx[j] != target) {
@@ -630,7 +633,12 @@ static std::unique_ptr<rlx_exec> plan_graph(const rlx_graph_desc *g, const rlx_c
     }
     for (size_t si = 0; si < e->steps.size(); si++) {
         const std::vector<uint32_t> &step = e->steps[si];
-        size_t step_ws = 0;
+        size_t step_ws = 0, step_parts = 0;  // operands of the widest matmul; partial results of every matmul whose K is split
+        auto need = [&](const Node &mm, uint32_t dt) {
+            const size_t ops_only = rlx_mi355x_gguf_matmul_workspace((int)mm.d.scheme, (int)dt, mm.m, mm.k, 0);
+            step_ws = std::max(step_ws, ops_only);
+            return rlx_mi355x_gguf_matmul_workspace((int)mm.d.scheme, (int)dt, mm.m, mm.k, mm.n) - ops_only;
+        };
         for (uint32_t id : step) {
             Node &nd = e->nodes[id];
             if (!(nd.img_step >= 0 && !nd.keep_f32) && !placed_early[id])  // a FakeQuantize result that only travels as a prefill image has no slot
@@ -649,10 +657,13 @@ static std::unique_ptr<rlx_exec> plan_graph(const rlx_graph_desc *g, const rlx_c
                 if (need) nd.aux = take(need, (int)si, (int)si);
             }
             if (nd.d.op_kind == RLX_OP_DEQUANT_MATMUL && nd.m > 16)  // may run the prefill kernels (which one is decided by the input dtype at run time): sized for f32
-                step_ws = std::max(step_ws, rlx_mi355x_gguf_matmul_workspace((int)nd.d.scheme, RLX_F32, nd.m, nd.k, nd.n));
-            if (nd.x_image)  // the code image a FakeQuantize writes, and this matrix scaled by its column scales
-                step_ws = std::max(step_ws, rlx_mi355x_gguf_matmul_workspace((int)nd.d.scheme, RLX_I8, nd.m, nd.k, nd.n));
+                step_parts += std::max(need(nd, RLX_F32), need(nd, RLX_BF16));
+            if (nd.x_image) {  // the code image a FakeQuantize writes, and this matrix scaled by its column scales
+                const size_t with_w = rlx_mi355x_gguf_matmul_workspace((int)nd.d.scheme, RLX_I8, nd.m, nd.k, nd.n);
+                step_ws = std::max(step_ws, with_w);  // holds that matmul's own partial results too
+            }
         }
+        step_ws += step_parts;
         if (step_ws) {  // one workspace for the whole step; it is born earlier when a FakeQuantize writes the step's image into it
             int birth = (int)si;
             for (const Node &fq : e->nodes)

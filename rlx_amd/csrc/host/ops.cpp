@@ -95,7 +95,7 @@ struct GemmArgs {
     int nseg;
     const void *xh;
     const void *sxh;
-    int m_rows, m_out, k_pad, units, pair_rows, steps_per_split, use_atomics, sc_off;
+    int m_rows, m_out, k_pad, units, pair_rows, steps_per_split, split_out, sc_off;
     const float *rowfac;
     const int *tile_expert;
     const int *perm;
@@ -122,6 +122,7 @@ struct MoeSortArgs {  // mirrors kernels/moe.hip
 // Kinds of activation operand: 0 f32, 1 bf16, 2 f16 tensors; XK_CODES: the workspace image a FakeQuantize left
 // (rlx_mi355x_fake_quantize_image: integer codes as binary16 plus the column scales), named RLX_I8 at the boundary.
 constexpr int XK_CODES = 3;
+static bool code_image_scheme(int scheme) { return scheme == SCHEME_Q4_0 || scheme == SCHEME_Q8_0; }
 static int x_kind(int x_dtype) {
     switch (x_dtype) {
     case RLX_F32: return 0;
@@ -316,17 +317,40 @@ static int launch_gemv(const void *const *xs, int xk, const rlx_qweight *const *
     return launch(id, (unsigned)sh.wg, 1, (unsigned)sh.nwaves * 64, (unsigned)sh.lds, stream, params);
 }
 
-// Workspace of a prefill matmul: [per-row factors][column scales][image of x][block sums][image of the scaled weights].
-// The second and the last exist only for a FakeQuantize code image (XK_CODES), whose matmul runs on ready binary16
-// weights W * diag(s) (n is the widest matrix multiplied from the image, one at a time).
+// How K is cut across workgroups when the output tiles alone would leave most of the chip idle: `split` slices of
+// `units_per_split` K units (whole groups of four 64-column steps). Each slice writes its partial result and
+// rlx_splitk_reduce adds the slices in ascending K.
+struct GemmSplit {
+    int split, units_per_split;
+};
+static GemmSplit gemm_split(long long tiles_x, long long tiles_y, int64_t k_units, int steps_per_unit, bool skinny, int max_split = 1 << 30) {
+    // workgroup slots to fill: one per CU for the 256-row tile (144 KB of LDS), two for the 64-row tile; sized for the
+    // 256 CUs of the part when no device has been opened (planning a graph needs none)
+    const int cus = device_props().cu_count > 0 ? device_props().cu_count : 256;
+    const long long slots = (long long)cus * (skinny ? 2 : 1);
+    int split = 1;
+    if (tiles_x * tiles_y * 5 < slots * 4) split = (int)std::min<long long>(k_units, slots / (tiles_x * tiles_y));
+    split = std::max(1, std::min(split, max_split));
+    int units_per_split = (int)((k_units + split - 1) / split);
+    const int upq = std::max(1, 4 / steps_per_unit);  // units in four steps: every slice is a multiple of that
+    units_per_split = (units_per_split + upq - 1) / upq * upq;
+    split = (int)((k_units + units_per_split - 1) / units_per_split);
+    return GemmSplit{split, units_per_split};
+}
+
+// Workspace of a prefill matmul: [per-row factors][column scales][image of x][block sums][image of the scaled weights]
+// [partial results of a split K]. The second and the fifth exist only for a FakeQuantize code image (XK_CODES), whose
+// matmul runs on ready binary16 weights W * diag(s) (n is the widest matrix multiplied from the image, one at a time).
 struct GemmPlan {
     int64_t m_rows, k_pad;
     size_t xh_bytes, sxh_bytes, fac_bytes;  // the image, the block sums (Q4_K / Q5_K per 32 columns, Q2_K per 16), the per-row prescale factors
     size_t cs_bytes, wimg_bytes;
+    size_t part_bytes;                      // split K of one [m, n] matmul on its own: split x m x n floats (0: no split)
     int sums_kind;                          // act_sums_kind of the scheme the plan was made for
     size_t image_end() const { return fac_bytes + cs_bytes + xh_bytes + sxh_bytes; }
-    size_t total() const { return image_end() + wimg_bytes; }
+    size_t total() const { return image_end() + wimg_bytes + part_bytes; }
 };
+static bool gemm_skinny(int xk, int64_t m) { return (xk == 0 ? 2 * m : m) <= 128; }
 static GemmPlan gemm_plan(int scheme, int xk, int64_t m, int64_t k, int64_t n = 0) {
     GemmPlan p;
     const int64_t rv = xk == 0 ? 2 * m : m;
@@ -338,6 +362,15 @@ static GemmPlan gemm_plan(int scheme, int xk, int64_t m, int64_t k, int64_t n = 
     p.fac_bytes = ((size_t)m * 8 + 255) & ~(size_t)255;
     p.cs_bytes = xk == XK_CODES ? (size_t)p.k_pad * 4 : 0;
     p.wimg_bytes = xk == XK_CODES ? (size_t)((n + 127) / 128 * 128) * p.k_pad * 2 : 0;
+    p.part_bytes = 0;
+    if (n > 0) {
+        const Layout L = layout_of(scheme);
+        const bool skinny = gemm_skinny(xk, m);
+        const int spu = xk == XK_CODES ? 1 : L.unit_k / 64;
+        const int64_t k_units = xk == XK_CODES ? p.k_pad / 64 : (k + L.unit_k - 1) / L.unit_k;
+        const GemmSplit sp = gemm_split((n + 127) / 128, skinny ? (rv + 63) / 64 : p.m_rows / 256, k_units, spu, skinny);
+        if (sp.split > 1) p.part_bytes = (size_t)sp.split * (size_t)m * (size_t)n * 4;
+    }
     return p;
 }
 
@@ -371,23 +404,24 @@ static int launch_gemm(const void *x, int xk, const rlx_qweight *const *ws, floa
     const rlx_qweight *w = ws[0];
     const bool codes = xk == XK_CODES;  // the workspace holds a FakeQuantize code image; the weights are scaled into it first
     const Layout L = codes ? Layout{64, 0, 0, 0, 0} : w->layout;
-    const GemmPlan p = gemm_plan(w->scheme, xk, m, w->dims.k, w->dims.n);
+    const GemmPlan p = gemm_plan(w->scheme, xk, m, w->dims.k, codes ? w->dims.n : 0);  // the operands; partial results are fitted below
     for (int i = 1; i < count; i++)
         if (ws[i]->scheme != w->scheme || ws[i]->dims.k != w->dims.k || ws[i]->dims.units != w->dims.units ||
             ws[i]->layout.unit_bytes != L.unit_bytes || ws[i]->sc_off() != w->sc_off()) {
             set_error("gguf_matmul_bt: matrices of one prefill launch differ in scheme or K");
             return RLX_ERR_INVALID;
         }
-    if (!workspace || workspace_bytes < p.total()) {
-        set_error("gguf_matmul_bt: m=%lld needs a %zu-byte workspace, got %zu", (long long)m, p.total(), workspace_bytes);
+    const size_t ops_end = p.image_end() + p.wimg_bytes;  // the operands; partial results of a split K follow
+    if (!workspace || workspace_bytes < ops_end) {
+        set_error("gguf_matmul_bt: m=%lld needs a %zu-byte workspace, got %zu", (long long)m, ops_end, workspace_bytes);
         return RLX_ERR_INVALID;
     }
     if ((uintptr_t)workspace % 16 != 0 || (uintptr_t)x % 16 != 0) {
         set_error("gguf_matmul_bt: activations and workspace must be 16-byte aligned");
         return RLX_ERR_INVALID;
     }
-    // workspace: [per-row prescale factors][binary16 image of x][block sums], so that an image made for a scheme with
-    // block sums is found at the same place by a scheme without
+    // workspace: [per-row prescale factors][binary16 image of x][block sums] ..., so that an image made for a scheme
+    // with block sums is found at the same place by a scheme without
     float *fac = (float *)workspace;
     void *xh = (uint8_t *)workspace + p.fac_bytes + p.cs_bytes;
     void *sxh = p.sxh_bytes ? (uint8_t *)workspace + p.fac_bytes + p.cs_bytes + p.xh_bytes : nullptr;
@@ -395,13 +429,7 @@ static int launch_gemm(const void *x, int xk, const rlx_qweight *const *ws, floa
     if (codes) {  // B = fl16(W * diag(s) / S) as stage images; fac holds (1 / S, S) for every row
         WScaleArgs wa{w->dev, wimg, (const float *)((uint8_t *)workspace + p.fac_bytes), fac, w->dims.row_tiles, w->dims.units, (int)p.k_pad, w->sc_off()};
         void *wparams[] = {&wa};
-        const KernelId wid = w->scheme == SCHEME_Q4K    ? K_WSCALE_Q4_K
-                             : w->scheme == SCHEME_Q4_0 ? K_WSCALE_Q4_0
-                             : w->scheme == SCHEME_Q6K  ? K_WSCALE_Q6_K
-                             : w->scheme == SCHEME_Q5K  ? K_WSCALE_Q5_K
-                             : w->scheme == SCHEME_Q8K  ? K_WSCALE_Q8_K
-                             : w->scheme == SCHEME_Q2K  ? K_WSCALE_Q2_K
-                                                        : K_WSCALE_Q8_0;
+        const KernelId wid = w->scheme == SCHEME_Q4_0 ? K_WSCALE_Q4_0 : K_WSCALE_Q8_0;
         RLX_TRY(launch(wid, (unsigned)(p.k_pad / w->layout.unit_k), (unsigned)((w->dims.n + 127) / 128 * 8), 64, 0, stream, wparams));
     } else if (!prepared) {
         RLX_TRY(launch_xprep(x, xk, m, w->dims.k, p, workspace, stream));
@@ -412,7 +440,7 @@ static int launch_gemm(const void *x, int xk, const rlx_qweight *const *ws, floa
     // Up to 128 activation rows run the 64-row tile (the weights are decoded once per 64 rows, but nothing is spent on
     // padding rows); beyond that the 256-row tile.
     const int64_t rv = xk == 0 ? 2 * m : m;
-    const bool skinny = rv <= 128;
+    const bool skinny = gemm_skinny(xk, m);
     GemmArgs a{};
     long long gx = 0;
     for (int i = 0; i < count; i++) {
@@ -421,17 +449,24 @@ static int launch_gemm(const void *x, int xk, const rlx_qweight *const *ws, floa
     }
     a.nseg = count;
     const int gy = skinny ? (int)((rv + 63) / 64) : (int)(p.m_rows / 256);
-    // workgroup slots to fill: one per CU for the 256-row tile (144 KB of LDS), two for the 64-row tile
-    const long long slots = (long long)std::max(1, device_props().cu_count) * (skinny ? 2 : 1);
-    int split = 1;
-    if (gx * gy * 5 < slots * 4) split = (int)std::min<long long>(k_units, slots / (gx * gy));
-    split = std::max(1, split);
-    int units_per_split = (int)((k_units + split - 1) / split);
-    const int upq = 4 / steps_per_unit;  // units in four steps: every split is a multiple of that
-    if (upq > 1) units_per_split = (units_per_split + upq - 1) / upq * upq;
-    split = (int)((k_units + units_per_split - 1) / units_per_split);
-    if (split > 1)
-        for (int i = 0; i < count; i++) RLX_TRY(rlx_mi355x_memset_u32(outs[i], 0, (size_t)m * ws[i]->dims.n, stream));
+    // Split K: every slice writes its partial result behind the operands in the workspace, then one reduce launch per
+    // matrix adds the slices in ascending K into the output. A workspace sized for fewer slices gets fewer.
+    size_t n_sum = 0;
+    for (int i = 0; i < count; i++) n_sum += (size_t)ws[i]->dims.n;
+    GemmSplit sp = gemm_split(gx, gy, k_units, steps_per_unit, skinny);
+    const size_t part_room = workspace_bytes - ops_end;
+    uint8_t *part_base = (uint8_t *)workspace + ops_end;  // every part of the workspace is a multiple of 256 bytes
+    if (sp.split > 1 && (size_t)sp.split * (size_t)m * n_sum * 4 > part_room)
+        sp = gemm_split(gx, gy, k_units, steps_per_unit, skinny, (int)std::max<size_t>(1, part_room / ((size_t)m * n_sum * 4)));
+    if (sp.split > 1 && (size_t)sp.split * (size_t)m * n_sum * 4 > part_room) sp = gemm_split(gx, gy, k_units, steps_per_unit, skinny, 1);
+    const int split = sp.split, units_per_split = sp.units_per_split;
+    if (split > 1) {
+        size_t off = 0;
+        for (int i = 0; i < count; i++) {
+            a.seg[i].out = (float *)(part_base + off);
+            off += (size_t)split * (size_t)m * (size_t)ws[i]->dims.n * 4;
+        }
+    }
     a.xh = xh;
     a.sxh = sxh;
     a.m_rows = (int)p.m_rows;
@@ -440,7 +475,7 @@ static int launch_gemm(const void *x, int xk, const rlx_qweight *const *ws, floa
     a.units = (int)k_units;
     a.pair_rows = xk == 0 ? 1 : 0;
     a.steps_per_split = units_per_split * steps_per_unit;
-    a.use_atomics = split > 1 ? 1 : 0;
+    a.split_out = split > 1 ? 1 : 0;
     a.sc_off = w->sc_off();
     a.rowfac = fac;
     void *params[] = {&a};
@@ -454,6 +489,16 @@ static int launch_gemm(const void *x, int xk, const rlx_qweight *const *ws, floa
                                                 : (skinny ? K_GEMM64_Q8_0 : K_GEMM_Q8_0);
     RLX_TRY(runtime_init());
     RLX_TRY(launch3(id, (unsigned)gx, (unsigned)gy, (unsigned)split, 512, skinny ? 3 * 24 * 1024 : 3 * 48 * 1024, stream, params));
+    if (split > 1)
+        for (int i = 0; i < count; i++) {
+            const float *part = a.seg[i].out;
+            float *out = outs[i];
+            long long elems = (long long)m * ws[i]->dims.n;
+            int nsl = split;
+            void *rparams[] = {&part, &out, &elems, &nsl};
+            const long long work = (elems + 3) / 4;
+            RLX_TRY(launch(K_SPLITK_REDUCE, (unsigned)std::min<long long>((work + 255) / 256, 2048), 1, 256, 0, stream, rparams));
+        }
     return RLX_OK;
 }
 
@@ -578,10 +623,10 @@ int rlx_mi355x_dequant(const rlx_qweight *w, float *out_dev, void *stream) {
 size_t rlx_mi355x_gguf_matmul_workspace(int scheme, int x_dtype, int64_t m, int64_t k, int64_t n) {
     using namespace rlx;
     if (x_dtype == RLX_I8)  // a FakeQuantize code image and the scaled weights of the widest matrix it is multiplied by
-        return layout_of(scheme).unit_k == 0 || m <= 0 || k <= 0 || n <= 0 ? 0 : gemm_plan(scheme, XK_CODES, m, k, n).total();
+        return !code_image_scheme(scheme) || m <= 0 || k <= 0 || n < 0 ? 0 : gemm_plan(scheme, XK_CODES, m, k, n).total();
     int xk = x_kind(x_dtype);
     if (xk < 0 || layout_of(scheme).unit_k == 0 || m <= decode_rows(xk)) return 0;  // decode path: no workspace
-    return gemm_plan(scheme, xk, m, k).total();
+    return gemm_plan(scheme, xk, m, k, n < 0 ? 0 : n).total();  // n = 0: the operand image alone (what ..._prepare writes)
 }
 
 int rlx_mi355x_gguf_matmul_bt_batch(const void *const *xs_dev, int x_dtype, const rlx_qweight *const *ws,
@@ -685,6 +730,12 @@ int rlx_mi355x_gguf_matmul_bt_prepared(const void *workspace, size_t workspace_b
             return RLX_ERR_INVALID;
         }
     if (xk == XK_CODES) {  // one matrix at a time: each is scaled into the workspace's weight image first
+        for (int i = 0; i < count; i++)
+            if (!code_image_scheme(ws[i]->scheme)) {
+                // the other schemes' prefill operands are exact integers; a weight rounded to binary16 would cost them accuracy
+                set_error("gguf_matmul_bt_prepared: a FakeQuantize code image multiplies Q4_0 / Q8_0 weights only (weight %d is scheme %d)", i, ws[i]->scheme);
+                return RLX_ERR_UNSUPPORTED;
+            }
         for (int i = 0; i < count; i++)
             RLX_TRY(launch_gemm(workspace, xk, ws + i, outs_dev + i, 1, m, const_cast<void *>(workspace), workspace_bytes, (hipStream_t)stream, true));
         return RLX_OK;
@@ -1078,7 +1129,7 @@ int rlx_mi355x_gguf_grouped_matmul_bt_ws(const void *x_dev, int x_dtype, const r
     a.units = (int)w->dims.units;
     a.pair_rows = xk == 0 ? 1 : 0;
     a.steps_per_split = (int)w->dims.units * (L.unit_k / 64);
-    a.use_atomics = 0;
+    a.split_out = 0;
     a.sc_off = w->sc_off();
     a.rowfac = (const float *)gws;
     a.tile_expert = tile_expert;

@@ -167,6 +167,8 @@ __device__ __forceinline__ void dequant_tile(const DequantArgs &a) {
 // ---- weights times per-column scales, as binary16 operand images of the prefill kernel ---------------------------
 // A FakeQuantize result with column channels is q[i][c] * s[c] with small integer codes q, so its product with W^T is
 // sum_c q[i][c] * (s[c] * W[j][c]): the codes are exact in binary16 and the per-column scale belongs with the weights.
+// Built for Q4_0 and Q8_0, whose own prefill kernels round d * code to binary16 as well, so nothing is lost; the schemes
+// whose prefill operands are exact integers keep the f32 route.
 // This kernel writes B[j][c] = fl16(W[j][c] * (s[c] * inv)) (W decoded in f32 with the reference's operation order, one
 // rounding), `inv` the power of two in rowfac[0] that brings the largest s[c] to [1, 2), in the order of the prefill
 // kernel's LDS stage: one contiguous 16 KB block per (128-row tile of W, 64-column step), [k-slice][32-row sub-tile]
@@ -216,11 +218,6 @@ __device__ __forceinline__ void wscale_tile(const WScaleArgs &a) {
 
 extern "C" __global__ __launch_bounds__(64) void rlx_wscale_q4_0(rlx::WScaleArgs a) { rlx::wscale_tile<rlx::SCHEME_Q4_0>(a); }
 extern "C" __global__ __launch_bounds__(64) void rlx_wscale_q8_0(rlx::WScaleArgs a) { rlx::wscale_tile<rlx::SCHEME_Q8_0>(a); }
-extern "C" __global__ __launch_bounds__(64) void rlx_wscale_q4_k(rlx::WScaleArgs a) { rlx::wscale_tile<rlx::SCHEME_Q4K>(a); }
-extern "C" __global__ __launch_bounds__(64) void rlx_wscale_q5_k(rlx::WScaleArgs a) { rlx::wscale_tile<rlx::SCHEME_Q5K>(a); }
-extern "C" __global__ __launch_bounds__(64) void rlx_wscale_q6_k(rlx::WScaleArgs a) { rlx::wscale_tile<rlx::SCHEME_Q6K>(a); }
-extern "C" __global__ __launch_bounds__(64) void rlx_wscale_q8_k(rlx::WScaleArgs a) { rlx::wscale_tile<rlx::SCHEME_Q8K>(a); }
-extern "C" __global__ __launch_bounds__(64) void rlx_wscale_q2_k(rlx::WScaleArgs a) { rlx::wscale_tile<rlx::SCHEME_Q2K>(a); }
 extern "C" __global__ __launch_bounds__(64) void rlx_dequant_q4_0(rlx::DequantArgs a) { rlx::dequant_tile<rlx::SCHEME_Q4_0>(a); }
 extern "C" __global__ __launch_bounds__(64) void rlx_dequant_q8_0(rlx::DequantArgs a) { rlx::dequant_tile<rlx::SCHEME_Q8_0>(a); }
 extern "C" __global__ __launch_bounds__(64) void rlx_dequant_q4_k(rlx::DequantArgs a) { rlx::dequant_tile<rlx::SCHEME_Q4K>(a); }

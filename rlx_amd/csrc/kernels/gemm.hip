@@ -40,7 +40,7 @@ struct GemmArgs {
     int units;          // K units of the device layout
     int pair_rows;      // 1: rows 2i, 2i+1 of xh are hi / lo*2048 of logical row i (f32 activations)
     int steps_per_split;  // 64-column steps per grid.z slice (a multiple of 4)
-    int use_atomics;      // split K: accumulate into a zeroed `out` with atomic adds
+    int split_out;        // split K: seg.out is [grid.z][m_out][n], slice z written by the workgroups of blockIdx.z (rlx_splitk_reduce folds them)
     int sc_off;           // Q6_K: a stored scale byte stands for byte - sc_off (0 unsigned reading, 128 signed)
     const float *rowfac;  // [m_out][2]: the power of two row i of x was multiplied by when it was converted, and its inverse
     // Expert-sorted launch (rlx_gemm64g_*): the image rows are tokens sorted by expert, every 64-row tile inside one
@@ -110,7 +110,8 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
 #pragma unroll
     for (int i = 1; i < GEMM_MAX_SEG; i++)
         if (i < a.nseg && (int)blockIdx.x >= a.seg[i].tile_begin) si = i;
-    const GemmSeg sg = a.seg[si];
+    GemmSeg sg = a.seg[si];
+    if (a.split_out) sg.out += (long long)blockIdx.z * a.m_out * sg.n;  // this K slice's partial result
     const uint8_t *w_base = sg.w + (GROUPED ? (long long)expert * a.slab_bytes : 0LL);  // this launch's matrix, or the tile's expert slab
     const int bx = (int)blockIdx.x - sg.tile_begin;
     const int n_tile0 = bx * GEMM_NT, m_tile0 = blockIdx.y * MT;
@@ -568,7 +569,7 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
     // rows can take 16-byte stores the wave turns its tile around through LDS instead (the stages are free by now):
     // 32 image rows at a time, every lane then owns four consecutive columns of a row and a store instruction covers four
     // whole rows of the wave tile.
-    if (!a.use_atomics && (sg.n & 3) == 0 && ((uintptr_t)sg.out & 15) == 0) {
+    if ((sg.n & 3) == 0 && ((uintptr_t)sg.out & 15) == 0) {
         constexpr int STRIDE = TJ * 32 + 8;  // floats per row: lanes 32-63 (four rows further) land 32 banks away
         __syncthreads();                     // the last stage has been read by every wave
         float *tile = (float *)smem + wave * (32 * STRIDE);
@@ -608,7 +609,7 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
         }
         return;
     }
-    // Otherwise (K split across workgroups, or a row length that is no multiple of four):
+    // Otherwise (a row length that is no multiple of four):
     // The four rows of a register quad are neighbours, so their output rows and factors come as one 16-byte LDS read
     // each (8 bytes with f32 activations, where two image rows make one output row), shared by the tiles j.
 #pragma unroll
@@ -648,11 +649,29 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
                 }
                 if (orow[e] >= 0) {
                     v *= ofac[e];  // undo the row's prescale (1 for a row binary16 carries as it is)
-                    float *p = sg.out + (long long)orow[e] * sg.n + col;
-                    if (a.use_atomics) atomicAdd(p, v);
-                    else __builtin_nontemporal_store(v, p);  // written once, read by another kernel: keep it out of the way of the operands
+                    __builtin_nontemporal_store(v, sg.out + (long long)orow[e] * sg.n + col);  // written once, read by another kernel: keep it out of the way of the operands
                 }
             }
+        }
+    }
+}
+
+// Split K: out[i] = part[0][i] + part[1][i] + ... in ascending K, the order the reference walks a row in
+// (rlx-cpu/src/gguf_matmul.rs:81-94), so a result does not depend on which workgroup finished first.
+__device__ __forceinline__ void splitk_reduce_body(const float *part, float *out, long long elems, int split) {
+    const long long stride = (long long)gridDim.x * blockDim.x;
+    long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if ((elems & 3) == 0 && (((uintptr_t)part | (uintptr_t)out) & 15) == 0) {
+        for (; i < (elems >> 2); i += stride) {
+            float4_t acc = __builtin_nontemporal_load((const float4_t *)part + i);
+            for (int z = 1; z < split; z++) acc += __builtin_nontemporal_load((const float4_t *)(part + z * elems) + i);
+            __builtin_nontemporal_store(acc, (float4_t *)out + i);
+        }
+    } else {
+        for (; i < elems; i += stride) {
+            float acc = part[i];
+            for (int z = 1; z < split; z++) acc += part[z * elems + i];
+            out[i] = acc;
         }
     }
 }
@@ -835,5 +854,8 @@ extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64g_q5_k(rlx::GemmA
 extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64g_q6_k(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q6K, 1, 1, true>(a); }
 extern "C" __global__ __launch_bounds__(512) void rlx_gemm_f16w(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_F16W, 2, 2>(a); }
 extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64_f16w(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_F16W, 1, 1>(a); }
+extern "C" __global__ __launch_bounds__(256) void rlx_splitk_reduce(const float *part, float *out, long long elems, int split) {
+    rlx::splitk_reduce_body(part, out, elems, split);
+}
 extern "C" __global__ __launch_bounds__(256) void rlx_xprep(rlx::XPrepArgs a) { rlx::xprep_body(a); }
 extern "C" __global__ __launch_bounds__(256) void rlx_xrowscale(rlx::XPrepArgs a) { rlx::xrowscale_body(a); }

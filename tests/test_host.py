@@ -179,7 +179,7 @@ def test_plan_reuses_dead_slots():
     assert slots[fq][1] == 0 and "f32 tensor not written" in text.splitlines()[1 + fq]
     assert slots[z2][0] == slots[y][0]                     # z2 reuses y's slot
     bump = sum((sz + 255) // 256 * 256 for _, sz in slots.values())
-    assert total < bump + 5 * 1024 * 1024                  # less than one private slot per buffer plus the workspaces (code image 2 MiB + scaled weights 2 MiB)
+    assert total < bump + 7 * 1024 * 1024                  # less than one private slot per buffer plus the workspaces (code image 2 MiB, scaled weights 2 MiB, K-slice partial results)
     for a in (x, w, w2, w3, w4, z3):                       # sources and outputs never share bytes with anything
         for b in slots:
             assert a == b or disjoint(slots, a, b), (a, b)
