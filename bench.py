@@ -82,10 +82,12 @@ def build_layer_graph(li, wiring):
 SETTLE_LAUNCHES = 400   # untimed layer passes in front of every timed GEMV region, whatever --warmup says: the
                         # clocks of a fresh box need a few milliseconds of load before they stop moving
 GEMM_SETTLE_CALLS = 100  # the same for the prefill GEMM leg (each call is ~80 us)
+TIMED_BLOCKS = 10        # the headline is timed as this many blocks of --steps launches; median, min and max are reported
 
 
-def time_layers(rlx_amd, ops, stream, base, wiring, n_layers, steps, warmup, use_graph, settle=SETTLE_LAUNCHES):
-    """Build n_layers executables (distinct weight bytes), replay them round-robin, return (ms_per_step, layers, xs)."""
+def time_layers(rlx_amd, ops, stream, base, wiring, n_layers, steps, warmup, use_graph, settle=SETTLE_LAUNCHES, blocks=TIMED_BLOCKS):
+    """Build n_layers executables (distinct weight bytes), replay them round-robin, return (median ms_per_step, layers,
+    xs, spread over the timed blocks)."""
     from rlx_amd import DType, Session
 
     x_of = WIRING[wiring]
@@ -114,13 +116,18 @@ def time_layers(rlx_amd, ops, stream, base, wiring, n_layers, steps, warmup, use
     run_steps(settle)
     run_steps(warmup, settle)
     ops.sync(stream)
-    ev0, ev1 = ops.Event(), ops.Event()
-    ev0.record(stream)
-    run_steps(steps, settle + warmup)
-    ev1.record(stream)
-    ms = ev0.elapsed_ms(ev1)
+    # `blocks` timed regions of `steps` launches each, one after another on the stream, an event at every boundary: the
+    # figure is the median block, with the fastest and the slowest beside it
+    evs = [ops.Event() for _ in range(blocks + 1)]
+    evs[0].record(stream)
+    for b in range(blocks):
+        run_steps(steps, settle + warmup + b * steps)
+        evs[b + 1].record(stream)
     ops.sync(stream)
-    return ms / steps, layers, xs
+    per_step = sorted(evs[b].elapsed_ms(evs[b + 1]) / steps for b in range(blocks))
+    spread = {"blocks": blocks, "steps_per_block": steps, "median_ms": round(per_step[len(per_step) // 2], 6),
+              "min_ms": round(per_step[0], 6), "max_ms": round(per_step[-1], 6)}
+    return per_step[len(per_step) // 2], layers, xs, spread
 
 
 def main():
@@ -170,8 +177,8 @@ def main():
         ops.sync(stream)
         src.free()
         dst.free()
-    ms_per_step, layers, xs = time_layers(rlx_amd, ops, stream, base, args.wiring, args.layers, args.steps, args.warmup,
-                                          args.graph)
+    ms_per_step, layers, xs, spread = time_layers(rlx_amd, ops, stream, base, args.wiring, args.layers, args.steps, args.warmup,
+                                                  args.graph)
     setup_s = time.time() - t0
     launches_per_step = 1 if args.wiring == "independent" else 4
     gbs = layer_bytes / (ms_per_step * 1e-3) / 1e9
@@ -206,7 +213,11 @@ def main():
                      "frac": round(gbs / HBM_PEAK_GBS, 4),
                      "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH if args.wiring == "independent" else None,
                      "kernel": "rlx_gemv_q4_0_u2_r2", "avg_launch_us": round(us_per_launch, 3),
-                     "algorithmic_bytes_per_launch": layer_bytes // launches_per_step},
+                     "algorithmic_bytes_per_launch": layer_bytes // launches_per_step,
+                     "timed": f"{TIMED_BLOCKS} blocks of {args.steps} launches, HIP events at the block boundaries; value, ms_per_step "
+                              "and avg_launch_us are the median block",
+                     "blocks": spread,
+                     "GB/s_min_max": [round(layer_bytes / spread["max_ms"] / 1e6, 1), round(layer_bytes / spread["min_ms"] / 1e6, 1)]},
         "parity_max_rel_err": parity,
         "device": info,
         "setup_s": round(setup_s, 1),
@@ -227,11 +238,12 @@ def main():
     del layers
     # the other wiring of the same layer, beside the headline: "layer" is what a decode loop gets (four launches, each
     # waiting for the one before)
-    ms_o, lay_o, _ = time_layers(rlx_amd, ops, stream, base, other, args.layers, max(args.steps, 200), args.warmup, args.graph)
+    ms_o, lay_o, _, spread_o = time_layers(rlx_amd, ops, stream, base, other, args.layers, max(args.steps, 100), args.warmup, args.graph)
     del lay_o
     result["config"][f"wiring_{other}_ms"] = round(ms_o, 6)
     result["config"][f"wiring_{other}_GB/s"] = round(layer_bytes / ms_o / 1e6, 1)
     result["config"][f"wiring_{other}_launches_per_step"] = 1 if other == "independent" else 4
+    result["config"][f"wiring_{other}_blocks"] = spread_o
     result["config"]["settle_launches"] = SETTLE_LAUNCHES
 
     # ---- second half of the metric: Q4_K prefill GEMM, M = 512, on the Llama-3-8B MLP shapes (bf16 activations)
@@ -240,14 +252,19 @@ def main():
     result["roofline"]["secondary"] = {
         "bound": "mfma", "kernel": "rlx_gemm_q4_k", "achieved": g0["TFLOP/s"], "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
         "frac": round(g0["TFLOP/s"] / MFMA_F16_PEAK_TFLOPS, 4), "flop_per_launch": g0["flop"], "avg_launch_us": g0["us"],
-        "timed": "rlx_gemm_q4_k launches only, back to back between two HIP events (activations converted beforehand by "
-                 "rlx_mi355x_gguf_matmul_prepare); the whole rlx_mi355x_gguf_matmul_bt call, rlx_xprep launch included: "
-                 f"{g0['us_call_with_xprep']} us = {g0['TFLOP/s_call_with_xprep']} TFLOP/s",
+        "whole_call": {"us": g0["us_call_with_xprep"], "TFLOP/s": g0["TFLOP/s_call_with_xprep"],
+                       "frac": round(g0["TFLOP/s_call_with_xprep"] / MFMA_F16_PEAK_TFLOPS, 4),
+                       "what": "one rlx_mi355x_gguf_matmul_bt call as the reference defines the op: rlx_xrowscale + rlx_xprep + rlx_gemm_q4_k"},
+        "timed": "frac / achieved / avg_launch_us: rlx_gemm_q4_k launches only, back to back between two HIP events (activations "
+                 "converted beforehand by rlx_mi355x_gguf_matmul_prepare); whole_call: the complete call, conversion launches included",
         "workload": "Q4_K GEMM M=512, 4096 -> 14336 (gate / up), bf16 activations ~N(0,1), weights ~N(0,0.02), f32 out; "
                     f"{GEMM_SETTLE_CALLS} untimed calls, then {g0['reps']} timed, two weight copies in rotation",
         "down_14336x4096": {k: gemm["down_14336x4096"][k] for k in ("us", "TFLOP/s", "frac_mfma_f16", "us_call_with_xprep")},
         "gate+up_pair_one_call": {k: gemm["gate+up_pair"][k] for k in ("us", "TFLOP/s", "frac_mfma_f16")},
     }
+
+    # ---- the other benchmark configurations (1, 4, 5), each with its roofline fraction
+    result["config"]["other_configs"] = other_configs(rlx_amd, stream, not args.no_cpu)
 
     if args.extra:
         result["extra"] = extra_configs(rlx_amd, stream)
@@ -258,8 +275,6 @@ def main():
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(base, xs)
         result["cpu_baseline"]["secondary"] = cpu_baseline_q4k_gemm()
-        if args.extra:
-            result["extra"]["cpu_baselines"] = cpu_baselines_extra()
     print(json.dumps(result), flush=True)
 
 
@@ -354,27 +369,6 @@ def extra_configs(rlx_amd, stream):
     for ws in sets:
         for q in ws.values():
             q.free()
-    # config 1: Q8_0 GEMV 4096x4096
-    n = k = 4096
-    w = (ops.philox_normal(7, n * k) * np.float32(0.02)).astype(np.float32)
-    packed = ops.quantize(QuantScheme.GgufQ8_0, w).reshape(n, -1)
-    copies = 34
-    qws = [ops.QWeight(QuantScheme.GgufQ8_0, np.roll(packed, i, axis=0).reshape(-1), n, k) for i in range(copies)]
-    x = ops.DeviceBuffer.from_numpy(ops.philox_normal(8, k))
-    y = ops.DeviceBuffer(n * 4)
-    state = {"i": 0}
-
-    def fn8():
-        q = qws[state["i"] % copies]
-        state["i"] += 1
-        rlx_amd._lib.check(L.rlx_mi355x_gguf_matmul_bt(x.ptr, int(DType.F32), q.ptr, y.ptr, 1, None, 0, stream))
-
-    ms = time_launches(ops, stream, fn8, 400, 50)
-    b = gemv_bytes(n, k, 34)
-    out["q8_0_gemv_4096x4096"] = {"us": round(ms * 1e3, 3), "GB/s": round(b / ms / 1e6, 1),
-                                  "frac_hbm": round(b / ms / 1e6 / HBM_PEAK_GBS, 4)}
-    for q in qws:
-        q.free()
     # the other K-quants on a gate/up projection [14336, 4096], all packed: Q6_K, Q5_K, Q8_K and Q2_K in kernels of their own
     # (48 / 40 / 61 / 20 MB per copy), Q3_K as Q6_K super-blocks (48 MB). Copies rotated: nothing cache-resident.
     n, k = 14336, 4096
@@ -464,33 +458,6 @@ def extra_configs(rlx_amd, stream):
                                                     "launches": "gemv (logits into scratch) + two (cap 8) or three (cap 40) selection passes, one wave per 1024 candidates"}
     for q in qws:
         q.free()
-    # config 4: FakeQuantize [8192, 4096], int8 per column, heavy-tailed input; three input / output sets in rotation
-    # (3 x 268 MB) so that no launch finds its input in the 256 MB last-level cache
-    rows, cols = 8192, 4096
-    sets = []
-    for i in range(3):
-        xq = ops.philox_normal(9 + i, rows * cols)
-        xq[ops.philox_uniform(19 + i, rows * cols) < np.float32(0.001)] *= np.float32(20.0)
-        sets.append((ops.DeviceBuffer.from_numpy(xq), ops.DeviceBuffer(rows * cols * 4)))
-    del xq
-    scratch = ops.DeviceBuffer(L.rlx_mi355x_fake_quantize_scratch_bytes(rows * cols, cols, 1))
-    state = {"i": 0}
-
-    def fq():
-        xd, od = sets[state["i"] % 3]
-        state["i"] += 1
-        rlx_amd._lib.check(L.rlx_mi355x_fake_quantize(xd.ptr, od.ptr, None, rows * cols, cols, 1, 8, 0, 0.0, None, 0,
-                                                      scratch.ptr, stream))
-
-    ms = time_launches(ops, stream, fq, 60, 6)
-    b = 2 * rows * cols * 4
-    out["fake_quantize_8192x4096_cols"] = {"us": round(ms * 1e3, 2), "GB/s_1R1W": round(b / ms / 1e6, 1),
-                                           "frac_hbm_1R1W": round(b / ms / 1e6 / HBM_PEAK_GBS, 4),
-                                           "GB/s_2R1W": round(1.5 * b / ms / 1e6, 1),
-                                           "launches": "col_absmax + scale_parts + col_apply"}
-    for xd, od in sets:
-        xd.free()
-        od.free()
     out.update(moe_config(rlx_amd, stream))
     out.update(gemm_configs(rlx_amd, stream))
     return out
@@ -668,83 +635,170 @@ def gemm_configs(rlx_amd, stream):
     for q in qw:
         q.free()
 
-    # config 4 (second half): the fake-quantized [8192, 4096] f32 tensor against a Q8_0 4096x4096 weight
-    qw = [tiled_weight(ops, QuantScheme.GgufQ8_0, 4096, 4096, 45, 0.02)]
-    ms = run_matmul(qw, 8192, 4096, DType.F32, 30, 5)
-    tf = 2.0 * 8192 * 4096 * 4096 / ms / 1e9
-    out["q8_0_gemm_m8192_4096x4096_f32"] = {"us": round(ms * 1e3, 2), "TFLOP/s": round(tf, 1),
-                                          "frac_mfma_f16": round(tf / MFMA_F16_PEAK_TFLOPS, 4),
-                                          "note": "f32 activations run as hi + lo f16 rows: two MFMA rows per token"}
-    # the whole chain both ways: FakeQuantize writing f32 and the matmul converting it again, against FakeQuantize
-    # writing the matmul's operand image directly (no f32 tensor, no conversion pass)
-    rows, cols = 8192, 4096
-    xq = ops.philox_normal(9, rows * cols)
-    xq[ops.philox_uniform(19, rows * cols) < np.float32(0.001)] *= np.float32(20.0)
-    xd, fd, yd = ops.DeviceBuffer.from_numpy(xq), ops.DeviceBuffer(rows * cols * 4), ops.DeviceBuffer(rows * 4096 * 4)
+    return out
+
+
+def other_configs(rlx_amd, stream, with_cpu):
+    """Benchmark configurations 1, 4 and 5 beside the headline (2) and the prefill GEMM (3): each with its roofline fraction
+    and, with `with_cpu`, a bounded sample of the reference's scalar CPU path (the oracle's C restatement, one thread)."""
+    import oracle
+    from rlx_amd import DType, QuantScheme, ops
+    L = rlx_amd._lib.lib()
+    chk = rlx_amd._lib.check
+    out = {}
+
+    def cpu(fn, unit_per_call, unit):
+        if not with_cpu:
+            return None
+        t0 = time.time()
+        fn()
+        dt = time.time() - t0
+        return {"value": round(unit_per_call / dt, 4), "unit": unit, "s": round(dt, 3), "cores": 1, "kind": "port"}
+
+    # ---- config 1: Q8_0 GEMV 4096 x 4096, f32 activations, 34 weight copies in rotation (606 MB: nothing cache-resident)
+    n = k = 4096
+    w = (ops.philox_normal(7, n * k) * np.float32(0.02)).astype(np.float32)
+    packed = ops.quantize(QuantScheme.GgufQ8_0, w).reshape(n, -1)
+    copies = 34
+    qws = [ops.QWeight(QuantScheme.GgufQ8_0, np.roll(packed, i, axis=0).reshape(-1), n, k) for i in range(copies)]
+    xv = ops.philox_normal(8, k)
+    x = ops.DeviceBuffer.from_numpy(xv)
+    y = ops.DeviceBuffer(n * 4)
+    state = {"i": 0}
+
+    def fn8():
+        q = qws[state["i"] % copies]
+        state["i"] += 1
+        chk(L.rlx_mi355x_gguf_matmul_bt(x.ptr, int(DType.F32), q.ptr, y.ptr, 1, None, 0, stream))
+
+    ms = time_launches(ops, stream, fn8, 400, 100)
+    b = gemv_bytes(n, k, 34)
+    out["config1_q8_0_gemv_4096x4096"] = {
+        "us": round(ms * 1e3, 3), "GB/s": round(b / ms / 1e6, 1), "roofline": {"bound": "hbm", "frac": round(b / ms / 1e6 / HBM_PEAK_GBS, 4)},
+        "algorithmic_bytes": b, "kernel": "rlx_gemv_q8_0_r2", "note": "one 17.8 MB matrix per launch, cold; a launch of nothing takes ~3 us",
+        "cpu_baseline": cpu(lambda: oracle.gguf_matmul_bt(xv, packed.reshape(-1), 1, k, n, oracle.Q8_0), b / 1e9, "GB/s")}
+    for q in qws:
+        q.free()
+    del qws, packed, w
+
+    # ---- config 4: FakeQuantize [8192, 4096] int8 per column (heavy-tailed input), alone and feeding a Q8_0 4096 x 4096 matmul
+    rows, cols, n = 8192, 4096, 4096
+    sets, xq0 = [], None
+    for i in range(3):  # three input / output sets in rotation (3 x 268 MB): no launch finds its input in the last-level cache
+        xq = ops.philox_normal(9 + i, rows * cols)
+        xq[ops.philox_uniform(19 + i, rows * cols) < np.float32(0.001)] *= np.float32(20.0)
+        xq0 = xq if xq0 is None else xq0
+        sets.append((ops.DeviceBuffer.from_numpy(xq), ops.DeviceBuffer(rows * cols * 4)))
+    del xq
     scratch = ops.DeviceBuffer(L.rlx_mi355x_fake_quantize_scratch_bytes(rows * cols, cols, 1))
-    need = max(ops.matmul_workspace_bytes(qw[0], DType.F32, rows),
-               L.rlx_mi355x_gguf_matmul_workspace(int(QuantScheme.GgufQ8_0), int(DType.I8), rows, cols, 4096))
+    state = {"i": 0}
+
+    def fq():
+        xd, od = sets[state["i"] % 3]
+        state["i"] += 1
+        chk(L.rlx_mi355x_fake_quantize(xd.ptr, od.ptr, None, rows * cols, cols, 1, 8, 0, 0.0, None, 0, scratch.ptr, stream))
+
+    ms = time_launches(ops, stream, fq, 60, 10)
+    b = 2 * rows * cols * 4
+    out["config4_fake_quantize_8192x4096_cols"] = {
+        "us": round(ms * 1e3, 2), "GB/s_1R1W": round(b / ms / 1e6, 1), "GB/s_2R1W": round(1.5 * b / ms / 1e6, 1),
+        "roofline": {"bound": "hbm", "frac": round(b / ms / 1e6 / HBM_PEAK_GBS, 4), "frac_2R1W": round(1.5 * b / ms / 1e6 / HBM_PEAK_GBS, 4)},
+        "algorithmic_bytes": b, "launches": "rlx_fq_col_absmax + rlx_fq_scale_parts + rlx_fq_col_apply",
+        "cpu_baseline": cpu(lambda: oracle.fake_quantize(xq0, (rows, cols), 1, 8), b / 1e9, "GB/s_1R1W")}
+    qw = tiled_weight(ops, QuantScheme.GgufQ8_0, n, cols, 45, 0.02)
+    yd = ops.DeviceBuffer(rows * n * 4)
+    need = L.rlx_mi355x_gguf_matmul_workspace(int(QuantScheme.GgufQ8_0), int(DType.I8), rows, cols, n)
     ws = ops.DeviceBuffer(need)
-    w_arr = (rlx_amd._lib.C.c_void_p * 1)(qw[0].ptr)
-    y_arr = (rlx_amd._lib.C.c_void_p * 1)(yd.ptr)
+    w_arr, y_arr = (C.c_void_p * 1)(qw.ptr), (C.c_void_p * 1)(yd.ptr)
 
-    def chain_f32():
-        rlx_amd._lib.check(L.rlx_mi355x_fake_quantize(xd.ptr, fd.ptr, None, rows * cols, cols, 1, 8, 0, 0.0, None, 0, scratch.ptr, stream))
-        rlx_amd._lib.check(L.rlx_mi355x_gguf_matmul_bt(fd.ptr, int(DType.F32), qw[0].ptr, yd.ptr, rows, ws.ptr, need, stream))
+    def fq_image():
+        xd, _ = sets[state["i"] % 3]
+        state["i"] += 1
+        chk(L.rlx_mi355x_fake_quantize_image(xd.ptr, None, None, rows, cols, 8, 0, 0.0, None, 0, scratch.ptr, ws.ptr, need, stream))
 
-    def chain_image():
-        rlx_amd._lib.check(L.rlx_mi355x_fake_quantize_image(xd.ptr, None, None, rows, cols, 8, 0, 0.0, None, 0, scratch.ptr, ws.ptr, need, stream))
-        rlx_amd._lib.check(L.rlx_mi355x_gguf_matmul_bt_prepared(ws.ptr, need, int(DType.I8), w_arr, y_arr, 1, rows, stream))
+    def mm_image():
+        chk(L.rlx_mi355x_gguf_matmul_bt_prepared(ws.ptr, need, int(DType.I8), w_arr, y_arr, 1, rows, stream))
 
-    def fq_image_only():
-        rlx_amd._lib.check(L.rlx_mi355x_fake_quantize_image(xd.ptr, None, None, rows, cols, 8, 0, 0.0, None, 0, scratch.ptr, ws.ptr, need, stream))
+    def chain():
+        fq_image()
+        mm_image()
 
-    ms_a = time_launches(ops, stream, chain_f32, 30, 5)
-    ms_b = time_launches(ops, stream, chain_image, 30, 5)
-    ms_c = time_launches(ops, stream, fq_image_only, 60, 10)
-    out["fq_then_q8_0_gemm_8192x4096x4096"] = {
-        "us_fq_f32_then_matmul": round(ms_a * 1e3, 2), "us_fq_image_then_prepared_matmul": round(ms_b * 1e3, 2),
-        "us_fq_image_alone": round(ms_c * 1e3, 2),
-        "note": "the image holds the integer codes (exact in binary16, one row per token); the column scales are multiplied into the weights"}
-    qw[0].free()
+    ms_chain = time_launches(ops, stream, chain, 30, 8)
+    ms_mm = time_launches(ops, stream, mm_image, 30, 5)
+    ms_fqi = time_launches(ops, stream, fq_image, 60, 5)
+    flop = 2.0 * rows * cols * n
+    cpu_rows = 8  # the scalar loop is linear in the rows of x
+    out["config4_fake_quantize_then_q8_0_gemm_8192x4096x4096"] = {
+        "us_chain": round(ms_chain * 1e3, 1), "us_fake_quantize_writing_the_code_image": round(ms_fqi * 1e3, 1),
+        "us_matmul_from_the_image": round(ms_mm * 1e3, 1), "TFLOP/s_matmul": round(flop / ms_mm / 1e9, 1),
+        "roofline": {"bound": "mfma", "frac": round(flop / ms_mm / 1e9 / MFMA_F16_PEAK_TFLOPS, 4),
+                     "frac_chain": round(flop / ms_chain / 1e9 / MFMA_F16_PEAK_TFLOPS, 4)},
+        "flop": flop, "launches": "rlx_fq_col_absmax + rlx_fq_scale_parts + rlx_fq_col_apply_img | rlx_wscale_q8_0 + rlx_gemm_f16w",
+        "note": "the matmul runs on the integer codes (exact in binary16, one MFMA row per token) against W * diag(s) rounded once to binary16",
+        "cpu_baseline": cpu(lambda: oracle.gguf_matmul_bt(xq0[:cpu_rows * cols], _packed_of(ops, QuantScheme.GgufQ8_0, n, cols, 45, 0.02), cpu_rows, cols, n,
+                                                          oracle.Q8_0), 2.0 * cpu_rows * cols * n / 1e12, "TFLOP/s")}
+    if out["config4_fake_quantize_then_q8_0_gemm_8192x4096x4096"]["cpu_baseline"]:
+        out["config4_fake_quantize_then_q8_0_gemm_8192x4096x4096"]["cpu_baseline"]["sample"] = f"{cpu_rows} of {rows} rows of the matmul (linear in rows)"
+    for xd, od in sets:
+        xd.free()
+        od.free()
+    for bfr in (scratch, ws, yd):
+        bfr.free()
+    qw.free()
 
-    # config 5: Q4_0 batch sweep over the seven projections of one Llama-3-70B layer, bf16 activations
+    # ---- config 5: Q4_0 batch sweep over the seven projections of one Llama-3-70B layer, bf16 activations
     shapes70 = [("q", 8192, 8192), ("k", 1024, 8192), ("v", 1024, 8192), ("o", 8192, 8192),
                 ("gate", 28672, 8192), ("up", 28672, 8192), ("down", 8192, 28672)]
-    weights = {name: tiled_weight(ops, QuantScheme.GgufQ4_0, n, k, 50 + i, 0.015) for i, (name, n, k) in enumerate(shapes70)}
-    wbytes = sum(n * k // 32 * 18 for _, n, k in shapes70)
+    weights = {name: tiled_weight(ops, QuantScheme.GgufQ4_0, nn, kk, 50 + i, 0.015) for i, (name, nn, kk) in enumerate(shapes70)}
+    wbytes = sum(nn * kk // 32 * 18 for _, nn, kk in shapes70)
     sweep = {}
-    for m in (1, 4, 16, 32, 64, 256):  # 32: the largest batch the decode kernels take
-        # one timed repetition = the seven projections in turn, so the 481 MB of weights go round the 256 MB last-level
-        # cache and every launch reads its matrix from HBM
+    for m in (1, 4, 16, 64, 256):
+        # one timed repetition = the seven projections in one batched call, so the 481 MB of weights go round the 256 MB
+        # last-level cache and every launch reads its matrix from HBM
         bufs = {}
-        for name, n, k in shapes70:
-            if k not in bufs:
-                bufs[k] = ops.DeviceBuffer.from_numpy(f32_to_bf16_bits(ops.philox_normal(31, m * k)))
-        outs = {name: ops.DeviceBuffer(m * n * 4) for name, n, k in shapes70}
-        need = max(ops.matmul_workspace_bytes(weights[name], DType.BF16, m) for name, _, _ in shapes70)
+        for name, nn, kk in shapes70:
+            if kk not in bufs:
+                bufs[kk] = ops.DeviceBuffer.from_numpy(f32_to_bf16_bits(ops.philox_normal(31, m * kk)))
+        outs = {name: ops.DeviceBuffer(m * nn * 4) for name, nn, kk in shapes70}
+        need = sum(ops.matmul_workspace_bytes(weights[name], DType.BF16, m) for name, _, _ in shapes70)
         ws = ops.DeviceBuffer(need) if need else None
-
-        C = rlx_amd._lib.C
-        xs_arr = (C.c_void_p * 7)(*[bufs[k].ptr for _, _, k in shapes70])
+        xs_arr = (C.c_void_p * 7)(*[bufs[kk].ptr for _, _, kk in shapes70])
         ws_arr = (C.c_void_p * 7)(*[weights[name].ptr for name, _, _ in shapes70])
         out_arr = (C.c_void_p * 7)(*[outs[name].ptr for name, _, _ in shapes70])
 
-        def layer():  # one call: the decode path issues the seven as one launch, the prefill path as seven GEMMs
-            rlx_amd._lib.check(L.rlx_mi355x_gguf_matmul_bt_batch(xs_arr, int(DType.BF16), ws_arr, out_arr, 7, m,
-                                                                 ws.ptr if ws else None, need, stream))
+        def layer():  # one call: the decode path issues the seven as one launch, the prefill path as GEMM launches of up to four matrices
+            chk(L.rlx_mi355x_gguf_matmul_bt_batch(xs_arr, int(DType.BF16), ws_arr, out_arr, 7, m, ws.ptr if ws else None, need, stream))
 
-        total_ms = time_launches(ops, stream, layer, 20 if m > 16 else 50, 3)
+        total_ms = time_launches(ops, stream, layer, 30 if m > 16 else 100, 10)
         ops.sync(stream)
-        flops = sum(2.0 * m * n * k for _, n, k in shapes70)
-        algo = wbytes + sum(2 * m * k + 4 * m * n for _, n, k in shapes70)
+        flops = sum(2.0 * m * nn * kk for _, nn, kk in shapes70)
+        algo = wbytes + sum(2 * m * kk + 4 * m * nn for _, nn, kk in shapes70)
+        t_hbm, t_mfma = algo / (HBM_PEAK_GBS * 1e9), flops / (MFMA_F16_PEAK_TFLOPS * 1e12)
         sweep[f"M={m}"] = {"us_layer": round(total_ms * 1e3, 1), "GB/s": round(algo / total_ms / 1e6, 1),
                            "TFLOP/s": round(flops / total_ms / 1e9, 2),
-                           "path": "gemv" if m <= 32 else "gemm"}
-    out["q4_0_batch_sweep_llama70b_layer"] = sweep
+                           "roofline": {"bound": "hbm" if t_hbm >= t_mfma else "mfma", "frac": round(max(t_hbm, t_mfma) / (total_ms * 1e-3), 4)},
+                           "kernels": "rlx_gemv_q4_0_* (one batched launch)" if m <= 32 else
+                                      ("rlx_xprep + rlx_gemm64_q4_0" if m <= 128 else "rlx_xprep + rlx_gemm_q4_0") + " (+ rlx_splitk_reduce where K is cut)"}
+        for bfr in list(bufs.values()) + list(outs.values()) + ([ws] if ws else []):
+            bfr.free()
+    if with_cpu:  # the q projection at M = 1, in full
+        pk = _packed_of(ops, QuantScheme.GgufQ4_0, 8192, 8192, 50, 0.015)
+        xv = oracle.bf16_round(ops.philox_normal(31, 8192))
+        sweep["cpu_baseline"] = cpu(lambda: oracle.gguf_matmul_bt(xv, pk, 1, 8192, 8192, oracle.Q4_0), gemv_bytes(8192, 8192) / 1e9, "GB/s")
+        sweep["cpu_baseline"]["sample"] = "the q projection (8192 x 8192) at M = 1, one pass"
+    out["config5_q4_0_batch_sweep_llama70b_layer"] = sweep
     for q in weights.values():
         q.free()
     return out
+
+
+def _packed_of(ops, scheme, n, k, seed, sigma):
+    """The GGUF bytes tiled_weight() uploads, for the CPU leg."""
+    slab_rows = min(n, 4096)
+    w = (ops.philox_normal(seed, slab_rows * k) * np.float32(sigma)).astype(np.float32)
+    slab = ops.quantize(scheme, w).reshape(slab_rows, -1)
+    reps = (n + slab_rows - 1) // slab_rows
+    return np.ascontiguousarray(np.concatenate([np.roll(slab, 131 * r, axis=0) for r in range(reps)], axis=0)[:n]).reshape(-1)
 
 
 def cpu_baseline(base, xs):
@@ -788,24 +842,6 @@ def cpu_baseline_q4k_gemm():
             "cores": 1, "kind": "port",
             "sample": f"{ncols} of {n} output columns of the M=512 Q4_K GEMM, {dt:.1f} s, C restatement of rlx-cpu "
                       f"gguf_matmul_bt (scalar, single thread); full size = this x {n // ncols}"}
-
-
-def cpu_baselines_extra():
-    """The reference CPU path (oracle restatement, scalar, one thread) on bounded samples of the other configs."""
-    import oracle
-    from rlx_amd import QuantScheme, ops
-
-    out = {}
-    # FakeQuantize [8192, 4096] per column, in full (two scalar passes over 33.5 M elements)
-    rows, cols = 8192, 4096
-    x = ops.philox_normal(9, rows * cols)
-    t0 = time.time()
-    oracle.fake_quantize(x, (rows, cols), 1, 8)
-    dt = time.time() - t0
-    out["fake_quantize_8192x4096_cols"] = {"s": round(dt, 3), "GB/s_1R1W": round(2 * rows * cols * 4 / dt / 1e9, 3), "cores": 1,
-                                           "kind": "port", "sample": "the whole tensor, one call"}
-    out["q4_k_gemm_m512_gate_up_4096x14336"] = cpu_baseline_q4k_gemm()
-    return out
 
 
 if __name__ == "__main__":

@@ -10,6 +10,7 @@ rlx_blob_\name:
     blob dequant
     blob fakequant
     blob gemm
+    blob gemm_big
     blob gemv
     blob moe
     blob rowops

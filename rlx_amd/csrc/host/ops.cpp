@@ -101,6 +101,13 @@ struct GemmArgs {
     const int *perm;
     long long slab_bytes;
 };
+struct GemmBigArgs {  // mirrors kernels/gemm_big.hip
+    const void *a_img;
+    const void *b_img;
+    float *out;
+    const float *rowfac;
+    int m_out, n, steps;
+};
 struct XPrepArgs {
     const void *x;
     void *xh;
@@ -361,7 +368,7 @@ static GemmPlan gemm_plan(int scheme, int xk, int64_t m, int64_t k, int64_t n = 
     p.sxh_bytes = (size_t)p.m_rows * (p.k_pad / 256) * 32 * p.sums_kind;  // 16 or 32 halfs per row and super-block
     p.fac_bytes = ((size_t)m * 8 + 255) & ~(size_t)255;
     p.cs_bytes = xk == XK_CODES ? (size_t)p.k_pad * 4 : 0;
-    p.wimg_bytes = xk == XK_CODES ? (size_t)((n + 127) / 128 * 128) * p.k_pad * 2 : 0;
+    p.wimg_bytes = xk == XK_CODES ? (size_t)((n + 255) / 256 * 256) * p.k_pad * 2 : 0;  // whole 256-row tiles of the large-m kernel
     p.part_bytes = 0;
     if (n > 0) {
         const Layout L = layout_of(scheme);
@@ -430,7 +437,15 @@ static int launch_gemm(const void *x, int xk, const rlx_qweight *const *ws, floa
         WScaleArgs wa{w->dev, wimg, (const float *)((uint8_t *)workspace + p.fac_bytes), fac, w->dims.row_tiles, w->dims.units, (int)p.k_pad, w->sc_off()};
         void *wparams[] = {&wa};
         const KernelId wid = w->scheme == SCHEME_Q4_0 ? K_WSCALE_Q4_0 : K_WSCALE_Q8_0;
-        RLX_TRY(launch(wid, (unsigned)(p.k_pad / w->layout.unit_k), (unsigned)((w->dims.n + 127) / 128 * 8), 64, 0, stream, wparams));
+        RLX_TRY(launch(wid, (unsigned)(p.k_pad / w->layout.unit_k), (unsigned)((w->dims.n + 255) / 256 * 16), 64, 0, stream, wparams));
+        // Many rows: the 256 x 256 tile kernel for ready operands (two rounds of workgroups or more, so that its larger
+        // tile does not leave the chip half empty)
+        const long long big_tiles = (p.m_rows / 256) * ((w->dims.n + 255) / 256);
+        if (big_tiles >= 2LL * std::max(1, device_props().cu_count)) {
+            GemmBigArgs ba{xh, wimg, outs[0], fac, (int)m, (int)w->dims.n, (int)(p.k_pad / 64)};
+            void *bparams[] = {&ba};
+            return launch3(K_GEMM_BIG_F16W, (unsigned)((w->dims.n + 255) / 256), (unsigned)(p.m_rows / 256), 1, 512, 2 * 65536, stream, bparams);
+        }
     } else if (!prepared) {
         RLX_TRY(launch_xprep(x, xk, m, w->dims.k, p, workspace, stream));
     }

@@ -179,6 +179,36 @@ def test_config4_chain_full_size(oracle, fq_is_output):
         assert err <= TOL
 
 
+def test_fq_code_image_many_rows_ragged(oracle):
+    # enough output tiles for the 256 x 256 kernel of ready operands (two rounds of workgroups), with nothing aligned: rows
+    # and columns that end inside a tile, k that is no multiple of 64. Column windows over all rows, bands of rows over
+    # all columns, the last row and column among them.
+    rows, k, n = 8000, 1056, 4000
+    rng = np.random.default_rng(71)
+    x = rng.standard_normal((rows, k)).astype(np.float32)
+    x[rng.random((rows, k)) < 0.001] *= np.float32(20.0)
+    packed = tiled_packed(Q4_0, n, k, 72, 0.02).reshape(-1)
+    g = Graph.new("cfg4_ragged_big")
+    xi = g.input("x", Shape.new([rows, k], DType.F32))
+    fq = g.add_node(Op.FakeQuantize(8, 1), [xi], Shape.new([rows, k], DType.F32))
+    w = g.param("w", Shape.new([len(packed)], DType.U8))
+    y = g.add_node(Op.DequantMatMul(QuantScheme.GgufQ4_0), [fq, w], Shape.new([rows, n], DType.F32))
+    g.set_outputs([y])
+    c = Session().compile(g)
+    assert "[x: code image]" in c.describe_plan()
+    c.set_param_typed("w", packed, DType.U8)
+    y_got = c.run([("x", x)])[0].reshape(rows, n)
+    fq_ref, _, _ = oracle.fake_quantize(x, x.shape, 1, 8)
+    for n0 in (0, 250, 2040, n - 16):
+        err = rel_err(y_got[:, n0:n0 + 16], oracle.gguf_matmul_f64(fq_ref, packed, rows, k, n, Q4_0, n0, n0 + 16))
+        say(f"   ragged code image, columns {n0}..{n0 + 16}, all rows: max rel err {err:.3e}")
+        assert err <= TOL
+    for r0 in (0, 254, 4095, rows - 4):
+        err = rel_err(y_got[r0:r0 + 4], oracle.gguf_matmul_f64(fq_ref[r0:r0 + 4], packed, 4, k, n, Q4_0))
+        say(f"   ragged code image, rows {r0}..{r0 + 4}, all columns: max rel err {err:.3e}")
+        assert err <= TOL
+
+
 def test_two_fake_quantize_producers_in_one_step(oracle):
     # Two FakeQuantize nodes of equal depth, each feeding a prefill matmul of the same scheme: the matmuls land in one step,
     # whose single workspace can hold one operand image. The first producer writes the image; the second keeps its f32
