@@ -161,6 +161,7 @@ struct rlx_exec {
     // (a copy from pageable memory is staged by the runtime one buffer at a time).
     size_t in_lo = 0, in_hi = 0, out_lo = 0, out_hi = 0;  // arena spans of all inputs / all outputs
     uint8_t *stage = nullptr;                             // pinned: [in span][out span], allocated on the first run()
+    uint8_t *stage_dev = nullptr;                         // the same memory as the device addresses it (null: copies go through hipMemcpyAsync)
     bool stage_tried = false;
 
     ~rlx_exec() {
@@ -1045,6 +1046,7 @@ static int check_input(rlx_exec *e, const char *name, const void *data, size_t n
 }
 
 constexpr size_t kStageCap = 16u << 20;  // beyond this a copy is long enough to hide how it is issued
+constexpr size_t kKernelCopyCap = 1u << 20;  // up to this the pinned staging area is read and written by a copy kernel
 
 static int run_common(rlx_exec *e, const rlx_named_buf *inputs, size_t n_inputs, rlx_out_buf *outputs, size_t n_outputs,
                       bool typed) {
@@ -1061,9 +1063,16 @@ static int run_common(rlx_exec *e, const rlx_named_buf *inputs, size_t n_inputs,
     if (!e->stage_tried) {
         e->stage_tried = true;
         if (in_span + out_span > 0 && in_span + out_span <= kStageCap &&
-            hipHostMalloc((void **)&e->stage, in_span + out_span, hipHostMallocDefault) != hipSuccess) {
+            hipHostMalloc((void **)&e->stage, in_span + out_span, hipHostMallocMapped) != hipSuccess) {
             (void)hipGetLastError();
             e->stage = nullptr;  // no pinned memory to be had: the copies go from the caller's buffers
+        }
+        // Small spans are moved by the library's copy kernel reading / writing the pinned memory itself: two more launches on
+        // the stream instead of two trips through the copy engine, whose set-up costs more than these few KB take to move.
+        if (e->stage && in_span + out_span <= kKernelCopyCap && in_span % 16 == 0 && out_span % 16 == 0 &&
+            hipHostGetDevicePointer((void **)&e->stage_dev, e->stage, 0) != hipSuccess) {
+            (void)hipGetLastError();
+            e->stage_dev = nullptr;
         }
     }
     int warn = RLX_OK;
@@ -1089,7 +1098,10 @@ static int run_common(rlx_exec *e, const rlx_named_buf *inputs, size_t n_inputs,
         if (nd->cur_dtype != dt) e->drop_graph();  // the captured launches were specialised on the old dtype
         nd->cur_dtype = dt;
     }
-    if (staged_in) RLX_HIP(hipMemcpyAsync(e->arena + e->in_lo, e->stage, in_span, hipMemcpyHostToDevice, e->stream));
+    if (staged_in) {
+        if (e->stage_dev) RLX_TRY(rlx_mi355x_memcpy_d2d(e->arena + e->in_lo, e->stage_dev, in_span, e->stream));
+        else RLX_HIP(hipMemcpyAsync(e->arena + e->in_lo, e->stage, in_span, hipMemcpyHostToDevice, e->stream));
+    }
     RLX_TRY(rlx_exec_launch(e));
     bool staged_out = e->stage && out_span > 0;
     for (size_t i = 0; i < n_outputs; i++) {
@@ -1101,7 +1113,10 @@ static int run_common(rlx_exec *e, const rlx_named_buf *inputs, size_t n_inputs,
         }
         if (nd.slot.offset < e->out_lo || nd.slot.offset + bytes > e->out_hi) staged_out = false;  // an input handed back as output
     }
-    if (staged_out) RLX_HIP(hipMemcpyAsync(e->stage + in_span, e->arena + e->out_lo, out_span, hipMemcpyDeviceToHost, e->stream));
+    if (staged_out) {
+        if (e->stage_dev) RLX_TRY(rlx_mi355x_memcpy_d2d(e->stage_dev + in_span, e->arena + e->out_lo, out_span, e->stream));
+        else RLX_HIP(hipMemcpyAsync(e->stage + in_span, e->arena + e->out_lo, out_span, hipMemcpyDeviceToHost, e->stream));
+    }
     for (size_t i = 0; i < n_outputs; i++) {
         Node &nd = e->nodes[e->outputs[i]];
         const size_t bytes = (size_t)nd.numel * dtype_size(nd.d.dtype);
