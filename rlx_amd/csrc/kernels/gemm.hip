@@ -95,6 +95,11 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
     constexpr int WN = GEMM_NT / (32 * TJ), WM = 8 / WN, MT = WM * TI * 32;  // wave grid and rows per workgroup
     constexpr int NSA = MT / 32, SA = 4 * NSA * 1024, ST = SA + GEMM_STAGE_B;  // LDS stage: activations [4][NSA][1 KB], then weights
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    // Q4_K / Q5_K: what the per-super-block scaling needs goes through LDS instead of living in registers for two steps.
+    // sb_meta_s[parity of the super-block][W row of the tile]: the row's 16 meta bytes, left by the wave that decodes the row;
+    // sb_sum_s[half][x row of the tile]: the eight leading / eight residual block sums of the super-block being multiplied.
+    __shared__ uint4_t sb_meta_s[K4 ? 2 * GEMM_NT : 1];
+    __shared__ uint4_t sb_sum_s[K4 ? 2 * MT : 1];
 
     const int tid = threadIdx.x, lane = tid & 63;
     int expert = 0;
@@ -226,6 +231,7 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
             if (q == 0 && jl == 0) {
                 uint32_t mn[2];
                 const uint4_t &m4 = b_meta[0];
+                if (b_g == 0) sb_meta_s[((step >> 2) & 1) * GEMM_NT + wave * 16 + b_n16] = m4;  // for scale_sb, several steps from now
                 q4k_scales(m4[1], m4[2], m4[3], b_sc, mn);
                 b_sc[0] &= b_keep;  // a dead tile decodes to zeros
                 b_sc[1] &= b_keep;
@@ -350,15 +356,24 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
             sb_now = sb;
             return;
         }
-#pragma unroll
-        for (int j = 0; j < TJ; j++) w_meta[j] = *(const uint4_t *)(my_meta[j] + (long long)sb * L.unit_bytes);
-#pragma unroll
-        for (int i = 0; i < TI; i++) {
-            long long row = m_tile0 + (wm * TI + i) * 32 + lr;
-            fs[i].u4 = *(const uint4_t *)(a.sxh + (row * (a.k_pad / 256) + sb) * 16 + lh * 8);
-        }
     };
-    auto scale_sb = [&]() {
+    // Q4_K / Q5_K: thread t carries 16 bytes of the tile's block sums (row t / 2, half t % 2) of a super-block from memory
+    // to sb_sum_s, one step ahead of its store like the activation chunks.
+    uint4_t sx_reg = {0, 0, 0, 0};
+    const __amdgpu_buffer_rsrc_t sx_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)(K4 ? a.sxh + (long long)m_tile0 * (a.k_pad / 256) * 16 : a.sxh), 0, (K4 && wave < 2 * MT / 64) ? 0x7FFFFFFF : 0, 0x00020000);  // wave-uniform
+    const int sx_voff = (tid >> 1) * (a.k_pad / 256) * 32 + (tid & 1) * 16;
+    auto fetch_sx = [&](int sb) { sx_reg = ld128(sx_rsrc, sx_voff, sb * 32); };
+    auto store_sx = [&]() {
+        if (tid < 2 * MT) sb_sum_s[(tid & 1) * MT + (tid >> 1)] = sx_reg;
+    };
+    auto scale_sb = [&](int sb) {
+        if constexpr (K4) {
+#pragma unroll
+            for (int j = 0; j < TJ; j++) w_meta[j] = sb_meta_s[(sb & 1) * GEMM_NT + (wn * TJ + j) * 32 + lr];
+#pragma unroll
+            for (int i = 0; i < TI; i++) fs[i].u4 = sb_sum_s[lh * MT + (wm * TI + i) * 32 + lr];
+        }
         if constexpr (K6 || K8) {  // total += d * P
 #pragma unroll
             for (int j = 0; j < TJ; j++) {
@@ -528,23 +543,35 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
                 const int step = sbase + q;
                 if (step < step1) {
                     if constexpr (GRP == 0) {
+                        if constexpr (K4) {
+                            if (q == 1) fetch_sx(step >> 2);
+                        }
                         compute(smem + s0, q, step + 1, (q + 1) & 3);
                         __syncthreads();
                         preload(smem + s1);
                         data(step + 2, (q + 2) & 3, smem + s2);
-                        if constexpr (SB) {
+                        if constexpr (K4) {
+                            if (q == 1) store_sx();
+                            if (q == 3) scale_sb(step >> 2);
+                        } else if constexpr (SB) {
                             if (q == 1) load_sb_meta(step >> 2);
-                            if (q == 3) scale_sb();
+                            if (q == 3) scale_sb(step >> 2);
                         }
                         __syncthreads();
                     } else {
                         preload(smem + s0);
                         data(step + 1, (q + 1) & 3, smem + s1);
-                        if constexpr (SB) {
+                        if constexpr (K4) {
+                            if (q == 1) store_sx();
+                            if (q == 0 && step > step0) scale_sb((step >> 2) - 1);  // the super-block finished in the last iteration
+                        } else if constexpr (SB) {
                             if (q == 1) load_sb_meta(step >> 2);
-                            if (q == 0 && step > step0) scale_sb();  // the super-block finished in the last iteration
+                            if (q == 0 && step > step0) scale_sb((step >> 2) - 1);
                         }
                         __syncthreads();
+                        if constexpr (K4) {
+                            if (q == 0) fetch_sx(step >> 2);
+                        }
                         compute(smem + s0, q, step + 1, (q + 1) & 3);
                         __syncthreads();
                     }
@@ -556,7 +583,7 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
             }
         }
         if constexpr (SB && GRP == 1) {
-            if (step0 < step1) scale_sb();
+            if (step0 < step1) scale_sb((step1 - 1) >> 2);
         }
     };
     if (grp == 0) run(std::integral_constant<int, 0>{});
