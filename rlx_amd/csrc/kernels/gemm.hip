@@ -148,7 +148,7 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
             b_dst[jl] = SA + frag_offset(4, 2 * jl + (b_g >> 1), row >> 5, row & 31, b_g & 1);
     }
 
-    // Register-resident prefetch: activations one step ahead, packed weights two.
+    // Register-resident prefetch (AD and FD below say how far ahead).
     uint4_t a_reg[2][4];                                // activations of the next steps, [step parity] (Q4_K: one set)
     uint4_t b_q[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};      // [chunk parity] packed codes of a two-step chunk (Q8_0: [step parity])
     uint4_t b_meta[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};   // Q4_K: [0] = meta of the super-block decoded next; else [chunk parity] .x/.y = four f16 scales
@@ -159,6 +159,10 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
     // Activations run AD steps ahead of their LDS store: two where registers allow (their loads come through L2 with
     // the whole workgroup's 32 KB per step behind them), one for Q4_K whose second accumulator set takes the room.
     constexpr int AD = SB ? 1 : 2;
+    // Packed weights: a register slot is refilled FD steps ahead of the step whose data half emptied it. Where a slot holds a
+    // two-step chunk and there are two of them (Q4_0, Q4_K / Q5_K, Q6_K), the slot that was emptied last takes the chunk after
+    // the one waiting in the other slot: three steps ahead, a full chunk of latency cover with no more registers.
+    constexpr int FD = (SCHEME == SCHEME_Q4_0 || K4 || K6) ? 3 : 1;
     // Buffer loads: wave-uniform descriptor and scalar offset, constant per-lane offset, so a fetch costs no VALU.
     // A wave that moves no activation chunk (64-row tile) gets an empty range: its loads return zeros without traffic.
     const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)a_base, 0, a_mine ? 0x7FFFFFFF : 0, 0x00020000);
@@ -455,7 +459,7 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
     // ---- the two halves of a step ------------------------------------------------------------------------
     // compute: the sixteen (TI = TJ = 2) MFMAs of one 64-column step.
     // It also issues, between the MFMAs, the global loads that refill the registers this wave's last data half emptied
-    // (step fstep, phase fq): activations of step fstep + AD and weights of step fstep + 1. Issuing a load can stall a
+    // (step fstep, phase fq): activations of step fstep + AD and weights of step fstep + FD. Issuing a load can stall a
     // wave for tens of cycles when the CU's vector-memory queue is full; here that time is MFMA shadow.
     auto compute = [&](const uint8_t *stage, int q, int fstep, int fq) {
         const int last = step1 - 1;
@@ -465,7 +469,7 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
             const int buf = ks % NB;
             if (ks + PD < 4) load_frags(stage, ks + PD, (ks + PD) % NB);
             if (ks == 0) fetch_a(min(fstep + AD, last), AD == 2 ? (fq & 1) : 0);
-            if (ks == 1) fetch_b(min(fstep + 1, last), (fq + 1) & 3);
+            if (ks == 1) fetch_b(min(fstep + FD, last), (fq + FD) & 3);
 #pragma unroll
             for (int i = 0; i < TI; i++)
 #pragma unroll
@@ -526,6 +530,10 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
         data(step0, 0, smem);
         fetch_a(min(step0 + AD, last), 0);
         fetch_b(min(step0 + 1, last), 1);
+        if constexpr (FD == 3) {
+            fetch_b(min(step0 + 2, last), 2);
+            fetch_b(min(step0 + 3, last), 3);
+        }
         if (grp == 0) data(step0 + 1, 1, smem + ST);
     }
     __syncthreads();
