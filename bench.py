@@ -228,12 +228,12 @@ def main():
     # memory, the launch, the outputs back in one copy, synchronous) - PCIe and call overhead included, reported beside
     # the headline, never as `value`
     ins = [(src, v) for src, v in {WIRING[args.wiring][n]: xs[n] for n, _, _ in LLAMA8B if xs[n] is not None}.items()]
-    for _ in range(5):
-        layers[0].run(ins)
-    t1 = time.time()
-    for i in range(100):
+    for i in range(40):  # every layer's staging area allocated and the allocator's pages warm before the clock starts
         layers[i % len(layers)].run(ins)
-    host_ms = (time.time() - t1) / 100 * 1e3
+    t1 = time.perf_counter()
+    for i in range(200):
+        layers[i % len(layers)].run(ins)
+    host_ms = (time.perf_counter() - t1) / 200 * 1e3
     result["config"]["host_boundary_ms_per_call"] = round(host_ms, 4)
     del layers
     # the other wiring of the same layer, beside the headline: "layer" is what a decode loop gets (four launches, each

@@ -6,6 +6,7 @@
 // rlx-compile/src/memory.rs:76-94,203-219) and extends it the way a quantized GPU backend needs: a packed U8
 // param owns a slot sized for the *device layout* of its weights, filled once by set_param_typed.
 #include <algorithm>
+#include <chrono>
 #include <cstring>
 #include <functional>
 #include <map>
@@ -163,6 +164,10 @@ struct rlx_exec {
     uint8_t *stage = nullptr;                             // pinned: [in span][out span], allocated on the first run()
     uint8_t *stage_dev = nullptr;                         // the same memory as the device addresses it (null: copies go through hipMemcpyAsync)
     bool stage_tried = false;
+    // While run() enqueues a schedule whose outputs nothing else reads, the output slots stand for their places in the
+    // pinned staging area: the kernels store the results where the host picks them up, and no copy follows them.
+    bool out_direct = false;
+    bool out_pure = false;  // no node of the graph reads an output slot (set with the staging area)
 
     ~rlx_exec() {
         for (auto &nd : nodes) {
@@ -181,7 +186,10 @@ struct rlx_exec {
         graph_exec = nullptr;
         graph = nullptr;
     }
-    void *ptr(const Slot &s) const { return arena + s.offset; }
+    void *ptr(const Slot &s) const {
+        if (out_direct && s.offset >= out_lo && s.offset < out_hi) return stage_dev + (in_hi - in_lo) + (s.offset - out_lo);
+        return arena + s.offset;
+    }
 };
 
 extern "C" {
@@ -1074,6 +1082,12 @@ static int run_common(rlx_exec *e, const rlx_named_buf *inputs, size_t n_inputs,
             (void)hipGetLastError();
             e->stage_dev = nullptr;
         }
+        e->out_pure = true;
+        for (const Node &nd : e->nodes)
+            for (uint32_t j = 0; j < nd.d.n_inputs; j++) {
+                const Slot &src = e->nodes[nd.d.inputs[j]].slot;
+                if (src.offset >= e->out_lo && src.offset < e->out_hi) e->out_pure = false;
+            }
     }
     int warn = RLX_OK;
     // every input of the graph named exactly once -> one copy of the whole input span out of pinned memory
@@ -1102,7 +1116,6 @@ static int run_common(rlx_exec *e, const rlx_named_buf *inputs, size_t n_inputs,
         if (e->stage_dev) RLX_TRY(rlx_mi355x_memcpy_d2d(e->arena + e->in_lo, e->stage_dev, in_span, e->stream));
         else RLX_HIP(hipMemcpyAsync(e->arena + e->in_lo, e->stage, in_span, hipMemcpyHostToDevice, e->stream));
     }
-    RLX_TRY(rlx_exec_launch(e));
     bool staged_out = e->stage && out_span > 0;
     for (size_t i = 0; i < n_outputs; i++) {
         Node &nd = e->nodes[e->outputs[i]];
@@ -1113,7 +1126,13 @@ static int run_common(rlx_exec *e, const rlx_named_buf *inputs, size_t n_inputs,
         }
         if (nd.slot.offset < e->out_lo || nd.slot.offset + bytes > e->out_hi) staged_out = false;  // an input handed back as output
     }
-    if (staged_out) {
+    // After such a run the arena's output slots do not hold the results (rlx_exec_launch puts them there).
+    const bool direct = staged_out && e->stage_dev && e->out_pure && !e->graph_exec;
+    e->out_direct = direct;
+    const int launched = rlx_exec_launch(e);
+    e->out_direct = false;
+    RLX_TRY(launched);
+    if (staged_out && !direct) {
         if (e->stage_dev) RLX_TRY(rlx_mi355x_memcpy_d2d(e->stage_dev + in_span, e->arena + e->out_lo, out_span, e->stream));
         else RLX_HIP(hipMemcpyAsync(e->stage + in_span, e->arena + e->out_lo, out_span, hipMemcpyDeviceToHost, e->stream));
     }
@@ -1123,6 +1142,14 @@ static int run_common(rlx_exec *e, const rlx_named_buf *inputs, size_t n_inputs,
         if (!staged_out) RLX_HIP(hipMemcpyAsync(outputs[i].data, e->ptr(nd.slot), bytes, hipMemcpyDeviceToHost, e->stream));
         outputs[i].nbytes = bytes;
         outputs[i].dtype = nd.d.dtype;
+    }
+    // The caller is waiting for these few dozen microseconds of work: poll the stream for a bounded time before handing
+    // the wait to the runtime (whose blocking wait wakes up later than the work ends).
+    if (staged_out && e->stage_dev) {
+        const auto t0 = std::chrono::steady_clock::now();
+        while (hipStreamQuery(e->stream) == hipErrorNotReady)
+            if (std::chrono::steady_clock::now() - t0 > std::chrono::microseconds(300)) break;
+        (void)hipGetLastError();
     }
     RLX_HIP(hipStreamSynchronize(e->stream));
     if (staged_out)
