@@ -427,7 +427,10 @@ typedef struct rlx_out_buf {
     uint32_t dtype;   /* dtype written (the output node's declared dtype) */
 } rlx_out_buf;
 
-/* ExecutableGraph::run(&[(name, &[f32])]) -> Vec<Vec<f32>>: host f32 in, host f32 out (synchronous). */
+/* ExecutableGraph::run(&[(name, &[f32])]) -> Vec<Vec<f32>>: host f32 in, host f32 out (synchronous).
+ * The results are returned in `outputs` only: when nothing in the graph reads an output and the spans are small, the
+ * kernels of this call store them straight into pinned host memory and the arena's output slots keep what the last
+ * rlx_exec_launch left there (rlx_exec_output_slot is the device-resident path's accessor, to be used after launch). */
 int rlx_exec_run(rlx_exec *e, const rlx_named_buf *inputs, size_t n_inputs, rlx_out_buf *outputs, size_t n_outputs);
 /* ExecutableGraph::run_typed: inputs in F32/F16/BF16 bytes. 16-bit inputs stay 16-bit on the device. */
 int rlx_exec_run_typed(rlx_exec *e, const rlx_named_buf *inputs, size_t n_inputs, rlx_out_buf *outputs,

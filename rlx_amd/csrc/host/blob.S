@@ -12,6 +12,7 @@ rlx_blob_\name:
     blob gemm
     blob gemm_big
     blob gemv
+    blob gemv_wide
     blob moe
     blob rowops
     blob topk

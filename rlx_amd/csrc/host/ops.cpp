@@ -108,6 +108,33 @@ struct GemmBigArgs {  // mirrors kernels/gemm_big.hip
     const float *rowfac;
     int m_out, n, steps;
 };
+constexpr int GEMVW_MAX_SEG = 8;
+struct GemvWSeg {  // mirrors kernels/gemv_wide.hip
+    const void *w;
+    float *out;
+    int n, row_tiles, wg_begin, k_slices, slice_units;
+};
+struct GemvWArgs {
+    GemvWSeg seg[GEMVW_MAX_SEG];
+    int nseg, m, pair_rows, units, k_steps;
+    const void *xh;
+    const float *rowfac;
+};
+struct SplitReduceArgs {  // mirrors kernels/gemm.hip
+    const float *part[8];
+    float *out[8];
+    long long elems[8];
+    int split[8];
+};
+// One launch adds the K slices of up to eight matrices (ascending K, fixed order) into their outputs.
+static int launch_split_reduce(const SplitReduceArgs &ra, int nseg, hipStream_t stream) {
+    if (nseg == 0) return RLX_OK;
+    long long most = 0;
+    for (int i = 0; i < nseg; i++) most = std::max(most, (ra.elems[i] + 3) / 4);
+    SplitReduceArgs a = ra;
+    void *rparams[] = {&a};
+    return launch3(K_SPLITK_REDUCE, (unsigned)std::min<long long>((most + 255) / 256, 2048), (unsigned)nseg, 1, 256, 0, stream, rparams);
+}
 struct XPrepArgs {
     const void *x;
     void *xh;
@@ -358,6 +385,26 @@ struct GemmPlan {
     size_t total() const { return image_end() + wimg_bytes + part_bytes; }
 };
 static bool gemm_skinny(int xk, int64_t m) { return (xk == 0 ? 2 * m : m) <= 128; }
+// Up to 64 image rows of Q4_0 / Q8_0 run rlx_gemvw_* (kernels/gemv_wide.hip): weights decoded in registers by the wave
+// that multiplies them, 256-row blocks of W per workgroup.
+static bool gemm_wide(int scheme, int xk, int64_t m) {
+    return (scheme == SCHEME_Q4_0 || scheme == SCHEME_Q8_0) && xk != XK_CODES && (xk == 0 ? 2 * m : m) <= 64;
+}
+// K slices of one matrix in a launch of `launch_bytes` packed bytes in all: a workgroup should get about one CU's share
+// of the launch, at least 512 KB (one 70B layer at 64 rows, us: 218 with half a CU's share and 256 KB, 203 with this, 230
+// with at least 1 MB); the slices' partial results (written and read once: 8 m n bytes per slice) may cost up to half
+// the matrix's own bytes. Slices are whole 256-column chunks of at least four units.
+static GemmSplit wide_split(const Layout &L, const WeightDims &D, int64_t m, size_t launch_bytes) {
+    const int cus = device_props().cu_count > 0 ? device_props().cu_count : 256;
+    const size_t target = std::max<size_t>(launch_bytes / (size_t)cus, 512u << 10);
+    const size_t block_bytes = (size_t)16 * (size_t)D.units * (size_t)L.unit_bytes;
+    int64_t split = (int64_t)((block_bytes + target / 2) / target);
+    split = std::min<int64_t>(split, (int64_t)((size_t)D.bytes / 2 / ((size_t)8 * (size_t)m * (size_t)D.n)));
+    split = std::max<int64_t>(1, std::min<int64_t>(split, D.units / 4));
+    int units_per_split = (int)((D.units + split - 1) / split);
+    units_per_split = (units_per_split + 1) / 2 * 2;
+    return GemmSplit{(int)((D.units + units_per_split - 1) / units_per_split), units_per_split};
+}
 static GemmPlan gemm_plan(int scheme, int xk, int64_t m, int64_t k, int64_t n = 0) {
     GemmPlan p;
     const int64_t rv = xk == 0 ? 2 * m : m;
@@ -370,7 +417,11 @@ static GemmPlan gemm_plan(int scheme, int xk, int64_t m, int64_t k, int64_t n = 
     p.cs_bytes = xk == XK_CODES ? (size_t)p.k_pad * 4 : 0;
     p.wimg_bytes = xk == XK_CODES ? (size_t)((n + 255) / 256 * 256) * p.k_pad * 2 : 0;  // whole 256-row tiles of the large-m kernel
     p.part_bytes = 0;
-    if (n > 0) {
+    if (n > 0 && gemm_wide(scheme, xk, m)) {
+        const WeightDims D = weight_dims(scheme, n, k);
+        const GemmSplit sp = wide_split(layout_of(scheme), D, m, (size_t)D.bytes);  // alone in its launch: the most slices it can get
+        if (sp.split > 1) p.part_bytes = (size_t)sp.split * (size_t)m * (size_t)n * 4;
+    } else if (n > 0) {
         const Layout L = layout_of(scheme);
         const bool skinny = gemm_skinny(xk, m);
         const int spu = xk == XK_CODES ? 1 : L.unit_k / 64;
@@ -404,7 +455,7 @@ static int launch_xprep(const void *x, int xk, int64_t m, int64_t k, const GemmP
 // them) from the previous launch of a batch on the same stream, so the conversion pass is skipped.
 static int launch_gemm(const void *x, int xk, const rlx_qweight *const *ws, float *const *outs, int count, int64_t m,
                        void *workspace, size_t workspace_bytes, hipStream_t stream, bool prepared = false) {
-    if (count < 1 || count > GEMM_MAX_SEG || (xk == XK_CODES && count != 1)) {
+    if (count < 1 || count > (gemm_wide(ws[0]->scheme, xk, m) ? GEMVW_MAX_SEG : GEMM_MAX_SEG) || (xk == XK_CODES && count != 1)) {
         set_error("gguf_matmul_bt: %d matrices in one prefill launch", count);
         return RLX_ERR_INVALID;
     }
@@ -450,6 +501,49 @@ static int launch_gemm(const void *x, int xk, const rlx_qweight *const *ws, floa
         RLX_TRY(launch_xprep(x, xk, m, w->dims.k, p, workspace, stream));
     }
     const int64_t k_units = codes ? p.k_pad / 64 : w->dims.units;  // K units of the operand the kernel reads
+
+    if (gemm_wide(w->scheme, xk, m)) {
+        size_t launch_bytes = 0, part_need = 0;
+        for (int i = 0; i < count; i++) launch_bytes += (size_t)ws[i]->dims.bytes;
+        GemmSplit sps[GEMVW_MAX_SEG];
+        for (int i = 0; i < count; i++) {
+            sps[i] = wide_split(ws[i]->layout, ws[i]->dims, m, launch_bytes);
+            if (sps[i].split > 1) part_need += (size_t)sps[i].split * (size_t)m * (size_t)ws[i]->dims.n * 4;
+        }
+        if (part_need > workspace_bytes - ops_end)  // a workspace without room for the slices: every matrix in one piece
+            for (int i = 0; i < count; i++) sps[i] = GemmSplit{1, (int)((ws[i]->dims.units + 1) / 2 * 2)};
+        GemvWArgs wa{};
+        long long wgs = 0;
+        size_t off = 0;
+        for (int i = 0; i < count; i++) {
+            float *dst = outs[i];
+            if (sps[i].split > 1) {
+                dst = (float *)((uint8_t *)workspace + ops_end + off);
+                off += (size_t)sps[i].split * (size_t)m * (size_t)ws[i]->dims.n * 4;
+            }
+            wa.seg[i] = GemvWSeg{ws[i]->dev, dst, (int)ws[i]->dims.n, (int)ws[i]->dims.row_tiles, (int)wgs, sps[i].split, sps[i].units_per_split};
+            wgs += (ws[i]->dims.row_tiles + 15) / 16 * sps[i].split;
+        }
+        wa.nseg = count;
+        wa.m = (int)m;
+        wa.pair_rows = xk == 0 ? 1 : 0;
+        wa.units = (int)w->dims.units;
+        wa.k_steps = (int)(p.k_pad / 64);
+        wa.xh = xh;
+        wa.rowfac = fac;
+        void *wparams[] = {&wa};
+        RLX_TRY(launch(w->scheme == SCHEME_Q4_0 ? K_GEMVW_Q4_0 : K_GEMVW_Q8_0, (unsigned)wgs, 1, 512, 2 * 32768, stream, wparams));
+        SplitReduceArgs ra{};
+        int nred = 0;
+        for (int i = 0; i < count; i++)
+            if (sps[i].split > 1) {
+                ra.part[nred] = wa.seg[i].out;
+                ra.out[nred] = outs[i];
+                ra.elems[nred] = (long long)m * ws[i]->dims.n;
+                ra.split[nred++] = sps[i].split;
+            }
+        return launch_split_reduce(ra, nred, stream);
+    }
 
     const int steps_per_unit = L.unit_k / 64;
     // Up to 128 activation rows run the 64-row tile (the weights are decoded once per 64 rows, but nothing is spent on
@@ -504,17 +598,15 @@ static int launch_gemm(const void *x, int xk, const rlx_qweight *const *ws, floa
                                                 : (skinny ? K_GEMM64_Q8_0 : K_GEMM_Q8_0);
     RLX_TRY(runtime_init());
     RLX_TRY(launch3(id, (unsigned)gx, (unsigned)gy, (unsigned)split, 512, skinny ? 3 * 24 * 1024 : 3 * 48 * 1024, stream, params));
+    SplitReduceArgs ra{};
     if (split > 1)
         for (int i = 0; i < count; i++) {
-            const float *part = a.seg[i].out;
-            float *out = outs[i];
-            long long elems = (long long)m * ws[i]->dims.n;
-            int nsl = split;
-            void *rparams[] = {&part, &out, &elems, &nsl};
-            const long long work = (elems + 3) / 4;
-            RLX_TRY(launch(K_SPLITK_REDUCE, (unsigned)std::min<long long>((work + 255) / 256, 2048), 1, 256, 0, stream, rparams));
+            ra.part[i] = a.seg[i].out;
+            ra.out[i] = outs[i];
+            ra.elems[i] = (long long)m * ws[i]->dims.n;
+            ra.split[i] = split;
         }
-    return RLX_OK;
+    return launch_split_reduce(ra, split > 1 ? count : 0, stream);
 }
 
 }  // namespace rlx
@@ -673,13 +765,14 @@ int rlx_mi355x_gguf_matmul_bt_batch(const void *const *xs_dev, int x_dtype, cons
         // q, k, v (and gate, up) of a layer share their input: its f16 image in the workspace is made once. An image
         // with block sums (Q4_K / Q5_K: per 32 columns; Q2_K: per 16) also serves a scheme that reads none, not the
         // other way round, and not a scheme that reads the other kind.
-        // Consecutive matrices with the same input and K go into one launch, up to GEMM_MAX_SEG at a time.
+        // Consecutive matrices with the same input and K go into one launch, up to GEMM_MAX_SEG at a time (GEMVW_MAX_SEG for the 33 - 64 row kernel).
         const void *have_x = nullptr;
         int64_t have_k = -1;
         int have_sums = 0;
         for (int i = 0; i < count;) {
             int c = 1;
-            while (i + c < count && c < GEMM_MAX_SEG && xs_dev[i + c] == xs_dev[i] && ws[i + c]->dims.k == ws[i]->dims.k &&
+            const int most = gemm_wide(ws[i]->scheme, xk, m) ? GEMVW_MAX_SEG : GEMM_MAX_SEG;
+            while (i + c < count && c < most && xs_dev[i + c] == xs_dev[i] && ws[i + c]->dims.k == ws[i]->dims.k &&
                    ws[i + c]->layout.unit_bytes == ws[i]->layout.unit_bytes && ws[i + c]->sc_off() == ws[i]->sc_off())
                 c++;
             const int sums = act_sums_kind(ws[i]->scheme);

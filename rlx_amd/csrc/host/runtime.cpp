@@ -3,7 +3,7 @@
 #include <cstring>
 #include <mutex>
 
-extern "C" const unsigned char rlx_blob_dequant[], rlx_blob_fakequant[], rlx_blob_gemm[], rlx_blob_gemm_big[], rlx_blob_gemv[], rlx_blob_moe[], rlx_blob_rowops[],
+extern "C" const unsigned char rlx_blob_dequant[], rlx_blob_fakequant[], rlx_blob_gemm[], rlx_blob_gemm_big[], rlx_blob_gemv[], rlx_blob_gemv_wide[], rlx_blob_moe[], rlx_blob_rowops[],
     rlx_blob_topk[];
 
 namespace rlx {
@@ -48,13 +48,13 @@ static const char *const kKernelNames[K_COUNT] = {
     "rlx_gemm_q4_k", "rlx_gemm_q4_0", "rlx_gemm_q8_0", "rlx_gemm64_q4_k", "rlx_gemm64_q4_0", "rlx_gemm64_q8_0", "rlx_gemm_q6_k", "rlx_gemm64_q6_k", "rlx_gemm_q5_k", "rlx_gemm64_q5_k", "rlx_xprep", "rlx_xrowscale", "rlx_argmax_finish", "rlx_topk_select", "rlx_rmsnorm_rows", "rlx_swiglu_rows",
     "rlx_gemm64g_q4_k", "rlx_gemm64g_q4_0", "rlx_gemm64g_q8_0", "rlx_gemm64g_q5_k", "rlx_gemm64g_q6_k", "rlx_moe_sort",
     "rlx_gemm_q8_k", "rlx_gemm64_q8_k", "rlx_gemm64g_q8_k", "rlx_gemm_q2_k", "rlx_gemm64_q2_k", "rlx_gemm64g_q2_k",
-    "rlx_gemm_f16w", "rlx_gemm64_f16w", "rlx_wscale_q4_0", "rlx_wscale_q8_0", "rlx_splitk_reduce", "rlx_gemm_big_f16w",
+    "rlx_gemm_f16w", "rlx_gemm64_f16w", "rlx_wscale_q4_0", "rlx_wscale_q8_0", "rlx_splitk_reduce", "rlx_gemm_big_f16w", "rlx_gemvw_q4_0", "rlx_gemvw_q8_0",
 };
 
 static std::once_flag g_once;
 static int g_init_rc = RLX_ERR_NO_DEVICE;
 static std::string g_init_error;
-static const unsigned char *const kBlobs[] = {rlx_blob_dequant, rlx_blob_fakequant, rlx_blob_gemm, rlx_blob_gemm_big, rlx_blob_gemv,
+static const unsigned char *const kBlobs[] = {rlx_blob_dequant, rlx_blob_fakequant, rlx_blob_gemm, rlx_blob_gemm_big, rlx_blob_gemv, rlx_blob_gemv_wide,
                                               rlx_blob_moe,     rlx_blob_rowops,    rlx_blob_topk};
 constexpr int kModules = (int)(sizeof kBlobs / sizeof kBlobs[0]);
 static hipModule_t g_module[kModules];

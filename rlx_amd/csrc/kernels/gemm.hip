@@ -693,7 +693,17 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
 
 // Split K: out[i] = part[0][i] + part[1][i] + ... in ascending K, the order the reference walks a row in
 // (rlx-cpu/src/gguf_matmul.rs:81-94), so a result does not depend on which workgroup finished first.
-__device__ __forceinline__ void splitk_reduce_body(const float *part, float *out, long long elems, int split) {
+struct SplitReduceArgs {  // up to eight matrices of one launch, one per blockIdx.y
+    const float *part[8];  // [split][elems]
+    float *out[8];
+    long long elems[8];
+    int split[8];
+};
+__device__ __forceinline__ void splitk_reduce_body(const SplitReduceArgs &a) {
+    const float *part = a.part[blockIdx.y];
+    float *out = a.out[blockIdx.y];
+    const long long elems = a.elems[blockIdx.y];
+    const int split = a.split[blockIdx.y];
     const long long stride = (long long)gridDim.x * blockDim.x;
     long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     if ((elems & 3) == 0 && (((uintptr_t)part | (uintptr_t)out) & 15) == 0) {
@@ -889,8 +899,6 @@ extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64g_q5_k(rlx::GemmA
 extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64g_q6_k(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_Q6K, 1, 1, true>(a); }
 extern "C" __global__ __launch_bounds__(512) void rlx_gemm_f16w(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_F16W, 2, 2>(a); }
 extern "C" __global__ __launch_bounds__(512, 4) void rlx_gemm64_f16w(rlx::GemmArgs a) { rlx::gemm_body<rlx::SCHEME_F16W, 1, 1>(a); }
-extern "C" __global__ __launch_bounds__(256) void rlx_splitk_reduce(const float *part, float *out, long long elems, int split) {
-    rlx::splitk_reduce_body(part, out, elems, split);
-}
+extern "C" __global__ __launch_bounds__(256) void rlx_splitk_reduce(rlx::SplitReduceArgs a) { rlx::splitk_reduce_body(a); }
 extern "C" __global__ __launch_bounds__(256) void rlx_xprep(rlx::XPrepArgs a) { rlx::xprep_body(a); }
 extern "C" __global__ __launch_bounds__(256) void rlx_xrowscale(rlx::XPrepArgs a) { rlx::xrowscale_body(a); }

@@ -486,6 +486,34 @@ def test_gemm_small(oracle, scheme, m, n, k, x_dtype):
     check_matmul(oracle, scheme, n, k, m, x_dtype=x_dtype, seed=m + n)
 
 
+@pytest.mark.parametrize("scheme", [Q4_0, Q8_0])
+@pytest.mark.parametrize("m,n,k,x_dtype", [(33, 272, 384, DType.BF16),    # ragged N (a dead tile in the block), three K units
+                                           (64, 4112, 8192, DType.BF16),  # seventeen 256-row blocks, K cut across workgroups
+                                           (20, 300, 1152, DType.F32),    # leading / residual row pairs, nine K units
+                                           (32, 512, 256, DType.F32), (48, 100, 128, DType.F16), (57, 16, 16384, DType.BF16)])
+def test_rows_33_to_64(oracle, scheme, m, n, k, x_dtype):
+    # the kernel between the decode kernel and the prefill tiles (Q4_0 / Q8_0, 33 - 64 binary16 rows or 17 - 32 f32 rows)
+    got, x, packed, _ = check_matmul(oracle, scheme, n, k, m, x_dtype=x_dtype, seed=3 * m + n,
+                                     cols=None if n * k * m < (1 << 27) else (n - 40, n))
+    xin = f32_to_bf16_bits(x) if x_dtype == DType.BF16 else x.astype(np.float16) if x_dtype == DType.F16 else x
+    w = ops.QWeight(scheme, packed, n, k)
+    again = ops.gguf_matmul_bt(xin, w, m, x_dtype)
+    assert np.array_equal(got.view(np.uint32), again.view(np.uint32))  # the slices of a cut K are added in a fixed order
+    # rows far outside binary16 keep the reference's f32 range (per-row powers of two in front of the image)
+    scale = np.ones((m, 1), np.float32)
+    scale[0], scale[m // 2], scale[m - 1] = 1e20, 3e-15, 7e7
+    xs = (x * scale).astype(np.float32)
+    if x_dtype == DType.BF16:
+        xs = oracle.bf16_round(xs)
+    if x_dtype != DType.F16:
+        big = ops.gguf_matmul_bt(f32_to_bf16_bits(xs) if x_dtype == DType.BF16 else xs, w, m, x_dtype)
+        n0 = max(0, n - 24)
+        ref = oracle.gguf_matmul_f64(xs, packed, m, k, n, scheme, n0, n)
+        rows = np.abs(big[:, n0:].astype(np.float64) - ref).max(axis=1) / np.maximum(np.abs(ref).max(axis=1), 1e-30)
+        assert np.all(np.isfinite(big)) and rows.max() <= 4e-3, rows.max()
+    w.free()
+
+
 def test_config3_q4k_gemm_m512_slices(oracle):
     # benchmark configuration 3 shapes at full size; the f64 oracle is run on column windows (it is O(m n k) scalar work)
     for n, k in [(14336, 4096), (4096, 14336)]:
@@ -852,3 +880,37 @@ def test_run_boundary_full_and_partial_inputs(oracle):
     check(c.run([("x2", b), ("x1", a2)]), a2, b, "all inputs again, other order")
     bf = c.run_typed([("x1", f32_to_bf16_bits(oracle.bf16_round(a)), DType.BF16), ("x2", b, DType.F32)])
     assert rel_err(bf[0][0].reshape(2, n), oracle.gguf_matmul_f64(oracle.bf16_round(a), p1, 2, k, n, Q4_0)) <= TOL
+
+
+def test_run_then_launch_read_the_same_results(oracle):
+    # run() lets the kernels store the results where the host picks them up; launch() + read_output() must still find them
+    # in the arena, whichever of the two came before, and a graph whose output feeds another node takes the copying path.
+    k, n = 384, 96
+    p1, p2 = make_weights(Q4_0, n, k, seed=211)[0], make_weights(Q8_0, k, n, seed=212)[0]
+    rng = np.random.default_rng(213)
+    for chained in (False, True):
+        g = Graph.new("pure_outputs" if not chained else "output_read_again")
+        x = g.input("x", Shape.new([3, k], DType.F32))
+        w1 = g.param("w1", Shape.new([len(p1)], DType.U8))
+        y1 = g.add_node(Op.DequantMatMul(QuantScheme.GgufQ4_0), [x, w1], Shape.new([3, n], DType.F32))
+        outs = [y1]
+        if chained:
+            w2 = g.param("w2", Shape.new([len(p2)], DType.U8))
+            outs.append(g.add_node(Op.DequantMatMul(QuantScheme.GgufQ8_0), [y1, w2], Shape.new([3, k], DType.F32)))
+        g.set_outputs(outs)
+        c = Session.new().compile(g)
+        c.set_param_typed("w1", p1, DType.U8)
+        if chained:
+            c.set_param_typed("w2", p2, DType.U8)
+        for rep in range(3):
+            a = rng.standard_normal((3, k)).astype(np.float32)
+            want = oracle.gguf_matmul_f64(a, p1, 3, k, n, Q4_0)
+            got = c.run([("x", a)])
+            assert rel_err(got[0].reshape(3, n), want) <= TOL, (chained, rep)
+            c.launch()
+            dev = c.read_output(0)
+            assert np.array_equal(dev.view(np.uint32), got[0].view(np.uint32)), (chained, rep)
+            if chained:
+                y1_f32 = got[0].reshape(3, n)
+                assert rel_err(got[1].reshape(3, k), oracle.gguf_matmul_f64(y1_f32, p2, 3, n, k, Q8_0)) <= TOL, rep
+                assert np.array_equal(c.read_output(1).view(np.uint32), got[1].view(np.uint32)), rep
