@@ -6,16 +6,21 @@ A step is one pass over one layer's seven projections (q, k, v, o, gate, up, dow
 compiled graph, each with its own f32 activation vector as the benchmark definition states, which the backend issues as
 one batched launch. The layers rotate through LAYERS distinct weight sets (~123 MB each), far more than the 256 MB of
 last-level cache, so every launch streams its weights from HBM. Inputs and weights are resident in HBM before the timed
-region, which is bracketed by HIP events on the launch stream after SETTLE_LAUNCHES untimed launches (the clocks of a
-fresh process take a few hundred launches to settle; a 20-step run then reads like a 2000-step one). One JSON line is
-printed; `value` is algorithmic bytes per second (packed weights + f32 activations in + f32 outputs out), the figure
-`roofline.frac` is taken from. Beside it in the same line:
+region: TIMED_BLOCKS blocks of --steps launches each, one after another on the launch stream with a HIP event at every
+block boundary, after SETTLE_LAUNCHES untimed launches (the clocks of a fresh process take a few hundred launches to
+settle; a 20-step run then reads like a 2000-step one). One JSON line is printed; `value` is algorithmic bytes per
+second (packed weights + f32 activations in + f32 outputs out) of the median block, the figure `roofline.frac` is taken
+from; `roofline.blocks` and `roofline.GB/s_min_max` give the fastest and the slowest block. Beside it in the same line:
   config.wiring_layer_ms            the same layer in dependency order (x -> q,k,v; q -> o; o -> gate,up; gate -> down):
                                     four dependent launches, what a decode loop gets;
   config.host_boundary_ms_per_call  the layer through rlx_exec_run with host buffers (PCIe and call overhead included);
   roofline.secondary                rlx_gemm_q4_k at M = 512 on 4096 -> 14336 (bf16 activations): the kernel's launches
-                                    alone between two events, the whole rlx_mi355x_gguf_matmul_bt call, the down
-                                    projection and the gate + up pair;
+                                    alone between two events, the whole rlx_mi355x_gguf_matmul_bt call with its own
+                                    fraction (whole_call), the down projection and the gate + up pair;
+  config.other_configs              the other benchmark configurations, each with its roofline fraction and a bounded CPU
+                                    sample: Q8_0 GEMV 4096 x 4096 (cold), FakeQuantize [8192, 4096] alone and as the
+                                    chain into the Q8_0 matmul, the Q4_0 batch sweep M = 1, 4, 16, 64, 256 over one
+                                    Llama-3-70B layer;
   cpu_baseline[.secondary]          the oracle's C restatement of the reference's scalar CPU path on a bounded sample.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--no-cpu] [--extra]
