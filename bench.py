@@ -513,7 +513,7 @@ def moe_config(rlx_amd, stream):
     tf = 2.0 * m * n * k / ms_s / 1e9
     out["q4_0_moe_grouped_1024_rows_of_8x14336x4096_bf16"] = {
         "us_expert_sorted": round(ms_s * 1e3, 1), "TFLOP/s": round(tf, 1), "us_launch_per_eight_rows": round(ms_r * 1e3, 1),
-        "launches": "sort + row scales + image (gathered) + one prefill launch over 64-row tiles"}
+        "launches": "sort + row scales + image (gathered) + one launch over 64-row tiles (rlx_gemvwg_q4_0: weights decoded in registers)"}
     qw.free()
     return out
 

@@ -60,7 +60,7 @@ enum KernelId : int {
     K_GEMM_Q4_K, K_GEMM_Q4_0, K_GEMM_Q8_0, K_GEMM64_Q4_K, K_GEMM64_Q4_0, K_GEMM64_Q8_0, K_GEMM_Q6_K, K_GEMM64_Q6_K, K_GEMM_Q5_K, K_GEMM64_Q5_K, K_XPREP, K_XROWSCALE, K_ARGMAX_FINISH, K_TOPK_SELECT, K_RMSNORM_ROWS, K_SWIGLU_ROWS,
     K_GEMM64G_Q4_K, K_GEMM64G_Q4_0, K_GEMM64G_Q8_0, K_GEMM64G_Q5_K, K_GEMM64G_Q6_K, K_MOE_SORT,
     K_GEMM_Q8_K, K_GEMM64_Q8_K, K_GEMM64G_Q8_K, K_GEMM_Q2_K, K_GEMM64_Q2_K, K_GEMM64G_Q2_K,
-    K_GEMM_F16W, K_GEMM64_F16W, K_WSCALE_Q4_0, K_WSCALE_Q8_0, K_SPLITK_REDUCE, K_GEMM_BIG_F16W, K_GEMVW_Q4_0, K_GEMVW_Q8_0,
+    K_GEMM_F16W, K_GEMM64_F16W, K_WSCALE_Q4_0, K_WSCALE_Q8_0, K_SPLITK_REDUCE, K_GEMM_BIG_F16W, K_GEMVW_Q4_0, K_GEMVW_Q8_0, K_GEMVWG_Q4_0, K_GEMVWG_Q8_0,
     K_COUNT
 };
 

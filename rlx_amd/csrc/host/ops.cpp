@@ -119,6 +119,9 @@ struct GemvWArgs {
     int nseg, m, pair_rows, units, k_steps;
     const void *xh;
     const float *rowfac;
+    const int *tile_expert;
+    const int *perm;
+    long long slab_bytes;
 };
 struct SplitReduceArgs {  // mirrors kernels/gemm.hip
     const float *part[8];
@@ -1225,6 +1228,23 @@ int rlx_mi355x_gguf_grouped_matmul_bt_ws(const void *x_dev, int x_dtype, const r
     void *sparams[] = {&sa};
     RLX_TRY(launch(K_MOE_SORT, 1, 1, 1024, 0, s, sparams));
     RLX_TRY(launch_xprep(x_dev, xk, m, w->dims.k, p.gemm, gws, s, perm, (int)p.perm_len));
+    if (w->scheme == SCHEME_Q4_0 || w->scheme == SCHEME_Q8_0) {  // a tile is 64 image rows: the 33 - 64 row kernel, one expert slab per tile
+        GemvWArgs wa{};
+        wa.seg[0] = GemvWSeg{w->dev, out_dev, (int)w->dims.n, (int)w->dims.row_tiles, 0, 1, (int)((w->dims.units + 1) / 2 * 2)};
+        wa.nseg = 1;
+        wa.m = (int)p.perm_len;  // bound of the sorted rows; every perm entry is a token below m <= perm_len
+        wa.pair_rows = xk == 0 ? 1 : 0;
+        wa.units = (int)w->dims.units;
+        wa.k_steps = (int)(p.gemm.k_pad / 64);
+        wa.xh = (uint8_t *)gws + p.gemm.fac_bytes;
+        wa.rowfac = (const float *)gws;
+        wa.tile_expert = tile_expert;
+        wa.perm = perm;
+        wa.slab_bytes = w->dims.bytes;
+        void *wparams[] = {&wa};
+        return launch3(w->scheme == SCHEME_Q4_0 ? K_GEMVWG_Q4_0 : K_GEMVWG_Q8_0, (unsigned)((w->dims.row_tiles + 15) / 16),
+                       (unsigned)(p.perm_len / p.group), 1, 512, 2 * 32768, s, wparams);
+    }
     const Layout L = w->layout;
     GemmArgs a{};
     a.seg[0] = GemmSeg{w->dev, out_dev, (int)w->dims.n, (int)w->dims.row_tiles, 0};

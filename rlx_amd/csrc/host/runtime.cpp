@@ -48,7 +48,7 @@ static const char *const kKernelNames[K_COUNT] = {
     "rlx_gemm_q4_k", "rlx_gemm_q4_0", "rlx_gemm_q8_0", "rlx_gemm64_q4_k", "rlx_gemm64_q4_0", "rlx_gemm64_q8_0", "rlx_gemm_q6_k", "rlx_gemm64_q6_k", "rlx_gemm_q5_k", "rlx_gemm64_q5_k", "rlx_xprep", "rlx_xrowscale", "rlx_argmax_finish", "rlx_topk_select", "rlx_rmsnorm_rows", "rlx_swiglu_rows",
     "rlx_gemm64g_q4_k", "rlx_gemm64g_q4_0", "rlx_gemm64g_q8_0", "rlx_gemm64g_q5_k", "rlx_gemm64g_q6_k", "rlx_moe_sort",
     "rlx_gemm_q8_k", "rlx_gemm64_q8_k", "rlx_gemm64g_q8_k", "rlx_gemm_q2_k", "rlx_gemm64_q2_k", "rlx_gemm64g_q2_k",
-    "rlx_gemm_f16w", "rlx_gemm64_f16w", "rlx_wscale_q4_0", "rlx_wscale_q8_0", "rlx_splitk_reduce", "rlx_gemm_big_f16w", "rlx_gemvw_q4_0", "rlx_gemvw_q8_0",
+    "rlx_gemm_f16w", "rlx_gemm64_f16w", "rlx_wscale_q4_0", "rlx_wscale_q8_0", "rlx_splitk_reduce", "rlx_gemm_big_f16w", "rlx_gemvw_q4_0", "rlx_gemvw_q8_0", "rlx_gemvwg_q4_0", "rlx_gemvwg_q8_0",
 };
 
 static std::once_flag g_once;

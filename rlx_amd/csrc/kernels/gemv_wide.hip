@@ -38,6 +38,12 @@ struct GemvWArgs {
     int k_steps;        // 64-column steps of the image (k_pad / 64)
     const uint8_t *xh;  // image of x: [k_steps][32 KB] for the first 256-row tile
     const float *rowfac;  // [m][2]: the power of two row i was multiplied by, and its inverse
+    // Expert-sorted launch (rlx_gemvwg_*; rlx-cpu/src/gguf_matmul.rs:101-139, 178-207): the image rows are tokens sorted by
+    // expert, every 64-row tile inside one expert's run (see rlx_moe_sort). blockIdx.y is the tile; it multiplies the
+    // slab tile_expert names (-1: past the last run) and writes row perm[.] of `out` (-1: a padding row).
+    const int *tile_expert;
+    const int *perm;
+    long long slab_bytes;
 };
 
 template <int SCHEME>
@@ -78,13 +84,18 @@ struct WideUnit<SCHEME_Q8_0> {
     }
 };
 
-template <int SCHEME>
+template <int SCHEME, bool GROUPED = false>
 __device__ __forceinline__ void gemv_wide_body(const GemvWArgs &a) {
     constexpr Layout L = layout_of(SCHEME);
     static_assert(L.unit_k == 128, "two 64-column image steps per unit");
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];  // two chunk buffers
 
     const int tid = threadIdx.x, l = tid & 63;
+    int expert = 0;
+    if constexpr (GROUPED) {
+        expert = a.tile_expert[blockIdx.y];  // workgroup-uniform
+        if (expert < 0) return;              // nothing to do, and no barrier has been reached
+    }
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int nrow = l & 15, g = l >> 4;
     int si = 0;
@@ -103,16 +114,20 @@ __device__ __forceinline__ void gemv_wide_body(const GemvWArgs &a) {
     for (int tt = 0; tt < 2; tt++) {
         const int tile = blk * 16 + wave * 2 + tt;
         keep[tt] = tile < sg.row_tiles ? 0xFFFFFFFFu : 0u;
-        wt[tt] = __builtin_amdgcn_make_buffer_rsrc((void *)(sg.w + (long long)(tile < sg.row_tiles ? tile : 0) * a.units * L.unit_bytes), 0,
-                                                   a.units * L.unit_bytes, 0x00020000);
+        wt[tt] = __builtin_amdgcn_make_buffer_rsrc((void *)(sg.w + (GROUPED ? (long long)expert * a.slab_bytes : 0LL) +
+                                                            (long long)(tile < sg.row_tiles ? tile : 0) * a.units * L.unit_bytes),
+                                                   0, a.units * L.unit_bytes, 0x00020000);
     }
 
     // Activation chunk: piece p = tid + 512 j of the 2048 16-byte pieces is (step j, k-slice (tid >> 7) & 3, sub-tile
     // (tid >> 6) & 1, lane): constant per-thread offset in the image, the step in the scalar offset; in LDS piece p sits
     // at 16 p, i.e. a wave's 64 pieces of a step are 1 KB in a row: one buffer load with the LDS bit per step and wave,
     // no registers in between.
-    const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)a.xh, 0, 0x7FFFFFFF, 0x00020000);
-    const int x_voff = ((tid >> 7) & 3) * 8192 + ((tid >> 6) & 1) * 1024 + l * 16;
+    // (expert-sorted: tile y of 64 rows is sub-tiles 2 (y % 4), + 1 of the image's 256-row tile y / 4)
+    const int ytile = GROUPED ? (int)blockIdx.y : 0;
+    const __amdgpu_buffer_rsrc_t x_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc((void *)(a.xh + (long long)(ytile >> 2) * a.k_steps * 32768), 0, 0x7FFFFFFF, 0x00020000);
+    const int x_voff = ((tid >> 7) & 3) * 8192 + (2 * (ytile & 3) + ((tid >> 6) & 1)) * 1024 + l * 16;
     typedef __attribute__((address_space(3))) void *lds_ptr;
     auto fetch_x = [&](int unit, uint8_t *buf) {  // the chunk that starts at K unit `unit` (even); past the image: its last steps again
 #pragma unroll
@@ -201,7 +216,14 @@ __device__ __forceinline__ void gemv_wide_body(const GemvWArgs &a) {
     // columns and eight lanes store one whole 128-byte row of the block; the rows' factors come through LDS as well.
     constexpr int STRIDE = 36;  // floats per row of the block in LDS: rows four apart land in different banks
     float *fac_s = (float *)(smem + 8 * 32 * STRIDE * 4);
-    if (tid < 64) fac_s[tid] = tid < a.m ? a.rowfac[2 * tid + 1] : 0.f;
+    int *orow_s = (int *)(fac_s + 64);  // output row of result row r of the tile (-1: none), and the factor that undoes its prescale
+    if (tid < 64) {
+        int orow = tid < (a.pair_rows ? 32 : 64) ? ytile * (a.pair_rows ? 32 : 64) + tid : -1;
+        if (orow >= a.m) orow = -1;
+        if constexpr (GROUPED) orow = orow >= 0 ? a.perm[orow] : -1;  // the token this sorted row is
+        orow_s[tid] = orow;
+        fac_s[tid] = orow >= 0 ? a.rowfac[2 * orow + 1] : 0.f;
+    }
     __syncthreads();
     float *tile = (float *)smem + wave * (32 * STRIDE);  // this wave's own: 32 image rows at a time
     float *out = sg.out + (sg.k_slices > 1 ? (long long)ks * a.m * sg.n : 0LL);
@@ -219,7 +241,7 @@ __device__ __forceinline__ void gemv_wide_body(const GemvWArgs &a) {
         for (int it = 0; it < 4; it++) {
             const int trow = it * 8 + (l >> 3), irow = 32 * p + trow;  // row of the tile, image row
             float4_t v = *(const float4_t *)(tile + trow * STRIDE + (l & 7) * 4);
-            int row = irow;
+            int rrow = irow;  // result row of the tile
             bool live = true;
             if (a.pair_rows) {  // leading row 2 i, residual row 2 i + 1: lanes eight apart
                 float4_t lo;
@@ -228,13 +250,14 @@ __device__ __forceinline__ void gemv_wide_body(const GemvWArgs &a) {
 #pragma unroll
                 for (int e = 0; e < 4; e++) v[e] += lo[e] * (1.0f / GEMVW_LO_SCALE);
                 live = (irow & 1) == 0;
-                row = irow >> 1;
+                rrow = irow >> 1;
             }
-            if (!live || row >= a.m) continue;
-            const float f = fac_s[row];
+            const int orow = orow_s[rrow];
+            if (!live || orow < 0) continue;
+            const float f = fac_s[rrow];
 #pragma unroll
             for (int e = 0; e < 4; e++) v[e] *= f;
-            float *dst = out + (long long)row * sg.n + col;
+            float *dst = out + (long long)orow * sg.n + col;
             if (vec_ok && col + 3 < sg.n) {
                 *(float4_t *)dst = v;
             } else {
@@ -251,3 +274,5 @@ __device__ __forceinline__ void gemv_wide_body(const GemvWArgs &a) {
 // four waves per SIMD: two workgroups share a CU, one multiplies while the other waits for its chunk
 extern "C" __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) void rlx_gemvw_q4_0(rlx::GemvWArgs a) { rlx::gemv_wide_body<rlx::SCHEME_Q4_0>(a); }
 extern "C" __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) void rlx_gemvw_q8_0(rlx::GemvWArgs a) { rlx::gemv_wide_body<rlx::SCHEME_Q8_0>(a); }
+extern "C" __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) void rlx_gemvwg_q4_0(rlx::GemvWArgs a) { rlx::gemv_wide_body<rlx::SCHEME_Q4_0, true>(a); }
+extern "C" __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) void rlx_gemvwg_q8_0(rlx::GemvWArgs a) { rlx::gemv_wide_body<rlx::SCHEME_Q8_0, true>(a); }
