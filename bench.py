@@ -783,8 +783,7 @@ def other_configs(rlx_amd, stream, with_cpu):
                            "TFLOP/s": round(flops / total_ms / 1e9, 2),
                            "roofline": {"bound": "hbm" if t_hbm >= t_mfma else "mfma", "frac": round(max(t_hbm, t_mfma) / (total_ms * 1e-3), 4)},
                            "kernels": "rlx_gemv_q4_0_* (one batched launch)" if m <= 32 else
-                                      ("rlx_xprep + rlx_gemvw_q4_0" if m <= 64 else "rlx_xprep + rlx_gemm64_q4_0" if m <= 128 else
-                                       "rlx_xprep + rlx_gemm_q4_0") + " (+ rlx_splitk_reduce where K is cut)"}
+                                      ("rlx_xprep + rlx_gemvw_q4_0" if m <= 192 else "rlx_xprep + rlx_gemm_q4_0") + " (+ rlx_splitk_reduce where K is cut)"}
         for bfr in list(bufs.values()) + list(outs.values()) + ([ws] if ws else []):
             bfr.free()
     if with_cpu:  # the q projection at M = 1, in full

@@ -388,10 +388,12 @@ struct GemmPlan {
     size_t total() const { return image_end() + wimg_bytes + part_bytes; }
 };
 static bool gemm_skinny(int xk, int64_t m) { return (xk == 0 ? 2 * m : m) <= 128; }
-// Up to 64 image rows of Q4_0 / Q8_0 run rlx_gemvw_* (kernels/gemv_wide.hip): weights decoded in registers by the wave
-// that multiplies them, 256-row blocks of W per workgroup.
+// Up to 192 image rows of Q4_0 / Q8_0 run rlx_gemvw_* (kernels/gemv_wide.hip): weights decoded in registers by the wave
+// that multiplies them, 256-row blocks of W per workgroup, one pass over the weights per 64 image rows (grid.y). One 70B
+// layer, us, against the 64-row / 256-row prefill tiles: 96 rows 333 against 476, 128 rows 348 against 491, 160 rows 474
+// against 514, 192 rows 486 against 527; at 256 rows (four passes) 575 against 552, so the 256-row tile takes over there.
 static bool gemm_wide(int scheme, int xk, int64_t m) {
-    return (scheme == SCHEME_Q4_0 || scheme == SCHEME_Q8_0) && xk != XK_CODES && (xk == 0 ? 2 * m : m) <= 64;
+    return (scheme == SCHEME_Q4_0 || scheme == SCHEME_Q8_0) && xk != XK_CODES && (xk == 0 ? 2 * m : m) <= 192;
 }
 // K slices of one matrix in a launch of `launch_bytes` packed bytes in all: a workgroup should get about one CU's share
 // of the launch, at least 512 KB (one 70B layer at 64 rows, us: 218 with half a CU's share and 256 KB, 203 with this, 230
@@ -422,7 +424,7 @@ static GemmPlan gemm_plan(int scheme, int xk, int64_t m, int64_t k, int64_t n = 
     p.part_bytes = 0;
     if (n > 0 && gemm_wide(scheme, xk, m)) {
         const WeightDims D = weight_dims(scheme, n, k);
-        const GemmSplit sp = wide_split(layout_of(scheme), D, m, (size_t)D.bytes);  // alone in its launch: the most slices it can get
+        const GemmSplit sp = wide_split(layout_of(scheme), D, m, (size_t)D.bytes * (size_t)((rv + 63) / 64));  // alone in its launch: the most slices it can get
         if (sp.split > 1) p.part_bytes = (size_t)sp.split * (size_t)m * (size_t)n * 4;
     } else if (n > 0) {
         const Layout L = layout_of(scheme);
@@ -506,8 +508,10 @@ static int launch_gemm(const void *x, int xk, const rlx_qweight *const *ws, floa
     const int64_t k_units = codes ? p.k_pad / 64 : w->dims.units;  // K units of the operand the kernel reads
 
     if (gemm_wide(w->scheme, xk, m)) {
+        // every 64 image rows are a pass of their own over the weights (a second one finds part of them in L2)
+        const int64_t gy = ((xk == 0 ? 2 * m : m) + 63) / 64;
         size_t launch_bytes = 0, part_need = 0;
-        for (int i = 0; i < count; i++) launch_bytes += (size_t)ws[i]->dims.bytes;
+        for (int i = 0; i < count; i++) launch_bytes += (size_t)ws[i]->dims.bytes * (size_t)gy;
         GemmSplit sps[GEMVW_MAX_SEG];
         for (int i = 0; i < count; i++) {
             sps[i] = wide_split(ws[i]->layout, ws[i]->dims, m, launch_bytes);
@@ -535,7 +539,7 @@ static int launch_gemm(const void *x, int xk, const rlx_qweight *const *ws, floa
         wa.xh = xh;
         wa.rowfac = fac;
         void *wparams[] = {&wa};
-        RLX_TRY(launch(w->scheme == SCHEME_Q4_0 ? K_GEMVW_Q4_0 : K_GEMVW_Q8_0, (unsigned)wgs, 1, 512, 2 * 32768, stream, wparams));
+        RLX_TRY(launch3(w->scheme == SCHEME_Q4_0 ? K_GEMVW_Q4_0 : K_GEMVW_Q8_0, (unsigned)wgs, (unsigned)gy, 1, 512, 2 * 32768, stream, wparams));
         SplitReduceArgs ra{};
         int nred = 0;
         for (int i = 0; i < count; i++)
@@ -768,7 +772,7 @@ int rlx_mi355x_gguf_matmul_bt_batch(const void *const *xs_dev, int x_dtype, cons
         // q, k, v (and gate, up) of a layer share their input: its f16 image in the workspace is made once. An image
         // with block sums (Q4_K / Q5_K: per 32 columns; Q2_K: per 16) also serves a scheme that reads none, not the
         // other way round, and not a scheme that reads the other kind.
-        // Consecutive matrices with the same input and K go into one launch, up to GEMM_MAX_SEG at a time (GEMVW_MAX_SEG for the 33 - 64 row kernel).
+        // Consecutive matrices with the same input and K go into one launch, up to GEMM_MAX_SEG at a time (GEMVW_MAX_SEG for the 64-rows-a-pass kernel).
         const void *have_x = nullptr;
         int64_t have_k = -1;
         int have_sums = 0;
@@ -1228,7 +1232,7 @@ int rlx_mi355x_gguf_grouped_matmul_bt_ws(const void *x_dev, int x_dtype, const r
     void *sparams[] = {&sa};
     RLX_TRY(launch(K_MOE_SORT, 1, 1, 1024, 0, s, sparams));
     RLX_TRY(launch_xprep(x_dev, xk, m, w->dims.k, p.gemm, gws, s, perm, (int)p.perm_len));
-    if (w->scheme == SCHEME_Q4_0 || w->scheme == SCHEME_Q8_0) {  // a tile is 64 image rows: the 33 - 64 row kernel, one expert slab per tile
+    if (w->scheme == SCHEME_Q4_0 || w->scheme == SCHEME_Q8_0) {  // a tile is 64 image rows: the 64-rows-a-pass kernel, one expert slab per tile
         GemvWArgs wa{};
         wa.seg[0] = GemvWSeg{w->dev, out_dev, (int)w->dims.n, (int)w->dims.row_tiles, 0, 1, (int)((w->dims.units + 1) / 2 * 2)};
         wa.nseg = 1;

@@ -1,6 +1,7 @@
-// Matmul for 33 - 64 activation rows (17 - 32 f32 rows), Q4_0 and Q8_0: out[m, n] = x[m, k] . W[n, k]^T, the same
+// Matmul for 64 activation rows at a time (32 f32 rows), Q4_0 and Q8_0: out[m, n] = x[m, k] . W[n, k]^T, the same
 // product as rlx-cpu/src/gguf_matmul.rs:81-94, between the decode kernel (kernels/gemv.hip, up to 32 rows) and the
-// prefill tiles of kernels/gemm.hip. At this height the job is still to stream the weights once, so the kernel is built
+// 256-row prefill tile of kernels/gemm.hip; blockIdx.y walks the 64-row tiles of a taller batch (up to three of them,
+// one pass over the weights each, is where this still beats the 256-row tile). At this height the job is still to stream the weights once, so the kernel is built
 // like the decode kernel: a wave reads packed units in the device layout, which is the B operand of
 // v_mfma_f32_16x16x32_f16, decodes them in registers (d * code rounded to binary16, as the prefill kernels do) and
 // multiplies them by four groups of 16 activation rows; nothing of W goes through LDS and no wave waits for another
@@ -123,8 +124,8 @@ __device__ __forceinline__ void gemv_wide_body(const GemvWArgs &a) {
     // (tid >> 6) & 1, lane): constant per-thread offset in the image, the step in the scalar offset; in LDS piece p sits
     // at 16 p, i.e. a wave's 64 pieces of a step are 1 KB in a row: one buffer load with the LDS bit per step and wave,
     // no registers in between.
-    // (expert-sorted: tile y of 64 rows is sub-tiles 2 (y % 4), + 1 of the image's 256-row tile y / 4)
-    const int ytile = GROUPED ? (int)blockIdx.y : 0;
+    // (tile y of 64 rows is sub-tiles 2 (y % 4), + 1 of the image's 256-row tile y / 4)
+    const int ytile = (int)blockIdx.y;  // 64-row tile of the image
     const __amdgpu_buffer_rsrc_t x_rsrc =
         __builtin_amdgcn_make_buffer_rsrc((void *)(a.xh + (long long)(ytile >> 2) * a.k_steps * 32768), 0, 0x7FFFFFFF, 0x00020000);
     const int x_voff = ((tid >> 7) & 3) * 8192 + (2 * (ytile & 3) + ((tid >> 6) & 1)) * 1024 + l * 16;

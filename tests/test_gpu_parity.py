@@ -490,9 +490,13 @@ def test_gemm_small(oracle, scheme, m, n, k, x_dtype):
 @pytest.mark.parametrize("m,n,k,x_dtype", [(33, 272, 384, DType.BF16),    # ragged N (a dead tile in the block), three K units
                                            (64, 4112, 8192, DType.BF16),  # seventeen 256-row blocks, K cut across workgroups
                                            (20, 300, 1152, DType.F32),    # leading / residual row pairs, nine K units
-                                           (32, 512, 256, DType.F32), (48, 100, 128, DType.F16), (57, 16, 16384, DType.BF16)])
-def test_rows_33_to_64(oracle, scheme, m, n, k, x_dtype):
-    # the kernel between the decode kernel and the prefill tiles (Q4_0 / Q8_0, 33 - 64 binary16 rows or 17 - 32 f32 rows)
+                                           (32, 512, 256, DType.F32), (48, 100, 128, DType.F16), (57, 16, 16384, DType.BF16),
+                                           # taller batches walk the image 64 rows at a pass: two and three passes, f32 pairs across passes
+                                           (100, 528, 1280, DType.BF16), (192, 272, 512, DType.F16), (70, 300, 640, DType.F32),
+                                           (131, 4112, 4096, DType.BF16)])
+def test_rows_33_to_192(oracle, scheme, m, n, k, x_dtype):
+    # the kernel between the decode kernel and the 256-row prefill tile (Q4_0 / Q8_0, 33 - 192 image rows: binary16 rows, or
+    # half as many f32 rows)
     got, x, packed, _ = check_matmul(oracle, scheme, n, k, m, x_dtype=x_dtype, seed=3 * m + n,
                                      cols=None if n * k * m < (1 << 27) else (n - 40, n))
     xin = f32_to_bf16_bits(x) if x_dtype == DType.BF16 else x.astype(np.float16) if x_dtype == DType.F16 else x
