@@ -160,7 +160,9 @@ int rlx_mi355x_dequant(const rlx_qweight *w, float *out_dev, void *stream);
  * results are the same bits on every run. A workspace that holds only the activations (n = 0 in the size call) is
  * accepted: K is then cut in fewer slices or not at all.
  * m <= 16 (f32 activations) or m <= 32 (bf16 / f16) runs the decode kernels (weights streamed once, MFMA 16x16x32, one
- * or two groups of 16 rows per decoded weight fragment, an f32 row taking two); larger m runs the prefill GEMM. */
+ * or two groups of 16 rows per decoded weight fragment, an f32 row taking two); larger m converts the activations once
+ * (binary16 image in the workspace) and runs, for Q4_0 / Q8_0 up to 192 image rows, a kernel that still decodes the
+ * weights in registers, 64 rows a pass, otherwise the prefill GEMM tiles. */
 int rlx_mi355x_gguf_matmul_bt(const void *x_dev, int x_dtype, const rlx_qweight *w, float *out_dev, int64_t m,
                               void *workspace, size_t workspace_bytes, void *stream);
 size_t rlx_mi355x_gguf_matmul_workspace(int scheme, int x_dtype, int64_t m, int64_t k, int64_t n);

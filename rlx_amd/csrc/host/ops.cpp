@@ -454,8 +454,8 @@ static int launch_xprep(const void *x, int xk, int64_t m, int64_t k, const GemmP
 // Prefill path: convert the activations once (xprep), then the MFMA GEMM over `count` (<= GEMM_MAX_SEG) matrices of one
 // scheme and K that multiply the same x (q, k, v or gate, up of a layer): one launch, their tiles side by side, so
 // a small matrix fills the chip together with its neighbours instead of being cut into slivers of K on its own.
-// K is split across workgroups (atomic accumulation into zeroed outputs) only when the tile grid alone would leave
-// most CUs idle.
+// K is split across workgroups (slices written to the workspace, added in ascending K by one reduce launch) only when
+// the tile grid alone would leave most CUs idle. Q4_0 / Q8_0 up to 192 image rows go to the register-decode kernel instead.
 // `prepared`: the workspace already holds this x (same pointer, k, m, dtype, and the block sums if this scheme needs
 // them) from the previous launch of a batch on the same stream, so the conversion pass is skipped.
 static int launch_gemm(const void *x, int xk, const rlx_qweight *const *ws, float *const *outs, int count, int64_t m,
