@@ -35,6 +35,10 @@ struct FqArgs {
     int k_pad, m_rows;
     int write_out;       // 0: only the image (and the codes, if wanted) is written
     float *colscale;     // rlx_fq_col_apply_img only: [k_pad] copy of the column scales for the weight-scaling pass
+    // Column layout with a maximum pass: one word that ends up holding the largest scale of all channels (its bits; scales
+    // are positive, so unsigned order is value order): cleared by the maximum pass, raised by the scale pass. Null: whoever
+    // needs the largest scale scans the scales.
+    uint32_t *smax_bits;
 };
 
 __device__ __forceinline__ float fq_scale_from_max(float max_abs, float q_max) {
@@ -55,6 +59,7 @@ __device__ __forceinline__ int8_t fq_i8(float q) { return (q != q) ? (int8_t)0 :
 // ---- pass A ------------------------------------------------------------------------------------------
 
 __device__ __forceinline__ void col_absmax(const FqArgs &a) {
+    if (a.smax_bits && blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) *a.smax_bits = 0;  // raised by the scale pass, the next launch
     const long long c4 = ((long long)blockIdx.x * blockDim.x + threadIdx.x) * 4;
     if (c4 >= a.chan_dim) return;
     const long long rows = a.len / a.chan_dim;
@@ -126,7 +131,7 @@ __device__ __forceinline__ void flat_absmax(const FqArgs &a) {
 // ---- scale --------------------------------------------------------------------------------------------
 
 // s[c] from the channel's max|x| (PerBatch), blended into the state (EMA) or read from it (Fixed).
-__device__ __forceinline__ void scale_from_max(const FqArgs &a, long long c, float max_abs) {
+__device__ __forceinline__ float scale_from_max(const FqArgs &a, long long c, float max_abs) {
     float s;
     if (a.scale_mode == 2) {  // Fixed
         float v = a.state[c];
@@ -149,6 +154,7 @@ __device__ __forceinline__ void scale_from_max(const FqArgs &a, long long c, flo
         }
     }
     a.scale[c] = s;
+    return s;
 }
 
 __device__ __forceinline__ void make_scale(const FqArgs &a) {
@@ -180,7 +186,16 @@ __device__ __forceinline__ void make_scale_parts(const FqArgs &a) {
             m = v > m ? v : m;
         }
         a.max_bits[c] = __builtin_bit_cast(uint32_t, m);
-        scale_from_max(a, c, m);
+        m = scale_from_max(a, c, m);
+    }
+    if (grp == 0 && a.smax_bits) {  // wave 0: the largest of its 64 scales, one atomic per workgroup
+        float s = c < a.chan_dim ? m : 0.f;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            const float o = __shfl_xor(s, off);
+            s = o > s ? o : s;
+        }
+        if (cl == 0) atomicMax(a.smax_bits, __builtin_bit_cast(uint32_t, s));
     }
 }
 
@@ -230,19 +245,23 @@ __device__ __forceinline__ void col_apply_img(const FqArgs &a) {
     __shared__ float wave_max[4];
     const int tid = threadIdx.x;
     float smax = 0.f;
-    for (long long c = tid; c < a.chan_dim; c += blockDim.x) {
-        const float v = a.scale[c];
-        smax = v > smax ? v : smax;
-    }
+    if (a.smax_bits) {  // left by the scale pass
+        smax = __builtin_bit_cast(float, *a.smax_bits);
+    } else {
+        for (long long c = tid; c < a.chan_dim; c += blockDim.x) {
+            const float v = a.scale[c];
+            smax = v > smax ? v : smax;
+        }
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-        const float o = __shfl_xor(smax, off);
-        smax = o > smax ? o : smax;
+        for (int off = 32; off > 0; off >>= 1) {
+            const float o = __shfl_xor(smax, off);
+            smax = o > smax ? o : smax;
+        }
+        if ((tid & 63) == 0) wave_max[tid >> 6] = smax;
+        __syncthreads();
+        smax = wave_max[0];
+        for (int w = 1; w < (int)(blockDim.x >> 6); w++) smax = wave_max[w] > smax ? wave_max[w] : smax;
     }
-    if ((tid & 63) == 0) wave_max[tid >> 6] = smax;
-    __syncthreads();
-    smax = wave_max[0];
-    for (int w = 1; w < (int)(blockDim.x >> 6); w++) smax = wave_max[w] > smax ? wave_max[w] : smax;
     float inv = 1.f, big = 1.f;
     const uint32_t mb = __builtin_bit_cast(uint32_t, smax);
     if (mb >= 0x00800000u && mb < 0x7F800000u) {  // a normal number: its exponent
