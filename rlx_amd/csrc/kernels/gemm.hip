@@ -96,9 +96,11 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
     constexpr int NSA = MT / 32, SA = 4 * NSA * 1024, ST = SA + GEMM_STAGE_B;  // LDS stage: activations [4][NSA][1 KB], then weights
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     // Q4_K / Q5_K: what the per-super-block scaling needs goes through LDS instead of living in registers for two steps.
-    // sb_meta_s[parity of the super-block][W row of the tile]: the row's 16 meta bytes, left by the wave that decodes the row;
+    // sb_min_s / sb_dd_s[parity of the super-block][W row of the tile]: the row's eight 6-bit mins as binary16 integers and its
+    // (d, dmin) pair, left by the wave that decodes the row so that the scaling step has no bytes to take apart;
     // sb_sum_s[half][x row of the tile]: the eight leading / eight residual block sums of the super-block being multiplied.
-    __shared__ uint4_t sb_meta_s[K4 ? 2 * GEMM_NT : 1];
+    __shared__ uint4_t sb_min_s[K4 ? 2 * GEMM_NT : 1];
+    __shared__ uint32_t sb_dd_s[K4 ? 2 * GEMM_NT : 1];
     __shared__ uint4_t sb_sum_s[K4 ? 2 * MT : 1];
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -235,10 +237,22 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
             if (q == 0 && jl == 0) {
                 uint32_t mn[2];
                 const uint4_t &m4 = b_meta[0];
-                if (b_g == 0) sb_meta_s[((step >> 2) & 1) * GEMM_NT + wave * 16 + b_n16] = m4;  // for scale_sb, several steps from now
                 q4k_scales(m4[1], m4[2], m4[3], b_sc, mn);
                 b_sc[0] &= b_keep;  // a dead tile decodes to zeros
                 b_sc[1] &= b_keep;
+                // for scale_sb, several steps from now: mn_0..7 in the k-slot order of its B' fragment, and d, dmin (0 for a dead tile)
+                Frag fm;
+                const half2_t k1024 = {(half_t)1024.0f, (half_t)1024.0f};
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const uint32_t sel = (e & 1) ? 0x04030402u : 0x04010400u;  // bytes (2,3) or (0,1) -> [b,0x64,b',0x64]
+                    fm.h2[e] = as_half2(__builtin_amdgcn_perm(0x64646464u, mn[e >> 1], sel)) - k1024;
+                }
+                if (b_g == 0) {
+                    const int at = ((step >> 2) & 1) * GEMM_NT + wave * 16 + b_n16;
+                    sb_min_s[at] = fm.u4;
+                    sb_dd_s[at] = m4[0] & b_keep;
+                }
             }
             if constexpr (K5)
                 unpack_q5_scaled(b_q[cp][t], __builtin_amdgcn_alignbit(b_hw[cp][0], b_hw[cp][0], q5k_rot(t)), splat_code_half(b_sc[q >> 1], t), f);
@@ -374,7 +388,10 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
     auto scale_sb = [&](int sb) {
         if constexpr (K4) {
 #pragma unroll
-            for (int j = 0; j < TJ; j++) w_meta[j] = sb_meta_s[(sb & 1) * GEMM_NT + (wn * TJ + j) * 32 + lr];
+            for (int j = 0; j < TJ; j++) {
+                w_meta[j] = sb_min_s[(sb & 1) * GEMM_NT + (wn * TJ + j) * 32 + lr];
+                w_dd[j] = sb_dd_s[(sb & 1) * GEMM_NT + (wn * TJ + j) * 32 + lr];
+            }
 #pragma unroll
             for (int i = 0; i < TI; i++) fs[i].u4 = sb_sum_s[lh * MT + (wm * TI + i) * 32 + lr];
         }
@@ -428,22 +445,16 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
         }
 #pragma unroll
         for (int j = 0; j < TJ; j++) {
-            const uint4_t meta = w_meta[j];
-            const float d = my_ok[j] ? half_bits_to_float(meta[0] & 0xFFFFu) : 0.f;
-            const float dmin = my_ok[j] ? half_bits_to_float(meta[0] >> 16) : 0.f;
-            uint32_t sc[2], mn[2];
-            q4k_scales(meta[1], meta[2], meta[3], sc, mn);
+            const float d = half_bits_to_float(w_dd[j] & 0xFFFFu);
+            const float dmin = half_bits_to_float(w_dd[j] >> 16);
             // B' fragment: half 0 holds mn_0..7, half 1 holds mn_0..7 / 2048 (pairs with the lo sums)
             Frag fm;
-            const half2_t k1024 = {(half_t)1024.0f, (half_t)1024.0f};
+            fm.u4 = w_meta[j];
+            const half2_t one2 = {(half_t)1.0f, (half_t)1.0f};
             const half2_t lo_scale = {(half_t)(1.0f / GEMM_LO_SCALE), (half_t)(1.0f / GEMM_LO_SCALE)};
+            const half2_t half_scale = lh ? lo_scale : one2;
 #pragma unroll
-            for (int e = 0; e < 4; e++) {
-                uint32_t src = (e < 2) ? mn[0] : mn[1];
-                uint32_t sel = (e & 1) ? 0x04030402u : 0x04010400u;  // bytes (2,3) or (0,1) -> [b,0x64,b',0x64]
-                half2_t v = as_half2(__builtin_amdgcn_perm(0x64646464u, src, sel)) - k1024;
-                fm.h2[e] = lh ? v * lo_scale : v;
-            }
+            for (int e = 0; e < 4; e++) fm.h2[e] = fm.h2[e] * half_scale;
 #pragma unroll
             for (int i = 0; i < TI; i++) {
                 float16_t qq = mfma32(fs[i], fm, zero16);
