@@ -443,27 +443,42 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a) {
             }
             return;
         }
+        // Per wave tile (i, j): A = the sixteen total += d * P, M = the matrix instruction Q = sums . mins, B = the sixteen
+        // total -= dmin * Q. Issued as A0 M0 | A1 M1 B0 | A2 M2 B1 | ... | B_last with fences between the groups: an MFMA's
+        // result is first read sixteen independent multiply-adds after its issue, and Q can take the registers of the P
+        // that A has just consumed. (Left to itself the compiler pairs A and B element by element behind an idle wait
+        // for M.) d and dmin are made plain f32 registers first: folded into v_fma_mix_f32 as binary16 operands, every
+        // dependent pair costs a wait state.
+        Frag fm[TJ];
+        float d[TJ], ndmin[TJ];
+        const half2_t one2 = {(half_t)1.0f, (half_t)1.0f};
+        const half2_t lo_scale = {(half_t)(1.0f / GEMM_LO_SCALE), (half_t)(1.0f / GEMM_LO_SCALE)};
+        const half2_t half_scale = lh ? lo_scale : one2;
 #pragma unroll
         for (int j = 0; j < TJ; j++) {
-            const float d = half_bits_to_float(w_dd[j] & 0xFFFFu);
-            const float dmin = half_bits_to_float(w_dd[j] >> 16);
+            d[j] = half_bits_to_float(w_dd[j] & 0xFFFFu);
+            ndmin[j] = -half_bits_to_float(w_dd[j] >> 16);
+            asm volatile("" : "+v"(d[j]), "+v"(ndmin[j]));
             // B' fragment: half 0 holds mn_0..7, half 1 holds mn_0..7 / 2048 (pairs with the lo sums)
-            Frag fm;
-            fm.u4 = w_meta[j];
-            const half2_t one2 = {(half_t)1.0f, (half_t)1.0f};
-            const half2_t lo_scale = {(half_t)(1.0f / GEMM_LO_SCALE), (half_t)(1.0f / GEMM_LO_SCALE)};
-            const half2_t half_scale = lh ? lo_scale : one2;
+            fm[j].u4 = w_meta[j];
 #pragma unroll
-            for (int e = 0; e < 4; e++) fm.h2[e] = fm.h2[e] * half_scale;
+            for (int e = 0; e < 4; e++) fm[j].h2[e] = fm[j].h2[e] * half_scale;
+        }
+        float16_t qq[2];
 #pragma unroll
-            for (int i = 0; i < TI; i++) {
-                float16_t qq = mfma32(fs[i], fm, zero16);
+        for (int t = 0; t <= TI * TJ; t++) {
+            if (t < TI * TJ) {
+                const int i = t % TI, j = t / TI;
 #pragma unroll
-                for (int e = 0; e < 16; e++) {
-                    total[i][j][e] = __builtin_fmaf(d, part[i][j][e], total[i][j][e]);
-                    total[i][j][e] = __builtin_fmaf(-dmin, qq[e], total[i][j][e]);
-                }
+                for (int e = 0; e < 16; e++) total[i][j][e] = __builtin_fmaf(d[j], part[i][j][e], total[i][j][e]);
+                qq[t & 1] = mfma32(fs[i], fm[j], zero16);
             }
+            if (t > 0) {
+                const int i = (t - 1) % TI, j = (t - 1) / TI;
+#pragma unroll
+                for (int e = 0; e < 16; e++) total[i][j][e] = __builtin_fmaf(ndmin[j], qq[(t - 1) & 1][e], total[i][j][e]);
+            }
+            __builtin_amdgcn_sched_barrier(0);
         }
     };
 
